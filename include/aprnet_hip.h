@@ -1,0 +1,140 @@
+/* aprnet_hip.h — C ABI of the MI355X (gfx950) particle-space CNN operators.
+ *
+ * Drop-in boundary for the native functions that APR-CNN registers on
+ * `_pyaprwrapper.aprnet.{conv,pool,upsample,utils,cuda}` (wrappers/pythonBind.cpp:144-182).
+ * Each entry point below names the reference function it replaces.
+ *
+ * Conventions
+ *  - Every function returns 0 on success and a negative aprnet_status otherwise; the message of
+ *    the last failure on the calling thread is available from aprnet_last_error().  Nothing throws.
+ *  - An `aprnet_plan` is the device-side image of one APR (what `APR::init_cuda()` /
+ *    `GPUAccessHelper` is in the reference, wrap_conv_gpu.hpp:23-28): the access arrays plus the
+ *    child table and tile lists derived from them.  It is created from HOST arrays and owns its
+ *    device memory.  All other pointers are DEVICE pointers owned by the caller.
+ *  - Operators work on ONE batch item: features are `C` channel planes of `n` particles, plane `c`
+ *    starting at `base + c*ld` (ld in elements).  The reference's batch loop
+ *    (conv.hpp:99, wrap_conv_gpu.hpp:23-28) stays on the caller's side.
+ *  - `level_delta` d is the number of finest levels pooled away (helpers.hpp:86-117);
+ *    Lc = level_max - d.  A feature vector at d holds aprnet_number_parts(plan, d) values.
+ *  - No function allocates caller-visible memory; work space is passed in.  Kernels are enqueued
+ *    on `stream` (a hipStream_t passed as void*) and the call returns without synchronising.
+ *  - Suffix _f32 / _f64 = element type of features, weights and gradients.
+ */
+#ifndef APRNET_HIP_H
+#define APRNET_HIP_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum aprnet_status {
+    APRNET_OK = 0,
+    APRNET_ERR_INVALID_ARGUMENT = -1,   /* std::invalid_argument in the reference (conv.hpp:63-66, upsample.hpp:49-54) */
+    APRNET_ERR_LEVEL_DELTA = -2,        /* CHECK_LEVEL_DELTA (cuda/src/common.hpp:17) */
+    APRNET_ERR_HIP = -3,                /* a HIP runtime call failed */
+    APRNET_ERR_UNSUPPORTED = -4
+} aprnet_status;
+
+/* One linear access structure, as LibAPR's LinearAccess / GPUAccessHelper expose it
+ * (row lookup idiom: conv333_gpu.cu:65-67; state: data_containers/src/BindAPR.hpp:72-108).
+ * All pointers are host pointers; the arrays are copied. */
+typedef struct aprnet_access_desc {
+    int32_t level_min, level_max;
+    const int32_t* z_num;            /* [level_max+1], indexed by level */
+    const int32_t* x_num;
+    const int32_t* y_num;
+    const uint64_t* level_xz_vec;    /* [level_max+2] */
+    const uint64_t* xz_end_vec;      /* [n_rows] with leading sentinel 0 */
+    const uint16_t* y_vec;           /* [n_particles] */
+    uint64_t n_rows;
+    uint64_t n_particles;
+} aprnet_access_desc;
+
+typedef struct aprnet_plan aprnet_plan;
+
+const char* aprnet_last_error(void);
+
+/* Replaces APR::init_cuda() + gpuAPRHelper()/gpuTreeHelper() (wrap_conv_gpu.hpp:25-26). */
+int aprnet_plan_create(const aprnet_access_desc* apr, const aprnet_access_desc* tree, int device, aprnet_plan** out);
+void aprnet_plan_destroy(aprnet_plan* plan);
+
+/* helpers::number_parts (helpers.hpp:86-101); also number_parts_after_pooling/_upsampling with d±1. */
+int64_t aprnet_number_parts(const aprnet_plan* plan, int level_delta);
+/* helpers::compute_tree_offset (helpers.hpp:113-117) for `level`. */
+int64_t aprnet_tree_offset(const aprnet_plan* plan, int level);
+/* tree_it.total_number_particles(Lc-1): length of the tree work space at d (helpers.hpp:166). */
+int64_t aprnet_tree_parts(const aprnet_plan* plan, int level_delta);
+/* Copies the child table to host: int32 [8][n_tree]; slot s = 4*dz+2*dx+dy of tree node t holds the
+ * particle index (>= 0), ~tree_index (< 0, != INT32_MIN) or INT32_MIN when the child cell lies outside
+ * the image.  This is the index map behind the parent walks of helpers.hpp:185-194, maxpool.hpp:106-117,
+ * upsample.hpp:112-118. */
+int aprnet_plan_children(const aprnet_plan* plan, int32_t* out_host);
+
+#define APRNET_DECL(T, SFX)                                                                                          \
+    /* helpers::fill_tree_mean (helpers.hpp:156-252): tree[c][t] for all tree nodes of level < Lc. */               \
+    int aprnet_fill_tree_mean_##SFX(const aprnet_plan*, int level_delta, const T* x, int64_t ldx, int C,            \
+                                    T* tree, int64_t ld_tree, void* stream);                                        \
+    /* helpers::fill_tree_mean_backward (helpers.hpp:255-350): pushes grad_tree root->leaf (grad_tree is            \
+     * modified) and ACCUMULATES into grad_x. */                                                                    \
+    int aprnet_fill_tree_mean_bwd_##SFX(const aprnet_plan*, int level_delta, T* grad_x, int64_t ldx, int C,         \
+                                        T* grad_tree, int64_t ld_tree, void* stream);                               \
+    /* Convolution<kz,kx,ky>::forward (conv.hpp:55-195), CUDA twin conv333_forward (wrap_conv_gpu.hpp:32-66).       \
+     * (kz,kx,ky) in {333,133,155,555}.  w: expanded stencils [S_exp][Cout][Cin][kz][kx][ky] (the layout of         \
+     * cuda/conv.py:77).  y is OVERWRITTEN for indices < number_parts(d).  tree_ws: [Cin][ld_tree] scratch,         \
+     * ld_tree >= aprnet_tree_parts(plan, d). */                                                                    \
+    int aprnet_conv_fwd_##SFX(const aprnet_plan*, int level_delta, int kz, int kx, int ky,                          \
+                              const T* x, int64_t ldx, int Cin, const T* w, int S_exp, int Cout,                    \
+                              T* y, int64_t ldy, T* tree_ws, int64_t ld_tree, void* stream);                        \
+    /* Convolution<kz,kx,ky>::backward (conv.hpp:261-481), CUDA twin conv333_backward.  grad_x is OVERWRITTEN,      \
+     * grad_w [S_exp][Cout][Cin][k] is ACCUMULATED into (zero it before the first batch item, as                    \
+     * torch::zeros_like does in conv.hpp:270).  tree_ws / grad_tree_ws: [Cin][ld_tree] scratch each. */            \
+    int aprnet_conv_bwd_##SFX(const aprnet_plan*, int level_delta, int kz, int kx, int ky,                          \
+                              const T* x, int64_t ldx, int Cin, const T* w, int S_exp, int Cout,                    \
+                              const T* grad_y, int64_t ldy, T* grad_x, int64_t ldgx, T* grad_w,                     \
+                              T* tree_ws, int64_t ld_tree, T* grad_tree_ws, int64_t ld_gtree, void* stream);        \
+    /* Convolution<1,1,1>::forward/backward (conv.hpp:199-256, 484-554); w: [S][Cout][Cin] (not expanded,           \
+     * stencil index min(S-1, Lc-level)).  grad_w is accumulated, grad_x overwritten. */                            \
+    int aprnet_conv111_fwd_##SFX(const aprnet_plan*, int level_delta, const T* x, int64_t ldx, int Cin,             \
+                                 const T* w, int S, int Cout, T* y, int64_t ldy, void* stream);                     \
+    int aprnet_conv111_bwd_##SFX(const aprnet_plan*, int level_delta, const T* x, int64_t ldx, int Cin,             \
+                                 const T* w, int S, int Cout, const T* grad_y, int64_t ldy,                         \
+                                 T* grad_x, int64_t ldgx, T* grad_w, void* stream);                                 \
+    /* MaxPool::forward (maxpool.hpp:43-146): y[c][0:number_parts(d+1)], argmax = INPUT index, ties resolved in     \
+     * the CPU traversal order (z, x, y; particles before downsampled particles; strict >). */                     \
+    int aprnet_maxpool_fwd_##SFX(const aprnet_plan*, int level_delta, const T* x, int64_t ldx, int C,               \
+                                 T* y, int64_t ldy, int64_t* argmax, int64_t ldi, void* stream);                    \
+    /* MaxPool::backward (maxpool.hpp:149-230): grad_x[0:number_parts(d)] overwritten. */                          \
+    int aprnet_maxpool_bwd_##SFX(const aprnet_plan*, int level_delta, const T* grad_y, int64_t ldy, int C,          \
+                                 T* grad_x, int64_t ldx, const int64_t* argmax, int64_t ldi, void* stream);         \
+    /* UpSampleConst::forward/backward (upsample.hpp:39-236); level_delta is that of the INPUT (> 0). */           \
+    int aprnet_upsample_fwd_##SFX(const aprnet_plan*, int level_delta, const T* x, int64_t ldx, int C,              \
+                                  T* y, int64_t ldy, void* stream);                                                 \
+    int aprnet_upsample_bwd_##SFX(const aprnet_plan*, int level_delta, const T* grad_y, int64_t ldy, int C,         \
+                                  T* grad_x, int64_t ldx, void* stream);                                            \
+    /* RestrictKernel<kz,kx,ky>::forward/backward (kernel.hpp:31-224) on [S][Cout][Cin][k] weights:                 \
+     * w [S][n_filters][k] -> w_exp [S_exp][n_filters][k] with n_filters = Cout*Cin; backward is the transpose. */  \
+    int aprnet_restrict_kernel_fwd_##SFX(const T* w, int S, int n_filters, int kz, int kx, int ky, int S_exp,       \
+                                         T* w_exp, void* stream);                                                   \
+    int aprnet_restrict_kernel_bwd_##SFX(const T* grad_w_exp, int S_exp, int n_filters, int kz, int kx, int ky,     \
+                                         int S, T* grad_w, void* stream);                                           \
+    /* reconstruct_forward/backward (cuda/src/reconstruct_gpu.cu:3-197): particles -> dense                         \
+     * [C][z_num(Lc)][x_num(Lc)][y_num(Lc)], plane stride ld_img; cells no particle covers keep their value. */     \
+    int aprnet_reconstruct_fwd_##SFX(const aprnet_plan*, int level_delta, const T* x, int64_t ldx, int C,           \
+                                     T* img, int64_t ld_img, void* stream);                                         \
+    int aprnet_reconstruct_bwd_##SFX(const aprnet_plan*, int level_delta, const T* grad_img, int64_t ld_img, int C, \
+                                     T* grad_x, int64_t ldx, void* stream);                                         \
+    /* sample_particles_forward/backward (cuda/src/sample_particles_gpu.cu:3-246): dense -> particles (cell mean). */\
+    int aprnet_sample_particles_fwd_##SFX(const aprnet_plan*, int level_delta, const T* img, int64_t ld_img, int C, \
+                                          T* y, int64_t ldy, void* stream);                                         \
+    int aprnet_sample_particles_bwd_##SFX(const aprnet_plan*, int level_delta, const T* grad_y, int64_t ldy, int C, \
+                                          T* grad_img, int64_t ld_img, void* stream);
+
+APRNET_DECL(float, f32)
+APRNET_DECL(double, f64)
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* APRNET_HIP_H */
