@@ -1,0 +1,51 @@
+#!/usr/bin/env python3
+"""Builds the native libraries in-tree:
+     libaprnet_hip.so  HIP operators for gfx950 (hipcc, one translation unit per .hip file)
+     libaprcore.so     host-only APR builder (g++ / OpenMP)
+Usage: python build.py [--force]"""
+import os
+import subprocess
+import sys
+from concurrent.futures import ThreadPoolExecutor
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+HIP_SOURCES = ["plan.hip", "tree_ops.hip", "conv.hip", "conv_bwd.hip", "conv111.hip", "restrict.hip", "pixels.hip"]
+HIP_FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fno-gpu-rdc",
+             "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+             "-Wno-unused-command-line-argument", "-Wno-unknown-attributes"]
+HEADERS = ["common.hpp", "conv_common.hpp", os.path.join("..", "..", "include", "aprnet_hip.h")]
+
+
+def _newer(target, deps):
+    if not os.path.exists(target):
+        return True
+    t = os.path.getmtime(target)
+    return any(os.path.getmtime(d) > t for d in deps if os.path.exists(d))
+
+
+def build(force=False, verbose=True):
+    os.chdir(HERE)
+    objs, jobs = [], []
+    for src in HIP_SOURCES:
+        if not os.path.exists(src):
+            continue
+        obj = src.replace(".hip", ".o")
+        objs.append(obj)
+        if force or _newer(obj, [src] + HEADERS):
+            jobs.append([HIPCC, *HIP_FLAGS, "-c", src, "-o", obj])
+    def run(cmd):
+        if verbose:
+            print(" ".join(cmd), flush=True)
+        subprocess.check_call(cmd)
+    with ThreadPoolExecutor(max_workers=min(8, max(1, len(jobs)))) as ex:
+        list(ex.map(run, jobs))
+    if force or jobs or not os.path.exists("libaprnet_hip.so"):
+        run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", "libaprnet_hip.so", *objs])
+    if force or _newer("libaprcore.so", ["aprcore.cpp"]):
+        run(["g++", "-O3", "-march=x86-64-v3", "-fopenmp", "-shared", "-fPIC", "-std=c++17", "-o", "libaprcore.so", "aprcore.cpp"])
+    return os.path.join(HERE, "libaprnet_hip.so"), os.path.join(HERE, "libaprcore.so")
+
+
+if __name__ == "__main__":
+    build(force="--force" in sys.argv)

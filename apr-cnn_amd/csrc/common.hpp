@@ -1,0 +1,105 @@
+// Shared declarations of the HIP operator library (gfx950 only).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <cstdint>
+#include <climits>
+#include <map>
+#include <string>
+#include <tuple>
+#include <vector>
+
+#include "../../include/aprnet_hip.h"
+
+namespace aprnet {
+
+constexpr int MAX_LEVELS = 18;          // levels 0..17 (y_vec is uint16 -> dims <= 65536 -> level_max <= 16)
+constexpr int32_t NO_CHILD = INT32_MIN; // child-table sentinel: cell outside the image
+
+// Device view of one linear access structure; passed to kernels by value.
+struct AccessDev {
+    const uint64_t* xz_end;             // device, row table with leading 0
+    const uint16_t* y;                  // device
+    uint64_t level_xz[MAX_LEVELS + 1];
+    int32_t z_num[MAX_LEVELS], x_num[MAX_LEVELS], y_num[MAX_LEVELS];
+    int32_t level_min, level_max;
+
+    __device__ __forceinline__ uint64_t row(int l, int z, int x) const { return level_xz[l] + (uint64_t)z * x_num[l] + x; }
+};
+
+struct HostAccess {
+    int level_min = 0, level_max = 0;
+    std::vector<int32_t> z_num, x_num, y_num;
+    std::vector<uint64_t> level_xz, xz_end;
+    std::vector<uint16_t> y;
+    uint64_t n = 0;
+    uint64_t row(int l, int z, int x) const { return level_xz[l] + (uint64_t)z * x_num[l] + x; }
+    // first index of level l / one past the last index of level l (levels outside the range are empty)
+    int64_t level_begin(int l) const {
+        if (l < level_min) return 0;
+        if (l > level_max) return (int64_t)n;
+        return (int64_t)xz_end[level_xz[l] - 1];
+    }
+    int64_t level_end(int l) const {
+        if (l < level_min) return 0;
+        if (l > level_max) return (int64_t)n;
+        return (int64_t)xz_end[level_xz[l + 1] - 1];
+    }
+};
+
+struct ConvTile { int32_t level, z0, x0, pad; };
+
+struct TileList { ConvTile* d_tiles = nullptr; int n = 0; };
+
+}  // namespace aprnet
+
+struct aprnet_plan {
+    int device = 0;
+    aprnet::HostAccess apr, tree;
+    aprnet::AccessDev dapr{}, dtree{};
+    void* d_apr_xz = nullptr; void* d_apr_y = nullptr; void* d_tree_xz = nullptr; void* d_tree_y = nullptr;
+    int32_t* d_children = nullptr;      // [8][n_tree], slot-major
+    int64_t n_tree = 0, n_apr = 0;
+    std::map<std::tuple<int, int, int>, aprnet::TileList> tiles;   // (level_delta, TZ, TX) -> non-empty row groups
+
+    int lc(int level_delta) const { return apr.level_max - level_delta; }
+    int64_t number_parts(int level_delta) const {
+        const int L = lc(level_delta);
+        int64_t n = apr.level_end(L);
+        if (L <= tree.level_max && L >= tree.level_min) n += tree.level_end(L) - tree.level_begin(L);
+        return n;
+    }
+    int64_t tree_offset(int level) const { return apr.level_end(level) - tree.level_begin(level); }
+    int64_t tree_parts(int level_delta) const { const int L = lc(level_delta); return L >= 1 ? tree.level_end(L - 1) : 0; }
+};
+
+namespace aprnet {
+
+void set_error(const std::string& msg);
+int fail(int code, const std::string& msg);
+// non-empty row groups for the convolution at `level_delta` (built on first use, cached in the plan)
+int get_tiles(aprnet_plan* plan, int level_delta, int TZ, int TX, TileList* out);
+
+#define APRNET_HIP_CHECK(expr)                                                                                  \
+    do {                                                                                                        \
+        hipError_t e_ = (expr);                                                                                 \
+        if (e_ != hipSuccess)                                                                                   \
+            return aprnet::fail(APRNET_ERR_HIP, std::string(#expr) + ": " + hipGetErrorString(e_));             \
+    } while (0)
+
+#define APRNET_LAUNCH_CHECK(name)                                                                               \
+    do {                                                                                                        \
+        hipError_t e_ = hipGetLastError();                                                                      \
+        if (e_ != hipSuccess)                                                                                   \
+            return aprnet::fail(APRNET_ERR_HIP, std::string("launch of ") + name + ": " + hipGetErrorString(e_)); \
+    } while (0)
+
+inline int check_level_delta(const aprnet_plan* p, int d, const char* who) {
+    if (!p) return fail(APRNET_ERR_INVALID_ARGUMENT, std::string(who) + ": null plan");
+    // CHECK_LEVEL_DELTA(dlvl, tree.level_max()+1): cuda/src/common.hpp:17, wrap_conv_gpu.hpp:46
+    if (d < 0 || d >= p->tree.level_max + 1)
+        return fail(APRNET_ERR_LEVEL_DELTA, std::string(who) + ": level delta " + std::to_string(d) +
+                    " is too large for APR with maximum level " + std::to_string(p->apr.level_max));
+    return 0;
+}
+
+}  // namespace aprnet

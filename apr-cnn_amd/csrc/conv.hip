@@ -1,0 +1,162 @@
+// Stencil convolution on APR particles, forward (VALU path): Convolution<kz,kx,ky>::forward
+// (conv.hpp:55-195) for stencils 3x3x3, 1x3x3, 1x5x5 and 5x5x5, fp32 and fp64.
+//
+// Per window (see conv_common.hpp) the block loops over chunks of CIB input channels: zero the LDS
+// patch, gather the chunk from the three sources, then every thread owns up to ITER output
+// positions ("columns") and COB output channels in registers.  The taps of a column come from LDS,
+// the weights are wave-uniform and are fetched through the scalar cache.  All input channels are
+// reduced inside the block, so each output element is written exactly once: no atomics, and the
+// result does not depend on scheduling.  As in the reference, the sum over the K taps of one input
+// channel is formed first and then added to the running output (helpers.hpp:537-544).
+#include "conv_common.hpp"
+
+namespace aprnet {
+
+template <typename T, class G, int CIB, int COB>
+__global__ void __launch_bounds__(G::NT)
+conv_fwd_kernel(const ConvArgs<T> a) {
+    __shared__ T patch[CIB * G::CH_STRIDE];
+    __shared__ ConvShared<G> sh;
+
+    const ConvTile tile = a.tiles[blockIdx.x];
+    const int L = tile.level, z0 = tile.z0, x0 = tile.x0;
+    const int co0 = blockIdx.y * COB;
+    const int yn = a.apr.y_num[L];
+    const int s_idx = min(a.S_exp - 1, a.Lc - L);
+    const bool out_tree = (L == a.Lc) && (L < a.apr.level_max);
+    const T* __restrict__ wl = a.w + (int64_t)s_idx * a.Cout * a.Cin * G::K;
+
+    open_segments<G, T>(a, L, z0, x0, sh);
+    __syncthreads();
+
+    int yv[G::SPW];
+    unsigned long long inw;
+    for (int y0 = 0; y0 < yn; y0 += G::TY) {
+        scan_window<G, T>(a, L, y0, out_tree, sh, yv, inw);
+        __syncthreads();
+        const int nc = sh.ncol;
+        if (nc > 0) {
+            T acc[G::ITER][COB];
+#pragma unroll
+            for (int it = 0; it < G::ITER; ++it)
+#pragma unroll
+                for (int co = 0; co < COB; ++co) acc[it][co] = 0;
+
+            for (int ci0 = 0; ci0 < a.Cin; ci0 += CIB) {
+                for (int i = threadIdx.x; i < CIB * G::CH_STRIDE; i += G::NT) patch[i] = 0;
+                __syncthreads();
+                stage_values<G, T, CIB>(a, L, y0, ci0, sh, yv, inw, patch);
+                __syncthreads();
+#pragma unroll
+                for (int it = 0; it < G::ITER; ++it) {
+                    const int col = threadIdx.x + it * G::NT;
+                    if (col >= nc) continue;
+                    const T* p0 = patch + (int)sh.col_pos[col] - G::TAP0;
+#pragma unroll 1
+                    for (int c = 0; c < CIB; ++c) {
+                        const int ci = ci0 + c;
+                        if (ci >= a.Cin) break;
+                        T v[G::K];
+#pragma unroll
+                        for (int sz = 0; sz < G::KZ; ++sz)
+#pragma unroll
+                            for (int sx = 0; sx < G::KX; ++sx)
+#pragma unroll
+                                for (int sy = 0; sy < G::KY; ++sy)
+                                    v[(sz * G::KX + sx) * G::KY + sy] = p0[c * G::CH_STRIDE + (sz * G::RX + sx) * G::WY + sy];
+#pragma unroll
+                        for (int co = 0; co < COB; ++co) {
+                            if (co0 + co >= a.Cout) break;
+                            const T* __restrict__ wp = wl + ((int64_t)(co0 + co) * a.Cin + ci) * G::K;
+                            T res = 0;
+#pragma unroll
+                            for (int t = 0; t < G::K; ++t) res += v[t] * wp[t];
+                            acc[it][co] += res;
+                        }
+                    }
+                }
+                __syncthreads();
+            }
+#pragma unroll
+            for (int it = 0; it < G::ITER; ++it) {
+                const int col = threadIdx.x + it * G::NT;
+                if (col >= nc) continue;
+                const int64_t o = sh.col_idx[col];
+#pragma unroll
+                for (int co = 0; co < COB; ++co)
+                    if (co0 + co < a.Cout) a.y[(int64_t)(co0 + co) * a.ldy + o] = acc[it][co];
+            }
+        }
+        __syncthreads();
+        advance_cursors<G, T>(y0, sh, yv);
+        __syncthreads();
+    }
+}
+
+template <typename T, class G, int CIB, int COB>
+static int launch_fwd(const ConvArgs<T>& a, int n_tiles, hipStream_t st) {
+    dim3 grid((unsigned)n_tiles, (unsigned)((a.Cout + COB - 1) / COB));
+    hipLaunchKernelGGL((conv_fwd_kernel<T, G, CIB, COB>), grid, dim3(G::NT), 0, st, a);
+    APRNET_LAUNCH_CHECK("conv_fwd_kernel");
+    return 0;
+}
+
+// tile shapes: 3-D stencils 2 x 4 rows, 2-D stencils (kz == 1) 1 x 8 rows
+using G333 = ConvGeom<3, 3, 3, 2, 4, 256>;
+using G133 = ConvGeom<1, 3, 3, 1, 8, 256>;
+using G155 = ConvGeom<1, 5, 5, 1, 8, 256>;
+using G555 = ConvGeom<5, 5, 5, 2, 4, 256>;
+
+template <typename T> struct Chunk;       // channels staged per pass so that the patch stays near 48 KB
+template <> struct Chunk<float>  { static constexpr int c333 = 8, c133 = 16, c155 = 12, c555 = 4; };
+template <> struct Chunk<double> { static constexpr int c333 = 4, c133 = 8,  c155 = 6,  c555 = 2; };
+
+int fill_tree_for_conv(const aprnet_plan* p, int d, const float* x, int64_t ldx, int C, float* tree, int64_t ldt, hipStream_t st);
+int fill_tree_for_conv(const aprnet_plan* p, int d, const double* x, int64_t ldx, int C, double* tree, int64_t ldt, hipStream_t st);
+
+template <typename T>
+int conv_fwd(const aprnet_plan* cp, int d, int kz, int kx, int ky, const T* x, int64_t ldx, int Cin, const T* w,
+             int S_exp, int Cout, T* y, int64_t ldy, T* tree_ws, int64_t ldt, hipStream_t st) {
+    aprnet_plan* p = const_cast<aprnet_plan*>(cp);
+    if (int rc = check_level_delta(p, d, "conv_forward")) return rc;
+    if (Cin <= 0 || Cout <= 0 || S_exp <= 0) return fail(APRNET_ERR_INVALID_ARGUMENT, "conv_forward: empty channel / stencil count");
+    const int code = kz * 100 + kx * 10 + ky;
+    if (code != 333 && code != 133 && code != 155 && code != 555)
+        return fail(APRNET_ERR_UNSUPPORTED, "conv_forward: stencil must be 333, 133, 155 or 555");
+    const int64_t nt = p->tree_parts(d);
+    if (nt > 0 && (!tree_ws || ldt < nt)) return fail(APRNET_ERR_INVALID_ARGUMENT, "conv_forward: tree work space too small");
+    APRNET_HIP_CHECK(hipSetDevice(p->device));
+    if (int rc = fill_tree_for_conv(p, d, x, ldx, Cin, tree_ws, ldt, st)) return rc;
+    const bool flat = (kz == 1);
+    TileList tl;
+    if (int rc = get_tiles(p, d, flat ? 1 : 2, flat ? 8 : 4, &tl)) return rc;
+    if (tl.n == 0) return 0;
+    ConvArgs<T> a{};
+    a.apr = p->dapr; a.tree = p->dtree; a.tiles = tl.d_tiles;
+    a.x = x; a.ldx = ldx; a.Cin = Cin; a.w = w; a.S_exp = S_exp; a.Cout = Cout; a.y = y; a.ldy = ldy;
+    a.tree_data = tree_ws; a.ldt = ldt; a.Lc = p->lc(d); a.tree_off = p->tree_offset(a.Lc);
+    // few output channels per thread keep the wave-uniform weights within the scalar register file;
+    // wider layers run more blocks along grid.y (each re-stages its patch)
+    switch (code) {
+        case 333: return launch_fwd<T, G333, Chunk<T>::c333, 4>(a, tl.n, st);
+        case 133: return launch_fwd<T, G133, Chunk<T>::c133, 4>(a, tl.n, st);
+        case 155: return launch_fwd<T, G155, Chunk<T>::c155, 4>(a, tl.n, st);
+        case 555: return launch_fwd<T, G555, Chunk<T>::c555, 4>(a, tl.n, st);
+    }
+    return 0;
+}
+
+}  // namespace aprnet
+
+using namespace aprnet;
+
+extern "C" {
+int aprnet_conv_fwd_f32(const aprnet_plan* p, int d, int kz, int kx, int ky, const float* x, int64_t ldx, int Cin,
+                        const float* w, int S_exp, int Cout, float* y, int64_t ldy, float* tree_ws, int64_t ldt, void* st) {
+    return conv_fwd<float>(p, d, kz, kx, ky, x, ldx, Cin, w, S_exp, Cout, y, ldy, tree_ws, ldt, (hipStream_t)st);
+}
+int aprnet_conv_fwd_f64(const aprnet_plan* p, int d, int kz, int kx, int ky, const double* x, int64_t ldx, int Cin,
+                        const double* w, int S_exp, int Cout, double* y, int64_t ldy, double* tree_ws, int64_t ldt, void* st) {
+    return conv_fwd<double>(p, d, kz, kx, ky, x, ldx, Cin, w, S_exp, Cout, y, ldy, tree_ws, ldt, (hipStream_t)st);
+}
+}

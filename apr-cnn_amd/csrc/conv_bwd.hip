@@ -1,0 +1,305 @@
+// Stencil convolution, backward: Convolution<kz,kx,ky>::backward (conv.hpp:261-481 with
+// helpers.hpp:423-478, 578-704).  Two kernels over the same tiles / windows as the forward pass.
+//
+// grad_input.  Per window and chunk of input channels every thread owns one output position and
+// forms its K tap gradients  g[c][t] = sum_co dO[co] * w[co][c][t]  (weights wave-uniform), adds
+// them into an LDS gradient patch (LDS atomics: neighbouring outputs overlap), and the patch is then
+// flushed along the three gather sources - the exact transpose of the forward gather, including the
+// two cells of a coarser particle.  Halo rows belong to neighbouring tiles as well, so the flush uses
+// global floating-point atomics; tree cells of levels < Lc go to the tree-gradient buffer that
+// fill_tree_mean_backward afterwards pushes down to the particles.
+//
+// grad_weights.  dW[s][co][ci][t] = sum over outputs of dO[co] * tap[ci][t].  A thread owns one
+// (co, ci) pair and keeps its K sums in registers while the (persistent) block walks over many
+// tiles; dO and the patch are staged in LDS.  Sums are flushed with one atomic per element when the
+// stencil index changes and at the end.
+#include "conv_common.hpp"
+
+namespace aprnet {
+
+template <typename T>
+__global__ void fill_kernel(T* __restrict__ p, int64_t ld, int64_t n, T v) {
+    T* row = p + (int64_t)blockIdx.y * ld;
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x) row[i] = v;
+}
+
+template <typename T>
+static void fill2d(T* p, int64_t ld, int64_t n, int rows, T v, hipStream_t st) {
+    if (n <= 0 || rows <= 0) return;
+    dim3 grid((unsigned)std::min<int64_t>((n + 255) / 256, 4096), (unsigned)rows);
+    hipLaunchKernelGGL(fill_kernel<T>, grid, dim3(256), 0, st, p, ld, n, v);
+}
+
+// Transpose of stage_values: add the gradient patch back to its sources.
+template <class G, typename T, int CIB>
+__device__ __forceinline__ void flush_values(const ConvArgs<T>& a, int L, int y0, int ci0, const ConvShared<G>& sh,
+                                             const int (&yv)[G::SPW], unsigned long long inw, const T* gpatch) {
+    const int wave = threadIdx.x >> 6, lane = lane_id();
+    const int lo = y0 - G::HY, hi = y0 + G::TY + G::HY;
+    const int yn = a.apr.y_num[L];
+    const bool tree_in_x = (L == a.Lc);
+#pragma unroll
+    for (int k = 0; k < G::SPW; ++k) {
+        if (!((inw >> k) & 1ull)) continue;
+        const int s = wave + k * G::NWAVE;
+        const int r = s / 3, src = s - 3 * r;
+        const int64_t i = sh.seg_cur[s] + lane;
+        const int yy = yv[k];
+        T* base;
+        int64_t ld;
+        if (src == 2 && !tree_in_x) { base = a.gtree + i; ld = a.ldgt; }
+        else { base = a.gx + i + (src == 2 ? a.tree_off : 0); ld = a.ldgx; }
+        const T* prow = gpatch + r * G::WY;
+#pragma unroll
+        for (int c = 0; c < CIB; ++c) {
+            if (ci0 + c >= a.Cin) break;
+            T v;
+            if (src != 1) {
+                v = prow[c * G::CH_STRIDE + (yy - lo)];
+            } else {
+                const int ya = 2 * yy, yb = ya + 1;
+                v = 0;
+                if (ya >= lo && ya < hi) v += prow[c * G::CH_STRIDE + (ya - lo)];
+                if (yb >= lo && yb < hi && yb < yn) v += prow[c * G::CH_STRIDE + (yb - lo)];
+            }
+            if (v != (T)0) atomicAdd(base + (int64_t)(ci0 + c) * ld, v);
+        }
+    }
+}
+
+template <typename T, class G, int CIB, int COBLK>
+__global__ void __launch_bounds__(G::NT)
+conv_bwd_dx_kernel(const ConvArgs<T> a) {
+    static_assert(G::ITER == 1, "one output position per thread");
+    __shared__ T gpatch[CIB * G::CH_STRIDE];
+    __shared__ T dOs[COBLK * G::MAXCOL];
+    __shared__ ConvShared<G> sh;
+
+    const ConvTile tile = a.tiles[blockIdx.x];
+    const int L = tile.level, z0 = tile.z0, x0 = tile.x0;
+    const int ci0 = blockIdx.y * CIB;
+    const int yn = a.apr.y_num[L];
+    const int s_idx = min(a.S_exp - 1, a.Lc - L);
+    const bool out_tree = (L == a.Lc) && (L < a.apr.level_max);
+    const T* __restrict__ wl = a.w + (int64_t)s_idx * a.Cout * a.Cin * G::K;
+
+    open_segments<G, T>(a, L, z0, x0, sh);
+    __syncthreads();
+
+    int yv[G::SPW];
+    unsigned long long inw;
+    for (int y0 = 0; y0 < yn; y0 += G::TY) {
+        scan_window<G, T>(a, L, y0, out_tree, sh, yv, inw);
+        __syncthreads();
+        const int nc = sh.ncol;
+        if (nc > 0) {
+            for (int i = threadIdx.x; i < CIB * G::CH_STRIDE; i += G::NT) gpatch[i] = 0;
+            T g[CIB][G::K];
+#pragma unroll
+            for (int c = 0; c < CIB; ++c)
+#pragma unroll
+                for (int t = 0; t < G::K; ++t) g[c][t] = 0;
+            const int col = threadIdx.x;
+            for (int co0 = 0; co0 < a.Cout; co0 += COBLK) {
+                __syncthreads();
+                const int nco = min(COBLK, a.Cout - co0);
+                for (int i = threadIdx.x; i < nco * nc; i += G::NT) {
+                    const int co = i / nc, cc = i - co * nc;
+                    dOs[co * G::MAXCOL + cc] = a.gy[(int64_t)(co0 + co) * a.ldy + sh.col_idx[cc]];
+                }
+                __syncthreads();
+                if (col < nc) {
+#pragma unroll 1
+                    for (int co = 0; co < nco; ++co) {
+                        const T dO = dOs[co * G::MAXCOL + col];
+#pragma unroll
+                        for (int c = 0; c < CIB; ++c) {
+                            if (ci0 + c >= a.Cin) break;
+                            const T* __restrict__ wp = wl + ((int64_t)(co0 + co) * a.Cin + ci0 + c) * G::K;
+#pragma unroll
+                            for (int t = 0; t < G::K; ++t) g[c][t] += dO * wp[t];
+                        }
+                    }
+                }
+            }
+            if (col < nc) {
+                T* p0 = gpatch + (int)sh.col_pos[col] - G::TAP0;
+#pragma unroll
+                for (int c = 0; c < CIB; ++c)
+#pragma unroll
+                    for (int sz = 0; sz < G::KZ; ++sz)
+#pragma unroll
+                        for (int sx = 0; sx < G::KX; ++sx)
+#pragma unroll
+                            for (int sy = 0; sy < G::KY; ++sy)
+                                atomicAdd(&p0[c * G::CH_STRIDE + (sz * G::RX + sx) * G::WY + sy],
+                                          g[c][(sz * G::KX + sx) * G::KY + sy]);
+            }
+            __syncthreads();
+            flush_values<G, T, CIB>(a, L, y0, ci0, sh, yv, inw, gpatch);
+        }
+        __syncthreads();
+        advance_cursors<G, T>(y0, sh, yv);
+        __syncthreads();
+    }
+}
+
+template <typename T, class G, int CIB, int COB>
+__global__ void __launch_bounds__(G::NT)
+conv_bwd_dw_kernel(const ConvArgs<T> a) {
+    static_assert(CIB * COB <= G::NT, "one thread per (co, ci) pair");
+    static_assert(G::SPW <= 64, "in-window mask holds one bit per segment of a wave");
+    constexpr int DOS_LD = COB + 1;
+    __shared__ T patch[CIB * G::CH_STRIDE];
+    __shared__ T dOs[G::MAXCOL * DOS_LD];
+    __shared__ ConvShared<G> sh;
+
+    const int ci0 = blockIdx.y * CIB, co0 = blockIdx.z * COB;
+    const int pco = threadIdx.x % COB, pc = threadIdx.x / COB;
+    const bool worker = threadIdx.x < CIB * COB && (co0 + pco) < a.Cout && (ci0 + pc) < a.Cin;
+    T acc[G::K];
+#pragma unroll
+    for (int t = 0; t < G::K; ++t) acc[t] = 0;
+    int cur_s = -1;
+
+    auto flush = [&](int s_idx) {
+        if (!worker || s_idx < 0) return;
+        T* dst = a.gw + (((int64_t)s_idx * a.Cout + co0 + pco) * a.Cin + ci0 + pc) * G::K;
+#pragma unroll
+        for (int t = 0; t < G::K; ++t) { if (acc[t] != (T)0) atomicAdd(dst + t, acc[t]); acc[t] = 0; }
+    };
+
+    for (int ti = blockIdx.x; ti < a.n_tiles; ti += gridDim.x) {
+        const ConvTile tile = a.tiles[ti];
+        const int L = tile.level, z0 = tile.z0, x0 = tile.x0;
+        const int yn = a.apr.y_num[L];
+        const int s_idx = min(a.S_exp - 1, a.Lc - L);
+        const bool out_tree = (L == a.Lc) && (L < a.apr.level_max);
+        if (s_idx != cur_s) { flush(cur_s); cur_s = s_idx; }
+
+        __syncthreads();
+        open_segments<G, T>(a, L, z0, x0, sh);
+        __syncthreads();
+
+        int yv[G::SPW];
+        unsigned long long inw;
+        for (int y0 = 0; y0 < yn; y0 += G::TY) {
+            scan_window<G, T>(a, L, y0, out_tree, sh, yv, inw);
+            __syncthreads();
+            const int nc = sh.ncol;
+            if (nc > 0) {
+                for (int i = threadIdx.x; i < CIB * G::CH_STRIDE; i += G::NT) patch[i] = 0;
+                const int nco = min(COB, a.Cout - co0);
+                for (int i = threadIdx.x; i < nco * nc; i += G::NT) {
+                    const int co = i / nc, cc = i - co * nc;
+                    dOs[cc * DOS_LD + co] = a.gy[(int64_t)(co0 + co) * a.ldy + sh.col_idx[cc]];
+                }
+                __syncthreads();
+                stage_values<G, T, CIB>(a, L, y0, ci0, sh, yv, inw, patch);
+                __syncthreads();
+                if (worker) {
+                    const T* pch = patch + pc * G::CH_STRIDE - G::TAP0;
+                    for (int col = 0; col < nc; ++col) {
+                        const T dO = dOs[col * DOS_LD + pco];
+                        const T* p0 = pch + (int)sh.col_pos[col];
+#pragma unroll
+                        for (int sz = 0; sz < G::KZ; ++sz)
+#pragma unroll
+                            for (int sx = 0; sx < G::KX; ++sx)
+#pragma unroll
+                                for (int sy = 0; sy < G::KY; ++sy)
+                                    acc[(sz * G::KX + sx) * G::KY + sy] += dO * p0[(sz * G::RX + sx) * G::WY + sy];
+                    }
+                }
+            }
+            __syncthreads();
+            advance_cursors<G, T>(y0, sh, yv);
+            __syncthreads();
+        }
+    }
+    flush(cur_s);
+}
+
+// geometries: 512 threads for grad_input (one output position per thread), 256 for grad_weights
+using X333 = ConvGeom<3, 3, 3, 2, 4, 512>;
+using X133 = ConvGeom<1, 3, 3, 1, 8, 512>;
+using X155 = ConvGeom<1, 5, 5, 1, 8, 512>;
+using X555 = ConvGeom<5, 5, 5, 2, 4, 512>;
+using W333 = ConvGeom<3, 3, 3, 2, 4, 256>;
+using W133 = ConvGeom<1, 3, 3, 1, 8, 256>;
+using W155 = ConvGeom<1, 5, 5, 1, 8, 256>;
+using W555 = ConvGeom<5, 5, 5, 2, 4, 256>;
+
+int fill_tree_for_conv(const aprnet_plan* p, int d, const float* x, int64_t ldx, int C, float* tree, int64_t ldt, hipStream_t st);
+int fill_tree_for_conv(const aprnet_plan* p, int d, const double* x, int64_t ldx, int C, double* tree, int64_t ldt, hipStream_t st);
+int fill_tree_bwd_for_conv(const aprnet_plan* p, int d, float* gx, int64_t ldx, int C, float* gt, int64_t ldt, hipStream_t st);
+int fill_tree_bwd_for_conv(const aprnet_plan* p, int d, double* gx, int64_t ldx, int C, double* gt, int64_t ldt, hipStream_t st);
+
+template <typename T, class GX, int XCIB, class GW, int WCIB, int WCOB>
+static int launch_bwd(ConvArgs<T>& a, hipStream_t st) {
+    constexpr int COBLK = 8;
+    dim3 gx((unsigned)a.n_tiles, (unsigned)((a.Cin + XCIB - 1) / XCIB));
+    hipLaunchKernelGGL((conv_bwd_dx_kernel<T, GX, XCIB, COBLK>), gx, dim3(GX::NT), 0, st, a);
+    APRNET_LAUNCH_CHECK("conv_bwd_dx_kernel");
+    dim3 gw((unsigned)std::min(a.n_tiles, 512), (unsigned)((a.Cin + WCIB - 1) / WCIB), (unsigned)((a.Cout + WCOB - 1) / WCOB));
+    hipLaunchKernelGGL((conv_bwd_dw_kernel<T, GW, WCIB, WCOB>), gw, dim3(GW::NT), 0, st, a);
+    APRNET_LAUNCH_CHECK("conv_bwd_dw_kernel");
+    return 0;
+}
+
+template <typename T>
+int conv_bwd(const aprnet_plan* cp, int d, int kz, int kx, int ky, const T* x, int64_t ldx, int Cin, const T* w, int S_exp,
+             int Cout, const T* gy, int64_t ldy, T* gx, int64_t ldgx, T* gw, T* tree_ws, int64_t ldt, T* gtree_ws,
+             int64_t ldgt, hipStream_t st) {
+    aprnet_plan* p = const_cast<aprnet_plan*>(cp);
+    if (int rc = check_level_delta(p, d, "conv_backward")) return rc;
+    if (Cin <= 0 || Cout <= 0 || S_exp <= 0) return fail(APRNET_ERR_INVALID_ARGUMENT, "conv_backward: empty channel / stencil count");
+    const int code = kz * 100 + kx * 10 + ky;
+    if (code != 333 && code != 133 && code != 155 && code != 555)
+        return fail(APRNET_ERR_UNSUPPORTED, "conv_backward: stencil must be 333, 133, 155 or 555");
+    const int64_t nt = p->tree_parts(d);
+    if (nt > 0 && (!tree_ws || !gtree_ws || ldt < nt || ldgt < nt))
+        return fail(APRNET_ERR_INVALID_ARGUMENT, "conv_backward: tree work space too small");
+    APRNET_HIP_CHECK(hipSetDevice(p->device));
+    if (int rc = fill_tree_for_conv(p, d, x, ldx, Cin, tree_ws, ldt, st)) return rc;
+    fill2d<T>(gx, ldgx, p->number_parts(d), Cin, (T)0, st);
+    fill2d<T>(gtree_ws, ldgt, nt, Cin, (T)0, st);
+    const bool flat = (kz == 1);
+    TileList tl;
+    if (int rc = get_tiles(p, d, flat ? 1 : 2, flat ? 8 : 4, &tl)) return rc;
+    if (tl.n > 0) {
+        ConvArgs<T> a{};
+        a.apr = p->dapr; a.tree = p->dtree; a.tiles = tl.d_tiles; a.n_tiles = tl.n;
+        a.x = x; a.ldx = ldx; a.Cin = Cin; a.w = w; a.S_exp = S_exp; a.Cout = Cout;
+        a.tree_data = tree_ws; a.ldt = ldt; a.Lc = p->lc(d); a.tree_off = p->tree_offset(a.Lc);
+        a.gy = gy; a.ldy = ldy; a.gx = gx; a.ldgx = ldgx; a.gtree = gtree_ws; a.ldgt = ldgt; a.gw = gw;
+        constexpr bool f32 = sizeof(T) == 4;
+        int rc = 0;
+        switch (code) {
+            case 333: rc = launch_bwd<T, X333, (f32 ? 4 : 2), W333, (f32 ? 8 : 4), (f32 ? 32 : 16)>(a, st); break;
+            case 133: rc = launch_bwd<T, X133, (f32 ? 8 : 4), W133, (f32 ? 8 : 4), (f32 ? 32 : 16)>(a, st); break;
+            case 155: rc = launch_bwd<T, X155, (f32 ? 4 : 2), W155, (f32 ? 8 : 4), (f32 ? 32 : 16)>(a, st); break;
+            case 555: rc = launch_bwd<T, X555, 1, W555, (f32 ? 4 : 2), (f32 ? 32 : 16)>(a, st); break;
+        }
+        if (rc) return rc;
+    }
+    return fill_tree_bwd_for_conv(p, d, gx, ldgx, Cin, gtree_ws, ldgt, st);
+}
+
+}  // namespace aprnet
+
+using namespace aprnet;
+extern "C" {
+int aprnet_conv_bwd_f32(const aprnet_plan* p, int d, int kz, int kx, int ky, const float* x, int64_t ldx, int Cin,
+                        const float* w, int S_exp, int Cout, const float* gy, int64_t ldy, float* gx, int64_t ldgx,
+                        float* gw, float* tree_ws, int64_t ldt, float* gtree_ws, int64_t ldgt, void* st) {
+    return conv_bwd<float>(p, d, kz, kx, ky, x, ldx, Cin, w, S_exp, Cout, gy, ldy, gx, ldgx, gw, tree_ws, ldt, gtree_ws,
+                           ldgt, (hipStream_t)st);
+}
+int aprnet_conv_bwd_f64(const aprnet_plan* p, int d, int kz, int kx, int ky, const double* x, int64_t ldx, int Cin,
+                        const double* w, int S_exp, int Cout, const double* gy, int64_t ldy, double* gx, int64_t ldgx,
+                        double* gw, double* tree_ws, int64_t ldt, double* gtree_ws, int64_t ldgt, void* st) {
+    return conv_bwd<double>(p, d, kz, kx, ky, x, ldx, Cin, w, S_exp, Cout, gy, ldy, gx, ldgx, gw, tree_ws, ldt, gtree_ws,
+                            ldgt, (hipStream_t)st);
+}
+}

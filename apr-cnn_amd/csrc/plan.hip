@@ -1,0 +1,204 @@
+// Plan = device image of one APR: access arrays, child table, convolution tile lists.
+// Host side of the C ABI for plan management (include/aprnet_hip.h).
+#include "common.hpp"
+
+#include <algorithm>
+#include <cstring>
+#include <thread>
+
+namespace aprnet {
+
+static thread_local std::string g_last_error;
+
+void set_error(const std::string& msg) { g_last_error = msg; }
+int fail(int code, const std::string& msg) { g_last_error = msg; return code; }
+
+static int copy_access(const aprnet_access_desc* d, HostAccess& h, int lmax_all) {
+    if (!d || !d->z_num || !d->x_num || !d->y_num || !d->level_xz_vec || !d->xz_end_vec)
+        return fail(APRNET_ERR_INVALID_ARGUMENT, "plan_create: null access array");
+    if (d->level_max + 1 > MAX_LEVELS || d->level_min < 0 || d->level_min > d->level_max)
+        return fail(APRNET_ERR_INVALID_ARGUMENT, "plan_create: level range out of bounds");
+    h.level_min = d->level_min; h.level_max = d->level_max; h.n = d->n_particles;
+    h.z_num.assign(d->z_num, d->z_num + lmax_all + 1);
+    h.x_num.assign(d->x_num, d->x_num + lmax_all + 1);
+    h.y_num.assign(d->y_num, d->y_num + lmax_all + 1);
+    h.level_xz.assign(d->level_xz_vec, d->level_xz_vec + d->level_max + 2);
+    if (h.level_xz[d->level_max + 1] != d->n_rows)
+        return fail(APRNET_ERR_INVALID_ARGUMENT, "plan_create: xz_end_vec length does not match level_xz_vec");
+    h.xz_end.assign(d->xz_end_vec, d->xz_end_vec + d->n_rows);
+    if (h.xz_end.empty() || h.xz_end[0] != 0 || h.xz_end.back() != d->n_particles)
+        return fail(APRNET_ERR_INVALID_ARGUMENT, "plan_create: xz_end_vec must start at 0 and end at n_particles");
+    if (d->n_particles >= (uint64_t)INT32_MAX)
+        return fail(APRNET_ERR_UNSUPPORTED, "plan_create: more than 2^31-1 particles per access");
+    if (d->n_particles) h.y.assign(d->y_vec, d->y_vec + d->n_particles);
+    return 0;
+}
+
+static void fill_dev(const HostAccess& h, AccessDev& d, const void* xz, const void* y, int lmax_all) {
+    std::memset(&d, 0, sizeof(d));
+    d.xz_end = (const uint64_t*)xz; d.y = (const uint16_t*)y;
+    d.level_min = h.level_min; d.level_max = h.level_max;
+    for (int l = 0; l <= lmax_all; ++l) { d.z_num[l] = h.z_num[l]; d.x_num[l] = h.x_num[l]; d.y_num[l] = h.y_num[l]; }
+    for (int l = 0; l <= h.level_max + 1; ++l) d.level_xz[l] = h.level_xz[l];
+    for (int l = h.level_max + 2; l <= MAX_LEVELS; ++l) d.level_xz[l] = h.level_xz[h.level_max + 1];
+}
+
+template <class F>
+static void parallel_for(int n, F f) {
+    const int nt = std::max(1u, std::min(16u, std::thread::hardware_concurrency()));
+    if (n < 64 || nt == 1) { for (int i = 0; i < n; ++i) f(i); return; }
+    std::vector<std::thread> th;
+    for (int t = 0; t < nt; ++t)
+        th.emplace_back([=]() { for (int i = t; i < n; i += nt) f(i); });
+    for (auto& t : th) t.join();
+}
+
+// children[s][t], s = 4*dz + 2*dx + dy: the merge walk of helpers.hpp:185-194 done once, from the
+// parents' side, for particles and for tree nodes.
+static void build_children(const HostAccess& apr, const HostAccess& tree, std::vector<int32_t>& ch) {
+    const int64_t T = (int64_t)tree.n;
+    ch.assign((size_t)8 * T, NO_CHILD);
+    for (int l = tree.level_min; l <= tree.level_max; ++l) {
+        const int cl = l + 1;
+        const int zn = tree.z_num[l], xn = tree.x_num[l];
+        const int czn = tree.z_num[cl], cxn = tree.x_num[cl];
+        const bool apr_has = cl >= apr.level_min && cl <= apr.level_max;
+        const bool tree_has = cl <= tree.level_max;
+        parallel_for(zn, [&](int z) {
+            for (int x = 0; x < xn; ++x) {
+                const uint64_t prow = tree.row(l, z, x);
+                const int64_t pb = (int64_t)tree.xz_end[prow - 1], pe = (int64_t)tree.xz_end[prow];
+                if (pb == pe) continue;
+                for (int dz = 0; dz < 2; ++dz) {
+                    const int cz = 2 * z + dz; if (cz >= czn) continue;
+                    for (int dx = 0; dx < 2; ++dx) {
+                        const int cx = 2 * x + dx; if (cx >= cxn) continue;
+                        const int s0 = 4 * dz + 2 * dx;
+                        if (apr_has) {
+                            const uint64_t r = apr.row(cl, cz, cx);
+                            int64_t p = pb;
+                            for (int64_t c = (int64_t)apr.xz_end[r - 1]; c < (int64_t)apr.xz_end[r]; ++c) {
+                                const int yp = apr.y[c] >> 1;
+                                while (p < pe && tree.y[p] < yp) ++p;
+                                if (p < pe && tree.y[p] == yp) ch[(size_t)(s0 + (apr.y[c] & 1)) * T + p] = (int32_t)c;
+                            }
+                        }
+                        if (tree_has) {
+                            const uint64_t r = tree.row(cl, cz, cx);
+                            int64_t p = pb;
+                            for (int64_t c = (int64_t)tree.xz_end[r - 1]; c < (int64_t)tree.xz_end[r]; ++c) {
+                                const int yp = tree.y[c] >> 1;
+                                while (p < pe && tree.y[p] < yp) ++p;
+                                if (p < pe && tree.y[p] == yp) ch[(size_t)(s0 + (tree.y[c] & 1)) * T + p] = ~(int32_t)c;
+                            }
+                        }
+                    }
+                }
+            }
+        });
+    }
+}
+
+int get_tiles(aprnet_plan* plan, int level_delta, int TZ, int TX, TileList* out) {
+    auto key = std::make_tuple(level_delta, TZ, TX);
+    auto it = plan->tiles.find(key);
+    if (it != plan->tiles.end()) { *out = it->second; return 0; }
+    const HostAccess& apr = plan->apr; const HostAccess& tree = plan->tree;
+    const int Lc = plan->lc(level_delta);
+    std::vector<ConvTile> tiles;
+    // finest level first: it holds most of the work, the coarse levels fill the tail of the launch
+    for (int l = Lc; l >= apr.level_min; --l) {
+        const bool with_tree = (l == Lc && l < apr.level_max);
+        const int zn = apr.z_num[l], xn = apr.x_num[l];
+        for (int z0 = 0; z0 < zn; z0 += TZ)
+            for (int x0 = 0; x0 < xn; x0 += TX) {
+                bool any = false;
+                for (int z = z0; z < std::min(z0 + TZ, zn) && !any; ++z) {
+                    const int x1 = std::min(x0 + TX, xn) - 1;
+                    // rows x0..x1 of one z are adjacent in the row table: one range test
+                    const uint64_t ra = apr.row(l, z, x0), rb = apr.row(l, z, x1);
+                    any = apr.xz_end[rb] > apr.xz_end[ra - 1];
+                    if (!any && with_tree) {
+                        const uint64_t ta = tree.row(l, z, x0), tb = tree.row(l, z, x1);
+                        any = tree.xz_end[tb] > tree.xz_end[ta - 1];
+                    }
+                }
+                if (any) tiles.push_back(ConvTile{l, z0, x0, 0});
+            }
+    }
+    TileList tl;
+    tl.n = (int)tiles.size();
+    if (tl.n) {
+        APRNET_HIP_CHECK(hipMalloc((void**)&tl.d_tiles, tiles.size() * sizeof(ConvTile)));
+        APRNET_HIP_CHECK(hipMemcpy(tl.d_tiles, tiles.data(), tiles.size() * sizeof(ConvTile), hipMemcpyHostToDevice));
+    }
+    plan->tiles[key] = tl;
+    *out = tl;
+    return 0;
+}
+
+}  // namespace aprnet
+
+using namespace aprnet;
+
+extern "C" {
+
+const char* aprnet_last_error(void) { return g_last_error.c_str(); }
+
+int aprnet_plan_create(const aprnet_access_desc* apr, const aprnet_access_desc* tree, int device, aprnet_plan** out) {
+    if (!out) return fail(APRNET_ERR_INVALID_ARGUMENT, "plan_create: null output");
+    *out = nullptr;
+    if (!apr || !tree) return fail(APRNET_ERR_INVALID_ARGUMENT, "plan_create: null access descriptor");
+    if (tree->level_max != apr->level_max - 1 || tree->level_min > apr->level_min - 1)
+        return fail(APRNET_ERR_INVALID_ARGUMENT, "plan_create: the tree must span levels <= level_min-1 .. level_max-1");
+    aprnet_plan* p = new aprnet_plan();
+    p->device = device;
+    const int lmax_all = apr->level_max;
+    int rc = copy_access(apr, p->apr, lmax_all);
+    if (!rc) rc = copy_access(tree, p->tree, lmax_all);
+    if (rc) { delete p; return rc; }
+    p->n_apr = (int64_t)p->apr.n; p->n_tree = (int64_t)p->tree.n;
+    // per row y must ascend strictly: the staging code relies on it
+    std::vector<int32_t> children;
+    build_children(p->apr, p->tree, children);
+
+    APRNET_HIP_CHECK(hipSetDevice(device));
+    auto upload = [&](void** dst, const void* src, size_t bytes) -> int {
+        APRNET_HIP_CHECK(hipMalloc(dst, std::max<size_t>(bytes, 16)));
+        if (bytes) APRNET_HIP_CHECK(hipMemcpy(*dst, src, bytes, hipMemcpyHostToDevice));
+        return 0;
+    };
+    rc = upload(&p->d_apr_xz, p->apr.xz_end.data(), p->apr.xz_end.size() * 8);
+    if (!rc) rc = upload(&p->d_apr_y, p->apr.y.data(), p->apr.y.size() * 2);
+    if (!rc) rc = upload(&p->d_tree_xz, p->tree.xz_end.data(), p->tree.xz_end.size() * 8);
+    if (!rc) rc = upload(&p->d_tree_y, p->tree.y.data(), p->tree.y.size() * 2);
+    if (!rc) rc = upload((void**)&p->d_children, children.data(), children.size() * 4);
+    if (rc) { aprnet_plan_destroy(p); return rc; }
+    fill_dev(p->apr, p->dapr, p->d_apr_xz, p->d_apr_y, lmax_all);
+    fill_dev(p->tree, p->dtree, p->d_tree_xz, p->d_tree_y, lmax_all);
+    // the host keeps only the row tables (for level ranges and tile lists), not y
+    *out = p;
+    return 0;
+}
+
+void aprnet_plan_destroy(aprnet_plan* p) {
+    if (!p) return;
+    (void)hipSetDevice(p->device);
+    for (void* q : {p->d_apr_xz, p->d_apr_y, p->d_tree_xz, p->d_tree_y, (void*)p->d_children})
+        if (q) (void)hipFree(q);
+    for (auto& kv : p->tiles) if (kv.second.d_tiles) (void)hipFree(kv.second.d_tiles);
+    delete p;
+}
+
+int64_t aprnet_number_parts(const aprnet_plan* p, int level_delta) { return p ? p->number_parts(level_delta) : -1; }
+int64_t aprnet_tree_offset(const aprnet_plan* p, int level) { return p ? p->tree_offset(level) : 0; }
+int64_t aprnet_tree_parts(const aprnet_plan* p, int level_delta) { return p ? p->tree_parts(level_delta) : -1; }
+
+int aprnet_plan_children(const aprnet_plan* p, int32_t* out_host) {
+    if (!p || !out_host) return fail(APRNET_ERR_INVALID_ARGUMENT, "plan_children: null argument");
+    APRNET_HIP_CHECK(hipSetDevice(p->device));
+    if (p->n_tree) APRNET_HIP_CHECK(hipMemcpy(out_host, p->d_children, (size_t)8 * p->n_tree * 4, hipMemcpyDeviceToHost));
+    return 0;
+}
+
+}  // extern "C"

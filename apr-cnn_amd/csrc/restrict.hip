@@ -1,0 +1,111 @@
+// RestrictKernel<kz,kx,ky>::forward/backward (kernel.hpp:31-224): stencils of levels >= S are the
+// last given stencil restricted by area overlap with step 2^(level-S+1) and divided by step^ndim
+// (ndim counts the non-singleton dimensions only, kernel.hpp:59).  Tiny: one thread per filter
+// element, gather form in both directions, so the result is deterministic.
+#include "common.hpp"
+
+namespace aprnet {
+
+__device__ __forceinline__ float overlap1(int o, int i, int k, int step) {
+    const int off = (k / 2) * step - k / 2;
+    const int v = min((o + 1) * step, off + i + step) - max(o * step, off + i);
+    return (float)max(v, 0);
+}
+
+// w [S][F][K] -> we [S_exp][F][K]
+template <typename T>
+__global__ void restrict_fwd_kernel(const T* __restrict__ w, T* __restrict__ we, int S, int S_exp, int F,
+                                    int kz, int kx, int ky, int ndim) {
+    const int K = kz * kx * ky;
+    const int64_t n = (int64_t)S_exp * F * K;
+    const int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (e >= n) return;
+    const int tap = (int)(e % K);
+    const int f = (int)((e / K) % F);
+    const int l = (int)(e / ((int64_t)K * F));
+    if (l < S) { we[e] = w[e]; return; }
+    const int step = 1 << (l - (S - 1));
+    const float factor = powf((float)step, (float)ndim);
+    const int zo = tap / (kx * ky), xo = (tap / ky) % kx, yo = tap % ky;
+    const T* src = w + ((int64_t)(S - 1) * F + f) * K;
+    T acc = 0;
+    // same tap order as the reference: z_in, x_in, y_in ascending
+    for (int zi = 0; zi < kz; ++zi) {
+        const float oz = overlap1(zo, zi, kz, step);
+        if (oz <= 0) continue;
+        for (int xi = 0; xi < kx; ++xi) {
+            const float ox = overlap1(xo, xi, kx, step);
+            if (ox <= 0) continue;
+            for (int yi = 0; yi < ky; ++yi) {
+                const float oy = overlap1(yo, yi, ky, step);
+                if (oy <= 0) continue;
+                const float ov = ox * oy * oz / factor;
+                acc += (T)ov * src[(zi * kx + xi) * ky + yi];
+            }
+        }
+    }
+    we[e] = acc;
+}
+
+// gwe [S_exp][F][K] -> gw [S][F][K]
+template <typename T>
+__global__ void restrict_bwd_kernel(const T* __restrict__ gwe, T* __restrict__ gw, int S, int S_exp, int F,
+                                    int kz, int kx, int ky, int ndim) {
+    const int K = kz * kx * ky;
+    const int64_t n = (int64_t)S * F * K;
+    const int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (e >= n) return;
+    const int tap = (int)(e % K);
+    const int f = (int)((e / K) % F);
+    const int l = (int)(e / ((int64_t)K * F));
+    T acc = gwe[e];
+    if (l == S - 1) {
+        const int zi = tap / (kx * ky), xi = (tap / ky) % kx, yi = tap % ky;
+        for (int le = S; le < S_exp; ++le) {
+            const int step = 1 << (le - (S - 1));
+            const float factor = powf((float)step, (float)ndim);
+            const T* src = gwe + ((int64_t)le * F + f) * K;
+            for (int zo = 0; zo < kz; ++zo) {
+                const float oz = overlap1(zo, zi, kz, step);
+                if (oz <= 0) continue;
+                for (int xo = 0; xo < kx; ++xo) {
+                    const float ox = overlap1(xo, xi, kx, step);
+                    if (ox <= 0) continue;
+                    for (int yo = 0; yo < ky; ++yo) {
+                        const float oy = overlap1(yo, yi, ky, step);
+                        if (oy <= 0) continue;
+                        const float ov = ox * oy * oz / factor;
+                        acc += (T)ov * src[(zo * kx + xo) * ky + yo];
+                    }
+                }
+            }
+        }
+    }
+    gw[e] = acc;
+}
+
+template <typename T, bool Backward>
+int restrict_kernel(const T* src, int S, int F, int kz, int kx, int ky, int S_exp, T* dst, hipStream_t st) {
+    if (S <= 0 || S_exp < S || F <= 0 || kz <= 0 || kx <= 0 || ky <= 0)
+        return fail(APRNET_ERR_INVALID_ARGUMENT, "restrict_kernel: need 0 < S <= S_exp and a non-empty filter bank");
+    const int ndim = (kz > 1) + (kx > 1) + (ky > 1);
+    const int64_t n = (int64_t)(Backward ? S : S_exp) * F * kz * kx * ky;
+    dim3 grid((unsigned)((n + 255) / 256));
+    if (!Backward) hipLaunchKernelGGL(restrict_fwd_kernel<T>, grid, dim3(256), 0, st, src, dst, S, S_exp, F, kz, kx, ky, ndim);
+    else hipLaunchKernelGGL(restrict_bwd_kernel<T>, grid, dim3(256), 0, st, src, dst, S, S_exp, F, kz, kx, ky, ndim);
+    APRNET_LAUNCH_CHECK("restrict_kernel");
+    return 0;
+}
+
+}  // namespace aprnet
+
+using namespace aprnet;
+extern "C" {
+#define RESTRICT_API(T, SFX)                                                                                           \
+    int aprnet_restrict_kernel_fwd_##SFX(const T* w, int S, int F, int kz, int kx, int ky, int S_exp, T* we, void* st) { \
+        return restrict_kernel<T, false>(w, S, F, kz, kx, ky, S_exp, we, (hipStream_t)st); }                           \
+    int aprnet_restrict_kernel_bwd_##SFX(const T* gwe, int S_exp, int F, int kz, int kx, int ky, int S, T* gw, void* st) { \
+        return restrict_kernel<T, true>(gwe, S, F, kz, kx, ky, S_exp, gw, (hipStream_t)st); }
+RESTRICT_API(float, f32)
+RESTRICT_API(double, f64)
+}

@@ -1,0 +1,383 @@
+"""Native operator calls: the functions APR-CNN binds on ``_pyaprwrapper.aprnet.{conv,pool,upsample,
+utils,cuda}`` (wrappers/pythonBind.cpp:144-182), here implemented on top of the C ABI of
+``libaprnet_hip.so``.  Same names, argument order, output allocation and exception types as the
+reference's wrappers; every tensor must live on the GPU ("cuda" device of PyTorch-ROCm) — there is no
+CPU path behind these functions.
+
+Weight layouts: the ``cuda`` flavour uses [S, Cout, Cin, kz, kx, ky] (cuda/conv.py:77) and is what the
+kernels consume; the CPU-flavour names (``convolve333_forward`` ...) take [Cin, S, Cout, kz, kx, ky]
+(conv.py:164) and are permuted on the way in and out.
+"""
+import ctypes as C
+
+import torch
+
+from .. import _native
+
+
+def _lib():
+    return _native.hip()
+
+
+def _raise(rc, what):
+    msg = _lib().aprnet_last_error().decode()
+    if rc == -1:
+        raise ValueError(msg or what)            # std::invalid_argument -> ValueError (pybind11)
+    raise RuntimeError(msg or what)              # TORCH_CHECK -> RuntimeError
+
+
+def _sfx(t):
+    if t.dtype == torch.float32:
+        return "f32"
+    if t.dtype == torch.float64:
+        return "f64"
+    raise TypeError(f"aprnet operators support float32 and float64 tensors, got {t.dtype}")
+
+
+def _check_input(t, name):
+    # CHECK_INPUT (cuda/src/common.hpp:14-16)
+    if not t.is_cuda:
+        raise RuntimeError(f"{name} must be a CUDA tensor")
+    if not t.is_contiguous():
+        raise RuntimeError(f"{name} must be contiguous")
+
+
+def _deltas(level_deltas, n):
+    d = [int(v) for v in level_deltas.tolist()]
+    if len(d) < n:
+        raise ValueError("level_deltas must hold one entry per APR")
+    return d
+
+
+def _plans(aprs, device):
+    return [a.plan(device.index if device.index is not None else torch.cuda.current_device()) for a in aprs]
+
+
+def _stream():
+    return C.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _ptr(t):
+    return C.c_void_p(t.data_ptr())
+
+
+def _zero_tails(out, sizes):
+    """Batch items shorter than the padded length keep zeros behind their last particle, as the
+    reference's zero-initialised outputs do (conv.hpp:68)."""
+    n = out.shape[-1]
+    for b, nb in enumerate(sizes):
+        if nb < n:
+            out[b, ..., nb:] = 0
+
+
+# ---------------------------------------------------------------------------------------- utils
+def number_particles(apr, level_delta):
+    """helpers::number_parts (helpers.hpp:86-101); pure host arithmetic on the row tables."""
+    it, tr = apr.iterator(), apr.tree_iterator()
+    lc = apr.level_max() - int(level_delta)
+    n = it.particles_level_end(lc)
+    if tr.level_min() <= lc <= tr.level_max():
+        n += tr.particles_level_end(lc) - tr.particles_level_begin(lc)
+    return n
+
+
+number_parts = number_particles
+
+
+def number_particles_after_pooling(apr, level_delta):
+    return number_particles(apr, int(level_delta) + 1)
+
+
+def number_particles_after_upsampling(apr, level_delta):
+    return number_particles(apr, int(level_delta) - 1)
+
+
+def tree_parts(apr, level_delta):
+    lc = apr.level_max() - int(level_delta)
+    return apr.tree_iterator().particles_level_end(lc - 1) if lc >= 1 else 0
+
+
+# ---------------------------------------------------------------------------------------- restrict kernel
+def _restrict(weights, n_other, backward):
+    _check_input(weights, "weights")
+    s_in, cout, cin, kz, kx, ky = weights.shape
+    out = torch.empty((n_other, cout, cin, kz, kx, ky), dtype=weights.dtype, device=weights.device)
+    fn = getattr(_lib(), f"aprnet_restrict_kernel_{'bwd' if backward else 'fwd'}_{_sfx(weights)}")
+    with torch.cuda.device(weights.device):
+        rc = fn(_ptr(weights), s_in, cout * cin, kz, kx, ky, n_other, _ptr(out), _stream())
+    if rc:
+        _raise(rc, "restrict_kernel failed")
+    return out
+
+
+def restrict_kernel_forward(weights, num_levels):
+    """[S, Cout, Cin, k] -> [num_levels, Cout, Cin, k] (restrict_kernel333_forward, restrict_gpu.cu:175-203)."""
+    return _restrict(weights, int(num_levels), False)
+
+
+def restrict_kernel_backward(grad_weights, num_stencils):
+    return _restrict(grad_weights, int(num_stencils), True)
+
+
+# ---------------------------------------------------------------------------------------- convolution
+def conv_forward(aprs, x, weights, level_delta):
+    """conv333_forward / conv111_forward (wrap_conv_gpu.hpp:32-66, 170-193) for any supported stencil.
+    weights: [S_exp, Cout, Cin, kz, kx, ky] (for 1x1x1: [S, Cout, Cin, 1, 1, 1], not expanded)."""
+    _check_input(x, "input")
+    _check_input(weights, "weights")
+    if x.size(1) != weights.size(2):
+        raise ValueError("convolve: input tensor shape does not match weights tensor!")   # conv.hpp:63-66
+    s_exp, cout, cin, kz, kx, ky = weights.shape
+    B, _, N = x.shape
+    d = _deltas(level_delta, len(aprs))
+    sizes = [number_particles(a, d[b]) for b, a in enumerate(aprs)]
+    if max(sizes) > N:
+        raise ValueError("input holds fewer particles than the APR at this level delta")
+    out = torch.empty((B, cout, N), dtype=x.dtype, device=x.device)
+    _zero_tails(out, sizes)
+    plans = _plans(aprs, x.device)
+    sfx = _sfx(x)
+    with torch.cuda.device(x.device):
+        st = _stream()
+        if (kz, kx, ky) == (1, 1, 1):
+            fn = getattr(_lib(), "aprnet_conv111_fwd_" + sfx)
+            for b in range(B):
+                rc = fn(plans[b], d[b], _ptr(x[b]), N, cin, _ptr(weights), s_exp, cout, _ptr(out[b]), N, st)
+                if rc:
+                    _raise(rc, "conv111_forward failed")
+        else:
+            ld_tree = max(max(tree_parts(a, d[b]) for b, a in enumerate(aprs)), 1)
+            tree_ws = torch.empty((cin, ld_tree), dtype=x.dtype, device=x.device)
+            fn = getattr(_lib(), "aprnet_conv_fwd_" + sfx)
+            for b in range(B):
+                rc = fn(plans[b], d[b], kz, kx, ky, _ptr(x[b]), N, cin, _ptr(weights), s_exp, cout, _ptr(out[b]), N,
+                        _ptr(tree_ws), ld_tree, st)
+                if rc:
+                    _raise(rc, "conv_forward failed")
+    return out
+
+
+def conv_backward(aprs, x, weights, grad_output, level_delta):
+    """conv333_backward / conv111_backward (wrap_conv_gpu.hpp:87-133, 216-246) -> [grad_input, grad_weights]."""
+    _check_input(x, "input")
+    _check_input(weights, "weights")
+    _check_input(grad_output, "grad_output")
+    s_exp, cout, cin, kz, kx, ky = weights.shape
+    B, _, N = x.shape
+    d = _deltas(level_delta, len(aprs))
+    sizes = [number_particles(a, d[b]) for b, a in enumerate(aprs)]
+    gx = torch.empty_like(x)
+    _zero_tails(gx, sizes)
+    gw = torch.zeros_like(weights)
+    plans = _plans(aprs, x.device)
+    sfx = _sfx(x)
+    with torch.cuda.device(x.device):
+        st = _stream()
+        if (kz, kx, ky) == (1, 1, 1):
+            fn = getattr(_lib(), "aprnet_conv111_bwd_" + sfx)
+            for b in range(B):
+                rc = fn(plans[b], d[b], _ptr(x[b]), N, cin, _ptr(weights), s_exp, cout, _ptr(grad_output[b]),
+                        grad_output.size(2), _ptr(gx[b]), N, _ptr(gw), st)
+                if rc:
+                    _raise(rc, "conv111_backward failed")
+        else:
+            ld_tree = max(max(tree_parts(a, d[b]) for b, a in enumerate(aprs)), 1)
+            tree_ws = torch.empty((cin, ld_tree), dtype=x.dtype, device=x.device)
+            gtree_ws = torch.empty((cin, ld_tree), dtype=x.dtype, device=x.device)
+            fn = getattr(_lib(), "aprnet_conv_bwd_" + sfx)
+            for b in range(B):
+                rc = fn(plans[b], d[b], kz, kx, ky, _ptr(x[b]), N, cin, _ptr(weights), s_exp, cout,
+                        _ptr(grad_output[b]), grad_output.size(2), _ptr(gx[b]), N, _ptr(gw),
+                        _ptr(tree_ws), ld_tree, _ptr(gtree_ws), ld_tree, st)
+                if rc:
+                    _raise(rc, "conv_backward failed")
+    return [gx, gw]
+
+
+# ---------------------------------------------------------------------------------------- pool / upsample
+def maxpool_forward(aprs, x, level_delta, pad_value=-1e17):
+    """maxpool_forward (maxpool.hpp:43-64) -> [output, max_indices].  Slots behind a batch item's last
+    particle hold ``pad_value``: -1e17 in the CPU flavour (maxpool.hpp:51), 0 in the CUDA flavour
+    (wrap_maxpool_gpu.hpp:42)."""
+    _check_input(x, "input")
+    B, Cn, N = x.shape
+    d = _deltas(level_delta, len(aprs))
+    sizes = [number_particles(a, d[b] + 1) for b, a in enumerate(aprs)]
+    n_out = max(sizes)
+    out = torch.empty((B, Cn, n_out), dtype=x.dtype, device=x.device)
+    idx = torch.empty((B, Cn, n_out), dtype=torch.int64, device=x.device)
+    for b, nb in enumerate(sizes):
+        if nb < n_out:
+            out[b, :, nb:] = pad_value
+            idx[b, :, nb:] = 0
+    plans = _plans(aprs, x.device)
+    fn = getattr(_lib(), "aprnet_maxpool_fwd_" + _sfx(x))
+    with torch.cuda.device(x.device):
+        st = _stream()
+        for b in range(B):
+            rc = fn(plans[b], d[b], _ptr(x[b]), N, Cn, _ptr(out[b]), n_out, _ptr(idx[b]), n_out, st)
+            if rc:
+                _raise(rc, "maxpool_forward failed")
+    return [out, idx]
+
+
+def maxpool_backward(aprs, grad_output, max_indices, level_delta):
+    _check_input(grad_output, "grad_output")
+    _check_input(max_indices, "max_indices")
+    B, Cn, n_out = grad_output.shape
+    d = _deltas(level_delta, len(aprs))
+    sizes = [number_particles(a, d[b]) for b, a in enumerate(aprs)]
+    n_in = max(sizes)
+    gx = torch.empty((B, Cn, n_in), dtype=grad_output.dtype, device=grad_output.device)
+    _zero_tails(gx, sizes)
+    plans = _plans(aprs, grad_output.device)
+    fn = getattr(_lib(), "aprnet_maxpool_bwd_" + _sfx(grad_output))
+    with torch.cuda.device(grad_output.device):
+        st = _stream()
+        for b in range(B):
+            rc = fn(plans[b], d[b], _ptr(grad_output[b]), n_out, Cn, _ptr(gx[b]), n_in, _ptr(max_indices[b]),
+                    max_indices.size(2), st)
+            if rc:
+                _raise(rc, "maxpool_backward failed")
+    return gx
+
+
+def upsample_const_forward(aprs, x, level_delta):
+    _check_input(x, "input")
+    B, Cn, N = x.shape
+    d = _deltas(level_delta, len(aprs))
+    if min(d[:len(aprs)]) <= 0:           # upsample.hpp:49-54
+        raise ValueError("UpSampleConst is only implemented for downsampled particles. It is currently "
+                         "not possible to go beyond the original resolution. That is, input must have "
+                         "`level_delta > 0`.")
+    sizes = [number_particles(a, d[b] - 1) for b, a in enumerate(aprs)]
+    n_out = max(sizes)
+    out = torch.empty((B, Cn, n_out), dtype=x.dtype, device=x.device)
+    _zero_tails(out, sizes)
+    plans = _plans(aprs, x.device)
+    fn = getattr(_lib(), "aprnet_upsample_fwd_" + _sfx(x))
+    with torch.cuda.device(x.device):
+        st = _stream()
+        for b in range(B):
+            rc = fn(plans[b], d[b], _ptr(x[b]), N, Cn, _ptr(out[b]), n_out, st)
+            if rc:
+                _raise(rc, "upsample_const_forward failed")
+    return out
+
+
+def upsample_const_backward(aprs, grad_output, level_delta):
+    _check_input(grad_output, "grad_output")
+    B, Cn, n_out = grad_output.shape
+    d = _deltas(level_delta, len(aprs))
+    sizes = [number_particles(a, d[b]) for b, a in enumerate(aprs)]
+    n_in = max(sizes)
+    gx = torch.empty((B, Cn, n_in), dtype=grad_output.dtype, device=grad_output.device)
+    _zero_tails(gx, sizes)
+    plans = _plans(aprs, grad_output.device)
+    fn = getattr(_lib(), "aprnet_upsample_bwd_" + _sfx(grad_output))
+    with torch.cuda.device(grad_output.device):
+        st = _stream()
+        for b in range(B):
+            rc = fn(plans[b], d[b], _ptr(grad_output[b]), n_out, Cn, _ptr(gx[b]), n_in, st)
+            if rc:
+                _raise(rc, "upsample_const_backward failed")
+    return gx
+
+
+# ---------------------------------------------------------------------------------------- pixels <-> particles
+def _dense_shape(aprs, d):
+    z = x = y = 0
+    for b, a in enumerate(aprs):
+        lc = a.level_max() - d[b]
+        z, x, y = max(z, a.z_num(lc)), max(x, a.x_num(lc)), max(y, a.y_num(lc))
+    return z, x, y
+
+
+def _same_dense_shape(aprs, d, shape):
+    for b, a in enumerate(aprs):
+        lc = a.level_max() - d[b]
+        if (a.z_num(lc), a.x_num(lc), a.y_num(lc)) != tuple(shape):
+            raise ValueError("reconstruct / sample_particles: all batch items must share the dense shape "
+                             f"{tuple(shape)} at their level delta")
+
+
+def reconstruct_forward(aprs, x, level_delta):
+    """reconstruct_forward (wrap_reconstruct_gpu.hpp:30-63): particles [B,C,N_d] -> [B,C,Z,X,Y] at level Lc."""
+    _check_input(x, "input")
+    B, Cn, N = x.shape
+    d = _deltas(level_delta, len(aprs))
+    shape = _dense_shape(aprs, d)
+    _same_dense_shape(aprs, d, shape)
+    out = torch.zeros((B, Cn, *shape), dtype=x.dtype, device=x.device)
+    plane = shape[0] * shape[1] * shape[2]
+    plans = _plans(aprs, x.device)
+    fn = getattr(_lib(), "aprnet_reconstruct_fwd_" + _sfx(x))
+    with torch.cuda.device(x.device):
+        st = _stream()
+        for b in range(B):
+            rc = fn(plans[b], d[b], _ptr(x[b]), N, Cn, _ptr(out[b]), plane, st)
+            if rc:
+                _raise(rc, "reconstruct_forward failed")
+    return out
+
+
+def reconstruct_backward(aprs, grad_output, level_delta):
+    _check_input(grad_output, "grad_output")
+    B, Cn = grad_output.shape[:2]
+    d = _deltas(level_delta, len(aprs))
+    _same_dense_shape(aprs, d, grad_output.shape[2:])
+    sizes = [number_particles(a, d[b]) for b, a in enumerate(aprs)]
+    n = max(sizes)
+    gx = torch.empty((B, Cn, n), dtype=grad_output.dtype, device=grad_output.device)
+    _zero_tails(gx, sizes)
+    plane = grad_output[0, 0].numel()
+    plans = _plans(aprs, grad_output.device)
+    fn = getattr(_lib(), "aprnet_reconstruct_bwd_" + _sfx(grad_output))
+    with torch.cuda.device(grad_output.device):
+        st = _stream()
+        for b in range(B):
+            rc = fn(plans[b], d[b], _ptr(grad_output[b]), plane, Cn, _ptr(gx[b]), n, st)
+            if rc:
+                _raise(rc, "reconstruct_backward failed")
+    return gx
+
+
+def sample_particles_forward(aprs, img, level_delta):
+    """sample_particles_forward (wrap_sample_particles_gpu.hpp:30-63): dense [B,C,Z,X,Y] -> particles (cell means)."""
+    _check_input(img, "input")
+    B, Cn = img.shape[:2]
+    d = _deltas(level_delta, len(aprs))
+    _same_dense_shape(aprs, d, img.shape[2:])
+    sizes = [number_particles(a, d[b]) for b, a in enumerate(aprs)]
+    n = max(sizes)
+    out = torch.empty((B, Cn, n), dtype=img.dtype, device=img.device)
+    _zero_tails(out, sizes)
+    plane = img[0, 0].numel()
+    plans = _plans(aprs, img.device)
+    fn = getattr(_lib(), "aprnet_sample_particles_fwd_" + _sfx(img))
+    with torch.cuda.device(img.device):
+        st = _stream()
+        for b in range(B):
+            rc = fn(plans[b], d[b], _ptr(img[b]), plane, Cn, _ptr(out[b]), n, st)
+            if rc:
+                _raise(rc, "sample_particles_forward failed")
+    return out
+
+
+def sample_particles_backward(aprs, grad_output, level_delta):
+    _check_input(grad_output, "grad_output")
+    B, Cn, N = grad_output.shape
+    d = _deltas(level_delta, len(aprs))
+    shape = _dense_shape(aprs, d)
+    _same_dense_shape(aprs, d, shape)
+    gimg = torch.zeros((B, Cn, *shape), dtype=grad_output.dtype, device=grad_output.device)
+    plane = shape[0] * shape[1] * shape[2]
+    plans = _plans(aprs, grad_output.device)
+    fn = getattr(_lib(), "aprnet_sample_particles_bwd_" + _sfx(grad_output))
+    with torch.cuda.device(grad_output.device):
+        st = _stream()
+        for b in range(B):
+            rc = fn(plans[b], d[b], _ptr(grad_output[b]), N, Cn, _ptr(gimg[b]), plane, st)
+            if rc:
+                _raise(rc, "sample_particles_backward failed")
+    return gimg

@@ -1,0 +1,121 @@
+"""torch.autograd.Functions of the particle-space operators, with the contracts of the reference's
+Functions (pyapr/aprnet/conv.py:18-138, pool.py:7-22, upsample.py:7-22; cuda/conv.py:12-54,
+cuda/maxpool.py:8-28, cuda/upsample.py:8-26, cuda/utils.py:10-47):
+
+* convolution: weights are expanded to one stencil per level before every call
+  (num_levels = max over the batch of level_max - level_min + 1, conv.py:95), the expanded weights and a
+  *clone* of ``level_deltas`` are saved for backward, the bias is added afterwards, backward returns
+  ``(grad_input, grad_weights, grad_bias, None, None)``;
+* max-pool / upsample mutate ``level_deltas`` in place *after* the native call (pool.py:13-14,
+  upsample.py:13-14) and use the saved pre-mutation copy in backward.
+
+One Function per operator, parameterised by the stencil size and the weight layout, instead of one
+class per stencil size.
+"""
+import torch
+from torch.autograd import Function
+
+from . import _ops
+
+CPU_LAYOUT = "cin_s_cout"      # [Cin, S, Cout, kz, kx, ky]   pyapr/aprnet/conv.py:164
+CUDA_LAYOUT = "s_cout_cin"     # [S, Cout, Cin, kz, kx, ky]   pyapr/aprnet/cuda/conv.py:77
+
+SUPPORTED_KERNELS = {(1, 1, 1), (1, 3, 3), (1, 5, 5), (3, 3, 3), (5, 5, 5)}
+
+
+def _to_device_layout(w, layout):
+    return w if layout == CUDA_LAYOUT else w.permute(1, 2, 0, 3, 4, 5).contiguous()
+
+
+def _from_device_layout(w, layout):
+    return w if layout == CUDA_LAYOUT else w.permute(2, 0, 1, 3, 4, 5).contiguous()
+
+
+class ConvFunction(Function):
+    @staticmethod
+    def forward(ctx, inputs, weights, bias, aprs, level_deltas, layout):
+        ctx.aprs = aprs
+        ctx.layout = layout
+        w = _to_device_layout(weights, layout).contiguous()
+        ctx.num_stencils = w.shape[0]
+        ksize = tuple(w.shape[3:])
+        if ksize not in SUPPORTED_KERNELS:
+            raise ValueError(f"unsupported kernel size {ksize}")
+        ctx.expand = ksize != (1, 1, 1)
+        if ctx.expand:
+            num_levels = max(a.level_max() - a.level_min() + 1 for a in aprs)
+            w = _ops.restrict_kernel_forward(w, num_levels)
+        inputs = inputs.contiguous()
+        ctx.save_for_backward(inputs, w, bias, level_deltas.clone())
+        output = _ops.conv_forward(aprs, inputs, w, level_deltas)
+        return output if bias is None else output + bias.view((1, -1, 1))
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        inputs, w_exp, bias, level_deltas = ctx.saved_tensors
+        grad_output = grad_output.contiguous()
+        grad_input, grad_w = _ops.conv_backward(ctx.aprs, inputs, w_exp, grad_output, level_deltas)
+        grad_bias = None if bias is None else torch.sum(grad_output, dim=(0, 2))
+        if ctx.expand:
+            grad_w = _ops.restrict_kernel_backward(grad_w, ctx.num_stencils)
+        return grad_input, _from_device_layout(grad_w, ctx.layout), grad_bias, None, None, None
+
+
+class MaxPoolFunction(Function):
+    @staticmethod
+    def forward(ctx, inputs, aprs, level_deltas, increment_level_deltas, pad_value):
+        ctx.aprs = aprs
+        output, max_indices = _ops.maxpool_forward(aprs, inputs.contiguous(), level_deltas, pad_value)
+        ctx.save_for_backward(max_indices, level_deltas.clone())
+        if increment_level_deltas:
+            level_deltas.add_(1)
+        return output
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        max_indices, level_deltas = ctx.saved_tensors
+        grad_input = _ops.maxpool_backward(ctx.aprs, grad_output.contiguous(), max_indices, level_deltas)
+        return grad_input, None, None, None, None
+
+
+class UpSampleConstFunction(Function):
+    @staticmethod
+    def forward(ctx, inputs, aprs, level_deltas, decrement_level_deltas):
+        ctx.aprs = aprs
+        ctx.save_for_backward(level_deltas.clone())
+        output = _ops.upsample_const_forward(aprs, inputs.contiguous(), level_deltas)
+        if decrement_level_deltas:
+            level_deltas.sub_(1)
+        return output
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        level_deltas, = ctx.saved_tensors
+        grad_input = _ops.upsample_const_backward(ctx.aprs, grad_output.contiguous(), level_deltas)
+        return grad_input, None, None, None
+
+
+class ReconstructFunction(Function):
+    @staticmethod
+    def forward(ctx, inputs, aprs, level_deltas):
+        ctx.aprs = aprs
+        ctx.save_for_backward(level_deltas.clone())
+        return _ops.reconstruct_forward(aprs, inputs.contiguous(), level_deltas)
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        level_deltas, = ctx.saved_tensors
+        return _ops.reconstruct_backward(ctx.aprs, grad_output.contiguous(), level_deltas), None, None
+
+
+class SampleParticlesFunction(Function):
+    @staticmethod
+    def forward(ctx, inputs, aprs, level_deltas):
+        ctx.aprs = aprs
+        ctx.save_for_backward(level_deltas.clone())
+        return _ops.sample_particles_forward(aprs, inputs.contiguous(), level_deltas)
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        level_deltas, = ctx.saved_tensors
+        return _ops.sample_particles_backward(ctx.aprs, grad_output.contiguous(), level_deltas), None, None

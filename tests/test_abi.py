@@ -1,0 +1,92 @@
+"""CPU-side checks of the drop-in boundary: the C-ABI library loads without a GPU and exports every
+symbol that include/aprnet_hip.h declares; the Python host layer mirrors the reference's module API and
+refuses to run without device tensors (no CPU fallback)."""
+import ctypes
+import os
+import re
+
+import pytest
+import torch
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "aprnet_hip.h")
+LIB = os.path.join(ROOT, "apr-cnn_amd", "csrc", "libaprnet_hip.so")
+
+
+def declared_symbols():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    names = set(re.findall(r"\b(aprnet_[a-z0-9_]+)\s*\(", text))
+    macro = re.search(r"#define APRNET_DECL\(T, SFX\)(.*?)\n\nAPRNET_DECL", text, flags=re.S).group(1)
+    for base in re.findall(r"\b(aprnet_[a-z0-9_]+_)##SFX", macro):
+        for sfx in ("f32", "f64"):
+            names.add(base + sfx)
+    return sorted(n for n in names if not n.endswith("_"))
+
+
+def test_library_exports_every_declared_symbol():
+    lib = ctypes.CDLL(LIB)
+    names = declared_symbols()
+    assert len(names) >= 39
+    missing = [n for n in names if not hasattr(lib, n)]
+    assert not missing, f"declared in aprnet_hip.h but not exported: {missing}"
+
+
+def test_module_api_mirrors_reference():
+    from pyapr import aprnet
+    from pyapr.aprnet import cuda
+    # constructor signature / parameter names / layouts (conv.py:154-166, cuda/conv.py:66-79)
+    m = aprnet.APRConv(3, 5, nstencils=2, kernel_size=(1, 5, 5), bias=True)
+    assert tuple(m.weight.shape) == (3, 2, 5, 1, 5, 5) and tuple(m.bias.shape) == (5,)
+    assert set(m.state_dict()) == {"weight", "bias"}
+    mc = cuda.APRConv(3, 5, nstencils=2, kernel_size=(3, 3, 3), bias=False)
+    assert tuple(mc.weight.shape) == (2, 5, 3, 3, 3, 3) and mc.bias is None
+    assert set(mc.state_dict()) == {"weight"}
+    # kaiming_uniform_(a=sqrt(5)) bound: sqrt(6 / ((1 + 5) * fan_in)) with fan_in = size(1) * receptive field
+    fan_in = mc.weight.shape[1] * 27
+    assert float(mc.weight.abs().max()) <= (1.0 / fan_in) ** 0.5 + 1e-6
+    assert aprnet.MaxPool().increment_level_deltas is True
+    assert aprnet.UpSampleConst().decrement_level_deltas is True
+    for name in ("APRConv", "MaxPool", "UpSampleConst", "Reconstruct", "SampleParticles"):
+        assert hasattr(cuda, name)
+    for name in ("number_particles", "number_parts", "number_particles_after_pooling", "number_particles_after_upsampling"):
+        assert hasattr(aprnet.utils, name)
+
+
+def test_no_cpu_fallback():
+    """Operators refuse host tensors (CHECK_CUDA, cuda/src/common.hpp:14) instead of computing on the CPU."""
+    import apr_cases
+    from pyapr import aprnet
+    apr = apr_cases.get("3d_a")
+    n = aprnet.utils.number_particles(apr, 0)
+    x = torch.zeros(1, 1, n)
+    ld = torch.zeros(1, dtype=torch.int32)
+    with pytest.raises(RuntimeError, match="CUDA tensor"):
+        aprnet.MaxPool()(x, [apr], ld)
+    with pytest.raises(RuntimeError, match="CUDA tensor"):
+        aprnet.cuda.APRConv(1, 1, kernel_size=(1, 1, 1))(x, [apr], ld)
+
+
+def test_number_particles_helpers():
+    import apr_cases
+    from oracle import oracle
+    from pyapr import aprnet
+    for name in ("3d_a", "2d_b", "1d_a", "3d_s"):
+        apr = apr_cases.get(name)
+        for d in range(apr.level_max() - 1):
+            assert aprnet.utils.number_particles(apr, d) == oracle.number_parts(apr, d)
+            assert aprnet.utils.number_particles_after_pooling(apr, d) == oracle.number_parts(apr, d + 1)
+        assert aprnet.utils.number_particles(apr, 0) == apr.total_number_particles()
+
+
+def test_apr_state_roundtrip():
+    """The serialisable state is the one of BindAPR.hpp:72-90; level_xz_vec is recomputed from the dims."""
+    import numpy as np
+    import apr_cases
+    from pyapr import APR
+    apr = apr_cases.get("3d_b")
+    oy, ox, oz, _params, xz, y, txz, ty = apr.get_state()
+    back = APR.from_state((oy, ox, oz), xz, y, txz, ty)
+    for a, b in ((apr.iterator(), back.iterator()), (apr.tree_iterator(), back.tree_iterator())):
+        assert np.array_equal(a.level_xz_vec, b.level_xz_vec) and np.array_equal(a.xz_end_vec, b.xz_end_vec)
+        assert np.array_equal(a.y_vec, b.y_vec) and a.level_min() == b.level_min() and a.level_max() == b.level_max()

@@ -1,0 +1,243 @@
+"""GPU parity tests: the HIP operators (through pyapr.aprnet -> C ABI of libaprnet_hip.so) against the
+CPU oracle on the same seeded inputs.  Bit-exact for index maps and pooling argmax; float64 to 1e-11
+and float32 to rel 1e-5 of the output scale for values (the sides differ in summation order only)."""
+import ctypes as C
+
+import numpy as np
+import pytest
+import torch
+
+import apr_cases
+from oracle import oracle
+from pyapr import _native
+from pyapr.aprnet import _ops
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda:0"
+ALL_CASES = list(apr_cases.TINY) + list(apr_cases.SMALL)
+KID = lambda k: "k%d%d%d" % tuple(k)
+
+
+def close(got, ref, dtype):
+    got = got.detach().cpu()
+    if dtype == torch.float64:
+        torch.testing.assert_close(got, ref, rtol=1e-11, atol=1e-11 * max(1.0, float(ref.abs().max())))
+    else:
+        # rel 1e-5 of the output scale (fp32 sums of up to a few thousand terms in a different order)
+        scale = max(float(ref.abs().max()), 1e-30)
+        err = float((got - ref).abs().max())
+        assert err <= 1e-5 * scale, f"max abs err {err:.3e} vs scale {scale:.3e}"
+
+
+def batch(names_d, channels, dtype, seed=0):
+    aprs = [apr_cases.get(n) for n, _ in names_d]
+    ld = torch.tensor([d for _, d in names_d], dtype=torch.int32)
+    sizes = [oracle.number_parts(a, int(d)) for a, d in zip(aprs, ld)]
+    g = torch.Generator().manual_seed(seed)
+    x = torch.randn(len(aprs), channels, max(sizes), dtype=dtype, generator=g)
+    for i, n in enumerate(sizes):
+        x[i, :, n:] = 0
+    return x, aprs, ld
+
+
+def max_delta(apr):
+    return min(2, apr.level_max() - 1)
+
+
+@pytest.mark.parametrize("name", ALL_CASES)
+def test_child_table_matches_reference_parent_walk(name):
+    """The index map behind pool / upsample / tree fill is bit-exact against the merge walk of
+    helpers.hpp:185-194 (restated in the oracle)."""
+    apr = apr_cases.get(name)
+    apr.init_cuda()
+    nt = apr.total_number_tree_particles()
+    ch = np.zeros((8, nt), np.int32)
+    assert _native.hip().aprnet_plan_children(apr.plan(0), ch.ctypes.data) == 0
+    parent_of_part = np.full(apr.total_number_particles(), -1, np.int64)
+    parent_of_tree = np.full(nt, -1, np.int64)
+    for s in range(8):
+        for t in range(nt):
+            v = int(ch[s, t])
+            if v == -2 ** 31:
+                continue
+            if v >= 0:
+                assert parent_of_part[v] == -1
+                parent_of_part[v] = t
+            else:
+                assert parent_of_tree[~v] == -1
+                parent_of_tree[~v] = t
+    it, tr = apr.iterator(), apr.tree_iterator()
+    for level in range(1, apr.level_max() + 1):
+        ref = oracle.parent_index(apr, 0, level)
+        b, e = it.particles_level_begin(level), it.particles_level_end(level)
+        assert np.array_equal(parent_of_part[b:e], ref[b:e])
+    for level in range(1, apr.level_max()):
+        ref = oracle.parent_index(apr, 1, level)
+        b, e = tr.particles_level_begin(level), tr.particles_level_end(level)
+        assert np.array_equal(parent_of_tree[b:e], ref[b:e])
+
+
+@pytest.mark.parametrize("name", ALL_CASES)
+def test_number_parts(name):
+    apr = apr_cases.get(name)
+    apr.init_cuda()
+    lib = _native.hip()
+    for d in range(apr.level_max()):
+        assert lib.aprnet_number_parts(apr.plan(0), d) == oracle.number_parts(apr, d) == _ops.number_particles(apr, d)
+        assert lib.aprnet_tree_offset(apr.plan(0), apr.level_max() - d) == oracle.tree_offset(apr, apr.level_max() - d)
+        assert lib.aprnet_tree_parts(apr.plan(0), d) == oracle.tree_parts(apr, d)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
+@pytest.mark.parametrize("name", ALL_CASES)
+def test_fill_tree_mean(name, dtype):
+    apr = apr_cases.get(name)
+    apr.init_cuda()
+    lib = _native.hip()
+    sfx = "f32" if dtype == torch.float32 else "f64"
+    for d in range(max_delta(apr) + 1):
+        n, nt = oracle.number_parts(apr, d), oracle.tree_parts(apr, d)
+        g = torch.Generator().manual_seed(d)
+        x = torch.randn(2, n, dtype=dtype, generator=g)
+        xd = x.to(DEV)
+        tree = torch.zeros(2, max(nt, 1), dtype=dtype, device=DEV)
+        rc = getattr(lib, "aprnet_fill_tree_mean_" + sfx)(apr.plan(0), d, xd.data_ptr(), n, 2, tree.data_ptr(), max(nt, 1),
+                                                         torch.cuda.current_stream().cuda_stream)
+        assert rc == 0, lib.aprnet_last_error()
+        for c in range(2):
+            ref = oracle.fill_tree_mean(apr, x[c], d)
+            # same summation order as the reference -> identical bits
+            assert torch.equal(tree[c, :nt].cpu(), ref)
+        # backward: adjoint of the forward
+        gt = torch.randn(2, max(nt, 1), dtype=dtype, generator=g)
+        gtd, gx = gt.to(DEV), torch.zeros(2, n, dtype=dtype, device=DEV)
+        rc = getattr(lib, "aprnet_fill_tree_mean_bwd_" + sfx)(apr.plan(0), d, gx.data_ptr(), n, 2, gtd.data_ptr(), max(nt, 1),
+                                                             torch.cuda.current_stream().cuda_stream)
+        assert rc == 0, lib.aprnet_last_error()
+        for c in range(2):
+            close(gx[c], oracle.fill_tree_mean_backward(apr, gt[c, :nt], n, d), dtype)
+
+
+CONV_BATCHES = [
+    [("3d_a", 0)], [("3d_b", 1)], [("3d_a", 2), ("3d_c", 2)], [("3d_s", 0), ("3d_a", 1)], [("3d_t", 1)],
+    [("2d_a", 0)], [("2d_a", 1), ("2d_b", 2)], [("2d_s", 0)], [("2d_t", 0), ("2d_t", 2)], [("1d_a", 0), ("1d_s", 1)],
+]
+
+
+def _conv_case(bt, ksize, nstencils, cin, cout, dtype):
+    x, aprs, ld = batch(bt, cin, dtype, seed=nstencils)
+    g = torch.Generator().manual_seed(17)
+    w = torch.randn(cin, nstencils, cout, *ksize, dtype=dtype, generator=g)      # CPU layout
+    num_levels = max(a.level_max() - a.level_min() + 1 for a in aprs)
+    w_exp = w if ksize == (1, 1, 1) else oracle.restrict_kernel_forward(w, num_levels)
+    return x, aprs, ld, w_exp
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
+@pytest.mark.parametrize("ksize", [(3, 3, 3), (1, 3, 3), (1, 5, 5), (5, 5, 5), (1, 1, 1)], ids=KID)
+@pytest.mark.parametrize("bt", CONV_BATCHES, ids=lambda b: "+".join(f"{n}@{d}" for n, d in b))
+def test_conv_forward(bt, ksize, dtype):
+    cin, cout, S = 5, 7, 3
+    x, aprs, ld, w_exp = _conv_case(bt, ksize, S, cin, cout, dtype)
+    ref = oracle.conv_forward(aprs, x, w_exp, ld)
+    wd = w_exp.permute(1, 2, 0, 3, 4, 5).contiguous().to(DEV)                    # -> [S, Cout, Cin, k]
+    got = _ops.conv_forward(aprs, x.to(DEV), wd, ld)
+    close(got, ref, dtype)
+
+
+@pytest.mark.parametrize("cin,cout", [(1, 16), (32, 32), (33, 33), (16, 3)])
+def test_conv333_forward_channel_shapes(cin, cout):
+    """Channel counts of the benchmark configurations and of the reference's CUDA-vs-CPU test
+    (33 -> 33, pyapr/tests/test_aprnet.py:137-138)."""
+    x, aprs, ld, w_exp = _conv_case([("3d_s", 0), ("3d_t", 1)], (3, 3, 3), 2, cin, cout, torch.float32)
+    ref = oracle.conv_forward(aprs, x, w_exp, ld)
+    got = _ops.conv_forward(aprs, x.to(DEV), w_exp.permute(1, 2, 0, 3, 4, 5).contiguous().to(DEV), ld)
+    close(got, ref, torch.float32)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
+@pytest.mark.parametrize("ksize", [(3, 3, 3), (1, 3, 3), (1, 5, 5), (5, 5, 5), (1, 1, 1)], ids=KID)
+@pytest.mark.parametrize("bt", [[("3d_a", 0)], [("3d_b", 1), ("3d_c", 2)], [("2d_a", 1), ("2d_b", 0)], [("3d_s", 0)]],
+                         ids=lambda b: "+".join(f"{n}@{d}" for n, d in b))
+def test_conv_backward(bt, ksize, dtype):
+    cin, cout, S = 3, 4, 2
+    x, aprs, ld, w_exp = _conv_case(bt, ksize, S, cin, cout, dtype)
+    g = torch.Generator().manual_seed(5)
+    go = torch.randn(x.size(0), cout, x.size(2), dtype=dtype, generator=g)
+    gx_ref, gw_ref = oracle.conv_backward(aprs, x, w_exp, go, ld)
+    wd = w_exp.permute(1, 2, 0, 3, 4, 5).contiguous().to(DEV)
+    gx, gw = _ops.conv_backward(aprs, x.to(DEV), wd, go.to(DEV), ld)
+    # the reference leaves gradients of padding slots at zero
+    close(gx, gx_ref, dtype)
+    close(gw.permute(2, 0, 1, 3, 4, 5), gw_ref, dtype)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
+@pytest.mark.parametrize("ksize", [(3, 3, 3), (1, 3, 3), (1, 5, 5), (5, 5, 5)], ids=KID)
+@pytest.mark.parametrize("s,levels", [(1, 4), (2, 5), (3, 3), (3, 7)])
+def test_restrict_kernel(ksize, s, levels, dtype):
+    g = torch.Generator().manual_seed(s + levels)
+    w = torch.randn(3, s, 4, *ksize, dtype=dtype, generator=g)                   # CPU layout [Cin, S, Cout, k]
+    ref = oracle.restrict_kernel_forward(w, levels)
+    got = _ops.restrict_kernel_forward(w.permute(1, 2, 0, 3, 4, 5).contiguous().to(DEV), levels)
+    close(got.permute(2, 0, 1, 3, 4, 5), ref, dtype)
+    gw = torch.randn(3, levels, 4, *ksize, dtype=dtype, generator=g)
+    ref_b = oracle.restrict_kernel_backward(gw, s)
+    got_b = _ops.restrict_kernel_backward(gw.permute(1, 2, 0, 3, 4, 5).contiguous().to(DEV), s)
+    close(got_b.permute(2, 0, 1, 3, 4, 5), ref_b, dtype)
+
+
+POOL_BATCHES = [[("3d_a", 0)], [("3d_b", 1)], [("3d_a", 1), ("3d_c", 0)], [("3d_s", 0), ("3d_t", 1)], [("2d_a", 0), ("2d_b", 1)],
+                [("2d_t", 2)], [("1d_a", 0), ("1d_s", 1)]]
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
+@pytest.mark.parametrize("bt", POOL_BATCHES, ids=lambda b: "+".join(f"{n}@{d}" for n, d in b))
+def test_maxpool_bit_exact_with_ties(bt, dtype):
+    x, aprs, ld = batch(bt, 3, dtype)
+    x = torch.clamp(torch.round(x * 1.5), min=0)          # few distinct values, zeros as after a ReLU
+    ref, ref_idx = oracle.maxpool_forward(aprs, x, ld)
+    out, idx = _ops.maxpool_forward(aprs, x.to(DEV), ld)
+    assert torch.equal(out.cpu(), ref)
+    assert torch.equal(idx.cpu(), ref_idx)
+    g = torch.Generator().manual_seed(3)
+    go = torch.randn(ref.shape, dtype=dtype, generator=g)
+    gref = oracle.maxpool_backward(aprs, go, ref_idx, ld)
+    got = _ops.maxpool_backward(aprs, go.to(DEV), idx, ld)
+    assert torch.equal(got.cpu(), gref)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
+@pytest.mark.parametrize("bt", [[("3d_a", 1)], [("3d_b", 2)], [("3d_a", 1), ("3d_c", 2)], [("3d_s", 1), ("3d_t", 2)],
+                                [("2d_a", 1), ("2d_b", 2)], [("1d_a", 1), ("1d_s", 2)]],
+                         ids=lambda b: "+".join(f"{n}@{d}" for n, d in b))
+def test_upsample(bt, dtype):
+    x, aprs, ld = batch(bt, 3, dtype)
+    ref = oracle.upsample_const_forward(aprs, x, ld)
+    got = _ops.upsample_const_forward(aprs, x.to(DEV), ld)
+    assert torch.equal(got.cpu(), ref)
+    g = torch.Generator().manual_seed(9)
+    go = torch.randn(ref.shape, dtype=dtype, generator=g)
+    sizes = [oracle.number_parts(a, int(d) - 1) for a, d in zip(aprs, ld)]
+    for i, n in enumerate(sizes):
+        go[i, :, n:] = 0
+    close(_ops.upsample_const_backward(aprs, go.to(DEV), ld), oracle.upsample_const_backward(aprs, go, ld), dtype)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
+@pytest.mark.parametrize("bt", [[("3d_a", 0)], [("3d_b", 1)], [("3d_c", 2), ("3d_c", 2)], [("2d_a", 1)], [("3d_s", 0)]],
+                         ids=lambda b: "+".join(f"{n}@{d}" for n, d in b))
+def test_reconstruct_and_sample(bt, dtype):
+    x, aprs, ld = batch(bt, 2, dtype)
+    xd = x.to(DEV)
+    img_ref = oracle.reconstruct_forward(aprs, x, ld)
+    img = _ops.reconstruct_forward(aprs, xd, ld)
+    assert torch.equal(img.cpu(), img_ref)
+    # SampleParticles(Reconstruct(x)) == x  (pyapr/tests/test_aprnet.py:272-285)
+    close(_ops.sample_particles_forward(aprs, img, ld), x, dtype)
+    g = torch.Generator().manual_seed(2)
+    im = torch.randn(img_ref.shape, dtype=dtype, generator=g)
+    close(_ops.sample_particles_forward(aprs, im.to(DEV), ld), oracle.sample_particles_forward(aprs, im, ld), dtype)
+    close(_ops.reconstruct_backward(aprs, im.to(DEV), ld), oracle.reconstruct_backward(aprs, im, ld), dtype)
+    close(_ops.sample_particles_backward(aprs, xd, ld), oracle.sample_particles_backward(aprs, x, ld), dtype)
