@@ -1,0 +1,4 @@
+"""Particle-space models built on ``pyapr.aprnet.cuda`` (apr_models/apr_models/__init__.py)."""
+from . import unet
+
+__all__ = ["unet"]

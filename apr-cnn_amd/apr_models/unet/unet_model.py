@@ -1,0 +1,70 @@
+"""APRUNet (apr_models/apr_models/unet/unet_model.py:7-94): encoder of ConvBlock + `depth` DownConv
+stages, decoder of UpConv stages with skip connections, 1x1x1 head with bias.  One int32 CPU
+``level_deltas`` tensor is shared and mutated in place by the pool / upsample modules."""
+import torch
+import torch.nn as nn
+
+from pyapr.aprnet import cuda as aprnet
+from .unet_parts import BasicBlock, ConvBlock, DownConv, UpConv
+
+
+class APRUNet(nn.Module):
+    def __init__(self, in_channels, out_channels, depth=3, kernel_size=3, dims=3, activation=nn.ReLU,
+                 n_filters_base=16, n_conv_per_block=2, n_stencils=2, decrement_stencils=False, num_groups=None,
+                 channels_per_group=None, norm="group"):
+        super().__init__()
+        self.in_channels, self.out_channels, self.depth = in_channels, out_channels, depth
+        self.num_groups = self.channels_per_group = None
+        if num_groups is None and channels_per_group is None:
+            self.num_groups = n_filters_base
+        elif channels_per_group:
+            self.channels_per_group = channels_per_group
+        else:
+            self.num_groups = num_groups
+
+        ks = (kernel_size,) * dims if isinstance(kernel_size, int) else tuple(kernel_size)
+        self.kernel_size = (1,) * (3 - len(ks)) + ks
+        stencils = [max(n_stencils - i, 1) if decrement_stencils else max(n_stencils, 1) for i in range(depth + 1)]
+        widths = [n_filters_base * 2 ** i for i in range(depth + 1)]
+
+        def groups(c):
+            return self.num_groups or c // self.channels_per_group
+
+        common = dict(kernel_size=self.kernel_size, activation=activation, norm=norm)
+        self.encoder = nn.ModuleList([ConvBlock(in_channels, widths[0], nstencils=stencils[0], num_blocks=n_conv_per_block,
+                                                num_groups=groups(widths[0]), **common)])
+        for i in range(depth):
+            self.encoder.append(DownConv(widths[i], widths[i + 1], nstencils=stencils[i + 1],
+                                         num_conv_blocks=n_conv_per_block, num_groups=groups(widths[i + 1]), **common))
+        self.decoder = nn.ModuleList()
+        for i in reversed(range(depth)):
+            self.decoder.append(UpConv(widths[i + 1], widths[i], nstencils=stencils[i], num_conv_blocks=n_conv_per_block,
+                                       num_groups=groups(widths[i]), **common))
+        self.head = aprnet.APRConv(widths[0], out_channels, nstencils=stencils[0], kernel_size=(1, 1, 1))
+
+    def forward(self, x, aprs, level_deltas=None):
+        if level_deltas is None:
+            level_deltas = torch.zeros(len(aprs), dtype=torch.int32, device=torch.device("cpu"))
+        skips = [self.encoder[0](x, aprs, level_deltas)]
+        for stage in self.encoder[1:]:
+            skips.append(stage(skips[-1], aprs, level_deltas))
+        y = skips[-1]
+        for i, stage in enumerate(self.decoder):
+            y = stage(y, skips[-(i + 2)], aprs, level_deltas)
+        return self.head(y, aprs, level_deltas)
+
+
+@torch.no_grad()
+def fold_norms(model):
+    """Inference-time folding of BatchNorm1d (running statistics) into the preceding bias-free APRConv:
+    w' = w * gamma / sqrt(var + eps) per output channel, bias' = beta - mean * gamma / sqrt(var + eps).
+    The conv gains a bias parameter and the norm becomes nn.Identity.  GroupNorm depends on the input
+    and cannot be folded; models meant for folded inference are built with norm='batch'."""
+    for m in model.modules():
+        if isinstance(m, BasicBlock) and isinstance(m.norm, nn.BatchNorm1d):
+            bn, conv = m.norm, m.conv
+            scale = bn.weight / torch.sqrt(bn.running_var + bn.eps)
+            conv.weight.mul_(scale.view(1, -1, 1, 1, 1, 1))        # device layout [S, Cout, Cin, kz, kx, ky]
+            conv.bias = nn.Parameter((bn.bias - bn.running_mean * scale).clone())
+            m.norm = nn.Identity()
+    return model

@@ -93,9 +93,28 @@ conv_fwd_kernel(const ConvArgs<T> a) {
     }
 }
 
+// Optional timing of the dominant kernel with HIP events on the launch stream (aprnet_profile_*).
+struct KernelTimer {
+    bool enabled = false, armed = false;
+    hipEvent_t start = nullptr, stop = nullptr;
+};
+static KernelTimer g_timer;
+
+struct TimedLaunch {
+    hipStream_t st;
+    bool on;
+    explicit TimedLaunch(hipStream_t s) : st(s), on(g_timer.enabled) {
+        if (!on) return;
+        if (!g_timer.start) { (void)hipEventCreate(&g_timer.start); (void)hipEventCreate(&g_timer.stop); }
+        (void)hipEventRecord(g_timer.start, st);
+    }
+    ~TimedLaunch() { if (on) { (void)hipEventRecord(g_timer.stop, st); g_timer.armed = true; } }
+};
+
 template <typename T, class G, int CIB, int COB>
 static int launch_fwd(const ConvArgs<T>& a, int n_tiles, hipStream_t st) {
     dim3 grid((unsigned)n_tiles, (unsigned)((a.Cout + COB - 1) / COB));
+    TimedLaunch timed(st);
     hipLaunchKernelGGL((conv_fwd_kernel<T, G, CIB, COB>), grid, dim3(G::NT), 0, st, a);
     APRNET_LAUNCH_CHECK("conv_fwd_kernel");
     return 0;
@@ -151,6 +170,14 @@ int conv_fwd(const aprnet_plan* cp, int d, int kz, int kx, int ky, const T* x, i
 using namespace aprnet;
 
 extern "C" {
+int aprnet_profile_enable(int on) { g_timer.enabled = on != 0; g_timer.armed = false; return 0; }
+float aprnet_profile_last_ms(void) {
+    if (!g_timer.armed) return -1.0f;
+    float ms = -1.0f;
+    if (hipEventSynchronize(g_timer.stop) != hipSuccess) return -1.0f;
+    if (hipEventElapsedTime(&ms, g_timer.start, g_timer.stop) != hipSuccess) return -1.0f;
+    return ms;
+}
 int aprnet_conv_fwd_f32(const aprnet_plan* p, int d, int kz, int kx, int ky, const float* x, int64_t ldx, int Cin,
                         const float* w, int S_exp, int Cout, float* y, int64_t ldy, float* tree_ws, int64_t ldt, void* st) {
     return conv_fwd<float>(p, d, kz, kx, ky, x, ldx, Cin, w, S_exp, Cout, y, ldy, tree_ws, ldt, (hipStream_t)st);

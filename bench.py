@@ -1,0 +1,145 @@
+#!/usr/bin/env python3
+"""Benchmark of the hot path on one MI355X: APRConv 3x3x3 forward, Cin = Cout = 32, fp32, on the APR of the
+seeded 512 x 512 x 256 blob volume (BASELINE.json configs[1]).
+
+  python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+A step is one `aprnet.cuda.APRConv.forward` on device-resident features: weight expansion
+(restrict kernel), tree fill of the 32 input channels, the convolution kernel and the bias add.
+Prints ONE JSON line.  `value` = particles/s of the whole step; `roofline` prices the convolution
+kernel alone (its duration is measured with HIP events recorded around the launch on its own stream,
+see aprnet_profile_enable in include/aprnet_hip.h); `cpu_baseline` times the CPU oracle (a restatement
+of the reference's OpenMP code) on a centre crop of the same volume.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+for _p in (ROOT, os.path.join(ROOT, "apr-cnn_amd")):
+    if _p not in sys.path:
+        sys.path.insert(0, _p)
+
+CIN = COUT = 32
+K_TAPS = 27
+FLOP_PER_PARTICLE = 2 * K_TAPS * CIN * COUT          # 55 296
+BYTES_PER_PARTICLE = 4 * (CIN + COUT) + 2            # features in + out, y_vec
+PEAK_FP32_MATRIX_TFLOPS = 157.3
+PEAK_HBM_GBS = 8000.0
+
+
+def build_workload(name, crop=None):
+    import numpy as np
+    from pyapr.synthetic import CONFIGS, synth_volume, pipeline_parameters
+    from pyapr.converter import get_apr
+    shape, kind, n, axes, amp, bg, iso, rel = CONFIGS[name]
+    img = synth_volume(shape, 0, kind, n, axes, amp, bg, iso)
+    if crop is not None:
+        z, x, y = (s // 2 for s in shape)
+        cz, cx, cy = (c // 2 for c in crop)
+        img = np.ascontiguousarray(img[z - cz:z + cz, x - cx:x + cx, y - cy:y + cy])
+    apr, _parts = get_apr(img, params=pipeline_parameters(rel))
+    return apr
+
+
+def cpu_baseline(nstencils):
+    """CPU oracle (port of pyapr/aprnet/src/conv.hpp + helpers.hpp, OpenMP over z) on a 128 x 256 x 256 centre
+    crop of the benchmark volume, same layer shape; a few seconds to tens of seconds of CPU work."""
+    import torch
+    from oracle import oracle
+    crop = (128, 256, 256)
+    apr = build_workload("blobs512", crop=crop)
+    n = apr.total_number_particles()
+    g = torch.Generator().manual_seed(1)
+    x = torch.randn(1, CIN, n, generator=g)
+    w = torch.randn(CIN, nstencils, COUT, 3, 3, 3, generator=g) * 0.1
+    ld = torch.zeros(1, dtype=torch.int32)
+    t0 = time.perf_counter()
+    w_exp = oracle.restrict_kernel_forward(w, apr.level_max() - apr.level_min() + 1)
+    oracle.conv_forward([apr], x, w_exp, ld)
+    dt = time.perf_counter() - t0
+    cores = int(os.environ.get("OMP_NUM_THREADS", 0)) or len(os.sched_getaffinity(0))
+    return {"value": n / dt, "unit": "particles/s", "cores": cores, "kind": "port",
+            "sample": f"centre crop {crop[0]}x{crop[1]}x{crop[2]} of the 256x512x512 volume, {n} particles, "
+                      f"conv 3x3x3 {CIN}->{COUT} fp32, 1 run, {dt:.1f} s"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build runs on one GPU; --gpus N with N > 1 is not supported "
+                 "(the path shards by batch item or by z-slabs, see DESIGN.md)")
+
+    import torch
+    from pyapr import aprnet, _native
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+
+    nstencils = 2
+    t0 = time.perf_counter()
+    apr = build_workload("blobs512")
+    t_build = time.perf_counter() - t0
+    t0 = time.perf_counter()
+    apr.init_cuda()
+    t_plan = time.perf_counter() - t0
+    n = apr.total_number_particles()
+
+    torch.manual_seed(0)
+    x = torch.randn(1, CIN, n, device=dev)
+    conv = aprnet.cuda.APRConv(CIN, COUT, nstencils=nstencils, kernel_size=(3, 3, 3), bias=True).to(dev)
+    ld = torch.zeros(1, dtype=torch.int32)
+    lib = _native.hip()
+
+    with torch.no_grad():
+        for _ in range(args.warmup):
+            y = conv(x, [apr], ld)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            y = conv(x, [apr], ld)
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t0
+
+        # duration of the convolution kernel alone: HIP events around its launch, on its stream
+        lib.aprnet_profile_enable(1)
+        kms = []
+        for _ in range(args.steps):
+            y = conv(x, [apr], ld)
+            kms.append(float(lib.aprnet_profile_last_ms()))
+        lib.aprnet_profile_enable(0)
+    kernel_ms = sum(kms) / len(kms)
+    assert torch.isfinite(y).all()
+
+    ms_per_step = dt / args.steps * 1e3
+    value = n / (dt / args.steps)
+    tflops = FLOP_PER_PARTICLE * n / (kernel_ms * 1e-3) / 1e12
+    gbs = BYTES_PER_PARTICLE * n / (kernel_ms * 1e-3) / 1e9
+    out = {
+        "metric": "APRConv 3x3x3 fwd particles/s (Cin=Cout=32)",
+        "value": value, "unit": "particles/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "APRConv 3x3x3 32->32 fp32 forward (restrict + tree fill + conv + bias), batch 1, "
+                               "APR of the seeded 512x512x256 volume with 2000 ellipsoidal blobs (configs[1])",
+                   "n_particles": n, "nstencils": nstencils, "level_max": apr.level_max(),
+                   "apr_build_s": round(t_build, 2), "plan_create_s": round(t_plan, 2)},
+        "roofline": {"bound": "mfma", "achieved": tflops, "peak": PEAK_FP32_MATRIX_TFLOPS, "unit": "TFLOP/s",
+                     "frac": tflops / PEAK_FP32_MATRIX_TFLOPS, "traffic": None,
+                     "kernel": "conv_fwd_kernel", "kernel_ms": kernel_ms,
+                     "hbm_achieved_GBs": gbs, "hbm_frac": gbs / PEAK_HBM_GBS},
+    }
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline(nstencils)
+    print(json.dumps(out), flush=True)
+
+
+if __name__ == "__main__":
+    main()

@@ -72,6 +72,13 @@ int64_t aprnet_tree_parts(const aprnet_plan* plan, int level_delta);
  * upsample.hpp:112-118. */
 int aprnet_plan_children(const aprnet_plan* plan, int32_t* out_host);
 
+/* No counterpart in the reference (it has no profiling hooks).
+ * When enabled, the main kernel of every aprnet_conv_fwd_* call is bracketed by two HIP events recorded on
+ * the call's stream; aprnet_profile_last_ms() waits for the last bracket and returns its duration in
+ * milliseconds (-1 if none).  Process-wide, not thread-safe; meant for benchmarks. */
+int aprnet_profile_enable(int on);
+float aprnet_profile_last_ms(void);
+
 #define APRNET_DECL(T, SFX)                                                                                          \
     /* helpers::fill_tree_mean (helpers.hpp:156-252): tree[c][t] for all tree nodes of level < Lc. */               \
     int aprnet_fill_tree_mean_##SFX(const aprnet_plan*, int level_delta, const T* x, int64_t ldx, int C,            \
