@@ -29,10 +29,8 @@ conv_fwd_kernel(const ConvArgs<T> a) {
     open_segments<G, T>(a, L, z0, x0, sh);
     __syncthreads();
 
-    int yv[G::SPW];
-    unsigned long long inw;
     for (int y0 = 0; y0 < yn; y0 += G::TY) {
-        scan_window<G, T>(a, L, y0, out_tree, sh, yv, inw);
+        scan_window<G, T>(a, L, y0, out_tree, sh);
         __syncthreads();
         const int nc = sh.ncol;
         if (nc > 0) {
@@ -45,7 +43,7 @@ conv_fwd_kernel(const ConvArgs<T> a) {
             for (int ci0 = 0; ci0 < a.Cin; ci0 += CIB) {
                 for (int i = threadIdx.x; i < CIB * G::CH_STRIDE; i += G::NT) patch[i] = 0;
                 __syncthreads();
-                stage_values<G, T, CIB>(a, L, y0, ci0, sh, yv, inw, patch);
+                stage_values<G, T, CIB>(a, L, y0, ci0, sh, patch);
                 __syncthreads();
 #pragma unroll
                 for (int it = 0; it < G::ITER; ++it) {
@@ -88,7 +86,7 @@ conv_fwd_kernel(const ConvArgs<T> a) {
             }
         }
         __syncthreads();
-        advance_cursors<G, T>(y0, sh, yv);
+        advance_cursors<G>(sh);
         __syncthreads();
     }
 }
@@ -130,6 +128,17 @@ template <typename T> struct Chunk;       // channels staged per pass so that th
 template <> struct Chunk<float>  { static constexpr int c333 = 8, c133 = 16, c155 = 12, c555 = 4; };
 template <> struct Chunk<double> { static constexpr int c333 = 4, c133 = 8,  c155 = 6,  c555 = 2; };
 
+int launch_conv333_mfma(const ConvArgs<float>& a, int n_tiles, hipStream_t st);
+static int g_conv_path = 0;      // 0: matrix cores where available, 1: VALU kernels only
+
+template <typename T> static int try_mfma(const ConvArgs<T>&, int, int, hipStream_t, bool*) { return 0; }
+template <> int try_mfma<float>(const ConvArgs<float>& a, int code, int n_tiles, hipStream_t st, bool* done) {
+    if (g_conv_path == 1 || code != 333) return 0;
+    *done = true;
+    TimedLaunch timed(st);
+    return launch_conv333_mfma(a, n_tiles, st);
+}
+
 int fill_tree_for_conv(const aprnet_plan* p, int d, const float* x, int64_t ldx, int C, float* tree, int64_t ldt, hipStream_t st);
 int fill_tree_for_conv(const aprnet_plan* p, int d, const double* x, int64_t ldx, int C, double* tree, int64_t ldt, hipStream_t st);
 
@@ -154,6 +163,9 @@ int conv_fwd(const aprnet_plan* cp, int d, int kz, int kx, int ky, const T* x, i
     a.apr = p->dapr; a.tree = p->dtree; a.tiles = tl.d_tiles;
     a.x = x; a.ldx = ldx; a.Cin = Cin; a.w = w; a.S_exp = S_exp; a.Cout = Cout; a.y = y; a.ldy = ldy;
     a.tree_data = tree_ws; a.ldt = ldt; a.Lc = p->lc(d); a.tree_off = p->tree_offset(a.Lc);
+    bool done = false;
+    if (int rc = try_mfma<T>(a, code, tl.n, st, &done)) return rc;
+    if (done) return 0;
     // few output channels per thread keep the wave-uniform weights within the scalar register file;
     // wider layers run more blocks along grid.y (each re-stages its patch)
     switch (code) {
@@ -170,6 +182,11 @@ int conv_fwd(const aprnet_plan* cp, int d, int kz, int kx, int ky, const T* x, i
 using namespace aprnet;
 
 extern "C" {
+int aprnet_set_conv_path(int path) {
+    if (path != 0 && path != 1) return fail(APRNET_ERR_INVALID_ARGUMENT, "set_conv_path: 0 (auto) or 1 (VALU only)");
+    g_conv_path = path;
+    return 0;
+}
 int aprnet_profile_enable(int on) { g_timer.enabled = on != 0; g_timer.armed = false; return 0; }
 float aprnet_profile_last_ms(void) {
     if (!g_timer.armed) return -1.0f;

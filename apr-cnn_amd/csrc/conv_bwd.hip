@@ -33,18 +33,11 @@ static void fill2d(T* p, int64_t ld, int64_t n, int rows, T v, hipStream_t st) {
 // Transpose of stage_values: add the gradient patch back to its sources.
 template <class G, typename T, int CIB>
 __device__ __forceinline__ void flush_values(const ConvArgs<T>& a, int L, int y0, int ci0, const ConvShared<G>& sh,
-                                             const int (&yv)[G::SPW], unsigned long long inw, const T* gpatch) {
-    const int wave = threadIdx.x >> 6, lane = lane_id();
+                                             const T* gpatch) {
     const int lo = y0 - G::HY, hi = y0 + G::TY + G::HY;
     const int yn = a.apr.y_num[L];
     const bool tree_in_x = (L == a.Lc);
-#pragma unroll
-    for (int k = 0; k < G::SPW; ++k) {
-        if (!((inw >> k) & 1ull)) continue;
-        const int s = wave + k * G::NWAVE;
-        const int r = s / 3, src = s - 3 * r;
-        const int64_t i = sh.seg_cur[s] + lane;
-        const int yy = yv[k];
+    for_window_particles<G, T>(a, sh, [&](int r, int src, int i, int yy) {
         T* base;
         int64_t ld;
         if (src == 2 && !tree_in_x) { base = a.gtree + i; ld = a.ldgt; }
@@ -64,7 +57,7 @@ __device__ __forceinline__ void flush_values(const ConvArgs<T>& a, int L, int y0
             }
             if (v != (T)0) atomicAdd(base + (int64_t)(ci0 + c) * ld, v);
         }
-    }
+    });
 }
 
 template <typename T, class G, int CIB, int COBLK>
@@ -86,10 +79,8 @@ conv_bwd_dx_kernel(const ConvArgs<T> a) {
     open_segments<G, T>(a, L, z0, x0, sh);
     __syncthreads();
 
-    int yv[G::SPW];
-    unsigned long long inw;
     for (int y0 = 0; y0 < yn; y0 += G::TY) {
-        scan_window<G, T>(a, L, y0, out_tree, sh, yv, inw);
+        scan_window<G, T>(a, L, y0, out_tree, sh);
         __syncthreads();
         const int nc = sh.ncol;
         if (nc > 0) {
@@ -136,10 +127,10 @@ conv_bwd_dx_kernel(const ConvArgs<T> a) {
                                           g[c][(sz * G::KX + sx) * G::KY + sy]);
             }
             __syncthreads();
-            flush_values<G, T, CIB>(a, L, y0, ci0, sh, yv, inw, gpatch);
+            flush_values<G, T, CIB>(a, L, y0, ci0, sh, gpatch);
         }
         __syncthreads();
-        advance_cursors<G, T>(y0, sh, yv);
+        advance_cursors<G>(sh);
         __syncthreads();
     }
 }
@@ -148,7 +139,6 @@ template <typename T, class G, int CIB, int COB>
 __global__ void __launch_bounds__(G::NT)
 conv_bwd_dw_kernel(const ConvArgs<T> a) {
     static_assert(CIB * COB <= G::NT, "one thread per (co, ci) pair");
-    static_assert(G::SPW <= 64, "in-window mask holds one bit per segment of a wave");
     constexpr int DOS_LD = COB + 1;
     __shared__ T patch[CIB * G::CH_STRIDE];
     __shared__ T dOs[G::MAXCOL * DOS_LD];
@@ -181,10 +171,8 @@ conv_bwd_dw_kernel(const ConvArgs<T> a) {
         open_segments<G, T>(a, L, z0, x0, sh);
         __syncthreads();
 
-        int yv[G::SPW];
-        unsigned long long inw;
         for (int y0 = 0; y0 < yn; y0 += G::TY) {
-            scan_window<G, T>(a, L, y0, out_tree, sh, yv, inw);
+            scan_window<G, T>(a, L, y0, out_tree, sh);
             __syncthreads();
             const int nc = sh.ncol;
             if (nc > 0) {
@@ -195,7 +183,7 @@ conv_bwd_dw_kernel(const ConvArgs<T> a) {
                     dOs[cc * DOS_LD + co] = a.gy[(int64_t)(co0 + co) * a.ldy + sh.col_idx[cc]];
                 }
                 __syncthreads();
-                stage_values<G, T, CIB>(a, L, y0, ci0, sh, yv, inw, patch);
+                stage_values<G, T, CIB>(a, L, y0, ci0, sh, patch);
                 __syncthreads();
                 if (worker) {
                     const T* pch = patch + pc * G::CH_STRIDE - G::TAP0;
@@ -213,7 +201,7 @@ conv_bwd_dw_kernel(const ConvArgs<T> a) {
                 }
             }
             __syncthreads();
-            advance_cursors<G, T>(y0, sh, yv);
+            advance_cursors<G>(sh);
             __syncthreads();
         }
     }

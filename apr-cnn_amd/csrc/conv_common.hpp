@@ -46,7 +46,6 @@ struct ConvGeom {
     static constexpr int NSEG = NROW * 3;
     static constexpr int NWAVE = NT / 64;
     static constexpr int SPW = (NSEG + NWAVE - 1) / NWAVE;     // segments per wave
-    static_assert(SPW <= 64, "the in-window mask holds one bit per segment of a wave");
     static constexpr int MAXCOL = TZ * TX * TY;
     static constexpr int ITER = (MAXCOL + NT - 1) / NT;        // output columns per thread
     static constexpr int CH_STRIDE = NROW * WY;                // patch elements per channel
@@ -58,12 +57,16 @@ __device__ __forceinline__ int lane_id() { return __lane_id(); }
 // Per-block bookkeeping kept in LDS.
 template <class G>
 struct ConvShared {
-    int seg_cur[G::NSEG];
+    int seg_cur[G::NSEG];            // cursor: first particle of the segment that can fall into the current window
     int seg_end[G::NSEG];
-    int col_idx[G::MAXCOL];
-    unsigned short col_pos[G::MAXCOL];
+    int seg_next[G::NSEG];           // cursor for the next window
+    unsigned char seg_nin[G::NSEG];  // particles of the segment inside the current window (a prefix of the 64 lanes)
+    int col_idx[G::MAXCOL];          // output positions of the window: feature index ...
+    unsigned short col_pos[G::MAXCOL];   // ... and centre cell inside one channel of the patch
     int ncol;
 };
+
+__device__ __forceinline__ int uniform(int v) { return __builtin_amdgcn_readfirstlane(v); }
 
 // Opens the 3 * NROW segments of a tile.
 template <class G, typename T>
@@ -95,30 +98,29 @@ __device__ __forceinline__ void open_segments(const ConvArgs<T>& a, int L, int z
     if (threadIdx.x == 0) sh.ncol = 0;
 }
 
-// Phase A of a window: every wave loads y_vec at the cursor of its segments, decides which lanes
-// hold in-window particles and appends the output positions (particles of the centre rows, plus
-// tree nodes when they are downsampled particles) to the column list.
-// yv[k] : y of the particle in this lane (own coordinates), or INT_MAX
-// inw   : bit k set <=> lane holds an in-window particle of its k-th segment
+// Phase A of a window.  Every wave loads y_vec at the cursor of its segments (64 lanes = every particle
+// that can fall into the 64-cell window), and from ballots over "y < bound" derives the number of
+// in-window particles (they are the first n lanes, y ascends) and the cursor of the next window.
+// Particles of the centre rows (plus tree nodes when they are downsampled particles) whose y lies in the
+// output range are appended to the column list.
 template <class G, typename T>
-__device__ __forceinline__ void scan_window(const ConvArgs<T>& a, int L, int y0, bool out_tree, ConvShared<G>& sh,
-                                            int (&yv)[G::SPW], unsigned long long& inw) {
+__device__ __forceinline__ void scan_window(const ConvArgs<T>& a, int L, int y0, bool out_tree, ConvShared<G>& sh) {
     const int wave = threadIdx.x >> 6, lane = lane_id();
-    const int lo = y0 - G::HY, hi = y0 + G::TY + G::HY;
-    inw = 0;
-#pragma unroll
+    const int lo = y0 - G::HY, hi = y0 + G::TY + G::HY, lo_next = y0 + G::TY - G::HY;
+#pragma unroll 6
     for (int k = 0; k < G::SPW; ++k) {
         const int s = wave + k * G::NWAVE;
-        yv[k] = INT_MAX;
-        if (s >= G::NSEG) continue;
+        if (s >= G::NSEG) break;
         const int r = s / 3, src = s - 3 * r;
-        const int i = sh.seg_cur[s] + lane;
+        const int cur = sh.seg_cur[s];
+        const int i = cur + lane;
         const bool valid = i < sh.seg_end[s];
         int yy = INT_MAX;
         if (valid) yy = (src == 2) ? (int)a.tree.y[i] : (int)a.apr.y[i];
         const bool in = valid && (src == 1 ? yy <= ((hi - 1) >> 1) : yy < hi);
-        yv[k] = yy;
-        if (in) inw |= 1ull << k;
+        const bool below = valid && (src == 1 ? yy < (lo_next >> 1) : yy < lo_next);
+        const int n_in = __popcll(__ballot(in)), n_adv = __popcll(__ballot(below));
+        if (lane == 0) { sh.seg_nin[s] = (unsigned char)n_in; sh.seg_next[s] = cur + n_adv; }
         const int rz = r / G::RX, rx = r - rz * G::RX;
         const bool centre = rz >= G::HZ && rz < G::HZ + G::TZ && rx >= G::HX && rx < G::HX + G::TX;
         const bool out_seg = centre && (src == 0 || (src == 2 && out_tree));
@@ -137,56 +139,61 @@ __device__ __forceinline__ void scan_window(const ConvArgs<T>& a, int L, int y0,
     }
 }
 
-// Phase C: move every cursor to the first particle that can fall into the next window.
-template <class G, typename T>
-__device__ __forceinline__ void advance_cursors(int y0, ConvShared<G>& sh, const int (&yv)[G::SPW]) {
+// Phase C: commit the cursors of the next window.
+template <class G>
+__device__ __forceinline__ void advance_cursors(ConvShared<G>& sh) {
+    for (int s = threadIdx.x; s < G::NSEG; s += G::NT) sh.seg_cur[s] = sh.seg_next[s];
+    if (threadIdx.x == 0) sh.ncol = 0;
+}
+
+// Walks the in-window particles of the wave's segments: f(r, src, i, yy) per lane that holds one.
+// The y of a particle is re-read here (it is hot in the cache) instead of being kept in registers
+// between the phases; the value loads do not depend on it, so both are issued together.
+template <class G, typename T, class F>
+__device__ __forceinline__ void for_window_particles(const ConvArgs<T>& a, const ConvShared<G>& sh, F f) {
     const int wave = threadIdx.x >> 6, lane = lane_id();
-    const int lo_next = y0 + G::TY - G::HY;
-#pragma unroll
+#pragma unroll 6
     for (int k = 0; k < G::SPW; ++k) {
         const int s = wave + k * G::NWAVE;
-        if (s >= G::NSEG) continue;
-        const int src = s % 3;
-        const bool below = yv[k] != INT_MAX && (src == 1 ? yv[k] < (lo_next >> 1) : yv[k] < lo_next);
-        const int cnt = __popcll(__ballot(below));
-        if (lane == 0 && cnt) sh.seg_cur[s] += cnt;
+        if (s >= G::NSEG) break;
+        if (lane < (int)sh.seg_nin[s]) {
+            const int r = s / 3, src = s - 3 * r;
+            const int i = sh.seg_cur[s] + lane;
+            const int yy = (src == 2) ? (int)a.tree.y[i] : (int)a.apr.y[i];
+            f(r, src, i, yy);
+        }
     }
-    if (threadIdx.x == 0) sh.ncol = 0;
 }
 
 // Gather of one channel chunk into the (already zeroed) patch.
 template <class G, typename T, int CIB>
 __device__ __forceinline__ void stage_values(const ConvArgs<T>& a, int L, int y0, int ci0, const ConvShared<G>& sh,
-                                             const int (&yv)[G::SPW], unsigned long long inw, T* patch) {
-    const int wave = threadIdx.x >> 6, lane = lane_id();
+                                             T* patch) {
     const int lo = y0 - G::HY, hi = y0 + G::TY + G::HY;
     const int yn = a.apr.y_num[L];
     const bool tree_from_x = (L == a.Lc);
-#pragma unroll
-    for (int k = 0; k < G::SPW; ++k) {
-        if (!((inw >> k) & 1ull)) continue;
-        const int s = wave + k * G::NWAVE;
-        const int r = s / 3, src = s - 3 * r;
-        const int64_t i = sh.seg_cur[s] + lane;
-        const int yy = yv[k];
+    for_window_particles<G, T>(a, sh, [&](int r, int src, int i, int yy) {
         const T* base;
         int64_t ld;
         if (src == 2 && !tree_from_x) { base = a.tree_data + i; ld = a.ldt; }
         else { base = a.x + i + (src == 2 ? a.tree_off : 0); ld = a.ldx; }
-        T* prow = patch + r * G::WY;
+        T v[CIB];
 #pragma unroll
-        for (int c = 0; c < CIB; ++c) {
-            if (ci0 + c >= a.Cin) break;
-            const T v = base[(int64_t)(ci0 + c) * ld];
-            if (src != 1) {
-                prow[c * G::CH_STRIDE + (yy - lo)] = v;
-            } else {
-                const int ya = 2 * yy, yb = ya + 1;
-                if (ya >= lo && ya < hi) prow[c * G::CH_STRIDE + (ya - lo)] = v;
-                if (yb >= lo && yb < hi && yb < yn) prow[c * G::CH_STRIDE + (yb - lo)] = v;
+        for (int c = 0; c < CIB; ++c) v[c] = (ci0 + c < a.Cin) ? base[(int64_t)(ci0 + c) * ld] : (T)0;
+        T* prow = patch + r * G::WY;
+        if (src != 1) {
+#pragma unroll
+            for (int c = 0; c < CIB; ++c) prow[c * G::CH_STRIDE + (yy - lo)] = v[c];
+        } else {
+            const int ya = 2 * yy, yb = ya + 1;
+            const bool wa = ya >= lo && ya < hi, wb = yb >= lo && yb < hi && yb < yn;
+#pragma unroll
+            for (int c = 0; c < CIB; ++c) {
+                if (wa) prow[c * G::CH_STRIDE + (ya - lo)] = v[c];
+                if (wb) prow[c * G::CH_STRIDE + (yb - lo)] = v[c];
             }
         }
-    }
+    });
 }
 
 }  // namespace aprnet

@@ -1,0 +1,148 @@
+// Stencil convolution forward on the matrix cores (fp32 MFMA), gfx950.
+//
+// Same tiles, windows and three-source LDS gather as the VALU path (conv_common.hpp); only the
+// contraction differs.  For one window the block holds nc output positions ("columns").  The
+// contraction  out[co][col] = sum_{ci,t} W[co][ci][t] * patch[ci][pos(col) + off(t)]  is an implicit
+// GEMM with M = 32 output channels, N = columns, K = (tap, input channel):
+//
+//     v_mfma_f32_32x32x2_f32:  D[32x32] += A[32x2] * B[2x32]
+//       A: lane l supplies W[co = l%32][k = l/32]        B: lane l supplies patch value of column l%32, k = l/32
+//       the two k of one instruction are the two input channels of a pair (ci = 2p, 2p+1), same tap
+//
+// so every lane owns one column and one channel parity: its B operand for step (p, t) sits at a fixed
+// per-lane LDS address plus a compile-time offset (channel-pair stride + tap offset), and its A operand
+// likewise in a transposed, padded weight chunk Wl[(c*K + t)][co] that is staged per channel chunk.
+// The K loop is fully unrolled: two ds_read_b32 with immediate offsets and one MFMA per step and column
+// block, no address arithmetic.  Columns are cut into blocks of 32; wave w owns blocks b with
+// (b + rotation) % 4 == w, up to NBW of them, and keeps their 32x32 accumulators in registers across all
+// channel chunks, so each output element is written once (no atomics, deterministic).
+#include "conv_common.hpp"
+
+namespace aprnet {
+
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+
+template <class G>
+__device__ __forceinline__ constexpr int tap_offset(int t) {
+    return ((t / (G::KX * G::KY)) * G::RX + (t / G::KY) % G::KX) * G::WY + (t % G::KY);
+}
+
+// One window for a block whose waves own NB column blocks each (NB = ceil(#blocks / 4), the same for
+// all waves, so every wave runs the same barrier sequence; a wave whose last block does not exist
+// multiplies zeros, which costs nothing extra because it would otherwise wait at the barrier).
+template <class G, int CIB, int NB>
+__device__ __forceinline__ void mfma_window(const ConvArgs<float>& a, int L, int y0, int co0, int nc, int first,
+                                            const float* __restrict__ wl, const ConvShared<G>& sh,
+                                            float* __restrict__ patch, float* __restrict__ Wl) {
+    constexpr int WLD = 33;                    // padded row of the transposed weight chunk
+    constexpr int KC = CIB * G::K;             // k rows per chunk
+    const int lane = lane_id();
+    int bbase[NB];
+#pragma unroll
+    for (int j = 0; j < NB; ++j) {
+        const int col = ((first + 4 * j) << 5) + (lane & 31);
+        const int pos = col < nc ? (int)sh.col_pos[col] - G::TAP0 : 0;
+        bbase[j] = pos + (lane >> 5) * G::CH_STRIDE;
+    }
+    floatx16 acc[NB];
+#pragma unroll
+    for (int j = 0; j < NB; ++j)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[j][r] = 0.f;
+    const float* ap = Wl + (lane >> 5) * G::K * WLD + (lane & 31);
+
+    for (int ci0 = 0; ci0 < a.Cin; ci0 += CIB) {
+        for (int i = threadIdx.x; i < CIB * G::CH_STRIDE; i += G::NT) patch[i] = 0.f;
+        // weight chunk, transposed: Wl[(c*K + t) * WLD + co] = w[co0+co][ci0+c][t]; for a fixed co the
+        // (c, t) run is contiguous in global memory
+        for (int i = threadIdx.x; i < 32 * KC; i += G::NT) {
+            const int co = i / KC, j = i - co * KC;
+            const int ci = ci0 + j / G::K;
+            float v = 0.f;
+            if (co0 + co < a.Cout && ci < a.Cin) v = wl[((int64_t)(co0 + co) * a.Cin + ci0) * G::K + j];
+            Wl[j * WLD + co] = v;
+        }
+        __syncthreads();
+        stage_values<G, float, CIB>(a, L, y0, ci0, sh, patch);
+        __syncthreads();
+#pragma unroll
+        for (int p = 0; p < CIB / 2; ++p) {
+#pragma unroll
+            for (int t = 0; t < G::K; ++t) {
+                const float av = ap[(2 * p * G::K + t) * WLD];
+#pragma unroll
+                for (int j = 0; j < NB; ++j) {
+                    const float bv = patch[bbase[j] + 2 * p * G::CH_STRIDE + tap_offset<G>(t)];
+                    acc[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(av, bv, acc[j], 0, 0, 0);
+                }
+            }
+        }
+        __syncthreads();
+    }
+    // D layout: lane l, register r -> column l%32, row 8*(r/4) + 4*(l/32) + r%4
+#pragma unroll
+    for (int j = 0; j < NB; ++j) {
+        const int col = ((first + 4 * j) << 5) + (lane & 31);
+        if (col >= nc) continue;
+        const int64_t o = sh.col_idx[col];
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const int co = co0 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+            if (co < a.Cout) a.y[(int64_t)co * a.ldy + o] = acc[j][r];
+        }
+    }
+}
+
+template <class G, int CIB, int NBW>
+__global__ void __launch_bounds__(G::NT)
+conv_fwd_mfma_kernel(const ConvArgs<float> a) {
+    static_assert(CIB % 2 == 0, "input channels are consumed in pairs");
+    static_assert(G::NWAVE == 4, "block assignment assumes four waves");
+    static_assert(NBW == 4 && (G::MAXCOL + 31) / 32 <= 4 * NBW, "a window must fit the accumulators of the block");
+    __shared__ float patch[CIB * G::CH_STRIDE];
+    __shared__ float Wl[CIB * G::K * 33];
+    __shared__ ConvShared<G> sh;
+
+    const ConvTile tile = a.tiles[blockIdx.x];
+    const int L = tile.level, z0 = tile.z0, x0 = tile.x0;
+    const int co0 = blockIdx.y * 32;
+    const int yn = a.apr.y_num[L];
+    const int s_idx = min(a.S_exp - 1, a.Lc - L);
+    const bool out_tree = (L == a.Lc) && (L < a.apr.level_max);
+    const float* __restrict__ wl = a.w + (int64_t)s_idx * a.Cout * a.Cin * G::K;
+    const int wave = threadIdx.x >> 6;
+
+    open_segments<G, float>(a, L, z0, x0, sh);
+    __syncthreads();
+
+    int win = 0;
+    for (int y0 = 0; y0 < yn; y0 += G::TY, ++win) {
+        scan_window<G, float>(a, L, y0, out_tree, sh);
+        __syncthreads();
+        const int nc = __builtin_amdgcn_readfirstlane(sh.ncol);
+        if (nc > 0) {
+            const int nblk = (nc + 31) >> 5;
+            const int first = (wave - (int)blockIdx.x - win) & 3;      // rotation: spread the partial blocks over the SIMDs
+            switch ((nblk + 3) >> 2) {
+                case 1: mfma_window<G, CIB, 1>(a, L, y0, co0, nc, first, wl, sh, patch, Wl); break;
+                case 2: mfma_window<G, CIB, 2>(a, L, y0, co0, nc, first, wl, sh, patch, Wl); break;
+                case 3: mfma_window<G, CIB, 3>(a, L, y0, co0, nc, first, wl, sh, patch, Wl); break;
+                default: mfma_window<G, CIB, 4>(a, L, y0, co0, nc, first, wl, sh, patch, Wl); break;
+            }
+        }
+        __syncthreads();
+        advance_cursors<G>(sh);
+        __syncthreads();
+    }
+}
+
+using M333 = ConvGeom<3, 3, 3, 2, 4, 256>;
+
+int launch_conv333_mfma(const ConvArgs<float>& a, int n_tiles, hipStream_t st) {
+    dim3 grid((unsigned)n_tiles, (unsigned)((a.Cout + 31) / 32));
+    hipLaunchKernelGGL((conv_fwd_mfma_kernel<M333, 4, 4>), grid, dim3(M333::NT), 0, st, a);
+    APRNET_LAUNCH_CHECK("conv_fwd_mfma_kernel");
+    return 0;
+}
+
+}  // namespace aprnet

@@ -74,6 +74,7 @@ def hip():
         getattr(lib, fn).argtypes = [vp, i32]
     lib.aprnet_plan_children.argtypes = [vp, vp]
     lib.aprnet_profile_enable.argtypes = [i32]
+    lib.aprnet_set_conv_path.argtypes = [i32]
     lib.aprnet_profile_last_ms.restype = C.c_float
     for t in ("f32", "f64"):
         getattr(lib, f"aprnet_fill_tree_mean_{t}").argtypes = [vp, i32, vp, i64, i32, vp, i64, vp]

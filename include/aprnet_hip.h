@@ -77,6 +77,10 @@ int aprnet_plan_children(const aprnet_plan* plan, int32_t* out_host);
  * the call's stream; aprnet_profile_last_ms() waits for the last bracket and returns its duration in
  * milliseconds (-1 if none).  Process-wide, not thread-safe; meant for benchmarks. */
 int aprnet_profile_enable(int on);
+/* No counterpart in the reference.  Selects the forward convolution kernels: 0 = matrix-core (MFMA) kernels
+ * where one exists for the stencil and element type, VALU kernels otherwise (default); 1 = VALU kernels only.
+ * Both are HIP kernels; the switch exists so that tests can cover both. */
+int aprnet_set_conv_path(int path);
 float aprnet_profile_last_ms(void);
 
 #define APRNET_DECL(T, SFX)                                                                                          \

@@ -146,14 +146,41 @@ def test_conv_forward(bt, ksize, dtype):
     close(got, ref, dtype)
 
 
-@pytest.mark.parametrize("cin,cout", [(1, 16), (32, 32), (33, 33), (16, 3)])
-def test_conv333_forward_channel_shapes(cin, cout):
+@pytest.mark.parametrize("path", [0, 1], ids=["mfma", "valu"])
+@pytest.mark.parametrize("cin,cout", [(1, 16), (32, 32), (33, 33), (16, 3), (64, 40)])
+def test_conv333_forward_channel_shapes(cin, cout, path):
     """Channel counts of the benchmark configurations and of the reference's CUDA-vs-CPU test
-    (33 -> 33, pyapr/tests/test_aprnet.py:137-138)."""
+    (33 -> 33, pyapr/tests/test_aprnet.py:137-138), on both fp32 kernels (matrix cores / VALU)."""
     x, aprs, ld, w_exp = _conv_case([("3d_s", 0), ("3d_t", 1)], (3, 3, 3), 2, cin, cout, torch.float32)
     ref = oracle.conv_forward(aprs, x, w_exp, ld)
-    got = _ops.conv_forward(aprs, x.to(DEV), w_exp.permute(1, 2, 0, 3, 4, 5).contiguous().to(DEV), ld)
+    lib = _native.hip()
+    assert lib.aprnet_set_conv_path(path) == 0
+    try:
+        got = _ops.conv_forward(aprs, x.to(DEV), w_exp.permute(1, 2, 0, 3, 4, 5).contiguous().to(DEV), ld)
+    finally:
+        lib.aprnet_set_conv_path(0)
     close(got, ref, torch.float32)
+
+
+def test_conv333_forward_dense_windows():
+    """A fully refined APR: every window holds the maximum number of output positions (all four column
+    blocks per wave of the matrix-core kernel), plus run-to-run bit equality (no atomics in the forward)."""
+    import numpy as np
+    from pyapr import APR
+    shape = (6, 10, 140)
+    apr = APR.from_level_field(shape, np.full(tuple((s + 1) // 2 for s in shape), 8, np.uint8))
+    assert apr.total_number_particles() == 6 * 10 * 140
+    g = torch.Generator().manual_seed(4)
+    x = torch.randn(1, 6, apr.total_number_particles(), generator=g)
+    w = torch.randn(6, 1, 10, 3, 3, 3, generator=g)
+    ld = torch.zeros(1, dtype=torch.int32)
+    w_exp = oracle.restrict_kernel_forward(w, apr.level_max() - apr.level_min() + 1)
+    ref = oracle.conv_forward([apr], x, w_exp, ld)
+    wd = w_exp.permute(1, 2, 0, 3, 4, 5).contiguous().to(DEV)
+    got = _ops.conv_forward([apr], x.to(DEV), wd, ld)
+    close(got, ref, torch.float32)
+    again = _ops.conv_forward([apr], x.to(DEV), wd, ld)
+    assert torch.equal(got, again)
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
