@@ -32,18 +32,18 @@ conv_fwd_kernel(const ConvArgs<T> a) {
     for (int y0 = 0; y0 < yn; y0 += G::TY) {
         scan_window<G, T>(a, L, y0, out_tree, sh);
         __syncthreads();
-        const int nc = sh.ncol;
+        const int nc = sh.ncol, nitem = sh.nitem;
         if (nc > 0) {
             T acc[G::ITER][COB];
 #pragma unroll
             for (int it = 0; it < G::ITER; ++it)
 #pragma unroll
                 for (int co = 0; co < COB; ++co) acc[it][co] = 0;
+            for (int i = threadIdx.x; i < CIB * G::CH_STRIDE; i += G::NT) patch[i] = 0;
 
             for (int ci0 = 0; ci0 < a.Cin; ci0 += CIB) {
-                for (int i = threadIdx.x; i < CIB * G::CH_STRIDE; i += G::NT) patch[i] = 0;
                 __syncthreads();
-                stage_values<G, T, CIB>(a, L, y0, ci0, sh, patch);
+                stage_values<G, T, CIB>(a, ci0, nitem, sh, patch);
                 __syncthreads();
 #pragma unroll
                 for (int it = 0; it < G::ITER; ++it) {
@@ -73,7 +73,6 @@ conv_fwd_kernel(const ConvArgs<T> a) {
                         }
                     }
                 }
-                __syncthreads();
             }
 #pragma unroll
             for (int it = 0; it < G::ITER; ++it) {
@@ -86,7 +85,7 @@ conv_fwd_kernel(const ConvArgs<T> a) {
             }
         }
         __syncthreads();
-        advance_cursors<G>(sh);
+        close_window<G>(sh);
         __syncthreads();
     }
 }

@@ -30,34 +30,24 @@ static void fill2d(T* p, int64_t ld, int64_t n, int rows, T v, hipStream_t st) {
     hipLaunchKernelGGL(fill_kernel<T>, grid, dim3(256), 0, st, p, ld, n, v);
 }
 
-// Transpose of stage_values: add the gradient patch back to its sources.
+// Transpose of stage_values: add the gradient patch back to its sources, item by item.
 template <class G, typename T, int CIB>
-__device__ __forceinline__ void flush_values(const ConvArgs<T>& a, int L, int y0, int ci0, const ConvShared<G>& sh,
+__device__ __forceinline__ void flush_values(const ConvArgs<T>& a, int ci0, int nitem, const ConvShared<G>& sh,
                                              const T* gpatch) {
-    const int lo = y0 - G::HY, hi = y0 + G::TY + G::HY;
-    const int yn = a.apr.y_num[L];
-    const bool tree_in_x = (L == a.Lc);
-    for_window_particles<G, T>(a, sh, [&](int r, int src, int i, int yy) {
-        T* base;
-        int64_t ld;
-        if (src == 2 && !tree_in_x) { base = a.gtree + i; ld = a.ldgt; }
-        else { base = a.gx + i + (src == 2 ? a.tree_off : 0); ld = a.ldgx; }
-        const T* prow = gpatch + r * G::WY;
+    for (int it = threadIdx.x; it < nitem; it += G::NT) {
+        const unsigned pos = sh.item_pos[it];
+        const int64_t idx = sh.item_idx[it];
+        T* base = (pos & ITEM_TREE) ? a.gtree + idx : a.gx + idx;
+        const int64_t ld = (pos & ITEM_TREE) ? a.ldgt : a.ldgx;
+        const T* cell = gpatch + (pos & ITEM_CELL);
 #pragma unroll
         for (int c = 0; c < CIB; ++c) {
             if (ci0 + c >= a.Cin) break;
-            T v;
-            if (src != 1) {
-                v = prow[c * G::CH_STRIDE + (yy - lo)];
-            } else {
-                const int ya = 2 * yy, yb = ya + 1;
-                v = 0;
-                if (ya >= lo && ya < hi) v += prow[c * G::CH_STRIDE + (ya - lo)];
-                if (yb >= lo && yb < hi && yb < yn) v += prow[c * G::CH_STRIDE + (yb - lo)];
-            }
+            T v = cell[c * G::CH_STRIDE];
+            if (pos & ITEM_PAIR) v += cell[c * G::CH_STRIDE + 1];
             if (v != (T)0) atomicAdd(base + (int64_t)(ci0 + c) * ld, v);
         }
-    });
+    }
 }
 
 template <typename T, class G, int CIB, int COBLK>
@@ -82,7 +72,7 @@ conv_bwd_dx_kernel(const ConvArgs<T> a) {
     for (int y0 = 0; y0 < yn; y0 += G::TY) {
         scan_window<G, T>(a, L, y0, out_tree, sh);
         __syncthreads();
-        const int nc = sh.ncol;
+        const int nc = sh.ncol, nitem = sh.nitem;
         if (nc > 0) {
             for (int i = threadIdx.x; i < CIB * G::CH_STRIDE; i += G::NT) gpatch[i] = 0;
             T g[CIB][G::K];
@@ -127,10 +117,10 @@ conv_bwd_dx_kernel(const ConvArgs<T> a) {
                                           g[c][(sz * G::KX + sx) * G::KY + sy]);
             }
             __syncthreads();
-            flush_values<G, T, CIB>(a, L, y0, ci0, sh, gpatch);
+            flush_values<G, T, CIB>(a, ci0, nitem, sh, gpatch);
         }
         __syncthreads();
-        advance_cursors<G>(sh);
+        close_window<G>(sh);
         __syncthreads();
     }
 }
@@ -174,7 +164,7 @@ conv_bwd_dw_kernel(const ConvArgs<T> a) {
         for (int y0 = 0; y0 < yn; y0 += G::TY) {
             scan_window<G, T>(a, L, y0, out_tree, sh);
             __syncthreads();
-            const int nc = sh.ncol;
+            const int nc = sh.ncol, nitem = sh.nitem;
             if (nc > 0) {
                 for (int i = threadIdx.x; i < CIB * G::CH_STRIDE; i += G::NT) patch[i] = 0;
                 const int nco = min(COB, a.Cout - co0);
@@ -183,7 +173,7 @@ conv_bwd_dw_kernel(const ConvArgs<T> a) {
                     dOs[cc * DOS_LD + co] = a.gy[(int64_t)(co0 + co) * a.ldy + sh.col_idx[cc]];
                 }
                 __syncthreads();
-                stage_values<G, T, CIB>(a, L, y0, ci0, sh, patch);
+                stage_values<G, T, CIB>(a, ci0, nitem, sh, patch);
                 __syncthreads();
                 if (worker) {
                     const T* pch = patch + pc * G::CH_STRIDE - G::TAP0;
@@ -201,7 +191,7 @@ conv_bwd_dw_kernel(const ConvArgs<T> a) {
                 }
             }
             __syncthreads();
-            advance_cursors<G>(sh);
+            close_window<G>(sh);
             __syncthreads();
         }
     }

@@ -47,6 +47,7 @@ struct ConvGeom {
     static constexpr int NWAVE = NT / 64;
     static constexpr int SPW = (NSEG + NWAVE - 1) / NWAVE;     // segments per wave
     static constexpr int MAXCOL = TZ * TX * TY;
+    static constexpr int MAXITEM = NROW * WY;                  // every staged cell is filled by at most one item
     static constexpr int ITER = (MAXCOL + NT - 1) / NT;        // output columns per thread
     static constexpr int CH_STRIDE = NROW * WY;                // patch elements per channel
     static constexpr int TAP0 = (HZ * RX + HX) * WY + HY;      // centre -> first tap
@@ -55,18 +56,29 @@ struct ConvGeom {
 __device__ __forceinline__ int lane_id() { return __lane_id(); }
 
 // Per-block bookkeeping kept in LDS.
+//
+// A window is described by two lists that phase A (scan_window) builds once and every channel chunk
+// reuses:
+//   items   every particle / tree node that falls into the staged window: where its value comes from
+//           (feature index, or tree index with ITEM_TREE) and which patch cell(s) it fills;
+//   columns the output positions: feature index and centre cell.
+// Staging a chunk is then a flat loop over the items with all lanes busy and every global load
+// independent of the others (one memory round trip per chunk), instead of one partially filled
+// 64-lane load per segment.
 template <class G>
 struct ConvShared {
-    int seg_cur[G::NSEG];            // cursor: first particle of the segment that can fall into the current window
+    int seg_cur[G::NSEG];            // cursor: first particle of the segment that can fall into the next window
     int seg_end[G::NSEG];
-    int seg_next[G::NSEG];           // cursor for the next window
-    unsigned char seg_nin[G::NSEG];  // particles of the segment inside the current window (a prefix of the 64 lanes)
-    int col_idx[G::MAXCOL];          // output positions of the window: feature index ...
-    unsigned short col_pos[G::MAXCOL];   // ... and centre cell inside one channel of the patch
-    int ncol;
+    int col_idx[G::MAXCOL];
+    unsigned short col_pos[G::MAXCOL];
+    int item_idx[G::MAXITEM];
+    unsigned short item_pos[G::MAXITEM];   // bits 0-11 cell inside one channel of the patch, ITEM_PAIR, ITEM_TREE
+    int ncol, nitem;
 };
 
-__device__ __forceinline__ int uniform(int v) { return __builtin_amdgcn_readfirstlane(v); }
+constexpr unsigned ITEM_CELL = 0x0fffu;   // first patch cell the value goes to
+constexpr unsigned ITEM_PAIR = 0x1000u;   // coarser particle: the value also fills the next cell
+constexpr unsigned ITEM_TREE = 0x2000u;   // value is read from the mean-filled tree, not from the features
 
 // Opens the 3 * NROW segments of a tile.
 template <class G, typename T>
@@ -95,105 +107,142 @@ __device__ __forceinline__ void open_segments(const ConvArgs<T>& a, int L, int z
         }
         sh.seg_cur[s] = b; sh.seg_end[s] = e;
     }
-    if (threadIdx.x == 0) sh.ncol = 0;
+    if (threadIdx.x == 0) { sh.ncol = 0; sh.nitem = 0; }
 }
+
+// Segments are scanned in groups of GRP: the y_vec loads of a group are issued before the first LDS
+// write of the group, so a group costs one memory round trip instead of one per segment.
+template <class G> struct SegGroup { static constexpr int GRP = G::SPW < 6 ? G::SPW : 6; };
 
 // Phase A of a window.  Every wave loads y_vec at the cursor of its segments (64 lanes = every particle
-// that can fall into the 64-cell window), and from ballots over "y < bound" derives the number of
-// in-window particles (they are the first n lanes, y ascends) and the cursor of the next window.
-// Particles of the centre rows (plus tree nodes when they are downsampled particles) whose y lies in the
-// output range are appended to the column list.
+// that can fall into the 64-cell window).  Ballots over "y < bound" give the number of in-window
+// particles (the first n lanes, y ascends) and the cursor of the next window, which is committed at
+// once.  In-window particles are appended to the item list; those of the centre rows (plus tree nodes
+// when they are downsampled particles) whose y lies in the output range also to the column list.
 template <class G, typename T>
 __device__ __forceinline__ void scan_window(const ConvArgs<T>& a, int L, int y0, bool out_tree, ConvShared<G>& sh) {
+    constexpr int GRP = SegGroup<G>::GRP;
     const int wave = threadIdx.x >> 6, lane = lane_id();
     const int lo = y0 - G::HY, hi = y0 + G::TY + G::HY, lo_next = y0 + G::TY - G::HY;
-#pragma unroll 6
-    for (int k = 0; k < G::SPW; ++k) {
-        const int s = wave + k * G::NWAVE;
-        if (s >= G::NSEG) break;
-        const int r = s / 3, src = s - 3 * r;
-        const int cur = sh.seg_cur[s];
-        const int i = cur + lane;
-        const bool valid = i < sh.seg_end[s];
-        int yy = INT_MAX;
-        if (valid) yy = (src == 2) ? (int)a.tree.y[i] : (int)a.apr.y[i];
-        const bool in = valid && (src == 1 ? yy <= ((hi - 1) >> 1) : yy < hi);
-        const bool below = valid && (src == 1 ? yy < (lo_next >> 1) : yy < lo_next);
-        const int n_in = __popcll(__ballot(in)), n_adv = __popcll(__ballot(below));
-        if (lane == 0) { sh.seg_nin[s] = (unsigned char)n_in; sh.seg_next[s] = cur + n_adv; }
-        const int rz = r / G::RX, rx = r - rz * G::RX;
-        const bool centre = rz >= G::HZ && rz < G::HZ + G::TZ && rx >= G::HX && rx < G::HX + G::TX;
-        const bool out_seg = centre && (src == 0 || (src == 2 && out_tree));
-        const bool outl = out_seg && in && yy >= y0 && yy < y0 + G::TY;
-        const unsigned long long m = __ballot(outl);
-        if (m) {
-            int base = 0;
-            if (lane == 0) base = atomicAdd(&sh.ncol, __popcll(m));
-            base = __shfl(base, 0);
-            if (outl) {
-                const int rank = __popcll(m & ((1ull << lane) - 1ull));
-                sh.col_idx[base + rank] = i + (src == 2 ? (int)a.tree_off : 0);
-                sh.col_pos[base + rank] = (unsigned short)(r * G::WY + (yy - lo));
-            }
-        }
-    }
-}
-
-// Phase C: commit the cursors of the next window.
-template <class G>
-__device__ __forceinline__ void advance_cursors(ConvShared<G>& sh) {
-    for (int s = threadIdx.x; s < G::NSEG; s += G::NT) sh.seg_cur[s] = sh.seg_next[s];
-    if (threadIdx.x == 0) sh.ncol = 0;
-}
-
-// Walks the in-window particles of the wave's segments: f(r, src, i, yy) per lane that holds one.
-// The y of a particle is re-read here (it is hot in the cache) instead of being kept in registers
-// between the phases; the value loads do not depend on it, so both are issued together.
-template <class G, typename T, class F>
-__device__ __forceinline__ void for_window_particles(const ConvArgs<T>& a, const ConvShared<G>& sh, F f) {
-    const int wave = threadIdx.x >> 6, lane = lane_id();
-#pragma unroll 6
-    for (int k = 0; k < G::SPW; ++k) {
-        const int s = wave + k * G::NWAVE;
-        if (s >= G::NSEG) break;
-        if (lane < (int)sh.seg_nin[s]) {
-            const int r = s / 3, src = s - 3 * r;
-            const int i = sh.seg_cur[s] + lane;
-            const int yy = (src == 2) ? (int)a.tree.y[i] : (int)a.apr.y[i];
-            f(r, src, i, yy);
-        }
-    }
-}
-
-// Gather of one channel chunk into the (already zeroed) patch.
-template <class G, typename T, int CIB>
-__device__ __forceinline__ void stage_values(const ConvArgs<T>& a, int L, int y0, int ci0, const ConvShared<G>& sh,
-                                             T* patch) {
-    const int lo = y0 - G::HY, hi = y0 + G::TY + G::HY;
     const int yn = a.apr.y_num[L];
     const bool tree_from_x = (L == a.Lc);
-    for_window_particles<G, T>(a, sh, [&](int r, int src, int i, int yy) {
-        const T* base;
-        int64_t ld;
-        if (src == 2 && !tree_from_x) { base = a.tree_data + i; ld = a.ldt; }
-        else { base = a.x + i + (src == 2 ? a.tree_off : 0); ld = a.ldx; }
-        T v[CIB];
+    for (int k0 = 0; k0 < G::SPW; k0 += GRP) {
+        int yy[GRP], cur[GRP];
 #pragma unroll
-        for (int c = 0; c < CIB; ++c) v[c] = (ci0 + c < a.Cin) ? base[(int64_t)(ci0 + c) * ld] : (T)0;
-        T* prow = patch + r * G::WY;
-        if (src != 1) {
-#pragma unroll
-            for (int c = 0; c < CIB; ++c) prow[c * G::CH_STRIDE + (yy - lo)] = v[c];
-        } else {
-            const int ya = 2 * yy, yb = ya + 1;
-            const bool wa = ya >= lo && ya < hi, wb = yb >= lo && yb < hi && yb < yn;
-#pragma unroll
-            for (int c = 0; c < CIB; ++c) {
-                if (wa) prow[c * G::CH_STRIDE + (ya - lo)] = v[c];
-                if (wb) prow[c * G::CH_STRIDE + (yb - lo)] = v[c];
+        for (int g = 0; g < GRP; ++g) {
+            const int s = wave + (k0 + g) * G::NWAVE;
+            yy[g] = INT_MAX; cur[g] = 0;
+            if (s < G::NSEG) {
+                cur[g] = sh.seg_cur[s];
+                const int i = cur[g] + lane;
+                if (i < sh.seg_end[s]) yy[g] = (s % 3 == 2) ? (int)a.tree.y[i] : (int)a.apr.y[i];
             }
         }
-    });
+#pragma unroll
+        for (int g = 0; g < GRP; ++g) {
+            const int s = wave + (k0 + g) * G::NWAVE;
+            if (s >= G::NSEG) break;
+            const int r = s / 3, src = s - 3 * r;
+            const bool valid = yy[g] != INT_MAX;
+            const bool in = valid && (src == 1 ? yy[g] <= ((hi - 1) >> 1) : yy[g] < hi);
+            const bool below = valid && (src == 1 ? yy[g] < (lo_next >> 1) : yy[g] < lo_next);
+            const unsigned long long m_in = __ballot(in);
+            const int n_adv = __popcll(__ballot(below));
+            if (lane == 0 && n_adv) sh.seg_cur[s] = cur[g] + n_adv;
+            if (m_in == 0) continue;                                    // wave-uniform
+            const int i = cur[g] + lane;
+            int ibase = 0;
+            if (lane == 0) ibase = atomicAdd(&sh.nitem, __popcll(m_in));
+            ibase = __shfl(ibase, 0);
+            if (in) {      // in-window lanes are lanes 0 .. n_in-1
+                unsigned pos;
+                if (src != 1) {
+                    pos = (unsigned)(r * G::WY + (yy[g] - lo));
+                    if (src == 2 && !tree_from_x) pos |= ITEM_TREE;
+                } else {
+                    const int ya = 2 * yy[g], yb = ya + 1;
+                    const bool wa = ya >= lo, wb = yb < hi && yb < yn;
+                    pos = (unsigned)(r * G::WY + ((wa ? ya : yb) - lo));
+                    if (wa && wb) pos |= ITEM_PAIR;
+                }
+                sh.item_idx[ibase + lane] = i + ((src == 2 && tree_from_x) ? (int)a.tree_off : 0);
+                sh.item_pos[ibase + lane] = (unsigned short)pos;
+            }
+            const int rz = r / G::RX, rx = r - rz * G::RX;
+            const bool centre = rz >= G::HZ && rz < G::HZ + G::TZ && rx >= G::HX && rx < G::HX + G::TX;
+            const bool out_seg = centre && (src == 0 || (src == 2 && out_tree));
+            const bool outl = out_seg && in && yy[g] >= y0 && yy[g] < y0 + G::TY;
+            const unsigned long long m = __ballot(outl);
+            if (m) {
+                int base = 0;
+                if (lane == 0) base = atomicAdd(&sh.ncol, __popcll(m));
+                base = __shfl(base, 0);
+                if (outl) {
+                    const int rank = __popcll(m & ((1ull << lane) - 1ull));
+                    sh.col_idx[base + rank] = i + (src == 2 ? (int)a.tree_off : 0);
+                    sh.col_pos[base + rank] = (unsigned short)(r * G::WY + (yy[g] - lo));
+                }
+            }
+        }
+    }
+}
+
+// End of a window: reset the list lengths (call between two barriers).
+template <class G>
+__device__ __forceinline__ void close_window(ConvShared<G>& sh) {
+    if (threadIdx.x == 0) { sh.ncol = 0; sh.nitem = 0; }
+}
+
+// Values of one channel chunk for the items of this thread, in registers.
+template <class G, typename T, int CIB>
+struct ItemRegs {
+    static constexpr int IPT = (G::MAXITEM + G::NT - 1) / G::NT;    // items per thread
+    T v[IPT][CIB];
+    unsigned short pos[IPT];
+};
+
+// Issues the loads of a chunk (no LDS writes: they may run ahead of the consumer of the patch).
+template <class G, typename T, int CIB>
+__device__ __forceinline__ void load_items(const ConvArgs<T>& a, int ci0, int nitem, const ConvShared<G>& sh,
+                                           ItemRegs<G, T, CIB>& R) {
+#pragma unroll
+    for (int k = 0; k < ItemRegs<G, T, CIB>::IPT; ++k) {
+        const int it = threadIdx.x + k * G::NT;
+        R.pos[k] = 0xffffu;
+        if (it < nitem) {
+            const unsigned pos = sh.item_pos[it];
+            const int64_t idx = sh.item_idx[it];
+            R.pos[k] = (unsigned short)pos;
+            const T* base = (pos & ITEM_TREE) ? a.tree_data + idx : a.x + idx;
+            const int64_t ld = (pos & ITEM_TREE) ? a.ldt : a.ldx;
+#pragma unroll
+            for (int c = 0; c < CIB; ++c) R.v[k][c] = (ci0 + c < a.Cin) ? base[(int64_t)(ci0 + c) * ld] : (T)0;
+        }
+    }
+}
+
+template <class G, typename T, int CIB>
+__device__ __forceinline__ void store_items(const ItemRegs<G, T, CIB>& R, T* patch) {
+#pragma unroll
+    for (int k = 0; k < ItemRegs<G, T, CIB>::IPT; ++k) {
+        if (R.pos[k] == 0xffffu) continue;
+        T* cell = patch + (R.pos[k] & ITEM_CELL);
+#pragma unroll
+        for (int c = 0; c < CIB; ++c) {
+            cell[c * G::CH_STRIDE] = R.v[k][c];
+            if (R.pos[k] & ITEM_PAIR) cell[c * G::CH_STRIDE + 1] = R.v[k][c];
+        }
+    }
+}
+
+// Gather of one channel chunk into the patch.  Cells that no item covers keep the zeros written once
+// per window (outside the image, or inside a particle two or more levels coarser, which a stencil of
+// half-width <= 2 never reads on a 2:1-balanced APR); covered cells are overwritten by every chunk.
+template <class G, typename T, int CIB>
+__device__ __forceinline__ void stage_values(const ConvArgs<T>& a, int ci0, int nitem, const ConvShared<G>& sh, T* patch) {
+    ItemRegs<G, T, CIB> R;
+    load_items<G, T, CIB>(a, ci0, nitem, sh, R);
+    store_items<G, T, CIB>(R, patch);
 }
 
 }  // namespace aprnet

@@ -31,7 +31,7 @@ __device__ __forceinline__ constexpr int tap_offset(int t) {
 // all waves, so every wave runs the same barrier sequence; a wave whose last block does not exist
 // multiplies zeros, which costs nothing extra because it would otherwise wait at the barrier).
 template <class G, int CIB, int NB>
-__device__ __forceinline__ void mfma_window(const ConvArgs<float>& a, int L, int y0, int co0, int nc, int first,
+__device__ __forceinline__ void mfma_window(const ConvArgs<float>& a, int co0, int nc, int nitem, int first,
                                             const float* __restrict__ wl, const ConvShared<G>& sh,
                                             float* __restrict__ patch, float* __restrict__ Wl) {
     constexpr int WLD = 33;                    // padded row of the transposed weight chunk
@@ -51,8 +51,9 @@ __device__ __forceinline__ void mfma_window(const ConvArgs<float>& a, int L, int
         for (int r = 0; r < 16; ++r) acc[j][r] = 0.f;
     const float* ap = Wl + (lane >> 5) * G::K * WLD + (lane & 31);
 
+    for (int i = threadIdx.x; i < CIB * G::CH_STRIDE; i += G::NT) patch[i] = 0.f;     // once per window
     for (int ci0 = 0; ci0 < a.Cin; ci0 += CIB) {
-        for (int i = threadIdx.x; i < CIB * G::CH_STRIDE; i += G::NT) patch[i] = 0.f;
+        __syncthreads();            // the previous chunk's MFMAs have read patch and Wl
         // weight chunk, transposed: Wl[(c*K + t) * WLD + co] = w[co0+co][ci0+c][t]; for a fixed co the
         // (c, t) run is contiguous in global memory
         for (int i = threadIdx.x; i < 32 * KC; i += G::NT) {
@@ -62,8 +63,7 @@ __device__ __forceinline__ void mfma_window(const ConvArgs<float>& a, int L, int
             if (co0 + co < a.Cout && ci < a.Cin) v = wl[((int64_t)(co0 + co) * a.Cin + ci0) * G::K + j];
             Wl[j * WLD + co] = v;
         }
-        __syncthreads();
-        stage_values<G, float, CIB>(a, L, y0, ci0, sh, patch);
+        stage_values<G, float, CIB>(a, ci0, nitem, sh, patch);
         __syncthreads();
 #pragma unroll
         for (int p = 0; p < CIB / 2; ++p) {
@@ -77,7 +77,6 @@ __device__ __forceinline__ void mfma_window(const ConvArgs<float>& a, int L, int
                 }
             }
         }
-        __syncthreads();
     }
     // D layout: lane l, register r -> column l%32, row 8*(r/4) + 4*(l/32) + r%4
 #pragma unroll
@@ -119,19 +118,19 @@ conv_fwd_mfma_kernel(const ConvArgs<float> a) {
     for (int y0 = 0; y0 < yn; y0 += G::TY, ++win) {
         scan_window<G, float>(a, L, y0, out_tree, sh);
         __syncthreads();
-        const int nc = __builtin_amdgcn_readfirstlane(sh.ncol);
+        const int nc = __builtin_amdgcn_readfirstlane(sh.ncol), nitem = __builtin_amdgcn_readfirstlane(sh.nitem);
         if (nc > 0) {
             const int nblk = (nc + 31) >> 5;
             const int first = (wave - (int)blockIdx.x - win) & 3;      // rotation: spread the partial blocks over the SIMDs
             switch ((nblk + 3) >> 2) {
-                case 1: mfma_window<G, CIB, 1>(a, L, y0, co0, nc, first, wl, sh, patch, Wl); break;
-                case 2: mfma_window<G, CIB, 2>(a, L, y0, co0, nc, first, wl, sh, patch, Wl); break;
-                case 3: mfma_window<G, CIB, 3>(a, L, y0, co0, nc, first, wl, sh, patch, Wl); break;
-                default: mfma_window<G, CIB, 4>(a, L, y0, co0, nc, first, wl, sh, patch, Wl); break;
+                case 1: mfma_window<G, CIB, 1>(a, co0, nc, nitem, first, wl, sh, patch, Wl); break;
+                case 2: mfma_window<G, CIB, 2>(a, co0, nc, nitem, first, wl, sh, patch, Wl); break;
+                case 3: mfma_window<G, CIB, 3>(a, co0, nc, nitem, first, wl, sh, patch, Wl); break;
+                default: mfma_window<G, CIB, 4>(a, co0, nc, nitem, first, wl, sh, patch, Wl); break;
             }
         }
         __syncthreads();
-        advance_cursors<G>(sh);
+        close_window<G>(sh);
         __syncthreads();
     }
 }

@@ -16,7 +16,8 @@ _hip = None
 
 
 def _load(name):
-    path = os.path.join(_CSRC, name)
+    # APRNET_LIB_DIR points at an alternative build of the two libraries (kernel experiments)
+    path = os.path.join(os.environ.get("APRNET_LIB_DIR", _CSRC), name)
     if not os.path.exists(path):
         raise ImportError(
             f"{name} is not built: run `python {os.path.join(_CSRC, 'build.py')}` "
