@@ -60,6 +60,7 @@ struct aprnet_plan {
     int32_t* d_children = nullptr;      // [8][n_tree], slot-major
     int64_t n_tree = 0, n_apr = 0;
     std::map<std::tuple<int, int, int>, aprnet::TileList> tiles;   // (level_delta, TZ, TX) -> non-empty row groups
+    void* d_scratch = nullptr; size_t scratch_bytes = 0;          // re-laid-out weights of the call in flight
 
     int lc(int level_delta) const { return apr.level_max - level_delta; }
     int64_t number_parts(int level_delta) const {

@@ -43,7 +43,7 @@ conv_fwd_kernel(const ConvArgs<T> a) {
 
             for (int ci0 = 0; ci0 < a.Cin; ci0 += CIB) {
                 __syncthreads();
-                stage_values<G, T, CIB>(a, ci0, nitem, sh, patch);
+                stage_values<G, T, CIB>(a, ci0, nitem, L < a.Lc, sh, patch);
                 __syncthreads();
 #pragma unroll
                 for (int it = 0; it < G::ITER; ++it) {
@@ -128,14 +128,27 @@ template <> struct Chunk<float>  { static constexpr int c333 = 8, c133 = 16, c15
 template <> struct Chunk<double> { static constexpr int c333 = 4, c133 = 8,  c155 = 6,  c555 = 2; };
 
 int launch_conv333_mfma(const ConvArgs<float>& a, int n_tiles, hipStream_t st);
+size_t conv333_packed_floats(int S_exp, int Cout, int Cin);
+int pack_conv333_weights(const float* w, int S_exp, int Cout, int Cin, float* packed, hipStream_t st);
 static int g_conv_path = 0;      // 0: matrix cores where available, 1: VALU kernels only
 
-template <typename T> static int try_mfma(const ConvArgs<T>&, int, int, hipStream_t, bool*) { return 0; }
-template <> int try_mfma<float>(const ConvArgs<float>& a, int code, int n_tiles, hipStream_t st, bool* done) {
+template <typename T> static int try_mfma(aprnet_plan*, const ConvArgs<T>&, int, int, hipStream_t, bool*) { return 0; }
+template <> int try_mfma<float>(aprnet_plan* p, const ConvArgs<float>& a, int code, int n_tiles, hipStream_t st, bool* done) {
     if (g_conv_path == 1 || code != 333) return 0;
     *done = true;
+    // plan-owned scratch for the re-laid-out weights, grown on demand
+    const size_t need = conv333_packed_floats(a.S_exp, a.Cout, a.Cin) * sizeof(float);
+    if (need > p->scratch_bytes) {
+        if (p->d_scratch) { APRNET_HIP_CHECK(hipStreamSynchronize(st)); APRNET_HIP_CHECK(hipFree(p->d_scratch)); }
+        p->d_scratch = nullptr; p->scratch_bytes = 0;
+        APRNET_HIP_CHECK(hipMalloc(&p->d_scratch, need));
+        p->scratch_bytes = need;
+    }
+    if (int rc = pack_conv333_weights(a.w, a.S_exp, a.Cout, a.Cin, (float*)p->d_scratch, st)) return rc;
+    ConvArgs<float> b = a;
+    b.w = (const float*)p->d_scratch;
     TimedLaunch timed(st);
-    return launch_conv333_mfma(a, n_tiles, st);
+    return launch_conv333_mfma(b, n_tiles, st);
 }
 
 int fill_tree_for_conv(const aprnet_plan* p, int d, const float* x, int64_t ldx, int C, float* tree, int64_t ldt, hipStream_t st);
@@ -162,8 +175,9 @@ int conv_fwd(const aprnet_plan* cp, int d, int kz, int kx, int ky, const T* x, i
     a.apr = p->dapr; a.tree = p->dtree; a.tiles = tl.d_tiles;
     a.x = x; a.ldx = ldx; a.Cin = Cin; a.w = w; a.S_exp = S_exp; a.Cout = Cout; a.y = y; a.ldy = ldy;
     a.tree_data = tree_ws; a.ldt = ldt; a.Lc = p->lc(d); a.tree_off = p->tree_offset(a.Lc);
+    a.x_count = p->number_parts(d); a.t_count = p->tree_parts(d);
     bool done = false;
-    if (int rc = try_mfma<T>(a, code, tl.n, st, &done)) return rc;
+    if (int rc = try_mfma<T>(p, a, code, tl.n, st, &done)) return rc;
     if (done) return 0;
     // few output channels per thread keep the wave-uniform weights within the scalar register file;
     // wider layers run more blocks along grid.y (each re-stages its patch)

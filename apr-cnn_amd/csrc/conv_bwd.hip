@@ -173,7 +173,7 @@ conv_bwd_dw_kernel(const ConvArgs<T> a) {
                     dOs[cc * DOS_LD + co] = a.gy[(int64_t)(co0 + co) * a.ldy + sh.col_idx[cc]];
                 }
                 __syncthreads();
-                stage_values<G, T, CIB>(a, ci0, nitem, sh, patch);
+                stage_values<G, T, CIB>(a, ci0, nitem, L < a.Lc, sh, patch);
                 __syncthreads();
                 if (worker) {
                     const T* pch = patch + pc * G::CH_STRIDE - G::TAP0;
@@ -250,6 +250,7 @@ int conv_bwd(const aprnet_plan* cp, int d, int kz, int kx, int ky, const T* x, i
         a.apr = p->dapr; a.tree = p->dtree; a.tiles = tl.d_tiles; a.n_tiles = tl.n;
         a.x = x; a.ldx = ldx; a.Cin = Cin; a.w = w; a.S_exp = S_exp; a.Cout = Cout;
         a.tree_data = tree_ws; a.ldt = ldt; a.Lc = p->lc(d); a.tree_off = p->tree_offset(a.Lc);
+    a.x_count = p->number_parts(d); a.t_count = p->tree_parts(d);
         a.gy = gy; a.ldy = ldy; a.gx = gx; a.ldgx = ldgx; a.gtree = gtree_ws; a.ldgt = ldgt; a.gw = gw;
         constexpr bool f32 = sizeof(T) == 4;
         int rc = 0;

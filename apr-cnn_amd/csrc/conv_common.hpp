@@ -30,6 +30,7 @@ struct ConvArgs {
     T* y; int64_t ldy;
     const T* tree_data; int64_t ldt;
     int Lc; int64_t tree_off;                  // tree_offset(Lc)
+    int64_t x_count, t_count;                  // valid elements per channel plane of x / tree_data
     // backward only
     const T* gy; T* gx; int64_t ldgx; T* gtree; int64_t ldgt; T* gw; int n_tiles;
 };
@@ -193,30 +194,68 @@ __device__ __forceinline__ void close_window(ConvShared<G>& sh) {
     if (threadIdx.x == 0) { sh.ncol = 0; sh.nitem = 0; }
 }
 
+// Buffer loads: the channel plane is described by a wave-uniform resource (base, size in bytes), the lane
+// supplies a 32-bit byte offset, and an offset outside the plane returns zero without touching memory.
+// That keeps the address registers to one per item and makes every predicate of the gather (item
+// exists / value lives in the tree buffer / channel exists) an out-of-range offset or an empty plane
+// instead of a branch.  plan_create limits an access to 2^29 particles so that offsets fit 32 bits.
+constexpr unsigned BUF_OOB = 0xffffffffu;
+
+template <typename T> struct RawLoad;
+template <> struct RawLoad<float> {
+    typedef int raw;
+    static __device__ __forceinline__ raw ld(__amdgpu_buffer_rsrc_t r, unsigned off) { return __builtin_amdgcn_raw_buffer_load_b32(r, (int)off, 0, 0); }
+    static __device__ __forceinline__ float cast(raw v) { return __builtin_bit_cast(float, v); }
+};
+template <> struct RawLoad<double> {
+    typedef int raw __attribute__((ext_vector_type(2)));
+    static __device__ __forceinline__ raw ld(__amdgpu_buffer_rsrc_t r, unsigned off) { return __builtin_amdgcn_raw_buffer_load_b64(r, (int)off, 0, 0); }
+    static __device__ __forceinline__ double cast(raw v) { return __builtin_bit_cast(double, v); }
+};
+
+template <typename T>
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t plane_rsrc(const T* base, int64_t ld, int c, int C, int64_t count) {
+    const int bytes = c < C ? (int)(count * (int64_t)sizeof(T)) : 0;      // a channel beyond C reads as zeros
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(base + (int64_t)c * ld), 0, bytes, 0x00020000);
+}
+
 // Values of one channel chunk for the items of this thread, in registers.
 template <class G, typename T, int CIB>
 struct ItemRegs {
     static constexpr int IPT = (G::MAXITEM + G::NT - 1) / G::NT;    // items per thread
-    T v[IPT][CIB];
+    typename RawLoad<T>::raw v[IPT][CIB];
     unsigned short pos[IPT];
 };
 
 // Issues the loads of a chunk (no LDS writes: they may run ahead of the consumer of the patch).
 template <class G, typename T, int CIB>
-__device__ __forceinline__ void load_items(const ConvArgs<T>& a, int ci0, int nitem, const ConvShared<G>& sh,
-                                           ItemRegs<G, T, CIB>& R) {
+__device__ __forceinline__ void load_items(const ConvArgs<T>& a, int ci0, int nitem, bool tree_items,
+                                           const ConvShared<G>& sh, ItemRegs<G, T, CIB>& R) {
+    constexpr int IPT = ItemRegs<G, T, CIB>::IPT;
+    unsigned offx[IPT], offt[IPT];
 #pragma unroll
-    for (int k = 0; k < ItemRegs<G, T, CIB>::IPT; ++k) {
+    for (int k = 0; k < IPT; ++k) {
         const int it = threadIdx.x + k * G::NT;
-        R.pos[k] = 0xffffu;
+        R.pos[k] = 0xffffu; offx[k] = BUF_OOB; offt[k] = BUF_OOB;
         if (it < nitem) {
             const unsigned pos = sh.item_pos[it];
-            const int64_t idx = sh.item_idx[it];
+            const unsigned off = (unsigned)sh.item_idx[it] * (unsigned)sizeof(T);
             R.pos[k] = (unsigned short)pos;
-            const T* base = (pos & ITEM_TREE) ? a.tree_data + idx : a.x + idx;
-            const int64_t ld = (pos & ITEM_TREE) ? a.ldt : a.ldx;
+            if (pos & ITEM_TREE) offt[k] = off; else offx[k] = off;
+        }
+    }
 #pragma unroll
-            for (int c = 0; c < CIB; ++c) R.v[k][c] = (ci0 + c < a.Cin) ? base[(int64_t)(ci0 + c) * ld] : (T)0;
+    for (int c = 0; c < CIB; ++c) {
+        const __amdgpu_buffer_rsrc_t rx = plane_rsrc<T>(a.x, a.ldx, ci0 + c, a.Cin, a.x_count);
+#pragma unroll
+        for (int k = 0; k < IPT; ++k) R.v[k][c] = RawLoad<T>::ld(rx, offx[k]);
+    }
+    if (tree_items) {      // tile-uniform: only levels below the current maximum read the mean-filled tree
+#pragma unroll
+        for (int c = 0; c < CIB; ++c) {
+            const __amdgpu_buffer_rsrc_t rt = plane_rsrc<T>(a.tree_data, a.ldt, ci0 + c, a.Cin, a.t_count);
+#pragma unroll
+            for (int k = 0; k < IPT; ++k) R.v[k][c] |= RawLoad<T>::ld(rt, offt[k]);
         }
     }
 }
@@ -229,8 +268,9 @@ __device__ __forceinline__ void store_items(const ItemRegs<G, T, CIB>& R, T* pat
         T* cell = patch + (R.pos[k] & ITEM_CELL);
 #pragma unroll
         for (int c = 0; c < CIB; ++c) {
-            cell[c * G::CH_STRIDE] = R.v[k][c];
-            if (R.pos[k] & ITEM_PAIR) cell[c * G::CH_STRIDE + 1] = R.v[k][c];
+            const T v = RawLoad<T>::cast(R.v[k][c]);
+            cell[c * G::CH_STRIDE] = v;
+            if (R.pos[k] & ITEM_PAIR) cell[c * G::CH_STRIDE + 1] = v;
         }
     }
 }
@@ -239,9 +279,10 @@ __device__ __forceinline__ void store_items(const ItemRegs<G, T, CIB>& R, T* pat
 // per window (outside the image, or inside a particle two or more levels coarser, which a stencil of
 // half-width <= 2 never reads on a 2:1-balanced APR); covered cells are overwritten by every chunk.
 template <class G, typename T, int CIB>
-__device__ __forceinline__ void stage_values(const ConvArgs<T>& a, int ci0, int nitem, const ConvShared<G>& sh, T* patch) {
+__device__ __forceinline__ void stage_values(const ConvArgs<T>& a, int ci0, int nitem, bool tree_items,
+                                             const ConvShared<G>& sh, T* patch) {
     ItemRegs<G, T, CIB> R;
-    load_items<G, T, CIB>(a, ci0, nitem, sh, R);
+    load_items<G, T, CIB>(a, ci0, nitem, tree_items, sh, R);
     store_items<G, T, CIB>(R, patch);
 }
 

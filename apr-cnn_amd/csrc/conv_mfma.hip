@@ -22,6 +22,25 @@ namespace aprnet {
 
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 
+// Weights are re-laid out once per call into the image the kernel keeps in LDS, so that staging a chunk
+// is a straight 16-byte copy:  packed[s][cb][q][(c*K + t)][co]  with co-blocks cb of 32 output channels and
+// chunks q of CIB input channels, zero where co or ci run past the layer.
+__global__ void pack_weights_kernel(const float* __restrict__ w, int S_exp, int Cout, int Cin, int K, int CIB,
+                                    float* __restrict__ out) {
+    const int ncb = (Cout + 31) / 32, nq = (Cin + CIB - 1) / CIB, KC = CIB * K;
+    const int64_t n = (int64_t)S_exp * ncb * nq * KC * 32;
+    for (int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; e < n; e += (int64_t)gridDim.x * blockDim.x) {
+        const int co = (int)(e % 32);
+        const int row = (int)((e / 32) % KC);
+        const int q = (int)((e / (32 * (int64_t)KC)) % nq);
+        const int cb = (int)((e / (32 * (int64_t)KC * nq)) % ncb);
+        const int s = (int)(e / (32 * (int64_t)KC * nq * ncb));
+        const int c = row / K, t = row - c * K;
+        const int ci = q * CIB + c, cog = cb * 32 + co;
+        out[e] = (ci < Cin && cog < Cout) ? w[(((int64_t)s * Cout + cog) * Cin + ci) * K + t] : 0.f;
+    }
+}
+
 template <class G>
 __device__ __forceinline__ constexpr int tap_offset(int t) {
     return ((t / (G::KX * G::KY)) * G::RX + (t / G::KY) % G::KX) * G::WY + (t % G::KY);
@@ -31,10 +50,10 @@ __device__ __forceinline__ constexpr int tap_offset(int t) {
 // all waves, so every wave runs the same barrier sequence; a wave whose last block does not exist
 // multiplies zeros, which costs nothing extra because it would otherwise wait at the barrier).
 template <class G, int CIB, int NB>
-__device__ __forceinline__ void mfma_window(const ConvArgs<float>& a, int co0, int nc, int nitem, int first,
-                                            const float* __restrict__ wl, const ConvShared<G>& sh,
+__device__ __forceinline__ void mfma_window(const ConvArgs<float>& a, int co0, int nc, int nitem, bool tree_items, int first,
+                                            const float4* __restrict__ wl, const ConvShared<G>& sh,
                                             float* __restrict__ patch, float* __restrict__ Wl) {
-    constexpr int WLD = 33;                    // padded row of the transposed weight chunk
+    constexpr int WLD = 32;                    // row of the weight chunk: 32 output channels
     constexpr int KC = CIB * G::K;             // k rows per chunk
     const int lane = lane_id();
     int bbase[NB];
@@ -51,20 +70,39 @@ __device__ __forceinline__ void mfma_window(const ConvArgs<float>& a, int co0, i
         for (int r = 0; r < 16; ++r) acc[j][r] = 0.f;
     const float* ap = Wl + (lane >> 5) * G::K * WLD + (lane & 31);
 
+    // Software pipeline over the channel chunks: the global loads of chunk c+1 (items and weights) are
+    // issued into registers before the MFMAs of chunk c and land in LDS after them.
+    constexpr int W4 = KC * 8;                                   // float4 elements of a weight chunk
+    constexpr int WPT = (W4 + G::NT - 1) / G::NT;
+    ItemRegs<G, float, CIB> R;
+    float4 wr[WPT];
+    auto load_weights = [&](int q) {
+        const float4* src = wl + (int64_t)q * W4;
+#pragma unroll
+        for (int k = 0; k < WPT; ++k) {
+            const int i = threadIdx.x + k * G::NT;
+            if (i < W4) wr[k] = src[i];
+        }
+    };
+    auto store_weights = [&]() {
+#pragma unroll
+        for (int k = 0; k < WPT; ++k) {
+            const int i = threadIdx.x + k * G::NT;
+            if (i < W4) reinterpret_cast<float4*>(Wl)[i] = wr[k];
+        }
+    };
+    load_items<G, float, CIB>(a, 0, nitem, tree_items, sh, R);
+    load_weights(0);
     for (int i = threadIdx.x; i < CIB * G::CH_STRIDE; i += G::NT) patch[i] = 0.f;     // once per window
     for (int ci0 = 0; ci0 < a.Cin; ci0 += CIB) {
-        __syncthreads();            // the previous chunk's MFMAs have read patch and Wl
-        // weight chunk, transposed: Wl[(c*K + t) * WLD + co] = w[co0+co][ci0+c][t]; for a fixed co the
-        // (c, t) run is contiguous in global memory
-        for (int i = threadIdx.x; i < 32 * KC; i += G::NT) {
-            const int co = i / KC, j = i - co * KC;
-            const int ci = ci0 + j / G::K;
-            float v = 0.f;
-            if (co0 + co < a.Cout && ci < a.Cin) v = wl[((int64_t)(co0 + co) * a.Cin + ci0) * G::K + j];
-            Wl[j * WLD + co] = v;
-        }
-        stage_values<G, float, CIB>(a, ci0, nitem, sh, patch);
+        __syncthreads();            // zeros are in place / the previous chunk's MFMAs have read patch and Wl
+        store_items<G, float, CIB>(R, patch);
+        store_weights();
         __syncthreads();
+        if (ci0 + CIB < a.Cin) {
+            load_items<G, float, CIB>(a, ci0 + CIB, nitem, tree_items, sh, R);
+            load_weights(ci0 / CIB + 1);
+        }
 #pragma unroll
         for (int p = 0; p < CIB / 2; ++p) {
 #pragma unroll
@@ -99,7 +137,7 @@ conv_fwd_mfma_kernel(const ConvArgs<float> a) {
     static_assert(G::NWAVE == 4, "block assignment assumes four waves");
     static_assert(NBW == 4 && (G::MAXCOL + 31) / 32 <= 4 * NBW, "a window must fit the accumulators of the block");
     __shared__ float patch[CIB * G::CH_STRIDE];
-    __shared__ float Wl[CIB * G::K * 33];
+    __shared__ __attribute__((aligned(16))) float Wl[CIB * G::K * 32];
     __shared__ ConvShared<G> sh;
 
     const ConvTile tile = a.tiles[blockIdx.x];
@@ -108,7 +146,10 @@ conv_fwd_mfma_kernel(const ConvArgs<float> a) {
     const int yn = a.apr.y_num[L];
     const int s_idx = min(a.S_exp - 1, a.Lc - L);
     const bool out_tree = (L == a.Lc) && (L < a.apr.level_max);
-    const float* __restrict__ wl = a.w + (int64_t)s_idx * a.Cout * a.Cin * G::K;
+    // packed weights of this level and block of 32 output channels: [chunk][CIB*K][32]
+    const int nq = (a.Cin + CIB - 1) / CIB;
+    const float4* __restrict__ wl = reinterpret_cast<const float4*>(a.w) +
+                                    ((int64_t)s_idx * gridDim.y + blockIdx.y) * nq * (CIB * G::K * 8);
     const int wave = threadIdx.x >> 6;
 
     open_segments<G, float>(a, L, z0, x0, sh);
@@ -123,10 +164,10 @@ conv_fwd_mfma_kernel(const ConvArgs<float> a) {
             const int nblk = (nc + 31) >> 5;
             const int first = (wave - (int)blockIdx.x - win) & 3;      // rotation: spread the partial blocks over the SIMDs
             switch ((nblk + 3) >> 2) {
-                case 1: mfma_window<G, CIB, 1>(a, co0, nc, nitem, first, wl, sh, patch, Wl); break;
-                case 2: mfma_window<G, CIB, 2>(a, co0, nc, nitem, first, wl, sh, patch, Wl); break;
-                case 3: mfma_window<G, CIB, 3>(a, co0, nc, nitem, first, wl, sh, patch, Wl); break;
-                default: mfma_window<G, CIB, 4>(a, co0, nc, nitem, first, wl, sh, patch, Wl); break;
+                case 1: mfma_window<G, CIB, 1>(a, co0, nc, nitem, L < a.Lc, first, wl, sh, patch, Wl); break;
+                case 2: mfma_window<G, CIB, 2>(a, co0, nc, nitem, L < a.Lc, first, wl, sh, patch, Wl); break;
+                case 3: mfma_window<G, CIB, 3>(a, co0, nc, nitem, L < a.Lc, first, wl, sh, patch, Wl); break;
+                default: mfma_window<G, CIB, 4>(a, co0, nc, nitem, L < a.Lc, first, wl, sh, patch, Wl); break;
             }
         }
         __syncthreads();
@@ -137,10 +178,25 @@ conv_fwd_mfma_kernel(const ConvArgs<float> a) {
 
 using M333 = ConvGeom<3, 3, 3, 2, 4, 256>;
 
+constexpr int MFMA_CIB = 4;
+
+// a.w must point at the packed weights (pack_conv333_weights)
 int launch_conv333_mfma(const ConvArgs<float>& a, int n_tiles, hipStream_t st) {
     dim3 grid((unsigned)n_tiles, (unsigned)((a.Cout + 31) / 32));
-    hipLaunchKernelGGL((conv_fwd_mfma_kernel<M333, 4, 4>), grid, dim3(M333::NT), 0, st, a);
+    hipLaunchKernelGGL((conv_fwd_mfma_kernel<M333, MFMA_CIB, 4>), grid, dim3(M333::NT), 0, st, a);
     APRNET_LAUNCH_CHECK("conv_fwd_mfma_kernel");
+    return 0;
+}
+
+size_t conv333_packed_floats(int S_exp, int Cout, int Cin) {
+    return (size_t)S_exp * ((Cout + 31) / 32) * ((Cin + MFMA_CIB - 1) / MFMA_CIB) * MFMA_CIB * 27 * 32;
+}
+
+int pack_conv333_weights(const float* w, int S_exp, int Cout, int Cin, float* packed, hipStream_t st) {
+    const size_t n = conv333_packed_floats(S_exp, Cout, Cin);
+    dim3 grid((unsigned)std::min<size_t>((n + 255) / 256, 2048));
+    hipLaunchKernelGGL(pack_weights_kernel, grid, dim3(256), 0, st, w, S_exp, Cout, Cin, 27, MFMA_CIB, packed);
+    APRNET_LAUNCH_CHECK("pack_weights_kernel");
     return 0;
 }
 

@@ -28,8 +28,9 @@ static int copy_access(const aprnet_access_desc* d, HostAccess& h, int lmax_all)
     h.xz_end.assign(d->xz_end_vec, d->xz_end_vec + d->n_rows);
     if (h.xz_end.empty() || h.xz_end[0] != 0 || h.xz_end.back() != d->n_particles)
         return fail(APRNET_ERR_INVALID_ARGUMENT, "plan_create: xz_end_vec must start at 0 and end at n_particles");
-    if (d->n_particles >= (uint64_t)INT32_MAX)
-        return fail(APRNET_ERR_UNSUPPORTED, "plan_create: more than 2^31-1 particles per access");
+    // kernels address a channel plane with 32-bit byte offsets (8-byte elements at most)
+    if (d->n_particles >= (1ull << 29))
+        return fail(APRNET_ERR_UNSUPPORTED, "plan_create: 2^29 or more particles per access");
     if (d->n_particles) h.y.assign(d->y_vec, d->y_vec + d->n_particles);
     return 0;
 }
@@ -187,6 +188,7 @@ void aprnet_plan_destroy(aprnet_plan* p) {
     for (void* q : {p->d_apr_xz, p->d_apr_y, p->d_tree_xz, p->d_tree_y, (void*)p->d_children})
         if (q) (void)hipFree(q);
     for (auto& kv : p->tiles) if (kv.second.d_tiles) (void)hipFree(kv.second.d_tiles);
+    if (p->d_scratch) (void)hipFree(p->d_scratch);
     delete p;
 }
 
