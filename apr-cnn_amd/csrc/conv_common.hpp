@@ -120,13 +120,33 @@ template <class G> struct SegGroup { static constexpr int GRP = G::SPW < 6 ? G::
 // particles (the first n lanes, y ascends) and the cursor of the next window, which is committed at
 // once.  In-window particles are appended to the item list; those of the centre rows (plus tree nodes
 // when they are downsampled particles) whose y lies in the output range also to the column list.
+// Not inlined on purpose: inlined, the per-segment constants of the unrolled loops are hoisted out of the
+// window loop and stay live through the contraction, which costs ~80 registers per lane.
+struct ScanArgs {
+    const uint16_t* apr_y;
+    const uint16_t* tree_y;
+    int tree_off, yn, y0;
+    bool tree_from_x, out_tree;
+};
+
+template <class G>
+__device__ __attribute__((noinline)) void scan_window_impl(const ScanArgs a, ConvShared<G>& sh);
+
 template <class G, typename T>
 __device__ __forceinline__ void scan_window(const ConvArgs<T>& a, int L, int y0, bool out_tree, ConvShared<G>& sh) {
+    ScanArgs s;
+    s.apr_y = a.apr.y; s.tree_y = a.tree.y; s.tree_off = (int)a.tree_off; s.yn = a.apr.y_num[L]; s.y0 = y0;
+    s.tree_from_x = (L == a.Lc); s.out_tree = out_tree;
+    scan_window_impl<G>(s, sh);
+}
+
+template <class G>
+__device__ __attribute__((noinline)) void scan_window_impl(const ScanArgs a, ConvShared<G>& sh) {
+    const int y0 = a.y0, yn = a.yn;
+    const bool tree_from_x = a.tree_from_x, out_tree = a.out_tree;
     constexpr int GRP = SegGroup<G>::GRP;
     const int wave = threadIdx.x >> 6, lane = lane_id();
     const int lo = y0 - G::HY, hi = y0 + G::TY + G::HY, lo_next = y0 + G::TY - G::HY;
-    const int yn = a.apr.y_num[L];
-    const bool tree_from_x = (L == a.Lc);
     for (int k0 = 0; k0 < G::SPW; k0 += GRP) {
         int yy[GRP], cur[GRP];
 #pragma unroll
@@ -136,7 +156,7 @@ __device__ __forceinline__ void scan_window(const ConvArgs<T>& a, int L, int y0,
             if (s < G::NSEG) {
                 cur[g] = sh.seg_cur[s];
                 const int i = cur[g] + lane;
-                if (i < sh.seg_end[s]) yy[g] = (s % 3 == 2) ? (int)a.tree.y[i] : (int)a.apr.y[i];
+                if (i < sh.seg_end[s]) yy[g] = (s % 3 == 2) ? (int)a.tree_y[i] : (int)a.apr_y[i];
             }
         }
 #pragma unroll

@@ -46,9 +46,9 @@ __device__ __forceinline__ constexpr int tap_offset(int t) {
     return ((t / (G::KX * G::KY)) * G::RX + (t / G::KY) % G::KX) * G::WY + (t % G::KY);
 }
 
-// One window for a block whose waves own NB column blocks each (NB = ceil(#blocks / 4), the same for
-// all waves, so every wave runs the same barrier sequence; a wave whose last block does not exist
-// multiplies zeros, which costs nothing extra because it would otherwise wait at the barrier).
+// One window for a wave that owns NB of the window's column blocks (blocks b with b % NWAVE == first).
+// Every instantiation runs the same staging and the same two barriers per channel chunk, so the waves
+// of a block may take different NB (0 included: the wave only helps with the staging).
 template <class G, int CIB, int NB>
 __device__ __forceinline__ void mfma_window(const ConvArgs<float>& a, int co0, int nc, int nitem, bool tree_items, int first,
                                             const float4* __restrict__ wl, const ConvShared<G>& sh,
@@ -56,14 +56,15 @@ __device__ __forceinline__ void mfma_window(const ConvArgs<float>& a, int co0, i
     constexpr int WLD = 32;                    // row of the weight chunk: 32 output channels
     constexpr int KC = CIB * G::K;             // k rows per chunk
     const int lane = lane_id();
-    int bbase[NB];
+    constexpr int NBA = NB > 0 ? NB : 1;
+    int bbase[NBA];
 #pragma unroll
     for (int j = 0; j < NB; ++j) {
-        const int col = ((first + 4 * j) << 5) + (lane & 31);
+        const int col = ((first + G::NWAVE * j) << 5) + (lane & 31);
         const int pos = col < nc ? (int)sh.col_pos[col] - G::TAP0 : 0;
         bbase[j] = pos + (lane >> 5) * G::CH_STRIDE;
     }
-    floatx16 acc[NB];
+    floatx16 acc[NBA];
 #pragma unroll
     for (int j = 0; j < NB; ++j)
 #pragma unroll
@@ -119,7 +120,7 @@ __device__ __forceinline__ void mfma_window(const ConvArgs<float>& a, int co0, i
     // D layout: lane l, register r -> column l%32, row 8*(r/4) + 4*(l/32) + r%4
 #pragma unroll
     for (int j = 0; j < NB; ++j) {
-        const int col = ((first + 4 * j) << 5) + (lane & 31);
+        const int col = ((first + G::NWAVE * j) << 5) + (lane & 31);
         if (col >= nc) continue;
         const int64_t o = sh.col_idx[col];
 #pragma unroll
@@ -134,8 +135,8 @@ template <class G, int CIB, int NBW>
 __global__ void __launch_bounds__(G::NT)
 conv_fwd_mfma_kernel(const ConvArgs<float> a) {
     static_assert(CIB % 2 == 0, "input channels are consumed in pairs");
-    static_assert(G::NWAVE == 4, "block assignment assumes four waves");
-    static_assert(NBW == 4 && (G::MAXCOL + 31) / 32 <= 4 * NBW, "a window must fit the accumulators of the block");
+    static_assert((G::NWAVE & (G::NWAVE - 1)) == 0, "block rotation assumes a power-of-two wave count");
+    static_assert(NBW == 2 && (G::MAXCOL + 31) / 32 <= G::NWAVE * NBW, "a window must fit the accumulators of the block");
     __shared__ float patch[CIB * G::CH_STRIDE];
     __shared__ __attribute__((aligned(16))) float Wl[CIB * G::K * 32];
     __shared__ ConvShared<G> sh;
@@ -162,12 +163,13 @@ conv_fwd_mfma_kernel(const ConvArgs<float> a) {
         const int nc = __builtin_amdgcn_readfirstlane(sh.ncol), nitem = __builtin_amdgcn_readfirstlane(sh.nitem);
         if (nc > 0) {
             const int nblk = (nc + 31) >> 5;
-            const int first = (wave - (int)blockIdx.x - win) & 3;      // rotation: spread the partial blocks over the SIMDs
-            switch ((nblk + 3) >> 2) {
+            // rotation: spread the waves that own one block more over the SIMDs
+            const int first = (wave - (int)blockIdx.x - win) & (G::NWAVE - 1);
+            const int nb = first < nblk ? (nblk - first + G::NWAVE - 1) / G::NWAVE : 0;
+            switch (__builtin_amdgcn_readfirstlane(nb)) {
+                case 0: mfma_window<G, CIB, 0>(a, co0, nc, nitem, L < a.Lc, first, wl, sh, patch, Wl); break;
                 case 1: mfma_window<G, CIB, 1>(a, co0, nc, nitem, L < a.Lc, first, wl, sh, patch, Wl); break;
-                case 2: mfma_window<G, CIB, 2>(a, co0, nc, nitem, L < a.Lc, first, wl, sh, patch, Wl); break;
-                case 3: mfma_window<G, CIB, 3>(a, co0, nc, nitem, L < a.Lc, first, wl, sh, patch, Wl); break;
-                default: mfma_window<G, CIB, 4>(a, co0, nc, nitem, L < a.Lc, first, wl, sh, patch, Wl); break;
+                default: mfma_window<G, CIB, 2>(a, co0, nc, nitem, L < a.Lc, first, wl, sh, patch, Wl); break;
             }
         }
         __syncthreads();
@@ -176,14 +178,14 @@ conv_fwd_mfma_kernel(const ConvArgs<float> a) {
     }
 }
 
-using M333 = ConvGeom<3, 3, 3, 2, 4, 256>;
+using M333 = ConvGeom<3, 3, 3, 2, 4, 512>;
 
 constexpr int MFMA_CIB = 4;
 
 // a.w must point at the packed weights (pack_conv333_weights)
 int launch_conv333_mfma(const ConvArgs<float>& a, int n_tiles, hipStream_t st) {
     dim3 grid((unsigned)n_tiles, (unsigned)((a.Cout + 31) / 32));
-    hipLaunchKernelGGL((conv_fwd_mfma_kernel<M333, MFMA_CIB, 4>), grid, dim3(M333::NT), 0, st, a);
+    hipLaunchKernelGGL((conv_fwd_mfma_kernel<M333, MFMA_CIB, 2>), grid, dim3(M333::NT), 0, st, a);
     APRNET_LAUNCH_CHECK("conv_fwd_mfma_kernel");
     return 0;
 }
