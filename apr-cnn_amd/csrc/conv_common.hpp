@@ -50,7 +50,9 @@ struct ConvGeom {
     static constexpr int MAXCOL = TZ * TX * TY;
     static constexpr int MAXITEM = NROW * WY;                  // every staged cell is filled by at most one item
     static constexpr int ITER = (MAXCOL + NT - 1) / NT;        // output columns per thread
-    static constexpr int CH_STRIDE = NROW * WY;                // patch elements per channel
+    // patch elements per channel; the extra 32 words put the two channels of an MFMA pair (lanes l and
+    // l+32 read the same cell of adjacent channels) on different halves of the LDS banks
+    static constexpr int CH_STRIDE = NROW * WY + 32;
     static constexpr int TAP0 = (HZ * RX + HX) * WY + HY;      // centre -> first tap
 };
 
@@ -271,12 +273,17 @@ __device__ __forceinline__ void load_items(const ConvArgs<T>& a, int ci0, int ni
         for (int k = 0; k < IPT; ++k) R.v[k][c] = RawLoad<T>::ld(rx, offx[k]);
     }
     if (tree_items) {      // tile-uniform: only levels below the current maximum read the mean-filled tree
+        typename RawLoad<T>::raw tv[IPT][CIB];
 #pragma unroll
         for (int c = 0; c < CIB; ++c) {
             const __amdgpu_buffer_rsrc_t rt = plane_rsrc<T>(a.tree_data, a.ldt, ci0 + c, a.Cin, a.t_count);
 #pragma unroll
-            for (int k = 0; k < IPT; ++k) R.v[k][c] |= RawLoad<T>::ld(rt, offt[k]);
+            for (int k = 0; k < IPT; ++k) tv[k][c] = RawLoad<T>::ld(rt, offt[k]);
         }
+#pragma unroll
+        for (int c = 0; c < CIB; ++c)
+#pragma unroll
+            for (int k = 0; k < IPT; ++k) R.v[k][c] |= tv[k][c];      // one of the two loads returned zero
     }
 }
 

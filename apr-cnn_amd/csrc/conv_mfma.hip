@@ -77,32 +77,27 @@ __device__ __forceinline__ void mfma_window(const ConvArgs<float>& a, int co0, i
     constexpr int WPT = (W4 + G::NT - 1) / G::NT;
     ItemRegs<G, float, CIB> R;
     float4 wr[WPT];
-    auto load_weights = [&](int q) {
-        const float4* src = wl + (int64_t)q * W4;
-#pragma unroll
-        for (int k = 0; k < WPT; ++k) {
-            const int i = threadIdx.x + k * G::NT;
-            if (i < W4) wr[k] = src[i];
-        }
-    };
-    auto store_weights = [&]() {
-#pragma unroll
-        for (int k = 0; k < WPT; ++k) {
-            const int i = threadIdx.x + k * G::NT;
-            if (i < W4) reinterpret_cast<float4*>(Wl)[i] = wr[k];
-        }
-    };
+#define APRNET_LOAD_WEIGHTS(q)                                                                     \
+    _Pragma("unroll") for (int k = 0; k < WPT; ++k) {                                              \
+        const int i = threadIdx.x + k * G::NT;                                                     \
+        wr[k] = (i < W4) ? (wl + (int64_t)(q) * W4)[i] : make_float4(0.f, 0.f, 0.f, 0.f);          \
+    }
+#define APRNET_STORE_WEIGHTS()                                                                     \
+    _Pragma("unroll") for (int k = 0; k < WPT; ++k) {                                              \
+        const int i = threadIdx.x + k * G::NT;                                                     \
+        if (i < W4) reinterpret_cast<float4*>(Wl)[i] = wr[k];                                      \
+    }
     load_items<G, float, CIB>(a, 0, nitem, tree_items, sh, R);
-    load_weights(0);
+    APRNET_LOAD_WEIGHTS(0)
     for (int i = threadIdx.x; i < CIB * G::CH_STRIDE; i += G::NT) patch[i] = 0.f;     // once per window
     for (int ci0 = 0; ci0 < a.Cin; ci0 += CIB) {
         __syncthreads();            // zeros are in place / the previous chunk's MFMAs have read patch and Wl
         store_items<G, float, CIB>(R, patch);
-        store_weights();
+        APRNET_STORE_WEIGHTS()
         __syncthreads();
         if (ci0 + CIB < a.Cin) {
             load_items<G, float, CIB>(a, ci0 + CIB, nitem, tree_items, sh, R);
-            load_weights(ci0 / CIB + 1);
+            APRNET_LOAD_WEIGHTS(ci0 / CIB + 1)
         }
 #pragma unroll
         for (int p = 0; p < CIB / 2; ++p) {
@@ -117,6 +112,8 @@ __device__ __forceinline__ void mfma_window(const ConvArgs<float>& a, int co0, i
             }
         }
     }
+#undef APRNET_LOAD_WEIGHTS
+#undef APRNET_STORE_WEIGHTS
     // D layout: lane l, register r -> column l%32, row 8*(r/4) + 4*(l/32) + r%4
 #pragma unroll
     for (int j = 0; j < NB; ++j) {
