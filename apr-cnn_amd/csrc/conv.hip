@@ -81,7 +81,8 @@ conv_fwd_kernel(const ConvArgs<T> a) {
                 const int64_t o = sh.col_idx[col];
 #pragma unroll
                 for (int co = 0; co < COB; ++co)
-                    if (co0 + co < a.Cout) a.y[(int64_t)(co0 + co) * a.ldy + o] = acc[it][co];
+                    if (co0 + co < a.Cout)
+                        a.y[(int64_t)(co0 + co) * a.ldy + o] = acc[it][co] + (a.bias ? a.bias[co0 + co] : (T)0);
             }
         }
         __syncthreads();
@@ -156,7 +157,7 @@ int fill_tree_for_conv(const aprnet_plan* p, int d, const double* x, int64_t ldx
 
 template <typename T>
 int conv_fwd(const aprnet_plan* cp, int d, int kz, int kx, int ky, const T* x, int64_t ldx, int Cin, const T* w,
-             int S_exp, int Cout, T* y, int64_t ldy, T* tree_ws, int64_t ldt, hipStream_t st) {
+             int S_exp, int Cout, const T* bias, T* y, int64_t ldy, T* tree_ws, int64_t ldt, hipStream_t st) {
     aprnet_plan* p = const_cast<aprnet_plan*>(cp);
     if (int rc = check_level_delta(p, d, "conv_forward")) return rc;
     if (Cin <= 0 || Cout <= 0 || S_exp <= 0) return fail(APRNET_ERR_INVALID_ARGUMENT, "conv_forward: empty channel / stencil count");
@@ -173,7 +174,7 @@ int conv_fwd(const aprnet_plan* cp, int d, int kz, int kx, int ky, const T* x, i
     if (tl.n == 0) return 0;
     ConvArgs<T> a{};
     a.apr = p->dapr; a.tree = p->dtree; a.tiles = tl.d_tiles;
-    a.x = x; a.ldx = ldx; a.Cin = Cin; a.w = w; a.S_exp = S_exp; a.Cout = Cout; a.y = y; a.ldy = ldy;
+    a.x = x; a.ldx = ldx; a.Cin = Cin; a.w = w; a.S_exp = S_exp; a.Cout = Cout; a.bias = bias; a.y = y; a.ldy = ldy;
     a.tree_data = tree_ws; a.ldt = ldt; a.Lc = p->lc(d); a.tree_off = p->tree_offset(a.Lc);
     a.x_count = p->number_parts(d); a.t_count = p->tree_parts(d);
     bool done = false;
@@ -209,11 +210,13 @@ float aprnet_profile_last_ms(void) {
     return ms;
 }
 int aprnet_conv_fwd_f32(const aprnet_plan* p, int d, int kz, int kx, int ky, const float* x, int64_t ldx, int Cin,
-                        const float* w, int S_exp, int Cout, float* y, int64_t ldy, float* tree_ws, int64_t ldt, void* st) {
-    return conv_fwd<float>(p, d, kz, kx, ky, x, ldx, Cin, w, S_exp, Cout, y, ldy, tree_ws, ldt, (hipStream_t)st);
+                        const float* w, int S_exp, int Cout, const float* bias, float* y, int64_t ldy, float* tree_ws,
+                        int64_t ldt, void* st) {
+    return conv_fwd<float>(p, d, kz, kx, ky, x, ldx, Cin, w, S_exp, Cout, bias, y, ldy, tree_ws, ldt, (hipStream_t)st);
 }
 int aprnet_conv_fwd_f64(const aprnet_plan* p, int d, int kz, int kx, int ky, const double* x, int64_t ldx, int Cin,
-                        const double* w, int S_exp, int Cout, double* y, int64_t ldy, double* tree_ws, int64_t ldt, void* st) {
-    return conv_fwd<double>(p, d, kz, kx, ky, x, ldx, Cin, w, S_exp, Cout, y, ldy, tree_ws, ldt, (hipStream_t)st);
+                        const double* w, int S_exp, int Cout, const double* bias, double* y, int64_t ldy, double* tree_ws,
+                        int64_t ldt, void* st) {
+    return conv_fwd<double>(p, d, kz, kx, ky, x, ldx, Cin, w, S_exp, Cout, bias, y, ldy, tree_ws, ldt, (hipStream_t)st);
 }
 }

@@ -13,7 +13,7 @@ constexpr int TB1 = 256;
 template <typename T, int OB>
 __global__ void __launch_bounds__(TB1)
 conv111_kernel(const T* __restrict__ src, int64_t lds, int Csrc, const T* __restrict__ w, int so, int sc,
-               T* __restrict__ dst, int64_t ldd, int Cdst, int64_t begin, int64_t end) {
+               const T* __restrict__ bias, T* __restrict__ dst, int64_t ldd, int Cdst, int64_t begin, int64_t end) {
     const int64_t i = begin + (int64_t)blockIdx.x * TB1 + threadIdx.x;
     if (i >= end) return;
     const int o0 = blockIdx.y * OB;
@@ -28,7 +28,7 @@ conv111_kernel(const T* __restrict__ src, int64_t lds, int Csrc, const T* __rest
     }
 #pragma unroll
     for (int o = 0; o < OB; ++o)
-        if (o0 + o < Cdst) dst[(int64_t)(o0 + o) * ldd + i] = acc[o];
+        if (o0 + o < Cdst) dst[(int64_t)(o0 + o) * ldd + i] = acc[o] + (bias ? bias[o0 + o] : (T)0);
 }
 
 // gw[co][ci] += sum_i gy[co][i] * x[ci][i] over [begin, end): 8x8 register tile per thread, block
@@ -94,8 +94,8 @@ static std::vector<Segment> segments(const aprnet_plan* p, int d, int S) {
 }
 
 template <typename T>
-int conv111_fwd(const aprnet_plan* p, int d, const T* x, int64_t ldx, int Cin, const T* w, int S, int Cout, T* y,
-                int64_t ldy, hipStream_t st) {
+int conv111_fwd(const aprnet_plan* p, int d, const T* x, int64_t ldx, int Cin, const T* w, int S, int Cout,
+                const T* bias, T* y, int64_t ldy, hipStream_t st) {
     if (int rc = check_level_delta(p, d, "conv111_forward")) return rc;
     if (Cin <= 0 || Cout <= 0 || S <= 0) return fail(APRNET_ERR_INVALID_ARGUMENT, "conv111_forward: empty channel / stencil count");
     APRNET_HIP_CHECK(hipSetDevice(p->device));
@@ -103,7 +103,7 @@ int conv111_fwd(const aprnet_plan* p, int d, const T* x, int64_t ldx, int Cin, c
     for (const Segment& sg : segments(p, d, S)) {
         dim3 grid((unsigned)((sg.end - sg.begin + TB1 - 1) / TB1), (unsigned)((Cout + OB - 1) / OB));
         hipLaunchKernelGGL((conv111_kernel<T, OB>), grid, dim3(TB1), 0, st, x, ldx, Cin, w + (int64_t)sg.stencil * Cout * Cin,
-                           Cin, 1, y, ldy, Cout, sg.begin, sg.end);
+                           Cin, 1, bias, y, ldy, Cout, sg.begin, sg.end);
     }
     APRNET_LAUNCH_CHECK("conv111_kernel");
     return 0;
@@ -120,7 +120,7 @@ int conv111_bwd(const aprnet_plan* p, int d, const T* x, int64_t ldx, int Cin, c
         const T* ws = w + (int64_t)sg.stencil * Cout * Cin;
         dim3 grid((unsigned)((sg.end - sg.begin + TB1 - 1) / TB1), (unsigned)((Cin + OB - 1) / OB));
         // grad_x[ci][i] = sum_co w[co][ci] * gy[co][i]: the same kernel with the weight strides swapped
-        hipLaunchKernelGGL((conv111_kernel<T, OB>), grid, dim3(TB1), 0, st, gy, ldy, Cout, ws, 1, Cin, gx, ldgx, Cin,
+        hipLaunchKernelGGL((conv111_kernel<T, OB>), grid, dim3(TB1), 0, st, gy, ldy, Cout, ws, 1, Cin, (const T*)nullptr, gx, ldgx, Cin,
                            sg.begin, sg.end);
         const int64_t n = sg.end - sg.begin;
         dim3 g2((unsigned)std::min<int64_t>((n + TB1 * 8 - 1) / (TB1 * 8), 256), (unsigned)((Cout + 7) / 8), (unsigned)((Cin + 7) / 8));
@@ -137,8 +137,8 @@ using namespace aprnet;
 extern "C" {
 #define CONV111_API(T, SFX)                                                                                        \
     int aprnet_conv111_fwd_##SFX(const aprnet_plan* p, int d, const T* x, int64_t ldx, int Cin, const T* w, int S,  \
-                                 int Cout, T* y, int64_t ldy, void* st) {                                           \
-        return conv111_fwd<T>(p, d, x, ldx, Cin, w, S, Cout, y, ldy, (hipStream_t)st); }                            \
+                                 int Cout, const T* bias, T* y, int64_t ldy, void* st) {                            \
+        return conv111_fwd<T>(p, d, x, ldx, Cin, w, S, Cout, bias, y, ldy, (hipStream_t)st); }                      \
     int aprnet_conv111_bwd_##SFX(const aprnet_plan* p, int d, const T* x, int64_t ldx, int Cin, const T* w, int S,  \
                                  int Cout, const T* gy, int64_t ldy, T* gx, int64_t ldgx, T* gw, void* st) {        \
         return conv111_bwd<T>(p, d, x, ldx, Cin, w, S, Cout, gy, ldy, gx, ldgx, gw, (hipStream_t)st); }

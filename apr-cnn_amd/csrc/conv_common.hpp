@@ -27,6 +27,7 @@ struct ConvArgs {
     const ConvTile* tiles;
     const T* x; int64_t ldx; int Cin;
     const T* w; int S_exp; int Cout;          // [S_exp][Cout][Cin][K]
+    const T* bias;                            // [Cout] or null
     T* y; int64_t ldy;
     const T* tree_data; int64_t ldt;
     int Lc; int64_t tree_off;                  // tree_offset(Lc)

@@ -52,7 +52,8 @@ __device__ __forceinline__ constexpr int tap_offset(int t) {
 template <class G, int CIB, int NB>
 __device__ __forceinline__ void mfma_window(const ConvArgs<float>& a, int co0, int nc, int nitem, bool tree_items, int first,
                                             const float4* __restrict__ wl, const ConvShared<G>& sh,
-                                            float* __restrict__ patch, float* __restrict__ Wl) {
+                                            float* __restrict__ patch, float* __restrict__ Wl,
+                                            const float* __restrict__ bias_l) {
     constexpr int WLD = 32;                    // row of the weight chunk: 32 output channels
     constexpr int KC = CIB * G::K;             // k rows per chunk
     const int lane = lane_id();
@@ -115,6 +116,9 @@ __device__ __forceinline__ void mfma_window(const ConvArgs<float>& a, int co0, i
 #undef APRNET_LOAD_WEIGHTS
 #undef APRNET_STORE_WEIGHTS
     // D layout: lane l, register r -> column l%32, row 8*(r/4) + 4*(l/32) + r%4
+    float bias[16];
+#pragma unroll
+    for (int r = 0; r < 16; ++r) bias[r] = bias_l[8 * (r >> 2) + 4 * (lane >> 5) + (r & 3)];
 #pragma unroll
     for (int j = 0; j < NB; ++j) {
         const int col = ((first + G::NWAVE * j) << 5) + (lane & 31);
@@ -123,7 +127,7 @@ __device__ __forceinline__ void mfma_window(const ConvArgs<float>& a, int co0, i
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
             const int co = co0 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
-            if (co < a.Cout) a.y[(int64_t)co * a.ldy + o] = acc[j][r];
+            if (co < a.Cout) a.y[(int64_t)co * a.ldy + o] = acc[j][r] + bias[r];
         }
     }
 }
@@ -137,6 +141,7 @@ conv_fwd_mfma_kernel(const ConvArgs<float> a) {
     __shared__ float patch[CIB * G::CH_STRIDE];
     __shared__ __attribute__((aligned(16))) float Wl[CIB * G::K * 32];
     __shared__ ConvShared<G> sh;
+    __shared__ __attribute__((aligned(16))) float bias_l[32];   // bias of this block's output channels (0 without bias)
 
     const ConvTile tile = a.tiles[blockIdx.x];
     const int L = tile.level, z0 = tile.z0, x0 = tile.x0;
@@ -150,6 +155,7 @@ conv_fwd_mfma_kernel(const ConvArgs<float> a) {
                                     ((int64_t)s_idx * gridDim.y + blockIdx.y) * nq * (CIB * G::K * 8);
     const int wave = threadIdx.x >> 6;
 
+    if (threadIdx.x < 32) bias_l[threadIdx.x] = (a.bias && co0 + (int)threadIdx.x < a.Cout) ? a.bias[co0 + threadIdx.x] : 0.f;
     open_segments<G, float>(a, L, z0, x0, sh);
     __syncthreads();
 
@@ -164,9 +170,9 @@ conv_fwd_mfma_kernel(const ConvArgs<float> a) {
             const int first = (wave - (int)blockIdx.x - win) & (G::NWAVE - 1);
             const int nb = first < nblk ? (nblk - first + G::NWAVE - 1) / G::NWAVE : 0;
             switch (__builtin_amdgcn_readfirstlane(nb)) {
-                case 0: mfma_window<G, CIB, 0>(a, co0, nc, nitem, L < a.Lc, first, wl, sh, patch, Wl); break;
-                case 1: mfma_window<G, CIB, 1>(a, co0, nc, nitem, L < a.Lc, first, wl, sh, patch, Wl); break;
-                default: mfma_window<G, CIB, 2>(a, co0, nc, nitem, L < a.Lc, first, wl, sh, patch, Wl); break;
+                case 0: mfma_window<G, CIB, 0>(a, co0, nc, nitem, L < a.Lc, first, wl, sh, patch, Wl, bias_l); break;
+                case 1: mfma_window<G, CIB, 1>(a, co0, nc, nitem, L < a.Lc, first, wl, sh, patch, Wl, bias_l); break;
+                default: mfma_window<G, CIB, 2>(a, co0, nc, nitem, L < a.Lc, first, wl, sh, patch, Wl, bias_l); break;
             }
         }
         __syncthreads();

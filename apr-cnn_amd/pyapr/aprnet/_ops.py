@@ -120,11 +120,17 @@ def restrict_kernel_backward(grad_weights, num_stencils):
 
 
 # ---------------------------------------------------------------------------------------- convolution
-def conv_forward(aprs, x, weights, level_delta):
+def conv_forward(aprs, x, weights, level_delta, bias=None):
     """conv333_forward / conv111_forward (wrap_conv_gpu.hpp:32-66, 170-193) for any supported stencil.
-    weights: [S_exp, Cout, Cin, kz, kx, ky] (for 1x1x1: [S, Cout, Cin, 1, 1, 1], not expanded)."""
+    weights: [S_exp, Cout, Cin, kz, kx, ky] (for 1x1x1: [S, Cout, Cin, 1, 1, 1], not expanded).
+    bias ([Cout], optional) is added inside the kernel instead of in a separate pass over the output."""
     _check_input(x, "input")
     _check_input(weights, "weights")
+    if bias is not None:
+        _check_input(bias, "bias")
+        if bias.dtype != x.dtype or bias.numel() != weights.size(1):
+            raise ValueError("bias must hold one value per output channel, in the dtype of the input")
+    bptr = _ptr(bias) if bias is not None else None
     if x.size(1) != weights.size(2):
         raise ValueError("convolve: input tensor shape does not match weights tensor!")   # conv.hpp:63-66
     s_exp, cout, cin, kz, kx, ky = weights.shape
@@ -135,6 +141,11 @@ def conv_forward(aprs, x, weights, level_delta):
         raise ValueError("input holds fewer particles than the APR at this level delta")
     out = torch.empty((B, cout, N), dtype=x.dtype, device=x.device)
     _zero_tails(out, sizes)
+    if bias is not None:
+        # the reference adds the bias to the whole padded tensor (conv.py:101): tails hold 0 + bias
+        for b, nb in enumerate(sizes):
+            if nb < N:
+                out[b, :, nb:] = bias.view(-1, 1)
     plans = _plans(aprs, x.device)
     sfx = _sfx(x)
     with torch.cuda.device(x.device):
@@ -142,7 +153,7 @@ def conv_forward(aprs, x, weights, level_delta):
         if (kz, kx, ky) == (1, 1, 1):
             fn = getattr(_lib(), "aprnet_conv111_fwd_" + sfx)
             for b in range(B):
-                rc = fn(plans[b], d[b], _ptr(x[b]), N, cin, _ptr(weights), s_exp, cout, _ptr(out[b]), N, st)
+                rc = fn(plans[b], d[b], _ptr(x[b]), N, cin, _ptr(weights), s_exp, cout, bptr, _ptr(out[b]), N, st)
                 if rc:
                     _raise(rc, "conv111_forward failed")
         else:
@@ -150,7 +161,7 @@ def conv_forward(aprs, x, weights, level_delta):
             tree_ws = torch.empty((cin, ld_tree), dtype=x.dtype, device=x.device)
             fn = getattr(_lib(), "aprnet_conv_fwd_" + sfx)
             for b in range(B):
-                rc = fn(plans[b], d[b], kz, kx, ky, _ptr(x[b]), N, cin, _ptr(weights), s_exp, cout, _ptr(out[b]), N,
+                rc = fn(plans[b], d[b], kz, kx, ky, _ptr(x[b]), N, cin, _ptr(weights), s_exp, cout, bptr, _ptr(out[b]), N,
                         _ptr(tree_ws), ld_tree, st)
                 if rc:
                     _raise(rc, "conv_forward failed")

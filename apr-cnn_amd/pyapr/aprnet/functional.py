@@ -47,8 +47,8 @@ class ConvFunction(Function):
             w = _ops.restrict_kernel_forward(w, num_levels)
         inputs = inputs.contiguous()
         ctx.save_for_backward(inputs, w, bias, level_deltas.clone())
-        output = _ops.conv_forward(aprs, inputs, w, level_deltas)
-        return output if bias is None else output + bias.view((1, -1, 1))
+        # the bias add of conv.py:101 is fused into the kernel's store
+        return _ops.conv_forward(aprs, inputs, w, level_deltas, None if bias is None else bias.contiguous())
 
     @staticmethod
     def backward(ctx, grad_output):

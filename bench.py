@@ -5,7 +5,7 @@ seeded 512 x 512 x 256 blob volume (BASELINE.json configs[1]).
   python bench.py [--gpus 1] [--steps K] [--warmup W]
 
 A step is one `aprnet.cuda.APRConv.forward` on device-resident features: weight expansion
-(restrict kernel), tree fill of the 32 input channels, the convolution kernel and the bias add.
+(restrict kernel), tree fill of the 32 input channels and the convolution kernel (bias fused into its store).
 Prints ONE JSON line.  `value` = particles/s of the whole step; `roofline` prices the convolution
 kernel alone (its duration is measured with HIP events recorded around the launch on its own stream,
 see aprnet_profile_enable in include/aprnet_hip.h); `cpu_baseline` times the CPU oracle (a restatement
@@ -66,12 +66,81 @@ def cpu_baseline(nstencils):
                       f"conv 3x3x3 {CIN}->{COUT} fp32, 1 run, {dt:.1f} s"}
 
 
+def _time(fn, iters=10, warmup=2):
+    import torch
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    a.record()
+    for _ in range(iters):
+        fn()
+    b.record()
+    torch.cuda.synchronize()
+    return a.elapsed_time(b) / iters
+
+
+def other_ops(apr, x, dev):
+    """Memory-bound operators at 32 channels on the same APR, priced against the HBM roofline with their
+    algorithmic bytes, the backward pass of the convolution, and the 4-level APR-UNet forward."""
+    import torch
+    from pyapr import aprnet
+    from pyapr.aprnet import _ops
+    from apr_models.unet import APRUNet, fold_norms
+    C, e = x.shape[1], 4
+    ld0, ld1 = torch.zeros(1, dtype=torch.int32), torch.ones(1, dtype=torch.int32)
+    n0, n1 = _ops.number_particles(apr, 0), _ops.number_particles(apr, 1)
+    nt = _ops.tree_parts(apr, 0)
+    res = []
+
+    def line(op, ms, nbytes, note):
+        res.append({"op": op, "ms": ms, "algorithmic_GB": nbytes / 1e9, "GBps": nbytes / ms / 1e6,
+                    "hbm_frac": nbytes / ms / 1e6 / PEAK_HBM_GBS, "note": note})
+
+    with torch.no_grad():
+        pooled, idx = _ops.maxpool_forward([apr], x, ld0, 0.0)
+        ms = _time(lambda: _ops.maxpool_forward([apr], x, ld0, 0.0))
+        line("maxpool_fwd", ms, e * C * n0 + (e + 8) * C * n1, f"C={C}, N {n0} -> {n1}, int64 argmax written")
+        ms = _time(lambda: _ops.maxpool_backward([apr], pooled, idx, ld0))
+        line("maxpool_bwd", ms, (e + 8) * C * n1 + e * C * n0, "reads grad + argmax, writes grad_input")
+        ms = _time(lambda: _ops.upsample_const_forward([apr], pooled, ld1))
+        line("upsample_fwd", ms, e * C * (n1 + n0), f"C={C}, N {n1} -> {n0}")
+        ms = _time(lambda: _ops.upsample_const_backward([apr], x, ld1))
+        line("upsample_bwd", ms, e * C * (n1 + n0), "sum of child gradients")
+        tree = torch.empty(C, max(nt, 1), device=dev)
+        lib, plan, st = _ops._lib(), apr.plan(0), torch.cuda.current_stream().cuda_stream
+        ms = _time(lambda: lib.aprnet_fill_tree_mean_f32(plan, 0, x.data_ptr(), x.shape[2], C, tree.data_ptr(), tree.shape[1], st))
+        line("fill_tree_mean", ms, e * C * (n0 + 2 * nt), f"C={C}, {nt} tree nodes")
+        w1 = torch.randn(1, C, C, 1, 1, 1, device=dev) * 0.1
+        ms = _time(lambda: _ops.conv_forward([apr], x, w1, ld0))
+        line("conv111_fwd", ms, e * 2 * C * n0, f"{C}->{C}")
+    conv = aprnet.cuda.APRConv(C, C, nstencils=2).to(dev)
+    xg = x.clone().requires_grad_(True)
+    y = conv(xg, [apr], ld0)
+    go = torch.randn_like(y)
+    ms = _time(lambda: torch.autograd.grad(y, (xg, conv.weight), go, retain_graph=True), iters=3, warmup=1)
+    res.append({"op": "conv333_bwd", "ms": ms, "particles_per_s": n0 / ms * 1e3, "note": f"{C}->{C} grad_input + grad_weight"})
+    del y, go, xg
+    torch.manual_seed(0)
+    net = fold_norms(APRUNet(1, 3, depth=3, n_filters_base=16, n_stencils=2, norm="batch").eval()).to(dev)
+    xin = x[:, :1].contiguous()
+    with torch.no_grad():
+        ms = _time(lambda: net(xin, [apr]), iters=3, warmup=1)
+    res.append({"op": "apr_unet_fwd", "ms": ms, "note": f"4 levels 16-32-64-128, fp32, {n0} particles, norms folded"})
+    return res
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="run one device-to-device copy of the input features (a kernel of known traffic, "
+                         "used to scale the FETCH_SIZE / WRITE_SIZE counters of a profiler run)")
+    ap.add_argument("--ops", action="store_true",
+                    help="also time the memory-bound operators and the APR-UNet forward (extra JSON lines on stderr)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU; --gpus N with N > 1 is not supported "
@@ -136,6 +205,14 @@ def main():
                      "kernel": "conv_fwd_kernel", "kernel_ms": kernel_ms,
                      "hbm_achieved_GBs": gbs, "hbm_frac": gbs / PEAK_HBM_GBS},
     }
+    if args.calibrate_copy:
+        torch.empty_like(x).copy_(x)
+        torch.cuda.synchronize()
+        print(json.dumps({"calibration_copy_bytes_read": x.numel() * 4, "calibration_copy_bytes_written": x.numel() * 4}),
+              file=sys.stderr, flush=True)
+    if args.ops:
+        for line in other_ops(apr, x, dev):
+            print(json.dumps(line), file=sys.stderr, flush=True)
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(nstencils)
     print(json.dumps(out), flush=True)

@@ -93,10 +93,11 @@ float aprnet_profile_last_ms(void);
                                         T* grad_tree, int64_t ld_tree, void* stream);                               \
     /* Convolution<kz,kx,ky>::forward (conv.hpp:55-195), CUDA twin conv333_forward (wrap_conv_gpu.hpp:32-66).       \
      * (kz,kx,ky) in {333,133,155,555}.  w: expanded stencils [S_exp][Cout][Cin][kz][kx][ky] (the layout of         \
-     * cuda/conv.py:77).  y is OVERWRITTEN for indices < number_parts(d).  tree_ws: [Cin][ld_tree] scratch,         \
-     * ld_tree >= aprnet_tree_parts(plan, d). */                                                                    \
+     * cuda/conv.py:77).  y is OVERWRITTEN for indices < number_parts(d).  bias: [Cout] or NULL; the reference     \
+     * adds it in a separate pass (conv.py:101), here it is fused into the store.  tree_ws: [Cin][ld_tree]         \
+     * scratch, ld_tree >= aprnet_tree_parts(plan, d). */                                                           \
     int aprnet_conv_fwd_##SFX(const aprnet_plan*, int level_delta, int kz, int kx, int ky,                          \
-                              const T* x, int64_t ldx, int Cin, const T* w, int S_exp, int Cout,                    \
+                              const T* x, int64_t ldx, int Cin, const T* w, int S_exp, int Cout, const T* bias,     \
                               T* y, int64_t ldy, T* tree_ws, int64_t ld_tree, void* stream);                        \
     /* Convolution<kz,kx,ky>::backward (conv.hpp:261-481), CUDA twin conv333_backward.  grad_x is OVERWRITTEN,      \
      * grad_w [S_exp][Cout][Cin][k] is ACCUMULATED into (zero it before the first batch item, as                    \
@@ -108,7 +109,7 @@ float aprnet_profile_last_ms(void);
     /* Convolution<1,1,1>::forward/backward (conv.hpp:199-256, 484-554); w: [S][Cout][Cin] (not expanded,           \
      * stencil index min(S-1, Lc-level)).  grad_w is accumulated, grad_x overwritten. */                            \
     int aprnet_conv111_fwd_##SFX(const aprnet_plan*, int level_delta, const T* x, int64_t ldx, int Cin,             \
-                                 const T* w, int S, int Cout, T* y, int64_t ldy, void* stream);                     \
+                                 const T* w, int S, int Cout, const T* bias, T* y, int64_t ldy, void* stream);      \
     int aprnet_conv111_bwd_##SFX(const aprnet_plan*, int level_delta, const T* x, int64_t ldx, int Cin,             \
                                  const T* w, int S, int Cout, const T* grad_y, int64_t ldy,                         \
                                  T* grad_x, int64_t ldgx, T* grad_w, void* stream);                                 \
