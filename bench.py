@@ -28,6 +28,11 @@ FLOP_PER_PARTICLE = 2 * K_TAPS * CIN * COUT          # 55 296
 BYTES_PER_PARTICLE = 4 * (CIN + COUT) + 2            # features in + out, y_vec
 PEAK_FP32_MATRIX_TFLOPS = 157.3
 PEAK_HBM_GBS = 8000.0
+# HBM-side bytes of one launch of the convolution kernel on this workload: FETCH_SIZE + WRITE_SIZE of two
+# profiler passes, scaled by what the same counters read for a device-to-device copy of known size
+# (profiles/conv333_fwd_32x32_f32_blobs512_hbm_traffic.txt).  Counters cannot be read from inside this
+# script; the figure is only reported when the workload is the one it was measured on.
+MEASURED_TRAFFIC_BYTES = {23245996: 28.98e9 + 3.79e9}
 
 
 def build_workload(name, crop=None):
@@ -201,8 +206,8 @@ def main():
                    "n_particles": n, "nstencils": nstencils, "level_max": apr.level_max(),
                    "apr_build_s": round(t_build, 2), "plan_create_s": round(t_plan, 2)},
         "roofline": {"bound": "mfma", "achieved": tflops, "peak": PEAK_FP32_MATRIX_TFLOPS, "unit": "TFLOP/s",
-                     "frac": tflops / PEAK_FP32_MATRIX_TFLOPS, "traffic": None,
-                     "kernel": "conv_fwd_kernel", "kernel_ms": kernel_ms,
+                     "frac": tflops / PEAK_FP32_MATRIX_TFLOPS, "traffic": MEASURED_TRAFFIC_BYTES.get(n),
+                     "kernel": "conv_fwd_mfma_kernel", "kernel_ms": kernel_ms,
                      "hbm_achieved_GBs": gbs, "hbm_frac": gbs / PEAK_HBM_GBS},
     }
     if args.calibrate_copy:
