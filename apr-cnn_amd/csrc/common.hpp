@@ -48,7 +48,11 @@ struct HostAccess {
 
 struct ConvTile { int32_t level, z0, x0, pad; };
 
-struct TileList { ConvTile* d_tiles = nullptr; int n = 0; };
+struct TileList {
+    ConvTile* d_tiles = nullptr; int n = 0;
+    int level_begin[MAX_LEVELS + 1] = {};   // tiles are sorted finest level first: level l owns
+    int level_count[MAX_LEVELS + 1] = {};   // [level_begin[l], level_begin[l] + level_count[l])
+};
 
 }  // namespace aprnet
 
@@ -59,7 +63,7 @@ struct aprnet_plan {
     void* d_apr_xz = nullptr; void* d_apr_y = nullptr; void* d_tree_xz = nullptr; void* d_tree_y = nullptr;
     int32_t* d_children = nullptr;      // [8][n_tree], slot-major
     int64_t n_tree = 0, n_apr = 0;
-    std::map<std::tuple<int, int, int>, aprnet::TileList> tiles;   // (level_delta, TZ, TX) -> non-empty row groups
+    std::map<std::tuple<int, int, int, int>, aprnet::TileList> tiles;   // (level_delta, TZ, TX, halo) -> row groups
     void* d_scratch = nullptr; size_t scratch_bytes = 0;          // re-laid-out weights of the call in flight
 
     int lc(int level_delta) const { return apr.level_max - level_delta; }
@@ -78,7 +82,10 @@ namespace aprnet {
 void set_error(const std::string& msg);
 int fail(int code, const std::string& msg);
 // non-empty row groups for the convolution at `level_delta` (built on first use, cached in the plan)
-int get_tiles(aprnet_plan* plan, int level_delta, int TZ, int TX, TileList* out);
+// `halo` > 0 also lists the row groups that lie within that many rows of a non-empty one
+int get_tiles(aprnet_plan* plan, int level_delta, int TZ, int TX, TileList* out, int halo = 0);
+// makes plan->d_scratch at least `bytes` large (contents are lost when it grows)
+int plan_scratch(aprnet_plan* plan, size_t bytes, hipStream_t st);
 
 #define APRNET_HIP_CHECK(expr)                                                                                  \
     do {                                                                                                        \

@@ -61,7 +61,7 @@ conv_fwd_kernel(const ConvArgs<T> a) {
                             for (int sx = 0; sx < G::KX; ++sx)
 #pragma unroll
                                 for (int sy = 0; sy < G::KY; ++sy)
-                                    v[(sz * G::KX + sx) * G::KY + sy] = p0[c * G::CH_STRIDE + (sz * G::RX + sx) * G::WY + sy];
+                                    v[(sz * G::KX + sx) * G::KY + sy] = p0[c * G::CH_STRIDE + (sz * G::RX + sx) * G::RS + sy];
 #pragma unroll
                         for (int co = 0; co < COB; ++co) {
                             if (co0 + co >= a.Cout) break;
@@ -130,22 +130,17 @@ template <> struct Chunk<double> { static constexpr int c333 = 4, c133 = 8,  c15
 
 int launch_conv333_mfma(const ConvArgs<float>& a, int n_tiles, hipStream_t st);
 size_t conv333_packed_floats(int S_exp, int Cout, int Cin);
-int pack_conv333_weights(const float* w, int S_exp, int Cout, int Cin, float* packed, hipStream_t st);
+int pack_conv333_weights(const float* w, int S_exp, int Cm, int Ck, bool transposed, float* packed, hipStream_t st);
 static int g_conv_path = 0;      // 0: matrix cores where available, 1: VALU kernels only
+int conv_path() { return g_conv_path; }
 
 template <typename T> static int try_mfma(aprnet_plan*, const ConvArgs<T>&, int, int, hipStream_t, bool*) { return 0; }
 template <> int try_mfma<float>(aprnet_plan* p, const ConvArgs<float>& a, int code, int n_tiles, hipStream_t st, bool* done) {
     if (g_conv_path == 1 || code != 333) return 0;
     *done = true;
     // plan-owned scratch for the re-laid-out weights, grown on demand
-    const size_t need = conv333_packed_floats(a.S_exp, a.Cout, a.Cin) * sizeof(float);
-    if (need > p->scratch_bytes) {
-        if (p->d_scratch) { APRNET_HIP_CHECK(hipStreamSynchronize(st)); APRNET_HIP_CHECK(hipFree(p->d_scratch)); }
-        p->d_scratch = nullptr; p->scratch_bytes = 0;
-        APRNET_HIP_CHECK(hipMalloc(&p->d_scratch, need));
-        p->scratch_bytes = need;
-    }
-    if (int rc = pack_conv333_weights(a.w, a.S_exp, a.Cout, a.Cin, (float*)p->d_scratch, st)) return rc;
+    if (int rc = plan_scratch(p, conv333_packed_floats(a.S_exp, a.Cout, a.Cin) * sizeof(float), st)) return rc;
+    if (int rc = pack_conv333_weights(a.w, a.S_exp, a.Cout, a.Cin, false, (float*)p->d_scratch, st)) return rc;
     ConvArgs<float> b = a;
     b.w = (const float*)p->d_scratch;
     TimedLaunch timed(st);

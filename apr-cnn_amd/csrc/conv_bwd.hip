@@ -113,7 +113,7 @@ conv_bwd_dx_kernel(const ConvArgs<T> a) {
                         for (int sx = 0; sx < G::KX; ++sx)
 #pragma unroll
                             for (int sy = 0; sy < G::KY; ++sy)
-                                atomicAdd(&p0[c * G::CH_STRIDE + (sz * G::RX + sx) * G::WY + sy],
+                                atomicAdd(&p0[c * G::CH_STRIDE + (sz * G::RX + sx) * G::RS + sy],
                                           g[c][(sz * G::KX + sx) * G::KY + sy]);
             }
             __syncthreads();
@@ -186,7 +186,7 @@ conv_bwd_dw_kernel(const ConvArgs<T> a) {
                             for (int sx = 0; sx < G::KX; ++sx)
 #pragma unroll
                                 for (int sy = 0; sy < G::KY; ++sy)
-                                    acc[(sz * G::KX + sx) * G::KY + sy] += dO * p0[(sz * G::RX + sx) * G::WY + sy];
+                                    acc[(sz * G::KX + sx) * G::KY + sy] += dO * p0[(sz * G::RX + sx) * G::RS + sy];
                     }
                 }
             }
@@ -225,6 +225,31 @@ static int launch_bwd(ConvArgs<T>& a, hipStream_t st) {
     return 0;
 }
 
+// matrix-core kernels (conv_mfma.hip, conv_bwd_mfma.hip)
+int launch_conv333_dx_mfma(const ConvArgs<float>& a, int n_tiles, hipStream_t st);
+int launch_conv333_dw_mfma(const ConvArgs<float>& a, const TileList& tl, int level_min, hipStream_t st);
+size_t conv333_packed_floats(int S_exp, int Cm, int Ck);
+int pack_conv333_weights(const float* w, int S_exp, int Cm, int Ck, bool transposed, float* packed, hipStream_t st);
+int conv_path();
+
+template <typename T> static int try_mfma_bwd(aprnet_plan*, const ConvArgs<T>&, const TileList&, int, int, hipStream_t, bool*) { return 0; }
+template <> int try_mfma_bwd<float>(aprnet_plan* p, const ConvArgs<float>& a, const TileList& tl, int code, int d, hipStream_t st, bool* done) {
+    if (conv_path() == 1 || code != 333) return 0;
+    *done = true;
+    // input gradient: the forward kernel on the output gradient with the transposed, flipped stencil;
+    // every row group within one row of an output takes part
+    TileList near;
+    if (int rc = get_tiles(p, d, 2, 4, &near, 1)) return rc;
+    if (int rc = plan_scratch(p, conv333_packed_floats(a.S_exp, a.Cin, a.Cout) * sizeof(float), st)) return rc;
+    if (int rc = pack_conv333_weights(a.w, a.S_exp, a.Cin, a.Cout, true, (float*)p->d_scratch, st)) return rc;
+    ConvArgs<float> b = a;
+    b.tiles = near.d_tiles; b.n_tiles = near.n;
+    b.x = a.gy; b.ldx = a.ldy; b.Cin = a.Cout; b.Cout = a.Cin; b.w = (const float*)p->d_scratch; b.bias = nullptr;
+    b.tree_data = nullptr; b.t_count = 0;
+    if (near.n > 0) if (int rc = launch_conv333_dx_mfma(b, near.n, st)) return rc;
+    return launch_conv333_dw_mfma(a, tl, p->apr.level_min, st);
+}
+
 template <typename T>
 int conv_bwd(const aprnet_plan* cp, int d, int kz, int kx, int ky, const T* x, int64_t ldx, int Cin, const T* w, int S_exp,
              int Cout, const T* gy, int64_t ldy, T* gx, int64_t ldgx, T* gw, T* tree_ws, int64_t ldt, T* gtree_ws,
@@ -254,7 +279,9 @@ int conv_bwd(const aprnet_plan* cp, int d, int kz, int kx, int ky, const T* x, i
         a.gy = gy; a.ldy = ldy; a.gx = gx; a.ldgx = ldgx; a.gtree = gtree_ws; a.ldgt = ldgt; a.gw = gw;
         constexpr bool f32 = sizeof(T) == 4;
         int rc = 0;
-        switch (code) {
+        bool done = false;
+        if ((rc = try_mfma_bwd<T>(p, a, tl, code, d, st, &done))) return rc;
+        if (!done) switch (code) {
             case 333: rc = launch_bwd<T, X333, (f32 ? 4 : 2), W333, (f32 ? 8 : 4), (f32 ? 32 : 16)>(a, st); break;
             case 133: rc = launch_bwd<T, X133, (f32 ? 8 : 4), W133, (f32 ? 8 : 4), (f32 ? 32 : 16)>(a, st); break;
             case 155: rc = launch_bwd<T, X155, (f32 ? 4 : 2), W155, (f32 ? 8 : 4), (f32 ? 32 : 16)>(a, st); break;

@@ -1,0 +1,144 @@
+// Stencil convolution backward on the matrix cores (fp32 MFMA), gfx950: gradient of the weights.
+// (The gradient of the input is the forward kernel run on the output gradient with the transposed,
+// flipped stencil, conv_mfma.hip.)
+//
+//   dW[s][co][ci][t] = sum over output positions (columns) of  gY[co][col] * patch[ci][pos(col) + off(t)]
+//
+// is a GEMM with M = 32 output channels, N = taps (27 of the 32 columns of the tile are used) and the
+// columns of the window as the contracted axis, one 32x32 accumulator per input channel:
+//
+//     v_mfma_f32_32x32x2_f32:  D[co][t] += A[co][k] * B[k][t],   k = two columns of the window
+//       A: lane l supplies gY[co = l%32] of column k = l/32      (LDS image gyl, laid out so that the
+//                                                                  read is linear in the lane index)
+//       B: lane l supplies patch[ci][pos(column k = l/32) + off(t = l%32)]
+//
+// A block owns 16 input channels (four staged chunks of 4) and 32 output channels.  Wave w takes input
+// channel w%4 of every chunk and half of the columns (w/4), so it holds four accumulators, and keeps them
+// in registers while the (persistent) block walks over many tiles of one stencil index (one launch per
+// stencil index); they are added to the result with one atomic per element at the end.  The patch rows are 67 words
+// apart so that the 27 tap offsets of a B read fall into 27 different LDS banks.
+#include "conv_common.hpp"
+
+namespace aprnet {
+
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+
+using W333M = ConvGeom<3, 3, 3, 2, 4, 512, 67>;
+constexpr int DW_CIB = 4;          // input channels per staged chunk
+constexpr int DW_NCH = 4;          // chunks per block
+constexpr int DW_GB = 256;         // columns of gY staged at a time
+constexpr int DW_GLD = 33;         // words per column of gyl (32 output channels + 1 against bank conflicts)
+
+template <class G, int CIB, int NCH>
+__global__ void __launch_bounds__(G::NT) __attribute__((amdgpu_waves_per_eu(4, 4)))
+conv_dw_mfma_kernel(const ConvArgs<float> a, const int s_idx) {
+    static_assert(G::NWAVE == 8 && CIB == 4, "wave w owns input channel w%4 and column half w/4");
+    __shared__ float patch[CIB * G::CH_STRIDE];
+    __shared__ float gyl[DW_GB * DW_GLD];
+    __shared__ ConvShared<G> sh;
+
+    const int cig0 = blockIdx.y * (CIB * NCH), co0 = blockIdx.z * 32;
+    const int lane = lane_id();
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int cil = wave & 3, kh = wave >> 2;
+    const int t = lane & 31, hi = lane >> 5;
+    const int tt = t < G::K ? t : 0;
+    const int toff = ((tt / (G::KX * G::KY)) * G::RX + (tt / G::KY) % G::KX) * G::RS + (tt % G::KY);
+    const int bl = cil * G::CH_STRIDE - G::TAP0 + toff;       // B operand: + cell of the column
+    const float* ap = gyl + lane + hi;                        // A operand: + (64 * batch + 2 * kk) * DW_GLD
+
+    floatx16 acc[NCH];
+#pragma unroll
+    for (int q = 0; q < NCH; ++q)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[q][r] = 0.f;
+
+    for (int ti = blockIdx.x; ti < a.n_tiles; ti += gridDim.x) {
+        const ConvTile tile = a.tiles[ti];
+        const int L = tile.level, z0 = tile.z0, x0 = tile.x0;
+        const int yn = a.apr.y_num[L];
+        const bool out_tree = (L == a.Lc) && (L < a.apr.level_max);
+
+        __syncthreads();
+        open_segments<G, float>(a, L, z0, x0, sh);
+        __syncthreads();
+
+        for (int y0 = 0; y0 < yn; y0 += G::TY) {
+            scan_window<G, float>(a, L, y0, out_tree, sh);
+            __syncthreads();
+            const int nc = __builtin_amdgcn_readfirstlane(sh.ncol), nitem = __builtin_amdgcn_readfirstlane(sh.nitem);
+            if (nc > 0) {
+                for (int i = threadIdx.x; i < CIB * G::CH_STRIDE; i += G::NT) patch[i] = 0.f;     // once per window
+                for (int g0 = 0; g0 < nc; g0 += DW_GB) {
+                    const int ng = min(DW_GB, nc - g0), nbatch = (ng + 63) >> 6;
+                    // output gradient of this group of columns -> gyl; a wave reads 64 columns of one channel
+                    for (int i = threadIdx.x; i < 32 * nbatch * 64; i += G::NT) {
+                        const int co = i / (nbatch * 64), c = i - co * (nbatch * 64);
+                        float v = 0.f;
+                        if (c < ng && co0 + co < a.Cout) v = a.gy[(int64_t)(co0 + co) * a.ldy + sh.col_idx[g0 + c]];
+                        const int slot = (c & ~63) + 2 * (c & 31) + ((c >> 5) & 1);
+                        gyl[slot * DW_GLD + co] = v;
+                    }
+#pragma unroll
+                    for (int q = 0; q < NCH; ++q) {
+                        __syncthreads();        // previous chunk's reads of the patch are done / gyl is written
+                        stage_values<G, float, CIB>(a, cig0 + q * CIB, nitem, L < a.Lc, sh, patch);
+                        __syncthreads();
+#pragma unroll 1
+                        for (int b = 0; b < nbatch; ++b) {
+                            // cell of column 64 b + lane; broadcast below with readlane
+                            const int c = b * 64 + lane;
+                            const int pb = c < ng ? (int)sh.col_pos[g0 + c] : G::TAP0;
+                            const float* apb = ap + (b * 64 + 32 * kh) * DW_GLD;
+#pragma unroll
+                            for (int k = 0; k < 16; ++k) {
+                                const int kk = kh * 16 + k;
+                                const int p0 = __builtin_amdgcn_readlane(pb, kk);
+                                const int p1 = __builtin_amdgcn_readlane(pb, kk + 32);
+                                const float av = apb[2 * k * DW_GLD];
+                                const float bv = patch[bl + (hi ? p1 : p0)];
+                                acc[q] = __builtin_amdgcn_mfma_f32_32x32x2f32(av, bv, acc[q], 0, 0, 0);
+                            }
+                        }
+                    }
+                    __syncthreads();            // gyl is rewritten by the next group
+                }
+            }
+            __syncthreads();
+            close_window<G>(sh);
+            __syncthreads();
+        }
+    }
+#pragma unroll
+    for (int q = 0; q < NCH; ++q) {
+        const int ci = cig0 + q * CIB + cil;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const int co = co0 + 8 * (r >> 2) + 4 * hi + (r & 3);
+            if (t < G::K && ci < a.Cin && co < a.Cout && acc[q][r] != 0.f)
+                unsafeAtomicAdd(a.gw + (((int64_t)s_idx * a.Cout + co) * a.Cin + ci) * G::K + t, acc[q][r]);
+        }
+    }
+}
+
+// Weight gradient of the 3x3x3 stencil; a.gw is accumulated into (the caller zeroes it).
+// One launch per stencil index: level Lc - s for s < S_exp - 1, every coarser level for the last one
+// (adjacent in the tile list, which is sorted finest level first).
+int launch_conv333_dw_mfma(const ConvArgs<float>& a0, const TileList& tl, int level_min, hipStream_t st) {
+    for (int s = 0; s < a0.S_exp; ++s) {
+        const int l_hi = a0.Lc - s, l_lo = (s == a0.S_exp - 1) ? level_min : l_hi;
+        if (l_hi < level_min) break;
+        int n = 0;
+        for (int l = l_lo; l <= l_hi; ++l) n += tl.level_count[l];
+        if (n == 0) continue;
+        ConvArgs<float> a = a0;
+        a.tiles = tl.d_tiles + tl.level_begin[l_hi]; a.n_tiles = n;
+        dim3 grid((unsigned)std::min(n, 512), (unsigned)((a.Cin + DW_CIB * DW_NCH - 1) / (DW_CIB * DW_NCH)),
+                  (unsigned)((a.Cout + 31) / 32));
+        hipLaunchKernelGGL((conv_dw_mfma_kernel<W333M, DW_CIB, DW_NCH>), grid, dim3(W333M::NT), 0, st, a, s);
+        APRNET_LAUNCH_CHECK("conv_dw_mfma_kernel");
+    }
+    return 0;
+}
+
+}  // namespace aprnet

@@ -36,9 +36,10 @@ struct ConvArgs {
     const T* gy; T* gx; int64_t ldgx; T* gtree; int64_t ldgt; T* gw; int n_tiles;
 };
 
-template <int KZ_, int KX_, int KY_, int TZ_, int TX_, int NT_>
+template <int KZ_, int KX_, int KY_, int TZ_, int TX_, int NT_, int RS_ = 64>
 struct ConvGeom {
     static constexpr int KZ = KZ_, KX = KX_, KY = KY_, TZ = TZ_, TX = TX_, NT = NT_;
+    static constexpr int RS = RS_;                // words between two staged rows of one channel (>= WY)
     static constexpr int K = KZ * KX * KY;
     static constexpr int HZ = (KZ - 1) / 2, HX = (KX - 1) / 2, HY = (KY - 1) / 2;
     static constexpr int RZ = TZ + KZ - 1, RX = TX + KX - 1;
@@ -53,8 +54,8 @@ struct ConvGeom {
     static constexpr int ITER = (MAXCOL + NT - 1) / NT;        // output columns per thread
     // patch elements per channel; the extra 32 words put the two channels of an MFMA pair (lanes l and
     // l+32 read the same cell of adjacent channels) on different halves of the LDS banks
-    static constexpr int CH_STRIDE = NROW * WY + 32;
-    static constexpr int TAP0 = (HZ * RX + HX) * WY + HY;      // centre -> first tap
+    static constexpr int CH_STRIDE = (NROW * RS + 63) / 64 * 64 + 32;
+    static constexpr int TAP0 = (HZ * RX + HX) * RS + HY;      // centre -> first tap
 };
 
 __device__ __forceinline__ int lane_id() { return __lane_id(); }
@@ -181,12 +182,12 @@ __device__ __attribute__((noinline)) void scan_window_impl(const ScanArgs a, Con
             if (in) {      // in-window lanes are lanes 0 .. n_in-1
                 unsigned pos;
                 if (src != 1) {
-                    pos = (unsigned)(r * G::WY + (yy[g] - lo));
+                    pos = (unsigned)(r * G::RS + (yy[g] - lo));
                     if (src == 2 && !tree_from_x) pos |= ITEM_TREE;
                 } else {
                     const int ya = 2 * yy[g], yb = ya + 1;
                     const bool wa = ya >= lo, wb = yb < hi && yb < yn;
-                    pos = (unsigned)(r * G::WY + ((wa ? ya : yb) - lo));
+                    pos = (unsigned)(r * G::RS + ((wa ? ya : yb) - lo));
                     if (wa && wb) pos |= ITEM_PAIR;
                 }
                 sh.item_idx[ibase + lane] = i + ((src == 2 && tree_from_x) ? (int)a.tree_off : 0);
@@ -204,11 +205,114 @@ __device__ __attribute__((noinline)) void scan_window_impl(const ScanArgs a, Con
                 if (outl) {
                     const int rank = __popcll(m & ((1ull << lane) - 1ull));
                     sh.col_idx[base + rank] = i + (src == 2 ? (int)a.tree_off : 0);
-                    sh.col_pos[base + rank] = (unsigned short)(r * G::WY + (yy[g] - lo));
+                    sh.col_pos[base + rank] = (unsigned short)(r * G::RS + (yy[g] - lo));
                 }
             }
         }
     }
+}
+
+// Phase A of a window for the gradient with respect to the input, in gather form.  The gradient of the
+// staged patch is  gV[ci][cell] = sum_{co,t} w[co][ci][t] * gY[co][cell - off(t)],  a convolution of the
+// output gradient laid out by position (zero where the level has no output) with the flipped stencil.
+//   items    the output positions of the window including the halo rows: same-level particles, and tree
+//            nodes where they are downsampled particles;  idx addresses the output gradient
+//   columns  every cell of the centre rows that some source covers, with the place its gradient goes to:
+//            the same-level particle, the coarser particle behind two cells (one column per cell), the
+//            downsampled particle, or (COL_TREE) the node of the tree-gradient buffer
+constexpr unsigned COL_CELL = 0x0fffu;
+constexpr unsigned COL_TREE = 0x8000u;
+
+template <class G>
+__device__ __attribute__((noinline)) void scan_window_dx_impl(const ScanArgs a, ConvShared<G>& sh) {
+    const int y0 = a.y0, yn = a.yn;
+    const bool tree_from_x = a.tree_from_x, out_tree = a.out_tree;
+    constexpr int GRP = SegGroup<G>::GRP;
+    const int wave = threadIdx.x >> 6, lane = lane_id();
+    const int lo = y0 - G::HY, hi = y0 + G::TY + G::HY, lo_next = y0 + G::TY - G::HY;
+    const unsigned long long below_me = (1ull << lane) - 1ull;
+    for (int k0 = 0; k0 < G::SPW; k0 += GRP) {
+        int yy[GRP], cur[GRP];
+#pragma unroll
+        for (int g = 0; g < GRP; ++g) {
+            const int s = wave + (k0 + g) * G::NWAVE;
+            yy[g] = INT_MAX; cur[g] = 0;
+            if (s < G::NSEG) {
+                cur[g] = sh.seg_cur[s];
+                const int i = cur[g] + lane;
+                if (i < sh.seg_end[s]) yy[g] = (s % 3 == 2) ? (int)a.tree_y[i] : (int)a.apr_y[i];
+            }
+        }
+#pragma unroll
+        for (int g = 0; g < GRP; ++g) {
+            const int s = wave + (k0 + g) * G::NWAVE;
+            if (s >= G::NSEG) break;
+            const int r = s / 3, src = s - 3 * r;
+            const bool valid = yy[g] != INT_MAX;
+            const bool in = valid && (src == 1 ? yy[g] <= ((hi - 1) >> 1) : yy[g] < hi);
+            const bool below = valid && (src == 1 ? yy[g] < (lo_next >> 1) : yy[g] < lo_next);
+            const unsigned long long m_in = __ballot(in);
+            const int n_adv = __popcll(__ballot(below));
+            if (lane == 0 && n_adv) sh.seg_cur[s] = cur[g] + n_adv;
+            if (m_in == 0) continue;                                    // wave-uniform
+            const int i = cur[g] + lane;
+            if (src == 0 || (src == 2 && out_tree)) {
+                int ibase = 0;
+                if (lane == 0) ibase = atomicAdd(&sh.nitem, __popcll(m_in));
+                ibase = __shfl(ibase, 0);
+                if (in) {
+                    sh.item_idx[ibase + lane] = i + (src == 2 ? (int)a.tree_off : 0);
+                    sh.item_pos[ibase + lane] = (unsigned short)(r * G::RS + (yy[g] - lo));
+                }
+            }
+            const int rz = r / G::RX, rx = r - rz * G::RX;
+            const bool centre = rz >= G::HZ && rz < G::HZ + G::TZ && rx >= G::HX && rx < G::HX + G::TX;
+            if (!centre) continue;
+            if (src != 1) {
+                const bool outl = in && yy[g] >= y0 && yy[g] < y0 + G::TY;
+                const unsigned long long m = __ballot(outl);
+                if (m) {
+                    int base = 0;
+                    if (lane == 0) base = atomicAdd(&sh.ncol, __popcll(m));
+                    base = __shfl(base, 0);
+                    if (outl) {
+                        const int rank = __popcll(m & below_me);
+                        const bool to_tree = src == 2 && !tree_from_x;
+                        sh.col_idx[base + rank] = i + ((src == 2 && tree_from_x) ? (int)a.tree_off : 0);
+                        sh.col_pos[base + rank] = (unsigned short)((r * G::RS + (yy[g] - lo)) | (to_tree ? COL_TREE : 0u));
+                    }
+                }
+            } else {
+                const int ya = 2 * yy[g], yb = ya + 1;
+                const bool oa = in && ya >= y0 && ya < y0 + G::TY;
+                const bool ob = in && yb >= y0 && yb < y0 + G::TY && yb < yn;
+                const unsigned long long ma = __ballot(oa), mb = __ballot(ob);
+                if (ma | mb) {
+                    int base = 0;
+                    if (lane == 0) base = atomicAdd(&sh.ncol, __popcll(ma) + __popcll(mb));
+                    base = __shfl(base, 0);
+                    if (oa) {
+                        const int rank = __popcll(ma & below_me);
+                        sh.col_idx[base + rank] = i;
+                        sh.col_pos[base + rank] = (unsigned short)(r * G::RS + (ya - lo));
+                    }
+                    if (ob) {
+                        const int rank = __popcll(ma) + __popcll(mb & below_me);
+                        sh.col_idx[base + rank] = i;
+                        sh.col_pos[base + rank] = (unsigned short)(r * G::RS + (yb - lo));
+                    }
+                }
+            }
+        }
+    }
+}
+
+template <class G, typename T>
+__device__ __forceinline__ void scan_window_dx(const ConvArgs<T>& a, int L, int y0, bool out_tree, ConvShared<G>& sh) {
+    ScanArgs s;
+    s.apr_y = a.apr.y; s.tree_y = a.tree.y; s.tree_off = (int)a.tree_off; s.yn = a.apr.y_num[L]; s.y0 = y0;
+    s.tree_from_x = (L == a.Lc); s.out_tree = out_tree;
+    scan_window_dx_impl<G>(s, sh);
 }
 
 // End of a window: reset the list lengths (call between two barriers).

@@ -25,9 +25,14 @@ typedef float floatx16 __attribute__((ext_vector_type(16)));
 // Weights are re-laid out once per call into the image the kernel keeps in LDS, so that staging a chunk
 // is a straight 16-byte copy:  packed[s][cb][q][(c*K + t)][co]  with co-blocks cb of 32 output channels and
 // chunks q of CIB input channels, zero where co or ci run past the layer.
-__global__ void pack_weights_kernel(const float* __restrict__ w, int S_exp, int Cout, int Cin, int K, int CIB,
-                                    float* __restrict__ out) {
-    const int ncb = (Cout + 31) / 32, nq = (Cin + CIB - 1) / CIB, KC = CIB * K;
+//
+// With `transposed` the roles of the two channel axes are swapped and the taps reversed: the image is that
+// of the stencil of the input gradient, M = input channels, contraction over (flipped tap, output channel).
+// Cm / Ck are the channel counts of the M axis and of the contracted axis.
+__global__ void pack_weights_kernel(const float* __restrict__ w, int S_exp, int Cm, int Ck, int K, int CIB,
+                                    int transposed, float* __restrict__ out) {
+    const int Cout = transposed ? Ck : Cm, Cin = transposed ? Cm : Ck;
+    const int ncb = (Cm + 31) / 32, nq = (Ck + CIB - 1) / CIB, KC = CIB * K;
     const int64_t n = (int64_t)S_exp * ncb * nq * KC * 32;
     for (int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; e < n; e += (int64_t)gridDim.x * blockDim.x) {
         const int co = (int)(e % 32);
@@ -36,20 +41,26 @@ __global__ void pack_weights_kernel(const float* __restrict__ w, int S_exp, int 
         const int cb = (int)((e / (32 * (int64_t)KC * nq)) % ncb);
         const int s = (int)(e / (32 * (int64_t)KC * nq * ncb));
         const int c = row / K, t = row - c * K;
-        const int ci = q * CIB + c, cog = cb * 32 + co;
-        out[e] = (ci < Cin && cog < Cout) ? w[(((int64_t)s * Cout + cog) * Cin + ci) * K + t] : 0.f;
+        const int ck = q * CIB + c, cm = cb * 32 + co;
+        float v = 0.f;
+        if (ck < Ck && cm < Cm)
+            v = transposed ? w[(((int64_t)s * Cout + ck) * Cin + cm) * K + (K - 1 - t)]
+                           : w[(((int64_t)s * Cout + cm) * Cin + ck) * K + t];
+        out[e] = v;
     }
 }
 
 template <class G>
 __device__ __forceinline__ constexpr int tap_offset(int t) {
-    return ((t / (G::KX * G::KY)) * G::RX + (t / G::KY) % G::KX) * G::WY + (t % G::KY);
+    return ((t / (G::KX * G::KY)) * G::RX + (t / G::KY) % G::KX) * G::RS + (t % G::KY);
 }
 
 // One window for a wave that owns NB of the window's column blocks (blocks b with b % NWAVE == first).
 // Every instantiation runs the same staging and the same two barriers per channel chunk, so the waves
 // of a block may take different NB (0 included: the wave only helps with the staging).
-template <class G, int CIB, int NB>
+// MODE 0: forward, results stored (plus bias).  MODE 1: input gradient, results added atomically to the
+// place each column names (feature gradient, or tree gradient with COL_TREE).
+template <class G, int CIB, int NB, int MODE>
 __device__ __forceinline__ void mfma_window(const ConvArgs<float>& a, int co0, int nc, int nitem, bool tree_items, int first,
                                             const float4* __restrict__ wl, const ConvShared<G>& sh,
                                             float* __restrict__ patch, float* __restrict__ Wl,
@@ -62,7 +73,7 @@ __device__ __forceinline__ void mfma_window(const ConvArgs<float>& a, int co0, i
 #pragma unroll
     for (int j = 0; j < NB; ++j) {
         const int col = ((first + G::NWAVE * j) << 5) + (lane & 31);
-        const int pos = col < nc ? (int)sh.col_pos[col] - G::TAP0 : 0;
+        const int pos = col < nc ? (int)(sh.col_pos[col] & COL_CELL) - G::TAP0 : 0;
         bbase[j] = pos + (lane >> 5) * G::CH_STRIDE;
     }
     floatx16 acc[NBA];
@@ -116,25 +127,41 @@ __device__ __forceinline__ void mfma_window(const ConvArgs<float>& a, int co0, i
 #undef APRNET_LOAD_WEIGHTS
 #undef APRNET_STORE_WEIGHTS
     // D layout: lane l, register r -> column l%32, row 8*(r/4) + 4*(l/32) + r%4
-    float bias[16];
+    if constexpr (MODE == 0) {
+        float bias[16];
 #pragma unroll
-    for (int r = 0; r < 16; ++r) bias[r] = bias_l[8 * (r >> 2) + 4 * (lane >> 5) + (r & 3)];
+        for (int r = 0; r < 16; ++r) bias[r] = bias_l[8 * (r >> 2) + 4 * (lane >> 5) + (r & 3)];
 #pragma unroll
-    for (int j = 0; j < NB; ++j) {
-        const int col = ((first + G::NWAVE * j) << 5) + (lane & 31);
-        if (col >= nc) continue;
-        const int64_t o = sh.col_idx[col];
+        for (int j = 0; j < NB; ++j) {
+            const int col = ((first + G::NWAVE * j) << 5) + (lane & 31);
+            if (col >= nc) continue;
+            const int64_t o = sh.col_idx[col];
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-            const int co = co0 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
-            if (co < a.Cout) a.y[(int64_t)co * a.ldy + o] = acc[j][r] + bias[r];
+            for (int r = 0; r < 16; ++r) {
+                const int co = co0 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+                if (co < a.Cout) a.y[(int64_t)co * a.ldy + o] = acc[j][r] + bias[r];
+            }
+        }
+    } else {
+#pragma unroll
+        for (int j = 0; j < NB; ++j) {
+            const int col = ((first + G::NWAVE * j) << 5) + (lane & 31);
+            if (col >= nc) continue;
+            const bool to_tree = (sh.col_pos[col] & COL_TREE) != 0;
+            float* dst = (to_tree ? a.gtree : a.gx) + sh.col_idx[col];
+            const int64_t ld = to_tree ? a.ldgt : a.ldgx;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int ci = co0 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+                if (ci < a.Cout) unsafeAtomicAdd(dst + (int64_t)ci * ld, acc[j][r]);
+            }
         }
     }
 }
 
-template <class G, int CIB, int NBW>
+template <class G, int CIB, int NBW, int MODE>
 __global__ void __launch_bounds__(G::NT)
-conv_fwd_mfma_kernel(const ConvArgs<float> a) {
+conv_mfma_kernel(const ConvArgs<float> a) {
     static_assert(CIB % 2 == 0, "input channels are consumed in pairs");
     static_assert((G::NWAVE & (G::NWAVE - 1)) == 0, "block rotation assumes a power-of-two wave count");
     static_assert(NBW == 2 && (G::MAXCOL + 31) / 32 <= G::NWAVE * NBW, "a window must fit the accumulators of the block");
@@ -155,24 +182,27 @@ conv_fwd_mfma_kernel(const ConvArgs<float> a) {
                                     ((int64_t)s_idx * gridDim.y + blockIdx.y) * nq * (CIB * G::K * 8);
     const int wave = threadIdx.x >> 6;
 
-    if (threadIdx.x < 32) bias_l[threadIdx.x] = (a.bias && co0 + (int)threadIdx.x < a.Cout) ? a.bias[co0 + threadIdx.x] : 0.f;
+    if (MODE == 0 && threadIdx.x < 32)
+        bias_l[threadIdx.x] = (a.bias && co0 + (int)threadIdx.x < a.Cout) ? a.bias[co0 + threadIdx.x] : 0.f;
     open_segments<G, float>(a, L, z0, x0, sh);
     __syncthreads();
 
     int win = 0;
     for (int y0 = 0; y0 < yn; y0 += G::TY, ++win) {
-        scan_window<G, float>(a, L, y0, out_tree, sh);
+        if constexpr (MODE == 0) scan_window<G, float>(a, L, y0, out_tree, sh);
+        else scan_window_dx<G, float>(a, L, y0, out_tree, sh);
         __syncthreads();
         const int nc = __builtin_amdgcn_readfirstlane(sh.ncol), nitem = __builtin_amdgcn_readfirstlane(sh.nitem);
-        if (nc > 0) {
+        const bool tree_items = MODE == 0 && L < a.Lc;       // the output gradient has no tree part
+        if (nc > 0 && nitem > 0) {
             const int nblk = (nc + 31) >> 5;
             // rotation: spread the waves that own one block more over the SIMDs
             const int first = (wave - (int)blockIdx.x - win) & (G::NWAVE - 1);
             const int nb = first < nblk ? (nblk - first + G::NWAVE - 1) / G::NWAVE : 0;
             switch (__builtin_amdgcn_readfirstlane(nb)) {
-                case 0: mfma_window<G, CIB, 0>(a, co0, nc, nitem, L < a.Lc, first, wl, sh, patch, Wl, bias_l); break;
-                case 1: mfma_window<G, CIB, 1>(a, co0, nc, nitem, L < a.Lc, first, wl, sh, patch, Wl, bias_l); break;
-                default: mfma_window<G, CIB, 2>(a, co0, nc, nitem, L < a.Lc, first, wl, sh, patch, Wl, bias_l); break;
+                case 0: mfma_window<G, CIB, 0, MODE>(a, co0, nc, nitem, tree_items, first, wl, sh, patch, Wl, bias_l); break;
+                case 1: mfma_window<G, CIB, 1, MODE>(a, co0, nc, nitem, tree_items, first, wl, sh, patch, Wl, bias_l); break;
+                default: mfma_window<G, CIB, 2, MODE>(a, co0, nc, nitem, tree_items, first, wl, sh, patch, Wl, bias_l); break;
             }
         }
         __syncthreads();
@@ -188,19 +218,29 @@ constexpr int MFMA_CIB = 4;
 // a.w must point at the packed weights (pack_conv333_weights)
 int launch_conv333_mfma(const ConvArgs<float>& a, int n_tiles, hipStream_t st) {
     dim3 grid((unsigned)n_tiles, (unsigned)((a.Cout + 31) / 32));
-    hipLaunchKernelGGL((conv_fwd_mfma_kernel<M333, MFMA_CIB, 2>), grid, dim3(M333::NT), 0, st, a);
-    APRNET_LAUNCH_CHECK("conv_fwd_mfma_kernel");
+    hipLaunchKernelGGL((conv_mfma_kernel<M333, MFMA_CIB, 2, 0>), grid, dim3(M333::NT), 0, st, a);
+    APRNET_LAUNCH_CHECK("conv_mfma_kernel (forward)");
     return 0;
 }
 
-size_t conv333_packed_floats(int S_exp, int Cout, int Cin) {
-    return (size_t)S_exp * ((Cout + 31) / 32) * ((Cin + MFMA_CIB - 1) / MFMA_CIB) * MFMA_CIB * 27 * 32;
+// Input gradient: a.x / a.Cin describe the output gradient, a.Cout the input channels, a.w the packed
+// transposed weights, a.tiles the row groups within one cell of an output (n_tiles of them).
+int launch_conv333_dx_mfma(const ConvArgs<float>& a, int n_tiles, hipStream_t st) {
+    dim3 grid((unsigned)n_tiles, (unsigned)((a.Cout + 31) / 32));
+    hipLaunchKernelGGL((conv_mfma_kernel<M333, MFMA_CIB, 2, 1>), grid, dim3(M333::NT), 0, st, a);
+    APRNET_LAUNCH_CHECK("conv_mfma_kernel (input gradient)");
+    return 0;
 }
 
-int pack_conv333_weights(const float* w, int S_exp, int Cout, int Cin, float* packed, hipStream_t st) {
-    const size_t n = conv333_packed_floats(S_exp, Cout, Cin);
+// Cm: channels on the M axis of the kernel, Ck: contracted channels (forward: Cout, Cin; transposed: Cin, Cout)
+size_t conv333_packed_floats(int S_exp, int Cm, int Ck) {
+    return (size_t)S_exp * ((Cm + 31) / 32) * ((Ck + MFMA_CIB - 1) / MFMA_CIB) * MFMA_CIB * 27 * 32;
+}
+
+int pack_conv333_weights(const float* w, int S_exp, int Cm, int Ck, bool transposed, float* packed, hipStream_t st) {
+    const size_t n = conv333_packed_floats(S_exp, Cm, Ck);
     dim3 grid((unsigned)std::min<size_t>((n + 255) / 256, 2048));
-    hipLaunchKernelGGL(pack_weights_kernel, grid, dim3(256), 0, st, w, S_exp, Cout, Cin, 27, MFMA_CIB, packed);
+    hipLaunchKernelGGL(pack_weights_kernel, grid, dim3(256), 0, st, w, S_exp, Cm, Ck, 27, MFMA_CIB, transposed ? 1 : 0, packed);
     APRNET_LAUNCH_CHECK("pack_weights_kernel");
     return 0;
 }

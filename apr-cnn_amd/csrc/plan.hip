@@ -100,34 +100,45 @@ static void build_children(const HostAccess& apr, const HostAccess& tree, std::v
     }
 }
 
-int get_tiles(aprnet_plan* plan, int level_delta, int TZ, int TX, TileList* out) {
-    auto key = std::make_tuple(level_delta, TZ, TX);
+int plan_scratch(aprnet_plan* p, size_t bytes, hipStream_t st) {
+    if (bytes <= p->scratch_bytes) return 0;
+    if (p->d_scratch) { APRNET_HIP_CHECK(hipStreamSynchronize(st)); APRNET_HIP_CHECK(hipFree(p->d_scratch)); }
+    p->d_scratch = nullptr; p->scratch_bytes = 0;
+    APRNET_HIP_CHECK(hipMalloc(&p->d_scratch, bytes));
+    p->scratch_bytes = bytes;
+    return 0;
+}
+
+int get_tiles(aprnet_plan* plan, int level_delta, int TZ, int TX, TileList* out, int halo) {
+    auto key = std::make_tuple(level_delta, TZ, TX, halo);
     auto it = plan->tiles.find(key);
     if (it != plan->tiles.end()) { *out = it->second; return 0; }
     const HostAccess& apr = plan->apr; const HostAccess& tree = plan->tree;
     const int Lc = plan->lc(level_delta);
     std::vector<ConvTile> tiles;
+    TileList tl;
     // finest level first: it holds most of the work, the coarse levels fill the tail of the launch
     for (int l = Lc; l >= apr.level_min; --l) {
+        tl.level_begin[l] = (int)tiles.size();
         const bool with_tree = (l == Lc && l < apr.level_max);
         const int zn = apr.z_num[l], xn = apr.x_num[l];
         for (int z0 = 0; z0 < zn; z0 += TZ)
             for (int x0 = 0; x0 < xn; x0 += TX) {
                 bool any = false;
-                for (int z = z0; z < std::min(z0 + TZ, zn) && !any; ++z) {
-                    const int x1 = std::min(x0 + TX, xn) - 1;
-                    // rows x0..x1 of one z are adjacent in the row table: one range test
-                    const uint64_t ra = apr.row(l, z, x0), rb = apr.row(l, z, x1);
+                for (int z = std::max(z0 - halo, 0); z < std::min(z0 + TZ + halo, zn) && !any; ++z) {
+                    const int xa = std::max(x0 - halo, 0), x1 = std::min(x0 + TX + halo, xn) - 1;
+                    // rows xa..x1 of one z are adjacent in the row table: one range test
+                    const uint64_t ra = apr.row(l, z, xa), rb = apr.row(l, z, x1);
                     any = apr.xz_end[rb] > apr.xz_end[ra - 1];
                     if (!any && with_tree) {
-                        const uint64_t ta = tree.row(l, z, x0), tb = tree.row(l, z, x1);
+                        const uint64_t ta = tree.row(l, z, xa), tb = tree.row(l, z, x1);
                         any = tree.xz_end[tb] > tree.xz_end[ta - 1];
                     }
                 }
                 if (any) tiles.push_back(ConvTile{l, z0, x0, 0});
             }
+        tl.level_count[l] = (int)tiles.size() - tl.level_begin[l];
     }
-    TileList tl;
     tl.n = (int)tiles.size();
     if (tl.n) {
         APRNET_HIP_CHECK(hipMalloc((void**)&tl.d_tiles, tiles.size() * sizeof(ConvTile)));

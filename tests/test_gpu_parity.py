@@ -200,6 +200,45 @@ def test_conv_backward(bt, ksize, dtype):
     close(gw.permute(2, 0, 1, 3, 4, 5), gw_ref, dtype)
 
 
+@pytest.mark.parametrize("path", [0, 1], ids=["mfma", "valu"])
+@pytest.mark.parametrize("cin,cout", [(1, 16), (32, 32), (33, 33), (16, 3), (40, 64)])
+def test_conv333_backward_channel_shapes(cin, cout, path):
+    """Gradients of input and weights on both fp32 kernel families, at channel counts that fill, straddle and
+    underfill the 32-channel blocks and the 16-channel groups of the matrix-core kernels."""
+    x, aprs, ld, w_exp = _conv_case([("3d_s", 0), ("3d_t", 1)], (3, 3, 3), 2, cin, cout, torch.float32)
+    g = torch.Generator().manual_seed(6)
+    go = torch.randn(x.size(0), cout, x.size(2), generator=g)
+    gx_ref, gw_ref = oracle.conv_backward(aprs, x, w_exp, go, ld)
+    lib = _native.hip()
+    assert lib.aprnet_set_conv_path(path) == 0
+    try:
+        gx, gw = _ops.conv_backward(aprs, x.to(DEV), w_exp.permute(1, 2, 0, 3, 4, 5).contiguous().to(DEV), go.to(DEV), ld)
+    finally:
+        lib.aprnet_set_conv_path(0)
+    close(gx, gx_ref, torch.float32)
+    close(gw.permute(2, 0, 1, 3, 4, 5), gw_ref, torch.float32)
+
+
+def test_conv333_backward_dense_windows():
+    """Fully refined APR: windows with the maximum number of columns (496 > one staged group of 256 in the
+    weight-gradient kernel, all column blocks in the input-gradient kernel)."""
+    import numpy as np
+    from pyapr import APR
+    shape = (6, 10, 140)
+    apr = APR.from_level_field(shape, np.full(tuple((s + 1) // 2 for s in shape), 8, np.uint8))
+    g = torch.Generator().manual_seed(7)
+    n = apr.total_number_particles()
+    x = torch.randn(1, 6, n, generator=g)
+    w = torch.randn(6, 1, 10, 3, 3, 3, generator=g)
+    go = torch.randn(1, 10, n, generator=g)
+    ld = torch.zeros(1, dtype=torch.int32)
+    w_exp = oracle.restrict_kernel_forward(w, apr.level_max() - apr.level_min() + 1)
+    gx_ref, gw_ref = oracle.conv_backward([apr], x, w_exp, go, ld)
+    gx, gw = _ops.conv_backward([apr], x.to(DEV), w_exp.permute(1, 2, 0, 3, 4, 5).contiguous().to(DEV), go.to(DEV), ld)
+    close(gx, gx_ref, torch.float32)
+    close(gw.permute(2, 0, 1, 3, 4, 5), gw_ref, torch.float32)
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
 @pytest.mark.parametrize("ksize", [(3, 3, 3), (1, 3, 3), (1, 5, 5), (5, 5, 5)], ids=KID)
 @pytest.mark.parametrize("s,levels", [(1, 4), (2, 5), (3, 3), (3, 7)])
