@@ -167,8 +167,9 @@ __device__ __attribute__((noinline)) void scan_window_impl(const ScanArgs a, Con
         for (int g = 0; g < GRP; ++g) {
             const int s = wave + (k0 + g) * G::NWAVE;
             if (s >= G::NSEG) break;
-            const int r = s / 3, src = s - 3 * r;
             const bool valid = yy[g] != INT_MAX;
+            if (__ballot(valid) == 0) continue;                         // wave-uniform: segment is exhausted
+            const int r = s / 3, src = s - 3 * r;
             const bool in = valid && (src == 1 ? yy[g] <= ((hi - 1) >> 1) : yy[g] < hi);
             const bool below = valid && (src == 1 ? yy[g] < (lo_next >> 1) : yy[g] < lo_next);
             const unsigned long long m_in = __ballot(in);
@@ -247,8 +248,9 @@ __device__ __attribute__((noinline)) void scan_window_dx_impl(const ScanArgs a, 
         for (int g = 0; g < GRP; ++g) {
             const int s = wave + (k0 + g) * G::NWAVE;
             if (s >= G::NSEG) break;
-            const int r = s / 3, src = s - 3 * r;
             const bool valid = yy[g] != INT_MAX;
+            if (__ballot(valid) == 0) continue;                         // wave-uniform: segment is exhausted
+            const int r = s / 3, src = s - 3 * r;
             const bool in = valid && (src == 1 ? yy[g] <= ((hi - 1) >> 1) : yy[g] < hi);
             const bool below = valid && (src == 1 ? yy[g] < (lo_next >> 1) : yy[g] < lo_next);
             const unsigned long long m_in = __ballot(in);
@@ -355,47 +357,44 @@ struct ItemRegs {
 };
 
 // Issues the loads of a chunk (no LDS writes: they may run ahead of the consumer of the patch).
+// Thread t owns items t, t + NT, ...; a round k that lies beyond the item count is skipped by a
+// wave-uniform branch (most windows hold fewer items than the block has threads).
 template <class G, typename T, int CIB>
 __device__ __forceinline__ void load_items(const ConvArgs<T>& a, int ci0, int nitem, bool tree_items,
                                            const ConvShared<G>& sh, ItemRegs<G, T, CIB>& R) {
     constexpr int IPT = ItemRegs<G, T, CIB>::IPT;
-    unsigned offx[IPT], offt[IPT];
+    __amdgpu_buffer_rsrc_t rx[CIB], rt[CIB];
+#pragma unroll
+    for (int c = 0; c < CIB; ++c) {
+        rx[c] = plane_rsrc<T>(a.x, a.ldx, ci0 + c, a.Cin, a.x_count);
+        rt[c] = plane_rsrc<T>(a.tree_data, a.ldt, ci0 + c, tree_items ? a.Cin : 0, a.t_count);
+    }
 #pragma unroll
     for (int k = 0; k < IPT; ++k) {
+        if (k * G::NT >= nitem) break;                  // wave-uniform
         const int it = threadIdx.x + k * G::NT;
-        R.pos[k] = 0xffffu; offx[k] = BUF_OOB; offt[k] = BUF_OOB;
+        unsigned offx = BUF_OOB, offt = BUF_OOB;
+        R.pos[k] = 0xffffu;
         if (it < nitem) {
             const unsigned pos = sh.item_pos[it];
             const unsigned off = (unsigned)sh.item_idx[it] * (unsigned)sizeof(T);
             R.pos[k] = (unsigned short)pos;
-            if (pos & ITEM_TREE) offt[k] = off; else offx[k] = off;
-        }
-    }
-#pragma unroll
-    for (int c = 0; c < CIB; ++c) {
-        const __amdgpu_buffer_rsrc_t rx = plane_rsrc<T>(a.x, a.ldx, ci0 + c, a.Cin, a.x_count);
-#pragma unroll
-        for (int k = 0; k < IPT; ++k) R.v[k][c] = RawLoad<T>::ld(rx, offx[k]);
-    }
-    if (tree_items) {      // tile-uniform: only levels below the current maximum read the mean-filled tree
-        typename RawLoad<T>::raw tv[IPT][CIB];
-#pragma unroll
-        for (int c = 0; c < CIB; ++c) {
-            const __amdgpu_buffer_rsrc_t rt = plane_rsrc<T>(a.tree_data, a.ldt, ci0 + c, a.Cin, a.t_count);
-#pragma unroll
-            for (int k = 0; k < IPT; ++k) tv[k][c] = RawLoad<T>::ld(rt, offt[k]);
+            if (pos & ITEM_TREE) offt = off; else offx = off;
         }
 #pragma unroll
-        for (int c = 0; c < CIB; ++c)
+        for (int c = 0; c < CIB; ++c) R.v[k][c] = RawLoad<T>::ld(rx[c], offx);
+        if (tree_items) {      // tile-uniform: only levels below the current maximum read the mean-filled tree
 #pragma unroll
-            for (int k = 0; k < IPT; ++k) R.v[k][c] |= tv[k][c];      // one of the two loads returned zero
+            for (int c = 0; c < CIB; ++c) R.v[k][c] |= RawLoad<T>::ld(rt[c], offt);     // one of the two returned zero
+        }
     }
 }
 
 template <class G, typename T, int CIB>
-__device__ __forceinline__ void store_items(const ItemRegs<G, T, CIB>& R, T* patch) {
+__device__ __forceinline__ void store_items(const ItemRegs<G, T, CIB>& R, int nitem, T* patch) {
 #pragma unroll
     for (int k = 0; k < ItemRegs<G, T, CIB>::IPT; ++k) {
+        if (k * G::NT >= nitem) break;                  // wave-uniform
         if (R.pos[k] == 0xffffu) continue;
         T* cell = patch + (R.pos[k] & ITEM_CELL);
 #pragma unroll
@@ -415,7 +414,7 @@ __device__ __forceinline__ void stage_values(const ConvArgs<T>& a, int ci0, int 
                                              const ConvShared<G>& sh, T* patch) {
     ItemRegs<G, T, CIB> R;
     load_items<G, T, CIB>(a, ci0, nitem, tree_items, sh, R);
-    store_items<G, T, CIB>(R, patch);
+    store_items<G, T, CIB>(R, nitem, patch);
 }
 
 }  // namespace aprnet

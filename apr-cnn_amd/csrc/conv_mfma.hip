@@ -104,7 +104,7 @@ __device__ __forceinline__ void mfma_window(const ConvArgs<float>& a, int co0, i
     for (int i = threadIdx.x; i < CIB * G::CH_STRIDE; i += G::NT) patch[i] = 0.f;     // once per window
     for (int ci0 = 0; ci0 < a.Cin; ci0 += CIB) {
         __syncthreads();            // zeros are in place / the previous chunk's MFMAs have read patch and Wl
-        store_items<G, float, CIB>(R, patch);
+        store_items<G, float, CIB>(R, nitem, patch);
         APRNET_STORE_WEIGHTS()
         __syncthreads();
         if (ci0 + CIB < a.Cin) {
