@@ -20,15 +20,106 @@ conv111_kernel(const T* __restrict__ src, int64_t lds, int Csrc, const T* __rest
     T acc[OB];
 #pragma unroll
     for (int o = 0; o < OB; ++o) acc[o] = 0;
-    for (int c = 0; c < Csrc; ++c) {
-        const T v = src[(int64_t)c * lds + i];
+    constexpr int CU = 8;            // input channels loaded together: eight independent loads in flight
+    for (int c0 = 0; c0 < Csrc; c0 += CU) {
+        T v[CU];
 #pragma unroll
-        for (int o = 0; o < OB; ++o)
-            if (o0 + o < Cdst) acc[o] += w[(int64_t)(o0 + o) * so + (int64_t)c * sc] * v;
+        for (int k = 0; k < CU; ++k) v[k] = c0 + k < Csrc ? src[(int64_t)(c0 + k) * lds + i] : (T)0;
+#pragma unroll
+        for (int k = 0; k < CU; ++k) {
+            if (c0 + k >= Csrc) break;
+#pragma unroll
+            for (int o = 0; o < OB; ++o)
+                if (o0 + o < Cdst) acc[o] += w[(int64_t)(o0 + o) * so + (int64_t)(c0 + k) * sc] * v[k];
+        }
     }
 #pragma unroll
     for (int o = 0; o < OB; ++o)
         if (o0 + o < Cdst) dst[(int64_t)(o0 + o) * ldd + i] = acc[o] + (bias ? bias[o0 + o] : (T)0);
+}
+
+// The same product on the matrix cores (fp32): M = 32 outputs, N = 32 positions, K = input channels two at a
+// time.  v_mfma_f32_32x32x2_f32 takes  A: lane l -> W(o = l%32, c = 2p + l/32)  (kept in registers for the
+// whole kernel) and  B: lane l -> src[c = 2p + l/32][i0 + l%32]  (two coalesced 128-byte rows per load), so
+// the kernel streams the input once per 32 output channels and is bound by HBM.
+typedef float floatx16_111 __attribute__((ext_vector_type(16)));
+
+template <int KP>      // KP = channel pairs held in registers (ceil(Csrc / 2) <= KP)
+__global__ void __launch_bounds__(TB1)
+conv111_mfma_kernel(const float* __restrict__ src, int64_t lds, int Csrc, const float* __restrict__ w, int so, int sc,
+                    const float* __restrict__ bias, float* __restrict__ dst, int64_t ldd, int Cdst, int64_t begin,
+                    int64_t end) {
+    const int lane = threadIdx.x & 63, hi = lane >> 5, col = lane & 31;
+    const int o0 = blockIdx.y * 32;
+    float aw[KP];
+#pragma unroll
+    for (int p = 0; p < KP; ++p) {
+        const int c = 2 * p + hi, o = o0 + col;
+        aw[p] = (c < Csrc && o < Cdst) ? w[(int64_t)o * so + (int64_t)c * sc] : 0.f;
+    }
+    float bs[16];
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+        const int o = o0 + 8 * (r >> 2) + 4 * hi + (r & 3);
+        bs[r] = (bias && o < Cdst) ? bias[o] : 0.f;
+    }
+    const int64_t nwave = (int64_t)gridDim.x * (TB1 / 64);
+    const int64_t wave = (int64_t)blockIdx.x * (TB1 / 64) + (threadIdx.x >> 6);
+    for (int64_t i0 = begin + wave * 64; i0 < end; i0 += nwave * 64) {
+        const int64_t ia = i0 + col, ib = i0 + 32 + col;
+        float va[KP], vb[KP];
+#pragma unroll
+        for (int p = 0; p < KP; ++p) {
+            const int c = 2 * p + hi;
+            const float* row = src + (int64_t)c * lds;
+            va[p] = (c < Csrc && ia < end) ? row[ia] : 0.f;
+            vb[p] = (c < Csrc && ib < end) ? row[ib] : 0.f;
+        }
+        floatx16_111 acca, accb;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) { acca[r] = bs[r]; accb[r] = bs[r]; }
+#pragma unroll
+        for (int p = 0; p < KP; ++p) {
+            acca = __builtin_amdgcn_mfma_f32_32x32x2f32(aw[p], va[p], acca, 0, 0, 0);
+            accb = __builtin_amdgcn_mfma_f32_32x32x2f32(aw[p], vb[p], accb, 0, 0, 0);
+        }
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const int o = o0 + 8 * (r >> 2) + 4 * hi + (r & 3);
+            if (o < Cdst) {
+                if (ia < end) dst[(int64_t)o * ldd + ia] = acca[r];
+                if (ib < end) dst[(int64_t)o * ldd + ib] = accb[r];
+            }
+        }
+    }
+}
+
+// dispatch on the number of channel pairs kept in registers; false when the layer is too wide for this kernel
+static bool launch_conv111_mfma(const float* src, int64_t lds, int Csrc, const float* w, int so, int sc, const float* bias,
+                                float* dst, int64_t ldd, int Cdst, int64_t begin, int64_t end, hipStream_t st) {
+    const int kp = (Csrc + 1) / 2;
+    const int64_t n = end - begin;
+    dim3 grid((unsigned)std::min<int64_t>((n + 255) / 256, 256 * 8), (unsigned)((Cdst + 31) / 32));
+#define APRNET_111(KP) hipLaunchKernelGGL((conv111_mfma_kernel<KP>), grid, dim3(TB1), 0, st, src, lds, Csrc, w, so, sc, bias, \
+                                          dst, ldd, Cdst, begin, end)
+    if (kp <= 8) APRNET_111(8);
+    else if (kp <= 16) APRNET_111(16);
+    else if (kp <= 32) APRNET_111(32);
+    else if (kp <= 64) APRNET_111(64);
+    else return false;
+#undef APRNET_111
+    return true;
+}
+template <typename T>
+static bool try_conv111_mfma(const T*, int64_t, int, const T*, int, int, const T*, T*, int64_t, int, int64_t, int64_t, hipStream_t) {
+    return false;
+}
+int conv_path();
+template <>
+bool try_conv111_mfma<float>(const float* src, int64_t lds, int Csrc, const float* w, int so, int sc, const float* bias,
+                             float* dst, int64_t ldd, int Cdst, int64_t begin, int64_t end, hipStream_t st) {
+    if (conv_path() == 1) return false;
+    return launch_conv111_mfma(src, lds, Csrc, w, so, sc, bias, dst, ldd, Cdst, begin, end, st);
 }
 
 // gw[co][ci] += sum_i gy[co][i] * x[ci][i] over [begin, end): 8x8 register tile per thread, block
@@ -99,11 +190,19 @@ int conv111_fwd(const aprnet_plan* p, int d, const T* x, int64_t ldx, int Cin, c
     if (int rc = check_level_delta(p, d, "conv111_forward")) return rc;
     if (Cin <= 0 || Cout <= 0 || S <= 0) return fail(APRNET_ERR_INVALID_ARGUMENT, "conv111_forward: empty channel / stencil count");
     APRNET_HIP_CHECK(hipSetDevice(p->device));
-    constexpr int OB = 16;
+    // 32 outputs per thread when the layer has more than 16: the input is then read once per 32 output channels
     for (const Segment& sg : segments(p, d, S)) {
-        dim3 grid((unsigned)((sg.end - sg.begin + TB1 - 1) / TB1), (unsigned)((Cout + OB - 1) / OB));
-        hipLaunchKernelGGL((conv111_kernel<T, OB>), grid, dim3(TB1), 0, st, x, ldx, Cin, w + (int64_t)sg.stencil * Cout * Cin,
-                           Cin, 1, bias, y, ldy, Cout, sg.begin, sg.end);
+        const T* ws = w + (int64_t)sg.stencil * Cout * Cin;
+        if (try_conv111_mfma<T>(x, ldx, Cin, ws, Cin, 1, bias, y, ldy, Cout, sg.begin, sg.end, st)) continue;
+        if (Cout > 16) {
+            dim3 grid((unsigned)((sg.end - sg.begin + TB1 - 1) / TB1), (unsigned)((Cout + 31) / 32));
+            hipLaunchKernelGGL((conv111_kernel<T, 32>), grid, dim3(TB1), 0, st, x, ldx, Cin, ws, Cin, 1, bias, y, ldy, Cout,
+                               sg.begin, sg.end);
+        } else {
+            dim3 grid((unsigned)((sg.end - sg.begin + TB1 - 1) / TB1), 1u);
+            hipLaunchKernelGGL((conv111_kernel<T, 16>), grid, dim3(TB1), 0, st, x, ldx, Cin, ws, Cin, 1, bias, y, ldy, Cout,
+                               sg.begin, sg.end);
+        }
     }
     APRNET_LAUNCH_CHECK("conv111_kernel");
     return 0;
@@ -120,8 +219,9 @@ int conv111_bwd(const aprnet_plan* p, int d, const T* x, int64_t ldx, int Cin, c
         const T* ws = w + (int64_t)sg.stencil * Cout * Cin;
         dim3 grid((unsigned)((sg.end - sg.begin + TB1 - 1) / TB1), (unsigned)((Cin + OB - 1) / OB));
         // grad_x[ci][i] = sum_co w[co][ci] * gy[co][i]: the same kernel with the weight strides swapped
-        hipLaunchKernelGGL((conv111_kernel<T, OB>), grid, dim3(TB1), 0, st, gy, ldy, Cout, ws, 1, Cin, (const T*)nullptr, gx, ldgx, Cin,
-                           sg.begin, sg.end);
+        if (!try_conv111_mfma<T>(gy, ldy, Cout, ws, 1, Cin, (const T*)nullptr, gx, ldgx, Cin, sg.begin, sg.end, st))
+            hipLaunchKernelGGL((conv111_kernel<T, OB>), grid, dim3(TB1), 0, st, gy, ldy, Cout, ws, 1, Cin, (const T*)nullptr, gx, ldgx, Cin,
+                               sg.begin, sg.end);
         const int64_t n = sg.end - sg.begin;
         dim3 g2((unsigned)std::min<int64_t>((n + TB1 * 8 - 1) / (TB1 * 8), 256), (unsigned)((Cout + 7) / 8), (unsigned)((Cin + 7) / 8));
         hipLaunchKernelGGL(conv111_dw_kernel<T>, g2, dim3(TB1), 0, st, x, ldx, Cin, gy, ldy, Cout,

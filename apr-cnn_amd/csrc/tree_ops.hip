@@ -1,12 +1,14 @@
 // Child-table operators: bottom-up tree fill (mean of children), max-pool with argmax, constant
 // upsampling, and their backward passes.  All are HBM-bound gathers/scatters: one thread per
-// (tree node, channel), tree nodes of one level are contiguous, so every access is coalesced
-// along the node index and the eight child slots are read from slot-major planes.
+// (tree node, group of CPT channels), tree nodes of one level are contiguous, so every access is
+// coalesced along the node index and the eight child slots are read from slot-major planes, once for
+// the CPT channels of the thread (the index traffic would otherwise equal the data traffic).
 #include "common.hpp"
 
 namespace aprnet {
 
 constexpr int TB = 256;
+constexpr int CPT = 4;          // channels per thread
 
 template <typename T>
 struct ChildView {
@@ -22,56 +24,66 @@ struct ChildView {
 template <typename T>
 __global__ void __launch_bounds__(TB)
 fill_tree_level_kernel(const int32_t* __restrict__ children, int64_t n_tree, int64_t t_begin, int64_t t_end,
-                       const T* __restrict__ x, int64_t ldx, T* __restrict__ tree, int64_t ldt,
+                       const T* __restrict__ x, int64_t ldx, int C, T* __restrict__ tree, int64_t ldt,
                        int64_t tree_off, int tree_child_from_x, int tree_first) {
     const int64_t t = t_begin + (int64_t)blockIdx.x * TB + threadIdx.x;
     if (t >= t_end) return;
-    const int c = blockIdx.y;
-    const T* xc = x + (int64_t)c * ldx;
-    T* tc = tree + (int64_t)c * ldt;
     int32_t ch[8];
     int cnt = 0;
 #pragma unroll
     for (int s = 0; s < 8; ++s) { ch[s] = children[(int64_t)s * n_tree + t]; cnt += ch[s] != NO_CHILD; }
-    T sum = 0;
-#pragma unroll
-    for (int pass = 0; pass < 2; ++pass) {
-        const bool want_tree = (pass == 0) == (tree_first != 0);
-#pragma unroll
-        for (int s = 0; s < 8; ++s) {
-            const int32_t v = ch[s];
-            if (v == NO_CHILD) continue;
-            if (want_tree && v < 0) sum += tree_child_from_x ? xc[(int64_t)(~v) + tree_off] : tc[~v];
-            if (!want_tree && v >= 0) sum += xc[v];
-        }
-    }
     // 1/cnt is a power of two (cnt = product of 1-or-2 per dimension, helpers.hpp:133-153)
-    tc[t] = sum * (T)(1.0f / (float)max(cnt, 1));
+    const T scale = (T)(1.0f / (float)max(cnt, 1));
+#pragma unroll
+    for (int k = 0; k < CPT; ++k) {
+        const int c = blockIdx.y * CPT + k;
+        if (c >= C) break;
+        const T* xc = x + (int64_t)c * ldx;
+        T* tc = tree + (int64_t)c * ldt;
+        T sum = 0;
+#pragma unroll
+        for (int pass = 0; pass < 2; ++pass) {
+            const bool want_tree = (pass == 0) == (tree_first != 0);
+#pragma unroll
+            for (int s = 0; s < 8; ++s) {
+                const int32_t v = ch[s];
+                if (v == NO_CHILD) continue;
+                if (want_tree && v < 0) sum += tree_child_from_x ? xc[(int64_t)(~v) + tree_off] : tc[~v];
+                if (!want_tree && v >= 0) sum += xc[v];
+            }
+        }
+        tc[t] = sum * scale;
+    }
 }
 
 // helpers.hpp:255-350, parent-driven: every child has exactly one parent, so no write conflicts.
 template <typename T>
 __global__ void __launch_bounds__(TB)
 fill_tree_bwd_level_kernel(const int32_t* __restrict__ children, int64_t n_tree, int64_t t_begin, int64_t t_end,
-                           T* __restrict__ gx, int64_t ldx, T* __restrict__ gtree, int64_t ldt,
+                           T* __restrict__ gx, int64_t ldx, int C, T* __restrict__ gtree, int64_t ldt,
                            int64_t tree_off, int tree_child_in_x) {
     const int64_t t = t_begin + (int64_t)blockIdx.x * TB + threadIdx.x;
     if (t >= t_end) return;
-    const int c = blockIdx.y;
-    T* gxc = gx + (int64_t)c * ldx;
-    T* gtc = gtree + (int64_t)c * ldt;
     int32_t ch[8];
     int cnt = 0;
 #pragma unroll
     for (int s = 0; s < 8; ++s) { ch[s] = children[(int64_t)s * n_tree + t]; cnt += ch[s] != NO_CHILD; }
-    const T g = gtc[t] * (T)(1.0f / (float)max(cnt, 1));
+    const T scale = (T)(1.0f / (float)max(cnt, 1));
 #pragma unroll
-    for (int s = 0; s < 8; ++s) {
-        const int32_t v = ch[s];
-        if (v == NO_CHILD) continue;
-        if (v >= 0) gxc[v] += g;
-        else if (tree_child_in_x) gxc[(int64_t)(~v) + tree_off] += g;
-        else gtc[~v] += g;
+    for (int k = 0; k < CPT; ++k) {
+        const int c = blockIdx.y * CPT + k;
+        if (c >= C) break;
+        T* gxc = gx + (int64_t)c * ldx;
+        T* gtc = gtree + (int64_t)c * ldt;
+        const T g = gtc[t] * scale;
+#pragma unroll
+        for (int s = 0; s < 8; ++s) {
+            const int32_t v = ch[s];
+            if (v == NO_CHILD) continue;
+            if (v >= 0) gxc[v] += g;
+            else if (tree_child_in_x) gxc[(int64_t)(~v) + tree_off] += g;
+            else gtc[~v] += g;
+        }
     }
 }
 
@@ -81,35 +93,47 @@ fill_tree_bwd_level_kernel(const int32_t* __restrict__ children, int64_t n_tree,
 template <typename T>
 __global__ void __launch_bounds__(TB)
 maxpool_fwd_kernel(const int32_t* __restrict__ children, int64_t n_tree, int64_t n_copy, int64_t n_out,
-                   int64_t t_begin, const T* __restrict__ x, int64_t ldx, T* __restrict__ y, int64_t ldy,
+                   int64_t t_begin, const T* __restrict__ x, int64_t ldx, int C, T* __restrict__ y, int64_t ldy,
                    int64_t* __restrict__ arg, int64_t ldi, int64_t in_tree_off) {
     const int64_t i = (int64_t)blockIdx.x * TB + threadIdx.x;
     if (i >= n_out) return;
-    const int c = blockIdx.y;
-    const T* xc = x + (int64_t)c * ldx;
-    if (i < n_copy) { y[(int64_t)c * ldy + i] = xc[i]; arg[(int64_t)c * ldi + i] = 0; return; }
+    if (i < n_copy) {
+#pragma unroll
+        for (int k = 0; k < CPT; ++k) {
+            const int c = blockIdx.y * CPT + k;
+            if (c >= C) break;
+            y[(int64_t)c * ldy + i] = x[(int64_t)c * ldx + i]; arg[(int64_t)c * ldi + i] = 0;
+        }
+        return;
+    }
     const int64_t t = t_begin + (i - n_copy);
-    T best = (T)(-1e17f);               // initial value of the output, maxpool.hpp:51
-    int64_t best_i = 0;
     int32_t ch[8];
 #pragma unroll
     for (int s = 0; s < 8; ++s) ch[s] = children[(int64_t)s * n_tree + t];
 #pragma unroll
-    for (int s = 0; s < 8; ++s) {
-        const int32_t v = ch[s];
-        if (v >= 0) { const T val = xc[v]; if (val > best) { best = val; best_i = v; } }
-    }
+    for (int k = 0; k < CPT; ++k) {
+        const int c = blockIdx.y * CPT + k;
+        if (c >= C) break;
+        const T* xc = x + (int64_t)c * ldx;
+        T best = (T)(-1e17f);               // initial value of the output, maxpool.hpp:51
+        int64_t best_i = 0;
 #pragma unroll
-    for (int s = 0; s < 8; ++s) {
-        const int32_t v = ch[s];
-        if (v < 0 && v != NO_CHILD) {
-            const int64_t j = (int64_t)(~v) + in_tree_off;
-            const T val = xc[j];
-            if (val > best) { best = val; best_i = j; }
+        for (int s = 0; s < 8; ++s) {
+            const int32_t v = ch[s];
+            if (v >= 0) { const T val = xc[v]; if (val > best) { best = val; best_i = v; } }
         }
+#pragma unroll
+        for (int s = 0; s < 8; ++s) {
+            const int32_t v = ch[s];
+            if (v < 0 && v != NO_CHILD) {
+                const int64_t j = (int64_t)(~v) + in_tree_off;
+                const T val = xc[j];
+                if (val > best) { best = val; best_i = j; }
+            }
+        }
+        y[(int64_t)c * ldy + i] = best;
+        arg[(int64_t)c * ldi + i] = best_i;
     }
-    y[(int64_t)c * ldy + i] = best;
-    arg[(int64_t)c * ldi + i] = best_i;
 }
 
 // maxpool.hpp:170-230 without the zero-fill pass: every input position of level Lc has exactly one
@@ -117,22 +141,37 @@ maxpool_fwd_kernel(const int32_t* __restrict__ children, int64_t n_tree, int64_t
 template <typename T>
 __global__ void __launch_bounds__(TB)
 maxpool_bwd_kernel(const int32_t* __restrict__ children, int64_t n_tree, int64_t n_copy, int64_t n_out,
-                   int64_t t_begin, const T* __restrict__ gy, int64_t ldy, T* __restrict__ gx, int64_t ldx,
+                   int64_t t_begin, const T* __restrict__ gy, int64_t ldy, int C, T* __restrict__ gx, int64_t ldx,
                    const int64_t* __restrict__ arg, int64_t ldi, int64_t in_tree_off) {
     const int64_t i = (int64_t)blockIdx.x * TB + threadIdx.x;
     if (i >= n_out) return;
-    const int c = blockIdx.y;
-    T* gxc = gx + (int64_t)c * ldx;
-    const T g = gy[(int64_t)c * ldy + i];
-    if (i < n_copy) { gxc[i] = g; return; }
-    const int64_t t = t_begin + (i - n_copy);
-    const int64_t m = arg[(int64_t)c * ldi + i];
+    if (i < n_copy) {
 #pragma unroll
-    for (int s = 0; s < 8; ++s) {
-        const int32_t v = children[(int64_t)s * n_tree + t];
-        if (v == NO_CHILD) continue;
-        const int64_t j = v >= 0 ? (int64_t)v : (int64_t)(~v) + in_tree_off;
-        gxc[j] = (j == m) ? g : (T)0;
+        for (int k = 0; k < CPT; ++k) {
+            const int c = blockIdx.y * CPT + k;
+            if (c >= C) break;
+            gx[(int64_t)c * ldx + i] = gy[(int64_t)c * ldy + i];
+        }
+        return;
+    }
+    const int64_t t = t_begin + (i - n_copy);
+    int32_t ch[8];
+#pragma unroll
+    for (int s = 0; s < 8; ++s) ch[s] = children[(int64_t)s * n_tree + t];
+#pragma unroll
+    for (int k = 0; k < CPT; ++k) {
+        const int c = blockIdx.y * CPT + k;
+        if (c >= C) break;
+        T* gxc = gx + (int64_t)c * ldx;
+        const T g = gy[(int64_t)c * ldy + i];
+        const int64_t m = arg[(int64_t)c * ldi + i];
+#pragma unroll
+        for (int s = 0; s < 8; ++s) {
+            const int32_t v = ch[s];
+            if (v == NO_CHILD) continue;
+            const int64_t j = v >= 0 ? (int64_t)v : (int64_t)(~v) + in_tree_off;
+            gxc[j] = (j == m) ? g : (T)0;
+        }
     }
 }
 
@@ -142,33 +181,45 @@ maxpool_bwd_kernel(const int32_t* __restrict__ children, int64_t n_tree, int64_t
 template <typename T, bool Backward>
 __global__ void __launch_bounds__(TB)
 upsample_kernel(const int32_t* __restrict__ children, int64_t n_tree, int64_t n_copy, int64_t n_in,
-                int64_t t_begin, const T* __restrict__ src, int64_t lds, T* __restrict__ dst, int64_t ldd,
+                int64_t t_begin, const T* __restrict__ src, int64_t lds, int C, T* __restrict__ dst, int64_t ldd,
                 int64_t out_tree_off) {
     const int64_t i = (int64_t)blockIdx.x * TB + threadIdx.x;
     if (i >= n_in) return;
-    const int c = blockIdx.y;
     // forward: src = input at d, dst = output at d-1.  backward: src = grad_output, dst = grad_input.
-    const T* s_ = src + (int64_t)c * lds;
-    T* d_ = dst + (int64_t)c * ldd;
-    if (i < n_copy) { d_[i] = s_[i]; return; }
+    if (i < n_copy) {
+#pragma unroll
+        for (int k = 0; k < CPT; ++k) {
+            const int c = blockIdx.y * CPT + k;
+            if (c >= C) break;
+            dst[(int64_t)c * ldd + i] = src[(int64_t)c * lds + i];
+        }
+        return;
+    }
     const int64_t t = t_begin + (i - n_copy);
     int32_t ch[8];
 #pragma unroll
     for (int s = 0; s < 8; ++s) ch[s] = children[(int64_t)s * n_tree + t];
-    if (!Backward) {
-        const T v = s_[i];
 #pragma unroll
-        for (int s = 0; s < 8; ++s) {
-            if (ch[s] == NO_CHILD) continue;
-            d_[ch[s] >= 0 ? (int64_t)ch[s] : (int64_t)(~ch[s]) + out_tree_off] = v;
+    for (int k = 0; k < CPT; ++k) {
+        const int c = blockIdx.y * CPT + k;
+        if (c >= C) break;
+        const T* s_ = src + (int64_t)c * lds;
+        T* d_ = dst + (int64_t)c * ldd;
+        if (!Backward) {
+            const T v = s_[i];
+#pragma unroll
+            for (int s = 0; s < 8; ++s) {
+                if (ch[s] == NO_CHILD) continue;
+                d_[ch[s] >= 0 ? (int64_t)ch[s] : (int64_t)(~ch[s]) + out_tree_off] = v;
+            }
+        } else {
+            T sum = 0;      // particles first, then tree nodes (upsample.hpp:199-232)
+#pragma unroll
+            for (int s = 0; s < 8; ++s) if (ch[s] >= 0) sum += s_[ch[s]];
+#pragma unroll
+            for (int s = 0; s < 8; ++s) if (ch[s] < 0 && ch[s] != NO_CHILD) sum += s_[(int64_t)(~ch[s]) + out_tree_off];
+            d_[i] = sum;
         }
-    } else {
-        T sum = 0;      // particles first, then tree nodes (upsample.hpp:199-232)
-#pragma unroll
-        for (int s = 0; s < 8; ++s) if (ch[s] >= 0) sum += s_[ch[s]];
-#pragma unroll
-        for (int s = 0; s < 8; ++s) if (ch[s] < 0 && ch[s] != NO_CHILD) sum += s_[(int64_t)(~ch[s]) + out_tree_off];
-        d_[i] = sum;
     }
 }
 
@@ -182,9 +233,9 @@ int fill_tree_mean(const aprnet_plan* p, int d, const T* x, int64_t ldx, int C, 
     for (int l = std::min(Lc - 1, p->tree.level_max); l >= p->tree.level_min; --l) {
         const int64_t b = p->tree.level_begin(l), e = p->tree.level_end(l);
         if (e <= b) continue;
-        dim3 grid((unsigned)((e - b + TB - 1) / TB), (unsigned)C);
+        dim3 grid((unsigned)((e - b + TB - 1) / TB), (unsigned)((C + CPT - 1) / CPT));
         const int from_x = (l + 1 == Lc);
-        hipLaunchKernelGGL(fill_tree_level_kernel<T>, grid, dim3(TB), 0, st, p->d_children, p->n_tree, b, e, x, ldx,
+        hipLaunchKernelGGL(fill_tree_level_kernel<T>, grid, dim3(TB), 0, st, p->d_children, p->n_tree, b, e, x, ldx, C,
                            tree, ldt, from_x ? p->tree_offset(Lc) : 0, from_x, from_x);
     }
     APRNET_LAUNCH_CHECK("fill_tree_level_kernel");
@@ -199,9 +250,9 @@ int fill_tree_mean_bwd(const aprnet_plan* p, int d, T* gx, int64_t ldx, int C, T
     for (int l = p->tree.level_min; l <= std::min(Lc - 1, p->tree.level_max); ++l) {
         const int64_t b = p->tree.level_begin(l), e = p->tree.level_end(l);
         if (e <= b) continue;
-        dim3 grid((unsigned)((e - b + TB - 1) / TB), (unsigned)C);
+        dim3 grid((unsigned)((e - b + TB - 1) / TB), (unsigned)((C + CPT - 1) / CPT));
         const int in_x = (l + 1 == Lc);
-        hipLaunchKernelGGL(fill_tree_bwd_level_kernel<T>, grid, dim3(TB), 0, st, p->d_children, p->n_tree, b, e, gx, ldx,
+        hipLaunchKernelGGL(fill_tree_bwd_level_kernel<T>, grid, dim3(TB), 0, st, p->d_children, p->n_tree, b, e, gx, ldx, C,
                            gtree, ldt, in_x ? p->tree_offset(Lc) : 0, in_x);
     }
     APRNET_LAUNCH_CHECK("fill_tree_bwd_level_kernel");
@@ -216,9 +267,9 @@ int maxpool_fwd(const aprnet_plan* p, int d, const T* x, int64_t ldx, int C, T* 
     if (Lc - 1 < p->tree.level_min) return fail(APRNET_ERR_LEVEL_DELTA, "maxpool_forward: nothing left to pool");
     const int64_t n_out = p->number_parts(d + 1), n_copy = p->apr.level_end(Lc - 1);
     if (C <= 0 || n_out <= 0) return 0;
-    dim3 grid((unsigned)((n_out + TB - 1) / TB), (unsigned)C);
+    dim3 grid((unsigned)((n_out + TB - 1) / TB), (unsigned)((C + CPT - 1) / CPT));
     hipLaunchKernelGGL(maxpool_fwd_kernel<T>, grid, dim3(TB), 0, st, p->d_children, p->n_tree, n_copy, n_out,
-                       p->tree.level_begin(Lc - 1), x, ldx, y, ldy, arg, ldi, p->tree_offset(Lc));
+                       p->tree.level_begin(Lc - 1), x, ldx, C, y, ldy, arg, ldi, p->tree_offset(Lc));
     APRNET_LAUNCH_CHECK("maxpool_fwd_kernel");
     return 0;
 }
@@ -231,9 +282,9 @@ int maxpool_bwd(const aprnet_plan* p, int d, const T* gy, int64_t ldy, int C, T*
     if (Lc - 1 < p->tree.level_min) return fail(APRNET_ERR_LEVEL_DELTA, "maxpool_backward: invalid level delta");
     const int64_t n_out = p->number_parts(d + 1), n_copy = p->apr.level_end(Lc - 1);
     if (C <= 0 || n_out <= 0) return 0;
-    dim3 grid((unsigned)((n_out + TB - 1) / TB), (unsigned)C);
+    dim3 grid((unsigned)((n_out + TB - 1) / TB), (unsigned)((C + CPT - 1) / CPT));
     hipLaunchKernelGGL(maxpool_bwd_kernel<T>, grid, dim3(TB), 0, st, p->d_children, p->n_tree, n_copy, n_out,
-                       p->tree.level_begin(Lc - 1), gy, ldy, gx, ldx, arg, ldi, p->tree_offset(Lc));
+                       p->tree.level_begin(Lc - 1), gy, ldy, C, gx, ldx, arg, ldi, p->tree_offset(Lc));
     APRNET_LAUNCH_CHECK("maxpool_bwd_kernel");
     return 0;
 }
@@ -247,9 +298,9 @@ int upsample(const aprnet_plan* p, int d, const T* src, int64_t lds, int C, T* d
     const int Lc = p->lc(d);
     const int64_t n_in = p->number_parts(d), n_copy = p->apr.level_end(Lc);
     if (C <= 0 || n_in <= 0) return 0;
-    dim3 grid((unsigned)((n_in + TB - 1) / TB), (unsigned)C);
+    dim3 grid((unsigned)((n_in + TB - 1) / TB), (unsigned)((C + CPT - 1) / CPT));
     hipLaunchKernelGGL((upsample_kernel<T, Backward>), grid, dim3(TB), 0, st, p->d_children, p->n_tree, n_copy, n_in,
-                       p->tree.level_begin(Lc), src, lds, dst, ldd, p->tree_offset(Lc + 1));
+                       p->tree.level_begin(Lc), src, lds, C, dst, ldd, p->tree_offset(Lc + 1));
     APRNET_LAUNCH_CHECK("upsample_kernel");
     return 0;
 }
