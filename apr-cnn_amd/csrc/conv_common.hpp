@@ -36,7 +36,7 @@ struct ConvArgs {
     const T* gy; T* gx; int64_t ldgx; T* gtree; int64_t ldgt; T* gw; int n_tiles;
 };
 
-template <int KZ_, int KX_, int KY_, int TZ_, int TX_, int NT_, int RS_ = 64>
+template <int KZ_, int KX_, int KY_, int TZ_, int TX_, int NT_, int RS_ = 64, int PAD_ = 32>
 struct ConvGeom {
     static constexpr int KZ = KZ_, KX = KX_, KY = KY_, TZ = TZ_, TX = TX_, NT = NT_;
     static constexpr int RS = RS_;                // words between two staged rows of one channel (>= WY)
@@ -52,9 +52,10 @@ struct ConvGeom {
     static constexpr int MAXCOL = TZ * TX * TY;
     static constexpr int MAXITEM = NROW * WY;                  // every staged cell is filled by at most one item
     static constexpr int ITER = (MAXCOL + NT - 1) / NT;        // output columns per thread
-    // patch elements per channel; the extra 32 words put the two channels of an MFMA pair (lanes l and
-    // l+32 read the same cell of adjacent channels) on different halves of the LDS banks
-    static constexpr int CH_STRIDE = (NROW * RS + 63) / 64 * 64 + 32;
+    // patch elements per channel; the extra PAD words put the channels that one MFMA operand read touches
+    // (lanes l and l+32 read the same cell of adjacent channels, PAD 32; four lane groups of 16 read four
+    // channels, PAD 16) on different parts of the 64 LDS banks
+    static constexpr int CH_STRIDE = (NROW * RS + 63) / 64 * 64 + PAD_;
     static constexpr int TAP0 = (HZ * RX + HX) * RS + HY;      // centre -> first tap
 };
 

@@ -211,6 +211,180 @@ conv_mfma_kernel(const ConvArgs<float> a) {
     }
 }
 
+// ---------------------------------------------------------------------------------------------------------
+// Layers with at most 16 output channels: v_mfma_f32_16x16x4_f32, M = 16 output channels, N = 16 columns,
+// K = the four input channels of a chunk at one tap.
+//     A: lane l -> W[co = l%16][ci = l/16]      B: lane l -> patch[ci = l/16][cell of column l%16 + off(t)]
+//     D: lane l, register r -> column l%16, output channel 4*(l/16) + r
+// Half the matrix work of the 32-row kernel for these layers; a wave owns up to four blocks of 16 columns.
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+
+// packed16[s][cb][q][t][c][16 co]: the chunk image is linear in (t, lane)
+__global__ void pack_weights16_kernel(const float* __restrict__ w, int S_exp, int Cout, int Cin, int K, int CIB,
+                                      float* __restrict__ out) {
+    const int ncb = (Cout + 15) / 16, nq = (Cin + CIB - 1) / CIB;
+    const int64_t n = (int64_t)S_exp * ncb * nq * K * CIB * 16;
+    for (int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; e < n; e += (int64_t)gridDim.x * blockDim.x) {
+        const int co = (int)(e % 16);
+        const int c = (int)((e / 16) % CIB);
+        const int t = (int)((e / (16 * CIB)) % K);
+        const int q = (int)((e / (16 * (int64_t)CIB * K)) % nq);
+        const int cb = (int)((e / (16 * (int64_t)CIB * K * nq)) % ncb);
+        const int s = (int)(e / (16 * (int64_t)CIB * K * nq * ncb));
+        const int ci = q * CIB + c, cog = cb * 16 + co;
+        out[e] = (ci < Cin && cog < Cout) ? w[(((int64_t)s * Cout + cog) * Cin + ci) * K + t] : 0.f;
+    }
+}
+
+template <class G, int NB>
+__device__ __forceinline__ void mfma16_window(const ConvArgs<float>& a, int co0, int nc, int nitem, bool tree_items, int first,
+                                              const float4* __restrict__ wl, const ConvShared<G>& sh,
+                                              float* __restrict__ patch, float* __restrict__ Wl,
+                                              const float* __restrict__ bias_l) {
+    constexpr int CIB = 4;
+    constexpr int KC = CIB * G::K;             // k rows per chunk
+    const int lane = lane_id();
+    constexpr int NBA = NB > 0 ? NB : 1;
+    int bbase[NBA];
+#pragma unroll
+    for (int j = 0; j < NB; ++j) {
+        const int col = ((first + G::NWAVE * j) << 4) + (lane & 15);
+        const int pos = col < nc ? (int)(sh.col_pos[col] & COL_CELL) - G::TAP0 : 0;
+        bbase[j] = pos + (lane >> 4) * G::CH_STRIDE;
+    }
+    floatx4 acc[NBA];
+#pragma unroll
+    for (int j = 0; j < NB; ++j)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) acc[j][r] = 0.f;
+    const float* ap = Wl + lane;
+
+    constexpr int W4 = KC * 4;                                   // float4 elements of a weight chunk (16 co wide)
+    constexpr int WPT = (W4 + G::NT - 1) / G::NT;
+    ItemRegs<G, float, CIB> R;
+    float4 wr[WPT];
+#define APRNET_LOAD_WEIGHTS(q)                                                                     \
+    _Pragma("unroll") for (int k = 0; k < WPT; ++k) {                                              \
+        const int i = threadIdx.x + k * G::NT;                                                     \
+        wr[k] = (i < W4) ? (wl + (int64_t)(q) * W4)[i] : make_float4(0.f, 0.f, 0.f, 0.f);          \
+    }
+#define APRNET_STORE_WEIGHTS()                                                                     \
+    _Pragma("unroll") for (int k = 0; k < WPT; ++k) {                                              \
+        const int i = threadIdx.x + k * G::NT;                                                     \
+        if (i < W4) reinterpret_cast<float4*>(Wl)[i] = wr[k];                                      \
+    }
+    load_items<G, float, CIB>(a, 0, nitem, tree_items, sh, R);
+    APRNET_LOAD_WEIGHTS(0)
+    for (int i = threadIdx.x; i < CIB * G::CH_STRIDE; i += G::NT) patch[i] = 0.f;     // once per window
+    for (int ci0 = 0; ci0 < a.Cin; ci0 += CIB) {
+        __syncthreads();
+        store_items<G, float, CIB>(R, nitem, patch);
+        APRNET_STORE_WEIGHTS()
+        __syncthreads();
+        if (ci0 + CIB < a.Cin) {
+            load_items<G, float, CIB>(a, ci0 + CIB, nitem, tree_items, sh, R);
+            APRNET_LOAD_WEIGHTS(ci0 / CIB + 1)
+        }
+#pragma unroll
+        for (int t = 0; t < G::K; ++t) {
+            const float av = ap[t * 64];
+#pragma unroll
+            for (int j = 0; j < NB; ++j) {
+                const float bv = patch[bbase[j] + tap_offset<G>(t)];
+                acc[j] = __builtin_amdgcn_mfma_f32_16x16x4f32(av, bv, acc[j], 0, 0, 0);
+            }
+        }
+    }
+#undef APRNET_LOAD_WEIGHTS
+#undef APRNET_STORE_WEIGHTS
+    float bias[4];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) bias[r] = bias_l[4 * (lane >> 4) + r];
+#pragma unroll
+    for (int j = 0; j < NB; ++j) {
+        const int col = ((first + G::NWAVE * j) << 4) + (lane & 15);
+        if (col >= nc) continue;
+        const int64_t o = sh.col_idx[col];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const int co = co0 + 4 * (lane >> 4) + r;
+            if (co < a.Cout) a.y[(int64_t)co * a.ldy + o] = acc[j][r] + bias[r];
+        }
+    }
+}
+
+template <class G>
+__global__ void __launch_bounds__(G::NT)
+conv_mfma16_kernel(const ConvArgs<float> a) {
+    constexpr int CIB = 4, NBW = 4;
+    static_assert((G::NWAVE & (G::NWAVE - 1)) == 0, "block rotation assumes a power-of-two wave count");
+    static_assert((G::MAXCOL + 15) / 16 <= G::NWAVE * NBW, "a window must fit the accumulators of the block");
+    static_assert(G::CH_STRIDE % 64 == 16, "four lane groups read four channels: a quarter of the banks each");
+    __shared__ float patch[CIB * G::CH_STRIDE];
+    __shared__ __attribute__((aligned(16))) float Wl[CIB * G::K * 16];
+    __shared__ ConvShared<G> sh;
+    __shared__ float bias_l[16];
+
+    const ConvTile tile = a.tiles[blockIdx.x];
+    const int L = tile.level, z0 = tile.z0, x0 = tile.x0;
+    const int co0 = blockIdx.y * 16;
+    const int yn = a.apr.y_num[L];
+    const int s_idx = min(a.S_exp - 1, a.Lc - L);
+    const bool out_tree = (L == a.Lc) && (L < a.apr.level_max);
+    const int nq = (a.Cin + CIB - 1) / CIB;
+    const float4* __restrict__ wl = reinterpret_cast<const float4*>(a.w) +
+                                    ((int64_t)s_idx * gridDim.y + blockIdx.y) * nq * (CIB * G::K * 4);
+    const int wave = threadIdx.x >> 6;
+
+    if (threadIdx.x < 16) bias_l[threadIdx.x] = (a.bias && co0 + (int)threadIdx.x < a.Cout) ? a.bias[co0 + threadIdx.x] : 0.f;
+    open_segments<G, float>(a, L, z0, x0, sh);
+    __syncthreads();
+
+    int win = 0;
+    for (int y0 = 0; y0 < yn; y0 += G::TY, ++win) {
+        scan_window<G, float>(a, L, y0, out_tree, sh);
+        __syncthreads();
+        const int nc = __builtin_amdgcn_readfirstlane(sh.ncol), nitem = __builtin_amdgcn_readfirstlane(sh.nitem);
+        const bool tree_items = L < a.Lc;
+        if (nc > 0) {
+            const int nblk = (nc + 15) >> 4;
+            const int first = (wave - (int)blockIdx.x - win) & (G::NWAVE - 1);
+            const int nb = first < nblk ? (nblk - first + G::NWAVE - 1) / G::NWAVE : 0;
+            switch (__builtin_amdgcn_readfirstlane(nb)) {
+                case 0: mfma16_window<G, 0>(a, co0, nc, nitem, tree_items, first, wl, sh, patch, Wl, bias_l); break;
+                case 1: mfma16_window<G, 1>(a, co0, nc, nitem, tree_items, first, wl, sh, patch, Wl, bias_l); break;
+                case 2: mfma16_window<G, 2>(a, co0, nc, nitem, tree_items, first, wl, sh, patch, Wl, bias_l); break;
+                case 3: mfma16_window<G, 3>(a, co0, nc, nitem, tree_items, first, wl, sh, patch, Wl, bias_l); break;
+                default: mfma16_window<G, 4>(a, co0, nc, nitem, tree_items, first, wl, sh, patch, Wl, bias_l); break;
+            }
+        }
+        __syncthreads();
+        close_window<G>(sh);
+        __syncthreads();
+    }
+}
+
+using M333N = ConvGeom<3, 3, 3, 2, 4, 512, 64, 16>;
+
+int launch_conv333_mfma16(const ConvArgs<float>& a, int n_tiles, hipStream_t st) {
+    dim3 grid((unsigned)n_tiles, (unsigned)((a.Cout + 15) / 16));
+    hipLaunchKernelGGL((conv_mfma16_kernel<M333N>), grid, dim3(M333N::NT), 0, st, a);
+    APRNET_LAUNCH_CHECK("conv_mfma16_kernel");
+    return 0;
+}
+
+size_t conv333_packed16_floats(int S_exp, int Cout, int Cin) {
+    return (size_t)S_exp * ((Cout + 15) / 16) * ((Cin + 3) / 4) * 4 * 27 * 16;
+}
+
+int pack_conv333_weights16(const float* w, int S_exp, int Cout, int Cin, float* packed, hipStream_t st) {
+    const size_t n = conv333_packed16_floats(S_exp, Cout, Cin);
+    dim3 grid((unsigned)std::min<size_t>((n + 255) / 256, 2048));
+    hipLaunchKernelGGL(pack_weights16_kernel, grid, dim3(256), 0, st, w, S_exp, Cout, Cin, 27, 4, packed);
+    APRNET_LAUNCH_CHECK("pack_weights16_kernel");
+    return 0;
+}
+
 using M333 = ConvGeom<3, 3, 3, 2, 4, 512>;
 
 constexpr int MFMA_CIB = 4;
