@@ -131,9 +131,7 @@ template <> struct Chunk<double> { static constexpr int c333 = 4, c133 = 8,  c15
 int launch_conv333_mfma(const ConvArgs<float>& a, int n_tiles, hipStream_t st);
 size_t conv333_packed_floats(int S_exp, int Cout, int Cin);
 int pack_conv333_weights(const float* w, int S_exp, int Cm, int Ck, bool transposed, float* packed, hipStream_t st);
-int launch_conv333_mfma16(const ConvArgs<float>& a, int n_tiles, hipStream_t st);
-size_t conv333_packed16_floats(int S_exp, int Cout, int Cin);
-int pack_conv333_weights16(const float* w, int S_exp, int Cout, int Cin, float* packed, hipStream_t st);
+
 static int g_conv_path = 0;      // 0: matrix cores where available, 1: VALU kernels only
 int conv_path() { return g_conv_path; }
 
@@ -141,14 +139,6 @@ template <typename T> static int try_mfma(aprnet_plan*, const ConvArgs<T>&, int,
 template <> int try_mfma<float>(aprnet_plan* p, const ConvArgs<float>& a, int code, int n_tiles, hipStream_t st, bool* done) {
     if (g_conv_path == 1 || code != 333) return 0;
     *done = true;
-    if (a.Cout <= 16) {      // narrow layers: 16-row matrix instruction, half the matrix work
-        if (int rc = plan_scratch(p, conv333_packed16_floats(a.S_exp, a.Cout, a.Cin) * sizeof(float), st)) return rc;
-        if (int rc = pack_conv333_weights16(a.w, a.S_exp, a.Cout, a.Cin, (float*)p->d_scratch, st)) return rc;
-        ConvArgs<float> b = a;
-        b.w = (const float*)p->d_scratch;
-        TimedLaunch timed(st);
-        return launch_conv333_mfma16(b, n_tiles, st);
-    }
     // plan-owned scratch for the re-laid-out weights, grown on demand
     if (int rc = plan_scratch(p, conv333_packed_floats(a.S_exp, a.Cout, a.Cin) * sizeof(float), st)) return rc;
     if (int rc = pack_conv333_weights(a.w, a.S_exp, a.Cout, a.Cin, false, (float*)p->d_scratch, st)) return rc;

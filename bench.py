@@ -207,7 +207,7 @@ def main():
                    "apr_build_s": round(t_build, 2), "plan_create_s": round(t_plan, 2)},
         "roofline": {"bound": "mfma", "achieved": tflops, "peak": PEAK_FP32_MATRIX_TFLOPS, "unit": "TFLOP/s",
                      "frac": tflops / PEAK_FP32_MATRIX_TFLOPS, "traffic": MEASURED_TRAFFIC_BYTES.get(n),
-                     "kernel": "conv_fwd_mfma_kernel", "kernel_ms": kernel_ms,
+                     "kernel": "conv_mfma16_kernel", "kernel_ms": kernel_ms,
                      "hbm_achieved_GBs": gbs, "hbm_frac": gbs / PEAK_HBM_GBS},
     }
     if args.calibrate_copy:
