@@ -161,8 +161,10 @@ __device__ __forceinline__ void mfma16_window(const ConvArgs<float>& a, int co0,
 }
 
 // COH = 16-channel parts of the output block: 1 for layers of at most 16 output channels, 2 otherwise
+// Three workgroups per CU (six waves per SIMD, 80 registers): the third group hides more of the latency of
+// the scan and staging phases than the few spilled registers cost.
 template <class G, int COH, int MODE>
-__global__ void __launch_bounds__(G::NT)
+__global__ void __launch_bounds__(G::NT) __attribute__((amdgpu_waves_per_eu(6, 6)))
 conv_mfma16_kernel(const ConvArgs<float> a) {
     constexpr int CIB = 4, NBW = 4;
     static_assert((G::NWAVE & (G::NWAVE - 1)) == 0, "block rotation assumes a power-of-two wave count");
