@@ -80,6 +80,7 @@ def hip():
     for t in ("f32", "f64"):
         getattr(lib, f"aprnet_fill_tree_mean_{t}").argtypes = [vp, i32, vp, i64, i32, vp, i64, vp]
         getattr(lib, f"aprnet_fill_tree_mean_bwd_{t}").argtypes = [vp, i32, vp, i64, i32, vp, i64, vp]
+        getattr(lib, f"aprnet_channel_sum_{t}").argtypes = [vp, i64, i32, i64, vp, i32, vp, vp]
         getattr(lib, f"aprnet_conv_fwd_{t}").argtypes = [vp, i32, i32, i32, i32, vp, i64, i32, vp, i32, i32, vp,
                                                          vp, i64, vp, i64, vp]
         getattr(lib, f"aprnet_conv_bwd_{t}").argtypes = [vp, i32, i32, i32, i32, vp, i64, i32, vp, i32, i32,

@@ -168,6 +168,23 @@ def conv_forward(aprs, x, weights, level_delta, bias=None):
     return out
 
 
+def channel_sum(x):
+    """sum over batch and positions of a [B, C, N] tensor -> [C] (the bias gradient, conv.py:33), deterministic."""
+    _check_input(x, "grad_output")
+    B, C, N = x.shape
+    out = torch.empty(C, dtype=x.dtype, device=x.device)
+    lib = _lib()
+    work = torch.empty(lib.aprnet_channel_sum_work_elems(C), dtype=x.dtype, device=x.device)
+    fn = getattr(lib, "aprnet_channel_sum_" + _sfx(x))
+    with torch.cuda.device(x.device):
+        st = _stream()
+        for b in range(B):
+            rc = fn(_ptr(x[b]), N, C, N, _ptr(out), 1 if b else 0, _ptr(work), st)
+            if rc:
+                _raise(rc, "channel_sum failed")
+    return out
+
+
 def conv_backward(aprs, x, weights, grad_output, level_delta):
     """conv333_backward / conv111_backward (wrap_conv_gpu.hpp:87-133, 216-246) -> [grad_input, grad_weights]."""
     _check_input(x, "input")

@@ -55,7 +55,7 @@ class ConvFunction(Function):
         inputs, w_exp, bias, level_deltas = ctx.saved_tensors
         grad_output = grad_output.contiguous()
         grad_input, grad_w = _ops.conv_backward(ctx.aprs, inputs, w_exp, grad_output, level_deltas)
-        grad_bias = None if bias is None else torch.sum(grad_output, dim=(0, 2))
+        grad_bias = None if bias is None else _ops.channel_sum(grad_output)
         if ctx.expand:
             grad_w = _ops.restrict_kernel_backward(grad_w, ctx.num_stencils)
         return grad_input, _from_device_layout(grad_w, ctx.layout), grad_bias, None, None, None

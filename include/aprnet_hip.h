@@ -83,6 +83,13 @@ int aprnet_profile_enable(int on);
 int aprnet_set_conv_path(int path);
 float aprnet_profile_last_ms(void);
 
+/* Bias gradient of a convolution: out[c] (+)= sum_i x[c*ld + i], i < n (replaces torch.sum(grad_output, dim=(0, 2)),
+ * conv.py:33, cuda/conv.py:33, one batch item per call; pass accumulate != 0 for the items after the first).
+ * Two passes in a fixed order, no atomics.  work: aprnet_channel_sum_work_elems(C) elements of scratch. */
+int aprnet_channel_sum_work_elems(int C);
+int aprnet_channel_sum_f32(const float* x, int64_t ld, int C, int64_t n, float* out, int accumulate, float* work, void* stream);
+int aprnet_channel_sum_f64(const double* x, int64_t ld, int C, int64_t n, double* out, int accumulate, double* work, void* stream);
+
 #define APRNET_DECL(T, SFX)                                                                                          \
     /* helpers::fill_tree_mean (helpers.hpp:156-252): tree[c][t] for all tree nodes of level < Lc. */               \
     int aprnet_fill_tree_mean_##SFX(const aprnet_plan*, int level_delta, const T* x, int64_t ldx, int C,            \
