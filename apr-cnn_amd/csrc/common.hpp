@@ -46,6 +46,27 @@ struct HostAccess {
     }
 };
 
+// bfloat16 as a storage type: kernels load it into fp32, compute in fp32 and round to nearest even on store.
+struct bf16_t { uint16_t bits; };
+__host__ __device__ inline float bf16_to_float(bf16_t v) { return __builtin_bit_cast(float, (uint32_t)v.bits << 16); }
+__host__ __device__ inline bf16_t float_to_bf16(float f) {
+    uint32_t u = __builtin_bit_cast(uint32_t, f);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return bf16_t{(uint16_t)((u >> 16) | 0x40u)};      // NaN stays NaN
+    u += 0x7fffu + ((u >> 16) & 1u);
+    return bf16_t{(uint16_t)(u >> 16)};
+}
+// element type -> the type it is computed in, with the conversions of a load and a store
+template <typename T> struct Num {
+    typedef T acc;
+    static __host__ __device__ __forceinline__ acc ld(T v) { return v; }
+    static __host__ __device__ __forceinline__ T st(acc v) { return v; }
+};
+template <> struct Num<bf16_t> {
+    typedef float acc;
+    static __host__ __device__ __forceinline__ float ld(bf16_t v) { return bf16_to_float(v); }
+    static __host__ __device__ __forceinline__ bf16_t st(float v) { return float_to_bf16(v); }
+};
+
 struct ConvTile { int32_t level, z0, x0, pad; };
 
 struct TileList {

@@ -129,6 +129,8 @@ template <> struct Chunk<float>  { static constexpr int c333 = 8, c133 = 16, c15
 template <> struct Chunk<double> { static constexpr int c333 = 4, c133 = 8,  c155 = 6,  c555 = 2; };
 
 int launch_conv333_mfma(const ConvArgs<float>& a, int n_tiles, hipStream_t st);
+int launch_conv333_mfma(const ConvArgs<bf16_t>& a, int n_tiles, hipStream_t st);
+int fill_tree_for_conv(const aprnet_plan* p, int d, const bf16_t* x, int64_t ldx, int C, bf16_t* tree, int64_t ldt, hipStream_t st);
 size_t conv333_packed_floats(int S_exp, int Cout, int Cin);
 int pack_conv333_weights(const float* w, int S_exp, int Cm, int Ck, bool transposed, float* packed, hipStream_t st);
 
@@ -187,11 +189,42 @@ int conv_fwd(const aprnet_plan* cp, int d, int kz, int kx, int ky, const T* x, i
     return 0;
 }
 
+// bfloat16 features, fp32 weights and bias, fp32 arithmetic: 3x3x3 on the matrix cores only
+int conv_fwd_bf16(const aprnet_plan* cp, int d, int kz, int kx, int ky, const bf16_t* x, int64_t ldx, int Cin, const float* w,
+                  int S_exp, int Cout, const float* bias, bf16_t* y, int64_t ldy, bf16_t* tree_ws, int64_t ldt, hipStream_t st) {
+    aprnet_plan* p = const_cast<aprnet_plan*>(cp);
+    if (int rc = check_level_delta(p, d, "conv_forward")) return rc;
+    if (Cin <= 0 || Cout <= 0 || S_exp <= 0) return fail(APRNET_ERR_INVALID_ARGUMENT, "conv_forward: empty channel / stencil count");
+    if (kz != 3 || kx != 3 || ky != 3) return fail(APRNET_ERR_UNSUPPORTED, "conv_forward: bfloat16 features are supported for the 3x3x3 stencil only");
+    const int64_t nt = p->tree_parts(d);
+    if (nt > 0 && (!tree_ws || ldt < nt)) return fail(APRNET_ERR_INVALID_ARGUMENT, "conv_forward: tree work space too small");
+    APRNET_HIP_CHECK(hipSetDevice(p->device));
+    if (int rc = fill_tree_for_conv(p, d, x, ldx, Cin, tree_ws, ldt, st)) return rc;
+    TileList tl;
+    if (int rc = get_tiles(p, d, 2, 4, &tl)) return rc;
+    if (tl.n == 0) return 0;
+    if (int rc = plan_scratch(p, conv333_packed_floats(S_exp, Cout, Cin) * sizeof(float), st)) return rc;
+    if (int rc = pack_conv333_weights(w, S_exp, Cout, Cin, false, (float*)p->d_scratch, st)) return rc;
+    ConvArgs<bf16_t> a{};
+    a.apr = p->dapr; a.tree = p->dtree; a.tiles = tl.d_tiles;
+    a.x = x; a.ldx = ldx; a.Cin = Cin; a.w = (const float*)p->d_scratch; a.S_exp = S_exp; a.Cout = Cout; a.bias = bias;
+    a.y = y; a.ldy = ldy; a.tree_data = tree_ws; a.ldt = ldt; a.Lc = p->lc(d); a.tree_off = p->tree_offset(a.Lc);
+    a.x_count = p->number_parts(d); a.t_count = p->tree_parts(d);
+    TimedLaunch timed(st);
+    return launch_conv333_mfma(a, tl.n, st);
+}
+
 }  // namespace aprnet
 
 using namespace aprnet;
 
 extern "C" {
+int aprnet_conv_fwd_bf16(const aprnet_plan* p, int d, int kz, int kx, int ky, const uint16_t* x, int64_t ldx, int Cin,
+                         const float* w, int S_exp, int Cout, const float* bias, uint16_t* y, int64_t ldy, uint16_t* tree_ws,
+                         int64_t ldt, void* st) {
+    return conv_fwd_bf16(p, d, kz, kx, ky, (const bf16_t*)x, ldx, Cin, w, S_exp, Cout, bias, (bf16_t*)y, ldy, (bf16_t*)tree_ws,
+                         ldt, (hipStream_t)st);
+}
 int aprnet_set_conv_path(int path) {
     if (path != 0 && path != 1) return fail(APRNET_ERR_INVALID_ARGUMENT, "set_conv_path: 0 (auto) or 1 (VALU only)");
     g_conv_path = path;

@@ -44,10 +44,11 @@ conv111_kernel(const T* __restrict__ src, int64_t lds, int Csrc, const T* __rest
 // the kernel streams the input once per 32 output channels and is bound by HBM.
 typedef float floatx16_111 __attribute__((ext_vector_type(16)));
 
-template <int KP>      // KP = channel pairs held in registers (ceil(Csrc / 2) <= KP)
+// T = storage type of the features (float, or bfloat16 with fp32 weights, bias and arithmetic)
+template <typename T, int KP>      // KP = channel pairs held in registers (ceil(Csrc / 2) <= KP)
 __global__ void __launch_bounds__(TB1)
-conv111_mfma_kernel(const float* __restrict__ src, int64_t lds, int Csrc, const float* __restrict__ w, int so, int sc,
-                    const float* __restrict__ bias, float* __restrict__ dst, int64_t ldd, int Cdst, int64_t begin,
+conv111_mfma_kernel(const T* __restrict__ src, int64_t lds, int Csrc, const float* __restrict__ w, int so, int sc,
+                    const float* __restrict__ bias, T* __restrict__ dst, int64_t ldd, int Cdst, int64_t begin,
                     int64_t end) {
     const int lane = threadIdx.x & 63, hi = lane >> 5, col = lane & 31;
     const int o0 = blockIdx.y * 32;
@@ -71,9 +72,9 @@ conv111_mfma_kernel(const float* __restrict__ src, int64_t lds, int Csrc, const 
 #pragma unroll
         for (int p = 0; p < KP; ++p) {
             const int c = 2 * p + hi;
-            const float* row = src + (int64_t)c * lds;
-            va[p] = (c < Csrc && ia < end) ? row[ia] : 0.f;
-            vb[p] = (c < Csrc && ib < end) ? row[ib] : 0.f;
+            const T* row = src + (int64_t)c * lds;
+            va[p] = (c < Csrc && ia < end) ? Num<T>::ld(row[ia]) : 0.f;
+            vb[p] = (c < Csrc && ib < end) ? Num<T>::ld(row[ib]) : 0.f;
         }
         floatx16_111 acca, accb;
 #pragma unroll
@@ -87,20 +88,21 @@ conv111_mfma_kernel(const float* __restrict__ src, int64_t lds, int Csrc, const 
         for (int r = 0; r < 16; ++r) {
             const int o = o0 + 8 * (r >> 2) + 4 * hi + (r & 3);
             if (o < Cdst) {
-                if (ia < end) dst[(int64_t)o * ldd + ia] = acca[r];
-                if (ib < end) dst[(int64_t)o * ldd + ib] = accb[r];
+                if (ia < end) dst[(int64_t)o * ldd + ia] = Num<T>::st(acca[r]);
+                if (ib < end) dst[(int64_t)o * ldd + ib] = Num<T>::st(accb[r]);
             }
         }
     }
 }
 
 // dispatch on the number of channel pairs kept in registers; false when the layer is too wide for this kernel
-static bool launch_conv111_mfma(const float* src, int64_t lds, int Csrc, const float* w, int so, int sc, const float* bias,
-                                float* dst, int64_t ldd, int Cdst, int64_t begin, int64_t end, hipStream_t st) {
+template <typename T>
+static bool launch_conv111_mfma(const T* src, int64_t lds, int Csrc, const float* w, int so, int sc, const float* bias,
+                                T* dst, int64_t ldd, int Cdst, int64_t begin, int64_t end, hipStream_t st) {
     const int kp = (Csrc + 1) / 2;
     const int64_t n = end - begin;
     dim3 grid((unsigned)std::min<int64_t>((n + 255) / 256, 256 * 8), (unsigned)((Cdst + 31) / 32));
-#define APRNET_111(KP) hipLaunchKernelGGL((conv111_mfma_kernel<KP>), grid, dim3(TB1), 0, st, src, lds, Csrc, w, so, sc, bias, \
+#define APRNET_111(KP) hipLaunchKernelGGL((conv111_mfma_kernel<T, KP>), grid, dim3(TB1), 0, st, src, lds, Csrc, w, so, sc, bias, \
                                           dst, ldd, Cdst, begin, end)
     if (kp <= 8) APRNET_111(8);
     else if (kp <= 16) APRNET_111(16);
@@ -119,7 +121,7 @@ template <>
 bool try_conv111_mfma<float>(const float* src, int64_t lds, int Csrc, const float* w, int so, int sc, const float* bias,
                              float* dst, int64_t ldd, int Cdst, int64_t begin, int64_t end, hipStream_t st) {
     if (conv_path() == 1) return false;
-    return launch_conv111_mfma(src, lds, Csrc, w, so, sc, bias, dst, ldd, Cdst, begin, end, st);
+    return launch_conv111_mfma<float>(src, lds, Csrc, w, so, sc, bias, dst, ldd, Cdst, begin, end, st);
 }
 
 // gw[co][ci] += sum_i gy[co][i] * x[ci][i] over [begin, end): 8x8 register tile per thread, block
@@ -231,10 +233,26 @@ int conv111_bwd(const aprnet_plan* p, int d, const T* x, int64_t ldx, int Cin, c
     return 0;
 }
 
+int conv111_fwd_bf16(const aprnet_plan* p, int d, const bf16_t* x, int64_t ldx, int Cin, const float* w, int S, int Cout,
+                     const float* bias, bf16_t* y, int64_t ldy, hipStream_t st) {
+    if (int rc = check_level_delta(p, d, "conv111_forward")) return rc;
+    if (Cin <= 0 || Cout <= 0 || S <= 0) return fail(APRNET_ERR_INVALID_ARGUMENT, "conv111_forward: empty channel / stencil count");
+    APRNET_HIP_CHECK(hipSetDevice(p->device));
+    for (const Segment& sg : segments(p, d, S))
+        if (!launch_conv111_mfma<bf16_t>(x, ldx, Cin, w + (int64_t)sg.stencil * Cout * Cin, Cin, 1, bias, y, ldy, Cout, sg.begin, sg.end, st))
+            return fail(APRNET_ERR_UNSUPPORTED, "conv111_forward: more than 128 input channels with bfloat16 features");
+    APRNET_LAUNCH_CHECK("conv111_mfma_kernel");
+    return 0;
+}
+
 }  // namespace aprnet
 
 using namespace aprnet;
 extern "C" {
+int aprnet_conv111_fwd_bf16(const aprnet_plan* p, int d, const uint16_t* x, int64_t ldx, int Cin, const float* w, int S,
+                            int Cout, const float* bias, uint16_t* y, int64_t ldy, void* st) {
+    return conv111_fwd_bf16(p, d, (const bf16_t*)x, ldx, Cin, w, S, Cout, bias, (bf16_t*)y, ldy, (hipStream_t)st);
+}
 #define CONV111_API(T, SFX)                                                                                        \
     int aprnet_conv111_fwd_##SFX(const aprnet_plan* p, int d, const T* x, int64_t ldx, int Cin, const T* w, int S,  \
                                  int Cout, const T* bias, T* y, int64_t ldy, void* st) {                            \

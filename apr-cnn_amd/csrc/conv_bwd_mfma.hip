@@ -72,12 +72,17 @@ conv_dw_mfma_kernel(const ConvArgs<float> a, const int s_idx) {
                 for (int g0 = 0; g0 < nc; g0 += DW_GB) {
                     const int ng = min(DW_GB, nc - g0), nbatch = (ng + 63) >> 6;
                     // output gradient of this group of columns -> gyl; a wave reads 64 columns of one channel
-                    for (int i = threadIdx.x; i < 32 * nbatch * 64; i += G::NT) {
-                        const int co = i / (nbatch * 64), c = i - co * (nbatch * 64);
-                        float v = 0.f;
-                        if (c < ng && co0 + co < a.Cout) v = a.gy[(int64_t)(co0 + co) * a.ldy + sh.col_idx[g0 + c]];
-                        const int slot = (c & ~63) + 2 * (c & 31) + ((c >> 5) & 1);
-                        gyl[slot * DW_GLD + co] = v;
+                    for (int b = 0; b < nbatch; ++b) {
+                        const int c = b * 64 + lane;
+                        const int64_t idx = c < ng ? sh.col_idx[g0 + c] : -1;
+                        const int slot = b * 64 + 2 * (lane & 31) + (lane >> 5);
+#pragma unroll
+                        for (int k = 0; k < 32 / G::NWAVE; ++k) {
+                            const int co = wave + k * G::NWAVE;
+                            float v = 0.f;
+                            if (idx >= 0 && co0 + co < a.Cout) v = a.gy[(int64_t)(co0 + co) * a.ldy + idx];
+                            gyl[slot * DW_GLD + co] = v;
+                        }
                     }
 #pragma unroll
                     for (int q = 0; q < NCH; ++q) {

@@ -26,8 +26,8 @@ struct ConvArgs {
     AccessDev apr, tree;
     const ConvTile* tiles;
     const T* x; int64_t ldx; int Cin;
-    const T* w; int S_exp; int Cout;          // [S_exp][Cout][Cin][K]
-    const T* bias;                            // [Cout] or null
+    const typename Num<T>::acc* w; int S_exp; int Cout;     // [S_exp][Cout][Cin][K]; fp32 for bfloat16 features
+    const typename Num<T>::acc* bias;                       // [Cout] or null
     T* y; int64_t ldy;
     const T* tree_data; int64_t ldt;
     int Lc; int64_t tree_off;                  // tree_offset(Lc)
@@ -337,6 +337,11 @@ template <> struct RawLoad<float> {
     static __device__ __forceinline__ raw ld(__amdgpu_buffer_rsrc_t r, unsigned off) { return __builtin_amdgcn_raw_buffer_load_b32(r, (int)off, 0, 0); }
     static __device__ __forceinline__ float cast(raw v) { return __builtin_bit_cast(float, v); }
 };
+template <> struct RawLoad<bf16_t> {      // 16-bit load, zero-extended; the value is the upper half of an fp32
+    typedef int raw;
+    static __device__ __forceinline__ raw ld(__amdgpu_buffer_rsrc_t r, unsigned off) { return (int)__builtin_amdgcn_raw_buffer_load_b16(r, (int)off, 0, 0); }
+    static __device__ __forceinline__ float cast(raw v) { return __builtin_bit_cast(float, v << 16); }
+};
 template <> struct RawLoad<double> {
     typedef int raw __attribute__((ext_vector_type(2)));
     static __device__ __forceinline__ raw ld(__amdgpu_buffer_rsrc_t r, unsigned off) { return __builtin_amdgcn_raw_buffer_load_b64(r, (int)off, 0, 0); }
@@ -392,15 +397,15 @@ __device__ __forceinline__ void load_items(const ConvArgs<T>& a, int ci0, int ni
 }
 
 template <class G, typename T, int CIB>
-__device__ __forceinline__ void store_items(const ItemRegs<G, T, CIB>& R, int nitem, T* patch) {
+__device__ __forceinline__ void store_items(const ItemRegs<G, T, CIB>& R, int nitem, typename Num<T>::acc* patch) {
 #pragma unroll
     for (int k = 0; k < ItemRegs<G, T, CIB>::IPT; ++k) {
         if (k * G::NT >= nitem) break;                  // wave-uniform
         if (R.pos[k] == 0xffffu) continue;
-        T* cell = patch + (R.pos[k] & ITEM_CELL);
+        typename Num<T>::acc* cell = patch + (R.pos[k] & ITEM_CELL);
 #pragma unroll
         for (int c = 0; c < CIB; ++c) {
-            const T v = RawLoad<T>::cast(R.v[k][c]);
+            const typename Num<T>::acc v = RawLoad<T>::cast(R.v[k][c]);
             cell[c * G::CH_STRIDE] = v;
             if (R.pos[k] & ITEM_PAIR) cell[c * G::CH_STRIDE + 1] = v;
         }
@@ -412,7 +417,7 @@ __device__ __forceinline__ void store_items(const ItemRegs<G, T, CIB>& R, int ni
 // half-width <= 2 never reads on a 2:1-balanced APR); covered cells are overwritten by every chunk.
 template <class G, typename T, int CIB>
 __device__ __forceinline__ void stage_values(const ConvArgs<T>& a, int ci0, int nitem, bool tree_items,
-                                             const ConvShared<G>& sh, T* patch) {
+                                             const ConvShared<G>& sh, typename Num<T>::acc* patch) {
     ItemRegs<G, T, CIB> R;
     load_items<G, T, CIB>(a, ci0, nitem, tree_items, sh, R);
     store_items<G, T, CIB>(R, nitem, patch);

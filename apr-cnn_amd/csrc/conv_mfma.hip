@@ -66,8 +66,8 @@ __global__ void pack_weights16_kernel(const float* __restrict__ w, int S_exp, in
 
 // MODE 0: forward, results stored (plus bias).  MODE 1: input gradient, results added atomically to the
 // place each column names (feature gradient, or tree gradient with COL_TREE).
-template <class G, int COH, int NB, int MODE>
-__device__ __forceinline__ void mfma16_window(const ConvArgs<float>& a, int co0, int nc, int nitem, bool tree_items, int first,
+template <typename T, class G, int COH, int NB, int MODE>
+__device__ __forceinline__ void mfma16_window(const ConvArgs<T>& a, int co0, int nc, int nitem, bool tree_items, int first,
                                               const float4* __restrict__ wl, const ConvShared<G>& sh,
                                               float* __restrict__ patch, float* __restrict__ Wl,
                                               const float* __restrict__ bias_l) {
@@ -93,7 +93,7 @@ __device__ __forceinline__ void mfma16_window(const ConvArgs<float>& a, int co0,
 
     constexpr int W4 = KC * 4 * COH;                             // float4 elements of a weight chunk
     constexpr int WPT = (W4 + G::NT - 1) / G::NT;
-    ItemRegs<G, float, CIB> R;
+    ItemRegs<G, T, CIB> R;
     float4 wr[WPT];
 #define APRNET_LOAD_WEIGHTS(q)                                                                     \
     _Pragma("unroll") for (int k = 0; k < WPT; ++k) {                                              \
@@ -105,16 +105,16 @@ __device__ __forceinline__ void mfma16_window(const ConvArgs<float>& a, int co0,
         const int i = threadIdx.x + k * G::NT;                                                     \
         if (i < W4) reinterpret_cast<float4*>(Wl)[i] = wr[k];                                      \
     }
-    load_items<G, float, CIB>(a, 0, nitem, tree_items, sh, R);
+    load_items<G, T, CIB>(a, 0, nitem, tree_items, sh, R);
     APRNET_LOAD_WEIGHTS(0)
     for (int i = threadIdx.x; i < CIB * G::CH_STRIDE; i += G::NT) patch[i] = 0.f;     // once per window
     for (int ci0 = 0; ci0 < a.Cin; ci0 += CIB) {
         __syncthreads();
-        store_items<G, float, CIB>(R, nitem, patch);
+        store_items<G, T, CIB>(R, nitem, patch);
         APRNET_STORE_WEIGHTS()
         __syncthreads();
         if (ci0 + CIB < a.Cin) {
-            load_items<G, float, CIB>(a, ci0 + CIB, nitem, tree_items, sh, R);
+            load_items<G, T, CIB>(a, ci0 + CIB, nitem, tree_items, sh, R);
             APRNET_LOAD_WEIGHTS(ci0 / CIB + 1)
         }
 #pragma unroll
@@ -143,9 +143,9 @@ __device__ __forceinline__ void mfma16_window(const ConvArgs<float>& a, int co0,
 #pragma unroll
                 for (int r = 0; r < 4; ++r) {
                     const int cl = h * 16 + 4 * (lane >> 4) + r;
-                    if (co0 + cl < a.Cout) a.y[(int64_t)(co0 + cl) * a.ldy + o] = acc[j][h][r] + bias_l[cl];
+                    if (co0 + cl < a.Cout) a.y[(int64_t)(co0 + cl) * a.ldy + o] = Num<T>::st(acc[j][h][r] + bias_l[cl]);
                 }
-        } else {
+        } else if constexpr (sizeof(T) == 4) {      // gradients are accumulated in fp32 only
             const bool to_tree = (sh.col_pos[col] & COL_TREE) != 0;
             float* dst = (to_tree ? a.gtree : a.gx) + o;
             const int64_t ld = to_tree ? a.ldgt : a.ldgx;
@@ -163,9 +163,9 @@ __device__ __forceinline__ void mfma16_window(const ConvArgs<float>& a, int co0,
 // COH = 16-channel parts of the output block: 1 for layers of at most 16 output channels, 2 otherwise
 // Three workgroups per CU (six waves per SIMD, 80 registers): the third group hides more of the latency of
 // the scan and staging phases than the few spilled registers cost.
-template <class G, int COH, int MODE>
+template <typename T, class G, int COH, int MODE>
 __global__ void __launch_bounds__(G::NT) __attribute__((amdgpu_waves_per_eu(6, 6)))
-conv_mfma16_kernel(const ConvArgs<float> a) {
+conv_mfma16_kernel(const ConvArgs<T> a) {
     constexpr int CIB = 4, NBW = 4;
     static_assert((G::NWAVE & (G::NWAVE - 1)) == 0, "block rotation assumes a power-of-two wave count");
     static_assert((G::MAXCOL + 15) / 16 <= G::NWAVE * NBW, "a window must fit the accumulators of the block");
@@ -188,13 +188,13 @@ conv_mfma16_kernel(const ConvArgs<float> a) {
 
     if (MODE == 0 && threadIdx.x < 16 * COH)
         bias_l[threadIdx.x] = (a.bias && co0 + (int)threadIdx.x < a.Cout) ? a.bias[co0 + threadIdx.x] : 0.f;
-    open_segments<G, float>(a, L, z0, x0, sh);
+    open_segments<G, T>(a, L, z0, x0, sh);
     __syncthreads();
 
     int win = 0;
     for (int y0 = 0; y0 < yn; y0 += G::TY, ++win) {
-        if constexpr (MODE == 0) scan_window<G, float>(a, L, y0, out_tree, sh);
-        else scan_window_dx<G, float>(a, L, y0, out_tree, sh);
+        if constexpr (MODE == 0) scan_window<G, T>(a, L, y0, out_tree, sh);
+        else scan_window_dx<G, T>(a, L, y0, out_tree, sh);
         __syncthreads();
         const int nc = __builtin_amdgcn_readfirstlane(sh.ncol), nitem = __builtin_amdgcn_readfirstlane(sh.nitem);
         const bool tree_items = MODE == 0 && L < a.Lc;       // the output gradient has no tree part
@@ -203,11 +203,11 @@ conv_mfma16_kernel(const ConvArgs<float> a) {
             const int first = (wave - (int)blockIdx.x - win) & (G::NWAVE - 1);
             const int nb = first < nblk ? (nblk - first + G::NWAVE - 1) / G::NWAVE : 0;
             switch (__builtin_amdgcn_readfirstlane(nb)) {
-                case 0: mfma16_window<G, COH, 0, MODE>(a, co0, nc, nitem, tree_items, first, wl, sh, patch, Wl, bias_l); break;
-                case 1: mfma16_window<G, COH, 1, MODE>(a, co0, nc, nitem, tree_items, first, wl, sh, patch, Wl, bias_l); break;
-                case 2: mfma16_window<G, COH, 2, MODE>(a, co0, nc, nitem, tree_items, first, wl, sh, patch, Wl, bias_l); break;
-                case 3: mfma16_window<G, COH, 3, MODE>(a, co0, nc, nitem, tree_items, first, wl, sh, patch, Wl, bias_l); break;
-                default: mfma16_window<G, COH, 4, MODE>(a, co0, nc, nitem, tree_items, first, wl, sh, patch, Wl, bias_l); break;
+                case 0: mfma16_window<T, G, COH, 0, MODE>(a, co0, nc, nitem, tree_items, first, wl, sh, patch, Wl, bias_l); break;
+                case 1: mfma16_window<T, G, COH, 1, MODE>(a, co0, nc, nitem, tree_items, first, wl, sh, patch, Wl, bias_l); break;
+                case 2: mfma16_window<T, G, COH, 2, MODE>(a, co0, nc, nitem, tree_items, first, wl, sh, patch, Wl, bias_l); break;
+                case 3: mfma16_window<T, G, COH, 3, MODE>(a, co0, nc, nitem, tree_items, first, wl, sh, patch, Wl, bias_l); break;
+                default: mfma16_window<T, G, COH, 4, MODE>(a, co0, nc, nitem, tree_items, first, wl, sh, patch, Wl, bias_l); break;
             }
         }
         __syncthreads();
@@ -221,22 +221,25 @@ using M333N = ConvGeom<3, 3, 3, 2, 4, 512, 64, 16>;
 static int conv333_coh(int Cm) { return Cm <= 16 ? 1 : 2; }
 
 // Forward.  a.w must point at the packed weights (pack_conv333_weights).
-int launch_conv333_mfma(const ConvArgs<float>& a, int n_tiles, hipStream_t st) {
+template <typename T>
+static int launch_fwd16(const ConvArgs<T>& a, int n_tiles, hipStream_t st) {
     const int coh = conv333_coh(a.Cout);
     dim3 grid((unsigned)n_tiles, (unsigned)((a.Cout + 16 * coh - 1) / (16 * coh)));
-    if (coh == 1) hipLaunchKernelGGL((conv_mfma16_kernel<M333N, 1, 0>), grid, dim3(M333N::NT), 0, st, a);
-    else hipLaunchKernelGGL((conv_mfma16_kernel<M333N, 2, 0>), grid, dim3(M333N::NT), 0, st, a);
+    if (coh == 1) hipLaunchKernelGGL((conv_mfma16_kernel<T, M333N, 1, 0>), grid, dim3(M333N::NT), 0, st, a);
+    else hipLaunchKernelGGL((conv_mfma16_kernel<T, M333N, 2, 0>), grid, dim3(M333N::NT), 0, st, a);
     APRNET_LAUNCH_CHECK("conv_mfma16_kernel (forward)");
     return 0;
 }
+int launch_conv333_mfma(const ConvArgs<float>& a, int n_tiles, hipStream_t st) { return launch_fwd16<float>(a, n_tiles, st); }
+int launch_conv333_mfma(const ConvArgs<bf16_t>& a, int n_tiles, hipStream_t st) { return launch_fwd16<bf16_t>(a, n_tiles, st); }
 
 // Input gradient: a.x / a.Cin describe the output gradient, a.Cout the input channels, a.w the packed
 // transposed weights, a.tiles the row groups within one row of an output (n_tiles of them).
 int launch_conv333_dx_mfma(const ConvArgs<float>& a, int n_tiles, hipStream_t st) {
     const int coh = conv333_coh(a.Cout);
     dim3 grid((unsigned)n_tiles, (unsigned)((a.Cout + 16 * coh - 1) / (16 * coh)));
-    if (coh == 1) hipLaunchKernelGGL((conv_mfma16_kernel<M333N, 1, 1>), grid, dim3(M333N::NT), 0, st, a);
-    else hipLaunchKernelGGL((conv_mfma16_kernel<M333N, 2, 1>), grid, dim3(M333N::NT), 0, st, a);
+    if (coh == 1) hipLaunchKernelGGL((conv_mfma16_kernel<float, M333N, 1, 1>), grid, dim3(M333N::NT), 0, st, a);
+    else hipLaunchKernelGGL((conv_mfma16_kernel<float, M333N, 2, 1>), grid, dim3(M333N::NT), 0, st, a);
     APRNET_LAUNCH_CHECK("conv_mfma16_kernel (input gradient)");
     return 0;
 }

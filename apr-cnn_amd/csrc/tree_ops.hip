@@ -33,14 +33,15 @@ fill_tree_level_kernel(const int32_t* __restrict__ children, int64_t n_tree, int
 #pragma unroll
     for (int s = 0; s < 8; ++s) { ch[s] = children[(int64_t)s * n_tree + t]; cnt += ch[s] != NO_CHILD; }
     // 1/cnt is a power of two (cnt = product of 1-or-2 per dimension, helpers.hpp:133-153)
-    const T scale = (T)(1.0f / (float)max(cnt, 1));
+    typedef typename Num<T>::acc A;
+    const A scale = (A)(1.0f / (float)max(cnt, 1));
 #pragma unroll
     for (int k = 0; k < CPT; ++k) {
         const int c = blockIdx.y * CPT + k;
         if (c >= C) break;
         const T* xc = x + (int64_t)c * ldx;
         T* tc = tree + (int64_t)c * ldt;
-        T sum = 0;
+        A sum = 0;
 #pragma unroll
         for (int pass = 0; pass < 2; ++pass) {
             const bool want_tree = (pass == 0) == (tree_first != 0);
@@ -48,11 +49,11 @@ fill_tree_level_kernel(const int32_t* __restrict__ children, int64_t n_tree, int
             for (int s = 0; s < 8; ++s) {
                 const int32_t v = ch[s];
                 if (v == NO_CHILD) continue;
-                if (want_tree && v < 0) sum += tree_child_from_x ? xc[(int64_t)(~v) + tree_off] : tc[~v];
-                if (!want_tree && v >= 0) sum += xc[v];
+                if (want_tree && v < 0) sum += Num<T>::ld(tree_child_from_x ? xc[(int64_t)(~v) + tree_off] : tc[~v]);
+                if (!want_tree && v >= 0) sum += Num<T>::ld(xc[v]);
             }
         }
-        tc[t] = sum * scale;
+        tc[t] = Num<T>::st(sum * scale);
     }
 }
 
@@ -68,21 +69,21 @@ fill_tree_bwd_level_kernel(const int32_t* __restrict__ children, int64_t n_tree,
     int cnt = 0;
 #pragma unroll
     for (int s = 0; s < 8; ++s) { ch[s] = children[(int64_t)s * n_tree + t]; cnt += ch[s] != NO_CHILD; }
-    const T scale = (T)(1.0f / (float)max(cnt, 1));
+    typedef typename Num<T>::acc A;
+    const A scale = (A)(1.0f / (float)max(cnt, 1));
 #pragma unroll
     for (int k = 0; k < CPT; ++k) {
         const int c = blockIdx.y * CPT + k;
         if (c >= C) break;
         T* gxc = gx + (int64_t)c * ldx;
         T* gtc = gtree + (int64_t)c * ldt;
-        const T g = gtc[t] * scale;
+        const A g = Num<T>::ld(gtc[t]) * scale;
 #pragma unroll
         for (int s = 0; s < 8; ++s) {
             const int32_t v = ch[s];
             if (v == NO_CHILD) continue;
-            if (v >= 0) gxc[v] += g;
-            else if (tree_child_in_x) gxc[(int64_t)(~v) + tree_off] += g;
-            else gtc[~v] += g;
+            T* dst = v >= 0 ? gxc + v : (tree_child_in_x ? gxc + ((int64_t)(~v) + tree_off) : gtc + ~v);
+            *dst = Num<T>::st(Num<T>::ld(*dst) + g);
         }
     }
 }
@@ -115,23 +116,24 @@ maxpool_fwd_kernel(const int32_t* __restrict__ children, int64_t n_tree, int64_t
         const int c = blockIdx.y * CPT + k;
         if (c >= C) break;
         const T* xc = x + (int64_t)c * ldx;
-        T best = (T)(-1e17f);               // initial value of the output, maxpool.hpp:51
+        typedef typename Num<T>::acc A;
+        A best = (A)(-1e17f);               // initial value of the output, maxpool.hpp:51
         int64_t best_i = 0;
 #pragma unroll
         for (int s = 0; s < 8; ++s) {
             const int32_t v = ch[s];
-            if (v >= 0) { const T val = xc[v]; if (val > best) { best = val; best_i = v; } }
+            if (v >= 0) { const A val = Num<T>::ld(xc[v]); if (val > best) { best = val; best_i = v; } }
         }
 #pragma unroll
         for (int s = 0; s < 8; ++s) {
             const int32_t v = ch[s];
             if (v < 0 && v != NO_CHILD) {
                 const int64_t j = (int64_t)(~v) + in_tree_off;
-                const T val = xc[j];
+                const A val = Num<T>::ld(xc[j]);
                 if (val > best) { best = val; best_i = j; }
             }
         }
-        y[(int64_t)c * ldy + i] = best;
+        y[(int64_t)c * ldy + i] = Num<T>::st(best);
         arg[(int64_t)c * ldi + i] = best_i;
     }
 }
@@ -170,7 +172,7 @@ maxpool_bwd_kernel(const int32_t* __restrict__ children, int64_t n_tree, int64_t
             const int32_t v = ch[s];
             if (v == NO_CHILD) continue;
             const int64_t j = v >= 0 ? (int64_t)v : (int64_t)(~v) + in_tree_off;
-            gxc[j] = (j == m) ? g : (T)0;
+            gxc[j] = (j == m) ? g : Num<T>::st(0);
         }
     }
 }
@@ -213,12 +215,12 @@ upsample_kernel(const int32_t* __restrict__ children, int64_t n_tree, int64_t n_
                 d_[ch[s] >= 0 ? (int64_t)ch[s] : (int64_t)(~ch[s]) + out_tree_off] = v;
             }
         } else {
-            T sum = 0;      // particles first, then tree nodes (upsample.hpp:199-232)
+            typename Num<T>::acc sum = 0;      // particles first, then tree nodes (upsample.hpp:199-232)
 #pragma unroll
-            for (int s = 0; s < 8; ++s) if (ch[s] >= 0) sum += s_[ch[s]];
+            for (int s = 0; s < 8; ++s) if (ch[s] >= 0) sum += Num<T>::ld(s_[ch[s]]);
 #pragma unroll
-            for (int s = 0; s < 8; ++s) if (ch[s] < 0 && ch[s] != NO_CHILD) sum += s_[(int64_t)(~ch[s]) + out_tree_off];
-            d_[i] = sum;
+            for (int s = 0; s < 8; ++s) if (ch[s] < 0 && ch[s] != NO_CHILD) sum += Num<T>::ld(s_[(int64_t)(~ch[s]) + out_tree_off]);
+            d_[i] = Num<T>::st(sum);
         }
     }
 }
@@ -329,6 +331,21 @@ extern "C" {
 
 TREE_OPS_API(float, f32)
 TREE_OPS_API(double, f64)
+// bfloat16 storage (uint16_t bit patterns at the boundary), fp32 arithmetic
+#define TREE_OPS_BF16(NAME, ARGS, CALL)                                                                              \
+    int aprnet_##NAME##_bf16 ARGS { typedef bf16_t B; return CALL; }
+TREE_OPS_BF16(fill_tree_mean, (const aprnet_plan* p, int d, const uint16_t* x, int64_t ldx, int C, uint16_t* tree, int64_t ldt, void* st),
+              fill_tree_mean<B>(p, d, (const B*)x, ldx, C, (B*)tree, ldt, (hipStream_t)st))
+TREE_OPS_BF16(fill_tree_mean_bwd, (const aprnet_plan* p, int d, uint16_t* gx, int64_t ldx, int C, uint16_t* gt, int64_t ldt, void* st),
+              fill_tree_mean_bwd<B>(p, d, (B*)gx, ldx, C, (B*)gt, ldt, (hipStream_t)st))
+TREE_OPS_BF16(maxpool_fwd, (const aprnet_plan* p, int d, const uint16_t* x, int64_t ldx, int C, uint16_t* y, int64_t ldy, int64_t* arg, int64_t ldi, void* st),
+              maxpool_fwd<B>(p, d, (const B*)x, ldx, C, (B*)y, ldy, arg, ldi, (hipStream_t)st))
+TREE_OPS_BF16(maxpool_bwd, (const aprnet_plan* p, int d, const uint16_t* gy, int64_t ldy, int C, uint16_t* gx, int64_t ldx, const int64_t* arg, int64_t ldi, void* st),
+              maxpool_bwd<B>(p, d, (const B*)gy, ldy, C, (B*)gx, ldx, arg, ldi, (hipStream_t)st))
+TREE_OPS_BF16(upsample_fwd, (const aprnet_plan* p, int d, const uint16_t* x, int64_t ldx, int C, uint16_t* y, int64_t ldy, void* st),
+              (upsample<B, false>(p, d, (const B*)x, ldx, C, (B*)y, ldy, (hipStream_t)st)))
+TREE_OPS_BF16(upsample_bwd, (const aprnet_plan* p, int d, const uint16_t* gy, int64_t ldy, int C, uint16_t* gx, int64_t ldx, void* st),
+              (upsample<B, true>(p, d, (const B*)gy, ldy, C, (B*)gx, ldx, (hipStream_t)st)))
 
 }  // extern "C"
 
@@ -339,6 +356,9 @@ int fill_tree_for_conv(const aprnet_plan* p, int d, const float* x, int64_t ldx,
 }
 int fill_tree_for_conv(const aprnet_plan* p, int d, const double* x, int64_t ldx, int C, double* tree, int64_t ldt, hipStream_t st) {
     return fill_tree_mean<double>(p, d, x, ldx, C, tree, ldt, st);
+}
+int fill_tree_for_conv(const aprnet_plan* p, int d, const bf16_t* x, int64_t ldx, int C, bf16_t* tree, int64_t ldt, hipStream_t st) {
+    return fill_tree_mean<bf16_t>(p, d, x, ldx, C, tree, ldt, st);
 }
 int fill_tree_bwd_for_conv(const aprnet_plan* p, int d, float* gx, int64_t ldx, int C, float* gt, int64_t ldt, hipStream_t st) {
     return fill_tree_mean_bwd<float>(p, d, gx, ldx, C, gt, ldt, st);

@@ -98,5 +98,15 @@ def hip():
         getattr(lib, f"aprnet_reconstruct_bwd_{t}").argtypes = [vp, i32, vp, i64, i32, vp, i64, vp]
         getattr(lib, f"aprnet_sample_particles_fwd_{t}").argtypes = [vp, i32, vp, i64, i32, vp, i64, vp]
         getattr(lib, f"aprnet_sample_particles_bwd_{t}").argtypes = [vp, i32, vp, i64, i32, vp, i64, vp]
+    # bfloat16 features: forward operators of the network, backward of pool / upsample / tree fill
+    lib.aprnet_conv_fwd_bf16.argtypes = [vp, i32, i32, i32, i32, vp, i64, i32, vp, i32, i32, vp, vp, i64, vp, i64, vp]
+    lib.aprnet_conv111_fwd_bf16.argtypes = [vp, i32, vp, i64, i32, vp, i32, i32, vp, vp, i64, vp]
+    lib.aprnet_fill_tree_mean_bf16.argtypes = [vp, i32, vp, i64, i32, vp, i64, vp]
+    lib.aprnet_fill_tree_mean_bwd_bf16.argtypes = [vp, i32, vp, i64, i32, vp, i64, vp]
+    lib.aprnet_maxpool_fwd_bf16.argtypes = [vp, i32, vp, i64, i32, vp, i64, vp, i64, vp]
+    lib.aprnet_maxpool_bwd_bf16.argtypes = [vp, i32, vp, i64, i32, vp, i64, vp, i64, vp]
+    lib.aprnet_upsample_fwd_bf16.argtypes = [vp, i32, vp, i64, i32, vp, i64, vp]
+    lib.aprnet_upsample_bwd_bf16.argtypes = [vp, i32, vp, i64, i32, vp, i64, vp]
+    lib.aprnet_channel_sum_work_elems.argtypes = [i32]
     _hip = lib
     return lib

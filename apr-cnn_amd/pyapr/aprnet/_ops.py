@@ -26,12 +26,16 @@ def _raise(rc, what):
     raise RuntimeError(msg or what)              # TORCH_CHECK -> RuntimeError
 
 
-def _sfx(t):
+def _sfx(t, bf16=False):
+    """Entry-point suffix of a tensor's element type.  bfloat16 is a storage type of the features for the
+    operators that pass bf16=True (forward operators of the network, backward of pool / upsample)."""
     if t.dtype == torch.float32:
         return "f32"
     if t.dtype == torch.float64:
         return "f64"
-    raise TypeError(f"aprnet operators support float32 and float64 tensors, got {t.dtype}")
+    if t.dtype == torch.bfloat16 and bf16:
+        return "bf16"
+    raise TypeError(f"this aprnet operator does not support {t.dtype} tensors")
 
 
 def _check_input(t, name):
@@ -126,10 +130,16 @@ def conv_forward(aprs, x, weights, level_delta, bias=None):
     bias ([Cout], optional) is added inside the kernel instead of in a separate pass over the output."""
     _check_input(x, "input")
     _check_input(weights, "weights")
+    if x.dtype == torch.bfloat16:
+        # bfloat16 is the storage type of the features only: weights and bias are used in fp32
+        weights = weights.float()
+        bias = None if bias is None else bias.float()
+    elif weights.dtype != x.dtype:
+        raise ValueError("weights must have the dtype of the input")
     if bias is not None:
         _check_input(bias, "bias")
-        if bias.dtype != x.dtype or bias.numel() != weights.size(1):
-            raise ValueError("bias must hold one value per output channel, in the dtype of the input")
+        if bias.dtype != weights.dtype or bias.numel() != weights.size(1):
+            raise ValueError("bias must hold one value per output channel, in the dtype of the weights")
     bptr = _ptr(bias) if bias is not None else None
     if x.size(1) != weights.size(2):
         raise ValueError("convolve: input tensor shape does not match weights tensor!")   # conv.hpp:63-66
@@ -147,7 +157,7 @@ def conv_forward(aprs, x, weights, level_delta, bias=None):
             if nb < N:
                 out[b, :, nb:] = bias.view(-1, 1)
     plans = _plans(aprs, x.device)
-    sfx = _sfx(x)
+    sfx = _sfx(x, bf16=True)
     with torch.cuda.device(x.device):
         st = _stream()
         if (kz, kx, ky) == (1, 1, 1):
@@ -239,7 +249,7 @@ def maxpool_forward(aprs, x, level_delta, pad_value=-1e17):
             out[b, :, nb:] = pad_value
             idx[b, :, nb:] = 0
     plans = _plans(aprs, x.device)
-    fn = getattr(_lib(), "aprnet_maxpool_fwd_" + _sfx(x))
+    fn = getattr(_lib(), "aprnet_maxpool_fwd_" + _sfx(x, bf16=True))
     with torch.cuda.device(x.device):
         st = _stream()
         for b in range(B):
@@ -259,7 +269,7 @@ def maxpool_backward(aprs, grad_output, max_indices, level_delta):
     gx = torch.empty((B, Cn, n_in), dtype=grad_output.dtype, device=grad_output.device)
     _zero_tails(gx, sizes)
     plans = _plans(aprs, grad_output.device)
-    fn = getattr(_lib(), "aprnet_maxpool_bwd_" + _sfx(grad_output))
+    fn = getattr(_lib(), "aprnet_maxpool_bwd_" + _sfx(grad_output, bf16=True))
     with torch.cuda.device(grad_output.device):
         st = _stream()
         for b in range(B):
@@ -283,7 +293,7 @@ def upsample_const_forward(aprs, x, level_delta):
     out = torch.empty((B, Cn, n_out), dtype=x.dtype, device=x.device)
     _zero_tails(out, sizes)
     plans = _plans(aprs, x.device)
-    fn = getattr(_lib(), "aprnet_upsample_fwd_" + _sfx(x))
+    fn = getattr(_lib(), "aprnet_upsample_fwd_" + _sfx(x, bf16=True))
     with torch.cuda.device(x.device):
         st = _stream()
         for b in range(B):
@@ -302,7 +312,7 @@ def upsample_const_backward(aprs, grad_output, level_delta):
     gx = torch.empty((B, Cn, n_in), dtype=grad_output.dtype, device=grad_output.device)
     _zero_tails(gx, sizes)
     plans = _plans(aprs, grad_output.device)
-    fn = getattr(_lib(), "aprnet_upsample_bwd_" + _sfx(grad_output))
+    fn = getattr(_lib(), "aprnet_upsample_bwd_" + _sfx(grad_output, bf16=True))
     with torch.cuda.device(grad_output.device):
         st = _stream()
         for b in range(B):

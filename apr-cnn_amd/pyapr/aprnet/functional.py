@@ -37,6 +37,8 @@ class ConvFunction(Function):
         ctx.aprs = aprs
         ctx.layout = layout
         w = _to_device_layout(weights, layout).contiguous()
+        if inputs.dtype == torch.bfloat16:
+            w = w.float()          # bfloat16 stores the features; stencils are restricted and applied in fp32
         ctx.num_stencils = w.shape[0]
         ksize = tuple(w.shape[3:])
         if ksize not in SUPPORTED_KERNELS:

@@ -132,6 +132,17 @@ def other_ops(apr, x, dev):
     with torch.no_grad():
         ms = _time(lambda: net(xin, [apr]), iters=3, warmup=1)
     res.append({"op": "apr_unet_fwd", "ms": ms, "note": f"4 levels 16-32-64-128, fp32, {n0} particles, norms folded"})
+    # bfloat16 features (fp32 weights and arithmetic inside the operators)
+    xb = x.to(torch.bfloat16)
+    with torch.no_grad():
+        ms = _time(lambda: conv(xb, [apr], ld0), iters=5, warmup=1)
+        res.append({"op": "conv333_fwd_bf16", "ms": ms, "particles_per_s": n0 / ms * 1e3,
+                    "note": f"{C}->{C}, bfloat16 features, fp32 matrix math, whole APRConv.forward"})
+        ms = _time(lambda: _ops.maxpool_forward([apr], xb, ld0, 0.0))
+        line("maxpool_fwd_bf16", ms, 2 * C * n0 + (2 + 8) * C * n1, "bfloat16 values, int64 argmax")
+        xinb = xin.to(torch.bfloat16)
+        ms = _time(lambda: net(xinb, [apr]), iters=3, warmup=1)
+    res.append({"op": "apr_unet_fwd_bf16", "ms": ms, "note": "same network, bfloat16 features"})
     return res
 
 

@@ -153,6 +153,29 @@ int aprnet_channel_sum_f64(const double* x, int64_t ld, int C, int64_t n, double
 APRNET_DECL(float, f32)
 APRNET_DECL(double, f64)
 
+/* bfloat16 features (uint16_t bit patterns; no counterpart in the reference, which has no 16-bit path).
+ * Storage only: values are widened to fp32 on load, all arithmetic is fp32, results are rounded to nearest
+ * even on store.  Weights and bias stay fp32.  Forward operators of the APR-UNet, plus the backward passes
+ * of pool / upsample / tree fill; the convolution backward is not available in bfloat16.  Argument meaning
+ * as for the _f32 entry points. */
+int aprnet_conv_fwd_bf16(const aprnet_plan*, int level_delta, int kz, int kx, int ky, const uint16_t* x, int64_t ldx, int Cin,
+                         const float* w, int S_exp, int Cout, const float* bias, uint16_t* y, int64_t ldy,
+                         uint16_t* tree_ws, int64_t ld_tree, void* stream);          /* 3x3x3 only */
+int aprnet_conv111_fwd_bf16(const aprnet_plan*, int level_delta, const uint16_t* x, int64_t ldx, int Cin, const float* w,
+                            int S, int Cout, const float* bias, uint16_t* y, int64_t ldy, void* stream);
+int aprnet_fill_tree_mean_bf16(const aprnet_plan*, int level_delta, const uint16_t* x, int64_t ldx, int C, uint16_t* tree,
+                               int64_t ld_tree, void* stream);
+int aprnet_fill_tree_mean_bwd_bf16(const aprnet_plan*, int level_delta, uint16_t* gx, int64_t ldx, int C, uint16_t* gtree,
+                                   int64_t ld_tree, void* stream);
+int aprnet_maxpool_fwd_bf16(const aprnet_plan*, int level_delta, const uint16_t* x, int64_t ldx, int C, uint16_t* y, int64_t ldy,
+                            int64_t* argmax, int64_t ldi, void* stream);
+int aprnet_maxpool_bwd_bf16(const aprnet_plan*, int level_delta, const uint16_t* gy, int64_t ldy, int C, uint16_t* gx,
+                            int64_t ldx, const int64_t* argmax, int64_t ldi, void* stream);
+int aprnet_upsample_fwd_bf16(const aprnet_plan*, int level_delta, const uint16_t* x, int64_t ldx, int C, uint16_t* y,
+                             int64_t ldy, void* stream);
+int aprnet_upsample_bwd_bf16(const aprnet_plan*, int level_delta, const uint16_t* gy, int64_t ldy, int C, uint16_t* gx,
+                             int64_t ldx, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -307,3 +307,63 @@ def test_reconstruct_and_sample(bt, dtype):
     close(_ops.sample_particles_forward(aprs, im.to(DEV), ld), oracle.sample_particles_forward(aprs, im, ld), dtype)
     close(_ops.reconstruct_backward(aprs, im.to(DEV), ld), oracle.reconstruct_backward(aprs, im, ld), dtype)
     close(_ops.sample_particles_backward(aprs, xd, ld), oracle.sample_particles_backward(aprs, x, ld), dtype)
+
+
+# ------------------------------------------------------------------------------------------- bfloat16 features
+def close_bf16(got, ref):
+    """bfloat16 storage, fp32 arithmetic: every stored value is within half a unit in the 8th mantissa bit of
+    the fp32 result; 2e-2 of the output scale is the stated bound, 1e-2 is asserted."""
+    assert got.dtype == torch.bfloat16
+    scale = max(float(ref.abs().max()), 1e-30)
+    err = float((got.detach().float().cpu() - ref).abs().max())
+    assert err <= 1e-2 * scale, f"max abs err {err:.3e} vs scale {scale:.3e}"
+
+
+@pytest.mark.parametrize("cin,cout", [(1, 16), (32, 32), (33, 17)])
+@pytest.mark.parametrize("bt", [[("3d_a", 0)], [("3d_b", 1), ("3d_c", 2)], [("3d_s", 0), ("3d_t", 1)]],
+                         ids=lambda b: "+".join(f"{n}@{d}" for n, d in b))
+def test_conv333_forward_bf16(bt, cin, cout):
+    x, aprs, ld, w_exp = _conv_case(bt, (3, 3, 3), 2, cin, cout, torch.float32)
+    xb = x.to(torch.bfloat16)
+    g = torch.Generator().manual_seed(11)
+    bias = torch.randn(cout, generator=g)
+    ref = oracle.conv_forward(aprs, xb.float(), w_exp, ld) + bias.view(1, -1, 1)
+    got = _ops.conv_forward(aprs, xb.to(DEV), w_exp.permute(1, 2, 0, 3, 4, 5).contiguous().to(DEV), ld, bias.to(DEV))
+    close_bf16(got, ref)
+
+
+def test_conv111_forward_bf16():
+    x, aprs, ld, w = _conv_case([("3d_b", 1), ("3d_c", 0)], (1, 1, 1), 3, 20, 9, torch.float32)
+    xb = x.to(torch.bfloat16)
+    ref = oracle.conv_forward(aprs, xb.float(), w, ld)
+    got = _ops.conv_forward(aprs, xb.to(DEV), w.permute(1, 2, 0, 3, 4, 5).contiguous().to(DEV), ld)
+    close_bf16(got, ref)
+
+
+@pytest.mark.parametrize("bt", POOL_BATCHES[:4], ids=lambda b: "+".join(f"{n}@{d}" for n, d in b))
+def test_maxpool_upsample_bf16_bit_exact(bt):
+    """Pool and upsample move values without arithmetic: bfloat16 results equal the oracle's on the same
+    (bfloat16-representable) values bit for bit, argmax included."""
+    x, aprs, ld = batch(bt, 5, torch.float32)
+    xb = x.to(torch.bfloat16)
+    ref, ref_idx = oracle.maxpool_forward(aprs, xb.float(), ld)
+    out, idx = _ops.maxpool_forward(aprs, xb.to(DEV), ld)
+    assert out.dtype == torch.bfloat16
+    ref = ref.to(torch.bfloat16).float()        # the -1e17 fill of padding slots (maxpool.hpp:51) rounds in bfloat16
+    assert torch.equal(out.float().cpu(), ref)
+    assert torch.equal(idx.cpu(), ref_idx)
+    ld1 = ld + 1
+    up_ref = oracle.upsample_const_forward(aprs, ref, ld1)
+    up = _ops.upsample_const_forward(aprs, out, ld1)
+    assert torch.equal(up.float().cpu(), up_ref)
+    g = torch.Generator().manual_seed(3)
+    go = torch.randn(ref.shape, generator=g).to(torch.bfloat16)
+    gref = oracle.maxpool_backward(aprs, go.float(), ref_idx, ld)
+    assert torch.equal(_ops.maxpool_backward(aprs, go.to(DEV), idx, ld).float().cpu(), gref)
+
+
+def test_conv_backward_bf16_is_refused():
+    x, aprs, ld, w_exp = _conv_case([("3d_a", 0)], (3, 3, 3), 1, 2, 2, torch.float32)
+    wd = w_exp.permute(1, 2, 0, 3, 4, 5).contiguous().to(DEV)
+    with pytest.raises(TypeError):
+        _ops.conv_backward(aprs, x.to(torch.bfloat16).to(DEV), wd, x.to(torch.bfloat16).to(DEV), ld)
