@@ -128,26 +128,27 @@ template <typename T> struct Chunk;       // channels staged per pass so that th
 template <> struct Chunk<float>  { static constexpr int c333 = 8, c133 = 16, c155 = 12, c555 = 4; };
 template <> struct Chunk<double> { static constexpr int c333 = 4, c133 = 8,  c155 = 6,  c555 = 2; };
 
-int launch_conv333_mfma(const ConvArgs<float>& a, int n_tiles, hipStream_t st);
-int launch_conv333_mfma(const ConvArgs<bf16_t>& a, int n_tiles, hipStream_t st);
+bool conv_mfma_supported(int code);
+int launch_conv_mfma(int code, const ConvArgs<float>& a, int n_tiles, hipStream_t st);
+int launch_conv_mfma(int code, const ConvArgs<bf16_t>& a, int n_tiles, hipStream_t st);
 int fill_tree_for_conv(const aprnet_plan* p, int d, const bf16_t* x, int64_t ldx, int C, bf16_t* tree, int64_t ldt, hipStream_t st);
-size_t conv333_packed_floats(int S_exp, int Cout, int Cin);
-int pack_conv333_weights(const float* w, int S_exp, int Cm, int Ck, bool transposed, float* packed, hipStream_t st);
+size_t conv_packed_floats(int code, int S_exp, int Cm, int Ck);
+int pack_conv_weights(int code, const float* w, int S_exp, int Cm, int Ck, bool transposed, float* packed, hipStream_t st);
 
 static int g_conv_path = 0;      // 0: matrix cores where available, 1: VALU kernels only
 int conv_path() { return g_conv_path; }
 
 template <typename T> static int try_mfma(aprnet_plan*, const ConvArgs<T>&, int, int, hipStream_t, bool*) { return 0; }
 template <> int try_mfma<float>(aprnet_plan* p, const ConvArgs<float>& a, int code, int n_tiles, hipStream_t st, bool* done) {
-    if (g_conv_path == 1 || code != 333) return 0;
+    if (g_conv_path == 1 || !conv_mfma_supported(code)) return 0;
     *done = true;
     // plan-owned scratch for the re-laid-out weights, grown on demand
-    if (int rc = plan_scratch(p, conv333_packed_floats(a.S_exp, a.Cout, a.Cin) * sizeof(float), st)) return rc;
-    if (int rc = pack_conv333_weights(a.w, a.S_exp, a.Cout, a.Cin, false, (float*)p->d_scratch, st)) return rc;
+    if (int rc = plan_scratch(p, conv_packed_floats(code, a.S_exp, a.Cout, a.Cin) * sizeof(float), st)) return rc;
+    if (int rc = pack_conv_weights(code, a.w, a.S_exp, a.Cout, a.Cin, false, (float*)p->d_scratch, st)) return rc;
     ConvArgs<float> b = a;
     b.w = (const float*)p->d_scratch;
     TimedLaunch timed(st);
-    return launch_conv333_mfma(b, n_tiles, st);
+    return launch_conv_mfma(code, b, n_tiles, st);
 }
 
 int fill_tree_for_conv(const aprnet_plan* p, int d, const float* x, int64_t ldx, int C, float* tree, int64_t ldt, hipStream_t st);
@@ -195,23 +196,25 @@ int conv_fwd_bf16(const aprnet_plan* cp, int d, int kz, int kx, int ky, const bf
     aprnet_plan* p = const_cast<aprnet_plan*>(cp);
     if (int rc = check_level_delta(p, d, "conv_forward")) return rc;
     if (Cin <= 0 || Cout <= 0 || S_exp <= 0) return fail(APRNET_ERR_INVALID_ARGUMENT, "conv_forward: empty channel / stencil count");
-    if (kz != 3 || kx != 3 || ky != 3) return fail(APRNET_ERR_UNSUPPORTED, "conv_forward: bfloat16 features are supported for the 3x3x3 stencil only");
+    const int code = kz * 100 + kx * 10 + ky;
+    if (!conv_mfma_supported(code))
+        return fail(APRNET_ERR_UNSUPPORTED, "conv_forward: bfloat16 features are supported for the 3x3x3, 1x3x3 and 1x5x5 stencils");
     const int64_t nt = p->tree_parts(d);
     if (nt > 0 && (!tree_ws || ldt < nt)) return fail(APRNET_ERR_INVALID_ARGUMENT, "conv_forward: tree work space too small");
     APRNET_HIP_CHECK(hipSetDevice(p->device));
     if (int rc = fill_tree_for_conv(p, d, x, ldx, Cin, tree_ws, ldt, st)) return rc;
     TileList tl;
-    if (int rc = get_tiles(p, d, 2, 4, &tl)) return rc;
+    if (int rc = get_tiles(p, d, kz == 1 ? 1 : 2, kz == 1 ? 8 : 4, &tl)) return rc;
     if (tl.n == 0) return 0;
-    if (int rc = plan_scratch(p, conv333_packed_floats(S_exp, Cout, Cin) * sizeof(float), st)) return rc;
-    if (int rc = pack_conv333_weights(w, S_exp, Cout, Cin, false, (float*)p->d_scratch, st)) return rc;
+    if (int rc = plan_scratch(p, conv_packed_floats(code, S_exp, Cout, Cin) * sizeof(float), st)) return rc;
+    if (int rc = pack_conv_weights(code, w, S_exp, Cout, Cin, false, (float*)p->d_scratch, st)) return rc;
     ConvArgs<bf16_t> a{};
     a.apr = p->dapr; a.tree = p->dtree; a.tiles = tl.d_tiles;
     a.x = x; a.ldx = ldx; a.Cin = Cin; a.w = (const float*)p->d_scratch; a.S_exp = S_exp; a.Cout = Cout; a.bias = bias;
     a.y = y; a.ldy = ldy; a.tree_data = tree_ws; a.ldt = ldt; a.Lc = p->lc(d); a.tree_off = p->tree_offset(a.Lc);
     a.x_count = p->number_parts(d); a.t_count = p->tree_parts(d);
     TimedLaunch timed(st);
-    return launch_conv333_mfma(a, tl.n, st);
+    return launch_conv_mfma(code, a, tl.n, st);
 }
 
 }  // namespace aprnet

@@ -226,28 +226,29 @@ static int launch_bwd(ConvArgs<T>& a, hipStream_t st) {
 }
 
 // matrix-core kernels (conv_mfma.hip, conv_bwd_mfma.hip)
-int launch_conv333_dx_mfma(const ConvArgs<float>& a, int n_tiles, hipStream_t st);
-int launch_conv333_dw_mfma(const ConvArgs<float>& a, const TileList& tl, int level_min, hipStream_t st);
-size_t conv333_packed_floats(int S_exp, int Cm, int Ck);
-int pack_conv333_weights(const float* w, int S_exp, int Cm, int Ck, bool transposed, float* packed, hipStream_t st);
+bool conv_mfma_supported(int code);
+int launch_conv_dx_mfma(int code, const ConvArgs<float>& a, int n_tiles, hipStream_t st);
+int launch_conv_dw_mfma(int code, const ConvArgs<float>& a, const TileList& tl, int level_min, hipStream_t st);
+size_t conv_packed_floats(int code, int S_exp, int Cm, int Ck);
+int pack_conv_weights(int code, const float* w, int S_exp, int Cm, int Ck, bool transposed, float* packed, hipStream_t st);
 int conv_path();
 
 template <typename T> static int try_mfma_bwd(aprnet_plan*, const ConvArgs<T>&, const TileList&, int, int, hipStream_t, bool*) { return 0; }
 template <> int try_mfma_bwd<float>(aprnet_plan* p, const ConvArgs<float>& a, const TileList& tl, int code, int d, hipStream_t st, bool* done) {
-    if (conv_path() == 1 || code != 333) return 0;
+    if (conv_path() == 1 || !conv_mfma_supported(code)) return 0;
     *done = true;
     // input gradient: the forward kernel on the output gradient with the transposed, flipped stencil;
     // every row group within one row of an output takes part
     TileList near;
-    if (int rc = get_tiles(p, d, 2, 4, &near, 1)) return rc;
-    if (int rc = plan_scratch(p, conv333_packed_floats(a.S_exp, a.Cin, a.Cout) * sizeof(float), st)) return rc;
-    if (int rc = pack_conv333_weights(a.w, a.S_exp, a.Cin, a.Cout, true, (float*)p->d_scratch, st)) return rc;
+    if (int rc = get_tiles(p, d, code == 333 ? 2 : 1, code == 333 ? 4 : 8, &near, 1)) return rc;
+    if (int rc = plan_scratch(p, conv_packed_floats(code, a.S_exp, a.Cin, a.Cout) * sizeof(float), st)) return rc;
+    if (int rc = pack_conv_weights(code, a.w, a.S_exp, a.Cin, a.Cout, true, (float*)p->d_scratch, st)) return rc;
     ConvArgs<float> b = a;
     b.tiles = near.d_tiles; b.n_tiles = near.n;
     b.x = a.gy; b.ldx = a.ldy; b.Cin = a.Cout; b.Cout = a.Cin; b.w = (const float*)p->d_scratch; b.bias = nullptr;
     b.tree_data = nullptr; b.t_count = 0;
-    if (near.n > 0) if (int rc = launch_conv333_dx_mfma(b, near.n, st)) return rc;
-    return launch_conv333_dw_mfma(a, tl, p->apr.level_min, st);
+    if (near.n > 0) if (int rc = launch_conv_dx_mfma(code, b, near.n, st)) return rc;
+    return launch_conv_dw_mfma(code, a, tl, p->apr.level_min, st);
 }
 
 template <typename T>

@@ -23,7 +23,10 @@ namespace aprnet {
 
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 
+// row strides that put the tap offsets of one B read into different banks: 67 for 3-wide, 69 for 5-wide rows
 using W333M = ConvGeom<3, 3, 3, 2, 4, 512, 67>;
+using W133M = ConvGeom<1, 3, 3, 1, 8, 512, 67>;
+using W155M = ConvGeom<1, 5, 5, 1, 8, 512, 69>;
 constexpr int DW_CIB = 4;          // input channels per staged chunk
 constexpr int DW_NCH = 4;          // chunks per block
 constexpr int DW_GB = 256;         // columns of gY staged at a time
@@ -126,10 +129,11 @@ conv_dw_mfma_kernel(const ConvArgs<float> a, const int s_idx) {
     }
 }
 
-// Weight gradient of the 3x3x3 stencil; a.gw is accumulated into (the caller zeroes it).
+// Weight gradient; a.gw is accumulated into (the caller zeroes it).
 // One launch per stencil index: level Lc - s for s < S_exp - 1, every coarser level for the last one
 // (adjacent in the tile list, which is sorted finest level first).
-int launch_conv333_dw_mfma(const ConvArgs<float>& a0, const TileList& tl, int level_min, hipStream_t st) {
+template <class G>
+static int launch_dw(const ConvArgs<float>& a0, const TileList& tl, int level_min, hipStream_t st) {
     for (int s = 0; s < a0.S_exp; ++s) {
         const int l_hi = a0.Lc - s, l_lo = (s == a0.S_exp - 1) ? level_min : l_hi;
         if (l_hi < level_min) break;
@@ -140,10 +144,19 @@ int launch_conv333_dw_mfma(const ConvArgs<float>& a0, const TileList& tl, int le
         a.tiles = tl.d_tiles + tl.level_begin[l_hi]; a.n_tiles = n;
         dim3 grid((unsigned)std::min(n, 512), (unsigned)((a.Cin + DW_CIB * DW_NCH - 1) / (DW_CIB * DW_NCH)),
                   (unsigned)((a.Cout + 31) / 32));
-        hipLaunchKernelGGL((conv_dw_mfma_kernel<W333M, DW_CIB, DW_NCH>), grid, dim3(W333M::NT), 0, st, a, s);
+        hipLaunchKernelGGL((conv_dw_mfma_kernel<G, DW_CIB, DW_NCH>), grid, dim3(G::NT), 0, st, a, s);
         APRNET_LAUNCH_CHECK("conv_dw_mfma_kernel");
     }
     return 0;
+}
+
+int launch_conv_dw_mfma(int code, const ConvArgs<float>& a, const TileList& tl, int level_min, hipStream_t st) {
+    switch (code) {
+        case 333: return launch_dw<W333M>(a, tl, level_min, st);
+        case 133: return launch_dw<W133M>(a, tl, level_min, st);
+        case 155: return launch_dw<W155M>(a, tl, level_min, st);
+    }
+    return fail(APRNET_ERR_UNSUPPORTED, "no matrix-core kernel for this stencil");
 }
 
 }  // namespace aprnet

@@ -217,43 +217,51 @@ conv_mfma16_kernel(const ConvArgs<T> a) {
 }
 
 using M333N = ConvGeom<3, 3, 3, 2, 4, 512, 64, 16>;
+using M133N = ConvGeom<1, 3, 3, 1, 8, 512, 64, 16>;
+using M155N = ConvGeom<1, 5, 5, 1, 8, 512, 64, 16>;
 
-static int conv333_coh(int Cm) { return Cm <= 16 ? 1 : 2; }
+// stencils with a matrix-core kernel (kz*100 + kx*10 + ky); 5x5x5 needs a weight chunk that does not fit LDS
+bool conv_mfma_supported(int code) { return code == 333 || code == 133 || code == 155; }
+static int conv_taps(int code) { return code == 333 ? 27 : code == 133 ? 9 : 25; }
+static int conv_coh(int Cm) { return Cm <= 16 ? 1 : 2; }
 
-// Forward.  a.w must point at the packed weights (pack_conv333_weights).
-template <typename T>
-static int launch_fwd16(const ConvArgs<T>& a, int n_tiles, hipStream_t st) {
-    const int coh = conv333_coh(a.Cout);
+template <typename T, class G, int MODE>
+static int launch16(const ConvArgs<T>& a, int n_tiles, hipStream_t st) {
+    const int coh = conv_coh(a.Cout);
     dim3 grid((unsigned)n_tiles, (unsigned)((a.Cout + 16 * coh - 1) / (16 * coh)));
-    if (coh == 1) hipLaunchKernelGGL((conv_mfma16_kernel<T, M333N, 1, 0>), grid, dim3(M333N::NT), 0, st, a);
-    else hipLaunchKernelGGL((conv_mfma16_kernel<T, M333N, 2, 0>), grid, dim3(M333N::NT), 0, st, a);
-    APRNET_LAUNCH_CHECK("conv_mfma16_kernel (forward)");
+    if (coh == 1) hipLaunchKernelGGL((conv_mfma16_kernel<T, G, 1, MODE>), grid, dim3(G::NT), 0, st, a);
+    else hipLaunchKernelGGL((conv_mfma16_kernel<T, G, 2, MODE>), grid, dim3(G::NT), 0, st, a);
+    APRNET_LAUNCH_CHECK("conv_mfma16_kernel");
     return 0;
 }
-int launch_conv333_mfma(const ConvArgs<float>& a, int n_tiles, hipStream_t st) { return launch_fwd16<float>(a, n_tiles, st); }
-int launch_conv333_mfma(const ConvArgs<bf16_t>& a, int n_tiles, hipStream_t st) { return launch_fwd16<bf16_t>(a, n_tiles, st); }
+template <typename T, int MODE>
+static int launch16_code(int code, const ConvArgs<T>& a, int n_tiles, hipStream_t st) {
+    switch (code) {
+        case 333: return launch16<T, M333N, MODE>(a, n_tiles, st);
+        case 133: return launch16<T, M133N, MODE>(a, n_tiles, st);
+        case 155: return launch16<T, M155N, MODE>(a, n_tiles, st);
+    }
+    return fail(APRNET_ERR_UNSUPPORTED, "no matrix-core kernel for this stencil");
+}
+
+// Forward.  a.w must point at the packed weights (pack_conv_weights).
+int launch_conv_mfma(int code, const ConvArgs<float>& a, int n_tiles, hipStream_t st) { return launch16_code<float, 0>(code, a, n_tiles, st); }
+int launch_conv_mfma(int code, const ConvArgs<bf16_t>& a, int n_tiles, hipStream_t st) { return launch16_code<bf16_t, 0>(code, a, n_tiles, st); }
 
 // Input gradient: a.x / a.Cin describe the output gradient, a.Cout the input channels, a.w the packed
 // transposed weights, a.tiles the row groups within one row of an output (n_tiles of them).
-int launch_conv333_dx_mfma(const ConvArgs<float>& a, int n_tiles, hipStream_t st) {
-    const int coh = conv333_coh(a.Cout);
-    dim3 grid((unsigned)n_tiles, (unsigned)((a.Cout + 16 * coh - 1) / (16 * coh)));
-    if (coh == 1) hipLaunchKernelGGL((conv_mfma16_kernel<float, M333N, 1, 1>), grid, dim3(M333N::NT), 0, st, a);
-    else hipLaunchKernelGGL((conv_mfma16_kernel<float, M333N, 2, 1>), grid, dim3(M333N::NT), 0, st, a);
-    APRNET_LAUNCH_CHECK("conv_mfma16_kernel (input gradient)");
-    return 0;
-}
+int launch_conv_dx_mfma(int code, const ConvArgs<float>& a, int n_tiles, hipStream_t st) { return launch16_code<float, 1>(code, a, n_tiles, st); }
 
 // Cm: channels on the M axis of the kernel, Ck: contracted channels (forward: Cout, Cin; transposed: Cin, Cout)
-size_t conv333_packed_floats(int S_exp, int Cm, int Ck) {
-    const int coh = conv333_coh(Cm);
-    return (size_t)S_exp * ((Cm + 16 * coh - 1) / (16 * coh)) * ((Ck + 3) / 4) * 4 * 27 * 16 * coh;
+size_t conv_packed_floats(int code, int S_exp, int Cm, int Ck) {
+    const int coh = conv_coh(Cm);
+    return (size_t)S_exp * ((Cm + 16 * coh - 1) / (16 * coh)) * ((Ck + 3) / 4) * 4 * conv_taps(code) * 16 * coh;
 }
 
-int pack_conv333_weights(const float* w, int S_exp, int Cm, int Ck, bool transposed, float* packed, hipStream_t st) {
-    const size_t n = conv333_packed_floats(S_exp, Cm, Ck);
+int pack_conv_weights(int code, const float* w, int S_exp, int Cm, int Ck, bool transposed, float* packed, hipStream_t st) {
+    const size_t n = conv_packed_floats(code, S_exp, Cm, Ck);
     dim3 grid((unsigned)std::min<size_t>((n + 255) / 256, 2048));
-    hipLaunchKernelGGL(pack_weights16_kernel, grid, dim3(256), 0, st, w, S_exp, Cm, Ck, 27, 4, conv333_coh(Cm),
+    hipLaunchKernelGGL(pack_weights16_kernel, grid, dim3(256), 0, st, w, S_exp, Cm, Ck, conv_taps(code), 4, conv_coh(Cm),
                        transposed ? 1 : 0, packed);
     APRNET_LAUNCH_CHECK("pack_weights16_kernel");
     return 0;

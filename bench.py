@@ -132,6 +132,20 @@ def other_ops(apr, x, dev):
     with torch.no_grad():
         ms = _time(lambda: net(xin, [apr]), iters=3, warmup=1)
     res.append({"op": "apr_unet_fwd", "ms": ms, "note": f"4 levels 16-32-64-128, fp32, {n0} particles, norms folded"})
+    # the wide 2-D stencil of configs[4] (1x5x5, 64 -> 64), here on the 3-D benchmark APR, fp32
+    conv5 = aprnet.cuda.APRConv(64, 64, nstencils=2, kernel_size=(1, 5, 5)).to(dev)
+    x64 = torch.randn(1, 64, x.shape[2], device=dev)
+    with torch.no_grad():
+        ms = _time(lambda: conv5(x64, [apr], ld0), iters=3, warmup=1)
+    fl = 2 * 25 * 64 * 64 * n0
+    res.append({"op": "conv155_fwd", "ms": ms, "particles_per_s": n0 / ms * 1e3, "TFLOPs": fl / ms / 1e9,
+                "mfma_frac": fl / ms / 1e9 / PEAK_FP32_MATRIX_TFLOPS, "note": "1x5x5 64->64 fp32, whole APRConv.forward"})
+    x64.requires_grad_(True)
+    y5 = conv5(x64, [apr], ld0)
+    go5 = torch.randn_like(y5)
+    ms = _time(lambda: torch.autograd.grad(y5, (x64, conv5.weight), go5, retain_graph=True), iters=2, warmup=1)
+    res.append({"op": "conv155_bwd", "ms": ms, "particles_per_s": n0 / ms * 1e3, "note": "1x5x5 64->64 grad_input + grad_weight"})
+    del y5, go5, x64, conv5
     # bfloat16 features (fp32 weights and arithmetic inside the operators)
     xb = x.to(torch.bfloat16)
     with torch.no_grad():

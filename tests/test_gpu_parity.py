@@ -219,6 +219,31 @@ def test_conv333_backward_channel_shapes(cin, cout, path):
     close(gw.permute(2, 0, 1, 3, 4, 5), gw_ref, torch.float32)
 
 
+@pytest.mark.parametrize("path", [0, 1], ids=["mfma", "valu"])
+@pytest.mark.parametrize("ksize", [(1, 3, 3), (1, 5, 5)], ids=KID)
+@pytest.mark.parametrize("bt", [[("2d_a", 0), ("2d_b", 1)], [("3d_s", 0)]], ids=lambda b: "+".join(f"{n}@{d}" for n, d in b))
+def test_conv_flat_stencils_wide_channels(bt, ksize, path):
+    """1x3x3 and 1x5x5 (the 2-D stencils) at channel counts that straddle the blocks of the matrix-core
+    kernels, forward and backward, on both fp32 kernel families."""
+    cin, cout = 20, 33
+    x, aprs, ld, w_exp = _conv_case(bt, ksize, 2, cin, cout, torch.float32)
+    g = torch.Generator().manual_seed(8)
+    go = torch.randn(x.size(0), cout, x.size(2), generator=g)
+    ref = oracle.conv_forward(aprs, x, w_exp, ld)
+    gx_ref, gw_ref = oracle.conv_backward(aprs, x, w_exp, go, ld)
+    wd = w_exp.permute(1, 2, 0, 3, 4, 5).contiguous().to(DEV)
+    lib = _native.hip()
+    assert lib.aprnet_set_conv_path(path) == 0
+    try:
+        got = _ops.conv_forward(aprs, x.to(DEV), wd, ld)
+        gx, gw = _ops.conv_backward(aprs, x.to(DEV), wd, go.to(DEV), ld)
+    finally:
+        lib.aprnet_set_conv_path(0)
+    close(got, ref, torch.float32)
+    close(gx, gx_ref, torch.float32)
+    close(gw.permute(2, 0, 1, 3, 4, 5), gw_ref, torch.float32)
+
+
 def test_conv333_backward_dense_windows():
     """Fully refined APR: windows with the maximum number of columns (496 > one staged group of 256 in the
     weight-gradient kernel, all column blocks in the input-gradient kernel)."""
