@@ -131,6 +131,10 @@ template <> struct Chunk<double> { static constexpr int c333 = 4, c133 = 8,  c15
 bool conv_mfma_supported(int code);
 int launch_conv_mfma(int code, const ConvArgs<float>& a, int n_tiles, hipStream_t st);
 int launch_conv_mfma(int code, const ConvArgs<bf16_t>& a, int n_tiles, hipStream_t st);
+int launch_conv_mfma_bf16(int code, const ConvArgs<bf16_t>& a, int n_tiles, hipStream_t st);
+size_t conv_packed_bf16_bytes(int code, int S_exp, int Cout, int Cin);
+int pack_conv_weights_bf16(int code, const float* w, int S_exp, int Cout, int Cin, void* packed, hipStream_t st);
+static int g_bf16_math = 1;      // bfloat16 features: 1 = bfloat16 matrix instructions, 0 = fp32 matrix instructions
 int fill_tree_for_conv(const aprnet_plan* p, int d, const bf16_t* x, int64_t ldx, int C, bf16_t* tree, int64_t ldt, hipStream_t st);
 size_t conv_packed_floats(int code, int S_exp, int Cm, int Ck);
 int pack_conv_weights(int code, const float* w, int S_exp, int Cm, int Ck, bool transposed, float* packed, hipStream_t st);
@@ -206,15 +210,20 @@ int conv_fwd_bf16(const aprnet_plan* cp, int d, int kz, int kx, int ky, const bf
     TileList tl;
     if (int rc = get_tiles(p, d, kz == 1 ? 1 : 2, kz == 1 ? 8 : 4, &tl)) return rc;
     if (tl.n == 0) return 0;
-    if (int rc = plan_scratch(p, conv_packed_floats(code, S_exp, Cout, Cin) * sizeof(float), st)) return rc;
-    if (int rc = pack_conv_weights(code, w, S_exp, Cout, Cin, false, (float*)p->d_scratch, st)) return rc;
+    if (g_bf16_math) {
+        if (int rc = plan_scratch(p, conv_packed_bf16_bytes(code, S_exp, Cout, Cin), st)) return rc;
+        if (int rc = pack_conv_weights_bf16(code, w, S_exp, Cout, Cin, p->d_scratch, st)) return rc;
+    } else {
+        if (int rc = plan_scratch(p, conv_packed_floats(code, S_exp, Cout, Cin) * sizeof(float), st)) return rc;
+        if (int rc = pack_conv_weights(code, w, S_exp, Cout, Cin, false, (float*)p->d_scratch, st)) return rc;
+    }
     ConvArgs<bf16_t> a{};
     a.apr = p->dapr; a.tree = p->dtree; a.tiles = tl.d_tiles;
     a.x = x; a.ldx = ldx; a.Cin = Cin; a.w = (const float*)p->d_scratch; a.S_exp = S_exp; a.Cout = Cout; a.bias = bias;
     a.y = y; a.ldy = ldy; a.tree_data = tree_ws; a.ldt = ldt; a.Lc = p->lc(d); a.tree_off = p->tree_offset(a.Lc);
     a.x_count = p->number_parts(d); a.t_count = p->tree_parts(d);
     TimedLaunch timed(st);
-    return launch_conv_mfma(code, a, tl.n, st);
+    return g_bf16_math ? launch_conv_mfma_bf16(code, a, tl.n, st) : launch_conv_mfma(code, a, tl.n, st);
 }
 
 }  // namespace aprnet
@@ -229,7 +238,9 @@ int aprnet_conv_fwd_bf16(const aprnet_plan* p, int d, int kz, int kx, int ky, co
                          ldt, (hipStream_t)st);
 }
 int aprnet_set_conv_path(int path) {
-    if (path != 0 && path != 1) return fail(APRNET_ERR_INVALID_ARGUMENT, "set_conv_path: 0 (auto) or 1 (VALU only)");
+    if (path == 2 || path == 3) { g_bf16_math = path == 2; return 0; }
+    if (path != 0 && path != 1)
+        return fail(APRNET_ERR_INVALID_ARGUMENT, "set_conv_path: 0 (auto), 1 (VALU only), 2 / 3 (bfloat16 features: bfloat16 / fp32 matrix math)");
     g_conv_path = path;
     return 0;
 }

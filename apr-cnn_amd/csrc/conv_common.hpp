@@ -354,10 +354,12 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t plane_rsrc(const T* base, int6
     return __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(base + (int64_t)c * ld), 0, bytes, 0x00020000);
 }
 
-// Values of one channel chunk for the items of this thread, in registers.
-template <class G, typename T, int CIB>
+// Values of one channel chunk for the items of this thread, in registers.  Thread t owns items t, t + NT, ...
+// ("rounds"); NR of the rounds are held at a time (all of them by default).
+template <class G, typename T, int CIB, int NR = (G::MAXITEM + G::NT - 1) / G::NT>
 struct ItemRegs {
-    static constexpr int IPT = (G::MAXITEM + G::NT - 1) / G::NT;    // items per thread
+    static constexpr int ROUNDS = (G::MAXITEM + G::NT - 1) / G::NT;  // items per thread
+    static constexpr int IPT = NR;
     typename RawLoad<T>::raw v[IPT][CIB];
     unsigned short pos[IPT];
 };
@@ -365,10 +367,10 @@ struct ItemRegs {
 // Issues the loads of a chunk (no LDS writes: they may run ahead of the consumer of the patch).
 // Thread t owns items t, t + NT, ...; a round k that lies beyond the item count is skipped by a
 // wave-uniform branch (most windows hold fewer items than the block has threads).
-template <class G, typename T, int CIB>
+template <class G, typename T, int CIB, int NR>
 __device__ __forceinline__ void load_items(const ConvArgs<T>& a, int ci0, int nitem, bool tree_items,
-                                           const ConvShared<G>& sh, ItemRegs<G, T, CIB>& R) {
-    constexpr int IPT = ItemRegs<G, T, CIB>::IPT;
+                                           const ConvShared<G>& sh, ItemRegs<G, T, CIB, NR>& R, int round0 = 0) {
+    constexpr int IPT = NR;
     __amdgpu_buffer_rsrc_t rx[CIB], rt[CIB];
 #pragma unroll
     for (int c = 0; c < CIB; ++c) {
@@ -377,8 +379,8 @@ __device__ __forceinline__ void load_items(const ConvArgs<T>& a, int ci0, int ni
     }
 #pragma unroll
     for (int k = 0; k < IPT; ++k) {
-        if (k * G::NT >= nitem) break;                  // wave-uniform
-        const int it = threadIdx.x + k * G::NT;
+        if ((round0 + k) * G::NT >= nitem) break;       // wave-uniform
+        const int it = threadIdx.x + (round0 + k) * G::NT;
         unsigned offx = BUF_OOB, offt = BUF_OOB;
         R.pos[k] = 0xffffu;
         if (it < nitem) {
@@ -396,11 +398,12 @@ __device__ __forceinline__ void load_items(const ConvArgs<T>& a, int ci0, int ni
     }
 }
 
-template <class G, typename T, int CIB>
-__device__ __forceinline__ void store_items(const ItemRegs<G, T, CIB>& R, int nitem, typename Num<T>::acc* patch) {
+template <class G, typename T, int CIB, int NR>
+__device__ __forceinline__ void store_items(const ItemRegs<G, T, CIB, NR>& R, int nitem, typename Num<T>::acc* patch,
+                                            int round0 = 0) {
 #pragma unroll
-    for (int k = 0; k < ItemRegs<G, T, CIB>::IPT; ++k) {
-        if (k * G::NT >= nitem) break;                  // wave-uniform
+    for (int k = 0; k < NR; ++k) {
+        if ((round0 + k) * G::NT >= nitem) break;       // wave-uniform
         if (R.pos[k] == 0xffffu) continue;
         typename Num<T>::acc* cell = patch + (R.pos[k] & ITEM_CELL);
 #pragma unroll

@@ -216,6 +216,200 @@ conv_mfma16_kernel(const ConvArgs<T> a) {
     }
 }
 
+// ---------------------------------------------------------------------------------------------------------
+// bfloat16 contraction (forward, bfloat16 features): v_mfma_f32_16x16x16_bf16, fp32 accumulation.
+// The 16 k of one instruction are 2 taps x 8 input channels: lane group g = l/16 supplies four consecutive
+// bfloat16 (8 bytes) of tap 2*step + g/2, channels 4*(g%2) .. +3 of the 8-channel chunk.
+//     patch8[cg][cell]   8 bytes = 4 channels of channel group cg (0, 1) at one cell
+//     Wl8[step][h][lane] 8 bytes = the A operand of that lane (weights rounded to bfloat16 when packed)
+// Channels of the two groups are CH_STRIDE (= 16 mod 32) cells apart, so the lanes of a half wave read
+// 32 different 8-byte bank pairs.  Same lists, same D layout and epilogue as the fp32 kernel; a window needs a
+// quarter of the channel chunks and 1/8 of the matrix instructions.
+typedef short bf16x4 __attribute__((ext_vector_type(4)));
+constexpr int BF_CIB = 8;
+
+template <class G> constexpr int bf16_steps() { return (G::K + 1) / 2; }
+
+// packedB[s][cb][q][step][h][lane] (8 bytes each), cb = block of 16 * COH output channels, q = chunk of 8 inputs
+__global__ void pack_weights_bf16_kernel(const float* __restrict__ w, int S_exp, int Cout, int Cin, int K, int COH,
+                                         uint2* __restrict__ out) {
+    const int ncb = (Cout + 16 * COH - 1) / (16 * COH), nq = (Cin + BF_CIB - 1) / BF_CIB, nstep = (K + 1) / 2;
+    const int64_t n = (int64_t)S_exp * ncb * nq * nstep * COH * 64;
+    for (int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; e < n; e += (int64_t)gridDim.x * blockDim.x) {
+        int64_t r = e;
+        const int lane = (int)(r % 64); r /= 64;
+        const int h = (int)(r % COH); r /= COH;
+        const int step = (int)(r % nstep); r /= nstep;
+        const int q = (int)(r % nq); r /= nq;
+        const int cb = (int)(r % ncb); r /= ncb;
+        const int s = (int)r;
+        const int g = lane >> 4, co = (cb * COH + h) * 16 + (lane & 15);
+        const int t = 2 * step + (g >> 1), ci0 = q * BF_CIB + 4 * (g & 1);
+        unsigned v[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            float f = 0.f;
+            if (t < K && co < Cout && ci0 + j < Cin) f = w[(((int64_t)s * Cout + co) * Cin + ci0 + j) * K + t];
+            v[j] = float_to_bf16(f).bits;
+        }
+        out[e] = make_uint2(v[0] | (v[1] << 16), v[2] | (v[3] << 16));
+    }
+}
+
+template <class G>
+__device__ __forceinline__ void store_items_bf16(const ItemRegs<G, bf16_t, BF_CIB>& R, int nitem, uint2* __restrict__ patch8) {
+#pragma unroll
+    for (int k = 0; k < ItemRegs<G, bf16_t, BF_CIB>::IPT; ++k) {
+        if (k * G::NT >= nitem) break;                  // wave-uniform
+        if (R.pos[k] == 0xffffu) continue;
+        uint2* cell = patch8 + (R.pos[k] & ITEM_CELL);
+#pragma unroll
+        for (int cg = 0; cg < 2; ++cg) {
+            const uint2 v = make_uint2((unsigned)R.v[k][4 * cg] | ((unsigned)R.v[k][4 * cg + 1] << 16),
+                                       (unsigned)R.v[k][4 * cg + 2] | ((unsigned)R.v[k][4 * cg + 3] << 16));
+            cell[cg * G::CH_STRIDE] = v;
+            if (R.pos[k] & ITEM_PAIR) cell[cg * G::CH_STRIDE + 1] = v;
+        }
+    }
+}
+
+template <class G, int COH, int NB>
+__device__ __forceinline__ void mfma_bf16_window(const ConvArgs<bf16_t>& a, int co0, int nc, int nitem, bool tree_items, int first,
+                                                 const uint4* __restrict__ wl, const ConvShared<G>& sh,
+                                                 uint2* __restrict__ patch8, uint2* __restrict__ Wl8,
+                                                 const float* __restrict__ bias_l) {
+    constexpr int NSTEP = bf16_steps<G>();
+    const int lane = lane_id();
+    const bool second_tap = lane >= 32;
+    constexpr int NBA = NB > 0 ? NB : 1;
+    int bbase[NBA];
+#pragma unroll
+    for (int j = 0; j < NB; ++j) {
+        const int col = ((first + G::NWAVE * j) << 4) + (lane & 15);
+        const int pos = col < nc ? (int)(sh.col_pos[col] & COL_CELL) - G::TAP0 : 0;
+        bbase[j] = pos + ((lane >> 4) & 1) * G::CH_STRIDE;
+    }
+    floatx4 acc[NBA][COH];
+#pragma unroll
+    for (int j = 0; j < NB; ++j)
+#pragma unroll
+        for (int h = 0; h < COH; ++h)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) acc[j][h][r] = 0.f;
+
+    constexpr int W16 = NSTEP * COH * 32;                        // 16-byte elements of a weight chunk
+    constexpr int WPT = (W16 + G::NT - 1) / G::NT;
+    ItemRegs<G, bf16_t, BF_CIB> R;
+    uint4 wr[WPT];
+#define APRNET_LOAD_WEIGHTS(q)                                                                     \
+    _Pragma("unroll") for (int k = 0; k < WPT; ++k) {                                              \
+        const int i = threadIdx.x + k * G::NT;                                                     \
+        wr[k] = (i < W16) ? (wl + (int64_t)(q) * W16)[i] : make_uint4(0u, 0u, 0u, 0u);             \
+    }
+#define APRNET_STORE_WEIGHTS()                                                                     \
+    _Pragma("unroll") for (int k = 0; k < WPT; ++k) {                                              \
+        const int i = threadIdx.x + k * G::NT;                                                     \
+        if (i < W16) reinterpret_cast<uint4*>(Wl8)[i] = wr[k];                                     \
+    }
+    load_items<G, bf16_t, BF_CIB>(a, 0, nitem, tree_items, sh, R);
+    APRNET_LOAD_WEIGHTS(0)
+    for (int i = threadIdx.x; i < 2 * G::CH_STRIDE; i += G::NT) patch8[i] = make_uint2(0u, 0u);     // once per window
+    for (int ci0 = 0; ci0 < a.Cin; ci0 += BF_CIB) {
+        __syncthreads();
+        // items -> patch: two 8-byte cells (channel groups) per item, four bfloat16 each
+        store_items_bf16<G>(R, nitem, patch8);
+        APRNET_STORE_WEIGHTS()
+        __syncthreads();
+        if (ci0 + BF_CIB < a.Cin) {
+            load_items<G, bf16_t, BF_CIB>(a, ci0 + BF_CIB, nitem, tree_items, sh, R);
+            APRNET_LOAD_WEIGHTS(ci0 / BF_CIB + 1)
+        }
+#pragma unroll
+        for (int st = 0; st < NSTEP; ++st) {
+            constexpr int dummy = 0; (void)dummy;
+            const int offA = tap_offset<G>(2 * st);
+            const int offB = (2 * st + 1 < G::K) ? tap_offset<G>(2 * st + 1) : offA;     // the weights of a missing tap are zero
+            const int off = second_tap ? offB : offA;
+            bf16x4 av[COH];
+#pragma unroll
+            for (int h = 0; h < COH; ++h) av[h] = __builtin_bit_cast(bf16x4, Wl8[(st * COH + h) * 64 + lane]);
+#pragma unroll
+            for (int j = 0; j < NB; ++j) {
+                const bf16x4 bv = __builtin_bit_cast(bf16x4, patch8[bbase[j] + off]);
+#pragma unroll
+                for (int h = 0; h < COH; ++h) acc[j][h] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(av[h], bv, acc[j][h], 0, 0, 0);
+            }
+        }
+    }
+#undef APRNET_LOAD_WEIGHTS
+#undef APRNET_STORE_WEIGHTS
+#pragma unroll
+    for (int j = 0; j < NB; ++j) {
+        const int col = ((first + G::NWAVE * j) << 4) + (lane & 15);
+        if (col >= nc) continue;
+        const int64_t o = sh.col_idx[col];
+#pragma unroll
+        for (int h = 0; h < COH; ++h)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int cl = h * 16 + 4 * (lane >> 4) + r;
+                if (co0 + cl < a.Cout) a.y[(int64_t)(co0 + cl) * a.ldy + o] = float_to_bf16(acc[j][h][r] + bias_l[cl]);
+            }
+    }
+}
+
+template <class G, int COH>
+__global__ void __launch_bounds__(G::NT) __attribute__((amdgpu_waves_per_eu(4, 4)))      // two workgroups per CU
+conv_mfma_bf16_kernel(const ConvArgs<bf16_t> a) {
+    constexpr int NBW = 4, NSTEP = bf16_steps<G>();
+    static_assert((G::MAXCOL + 15) / 16 <= G::NWAVE * NBW, "a window must fit the accumulators of the block");
+    static_assert(G::CH_STRIDE % 32 == 16, "the two channel groups of a half wave must fall on different bank pairs");
+    __shared__ uint2 patch8[2 * G::CH_STRIDE];
+    __shared__ __attribute__((aligned(16))) uint2 Wl8[NSTEP * COH * 64];
+    __shared__ ConvShared<G> sh;
+    __shared__ float bias_l[16 * COH];
+
+    const ConvTile tile = a.tiles[blockIdx.x];
+    const int L = tile.level, z0 = tile.z0, x0 = tile.x0;
+    const int co0 = blockIdx.y * 16 * COH;
+    const int yn = a.apr.y_num[L];
+    const int s_idx = min(a.S_exp - 1, a.Lc - L);
+    const bool out_tree = (L == a.Lc) && (L < a.apr.level_max);
+    const int nq = (a.Cin + BF_CIB - 1) / BF_CIB;
+    // a.w carries the packed bfloat16 image
+    const uint4* __restrict__ wl = reinterpret_cast<const uint4*>(a.w) +
+                                   ((int64_t)s_idx * gridDim.y + blockIdx.y) * nq * (NSTEP * COH * 32);
+    const int wave = threadIdx.x >> 6;
+
+    if (threadIdx.x < 16 * COH)
+        bias_l[threadIdx.x] = (a.bias && co0 + (int)threadIdx.x < a.Cout) ? a.bias[co0 + threadIdx.x] : 0.f;
+    open_segments<G, bf16_t>(a, L, z0, x0, sh);
+    __syncthreads();
+
+    int win = 0;
+    for (int y0 = 0; y0 < yn; y0 += G::TY, ++win) {
+        scan_window<G, bf16_t>(a, L, y0, out_tree, sh);
+        __syncthreads();
+        const int nc = __builtin_amdgcn_readfirstlane(sh.ncol), nitem = __builtin_amdgcn_readfirstlane(sh.nitem);
+        const bool tree_items = L < a.Lc;
+        if (nc > 0) {
+            const int nblk = (nc + 15) >> 4;
+            const int first = (wave - (int)blockIdx.x - win) & (G::NWAVE - 1);
+            const int nb = first < nblk ? (nblk - first + G::NWAVE - 1) / G::NWAVE : 0;
+            switch (__builtin_amdgcn_readfirstlane(nb)) {
+                case 0: mfma_bf16_window<G, COH, 0>(a, co0, nc, nitem, tree_items, first, wl, sh, patch8, Wl8, bias_l); break;
+                case 1: mfma_bf16_window<G, COH, 1>(a, co0, nc, nitem, tree_items, first, wl, sh, patch8, Wl8, bias_l); break;
+                case 2: mfma_bf16_window<G, COH, 2>(a, co0, nc, nitem, tree_items, first, wl, sh, patch8, Wl8, bias_l); break;
+                case 3: mfma_bf16_window<G, COH, 3>(a, co0, nc, nitem, tree_items, first, wl, sh, patch8, Wl8, bias_l); break;
+                default: mfma_bf16_window<G, COH, 4>(a, co0, nc, nitem, tree_items, first, wl, sh, patch8, Wl8, bias_l); break;
+            }
+        }
+        __syncthreads();
+        close_window<G>(sh);
+        __syncthreads();
+    }
+}
+
 using M333N = ConvGeom<3, 3, 3, 2, 4, 512, 64, 16>;
 using M133N = ConvGeom<1, 3, 3, 1, 8, 512, 64, 16>;
 using M155N = ConvGeom<1, 5, 5, 1, 8, 512, 64, 16>;
@@ -246,7 +440,39 @@ static int launch16_code(int code, const ConvArgs<T>& a, int n_tiles, hipStream_
 
 // Forward.  a.w must point at the packed weights (pack_conv_weights).
 int launch_conv_mfma(int code, const ConvArgs<float>& a, int n_tiles, hipStream_t st) { return launch16_code<float, 0>(code, a, n_tiles, st); }
+// bfloat16 features, fp32 contraction (weights packed by pack_conv_weights)
 int launch_conv_mfma(int code, const ConvArgs<bf16_t>& a, int n_tiles, hipStream_t st) { return launch16_code<bf16_t, 0>(code, a, n_tiles, st); }
+
+// bfloat16 features, bfloat16 contraction (a.w = image of pack_conv_weights_bf16)
+template <class G>
+static int launch_bf16(const ConvArgs<bf16_t>& a, int n_tiles, hipStream_t st) {
+    const int coh = conv_coh(a.Cout);
+    dim3 grid((unsigned)n_tiles, (unsigned)((a.Cout + 16 * coh - 1) / (16 * coh)));
+    if (coh == 1) hipLaunchKernelGGL((conv_mfma_bf16_kernel<G, 1>), grid, dim3(G::NT), 0, st, a);
+    else hipLaunchKernelGGL((conv_mfma_bf16_kernel<G, 2>), grid, dim3(G::NT), 0, st, a);
+    APRNET_LAUNCH_CHECK("conv_mfma_bf16_kernel");
+    return 0;
+}
+int launch_conv_mfma_bf16(int code, const ConvArgs<bf16_t>& a, int n_tiles, hipStream_t st) {
+    switch (code) {
+        case 333: return launch_bf16<M333N>(a, n_tiles, st);
+        case 133: return launch_bf16<M133N>(a, n_tiles, st);
+        case 155: return launch_bf16<M155N>(a, n_tiles, st);
+    }
+    return fail(APRNET_ERR_UNSUPPORTED, "no matrix-core kernel for this stencil");
+}
+size_t conv_packed_bf16_bytes(int code, int S_exp, int Cout, int Cin) {
+    const int coh = conv_coh(Cout), nstep = (conv_taps(code) + 1) / 2;
+    return (size_t)S_exp * ((Cout + 16 * coh - 1) / (16 * coh)) * ((Cin + BF_CIB - 1) / BF_CIB) * nstep * coh * 64 * sizeof(uint2);
+}
+int pack_conv_weights_bf16(int code, const float* w, int S_exp, int Cout, int Cin, void* packed, hipStream_t st) {
+    const size_t n = conv_packed_bf16_bytes(code, S_exp, Cout, Cin) / sizeof(uint2);
+    dim3 grid((unsigned)std::min<size_t>((n + 255) / 256, 2048));
+    hipLaunchKernelGGL(pack_weights_bf16_kernel, grid, dim3(256), 0, st, w, S_exp, Cout, Cin, conv_taps(code), conv_coh(Cout),
+                       (uint2*)packed);
+    APRNET_LAUNCH_CHECK("pack_weights_bf16_kernel");
+    return 0;
+}
 
 // Input gradient: a.x / a.Cin describe the output gradient, a.Cout the input channels, a.w the packed
 // transposed weights, a.tiles the row groups within one row of an output (n_tiles of them).

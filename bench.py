@@ -146,12 +146,12 @@ def other_ops(apr, x, dev):
     ms = _time(lambda: torch.autograd.grad(y5, (x64, conv5.weight), go5, retain_graph=True), iters=2, warmup=1)
     res.append({"op": "conv155_bwd", "ms": ms, "particles_per_s": n0 / ms * 1e3, "note": "1x5x5 64->64 grad_input + grad_weight"})
     del y5, go5, x64, conv5
-    # bfloat16 features (fp32 weights and arithmetic inside the operators)
+    # bfloat16 features (convolutions: bfloat16 matrix instructions with fp32 accumulation)
     xb = x.to(torch.bfloat16)
     with torch.no_grad():
         ms = _time(lambda: conv(xb, [apr], ld0), iters=5, warmup=1)
         res.append({"op": "conv333_fwd_bf16", "ms": ms, "particles_per_s": n0 / ms * 1e3,
-                    "note": f"{C}->{C}, bfloat16 features, fp32 matrix math, whole APRConv.forward"})
+                    "note": f"{C}->{C}, bfloat16 features and matrix math (fp32 accumulate), whole APRConv.forward"})
         ms = _time(lambda: _ops.maxpool_forward([apr], xb, ld0, 0.0))
         line("maxpool_fwd_bf16", ms, 2 * C * n0 + (2 + 8) * C * n1, "bfloat16 values, int64 argmax")
         xinb = xin.to(torch.bfloat16)

@@ -77,9 +77,10 @@ int aprnet_plan_children(const aprnet_plan* plan, int32_t* out_host);
  * the call's stream; aprnet_profile_last_ms() waits for the last bracket and returns its duration in
  * milliseconds (-1 if none).  Process-wide, not thread-safe; meant for benchmarks. */
 int aprnet_profile_enable(int on);
-/* No counterpart in the reference.  Selects the forward convolution kernels: 0 = matrix-core (MFMA) kernels
- * where one exists for the stencil and element type, VALU kernels otherwise (default); 1 = VALU kernels only.
- * Both are HIP kernels; the switch exists so that tests can cover both. */
+/* No counterpart in the reference.  Selects the convolution kernels: 0 = matrix-core (MFMA) kernels where one
+ * exists for the stencil and element type, VALU kernels otherwise (default); 1 = VALU kernels only.
+ * Independently, for bfloat16 features: 2 = bfloat16 matrix instructions (default), 3 = fp32 matrix
+ * instructions.  All are HIP kernels; the switch exists so that tests can cover them. */
 int aprnet_set_conv_path(int path);
 float aprnet_profile_last_ms(void);
 
@@ -154,13 +155,15 @@ APRNET_DECL(float, f32)
 APRNET_DECL(double, f64)
 
 /* bfloat16 features (uint16_t bit patterns; no counterpart in the reference, which has no 16-bit path).
- * Storage only: values are widened to fp32 on load, all arithmetic is fp32, results are rounded to nearest
- * even on store.  Weights and bias stay fp32.  Forward operators of the APR-UNet, plus the backward passes
+ * Values are widened to fp32 on load, accumulated in fp32 and rounded to nearest even on store.  Weights
+ * and bias are passed in fp32; the stencil convolution (3x3x3, 1x3x3, 1x5x5) rounds the weights to bfloat16
+ * and multiplies on the bfloat16 matrix cores (aprnet_set_conv_path(3) keeps the weights and the products
+ * in fp32).  Forward operators of the APR-UNet, plus the backward passes
  * of pool / upsample / tree fill; the convolution backward is not available in bfloat16.  Argument meaning
  * as for the _f32 entry points. */
 int aprnet_conv_fwd_bf16(const aprnet_plan*, int level_delta, int kz, int kx, int ky, const uint16_t* x, int64_t ldx, int Cin,
                          const float* w, int S_exp, int Cout, const float* bias, uint16_t* y, int64_t ldy,
-                         uint16_t* tree_ws, int64_t ld_tree, void* stream);          /* 3x3x3 only */
+                         uint16_t* tree_ws, int64_t ld_tree, void* stream);          /* not 5x5x5 */
 int aprnet_conv111_fwd_bf16(const aprnet_plan*, int level_delta, const uint16_t* x, int64_t ldx, int Cin, const float* w,
                             int S, int Cout, const float* bias, uint16_t* y, int64_t ldy, void* stream);
 int aprnet_fill_tree_mean_bf16(const aprnet_plan*, int level_delta, const uint16_t* x, int64_t ldx, int C, uint16_t* tree,

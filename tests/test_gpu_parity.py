@@ -344,16 +344,33 @@ def close_bf16(got, ref):
     assert err <= 1e-2 * scale, f"max abs err {err:.3e} vs scale {scale:.3e}"
 
 
+@pytest.mark.parametrize("math", [2, 3], ids=["bf16math", "fp32math"])
 @pytest.mark.parametrize("cin,cout", [(1, 16), (32, 32), (33, 17)])
 @pytest.mark.parametrize("bt", [[("3d_a", 0)], [("3d_b", 1), ("3d_c", 2)], [("3d_s", 0), ("3d_t", 1)]],
                          ids=lambda b: "+".join(f"{n}@{d}" for n, d in b))
-def test_conv333_forward_bf16(bt, cin, cout):
+def test_conv333_forward_bf16(bt, cin, cout, math):
+    """bfloat16 features against the fp32 oracle on the same (bfloat16-representable) inputs and fp32 weights,
+    with the products on the bfloat16 matrix cores (weights rounded to bfloat16) and on the fp32 ones."""
     x, aprs, ld, w_exp = _conv_case(bt, (3, 3, 3), 2, cin, cout, torch.float32)
     xb = x.to(torch.bfloat16)
     g = torch.Generator().manual_seed(11)
     bias = torch.randn(cout, generator=g)
     ref = oracle.conv_forward(aprs, xb.float(), w_exp, ld) + bias.view(1, -1, 1)
-    got = _ops.conv_forward(aprs, xb.to(DEV), w_exp.permute(1, 2, 0, 3, 4, 5).contiguous().to(DEV), ld, bias.to(DEV))
+    lib = _native.hip()
+    assert lib.aprnet_set_conv_path(math) == 0
+    try:
+        got = _ops.conv_forward(aprs, xb.to(DEV), w_exp.permute(1, 2, 0, 3, 4, 5).contiguous().to(DEV), ld, bias.to(DEV))
+    finally:
+        lib.aprnet_set_conv_path(2)
+    close_bf16(got, ref)
+
+
+@pytest.mark.parametrize("ksize", [(1, 3, 3), (1, 5, 5)], ids=KID)
+def test_conv_flat_forward_bf16(ksize):
+    x, aprs, ld, w_exp = _conv_case([("2d_a", 0), ("2d_b", 1)], ksize, 2, 20, 33, torch.float32)
+    xb = x.to(torch.bfloat16)
+    ref = oracle.conv_forward(aprs, xb.float(), w_exp, ld)
+    got = _ops.conv_forward(aprs, xb.to(DEV), w_exp.permute(1, 2, 0, 3, 4, 5).contiguous().to(DEV), ld)
     close_bf16(got, ref)
 
 
