@@ -75,6 +75,15 @@ struct TileList {
     int level_count[MAX_LEVELS + 1] = {};   // [level_begin[l], level_begin[l] + level_count[l])
 };
 
+// Precomputed window lists of the forward convolution (lists.hip), device arrays owned by the plan.
+struct WinLists {
+    int* d_tile_win = nullptr;                  // [n_tiles + 1]
+    int4* d_win = nullptr;                      // [n_win] {first item, items, first column, columns}
+    int* d_item_idx = nullptr; unsigned short* d_item_pos = nullptr;
+    int* d_col_idx = nullptr; unsigned short* d_col_pos = nullptr;
+    int n_win = 0; int64_t n_items = 0, n_cols = 0;
+};
+
 }  // namespace aprnet
 
 struct aprnet_plan {
@@ -86,6 +95,7 @@ struct aprnet_plan {
     int64_t n_tree = 0, n_apr = 0;
     std::map<std::tuple<int, int, int, int>, aprnet::TileList> tiles;   // (level_delta, TZ, TX, halo) -> row groups
     void* d_scratch = nullptr; size_t scratch_bytes = 0;          // re-laid-out weights of the call in flight
+    std::map<std::pair<int, int>, aprnet::WinLists> lists;        // (level_delta, stencil code) -> window lists
 
     int lc(int level_delta) const { return apr.level_max - level_delta; }
     int64_t number_parts(int level_delta) const {
@@ -105,6 +115,8 @@ int fail(int code, const std::string& msg);
 // non-empty row groups for the convolution at `level_delta` (built on first use, cached in the plan)
 // `halo` > 0 also lists the row groups that lie within that many rows of a non-empty one
 int get_tiles(aprnet_plan* plan, int level_delta, int TZ, int TX, TileList* out, int halo = 0);
+int get_lists(aprnet_plan* plan, int level_delta, int code, const TileList& tl, WinLists* out, hipStream_t st);
+void free_lists(WinLists& wl);
 // makes plan->d_scratch at least `bytes` large (contents are lost when it grows)
 int plan_scratch(aprnet_plan* plan, size_t bytes, hipStream_t st);
 

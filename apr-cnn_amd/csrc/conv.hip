@@ -136,21 +136,32 @@ size_t conv_packed_bf16_bytes(int code, int S_exp, int Cout, int Cin);
 int pack_conv_weights_bf16(int code, const float* w, int S_exp, int Cout, int Cin, void* packed, hipStream_t st);
 static int g_bf16_math = 1;      // bfloat16 features: 1 = bfloat16 matrix instructions, 0 = fp32 matrix instructions
 int fill_tree_for_conv(const aprnet_plan* p, int d, const bf16_t* x, int64_t ldx, int C, bf16_t* tree, int64_t ldt, hipStream_t st);
-size_t conv_packed_floats(int code, int S_exp, int Cm, int Ck);
+size_t conv_packed_floats(int code, int S_exp, int Cm, int Ck, bool transposed);
 int pack_conv_weights(int code, const float* w, int S_exp, int Cm, int Ck, bool transposed, float* packed, hipStream_t st);
 
 static int g_conv_path = 0;      // 0: matrix cores where available, 1: VALU kernels only
 int conv_path() { return g_conv_path; }
 
-template <typename T> static int try_mfma(aprnet_plan*, const ConvArgs<T>&, int, int, hipStream_t, bool*) { return 0; }
-template <> int try_mfma<float>(aprnet_plan* p, const ConvArgs<float>& a, int code, int n_tiles, hipStream_t st, bool* done) {
+template <typename T>
+static int set_lists(aprnet_plan* p, int d, int code, const TileList& tl, ConvArgs<T>& a, hipStream_t st) {
+    WinLists wl;
+    if (int rc = get_lists(p, d, code, tl, &wl, st)) return rc;
+    a.tile_win = wl.d_tile_win; a.win = wl.d_win;
+    a.l_item_idx = wl.d_item_idx; a.l_item_pos = wl.d_item_pos; a.l_col_idx = wl.d_col_idx; a.l_col_pos = wl.d_col_pos;
+    return 0;
+}
+
+template <typename T> static int try_mfma(aprnet_plan*, const ConvArgs<T>&, int, int, const TileList&, int, hipStream_t, bool*) { return 0; }
+template <> int try_mfma<float>(aprnet_plan* p, const ConvArgs<float>& a, int code, int d, const TileList& tl, int n_tiles,
+                                hipStream_t st, bool* done) {
     if (g_conv_path == 1 || !conv_mfma_supported(code)) return 0;
     *done = true;
     // plan-owned scratch for the re-laid-out weights, grown on demand
-    if (int rc = plan_scratch(p, conv_packed_floats(code, a.S_exp, a.Cout, a.Cin) * sizeof(float), st)) return rc;
+    if (int rc = plan_scratch(p, conv_packed_floats(code, a.S_exp, a.Cout, a.Cin, false) * sizeof(float), st)) return rc;
     if (int rc = pack_conv_weights(code, a.w, a.S_exp, a.Cout, a.Cin, false, (float*)p->d_scratch, st)) return rc;
     ConvArgs<float> b = a;
     b.w = (const float*)p->d_scratch;
+    if (int rc = set_lists(p, d, code, tl, b, st)) return rc;
     TimedLaunch timed(st);
     return launch_conv_mfma(code, b, n_tiles, st);
 }
@@ -181,7 +192,7 @@ int conv_fwd(const aprnet_plan* cp, int d, int kz, int kx, int ky, const T* x, i
     a.tree_data = tree_ws; a.ldt = ldt; a.Lc = p->lc(d); a.tree_off = p->tree_offset(a.Lc);
     a.x_count = p->number_parts(d); a.t_count = p->tree_parts(d);
     bool done = false;
-    if (int rc = try_mfma<T>(p, a, code, tl.n, st, &done)) return rc;
+    if (int rc = try_mfma<T>(p, a, code, d, tl, tl.n, st, &done)) return rc;
     if (done) return 0;
     // few output channels per thread keep the wave-uniform weights within the scalar register file;
     // wider layers run more blocks along grid.y (each re-stages its patch)
@@ -214,7 +225,7 @@ int conv_fwd_bf16(const aprnet_plan* cp, int d, int kz, int kx, int ky, const bf
         if (int rc = plan_scratch(p, conv_packed_bf16_bytes(code, S_exp, Cout, Cin), st)) return rc;
         if (int rc = pack_conv_weights_bf16(code, w, S_exp, Cout, Cin, p->d_scratch, st)) return rc;
     } else {
-        if (int rc = plan_scratch(p, conv_packed_floats(code, S_exp, Cout, Cin) * sizeof(float), st)) return rc;
+        if (int rc = plan_scratch(p, conv_packed_floats(code, S_exp, Cout, Cin, false) * sizeof(float), st)) return rc;
         if (int rc = pack_conv_weights(code, w, S_exp, Cout, Cin, false, (float*)p->d_scratch, st)) return rc;
     }
     ConvArgs<bf16_t> a{};
@@ -222,6 +233,7 @@ int conv_fwd_bf16(const aprnet_plan* cp, int d, int kz, int kx, int ky, const bf
     a.x = x; a.ldx = ldx; a.Cin = Cin; a.w = (const float*)p->d_scratch; a.S_exp = S_exp; a.Cout = Cout; a.bias = bias;
     a.y = y; a.ldy = ldy; a.tree_data = tree_ws; a.ldt = ldt; a.Lc = p->lc(d); a.tree_off = p->tree_offset(a.Lc);
     a.x_count = p->number_parts(d); a.t_count = p->tree_parts(d);
+    if (int rc = set_lists(p, d, code, tl, a, st)) return rc;
     TimedLaunch timed(st);
     return g_bf16_math ? launch_conv_mfma_bf16(code, a, tl.n, st) : launch_conv_mfma(code, a, tl.n, st);
 }

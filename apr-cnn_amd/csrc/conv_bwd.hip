@@ -229,7 +229,7 @@ static int launch_bwd(ConvArgs<T>& a, hipStream_t st) {
 bool conv_mfma_supported(int code);
 int launch_conv_dx_mfma(int code, const ConvArgs<float>& a, int n_tiles, hipStream_t st);
 int launch_conv_dw_mfma(int code, const ConvArgs<float>& a, const TileList& tl, int level_min, hipStream_t st);
-size_t conv_packed_floats(int code, int S_exp, int Cm, int Ck);
+size_t conv_packed_floats(int code, int S_exp, int Cm, int Ck, bool transposed);
 int pack_conv_weights(int code, const float* w, int S_exp, int Cm, int Ck, bool transposed, float* packed, hipStream_t st);
 int conv_path();
 
@@ -241,7 +241,7 @@ template <> int try_mfma_bwd<float>(aprnet_plan* p, const ConvArgs<float>& a, co
     // every row group within one row of an output takes part
     TileList near;
     if (int rc = get_tiles(p, d, code == 333 ? 2 : 1, code == 333 ? 4 : 8, &near, 1)) return rc;
-    if (int rc = plan_scratch(p, conv_packed_floats(code, a.S_exp, a.Cin, a.Cout) * sizeof(float), st)) return rc;
+    if (int rc = plan_scratch(p, conv_packed_floats(code, a.S_exp, a.Cin, a.Cout, true) * sizeof(float), st)) return rc;
     if (int rc = pack_conv_weights(code, a.w, a.S_exp, a.Cin, a.Cout, true, (float*)p->d_scratch, st)) return rc;
     ConvArgs<float> b = a;
     b.tiles = near.d_tiles; b.n_tiles = near.n;

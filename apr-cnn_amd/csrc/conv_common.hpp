@@ -34,6 +34,17 @@ struct ConvArgs {
     int64_t x_count, t_count;                  // valid elements per channel plane of x / tree_data
     // backward only
     const T* gy; T* gx; int64_t ldgx; T* gtree; int64_t ldgt; T* gw; int n_tiles;
+    // window lists built once per APR and kept in the plan (kernels that do not scan)
+    const int* tile_win;                       // [n_tiles + 1] first stored window of every tile
+    const int4* win;                           // per stored window: {first item, items, first column, columns}
+    const int* l_item_idx; const unsigned short* l_item_pos;
+    const int* l_col_idx; const unsigned short* l_col_pos;
+};
+
+// The lists of one window in global memory; same member names as ConvShared, so the staging code takes either.
+struct WindowLists {
+    const int* item_idx; const unsigned short* item_pos;
+    const int* col_idx; const unsigned short* col_pos;
 };
 
 template <int KZ_, int KX_, int KY_, int TZ_, int TX_, int NT_, int RS_ = 64, int PAD_ = 32>
@@ -361,16 +372,32 @@ struct ItemRegs {
     static constexpr int ROUNDS = (G::MAXITEM + G::NT - 1) / G::NT;  // items per thread
     static constexpr int IPT = NR;
     typename RawLoad<T>::raw v[IPT][CIB];
-    unsigned short pos[IPT];
+    unsigned off[IPT];                 // byte offset of the item inside a channel plane (BUF_OOB: no item)
+    unsigned short pos[IPT];           // patch cell and flags (0xffff: no item)
 };
 
 // Issues the loads of a chunk (no LDS writes: they may run ahead of the consumer of the patch).
 // Thread t owns items t, t + NT, ...; a round k that lies beyond the item count is skipped by a
 // wave-uniform branch (most windows hold fewer items than the block has threads).
+// Which items this thread stages, and where they go: read once per window from the lists (LDS or global).
+template <class G, typename T, int CIB, int NR, class Lists>
+__device__ __forceinline__ void fetch_slots(const Lists& sh, int nitem, ItemRegs<G, T, CIB, NR>& R, int round0 = 0) {
+#pragma unroll
+    for (int k = 0; k < NR; ++k) {
+        R.pos[k] = 0xffffu; R.off[k] = BUF_OOB;
+        if ((round0 + k) * G::NT >= nitem) continue;    // wave-uniform
+        const int it = threadIdx.x + (round0 + k) * G::NT;
+        if (it < nitem) {
+            R.pos[k] = sh.item_pos[it];
+            R.off[k] = (unsigned)sh.item_idx[it] * (unsigned)sizeof(T);
+        }
+    }
+}
+
+// Issues the value loads of one chunk for the fetched slots.
 template <class G, typename T, int CIB, int NR>
-__device__ __forceinline__ void load_items(const ConvArgs<T>& a, int ci0, int nitem, bool tree_items,
-                                           const ConvShared<G>& sh, ItemRegs<G, T, CIB, NR>& R, int round0 = 0) {
-    constexpr int IPT = NR;
+__device__ __forceinline__ void load_values(const ConvArgs<T>& a, int ci0, int nitem, bool tree_items,
+                                            ItemRegs<G, T, CIB, NR>& R, int round0 = 0) {
     __amdgpu_buffer_rsrc_t rx[CIB], rt[CIB];
 #pragma unroll
     for (int c = 0; c < CIB; ++c) {
@@ -378,17 +405,10 @@ __device__ __forceinline__ void load_items(const ConvArgs<T>& a, int ci0, int ni
         rt[c] = plane_rsrc<T>(a.tree_data, a.ldt, ci0 + c, tree_items ? a.Cin : 0, a.t_count);
     }
 #pragma unroll
-    for (int k = 0; k < IPT; ++k) {
+    for (int k = 0; k < NR; ++k) {
         if ((round0 + k) * G::NT >= nitem) break;       // wave-uniform
-        const int it = threadIdx.x + (round0 + k) * G::NT;
-        unsigned offx = BUF_OOB, offt = BUF_OOB;
-        R.pos[k] = 0xffffu;
-        if (it < nitem) {
-            const unsigned pos = sh.item_pos[it];
-            const unsigned off = (unsigned)sh.item_idx[it] * (unsigned)sizeof(T);
-            R.pos[k] = (unsigned short)pos;
-            if (pos & ITEM_TREE) offt = off; else offx = off;
-        }
+        const bool from_tree = (R.pos[k] & ITEM_TREE) != 0 && R.pos[k] != 0xffffu;
+        const unsigned offx = from_tree ? BUF_OOB : R.off[k], offt = from_tree ? R.off[k] : BUF_OOB;
 #pragma unroll
         for (int c = 0; c < CIB; ++c) R.v[k][c] = RawLoad<T>::ld(rx[c], offx);
         if (tree_items) {      // tile-uniform: only levels below the current maximum read the mean-filled tree
@@ -396,6 +416,16 @@ __device__ __forceinline__ void load_items(const ConvArgs<T>& a, int ci0, int ni
             for (int c = 0; c < CIB; ++c) R.v[k][c] |= RawLoad<T>::ld(rt[c], offt);     // one of the two returned zero
         }
     }
+}
+
+// Issues the loads of a chunk (no LDS writes: they may run ahead of the consumer of the patch).
+// Thread t owns items t, t + NT, ...; a round k that lies beyond the item count is skipped by a
+// wave-uniform branch (most windows hold fewer items than the block has threads).
+template <class G, typename T, int CIB, int NR, class Lists>
+__device__ __forceinline__ void load_items(const ConvArgs<T>& a, int ci0, int nitem, bool tree_items,
+                                           const Lists& sh, ItemRegs<G, T, CIB, NR>& R, int round0 = 0) {
+    fetch_slots<G, T, CIB, NR>(sh, nitem, R, round0);
+    load_values<G, T, CIB, NR>(a, ci0, nitem, tree_items, R, round0);
 }
 
 template <class G, typename T, int CIB, int NR>

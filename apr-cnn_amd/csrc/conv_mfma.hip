@@ -35,6 +35,12 @@ __device__ __forceinline__ constexpr int tap_offset(int t) {
 // the B operand; a wave owns up to four blocks of 16 columns.  Blocks of 16 columns instead of 32 waste
 // less of the last block of a window and spread more evenly over the four SIMDs.
 typedef float floatx4 __attribute__((ext_vector_type(4)));
+// Input channels per staged chunk (a multiple of the 4 of one instruction) and waves per SIMD the kernels are
+// compiled for.  Three workgroups per CU (six waves per SIMD, 80 registers) beat two with chunks of 8: the
+// third group hides more of the latency between the matrix phases than the few spilled registers cost.
+// Forward takes its window lists from the plan; the input gradient scans and keeps its lists in LDS.
+constexpr int FWD_CIB = 4, FWD_WAVES = 6;
+constexpr int DX_CIB = 4, DX_WAVES = 6;
 
 // packed16[s][cb][q][t][h][c][16 co], cb = block of 16 * COH output channels, h = its 16-channel part:
 // the chunk image is linear in (t, h, lane)
@@ -66,12 +72,12 @@ __global__ void pack_weights16_kernel(const float* __restrict__ w, int S_exp, in
 
 // MODE 0: forward, results stored (plus bias).  MODE 1: input gradient, results added atomically to the
 // place each column names (feature gradient, or tree gradient with COL_TREE).
-template <typename T, class G, int COH, int NB, int MODE>
+template <typename T, class G, int CIB, int COH, int NB, int MODE, class Lists>
 __device__ __forceinline__ void mfma16_window(const ConvArgs<T>& a, int co0, int nc, int nitem, bool tree_items, int first,
-                                              const float4* __restrict__ wl, const ConvShared<G>& sh,
+                                              const float4* __restrict__ wl, const Lists& sh,
                                               float* __restrict__ patch, float* __restrict__ Wl,
                                               const float* __restrict__ bias_l) {
-    constexpr int CIB = 4;
+    constexpr int NSUB = CIB / 4;
     constexpr int KC = CIB * G::K;             // k rows per chunk
     const int lane = lane_id();
     constexpr int NBA = NB > 0 ? NB : 1;
@@ -114,19 +120,22 @@ __device__ __forceinline__ void mfma16_window(const ConvArgs<T>& a, int co0, int
         APRNET_STORE_WEIGHTS()
         __syncthreads();
         if (ci0 + CIB < a.Cin) {
-            load_items<G, T, CIB>(a, ci0 + CIB, nitem, tree_items, sh, R);
+            load_values<G, T, CIB>(a, ci0 + CIB, nitem, tree_items, R);
             APRNET_LOAD_WEIGHTS(ci0 / CIB + 1)
         }
 #pragma unroll
         for (int t = 0; t < G::K; ++t) {
-            float av[COH];
 #pragma unroll
-            for (int h = 0; h < COH; ++h) av[h] = ap[(t * COH + h) * 64];
+            for (int sb = 0; sb < NSUB; ++sb) {
+                float av[COH];
 #pragma unroll
-            for (int j = 0; j < NB; ++j) {
-                const float bv = patch[bbase[j] + tap_offset<G>(t)];
+                for (int h = 0; h < COH; ++h) av[h] = ap[((t * COH + h) * NSUB + sb) * 64];
 #pragma unroll
-                for (int h = 0; h < COH; ++h) acc[j][h] = __builtin_amdgcn_mfma_f32_16x16x4f32(av[h], bv, acc[j][h], 0, 0, 0);
+                for (int j = 0; j < NB; ++j) {
+                    const float bv = patch[bbase[j] + 4 * sb * G::CH_STRIDE + tap_offset<G>(t)];
+#pragma unroll
+                    for (int h = 0; h < COH; ++h) acc[j][h] = __builtin_amdgcn_mfma_f32_16x16x4f32(av[h], bv, acc[j][h], 0, 0, 0);
+                }
             }
         }
     }
@@ -161,18 +170,18 @@ __device__ __forceinline__ void mfma16_window(const ConvArgs<T>& a, int co0, int
 }
 
 // COH = 16-channel parts of the output block: 1 for layers of at most 16 output channels, 2 otherwise
-// Three workgroups per CU (six waves per SIMD, 80 registers): the third group hides more of the latency of
-// the scan and staging phases than the few spilled registers cost.
-template <typename T, class G, int COH, int MODE>
-__global__ void __launch_bounds__(G::NT) __attribute__((amdgpu_waves_per_eu(6, 6)))
+// LISTS: the windows of the tile come as precomputed lists from the plan (forward); otherwise the block scans
+// the access arrays itself (input gradient).
+template <typename T, class G, int COH, int MODE, bool LISTS>
+__global__ void __launch_bounds__(G::NT)
+__attribute__((amdgpu_waves_per_eu(LISTS ? FWD_WAVES : DX_WAVES, LISTS ? FWD_WAVES : DX_WAVES)))
 conv_mfma16_kernel(const ConvArgs<T> a) {
-    constexpr int CIB = 4, NBW = 4;
+    constexpr int CIB = LISTS ? FWD_CIB : DX_CIB, NBW = 4;
     static_assert((G::NWAVE & (G::NWAVE - 1)) == 0, "block rotation assumes a power-of-two wave count");
     static_assert((G::MAXCOL + 15) / 16 <= G::NWAVE * NBW, "a window must fit the accumulators of the block");
     static_assert(G::CH_STRIDE % 64 == 16, "four lane groups read four channels: a quarter of the banks each");
     __shared__ float patch[CIB * G::CH_STRIDE];
     __shared__ __attribute__((aligned(16))) float Wl[CIB * G::K * 16 * COH];
-    __shared__ ConvShared<G> sh;
     __shared__ float bias_l[16 * COH];
 
     const ConvTile tile = a.tiles[blockIdx.x];
@@ -185,35 +194,54 @@ conv_mfma16_kernel(const ConvArgs<T> a) {
     const float4* __restrict__ wl = reinterpret_cast<const float4*>(a.w) +
                                     ((int64_t)s_idx * gridDim.y + blockIdx.y) * nq * (CIB * G::K * 4 * COH);
     const int wave = threadIdx.x >> 6;
+    const bool tree_items = MODE == 0 && L < a.Lc;       // the output gradient has no tree part
 
     if (MODE == 0 && threadIdx.x < 16 * COH)
         bias_l[threadIdx.x] = (a.bias && co0 + (int)threadIdx.x < a.Cout) ? a.bias[co0 + threadIdx.x] : 0.f;
-    open_segments<G, T>(a, L, z0, x0, sh);
-    __syncthreads();
 
-    int win = 0;
-    for (int y0 = 0; y0 < yn; y0 += G::TY, ++win) {
-        if constexpr (MODE == 0) scan_window<G, T>(a, L, y0, out_tree, sh);
-        else scan_window_dx<G, T>(a, L, y0, out_tree, sh);
-        __syncthreads();
-        const int nc = __builtin_amdgcn_readfirstlane(sh.ncol), nitem = __builtin_amdgcn_readfirstlane(sh.nitem);
-        const bool tree_items = MODE == 0 && L < a.Lc;       // the output gradient has no tree part
-        if (nc > 0 && nitem > 0) {
-            const int nblk = (nc + 15) >> 4;
-            const int first = (wave - (int)blockIdx.x - win) & (G::NWAVE - 1);
-            const int nb = first < nblk ? (nblk - first + G::NWAVE - 1) / G::NWAVE : 0;
-            switch (__builtin_amdgcn_readfirstlane(nb)) {
-                case 0: mfma16_window<T, G, COH, 0, MODE>(a, co0, nc, nitem, tree_items, first, wl, sh, patch, Wl, bias_l); break;
-                case 1: mfma16_window<T, G, COH, 1, MODE>(a, co0, nc, nitem, tree_items, first, wl, sh, patch, Wl, bias_l); break;
-                case 2: mfma16_window<T, G, COH, 2, MODE>(a, co0, nc, nitem, tree_items, first, wl, sh, patch, Wl, bias_l); break;
-                case 3: mfma16_window<T, G, COH, 3, MODE>(a, co0, nc, nitem, tree_items, first, wl, sh, patch, Wl, bias_l); break;
-                default: mfma16_window<T, G, COH, 4, MODE>(a, co0, nc, nitem, tree_items, first, wl, sh, patch, Wl, bias_l); break;
-            }
-        }
-        __syncthreads();
-        close_window<G>(sh);
-        __syncthreads();
+#define APRNET_WINDOW(LISTS_OBJ)                                                                                          \
+    {                                                                                                                     \
+        const int nblk = (nc + 15) >> 4;                                                                                  \
+        /* rotation: spread the waves that own one block more over the SIMDs */                                           \
+        const int first = (wave - (int)blockIdx.x - win) & (G::NWAVE - 1);                                                \
+        const int nb = first < nblk ? (nblk - first + G::NWAVE - 1) / G::NWAVE : 0;                                       \
+        switch (__builtin_amdgcn_readfirstlane(nb)) {                                                                     \
+            case 0: mfma16_window<T, G, CIB, COH, 0, MODE>(a, co0, nc, nitem, tree_items, first, wl, LISTS_OBJ, patch, Wl, bias_l); break; \
+            case 1: mfma16_window<T, G, CIB, COH, 1, MODE>(a, co0, nc, nitem, tree_items, first, wl, LISTS_OBJ, patch, Wl, bias_l); break; \
+            case 2: mfma16_window<T, G, CIB, COH, 2, MODE>(a, co0, nc, nitem, tree_items, first, wl, LISTS_OBJ, patch, Wl, bias_l); break; \
+            case 3: mfma16_window<T, G, CIB, COH, 3, MODE>(a, co0, nc, nitem, tree_items, first, wl, LISTS_OBJ, patch, Wl, bias_l); break; \
+            default: mfma16_window<T, G, CIB, COH, 4, MODE>(a, co0, nc, nitem, tree_items, first, wl, LISTS_OBJ, patch, Wl, bias_l); break; \
+        }                                                                                                                 \
     }
+
+    if constexpr (LISTS) {
+        (void)z0; (void)x0; (void)yn; (void)out_tree;
+        const int wb = a.tile_win[blockIdx.x], we = a.tile_win[blockIdx.x + 1];
+        for (int w = wb; w < we; ++w) {
+            const int win = w - wb;
+            const int4 hd = a.win[w];
+            const int nitem = __builtin_amdgcn_readfirstlane(hd.y), nc = __builtin_amdgcn_readfirstlane(hd.w);
+            const WindowLists gl{a.l_item_idx + hd.x, a.l_item_pos + hd.x, a.l_col_idx + hd.z, a.l_col_pos + hd.z};
+            APRNET_WINDOW(gl)
+            __syncthreads();        // the next window rewrites the patch
+        }
+    } else {
+        __shared__ ConvShared<G> sh;
+        open_segments<G, T>(a, L, z0, x0, sh);
+        __syncthreads();
+        int win = 0;
+        for (int y0 = 0; y0 < yn; y0 += G::TY, ++win) {
+            if constexpr (MODE == 0) scan_window<G, T>(a, L, y0, out_tree, sh);
+            else scan_window_dx<G, T>(a, L, y0, out_tree, sh);
+            __syncthreads();
+            const int nc = __builtin_amdgcn_readfirstlane(sh.ncol), nitem = __builtin_amdgcn_readfirstlane(sh.nitem);
+            if (nc > 0 && nitem > 0) APRNET_WINDOW(sh)
+            __syncthreads();
+            close_window<G>(sh);
+            __syncthreads();
+        }
+    }
+#undef APRNET_WINDOW
 }
 
 // ---------------------------------------------------------------------------------------------------------
@@ -273,9 +301,9 @@ __device__ __forceinline__ void store_items_bf16(const ItemRegs<G, bf16_t, BF_CI
     }
 }
 
-template <class G, int COH, int NB>
+template <class G, int COH, int NB, class Lists>
 __device__ __forceinline__ void mfma_bf16_window(const ConvArgs<bf16_t>& a, int co0, int nc, int nitem, bool tree_items, int first,
-                                                 const uint4* __restrict__ wl, const ConvShared<G>& sh,
+                                                 const uint4* __restrict__ wl, const Lists& sh,
                                                  uint2* __restrict__ patch8, uint2* __restrict__ Wl8,
                                                  const float* __restrict__ bias_l) {
     constexpr int NSTEP = bf16_steps<G>();
@@ -321,7 +349,7 @@ __device__ __forceinline__ void mfma_bf16_window(const ConvArgs<bf16_t>& a, int 
         APRNET_STORE_WEIGHTS()
         __syncthreads();
         if (ci0 + BF_CIB < a.Cin) {
-            load_items<G, bf16_t, BF_CIB>(a, ci0 + BF_CIB, nitem, tree_items, sh, R);
+            load_values<G, bf16_t, BF_CIB>(a, ci0 + BF_CIB, nitem, tree_items, R);
             APRNET_LOAD_WEIGHTS(ci0 / BF_CIB + 1)
         }
 #pragma unroll
@@ -358,6 +386,7 @@ __device__ __forceinline__ void mfma_bf16_window(const ConvArgs<bf16_t>& a, int 
     }
 }
 
+// The windows of the tile come as precomputed lists from the plan.
 template <class G, int COH>
 __global__ void __launch_bounds__(G::NT) __attribute__((amdgpu_waves_per_eu(4, 4)))      // two workgroups per CU
 conv_mfma_bf16_kernel(const ConvArgs<bf16_t> a) {
@@ -366,47 +395,39 @@ conv_mfma_bf16_kernel(const ConvArgs<bf16_t> a) {
     static_assert(G::CH_STRIDE % 32 == 16, "the two channel groups of a half wave must fall on different bank pairs");
     __shared__ uint2 patch8[2 * G::CH_STRIDE];
     __shared__ __attribute__((aligned(16))) uint2 Wl8[NSTEP * COH * 64];
-    __shared__ ConvShared<G> sh;
     __shared__ float bias_l[16 * COH];
 
     const ConvTile tile = a.tiles[blockIdx.x];
-    const int L = tile.level, z0 = tile.z0, x0 = tile.x0;
+    const int L = tile.level;
     const int co0 = blockIdx.y * 16 * COH;
-    const int yn = a.apr.y_num[L];
     const int s_idx = min(a.S_exp - 1, a.Lc - L);
-    const bool out_tree = (L == a.Lc) && (L < a.apr.level_max);
     const int nq = (a.Cin + BF_CIB - 1) / BF_CIB;
     // a.w carries the packed bfloat16 image
     const uint4* __restrict__ wl = reinterpret_cast<const uint4*>(a.w) +
                                    ((int64_t)s_idx * gridDim.y + blockIdx.y) * nq * (NSTEP * COH * 32);
     const int wave = threadIdx.x >> 6;
+    const bool tree_items = L < a.Lc;
 
     if (threadIdx.x < 16 * COH)
         bias_l[threadIdx.x] = (a.bias && co0 + (int)threadIdx.x < a.Cout) ? a.bias[co0 + threadIdx.x] : 0.f;
-    open_segments<G, bf16_t>(a, L, z0, x0, sh);
-    __syncthreads();
 
-    int win = 0;
-    for (int y0 = 0; y0 < yn; y0 += G::TY, ++win) {
-        scan_window<G, bf16_t>(a, L, y0, out_tree, sh);
-        __syncthreads();
-        const int nc = __builtin_amdgcn_readfirstlane(sh.ncol), nitem = __builtin_amdgcn_readfirstlane(sh.nitem);
-        const bool tree_items = L < a.Lc;
-        if (nc > 0) {
-            const int nblk = (nc + 15) >> 4;
-            const int first = (wave - (int)blockIdx.x - win) & (G::NWAVE - 1);
-            const int nb = first < nblk ? (nblk - first + G::NWAVE - 1) / G::NWAVE : 0;
-            switch (__builtin_amdgcn_readfirstlane(nb)) {
-                case 0: mfma_bf16_window<G, COH, 0>(a, co0, nc, nitem, tree_items, first, wl, sh, patch8, Wl8, bias_l); break;
-                case 1: mfma_bf16_window<G, COH, 1>(a, co0, nc, nitem, tree_items, first, wl, sh, patch8, Wl8, bias_l); break;
-                case 2: mfma_bf16_window<G, COH, 2>(a, co0, nc, nitem, tree_items, first, wl, sh, patch8, Wl8, bias_l); break;
-                case 3: mfma_bf16_window<G, COH, 3>(a, co0, nc, nitem, tree_items, first, wl, sh, patch8, Wl8, bias_l); break;
-                default: mfma_bf16_window<G, COH, 4>(a, co0, nc, nitem, tree_items, first, wl, sh, patch8, Wl8, bias_l); break;
-            }
+    const int wb = a.tile_win[blockIdx.x], we = a.tile_win[blockIdx.x + 1];
+    for (int w = wb; w < we; ++w) {
+        const int win = w - wb;
+        const int4 hd = a.win[w];
+        const int nitem = __builtin_amdgcn_readfirstlane(hd.y), nc = __builtin_amdgcn_readfirstlane(hd.w);
+        const WindowLists gl{a.l_item_idx + hd.x, a.l_item_pos + hd.x, a.l_col_idx + hd.z, a.l_col_pos + hd.z};
+        const int nblk = (nc + 15) >> 4;
+        const int first = (wave - (int)blockIdx.x - win) & (G::NWAVE - 1);
+        const int nb = first < nblk ? (nblk - first + G::NWAVE - 1) / G::NWAVE : 0;
+        switch (__builtin_amdgcn_readfirstlane(nb)) {
+            case 0: mfma_bf16_window<G, COH, 0>(a, co0, nc, nitem, tree_items, first, wl, gl, patch8, Wl8, bias_l); break;
+            case 1: mfma_bf16_window<G, COH, 1>(a, co0, nc, nitem, tree_items, first, wl, gl, patch8, Wl8, bias_l); break;
+            case 2: mfma_bf16_window<G, COH, 2>(a, co0, nc, nitem, tree_items, first, wl, gl, patch8, Wl8, bias_l); break;
+            case 3: mfma_bf16_window<G, COH, 3>(a, co0, nc, nitem, tree_items, first, wl, gl, patch8, Wl8, bias_l); break;
+            default: mfma_bf16_window<G, COH, 4>(a, co0, nc, nitem, tree_items, first, wl, gl, patch8, Wl8, bias_l); break;
         }
-        __syncthreads();
-        close_window<G>(sh);
-        __syncthreads();
+        __syncthreads();        // the next window rewrites the patch
     }
 }
 
@@ -423,8 +444,9 @@ template <typename T, class G, int MODE>
 static int launch16(const ConvArgs<T>& a, int n_tiles, hipStream_t st) {
     const int coh = conv_coh(a.Cout);
     dim3 grid((unsigned)n_tiles, (unsigned)((a.Cout + 16 * coh - 1) / (16 * coh)));
-    if (coh == 1) hipLaunchKernelGGL((conv_mfma16_kernel<T, G, 1, MODE>), grid, dim3(G::NT), 0, st, a);
-    else hipLaunchKernelGGL((conv_mfma16_kernel<T, G, 2, MODE>), grid, dim3(G::NT), 0, st, a);
+    constexpr bool LISTS = MODE == 0;      // forward: precomputed window lists; input gradient: scans
+    if (coh == 1) hipLaunchKernelGGL((conv_mfma16_kernel<T, G, 1, MODE, LISTS>), grid, dim3(G::NT), 0, st, a);
+    else hipLaunchKernelGGL((conv_mfma16_kernel<T, G, 2, MODE, LISTS>), grid, dim3(G::NT), 0, st, a);
     APRNET_LAUNCH_CHECK("conv_mfma16_kernel");
     return 0;
 }
@@ -479,15 +501,16 @@ int pack_conv_weights_bf16(int code, const float* w, int S_exp, int Cout, int Ci
 int launch_conv_dx_mfma(int code, const ConvArgs<float>& a, int n_tiles, hipStream_t st) { return launch16_code<float, 1>(code, a, n_tiles, st); }
 
 // Cm: channels on the M axis of the kernel, Ck: contracted channels (forward: Cout, Cin; transposed: Cin, Cout)
-size_t conv_packed_floats(int code, int S_exp, int Cm, int Ck) {
-    const int coh = conv_coh(Cm);
-    return (size_t)S_exp * ((Cm + 16 * coh - 1) / (16 * coh)) * ((Ck + 3) / 4) * 4 * conv_taps(code) * 16 * coh;
+// `transposed`: image for the input gradient (chunks of DX_CIB), otherwise for the forward pass (chunks of FWD_CIB)
+size_t conv_packed_floats(int code, int S_exp, int Cm, int Ck, bool transposed) {
+    const int coh = conv_coh(Cm), cib = transposed ? DX_CIB : FWD_CIB;
+    return (size_t)S_exp * ((Cm + 16 * coh - 1) / (16 * coh)) * ((Ck + cib - 1) / cib) * cib * conv_taps(code) * 16 * coh;
 }
 
 int pack_conv_weights(int code, const float* w, int S_exp, int Cm, int Ck, bool transposed, float* packed, hipStream_t st) {
-    const size_t n = conv_packed_floats(code, S_exp, Cm, Ck);
+    const size_t n = conv_packed_floats(code, S_exp, Cm, Ck, transposed);
     dim3 grid((unsigned)std::min<size_t>((n + 255) / 256, 2048));
-    hipLaunchKernelGGL(pack_weights16_kernel, grid, dim3(256), 0, st, w, S_exp, Cm, Ck, conv_taps(code), 4, conv_coh(Cm),
+    hipLaunchKernelGGL(pack_weights16_kernel, grid, dim3(256), 0, st, w, S_exp, Cm, Ck, conv_taps(code), transposed ? DX_CIB : FWD_CIB, conv_coh(Cm),
                        transposed ? 1 : 0, packed);
     APRNET_LAUNCH_CHECK("pack_weights16_kernel");
     return 0;

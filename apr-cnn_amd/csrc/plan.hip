@@ -200,6 +200,7 @@ void aprnet_plan_destroy(aprnet_plan* p) {
         if (q) (void)hipFree(q);
     for (auto& kv : p->tiles) if (kv.second.d_tiles) (void)hipFree(kv.second.d_tiles);
     if (p->d_scratch) (void)hipFree(p->d_scratch);
+    for (auto& kv : p->lists) free_lists(kv.second);
     delete p;
 }
 
