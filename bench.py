@@ -27,12 +27,13 @@ K_TAPS = 27
 FLOP_PER_PARTICLE = 2 * K_TAPS * CIN * COUT          # 55 296
 BYTES_PER_PARTICLE = 4 * (CIN + COUT) + 2            # features in + out, y_vec
 PEAK_FP32_MATRIX_TFLOPS = 157.3
+PEAK_BF16_MATRIX_TFLOPS = 2500.0
 PEAK_HBM_GBS = 8000.0
 # HBM-side bytes of one launch of the convolution kernel on this workload: FETCH_SIZE + WRITE_SIZE of two
 # profiler passes, scaled by what the same counters read for a device-to-device copy of known size
 # (profiles/conv333_fwd_32x32_f32_blobs512_hbm_traffic.txt).  Counters cannot be read from inside this
 # script; the figure is only reported when the workload is the one it was measured on.
-MEASURED_TRAFFIC_BYTES = {23245996: 28.98e9 + 3.79e9}
+MEASURED_TRAFFIC_BYTES = {23245996: 35.52e9 + 6.27e9}
 
 
 def build_workload(name, crop=None):
@@ -166,6 +167,9 @@ def main():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--features", choices=["f32", "bf16"], default="f32",
+                    help="element type of the feature tensors; bf16 runs the bfloat16 matrix-core kernel "
+                         "(the headline figure is the f32 one)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="run one device-to-device copy of the input features (a kernel of known traffic, "
                          "used to scale the FETCH_SIZE / WRITE_SIZE counters of a profiler run)")
@@ -193,6 +197,8 @@ def main():
 
     torch.manual_seed(0)
     x = torch.randn(1, CIN, n, device=dev)
+    if args.features == "bf16":
+        x = x.to(torch.bfloat16)
     conv = aprnet.cuda.APRConv(CIN, COUT, nstencils=nstencils, kernel_size=(3, 3, 3), bias=True).to(dev)
     ld = torch.zeros(1, dtype=torch.int32)
     lib = _native.hip()
@@ -215,24 +221,26 @@ def main():
             kms.append(float(lib.aprnet_profile_last_ms()))
         lib.aprnet_profile_enable(0)
     kernel_ms = sum(kms) / len(kms)
-    assert torch.isfinite(y).all()
+    assert torch.isfinite(y.float()).all()
+    bf16 = args.features == "bf16"
 
     ms_per_step = dt / args.steps * 1e3
     value = n / (dt / args.steps)
     tflops = FLOP_PER_PARTICLE * n / (kernel_ms * 1e-3) / 1e12
-    gbs = BYTES_PER_PARTICLE * n / (kernel_ms * 1e-3) / 1e9
+    gbs = (BYTES_PER_PARTICLE if args.features == "f32" else BYTES_PER_PARTICLE // 2 + 1) * n / (kernel_ms * 1e-3) / 1e9
     out = {
         "metric": "APRConv 3x3x3 fwd particles/s (Cin=Cout=32)",
         "value": value, "unit": "particles/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "f32", "data": "synthetic",
-        "config": {"workload": "APRConv 3x3x3 32->32 fp32 forward (restrict + tree fill + conv + bias), batch 1, "
+        "dtype": "bf16" if bf16 else "f32", "data": "synthetic",
+        "config": {"workload": f"APRConv 3x3x3 32->32 {'bf16' if bf16 else 'fp32'} forward (restrict + tree fill + conv + bias), batch 1, "
                                "APR of the seeded 512x512x256 volume with 2000 ellipsoidal blobs (configs[1])",
                    "n_particles": n, "nstencils": nstencils, "level_max": apr.level_max(),
                    "apr_build_s": round(t_build, 2), "plan_create_s": round(t_plan, 2)},
-        "roofline": {"bound": "mfma", "achieved": tflops, "peak": PEAK_FP32_MATRIX_TFLOPS, "unit": "TFLOP/s",
-                     "frac": tflops / PEAK_FP32_MATRIX_TFLOPS, "traffic": MEASURED_TRAFFIC_BYTES.get(n),
-                     "kernel": "conv_mfma16_kernel", "kernel_ms": kernel_ms,
+        "roofline": {"bound": "mfma", "achieved": tflops, "peak": PEAK_BF16_MATRIX_TFLOPS if bf16 else PEAK_FP32_MATRIX_TFLOPS,
+                     "unit": "TFLOP/s", "frac": tflops / (PEAK_BF16_MATRIX_TFLOPS if bf16 else PEAK_FP32_MATRIX_TFLOPS),
+                     "traffic": None if bf16 else MEASURED_TRAFFIC_BYTES.get(n),
+                     "kernel": "conv_mfma_bf16_kernel" if bf16 else "conv_mfma16_kernel", "kernel_ms": kernel_ms,
                      "hbm_achieved_GBs": gbs, "hbm_frac": gbs / PEAK_HBM_GBS},
     }
     if args.calibrate_copy:
