@@ -1,0 +1,107 @@
+"""Size-independent properties at the benchmark size (BASELINE configs[1]: APR of the seeded 256x512x512 blob
+volume, 23 M particles), where the CPU oracle is too slow to be the checker: identity stencils, linearity,
+adjointness of forward and backward, gather consistency of the pooling argmax, pool/upsample round trips.
+A centre crop of the same volume is compared with the oracle directly."""
+import pytest
+import torch
+
+from bench import build_workload
+from pyapr import aprnet
+from pyapr.aprnet import _ops
+from oracle import oracle
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+@pytest.fixture(scope="module")
+def apr():
+    a = build_workload("blobs512")
+    a.init_cuda()
+    return a
+
+
+def _identity_weights(c, ksize, dtype=torch.float32):
+    kz, kx, ky = ksize
+    w = torch.zeros(1, c, c, kz, kx, ky, dtype=dtype)           # [S, Cout, Cin, k], one stencil for all levels
+    for i in range(c):
+        w[0, i, i, kz // 2, kx // 2, ky // 2] = 1
+    return w
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
+@pytest.mark.parametrize("ksize", [(3, 3, 3), (1, 5, 5)], ids=["333", "155"])
+def test_identity_stencil_returns_input(apr, ksize, dtype):
+    """A stencil whose only non-zero tap is the centre copies every particle and every downsampled particle:
+    exact in both element types (one product with 1.0 per output)."""
+    n, c = apr.total_number_particles(), 20
+    g = torch.Generator().manual_seed(0)
+    x = torch.randn(1, c, n, generator=g).to(dtype).to(DEV)
+    levels = apr.level_max() - apr.level_min() + 1
+    w = _identity_weights(c, ksize).expand(levels, -1, -1, -1, -1, -1).contiguous().to(DEV)
+    for d in (0, 1):
+        nd = _ops.number_particles(apr, d)
+        xd = x[:, :, :nd].contiguous()
+        y = _ops.conv_forward([apr], xd, w, torch.tensor([d], dtype=torch.int32))
+        assert torch.equal(y, xd)
+
+
+def test_forward_is_linear_and_backward_is_its_adjoint(apr):
+    n, cin, cout = apr.total_number_particles(), 8, 24
+    g = torch.Generator().manual_seed(1)
+    ld = torch.zeros(1, dtype=torch.int32)
+    levels = apr.level_max() - apr.level_min() + 1
+    w = (torch.randn(levels, cout, cin, 3, 3, 3, generator=g) * 0.2).to(DEV)
+    x1 = torch.randn(1, cin, n, generator=g).to(DEV)
+    x2 = torch.randn(1, cin, n, generator=g).to(DEV)
+    y1, y2 = _ops.conv_forward([apr], x1, w, ld), _ops.conv_forward([apr], x2, w, ld)
+    y12 = _ops.conv_forward([apr], 2 * x1 - 3 * x2, w, ld)
+    scale = float(y12.abs().max())
+    assert float((y12 - (2 * y1 - 3 * y2)).abs().max()) <= 2e-5 * scale
+    gy = torch.randn(1, cout, n, generator=g).to(DEV)
+    gx, gw = _ops.conv_backward([apr], x1, w, gy, ld)
+    # <conv(x), gy> == <x, conv'(gy)> == <w, dW>   (float64 accumulation of the inner products)
+    lhs = float((y1.double() * gy.double()).sum())
+    rhs_x = float((x1.double() * gx.double()).sum())
+    rhs_w = float((w.double() * gw.double()).sum())
+    ref = float((y1.double().abs() * gy.double().abs()).sum())
+    assert abs(lhs - rhs_x) <= 1e-5 * ref
+    assert abs(lhs - rhs_w) <= 1e-5 * ref
+
+
+def test_pool_argmax_gathers_and_upsample_round_trip(apr):
+    n, c = apr.total_number_particles(), 6
+    g = torch.Generator().manual_seed(2)
+    x = torch.randn(1, c, n, generator=g).to(DEV)
+    ld = torch.zeros(1, dtype=torch.int32)
+    out, idx = _ops.maxpool_forward([apr], x, ld, 0.0)
+    n1, ncopy = _ops.number_particles(apr, 1), apr.iterator().particles_level_end(apr.level_max() - 1)
+    assert out.shape[2] == n1
+    assert torch.equal(out[:, :, :ncopy], x[:, :, :ncopy])                     # coarser particles pass through
+    pooled = out[:, :, ncopy:]
+    assert torch.equal(pooled, torch.gather(x, 2, idx[:, :, ncopy:]))          # the value at the reported argmax
+    up = _ops.upsample_const_forward([apr], out, torch.ones(1, dtype=torch.int32))
+    assert up.shape[2] == n
+    assert torch.equal(up[:, :, :ncopy], x[:, :, :ncopy])
+    assert bool((up[:, :, ncopy:] >= x[:, :, ncopy:]).all())                   # every child sees its block's maximum
+    again, idx2 = _ops.maxpool_forward([apr], up, ld, 0.0)
+    assert torch.equal(again, out)                                             # pool(upsample(pool(x))) == pool(x)
+    # backward of the pool scatters exactly the pooled gradients: sums agree per channel
+    go = torch.randn(1, c, n1, generator=g).to(DEV)
+    gi = _ops.maxpool_backward([apr], go, idx, ld)
+    torch.testing.assert_close(gi.double().sum(dim=2), go.double().sum(dim=2), rtol=1e-9, atol=1e-6)
+
+
+def test_centre_crop_against_oracle():
+    """The benchmark's CPU-baseline sample (128x256x256 crop, 3 M particles) through both implementations."""
+    apr = build_workload("blobs512", crop=(128, 256, 256))
+    apr.init_cuda()
+    n, cin, cout = apr.total_number_particles(), 4, 6
+    g = torch.Generator().manual_seed(3)
+    x = torch.randn(1, cin, n, generator=g)
+    w = torch.randn(cin, 2, cout, 3, 3, 3, generator=g) * 0.2
+    ld = torch.zeros(1, dtype=torch.int32)
+    w_exp = oracle.restrict_kernel_forward(w, apr.level_max() - apr.level_min() + 1)
+    ref = oracle.conv_forward([apr], x, w_exp, ld)
+    got = _ops.conv_forward([apr], x.to(DEV), w_exp.permute(1, 2, 0, 3, 4, 5).contiguous().to(DEV), ld)
+    assert float((got.cpu() - ref).abs().max()) <= 1e-5 * float(ref.abs().max())
