@@ -134,6 +134,13 @@ int plan_scratch(aprnet_plan* plan, size_t bytes, hipStream_t st);
             return aprnet::fail(APRNET_ERR_HIP, std::string("launch of ") + name + ": " + hipGetErrorString(e_)); \
     } while (0)
 
+// buffer loads of the convolution kernels use 32-bit byte offsets inside a channel plane
+inline int check_plane_size(const aprnet_plan* p, int d, size_t elem, const char* who) {
+    if ((uint64_t)p->number_parts(d) * elem >= (1ull << 32) || (uint64_t)p->tree_parts(d) * elem >= (1ull << 32))
+        return fail(APRNET_ERR_UNSUPPORTED, std::string(who) + ": a channel plane of this element size exceeds 4 GiB");
+    return 0;
+}
+
 inline int check_level_delta(const aprnet_plan* p, int d, const char* who) {
     if (!p) return fail(APRNET_ERR_INVALID_ARGUMENT, std::string(who) + ": null plan");
     // CHECK_LEVEL_DELTA(dlvl, tree.level_max()+1): cuda/src/common.hpp:17, wrap_conv_gpu.hpp:46

@@ -174,6 +174,7 @@ int conv_fwd(const aprnet_plan* cp, int d, int kz, int kx, int ky, const T* x, i
              int S_exp, int Cout, const T* bias, T* y, int64_t ldy, T* tree_ws, int64_t ldt, hipStream_t st) {
     aprnet_plan* p = const_cast<aprnet_plan*>(cp);
     if (int rc = check_level_delta(p, d, "conv_forward")) return rc;
+    if (int rc = check_plane_size(p, d, sizeof(*x), "conv_forward")) return rc;
     if (Cin <= 0 || Cout <= 0 || S_exp <= 0) return fail(APRNET_ERR_INVALID_ARGUMENT, "conv_forward: empty channel / stencil count");
     const int code = kz * 100 + kx * 10 + ky;
     if (code != 333 && code != 133 && code != 155 && code != 555)
@@ -210,6 +211,7 @@ int conv_fwd_bf16(const aprnet_plan* cp, int d, int kz, int kx, int ky, const bf
                   int S_exp, int Cout, const float* bias, bf16_t* y, int64_t ldy, bf16_t* tree_ws, int64_t ldt, hipStream_t st) {
     aprnet_plan* p = const_cast<aprnet_plan*>(cp);
     if (int rc = check_level_delta(p, d, "conv_forward")) return rc;
+    if (int rc = check_plane_size(p, d, sizeof(*x), "conv_forward")) return rc;
     if (Cin <= 0 || Cout <= 0 || S_exp <= 0) return fail(APRNET_ERR_INVALID_ARGUMENT, "conv_forward: empty channel / stencil count");
     const int code = kz * 100 + kx * 10 + ky;
     if (!conv_mfma_supported(code))

@@ -257,6 +257,7 @@ int conv_bwd(const aprnet_plan* cp, int d, int kz, int kx, int ky, const T* x, i
              int64_t ldgt, hipStream_t st) {
     aprnet_plan* p = const_cast<aprnet_plan*>(cp);
     if (int rc = check_level_delta(p, d, "conv_backward")) return rc;
+    if (int rc = check_plane_size(p, d, sizeof(*x), "conv_backward")) return rc;
     if (Cin <= 0 || Cout <= 0 || S_exp <= 0) return fail(APRNET_ERR_INVALID_ARGUMENT, "conv_backward: empty channel / stencil count");
     const int code = kz * 100 + kx * 10 + ky;
     if (code != 333 && code != 133 && code != 155 && code != 555)

@@ -36,7 +36,8 @@ struct ConvArgs {
     const T* gy; T* gx; int64_t ldgx; T* gtree; int64_t ldgt; T* gw; int n_tiles;
     // window lists built once per APR and kept in the plan (kernels that do not scan)
     const int* tile_win;                       // [n_tiles + 1] first stored window of every tile
-    const int4* win;                           // per stored window: {first item, items, first column, columns}
+    const int4* win;                           // per stored window: {first item, items, first column, columns}; the two
+                                               // "first" fields are unsigned 32-bit offsets
     const int* l_item_idx; const unsigned short* l_item_pos;
     const int* l_col_idx; const unsigned short* l_col_pos;
 };
@@ -339,7 +340,7 @@ __device__ __forceinline__ void close_window(ConvShared<G>& sh) {
 // supplies a 32-bit byte offset, and an offset outside the plane returns zero without touching memory.
 // That keeps the address registers to one per item and makes every predicate of the gather (item
 // exists / value lives in the tree buffer / channel exists) an out-of-range offset or an empty plane
-// instead of a branch.  plan_create limits an access to 2^29 particles so that offsets fit 32 bits.
+// instead of a branch.  The entry points refuse channel planes of 4 GiB or more so that offsets fit 32 bits.
 constexpr unsigned BUF_OOB = 0xffffffffu;
 
 template <typename T> struct RawLoad;

@@ -221,7 +221,7 @@ conv_mfma16_kernel(const ConvArgs<T> a) {
             const int win = w - wb;
             const int4 hd = a.win[w];
             const int nitem = __builtin_amdgcn_readfirstlane(hd.y), nc = __builtin_amdgcn_readfirstlane(hd.w);
-            const WindowLists gl{a.l_item_idx + hd.x, a.l_item_pos + hd.x, a.l_col_idx + hd.z, a.l_col_pos + hd.z};
+            const WindowLists gl{a.l_item_idx + (unsigned)hd.x, a.l_item_pos + (unsigned)hd.x, a.l_col_idx + (unsigned)hd.z, a.l_col_pos + (unsigned)hd.z};
             APRNET_WINDOW(gl)
             __syncthreads();        // the next window rewrites the patch
         }
@@ -416,7 +416,7 @@ conv_mfma_bf16_kernel(const ConvArgs<bf16_t> a) {
         const int win = w - wb;
         const int4 hd = a.win[w];
         const int nitem = __builtin_amdgcn_readfirstlane(hd.y), nc = __builtin_amdgcn_readfirstlane(hd.w);
-        const WindowLists gl{a.l_item_idx + hd.x, a.l_item_pos + hd.x, a.l_col_idx + hd.z, a.l_col_pos + hd.z};
+        const WindowLists gl{a.l_item_idx + (unsigned)hd.x, a.l_item_pos + (unsigned)hd.x, a.l_col_idx + (unsigned)hd.z, a.l_col_pos + (unsigned)hd.z};
         const int nblk = (nc + 15) >> 4;
         const int first = (wave - (int)blockIdx.x - win) & (G::NWAVE - 1);
         const int nb = first < nblk ? (nblk - first + G::NWAVE - 1) / G::NWAVE : 0;

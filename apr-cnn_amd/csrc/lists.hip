@@ -33,10 +33,11 @@ build_lists_kernel(const ConvArgs<float> a, const int pass, int4* __restrict__ t
         const int nc = sh.ncol, nitem = sh.nitem;
         if (nc > 0) {
             if (pass == 1) {
-                const int ib = off.y + ni, cb = off.z + ncl;
-                if (threadIdx.x == 0) win[off.x + nwin] = make_int4(ib, nitem, cb, nc);
-                for (int i = threadIdx.x; i < nitem; i += G::NT) { item_idx[ib + i] = sh.item_idx[i]; item_pos[ib + i] = sh.item_pos[i]; }
-                for (int i = threadIdx.x; i < nc; i += G::NT) { col_idx[cb + i] = sh.col_idx[i]; col_pos[cb + i] = sh.col_pos[i]; }
+                // list offsets are unsigned 32-bit numbers stored in the int fields of the header
+                const unsigned ib = (unsigned)off.y + (unsigned)ni, cb = (unsigned)off.z + (unsigned)ncl;
+                if (threadIdx.x == 0) win[off.x + nwin] = make_int4((int)ib, nitem, (int)cb, nc);
+                for (int i = threadIdx.x; i < nitem; i += G::NT) { item_idx[(size_t)ib + i] = sh.item_idx[i]; item_pos[(size_t)ib + i] = sh.item_pos[i]; }
+                for (int i = threadIdx.x; i < nc; i += G::NT) { col_idx[(size_t)cb + i] = sh.col_idx[i]; col_pos[(size_t)cb + i] = sh.col_pos[i]; }
             }
             ++nwin; ni += nitem; ncl += nc;
         }
@@ -92,14 +93,14 @@ int get_lists(aprnet_plan* p, int level_delta, int code, const TileList& tl, Win
         std::vector<int> tile_win(tl.n + 1);
         int64_t nw = 0, ni = 0, nc = 0;
         for (int t = 0; t < tl.n; ++t) {
-            offs[t] = make_int4((int)nw, (int)ni, (int)nc, 0);
+            offs[t] = make_int4((int)nw, (int)(uint32_t)ni, (int)(uint32_t)nc, 0);
             tile_win[t] = (int)nw;
             nw += counts[t].x; ni += counts[t].y; nc += counts[t].z;
         }
         tile_win[tl.n] = (int)nw;
-        if (ni >= (int64_t)INT32_MAX || nc >= (int64_t)INT32_MAX) {
+        if (ni >= (int64_t)UINT32_MAX || nc >= (int64_t)UINT32_MAX || nw >= (int64_t)INT32_MAX) {
             (void)hipFree(d_counts);
-            return fail(APRNET_ERR_UNSUPPORTED, "window lists: more than 2^31 entries");
+            return fail(APRNET_ERR_UNSUPPORTED, "window lists: more than 2^32 entries");
         }
         wl.n_win = (int)nw; wl.n_items = ni; wl.n_cols = nc;
         auto alloc = [&](void** q, size_t bytes) -> int { APRNET_HIP_CHECK(hipMalloc(q, std::max<size_t>(bytes, 16))); return 0; };

@@ -28,9 +28,10 @@ static int copy_access(const aprnet_access_desc* d, HostAccess& h, int lmax_all)
     h.xz_end.assign(d->xz_end_vec, d->xz_end_vec + d->n_rows);
     if (h.xz_end.empty() || h.xz_end[0] != 0 || h.xz_end.back() != d->n_particles)
         return fail(APRNET_ERR_INVALID_ARGUMENT, "plan_create: xz_end_vec must start at 0 and end at n_particles");
-    // kernels address a channel plane with 32-bit byte offsets (8-byte elements at most)
-    if (d->n_particles >= (1ull << 29))
-        return fail(APRNET_ERR_UNSUPPORTED, "plan_create: 2^29 or more particles per access");
+    // the convolution kernels address a channel plane with 32-bit byte offsets: 2^30 elements of 4 bytes
+    // (conv entry points check the element size of the call, check_plane_size)
+    if (d->n_particles >= (1ull << 30))
+        return fail(APRNET_ERR_UNSUPPORTED, "plan_create: 2^30 or more particles per access");
     if (d->n_particles) h.y.assign(d->y_vec, d->y_vec + d->n_particles);
     return 0;
 }
