@@ -229,6 +229,9 @@ static int launch_bwd(ConvArgs<T>& a, hipStream_t st) {
 bool conv_mfma_supported(int code);
 int launch_conv_dx_mfma(int code, const ConvArgs<float>& a, int n_tiles, hipStream_t st);
 int launch_conv_dw_mfma(int code, const ConvArgs<float>& a, const TileList& tl, int level_min, hipStream_t st);
+int launch_conv_dx_mfma(int code, const ConvArgs<bf16_t>& a, int n_tiles, hipStream_t st);
+int launch_conv_dw_mfma(int code, const ConvArgs<bf16_t>& a, const TileList& tl, int level_min, hipStream_t st);
+int fill_tree_for_conv(const aprnet_plan* p, int d, const bf16_t* x, int64_t ldx, int C, bf16_t* tree, int64_t ldt, hipStream_t st);
 size_t conv_packed_floats(int code, int S_exp, int Cm, int Ck, bool transposed);
 int pack_conv_weights(int code, const float* w, int S_exp, int Cm, int Ck, bool transposed, float* packed, hipStream_t st);
 int conv_path();
@@ -294,10 +297,72 @@ int conv_bwd(const aprnet_plan* cp, int d, int kz, int kx, int ky, const T* x, i
     return fill_tree_bwd_for_conv(p, d, gx, ldgx, Cin, gtree_ws, ldgt, st);
 }
 
+__global__ void round_to_bf16_kernel(const float* __restrict__ src, int64_t lds, bf16_t* __restrict__ dst, int64_t ldd, int64_t n) {
+    const float* s = src + (int64_t)blockIdx.y * lds;
+    bf16_t* d = dst + (int64_t)blockIdx.y * ldd;
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x) d[i] = float_to_bf16(s[i]);
+}
+
+// bfloat16 features and output gradient; weights, weight gradient and all accumulation in fp32 (the fp32
+// matrix-core kernels with 16-bit loads).  gx32_ws [Cin][ldgx32] and gtree_ws [Cin][ldgt] are fp32 work space:
+// the input gradient is accumulated there and rounded to bfloat16 at the end.
+int conv_bwd_bf16(const aprnet_plan* cp, int d, int kz, int kx, int ky, const bf16_t* x, int64_t ldx, int Cin, const float* w,
+                  int S_exp, int Cout, const bf16_t* gy, int64_t ldy, bf16_t* gx, int64_t ldgx, float* gw, bf16_t* tree_ws,
+                  int64_t ldt, float* gx32_ws, int64_t ldgx32, float* gtree_ws, int64_t ldgt, hipStream_t st) {
+    aprnet_plan* p = const_cast<aprnet_plan*>(cp);
+    if (int rc = check_level_delta(p, d, "conv_backward")) return rc;
+    if (int rc = check_plane_size(p, d, sizeof(float), "conv_backward")) return rc;
+    if (Cin <= 0 || Cout <= 0 || S_exp <= 0) return fail(APRNET_ERR_INVALID_ARGUMENT, "conv_backward: empty channel / stencil count");
+    const int code = kz * 100 + kx * 10 + ky;
+    if (!conv_mfma_supported(code))
+        return fail(APRNET_ERR_UNSUPPORTED, "conv_backward: bfloat16 features are supported for the 3x3x3, 1x3x3 and 1x5x5 stencils");
+    const int64_t nt = p->tree_parts(d), np = p->number_parts(d);
+    if (!gx32_ws || ldgx32 < np || (nt > 0 && (!tree_ws || !gtree_ws || ldt < nt || ldgt < nt)))
+        return fail(APRNET_ERR_INVALID_ARGUMENT, "conv_backward: work space too small");
+    APRNET_HIP_CHECK(hipSetDevice(p->device));
+    if (int rc = fill_tree_for_conv(p, d, x, ldx, Cin, tree_ws, ldt, st)) return rc;
+    fill2d<float>(gx32_ws, ldgx32, np, Cin, 0.f, st);
+    fill2d<float>(gtree_ws, ldgt, nt, Cin, 0.f, st);
+    const bool flat = (kz == 1);
+    TileList tl, near;
+    if (int rc = get_tiles(p, d, flat ? 1 : 2, flat ? 8 : 4, &tl)) return rc;
+    if (int rc = get_tiles(p, d, flat ? 1 : 2, flat ? 8 : 4, &near, 1)) return rc;
+    if (tl.n > 0) {
+        ConvArgs<bf16_t> a{};
+        a.apr = p->dapr; a.tree = p->dtree; a.tiles = tl.d_tiles; a.n_tiles = tl.n;
+        a.x = x; a.ldx = ldx; a.Cin = Cin; a.w = w; a.S_exp = S_exp; a.Cout = Cout;
+        a.tree_data = tree_ws; a.ldt = ldt; a.Lc = p->lc(d); a.tree_off = p->tree_offset(a.Lc);
+        a.x_count = np; a.t_count = nt;
+        a.gy = gy; a.ldy = ldy; a.gx = gx32_ws; a.ldgx = ldgx32; a.gtree = gtree_ws; a.ldgt = ldgt; a.gw = gw;
+        if (int rc = plan_scratch(p, conv_packed_floats(code, S_exp, Cin, Cout, true) * sizeof(float), st)) return rc;
+        if (int rc = pack_conv_weights(code, w, S_exp, Cin, Cout, true, (float*)p->d_scratch, st)) return rc;
+        ConvArgs<bf16_t> b = a;
+        b.tiles = near.d_tiles; b.n_tiles = near.n;
+        b.x = gy; b.ldx = ldy; b.Cin = Cout; b.Cout = Cin; b.w = (const float*)p->d_scratch; b.bias = nullptr;
+        b.tree_data = nullptr; b.t_count = 0;
+        if (near.n > 0) if (int rc = launch_conv_dx_mfma(code, b, near.n, st)) return rc;
+        if (int rc = launch_conv_dw_mfma(code, a, tl, p->apr.level_min, st)) return rc;
+    }
+    if (int rc = fill_tree_bwd_for_conv(p, d, gx32_ws, ldgx32, Cin, gtree_ws, ldgt, st)) return rc;
+    if (np > 0) {
+        dim3 grid((unsigned)std::min<int64_t>((np + 255) / 256, 4096), (unsigned)Cin);
+        hipLaunchKernelGGL(round_to_bf16_kernel, grid, dim3(256), 0, st, gx32_ws, ldgx32, gx, ldgx, np);
+        APRNET_LAUNCH_CHECK("round_to_bf16_kernel");
+    }
+    return 0;
+}
+
 }  // namespace aprnet
 
 using namespace aprnet;
 extern "C" {
+int aprnet_conv_bwd_bf16(const aprnet_plan* p, int d, int kz, int kx, int ky, const uint16_t* x, int64_t ldx, int Cin,
+                         const float* w, int S_exp, int Cout, const uint16_t* gy, int64_t ldy, uint16_t* gx, int64_t ldgx,
+                         float* gw, uint16_t* tree_ws, int64_t ldt, float* gx32_ws, int64_t ldgx32, float* gtree_ws,
+                         int64_t ldgt, void* st) {
+    return conv_bwd_bf16(p, d, kz, kx, ky, (const bf16_t*)x, ldx, Cin, w, S_exp, Cout, (const bf16_t*)gy, ldy, (bf16_t*)gx, ldgx,
+                         gw, (bf16_t*)tree_ws, ldt, gx32_ws, ldgx32, gtree_ws, ldgt, (hipStream_t)st);
+}
 int aprnet_conv_bwd_f32(const aprnet_plan* p, int d, int kz, int kx, int ky, const float* x, int64_t ldx, int Cin,
                         const float* w, int S_exp, int Cout, const float* gy, int64_t ldy, float* gx, int64_t ldgx,
                         float* gw, float* tree_ws, int64_t ldt, float* gtree_ws, int64_t ldgt, void* st) {

@@ -32,9 +32,10 @@ constexpr int DW_NCH = 4;          // chunks per block
 constexpr int DW_GB = 256;         // columns of gY staged at a time
 constexpr int DW_GLD = 33;         // words per column of gyl (32 output channels + 1 against bank conflicts)
 
-template <class G, int CIB, int NCH>
+// T: storage type of the features and of the output gradient (float, or bfloat16 widened to fp32 on load)
+template <typename T, class G, int CIB, int NCH>
 __global__ void __launch_bounds__(G::NT) __attribute__((amdgpu_waves_per_eu(4, 4)))
-conv_dw_mfma_kernel(const ConvArgs<float> a, const int s_idx) {
+conv_dw_mfma_kernel(const ConvArgs<T> a, const int s_idx) {
     static_assert(G::NWAVE == 8 && CIB == 4, "wave w owns input channel w%4 and column half w/4");
     __shared__ float patch[CIB * G::CH_STRIDE];
     __shared__ float gyl[DW_GB * DW_GLD];
@@ -63,11 +64,11 @@ conv_dw_mfma_kernel(const ConvArgs<float> a, const int s_idx) {
         const bool out_tree = (L == a.Lc) && (L < a.apr.level_max);
 
         __syncthreads();
-        open_segments<G, float>(a, L, z0, x0, sh);
+        open_segments<G, T>(a, L, z0, x0, sh);
         __syncthreads();
 
         for (int y0 = 0; y0 < yn; y0 += G::TY) {
-            scan_window<G, float>(a, L, y0, out_tree, sh);
+            scan_window<G, T>(a, L, y0, out_tree, sh);
             __syncthreads();
             const int nc = __builtin_amdgcn_readfirstlane(sh.ncol), nitem = __builtin_amdgcn_readfirstlane(sh.nitem);
             if (nc > 0) {
@@ -83,14 +84,14 @@ conv_dw_mfma_kernel(const ConvArgs<float> a, const int s_idx) {
                         for (int k = 0; k < 32 / G::NWAVE; ++k) {
                             const int co = wave + k * G::NWAVE;
                             float v = 0.f;
-                            if (idx >= 0 && co0 + co < a.Cout) v = a.gy[(int64_t)(co0 + co) * a.ldy + idx];
+                            if (idx >= 0 && co0 + co < a.Cout) v = Num<T>::ld(a.gy[(int64_t)(co0 + co) * a.ldy + idx]);
                             gyl[slot * DW_GLD + co] = v;
                         }
                     }
 #pragma unroll
                     for (int q = 0; q < NCH; ++q) {
                         __syncthreads();        // previous chunk's reads of the patch are done / gyl is written
-                        stage_values<G, float, CIB>(a, cig0 + q * CIB, nitem, L < a.Lc, sh, patch);
+                        stage_values<G, T, CIB>(a, cig0 + q * CIB, nitem, L < a.Lc, sh, patch);
                         __syncthreads();
 #pragma unroll 1
                         for (int b = 0; b < nbatch; ++b) {
@@ -132,31 +133,38 @@ conv_dw_mfma_kernel(const ConvArgs<float> a, const int s_idx) {
 // Weight gradient; a.gw is accumulated into (the caller zeroes it).
 // One launch per stencil index: level Lc - s for s < S_exp - 1, every coarser level for the last one
 // (adjacent in the tile list, which is sorted finest level first).
-template <class G>
-static int launch_dw(const ConvArgs<float>& a0, const TileList& tl, int level_min, hipStream_t st) {
+template <typename T, class G>
+static int launch_dw(const ConvArgs<T>& a0, const TileList& tl, int level_min, hipStream_t st) {
     for (int s = 0; s < a0.S_exp; ++s) {
         const int l_hi = a0.Lc - s, l_lo = (s == a0.S_exp - 1) ? level_min : l_hi;
         if (l_hi < level_min) break;
         int n = 0;
         for (int l = l_lo; l <= l_hi; ++l) n += tl.level_count[l];
         if (n == 0) continue;
-        ConvArgs<float> a = a0;
+        ConvArgs<T> a = a0;
         a.tiles = tl.d_tiles + tl.level_begin[l_hi]; a.n_tiles = n;
         dim3 grid((unsigned)std::min(n, 512), (unsigned)((a.Cin + DW_CIB * DW_NCH - 1) / (DW_CIB * DW_NCH)),
                   (unsigned)((a.Cout + 31) / 32));
-        hipLaunchKernelGGL((conv_dw_mfma_kernel<G, DW_CIB, DW_NCH>), grid, dim3(G::NT), 0, st, a, s);
+        hipLaunchKernelGGL((conv_dw_mfma_kernel<T, G, DW_CIB, DW_NCH>), grid, dim3(G::NT), 0, st, a, s);
         APRNET_LAUNCH_CHECK("conv_dw_mfma_kernel");
     }
     return 0;
 }
 
-int launch_conv_dw_mfma(int code, const ConvArgs<float>& a, const TileList& tl, int level_min, hipStream_t st) {
+template <typename T>
+static int launch_dw_code(int code, const ConvArgs<T>& a, const TileList& tl, int level_min, hipStream_t st) {
     switch (code) {
-        case 333: return launch_dw<W333M>(a, tl, level_min, st);
-        case 133: return launch_dw<W133M>(a, tl, level_min, st);
-        case 155: return launch_dw<W155M>(a, tl, level_min, st);
+        case 333: return launch_dw<T, W333M>(a, tl, level_min, st);
+        case 133: return launch_dw<T, W133M>(a, tl, level_min, st);
+        case 155: return launch_dw<T, W155M>(a, tl, level_min, st);
     }
     return fail(APRNET_ERR_UNSUPPORTED, "no matrix-core kernel for this stencil");
+}
+int launch_conv_dw_mfma(int code, const ConvArgs<float>& a, const TileList& tl, int level_min, hipStream_t st) {
+    return launch_dw_code<float>(code, a, tl, level_min, st);
+}
+int launch_conv_dw_mfma(int code, const ConvArgs<bf16_t>& a, const TileList& tl, int level_min, hipStream_t st) {
+    return launch_dw_code<bf16_t>(code, a, tl, level_min, st);
 }
 
 }  // namespace aprnet

@@ -33,7 +33,9 @@ struct ConvArgs {
     int Lc; int64_t tree_off;                  // tree_offset(Lc)
     int64_t x_count, t_count;                  // valid elements per channel plane of x / tree_data
     // backward only
-    const T* gy; T* gx; int64_t ldgx; T* gtree; int64_t ldgt; T* gw; int n_tiles;
+    // gradients are accumulated in the computation type (fp32 for bfloat16 features)
+    const T* gy; typename Num<T>::acc* gx; int64_t ldgx; typename Num<T>::acc* gtree; int64_t ldgt;
+    typename Num<T>::acc* gw; int n_tiles;
     // window lists built once per APR and kept in the plan (kernels that do not scan)
     const int* tile_win;                       // [n_tiles + 1] first stored window of every tile
     const int4* win;                           // per stored window: {first item, items, first column, columns}; the two

@@ -154,7 +154,7 @@ __device__ __forceinline__ void mfma16_window(const ConvArgs<T>& a, int co0, int
                     const int cl = h * 16 + 4 * (lane >> 4) + r;
                     if (co0 + cl < a.Cout) a.y[(int64_t)(co0 + cl) * a.ldy + o] = Num<T>::st(acc[j][h][r] + bias_l[cl]);
                 }
-        } else if constexpr (sizeof(T) == 4) {      // gradients are accumulated in fp32 only
+        } else {
             const bool to_tree = (sh.col_pos[col] & COL_TREE) != 0;
             float* dst = (to_tree ? a.gtree : a.gx) + o;
             const int64_t ld = to_tree ? a.ldgt : a.ldgx;
@@ -499,6 +499,7 @@ int pack_conv_weights_bf16(int code, const float* w, int S_exp, int Cout, int Ci
 // Input gradient: a.x / a.Cin describe the output gradient, a.Cout the input channels, a.w the packed
 // transposed weights, a.tiles the row groups within one row of an output (n_tiles of them).
 int launch_conv_dx_mfma(int code, const ConvArgs<float>& a, int n_tiles, hipStream_t st) { return launch16_code<float, 1>(code, a, n_tiles, st); }
+int launch_conv_dx_mfma(int code, const ConvArgs<bf16_t>& a, int n_tiles, hipStream_t st) { return launch16_code<bf16_t, 1>(code, a, n_tiles, st); }
 
 // Cm: channels on the M axis of the kernel, Ck: contracted channels (forward: Cout, Cin; transposed: Cin, Cout)
 // `transposed`: image for the input gradient (chunks of DX_CIB), otherwise for the forward pass (chunks of FWD_CIB)

@@ -104,21 +104,25 @@ constexpr int CS_BLOCKS = 256, CS_TB = 256;
 
 template <typename T>
 __global__ void __launch_bounds__(CS_TB)
-channel_sum_partial_kernel(const T* __restrict__ x, int64_t ld, int64_t n, T* __restrict__ partial) {
-    __shared__ T red[CS_TB / 64];
+channel_sum_partial_kernel(const T* __restrict__ x, int64_t ld, int64_t n, typename Num<T>::acc* __restrict__ partial) {
+    typedef typename Num<T>::acc A;
+    __shared__ A red[CS_TB / 64];
     const T* row = x + (int64_t)blockIdx.y * ld;
-    T s0 = 0, s1 = 0, s2 = 0, s3 = 0;
+    A s0 = 0, s1 = 0, s2 = 0, s3 = 0;
     const int64_t stride = (int64_t)gridDim.x * CS_TB;
     int64_t i = (int64_t)blockIdx.x * CS_TB + threadIdx.x;
-    for (; i + 3 * stride < n; i += 4 * stride) { s0 += row[i]; s1 += row[i + stride]; s2 += row[i + 2 * stride]; s3 += row[i + 3 * stride]; }
-    for (; i < n; i += stride) s0 += row[i];
-    T s = (s0 + s1) + (s2 + s3);
+    for (; i + 3 * stride < n; i += 4 * stride) {
+        s0 += Num<T>::ld(row[i]); s1 += Num<T>::ld(row[i + stride]);
+        s2 += Num<T>::ld(row[i + 2 * stride]); s3 += Num<T>::ld(row[i + 3 * stride]);
+    }
+    for (; i < n; i += stride) s0 += Num<T>::ld(row[i]);
+    A s = (s0 + s1) + (s2 + s3);
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) s += __shfl_down(s, off);
     if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = s;
     __syncthreads();
     if (threadIdx.x == 0) {
-        T t = 0;
+        A t = 0;
 #pragma unroll
         for (int w = 0; w < CS_TB / 64; ++w) t += red[w];
         partial[(int64_t)blockIdx.y * gridDim.x + blockIdx.x] = t;
@@ -136,11 +140,12 @@ channel_sum_final_kernel(const T* __restrict__ partial, int nb, T* __restrict__ 
 }
 
 template <typename T>
-int channel_sum(const T* x, int64_t ld, int C, int64_t n, T* out, int accumulate, T* work, hipStream_t st) {
+int channel_sum(const T* x, int64_t ld, int C, int64_t n, typename Num<T>::acc* out, int accumulate, typename Num<T>::acc* work,
+                hipStream_t st) {
     if (C <= 0) return 0;
     if (!x || !out || !work || n < 0) return fail(APRNET_ERR_INVALID_ARGUMENT, "channel_sum: null argument");
     hipLaunchKernelGGL(channel_sum_partial_kernel<T>, dim3(CS_BLOCKS, (unsigned)C), dim3(CS_TB), 0, st, x, ld, n, work);
-    hipLaunchKernelGGL(channel_sum_final_kernel<T>, dim3((unsigned)C), dim3(64), 0, st, work, CS_BLOCKS, out, accumulate);
+    hipLaunchKernelGGL(channel_sum_final_kernel<typename Num<T>::acc>, dim3((unsigned)C), dim3(64), 0, st, work, CS_BLOCKS, out, accumulate);
     APRNET_LAUNCH_CHECK("channel_sum kernels");
     return 0;
 }
@@ -152,6 +157,9 @@ extern "C" {
 int aprnet_channel_sum_work_elems(int C) { return C * CS_BLOCKS; }
 int aprnet_channel_sum_f32(const float* x, int64_t ld, int C, int64_t n, float* out, int accumulate, float* work, void* st) {
     return channel_sum<float>(x, ld, C, n, out, accumulate, work, (hipStream_t)st);
+}
+int aprnet_channel_sum_bf16(const uint16_t* x, int64_t ld, int C, int64_t n, float* out, int accumulate, float* work, void* st) {
+    return channel_sum<bf16_t>((const bf16_t*)x, ld, C, n, out, accumulate, work, (hipStream_t)st);
 }
 int aprnet_channel_sum_f64(const double* x, int64_t ld, int C, int64_t n, double* out, int accumulate, double* work, void* st) {
     return channel_sum<double>(x, ld, C, n, out, accumulate, work, (hipStream_t)st);

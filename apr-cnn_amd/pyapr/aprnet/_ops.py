@@ -182,10 +182,11 @@ def channel_sum(x):
     """sum over batch and positions of a [B, C, N] tensor -> [C] (the bias gradient, conv.py:33), deterministic."""
     _check_input(x, "grad_output")
     B, C, N = x.shape
-    out = torch.empty(C, dtype=x.dtype, device=x.device)
+    acc = torch.float32 if x.dtype == torch.bfloat16 else x.dtype      # bfloat16 is summed in fp32
+    out = torch.empty(C, dtype=acc, device=x.device)
     lib = _lib()
-    work = torch.empty(lib.aprnet_channel_sum_work_elems(C), dtype=x.dtype, device=x.device)
-    fn = getattr(lib, "aprnet_channel_sum_" + _sfx(x))
+    work = torch.empty(lib.aprnet_channel_sum_work_elems(C), dtype=acc, device=x.device)
+    fn = getattr(lib, "aprnet_channel_sum_" + _sfx(x, bf16=True))
     with torch.cuda.device(x.device):
         st = _stream()
         for b in range(B):
@@ -206,8 +207,27 @@ def conv_backward(aprs, x, weights, grad_output, level_delta):
     sizes = [number_particles(a, d[b]) for b, a in enumerate(aprs)]
     gx = torch.empty_like(x)
     _zero_tails(gx, sizes)
-    gw = torch.zeros_like(weights)
     plans = _plans(aprs, x.device)
+    if x.dtype == torch.bfloat16:
+        # bfloat16 features and output gradient; weights and their gradient in fp32, fp32 accumulation
+        if (kz, kx, ky) == (1, 1, 1) or grad_output.dtype != torch.bfloat16:
+            raise TypeError("bfloat16 backward exists for the stencil convolutions with a bfloat16 output gradient")
+        weights = weights.float()
+        gw = torch.zeros_like(weights)
+        ld_tree = max(max(tree_parts(a, d[b]) for b, a in enumerate(aprs)), 1)
+        tree_ws = torch.empty((cin, ld_tree), dtype=x.dtype, device=x.device)
+        gtree_ws = torch.empty((cin, ld_tree), dtype=torch.float32, device=x.device)
+        gx32_ws = torch.empty((cin, N), dtype=torch.float32, device=x.device)
+        with torch.cuda.device(x.device):
+            st = _stream()
+            for b in range(B):
+                rc = _lib().aprnet_conv_bwd_bf16(plans[b], d[b], kz, kx, ky, _ptr(x[b]), N, cin, _ptr(weights), s_exp, cout,
+                                                 _ptr(grad_output[b]), grad_output.size(2), _ptr(gx[b]), N, _ptr(gw),
+                                                 _ptr(tree_ws), ld_tree, _ptr(gx32_ws), N, _ptr(gtree_ws), ld_tree, st)
+                if rc:
+                    _raise(rc, "conv_backward failed")
+        return [gx, gw]
+    gw = torch.zeros_like(weights)
     sfx = _sfx(x)
     with torch.cuda.device(x.device):
         st = _stream()

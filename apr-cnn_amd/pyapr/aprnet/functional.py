@@ -36,6 +36,7 @@ class ConvFunction(Function):
     def forward(ctx, inputs, weights, bias, aprs, level_deltas, layout):
         ctx.aprs = aprs
         ctx.layout = layout
+        ctx.param_dtypes = (weights.dtype, None if bias is None else bias.dtype)
         w = _to_device_layout(weights, layout).contiguous()
         if inputs.dtype == torch.bfloat16:
             w = w.float()          # bfloat16 stores the features; stencils are restricted and applied in fp32
@@ -60,7 +61,10 @@ class ConvFunction(Function):
         grad_bias = None if bias is None else _ops.channel_sum(grad_output)
         if ctx.expand:
             grad_w = _ops.restrict_kernel_backward(grad_w, ctx.num_stencils)
-        return grad_input, _from_device_layout(grad_w, ctx.layout), grad_bias, None, None, None
+        grad_w = _from_device_layout(grad_w, ctx.layout).to(ctx.param_dtypes[0])     # fp32 sums for bfloat16 features
+        if grad_bias is not None:
+            grad_bias = grad_bias.to(ctx.param_dtypes[1])
+        return grad_input, grad_w, grad_bias, None, None, None
 
 
 class MaxPoolFunction(Function):

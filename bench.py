@@ -155,6 +155,19 @@ def other_ops(apr, x, dev):
                     "note": f"{C}->{C}, bfloat16 features and matrix math (fp32 accumulate), whole APRConv.forward"})
         ms = _time(lambda: _ops.maxpool_forward([apr], xb, ld0, 0.0))
         line("maxpool_fwd_bf16", ms, 2 * C * n0 + (2 + 8) * C * n1, "bfloat16 values, int64 argmax")
+        x64b = torch.randn(1, 64, x.shape[2], device=dev).to(torch.bfloat16)
+        conv5b = aprnet.cuda.APRConv(64, 64, nstencils=2, kernel_size=(1, 5, 5)).to(dev)
+        ms = _time(lambda: conv5b(x64b, [apr], ld0), iters=3, warmup=1)
+        res.append({"op": "conv155_fwd_bf16", "ms": ms, "particles_per_s": n0 / ms * 1e3, "TFLOPs": 2 * 25 * 64 * 64 * n0 / ms / 1e9,
+                    "note": "1x5x5 64->64, bfloat16 features and matrix math (configs[4] layer), whole APRConv.forward"})
+    x64b.requires_grad_(True)
+    y5b = conv5b(x64b, [apr], ld0)
+    go5b = torch.randn_like(y5b)
+    ms = _time(lambda: torch.autograd.grad(y5b, (x64b, conv5b.weight), go5b, retain_graph=True), iters=2, warmup=1)
+    res.append({"op": "conv155_bwd_bf16", "ms": ms, "particles_per_s": n0 / ms * 1e3,
+                "note": "1x5x5 64->64 backward, bfloat16 features and gradients, fp32 matrix math and accumulation"})
+    del y5b, go5b, x64b, conv5b
+    with torch.no_grad():
         xinb = xin.to(torch.bfloat16)
         ms = _time(lambda: net(xinb, [apr]), iters=3, warmup=1)
     res.append({"op": "apr_unet_fwd_bf16", "ms": ms, "note": "same network, bfloat16 features"})

@@ -156,3 +156,24 @@ def test_maxpool_padding_values_per_flavour():
     ya, yb = a(x, aprs, ld), b(x, aprs, ld)
     assert torch.all(ya[0, :, n0:] == -1e17) and torch.all(yb[0, :, n0:] == 0)
     assert torch.equal(ya[:, :, :n0], yb[:, :, :n0])
+
+
+def test_aprconv_bf16_training_step():
+    """APRConv with bfloat16 features end to end through autograd: fp32 parameters get fp32 gradients, the input
+    gets a bfloat16 gradient, all within bfloat16 tolerance of the fp32 run."""
+    apr = apr_cases.get("3d_b")
+    n = oracle.number_parts(apr, 0)
+    torch.manual_seed(3)
+    model = aprnet.cuda.APRConv(6, 5, nstencils=2).to(DEV)
+    x32 = torch.randn(1, 6, n, device=DEV).to(torch.bfloat16).float().requires_grad_(True)
+    xb = x32.detach().to(torch.bfloat16).requires_grad_(True)
+    ld = torch.zeros(1, dtype=torch.int32)
+    go = torch.randn(1, 5, n, device=DEV).to(torch.bfloat16)
+    y32 = model(x32, [apr], ld)
+    g32 = torch.autograd.grad(y32, (x32, model.weight, model.bias), go.float())
+    yb = model(xb, [apr], ld)
+    gb = torch.autograd.grad(yb, (xb, model.weight, model.bias), go)
+    assert yb.dtype == torch.bfloat16 and gb[0].dtype == torch.bfloat16
+    assert gb[1].dtype == torch.float32 and gb[2].dtype == torch.float32
+    for a, b in zip(gb, g32):
+        assert float((a.float() - b).abs().max()) <= 1e-2 * float(b.abs().max())

@@ -404,8 +404,27 @@ def test_maxpool_upsample_bf16_bit_exact(bt):
     assert torch.equal(_ops.maxpool_backward(aprs, go.to(DEV), idx, ld).float().cpu(), gref)
 
 
-def test_conv_backward_bf16_is_refused():
-    x, aprs, ld, w_exp = _conv_case([("3d_a", 0)], (3, 3, 3), 1, 2, 2, torch.float32)
-    wd = w_exp.permute(1, 2, 0, 3, 4, 5).contiguous().to(DEV)
+@pytest.mark.parametrize("ksize", [(3, 3, 3), (1, 5, 5)], ids=KID)
+@pytest.mark.parametrize("bt", [[("3d_b", 1), ("3d_c", 0)], [("2d_a", 0), ("2d_b", 1)]], ids=lambda b: "+".join(f"{n}@{d}" for n, d in b))
+def test_conv_backward_bf16(bt, ksize):
+    """bfloat16 features and output gradient, fp32 weights and accumulation: gradients against the fp32 oracle on
+    the same (bfloat16-representable) inputs; the input gradient comes back in bfloat16, the weight gradient in fp32."""
+    cin, cout = 20, 33
+    x, aprs, ld, w_exp = _conv_case(bt, ksize, 2, cin, cout, torch.float32)
+    xb = x.to(torch.bfloat16)
+    g = torch.Generator().manual_seed(12)
+    gob = torch.randn(x.size(0), cout, x.size(2), generator=g).to(torch.bfloat16)
+    gx_ref, gw_ref = oracle.conv_backward(aprs, xb.float(), w_exp, gob.float(), ld)
+    gx, gw = _ops.conv_backward(aprs, xb.to(DEV), w_exp.permute(1, 2, 0, 3, 4, 5).contiguous().to(DEV), gob.to(DEV), ld)
+    close_bf16(gx, gx_ref)
+    assert gw.dtype == torch.float32
+    # fp32 sums; the mean-filled tree values they read are stored in bfloat16, hence the bfloat16 tolerance
+    gwc = gw.permute(2, 0, 1, 3, 4, 5).cpu()
+    assert float((gwc - gw_ref).abs().max()) <= 1e-2 * float(gw_ref.abs().max())
+
+
+def test_conv111_backward_bf16_is_refused():
+    x, aprs, ld, w = _conv_case([("3d_a", 0)], (1, 1, 1), 1, 2, 2, torch.float32)
+    wd = w.permute(1, 2, 0, 3, 4, 5).contiguous().to(DEV)
     with pytest.raises(TypeError):
         _ops.conv_backward(aprs, x.to(torch.bfloat16).to(DEV), wd, x.to(torch.bfloat16).to(DEV), ld)
