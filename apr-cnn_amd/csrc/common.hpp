@@ -82,6 +82,7 @@ struct WinLists {
     int* d_item_idx = nullptr; unsigned short* d_item_pos = nullptr;
     int* d_col_idx = nullptr; unsigned short* d_col_pos = nullptr;
     int n_win = 0; int64_t n_items = 0, n_cols = 0;
+    bool unavailable = false;                   // building them failed once (no memory, too many entries): do not retry
 };
 
 }  // namespace aprnet

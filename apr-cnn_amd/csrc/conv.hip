@@ -142,10 +142,16 @@ int pack_conv_weights(int code, const float* w, int S_exp, int Cm, int Ck, bool 
 static int g_conv_path = 0;      // 0: matrix cores where available, 1: VALU kernels only
 int conv_path() { return g_conv_path; }
 
+static int g_use_lists = 1;      // 1: forward kernels take the window lists of the plan, 0: they scan per call
+
+// Points the kernel at the plan's window lists.  When the lists are switched off, or cannot be built (no device
+// memory for them, too many entries), a.tile_win stays null and the kernel scans the access arrays itself.
 template <typename T>
 static int set_lists(aprnet_plan* p, int d, int code, const TileList& tl, ConvArgs<T>& a, hipStream_t st) {
+    a.tile_win = nullptr;
+    if (!g_use_lists) return 0;
     WinLists wl;
-    if (int rc = get_lists(p, d, code, tl, &wl, st)) return rc;
+    if (get_lists(p, d, code, tl, &wl, st) != 0) { (void)hipGetLastError(); return 0; }
     a.tile_win = wl.d_tile_win; a.win = wl.d_win;
     a.l_item_idx = wl.d_item_idx; a.l_item_pos = wl.d_item_pos; a.l_col_idx = wl.d_col_idx; a.l_col_pos = wl.d_col_pos;
     return 0;
@@ -223,21 +229,22 @@ int conv_fwd_bf16(const aprnet_plan* cp, int d, int kz, int kx, int ky, const bf
     TileList tl;
     if (int rc = get_tiles(p, d, kz == 1 ? 1 : 2, kz == 1 ? 8 : 4, &tl)) return rc;
     if (tl.n == 0) return 0;
-    if (g_bf16_math) {
+    ConvArgs<bf16_t> a{};
+    if (int rc = set_lists(p, d, code, tl, a, st)) return rc;
+    const bool bf16_math = g_bf16_math && a.tile_win;      // the bfloat16 contraction exists with window lists only
+    if (bf16_math) {
         if (int rc = plan_scratch(p, conv_packed_bf16_bytes(code, S_exp, Cout, Cin), st)) return rc;
         if (int rc = pack_conv_weights_bf16(code, w, S_exp, Cout, Cin, p->d_scratch, st)) return rc;
     } else {
         if (int rc = plan_scratch(p, conv_packed_floats(code, S_exp, Cout, Cin, false) * sizeof(float), st)) return rc;
         if (int rc = pack_conv_weights(code, w, S_exp, Cout, Cin, false, (float*)p->d_scratch, st)) return rc;
     }
-    ConvArgs<bf16_t> a{};
     a.apr = p->dapr; a.tree = p->dtree; a.tiles = tl.d_tiles;
     a.x = x; a.ldx = ldx; a.Cin = Cin; a.w = (const float*)p->d_scratch; a.S_exp = S_exp; a.Cout = Cout; a.bias = bias;
     a.y = y; a.ldy = ldy; a.tree_data = tree_ws; a.ldt = ldt; a.Lc = p->lc(d); a.tree_off = p->tree_offset(a.Lc);
     a.x_count = p->number_parts(d); a.t_count = p->tree_parts(d);
-    if (int rc = set_lists(p, d, code, tl, a, st)) return rc;
     TimedLaunch timed(st);
-    return g_bf16_math ? launch_conv_mfma_bf16(code, a, tl.n, st) : launch_conv_mfma(code, a, tl.n, st);
+    return bf16_math ? launch_conv_mfma_bf16(code, a, tl.n, st) : launch_conv_mfma(code, a, tl.n, st);
 }
 
 }  // namespace aprnet
@@ -253,8 +260,10 @@ int aprnet_conv_fwd_bf16(const aprnet_plan* p, int d, int kz, int kx, int ky, co
 }
 int aprnet_set_conv_path(int path) {
     if (path == 2 || path == 3) { g_bf16_math = path == 2; return 0; }
+    if (path == 4 || path == 5) { g_use_lists = path == 4; return 0; }
     if (path != 0 && path != 1)
-        return fail(APRNET_ERR_INVALID_ARGUMENT, "set_conv_path: 0 (auto), 1 (VALU only), 2 / 3 (bfloat16 features: bfloat16 / fp32 matrix math)");
+        return fail(APRNET_ERR_INVALID_ARGUMENT, "set_conv_path: 0 (auto), 1 (VALU only), 2 / 3 (bfloat16 features: bfloat16 / fp32 "
+                                                 "matrix math), 4 / 5 (forward: window lists of the plan / scan per call)");
     g_conv_path = path;
     return 0;
 }

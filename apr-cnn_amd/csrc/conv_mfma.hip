@@ -440,13 +440,16 @@ bool conv_mfma_supported(int code) { return code == 333 || code == 133 || code =
 static int conv_taps(int code) { return code == 333 ? 27 : code == 133 ? 9 : 25; }
 static int conv_coh(int Cm) { return Cm <= 16 ? 1 : 2; }
 
+// a.tile_win set: forward with the window lists of the plan; otherwise the kernel scans (always for the input gradient)
 template <typename T, class G, int MODE>
 static int launch16(const ConvArgs<T>& a, int n_tiles, hipStream_t st) {
     const int coh = conv_coh(a.Cout);
     dim3 grid((unsigned)n_tiles, (unsigned)((a.Cout + 16 * coh - 1) / (16 * coh)));
-    constexpr bool LISTS = MODE == 0;      // forward: precomputed window lists; input gradient: scans
-    if (coh == 1) hipLaunchKernelGGL((conv_mfma16_kernel<T, G, 1, MODE, LISTS>), grid, dim3(G::NT), 0, st, a);
-    else hipLaunchKernelGGL((conv_mfma16_kernel<T, G, 2, MODE, LISTS>), grid, dim3(G::NT), 0, st, a);
+    if (MODE == 0 && a.tile_win) {
+        if (coh == 1) hipLaunchKernelGGL((conv_mfma16_kernel<T, G, 1, 0, true>), grid, dim3(G::NT), 0, st, a);
+        else hipLaunchKernelGGL((conv_mfma16_kernel<T, G, 2, 0, true>), grid, dim3(G::NT), 0, st, a);
+    } else if (coh == 1) hipLaunchKernelGGL((conv_mfma16_kernel<T, G, 1, MODE, false>), grid, dim3(G::NT), 0, st, a);
+    else hipLaunchKernelGGL((conv_mfma16_kernel<T, G, 2, MODE, false>), grid, dim3(G::NT), 0, st, a);
     APRNET_LAUNCH_CHECK("conv_mfma16_kernel");
     return 0;
 }

@@ -78,8 +78,13 @@ void free_lists(WinLists& wl) {
 int get_lists(aprnet_plan* p, int level_delta, int code, const TileList& tl, WinLists* out, hipStream_t st) {
     auto key = std::make_pair(level_delta, code);
     auto it = p->lists.find(key);
-    if (it != p->lists.end()) { *out = it->second; return 0; }
+    if (it != p->lists.end()) {
+        *out = it->second;
+        return it->second.unavailable ? fail(APRNET_ERR_UNSUPPORTED, "window lists are not available for this plan") : 0;
+    }
     WinLists wl{};
+    WinLists none{}; none.unavailable = true;
+    p->lists[key] = none;             // replaced below when the build succeeds
     if (tl.n > 0) {
         ConvArgs<float> a{};
         a.apr = p->dapr; a.tree = p->dtree; a.tiles = tl.d_tiles; a.Lc = p->lc(level_delta); a.tree_off = p->tree_offset(a.Lc);

@@ -80,7 +80,10 @@ int aprnet_profile_enable(int on);
 /* No counterpart in the reference.  Selects the convolution kernels: 0 = matrix-core (MFMA) kernels where one
  * exists for the stencil and element type, VALU kernels otherwise (default); 1 = VALU kernels only.
  * Independently, for bfloat16 features: 2 = bfloat16 matrix instructions (default), 3 = fp32 matrix
- * instructions.  All are HIP kernels; the switch exists so that tests can cover them. */
+ * instructions; and for the forward matrix-core kernels: 4 = take the window lists that the plan builds on first
+ * use and keeps (about 20 bytes of device memory per particle and level delta; default), 5 = scan the access arrays
+ * in every call (also the fallback when the lists cannot be allocated).  All are HIP kernels; the switch exists so
+ * that tests can cover them and memory-bound callers can do without the lists. */
 int aprnet_set_conv_path(int path);
 float aprnet_profile_last_ms(void);
 

@@ -162,6 +162,30 @@ def test_conv333_forward_channel_shapes(cin, cout, path):
     close(got, ref, torch.float32)
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
+@pytest.mark.parametrize("ksize", [(3, 3, 3), (1, 5, 5)], ids=KID)
+def test_conv_forward_without_plan_lists(ksize, dtype):
+    """The forward matrix-core kernels scanning the access arrays per call (the path taken when the plan's
+    window lists are switched off or do not fit) give the same result as with the lists."""
+    x, aprs, ld, w_exp = _conv_case([("3d_s", 0), ("3d_t", 1)], ksize, 2, 12, 20, torch.float32)
+    xd = x.to(dtype).to(DEV)
+    wd = w_exp.permute(1, 2, 0, 3, 4, 5).contiguous().to(DEV)
+    lib = _native.hip()
+    with_lists = _ops.conv_forward(aprs, xd, wd, ld)
+    assert lib.aprnet_set_conv_path(5) == 0
+    try:
+        scanned = _ops.conv_forward(aprs, xd, wd, ld)
+    finally:
+        lib.aprnet_set_conv_path(4)
+    ref = oracle.conv_forward(aprs, xd.float().cpu(), w_exp, ld)
+    if dtype == torch.float32:
+        assert torch.equal(with_lists, scanned)            # same kernel body, same summation order
+        close(scanned, ref, torch.float32)
+    else:
+        close_bf16(scanned, ref)                           # fp32 products here, bfloat16 products with the lists
+        close_bf16(with_lists, ref)
+
+
 def test_conv333_forward_dense_windows():
     """A fully refined APR: every window holds the maximum number of output positions (all four column
     blocks per wave of the matrix-core kernel), plus run-to-run bit equality (no atomics in the forward)."""
