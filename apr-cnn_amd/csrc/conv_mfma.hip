@@ -96,6 +96,11 @@ __device__ __forceinline__ void mfma16_window(const ConvArgs<T>& a, int co0, int
 #pragma unroll
             for (int r = 0; r < 4; ++r) acc[j][h][r] = 0.f;
     const float* ap = Wl + lane;
+    // B operands are read through a volatile LDS pointer: that keeps them single ds_read_b32 with immediate
+    // offsets.  Paired into ds_read2 they need vector adds for their bases inside the matrix loop, and a vector
+    // instruction between two MFMAs costs a pipeline switch; it also keeps the loop within 80 registers.
+    typedef const volatile __attribute__((address_space(3))) float lds_float;
+    lds_float* lpatch = (lds_float*)patch;
 
     constexpr int W4 = KC * 4 * COH;                             // float4 elements of a weight chunk
     constexpr int WPT = (W4 + G::NT - 1) / G::NT;
@@ -132,7 +137,7 @@ __device__ __forceinline__ void mfma16_window(const ConvArgs<T>& a, int co0, int
                 for (int h = 0; h < COH; ++h) av[h] = ap[((t * COH + h) * NSUB + sb) * 64];
 #pragma unroll
                 for (int j = 0; j < NB; ++j) {
-                    const float bv = patch[bbase[j] + 4 * sb * G::CH_STRIDE + tap_offset<G>(t)];
+                    const float bv = lpatch[bbase[j] + 4 * sb * G::CH_STRIDE + tap_offset<G>(t)];
 #pragma unroll
                     for (int h = 0; h < COH; ++h) acc[j][h] = __builtin_amdgcn_mfma_f32_16x16x4f32(av[h], bv, acc[j][h], 0, 0, 0);
                 }
