@@ -157,6 +157,9 @@ static int set_lists(aprnet_plan* p, int d, int code, const TileList& tl, ConvAr
     return 0;
 }
 
+int set_conv_lists(aprnet_plan* p, int d, int code, const TileList& tl, ConvArgs<float>& a, hipStream_t st) { return set_lists(p, d, code, tl, a, st); }
+int set_conv_lists(aprnet_plan* p, int d, int code, const TileList& tl, ConvArgs<bf16_t>& a, hipStream_t st) { return set_lists(p, d, code, tl, a, st); }
+
 template <typename T> static int try_mfma(aprnet_plan*, const ConvArgs<T>&, int, int, const TileList&, int, hipStream_t, bool*) { return 0; }
 template <> int try_mfma<float>(aprnet_plan* p, const ConvArgs<float>& a, int code, int d, const TileList& tl, int n_tiles,
                                 hipStream_t st, bool* done) {

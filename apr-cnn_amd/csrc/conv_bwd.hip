@@ -235,6 +235,9 @@ int fill_tree_for_conv(const aprnet_plan* p, int d, const bf16_t* x, int64_t ldx
 size_t conv_packed_floats(int code, int S_exp, int Cm, int Ck, bool transposed);
 int pack_conv_weights(int code, const float* w, int S_exp, int Cm, int Ck, bool transposed, float* packed, hipStream_t st);
 int conv_path();
+// points a at the plan's window lists (conv.hip); leaves a.tile_win null when they are off or unavailable
+int set_conv_lists(aprnet_plan* p, int d, int code, const TileList& tl, ConvArgs<float>& a, hipStream_t st);
+int set_conv_lists(aprnet_plan* p, int d, int code, const TileList& tl, ConvArgs<bf16_t>& a, hipStream_t st);
 
 template <typename T> static int try_mfma_bwd(aprnet_plan*, const ConvArgs<T>&, const TileList&, int, int, hipStream_t, bool*) { return 0; }
 template <> int try_mfma_bwd<float>(aprnet_plan* p, const ConvArgs<float>& a, const TileList& tl, int code, int d, hipStream_t st, bool* done) {
@@ -251,7 +254,9 @@ template <> int try_mfma_bwd<float>(aprnet_plan* p, const ConvArgs<float>& a, co
     b.x = a.gy; b.ldx = a.ldy; b.Cin = a.Cout; b.Cout = a.Cin; b.w = (const float*)p->d_scratch; b.bias = nullptr;
     b.tree_data = nullptr; b.t_count = 0;
     if (near.n > 0) if (int rc = launch_conv_dx_mfma(code, b, near.n, st)) return rc;
-    return launch_conv_dw_mfma(code, a, tl, p->apr.level_min, st);
+    ConvArgs<float> c = a;
+    if (int rc = set_conv_lists(p, d, code, tl, c, st)) return rc;
+    return launch_conv_dw_mfma(code, c, tl, p->apr.level_min, st);
 }
 
 template <typename T>
@@ -341,6 +346,7 @@ int conv_bwd_bf16(const aprnet_plan* cp, int d, int kz, int kx, int ky, const bf
         b.x = gy; b.ldx = ldy; b.Cin = Cout; b.Cout = Cin; b.w = (const float*)p->d_scratch; b.bias = nullptr;
         b.tree_data = nullptr; b.t_count = 0;
         if (near.n > 0) if (int rc = launch_conv_dx_mfma(code, b, near.n, st)) return rc;
+        if (int rc = set_conv_lists(p, d, code, tl, a, st)) return rc;
         if (int rc = launch_conv_dw_mfma(code, a, tl, p->apr.level_min, st)) return rc;
     }
     if (int rc = fill_tree_bwd_for_conv(p, d, gx32_ws, ldgx32, Cin, gtree_ws, ldgt, st)) return rc;

@@ -32,14 +32,88 @@ constexpr int DW_NCH = 4;          // chunks per block
 constexpr int DW_GB = 256;         // columns of gY staged at a time
 constexpr int DW_GLD = 33;         // words per column of gyl (32 output channels + 1 against bank conflicts)
 
-// T: storage type of the features and of the output gradient (float, or bfloat16 widened to fp32 on load)
-template <typename T, class G, int CIB, int NCH>
+// Lists of the plan carry patch cells for rows of 64 words; this kernel's rows are RS words apart.
+template <class G> __device__ __forceinline__ unsigned restride(unsigned pos) {
+    return (pos & ~ITEM_CELL) | (((pos & ITEM_CELL) >> 6) * G::RS + (pos & 63u));
+}
+
+// One window: its output gradient goes to gyl in groups of DW_GB columns; per group the four channel chunks of
+// the block are staged one after the other (the loads of the next chunk are issued before the matrix phase of
+// the current one) and contracted with the group's columns.
+template <typename T, class G, int CIB, int NCH, bool LISTS, class Lists>
+__device__ __forceinline__ void dw_window(const ConvArgs<T>& a, const Lists& sh, int nc, int nitem, bool tree_items,
+                                          int cig0, int co0, int bl, int kh, int hi, int wave, int lane,
+                                          float* __restrict__ patch, float* __restrict__ gyl, int* __restrict__ cpl,
+                                          const float* ap, floatx16 (&acc)[NCH]) {
+    for (int i = threadIdx.x; i < CIB * G::CH_STRIDE; i += G::NT) patch[i] = 0.f;     // once per window
+    ItemRegs<G, T, CIB> R;
+    fetch_slots<G, T, CIB>(sh, nitem, R);
+    if constexpr (LISTS) {
+#pragma unroll
+        for (int k = 0; k < ItemRegs<G, T, CIB>::IPT; ++k)
+            if (R.pos[k] != 0xffffu) R.pos[k] = (unsigned short)restride<G>(R.pos[k]);
+    }
+    load_values<G, T, CIB>(a, cig0, nitem, tree_items, R);
+    for (int g0 = 0; g0 < nc; g0 += DW_GB) {
+        const int ng = min(DW_GB, nc - g0), nbatch = (ng + 63) >> 6;
+        // output gradient of this group of columns -> gyl; a wave reads 64 columns of one channel
+        for (int b = 0; b < nbatch; ++b) {
+            const int c = b * 64 + lane;
+            const int64_t idx = c < ng ? sh.col_idx[g0 + c] : -1;
+            const int slot = b * 64 + 2 * (lane & 31) + (lane >> 5);
+            if (wave == 0) {        // patch cell of every column of the group, as a word offset
+                int pb = G::TAP0;
+                if (c < ng) pb = LISTS ? (int)restride<G>(sh.col_pos[g0 + c]) : (int)sh.col_pos[g0 + c];
+                cpl[c] = pb;
+            }
+#pragma unroll
+            for (int k = 0; k < 32 / G::NWAVE; ++k) {
+                const int co = wave + k * G::NWAVE;
+                float v = 0.f;
+                if (idx >= 0 && co0 + co < a.Cout) v = Num<T>::ld(a.gy[(int64_t)(co0 + co) * a.ldy + idx]);
+                gyl[slot * DW_GLD + co] = v;
+            }
+        }
+#pragma unroll
+        for (int q = 0; q < NCH; ++q) {
+            __syncthreads();        // previous chunk's reads of the patch are done / gyl is written
+            store_items<G, T, CIB>(R, nitem, patch);
+            __syncthreads();
+            if (q + 1 < NCH) load_values<G, T, CIB>(a, cig0 + (q + 1) * CIB, nitem, tree_items, R);
+            else if (g0 + DW_GB < nc) load_values<G, T, CIB>(a, cig0, nitem, tree_items, R);     // next group starts over
+#pragma unroll 1
+            for (int b = 0; b < nbatch; ++b) {
+                const float* apb = ap + (b * 64 + 32 * kh) * DW_GLD;
+                // Three separate phases, kept apart by scheduling barriers: operand addresses (one LDS read of the
+                // column's cell and one vector add each), then all operand reads, then 16 MFMAs back to back.  A
+                // vector instruction between two fp32 MFMAs costs a pipeline switch each time.
+                const int* cp = cpl + b * 64 + 32 * hi + 16 * kh;      // lanes of the upper half take column k + 32
+                int addr[16];
+#pragma unroll
+                for (int k = 0; k < 16; ++k) addr[k] = bl + cp[k];
+                __builtin_amdgcn_sched_barrier(0);
+                float av[16], bv[16];
+#pragma unroll
+                for (int k = 0; k < 16; ++k) { av[k] = apb[2 * k * DW_GLD]; bv[k] = patch[addr[k]]; }
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int k = 0; k < 16; ++k) acc[q] = __builtin_amdgcn_mfma_f32_32x32x2f32(av[k], bv[k], acc[q], 0, 0, 0);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        }
+        __syncthreads();            // gyl is rewritten by the next group, the patch by the next window
+    }
+}
+
+// T: storage type of the features and of the output gradient (float, or bfloat16 widened to fp32 on load).
+// LISTS: the windows come from the plan's lists; otherwise the block scans the access arrays.
+template <typename T, class G, int CIB, int NCH, bool LISTS>
 __global__ void __launch_bounds__(G::NT) __attribute__((amdgpu_waves_per_eu(4, 4)))
 conv_dw_mfma_kernel(const ConvArgs<T> a, const int s_idx) {
     static_assert(G::NWAVE == 8 && CIB == 4, "wave w owns input channel w%4 and column half w/4");
     __shared__ float patch[CIB * G::CH_STRIDE];
     __shared__ float gyl[DW_GB * DW_GLD];
-    __shared__ ConvShared<G> sh;
+    __shared__ int cpl[DW_GB];
 
     const int cig0 = blockIdx.y * (CIB * NCH), co0 = blockIdx.z * 32;
     const int lane = lane_id();
@@ -59,63 +133,33 @@ conv_dw_mfma_kernel(const ConvArgs<T> a, const int s_idx) {
 
     for (int ti = blockIdx.x; ti < a.n_tiles; ti += gridDim.x) {
         const ConvTile tile = a.tiles[ti];
-        const int L = tile.level, z0 = tile.z0, x0 = tile.x0;
-        const int yn = a.apr.y_num[L];
-        const bool out_tree = (L == a.Lc) && (L < a.apr.level_max);
-
-        __syncthreads();
-        open_segments<G, T>(a, L, z0, x0, sh);
-        __syncthreads();
-
-        for (int y0 = 0; y0 < yn; y0 += G::TY) {
-            scan_window<G, T>(a, L, y0, out_tree, sh);
-            __syncthreads();
-            const int nc = __builtin_amdgcn_readfirstlane(sh.ncol), nitem = __builtin_amdgcn_readfirstlane(sh.nitem);
-            if (nc > 0) {
-                for (int i = threadIdx.x; i < CIB * G::CH_STRIDE; i += G::NT) patch[i] = 0.f;     // once per window
-                for (int g0 = 0; g0 < nc; g0 += DW_GB) {
-                    const int ng = min(DW_GB, nc - g0), nbatch = (ng + 63) >> 6;
-                    // output gradient of this group of columns -> gyl; a wave reads 64 columns of one channel
-                    for (int b = 0; b < nbatch; ++b) {
-                        const int c = b * 64 + lane;
-                        const int64_t idx = c < ng ? sh.col_idx[g0 + c] : -1;
-                        const int slot = b * 64 + 2 * (lane & 31) + (lane >> 5);
-#pragma unroll
-                        for (int k = 0; k < 32 / G::NWAVE; ++k) {
-                            const int co = wave + k * G::NWAVE;
-                            float v = 0.f;
-                            if (idx >= 0 && co0 + co < a.Cout) v = Num<T>::ld(a.gy[(int64_t)(co0 + co) * a.ldy + idx]);
-                            gyl[slot * DW_GLD + co] = v;
-                        }
-                    }
-#pragma unroll
-                    for (int q = 0; q < NCH; ++q) {
-                        __syncthreads();        // previous chunk's reads of the patch are done / gyl is written
-                        stage_values<G, T, CIB>(a, cig0 + q * CIB, nitem, L < a.Lc, sh, patch);
-                        __syncthreads();
-#pragma unroll 1
-                        for (int b = 0; b < nbatch; ++b) {
-                            // cell of column 64 b + lane; broadcast below with readlane
-                            const int c = b * 64 + lane;
-                            const int pb = c < ng ? (int)sh.col_pos[g0 + c] : G::TAP0;
-                            const float* apb = ap + (b * 64 + 32 * kh) * DW_GLD;
-#pragma unroll
-                            for (int k = 0; k < 16; ++k) {
-                                const int kk = kh * 16 + k;
-                                const int p0 = __builtin_amdgcn_readlane(pb, kk);
-                                const int p1 = __builtin_amdgcn_readlane(pb, kk + 32);
-                                const float av = apb[2 * k * DW_GLD];
-                                const float bv = patch[bl + (hi ? p1 : p0)];
-                                acc[q] = __builtin_amdgcn_mfma_f32_32x32x2f32(av, bv, acc[q], 0, 0, 0);
-                            }
-                        }
-                    }
-                    __syncthreads();            // gyl is rewritten by the next group
-                }
+        const int L = tile.level;
+        const bool tree_items = L < a.Lc;
+        if constexpr (LISTS) {
+            const int wb = a.tile_win[ti], we = a.tile_win[ti + 1];
+            for (int w = wb; w < we; ++w) {
+                const int4 hd = a.win[w];
+                const int nitem = __builtin_amdgcn_readfirstlane(hd.y), nc = __builtin_amdgcn_readfirstlane(hd.w);
+                const WindowLists gl{a.l_item_idx + (unsigned)hd.x, a.l_item_pos + (unsigned)hd.x, a.l_col_idx + (unsigned)hd.z,
+                                     a.l_col_pos + (unsigned)hd.z};
+                dw_window<T, G, CIB, NCH, true>(a, gl, nc, nitem, tree_items, cig0, co0, bl, kh, hi, wave, lane, patch, gyl, cpl, ap, acc);
             }
+        } else {
+            __shared__ ConvShared<G> sh;
+            const int yn = a.apr.y_num[L];
+            const bool out_tree = (L == a.Lc) && (L < a.apr.level_max);
             __syncthreads();
-            close_window<G>(sh);
+            open_segments<G, T>(a, L, tile.z0, tile.x0, sh);
             __syncthreads();
+            for (int y0 = 0; y0 < yn; y0 += G::TY) {
+                scan_window<G, T>(a, L, y0, out_tree, sh);
+                __syncthreads();
+                const int nc = __builtin_amdgcn_readfirstlane(sh.ncol), nitem = __builtin_amdgcn_readfirstlane(sh.nitem);
+                if (nc > 0) dw_window<T, G, CIB, NCH, false>(a, sh, nc, nitem, tree_items, cig0, co0, bl, kh, hi, wave, lane, patch, gyl, cpl, ap, acc);
+                __syncthreads();
+                close_window<G>(sh);
+                __syncthreads();
+            }
         }
     }
 #pragma unroll
@@ -143,9 +187,11 @@ static int launch_dw(const ConvArgs<T>& a0, const TileList& tl, int level_min, h
         if (n == 0) continue;
         ConvArgs<T> a = a0;
         a.tiles = tl.d_tiles + tl.level_begin[l_hi]; a.n_tiles = n;
+        if (a.tile_win) a.tile_win += tl.level_begin[l_hi];
         dim3 grid((unsigned)std::min(n, 512), (unsigned)((a.Cin + DW_CIB * DW_NCH - 1) / (DW_CIB * DW_NCH)),
                   (unsigned)((a.Cout + 31) / 32));
-        hipLaunchKernelGGL((conv_dw_mfma_kernel<T, G, DW_CIB, DW_NCH>), grid, dim3(G::NT), 0, st, a, s);
+        if (a.tile_win) hipLaunchKernelGGL((conv_dw_mfma_kernel<T, G, DW_CIB, DW_NCH, true>), grid, dim3(G::NT), 0, st, a, s);
+        else hipLaunchKernelGGL((conv_dw_mfma_kernel<T, G, DW_CIB, DW_NCH, false>), grid, dim3(G::NT), 0, st, a, s);
         APRNET_LAUNCH_CHECK("conv_dw_mfma_kernel");
     }
     return 0;
