@@ -94,6 +94,7 @@ struct ConvShared {
     int item_idx[G::MAXITEM];
     unsigned short item_pos[G::MAXITEM];   // bits 0-11 cell inside one channel of the patch, ITEM_PAIR, ITEM_TREE
     int ncol, nitem;
+    int nbox;                        // input gradient: pooled columns (COL_BOX) of the window
 };
 
 constexpr unsigned ITEM_CELL = 0x0fffu;   // first patch cell the value goes to
@@ -127,7 +128,7 @@ __device__ __forceinline__ void open_segments(const ConvArgs<T>& a, int L, int z
         }
         sh.seg_cur[s] = b; sh.seg_end[s] = e;
     }
-    if (threadIdx.x == 0) { sh.ncol = 0; sh.nitem = 0; }
+    if (threadIdx.x == 0) { sh.ncol = 0; sh.nitem = 0; sh.nbox = 0; }
 }
 
 // Segments are scanned in groups of GRP: the y_vec loads of a group are issued before the first LDS
@@ -146,6 +147,7 @@ struct ScanArgs {
     const uint16_t* tree_y;
     int tree_off, yn, y0;
     bool tree_from_x, out_tree;
+    int z0, x0, zn, xn;             // tile origin and level extent (input-gradient scan only)
 };
 
 template <class G>
@@ -234,9 +236,14 @@ __device__ __attribute__((noinline)) void scan_window_impl(const ScanArgs a, Con
 //   items    the output positions of the window including the halo rows: same-level particles, and tree
 //            nodes where they are downsampled particles;  idx addresses the output gradient
 //   columns  every cell of the centre rows that some source covers, with the place its gradient goes to:
-//            the same-level particle, the coarser particle behind two cells (one column per cell), the
-//            downsampled particle, or (COL_TREE) the node of the tree-gradient buffer
+//            the same-level particle, the coarser particle, the downsampled particle, or (COL_TREE) the node
+//            of the tree-gradient buffer.  A coarser particle collects the gradients of the BOXZ x 2 x 2 cells
+//            it covers inside the tile; by linearity that sum is the stencil applied to the box-summed output
+//            gradient, so it takes ONE column (COL_BOX, at its first cell) that reads a second patch holding
+//            those box sums.  Only at the far faces of the image, where some of the cells do not exist, it
+//            takes one column per cell.
 constexpr unsigned COL_CELL = 0x0fffu;
+constexpr unsigned COL_BOX = 0x4000u;
 constexpr unsigned COL_TREE = 0x8000u;
 
 template <class G>
@@ -300,18 +307,29 @@ __device__ __attribute__((noinline)) void scan_window_dx_impl(const ScanArgs a, 
                     }
                 }
             } else {
+                constexpr int BOXZ = G::TZ >= 2 ? 2 : 1;         // a flat tile sees one z-slice of the coarser particle
+                const int z = a.z0 - G::HZ + rz, x = a.x0 - G::HX + rx;
                 const int ya = 2 * yy[g], yb = ya + 1;
-                const bool oa = in && ya >= y0 && ya < y0 + G::TY;
-                const bool ob = in && yb >= y0 && yb < y0 + G::TY && yb < yn;
+                // all cells of the coarser particle inside this tile exist (wave-uniform in z and x)
+                const bool rows_full = (BOXZ == 1 || (z | 1) < a.zn) && (x | 1) < a.xn;
+                const bool first_row = (BOXZ == 1 || (z & 1) == 0) && (x & 1) == 0;
+                const bool ina = in && ya >= y0 && ya < y0 + G::TY;
+                const bool pooled = rows_full && yb < yn;
+                const bool oa = ina && (!pooled || first_row);
+                const bool ob = in && !pooled && yb >= y0 && yb < y0 + G::TY && yb < yn;
                 const unsigned long long ma = __ballot(oa), mb = __ballot(ob);
                 if (ma | mb) {
                     int base = 0;
-                    if (lane == 0) base = atomicAdd(&sh.ncol, __popcll(ma) + __popcll(mb));
+                    const int n_pooled = __popcll(__ballot(oa && pooled));
+                    if (lane == 0) {
+                        base = atomicAdd(&sh.ncol, __popcll(ma) + __popcll(mb));
+                        if (n_pooled) atomicAdd(&sh.nbox, n_pooled);
+                    }
                     base = __shfl(base, 0);
                     if (oa) {
                         const int rank = __popcll(ma & below_me);
                         sh.col_idx[base + rank] = i;
-                        sh.col_pos[base + rank] = (unsigned short)(r * G::RS + (ya - lo));
+                        sh.col_pos[base + rank] = (unsigned short)((r * G::RS + (ya - lo)) | (pooled ? COL_BOX : 0u));
                     }
                     if (ob) {
                         const int rank = __popcll(ma) + __popcll(mb & below_me);
@@ -325,17 +343,19 @@ __device__ __attribute__((noinline)) void scan_window_dx_impl(const ScanArgs a, 
 }
 
 template <class G, typename T>
-__device__ __forceinline__ void scan_window_dx(const ConvArgs<T>& a, int L, int y0, bool out_tree, ConvShared<G>& sh) {
+__device__ __forceinline__ void scan_window_dx(const ConvArgs<T>& a, int L, int z0, int x0, int y0, bool out_tree,
+                                               ConvShared<G>& sh) {
     ScanArgs s;
     s.apr_y = a.apr.y; s.tree_y = a.tree.y; s.tree_off = (int)a.tree_off; s.yn = a.apr.y_num[L]; s.y0 = y0;
     s.tree_from_x = (L == a.Lc); s.out_tree = out_tree;
+    s.z0 = z0; s.x0 = x0; s.zn = a.apr.z_num[L]; s.xn = a.apr.x_num[L];
     scan_window_dx_impl<G>(s, sh);
 }
 
 // End of a window: reset the list lengths (call between two barriers).
 template <class G>
 __device__ __forceinline__ void close_window(ConvShared<G>& sh) {
-    if (threadIdx.x == 0) { sh.ncol = 0; sh.nitem = 0; }
+    if (threadIdx.x == 0) { sh.ncol = 0; sh.nitem = 0; sh.nbox = 0; }
 }
 
 // Buffer loads: the channel plane is described by a wave-uniform resource (base, size in bytes), the lane

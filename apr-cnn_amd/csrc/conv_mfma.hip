@@ -85,8 +85,9 @@ __device__ __forceinline__ void mfma16_window(const ConvArgs<T>& a, int co0, int
 #pragma unroll
     for (int j = 0; j < NB; ++j) {
         const int col = ((first + G::NWAVE * j) << 4) + (lane & 15);
-        const int pos = col < nc ? (int)(sh.col_pos[col] & COL_CELL) - G::TAP0 : 0;
-        bbase[j] = pos + (lane >> 4) * G::CH_STRIDE;
+        const unsigned cp = col < nc ? (unsigned)sh.col_pos[col] : (unsigned)G::TAP0;
+        // pooled columns of the input gradient read the box-summed patch that follows the patch in LDS
+        bbase[j] = (int)(cp & COL_CELL) - G::TAP0 + (lane >> 4) * G::CH_STRIDE + ((MODE == 1 && (cp & COL_BOX)) ? CIB * G::CH_STRIDE : 0);
     }
     floatx4 acc[NBA][COH];
 #pragma unroll
@@ -127,6 +128,34 @@ __device__ __forceinline__ void mfma16_window(const ConvArgs<T>& a, int co0, int
         if (ci0 + CIB < a.Cin) {
             load_values<G, T, CIB>(a, ci0 + CIB, nitem, tree_items, R);
             APRNET_LOAD_WEIGHTS(ci0 / CIB + 1)
+        }
+        if constexpr (MODE == 1) {
+            // Box sums over the cells of a coarser particle, for the pooled columns.  One wave per task
+            // (channel, pair of z rows, part of the x range), one lane per y: the sums over y and z of every x
+            // row are formed in registers, neighbouring x rows added, so each cell is read once per task.
+            if (sh.nbox > 0) {
+                constexpr int BOXZ = G::TZ >= 2 ? 2 : 1;
+                constexpr int NZP = G::RZ - (BOXZ - 1);                 // first z rows of a box
+                constexpr int XP = BOXZ == 1 ? 2 : 1, XW = (G::RX - 1 + XP - 1) / XP;      // x rows of boxes per task
+                float* box = patch + CIB * G::CH_STRIDE;
+                for (int task = threadIdx.x >> 6; task < CIB * NZP * XP; task += G::NWAVE) {
+                    const int c = task / (NZP * XP), zp = (task / XP) % NZP, xb = (task % XP) * XW;
+                    const float* p = patch + c * G::CH_STRIDE + (zp * G::RX + xb) * G::RS + lane;
+                    float* q = box + c * G::CH_STRIDE + (zp * G::RX + xb) * G::RS + lane;
+                    if (lane < G::RS - 1 && lane < 63) {
+                        float prev = 0.f;
+#pragma unroll
+                        for (int x = 0; x <= XW; ++x) {
+                            if (xb + x >= G::RX) break;
+                            float s = p[x * G::RS] + p[x * G::RS + 1];
+                            if (BOXZ == 2) s += p[(G::RX + x) * G::RS] + p[(G::RX + x) * G::RS + 1];
+                            if (x > 0) q[(x - 1) * G::RS] = prev + s;
+                            prev = s;
+                        }
+                    }
+                }
+                __syncthreads();
+            }
         }
 #pragma unroll
         for (int t = 0; t < G::K; ++t) {
@@ -182,10 +211,9 @@ __global__ void __launch_bounds__(G::NT)
 __attribute__((amdgpu_waves_per_eu(LISTS ? FWD_WAVES : DX_WAVES, LISTS ? FWD_WAVES : DX_WAVES)))
 conv_mfma16_kernel(const ConvArgs<T> a) {
     constexpr int CIB = LISTS ? FWD_CIB : DX_CIB, NBW = 4;
-    static_assert((G::NWAVE & (G::NWAVE - 1)) == 0, "block rotation assumes a power-of-two wave count");
     static_assert((G::MAXCOL + 15) / 16 <= G::NWAVE * NBW, "a window must fit the accumulators of the block");
     static_assert(G::CH_STRIDE % 64 == 16, "four lane groups read four channels: a quarter of the banks each");
-    __shared__ float patch[CIB * G::CH_STRIDE];
+    __shared__ float patch[(MODE == 1 ? 2 : 1) * CIB * G::CH_STRIDE];      // input gradient: patch + box sums
     __shared__ __attribute__((aligned(16))) float Wl[CIB * G::K * 16 * COH];
     __shared__ float bias_l[16 * COH];
 
@@ -208,7 +236,7 @@ conv_mfma16_kernel(const ConvArgs<T> a) {
     {                                                                                                                     \
         const int nblk = (nc + 15) >> 4;                                                                                  \
         /* rotation: spread the waves that own one block more over the SIMDs */                                           \
-        const int first = (wave - (int)blockIdx.x - win) & (G::NWAVE - 1);                                                \
+        const int first = (wave + G::NWAVE - (int)((blockIdx.x + win) % G::NWAVE)) % G::NWAVE;                            \
         const int nb = first < nblk ? (nblk - first + G::NWAVE - 1) / G::NWAVE : 0;                                       \
         switch (__builtin_amdgcn_readfirstlane(nb)) {                                                                     \
             case 0: mfma16_window<T, G, CIB, COH, 0, MODE>(a, co0, nc, nitem, tree_items, first, wl, LISTS_OBJ, patch, Wl, bias_l); break; \
@@ -237,7 +265,7 @@ conv_mfma16_kernel(const ConvArgs<T> a) {
         int win = 0;
         for (int y0 = 0; y0 < yn; y0 += G::TY, ++win) {
             if constexpr (MODE == 0) scan_window<G, T>(a, L, y0, out_tree, sh);
-            else scan_window_dx<G, T>(a, L, y0, out_tree, sh);
+            else scan_window_dx<G, T>(a, L, z0, x0, y0, out_tree, sh);
             __syncthreads();
             const int nc = __builtin_amdgcn_readfirstlane(sh.ncol), nitem = __builtin_amdgcn_readfirstlane(sh.nitem);
             if (nc > 0 && nitem > 0) APRNET_WINDOW(sh)
@@ -439,6 +467,9 @@ conv_mfma_bf16_kernel(const ConvArgs<bf16_t> a) {
 using M333N = ConvGeom<3, 3, 3, 2, 4, 512, 64, 16>;
 using M133N = ConvGeom<1, 3, 3, 1, 8, 512, 64, 16>;
 using M155N = ConvGeom<1, 5, 5, 1, 8, 512, 64, 16>;
+// input gradient of the 3x3x3 stencil: the second patch (box sums) leaves room for two workgroups per CU, so
+// each gets 12 waves
+using D333N = ConvGeom<3, 3, 3, 2, 4, 768, 64, 16>;
 
 // stencils with a matrix-core kernel (kz*100 + kx*10 + ky); 5x5x5 needs a weight chunk that does not fit LDS
 bool conv_mfma_supported(int code) { return code == 333 || code == 133 || code == 155; }
@@ -461,7 +492,9 @@ static int launch16(const ConvArgs<T>& a, int n_tiles, hipStream_t st) {
 template <typename T, int MODE>
 static int launch16_code(int code, const ConvArgs<T>& a, int n_tiles, hipStream_t st) {
     switch (code) {
-        case 333: return launch16<T, M333N, MODE>(a, n_tiles, st);
+        case 333:
+            if constexpr (MODE == 1) return launch16<T, D333N, MODE>(a, n_tiles, st);
+            else return launch16<T, M333N, MODE>(a, n_tiles, st);
         case 133: return launch16<T, M133N, MODE>(a, n_tiles, st);
         case 155: return launch16<T, M155N, MODE>(a, n_tiles, st);
     }
