@@ -30,7 +30,14 @@ class BasicBlock(nn.Module):
         self.norm = _make_norm(norm, out_channels, num_groups, bn_momentum)
         self.activation = activation if isinstance(activation, nn.Module) else activation()
 
-    def forward(self, x, aprs, level_deltas):
+    def forward(self, x, aprs, level_deltas, x2=None):
+        """x2: optional second input whose channels follow those of x (the concatenation of UpConv)."""
+        # Inference with the norm folded away: ReLU and the concatenation are done inside the convolution kernel
+        if (not torch.is_grad_enabled() and isinstance(self.norm, nn.Identity) and type(self.activation) is nn.ReLU
+                and x.is_cuda):
+            return self.conv.forward_fused(x, aprs, level_deltas, relu=True, second_input=x2)
+        if x2 is not None:
+            x = torch.cat([x, x2], dim=1)
         return self.activation(self.norm(self.conv(x, aprs, level_deltas)))
 
 
@@ -44,9 +51,9 @@ class ConvBlock(nn.Module):
             BasicBlock(widths[i], widths[i + 1], nstencils=nstencils, kernel_size=kernel_size, activation=activation,
                        num_groups=num_groups, norm=norm, bn_momentum=bn_momentum) for i in range(num_blocks))
 
-    def forward(self, x, aprs, level_deltas):
-        for block in self.blocks:
-            x = block(x, aprs, level_deltas)
+    def forward(self, x, aprs, level_deltas, x2=None):
+        for i, block in enumerate(self.blocks):
+            x = block(x, aprs, level_deltas, x2 if i == 0 else None)
         return x
 
 
@@ -82,4 +89,4 @@ class UpConv(nn.Module):
     def forward(self, x1, x2, aprs, level_deltas):
         x1 = self.reduce_ch(x1, aprs, level_deltas)
         x1 = self.upsample(x1, aprs, level_deltas)
-        return self.conv(torch.cat([x2, x1], dim=1), aprs, level_deltas)
+        return self.conv(x2, aprs, level_deltas, x1)          # = conv(torch.cat([x2, x1], dim=1)), unet_parts.py:82

@@ -81,8 +81,11 @@ conv_fwd_kernel(const ConvArgs<T> a) {
                 const int64_t o = sh.col_idx[col];
 #pragma unroll
                 for (int co = 0; co < COB; ++co)
-                    if (co0 + co < a.Cout)
-                        a.y[(int64_t)(co0 + co) * a.ldy + o] = acc[it][co] + (a.bias ? a.bias[co0 + co] : (T)0);
+                    if (co0 + co < a.Cout) {
+                        T v = acc[it][co] + (a.bias ? a.bias[co0 + co] : (T)0);
+                        if (a.relu) v = v < (T)0 ? (T)0 : v;
+                        a.y[(int64_t)(co0 + co) * a.ldy + o] = v;
+                    }
             }
         }
         __syncthreads();
@@ -178,20 +181,40 @@ template <> int try_mfma<float>(aprnet_plan* p, const ConvArgs<float>& a, int co
 int fill_tree_for_conv(const aprnet_plan* p, int d, const float* x, int64_t ldx, int C, float* tree, int64_t ldt, hipStream_t st);
 int fill_tree_for_conv(const aprnet_plan* p, int d, const double* x, int64_t ldx, int C, double* tree, int64_t ldt, hipStream_t st);
 
+// Optional parts of the fused forward entry points: a second input tensor whose C2 channels follow the Cin of x
+// in the contraction, and a clamp at zero of the result.
 template <typename T>
-int conv_fwd(const aprnet_plan* cp, int d, int kz, int kx, int ky, const T* x, int64_t ldx, int Cin, const T* w,
-             int S_exp, int Cout, const T* bias, T* y, int64_t ldy, T* tree_ws, int64_t ldt, hipStream_t st) {
+struct Fusion {
+    const T* x2 = nullptr; int64_t ldx2 = 0; int C2 = 0; int relu = 0;
+};
+template <typename T>
+static int read_fusion(const aprnet_conv_fusion* f, Fusion<T>* out) {
+    *out = Fusion<T>{};
+    if (!f) return 0;
+    if (f->C2 < 0 || (f->C2 > 0 && !f->x2)) return fail(APRNET_ERR_INVALID_ARGUMENT, "conv_forward: second input without data");
+    if (f->C2 > 0) { out->x2 = (const T*)f->x2; out->ldx2 = f->ldx2; out->C2 = f->C2; }
+    out->relu = f->relu != 0;
+    return 0;
+}
+
+template <typename T>
+int conv_fwd(const aprnet_plan* cp, int d, int kz, int kx, int ky, const T* x, int64_t ldx, int C1, const T* w,
+             int S_exp, int Cout, const T* bias, T* y, int64_t ldy, T* tree_ws, int64_t ldt, hipStream_t st,
+             const Fusion<T>& fu = Fusion<T>{}) {
     aprnet_plan* p = const_cast<aprnet_plan*>(cp);
     if (int rc = check_level_delta(p, d, "conv_forward")) return rc;
     if (int rc = check_plane_size(p, d, sizeof(*x), "conv_forward")) return rc;
-    if (Cin <= 0 || Cout <= 0 || S_exp <= 0) return fail(APRNET_ERR_INVALID_ARGUMENT, "conv_forward: empty channel / stencil count");
+    const int Cin = C1 + fu.C2;
+    if (C1 <= 0 || Cout <= 0 || S_exp <= 0) return fail(APRNET_ERR_INVALID_ARGUMENT, "conv_forward: empty channel / stencil count");
     const int code = kz * 100 + kx * 10 + ky;
     if (code != 333 && code != 133 && code != 155 && code != 555)
         return fail(APRNET_ERR_UNSUPPORTED, "conv_forward: stencil must be 333, 133, 155 or 555");
     const int64_t nt = p->tree_parts(d);
     if (nt > 0 && (!tree_ws || ldt < nt)) return fail(APRNET_ERR_INVALID_ARGUMENT, "conv_forward: tree work space too small");
     APRNET_HIP_CHECK(hipSetDevice(p->device));
-    if (int rc = fill_tree_for_conv(p, d, x, ldx, Cin, tree_ws, ldt, st)) return rc;
+    if (int rc = fill_tree_for_conv(p, d, x, ldx, C1, tree_ws, ldt, st)) return rc;
+    if (fu.C2 > 0)
+        if (int rc = fill_tree_for_conv(p, d, fu.x2, fu.ldx2, fu.C2, tree_ws + (int64_t)C1 * ldt, ldt, st)) return rc;
     const bool flat = (kz == 1);
     TileList tl;
     if (int rc = get_tiles(p, d, flat ? 1 : 2, flat ? 8 : 4, &tl)) return rc;
@@ -199,6 +222,7 @@ int conv_fwd(const aprnet_plan* cp, int d, int kz, int kx, int ky, const T* x, i
     ConvArgs<T> a{};
     a.apr = p->dapr; a.tree = p->dtree; a.tiles = tl.d_tiles;
     a.x = x; a.ldx = ldx; a.Cin = Cin; a.w = w; a.S_exp = S_exp; a.Cout = Cout; a.bias = bias; a.y = y; a.ldy = ldy;
+    a.x2 = fu.x2; a.ldx2 = fu.ldx2; a.c_split = C1; a.relu = fu.relu;
     a.tree_data = tree_ws; a.ldt = ldt; a.Lc = p->lc(d); a.tree_off = p->tree_offset(a.Lc);
     a.x_count = p->number_parts(d); a.t_count = p->tree_parts(d);
     bool done = false;
@@ -216,19 +240,23 @@ int conv_fwd(const aprnet_plan* cp, int d, int kz, int kx, int ky, const T* x, i
 }
 
 // bfloat16 features, fp32 weights and bias, fp32 arithmetic: 3x3x3 on the matrix cores only
-int conv_fwd_bf16(const aprnet_plan* cp, int d, int kz, int kx, int ky, const bf16_t* x, int64_t ldx, int Cin, const float* w,
-                  int S_exp, int Cout, const float* bias, bf16_t* y, int64_t ldy, bf16_t* tree_ws, int64_t ldt, hipStream_t st) {
+int conv_fwd_bf16(const aprnet_plan* cp, int d, int kz, int kx, int ky, const bf16_t* x, int64_t ldx, int C1, const float* w,
+                  int S_exp, int Cout, const float* bias, bf16_t* y, int64_t ldy, bf16_t* tree_ws, int64_t ldt, hipStream_t st,
+                  const Fusion<bf16_t>& fu = Fusion<bf16_t>{}) {
     aprnet_plan* p = const_cast<aprnet_plan*>(cp);
     if (int rc = check_level_delta(p, d, "conv_forward")) return rc;
     if (int rc = check_plane_size(p, d, sizeof(*x), "conv_forward")) return rc;
-    if (Cin <= 0 || Cout <= 0 || S_exp <= 0) return fail(APRNET_ERR_INVALID_ARGUMENT, "conv_forward: empty channel / stencil count");
+    const int Cin = C1 + fu.C2;
+    if (C1 <= 0 || Cout <= 0 || S_exp <= 0) return fail(APRNET_ERR_INVALID_ARGUMENT, "conv_forward: empty channel / stencil count");
     const int code = kz * 100 + kx * 10 + ky;
     if (!conv_mfma_supported(code))
         return fail(APRNET_ERR_UNSUPPORTED, "conv_forward: bfloat16 features are supported for the 3x3x3, 1x3x3 and 1x5x5 stencils");
     const int64_t nt = p->tree_parts(d);
     if (nt > 0 && (!tree_ws || ldt < nt)) return fail(APRNET_ERR_INVALID_ARGUMENT, "conv_forward: tree work space too small");
     APRNET_HIP_CHECK(hipSetDevice(p->device));
-    if (int rc = fill_tree_for_conv(p, d, x, ldx, Cin, tree_ws, ldt, st)) return rc;
+    if (int rc = fill_tree_for_conv(p, d, x, ldx, C1, tree_ws, ldt, st)) return rc;
+    if (fu.C2 > 0)
+        if (int rc = fill_tree_for_conv(p, d, fu.x2, fu.ldx2, fu.C2, tree_ws + (int64_t)C1 * ldt, ldt, st)) return rc;
     TileList tl;
     if (int rc = get_tiles(p, d, kz == 1 ? 1 : 2, kz == 1 ? 8 : 4, &tl)) return rc;
     if (tl.n == 0) return 0;
@@ -244,11 +272,16 @@ int conv_fwd_bf16(const aprnet_plan* cp, int d, int kz, int kx, int ky, const bf
     }
     a.apr = p->dapr; a.tree = p->dtree; a.tiles = tl.d_tiles;
     a.x = x; a.ldx = ldx; a.Cin = Cin; a.w = (const float*)p->d_scratch; a.S_exp = S_exp; a.Cout = Cout; a.bias = bias;
+    a.x2 = fu.x2; a.ldx2 = fu.ldx2; a.c_split = C1; a.relu = fu.relu;
     a.y = y; a.ldy = ldy; a.tree_data = tree_ws; a.ldt = ldt; a.Lc = p->lc(d); a.tree_off = p->tree_offset(a.Lc);
     a.x_count = p->number_parts(d); a.t_count = p->tree_parts(d);
     TimedLaunch timed(st);
     return bf16_math ? launch_conv_mfma_bf16(code, a, tl.n, st) : launch_conv_mfma(code, a, tl.n, st);
 }
+
+int conv111_fwd_relu(const aprnet_plan*, int, const float*, int64_t, int, const float*, int, int, const float*, float*, int64_t, hipStream_t, int);
+int conv111_fwd_relu(const aprnet_plan*, int, const double*, int64_t, int, const double*, int, int, const double*, double*, int64_t, hipStream_t, int);
+int conv111_fwd_relu(const aprnet_plan*, int, const bf16_t*, int64_t, int, const float*, int, int, const float*, bf16_t*, int64_t, hipStream_t, int);
 
 }  // namespace aprnet
 
@@ -260,6 +293,36 @@ int aprnet_conv_fwd_bf16(const aprnet_plan* p, int d, int kz, int kx, int ky, co
                          int64_t ldt, void* st) {
     return conv_fwd_bf16(p, d, kz, kx, ky, (const bf16_t*)x, ldx, Cin, w, S_exp, Cout, bias, (bf16_t*)y, ldy, (bf16_t*)tree_ws,
                          ldt, (hipStream_t)st);
+}
+#define APRNET_FUSED_111(T)                                                                                              \
+    if (kz == 1 && kx == 1 && ky == 1) {                                                                                 \
+        if (fu.C2 > 0) return fail(APRNET_ERR_UNSUPPORTED, "conv_forward: the 1x1x1 convolution takes a single input");  \
+        return conv111_fwd_relu(p, d, (const T*)x, ldx, Cin, w, S_exp, Cout, bias, (T*)y, ldy, (hipStream_t)st, fu.relu); \
+    }
+int aprnet_conv_fwd_fused_bf16(const aprnet_plan* p, int d, int kz, int kx, int ky, const uint16_t* x, int64_t ldx, int Cin,
+                               const float* w, int S_exp, int Cout, const float* bias, uint16_t* y, int64_t ldy,
+                               uint16_t* tree_ws, int64_t ldt, const aprnet_conv_fusion* fusion, void* st) {
+    Fusion<bf16_t> fu;
+    if (int rc = read_fusion(fusion, &fu)) return rc;
+    APRNET_FUSED_111(bf16_t)
+    return conv_fwd_bf16(p, d, kz, kx, ky, (const bf16_t*)x, ldx, Cin, w, S_exp, Cout, bias, (bf16_t*)y, ldy, (bf16_t*)tree_ws,
+                         ldt, (hipStream_t)st, fu);
+}
+int aprnet_conv_fwd_fused_f32(const aprnet_plan* p, int d, int kz, int kx, int ky, const float* x, int64_t ldx, int Cin,
+                              const float* w, int S_exp, int Cout, const float* bias, float* y, int64_t ldy, float* tree_ws,
+                              int64_t ldt, const aprnet_conv_fusion* fusion, void* st) {
+    Fusion<float> fu;
+    if (int rc = read_fusion(fusion, &fu)) return rc;
+    APRNET_FUSED_111(float)
+    return conv_fwd<float>(p, d, kz, kx, ky, x, ldx, Cin, w, S_exp, Cout, bias, y, ldy, tree_ws, ldt, (hipStream_t)st, fu);
+}
+int aprnet_conv_fwd_fused_f64(const aprnet_plan* p, int d, int kz, int kx, int ky, const double* x, int64_t ldx, int Cin,
+                              const double* w, int S_exp, int Cout, const double* bias, double* y, int64_t ldy, double* tree_ws,
+                              int64_t ldt, const aprnet_conv_fusion* fusion, void* st) {
+    Fusion<double> fu;
+    if (int rc = read_fusion(fusion, &fu)) return rc;
+    APRNET_FUSED_111(double)
+    return conv_fwd<double>(p, d, kz, kx, ky, x, ldx, Cin, w, S_exp, Cout, bias, y, ldy, tree_ws, ldt, (hipStream_t)st, fu);
 }
 int aprnet_set_conv_path(int path) {
     if (path == 2 || path == 3) { g_bf16_math = path == 2; return 0; }

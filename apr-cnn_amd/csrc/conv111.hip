@@ -13,7 +13,8 @@ constexpr int TB1 = 256;
 template <typename T, int OB>
 __global__ void __launch_bounds__(TB1)
 conv111_kernel(const T* __restrict__ src, int64_t lds, int Csrc, const T* __restrict__ w, int so, int sc,
-               const T* __restrict__ bias, T* __restrict__ dst, int64_t ldd, int Cdst, int64_t begin, int64_t end) {
+               const T* __restrict__ bias, T* __restrict__ dst, int64_t ldd, int Cdst, int64_t begin, int64_t end,
+               int relu) {
     const int64_t i = begin + (int64_t)blockIdx.x * TB1 + threadIdx.x;
     if (i >= end) return;
     const int o0 = blockIdx.y * OB;
@@ -35,7 +36,11 @@ conv111_kernel(const T* __restrict__ src, int64_t lds, int Csrc, const T* __rest
     }
 #pragma unroll
     for (int o = 0; o < OB; ++o)
-        if (o0 + o < Cdst) dst[(int64_t)(o0 + o) * ldd + i] = acc[o] + (bias ? bias[o0 + o] : (T)0);
+        if (o0 + o < Cdst) {
+            T v = acc[o] + (bias ? bias[o0 + o] : (T)0);
+            if (relu) v = v < (T)0 ? (T)0 : v;
+            dst[(int64_t)(o0 + o) * ldd + i] = v;
+        }
 }
 
 // The same product on the matrix cores (fp32): M = 32 outputs, N = 32 positions, K = input channels two at a
@@ -49,7 +54,7 @@ template <typename T, int KP>      // KP = channel pairs held in registers (ceil
 __global__ void __launch_bounds__(TB1)
 conv111_mfma_kernel(const T* __restrict__ src, int64_t lds, int Csrc, const float* __restrict__ w, int so, int sc,
                     const float* __restrict__ bias, T* __restrict__ dst, int64_t ldd, int Cdst, int64_t begin,
-                    int64_t end) {
+                    int64_t end, int relu) {
     const int lane = threadIdx.x & 63, hi = lane >> 5, col = lane & 31;
     const int o0 = blockIdx.y * 32;
     float aw[KP];
@@ -88,8 +93,10 @@ conv111_mfma_kernel(const T* __restrict__ src, int64_t lds, int Csrc, const floa
         for (int r = 0; r < 16; ++r) {
             const int o = o0 + 8 * (r >> 2) + 4 * hi + (r & 3);
             if (o < Cdst) {
-                if (ia < end) dst[(int64_t)o * ldd + ia] = Num<T>::st(acca[r]);
-                if (ib < end) dst[(int64_t)o * ldd + ib] = Num<T>::st(accb[r]);
+                float ya = acca[r], yb = accb[r];
+                if (relu) { ya = ya < 0.f ? 0.f : ya; yb = yb < 0.f ? 0.f : yb; }
+                if (ia < end) dst[(int64_t)o * ldd + ia] = Num<T>::st(ya);
+                if (ib < end) dst[(int64_t)o * ldd + ib] = Num<T>::st(yb);
             }
         }
     }
@@ -98,12 +105,12 @@ conv111_mfma_kernel(const T* __restrict__ src, int64_t lds, int Csrc, const floa
 // dispatch on the number of channel pairs kept in registers; false when the layer is too wide for this kernel
 template <typename T>
 static bool launch_conv111_mfma(const T* src, int64_t lds, int Csrc, const float* w, int so, int sc, const float* bias,
-                                T* dst, int64_t ldd, int Cdst, int64_t begin, int64_t end, hipStream_t st) {
+                                T* dst, int64_t ldd, int Cdst, int64_t begin, int64_t end, hipStream_t st, int relu = 0) {
     const int kp = (Csrc + 1) / 2;
     const int64_t n = end - begin;
     dim3 grid((unsigned)std::min<int64_t>((n + 255) / 256, 256 * 8), (unsigned)((Cdst + 31) / 32));
 #define APRNET_111(KP) hipLaunchKernelGGL((conv111_mfma_kernel<T, KP>), grid, dim3(TB1), 0, st, src, lds, Csrc, w, so, sc, bias, \
-                                          dst, ldd, Cdst, begin, end)
+                                          dst, ldd, Cdst, begin, end, relu)
     if (kp <= 8) APRNET_111(8);
     else if (kp <= 16) APRNET_111(16);
     else if (kp <= 32) APRNET_111(32);
@@ -113,15 +120,16 @@ static bool launch_conv111_mfma(const T* src, int64_t lds, int Csrc, const float
     return true;
 }
 template <typename T>
-static bool try_conv111_mfma(const T*, int64_t, int, const T*, int, int, const T*, T*, int64_t, int, int64_t, int64_t, hipStream_t) {
+static bool try_conv111_mfma(const T*, int64_t, int, const T*, int, int, const T*, T*, int64_t, int, int64_t, int64_t, hipStream_t,
+                             int = 0) {
     return false;
 }
 int conv_path();
 template <>
 bool try_conv111_mfma<float>(const float* src, int64_t lds, int Csrc, const float* w, int so, int sc, const float* bias,
-                             float* dst, int64_t ldd, int Cdst, int64_t begin, int64_t end, hipStream_t st) {
+                             float* dst, int64_t ldd, int Cdst, int64_t begin, int64_t end, hipStream_t st, int relu) {
     if (conv_path() == 1) return false;
-    return launch_conv111_mfma<float>(src, lds, Csrc, w, so, sc, bias, dst, ldd, Cdst, begin, end, st);
+    return launch_conv111_mfma<float>(src, lds, Csrc, w, so, sc, bias, dst, ldd, Cdst, begin, end, st, relu);
 }
 
 // gw[co][ci] += sum_i gy[co][i] * x[ci][i] over [begin, end): 8x8 register tile per thread, block
@@ -188,22 +196,22 @@ static std::vector<Segment> segments(const aprnet_plan* p, int d, int S) {
 
 template <typename T>
 int conv111_fwd(const aprnet_plan* p, int d, const T* x, int64_t ldx, int Cin, const T* w, int S, int Cout,
-                const T* bias, T* y, int64_t ldy, hipStream_t st) {
+                const T* bias, T* y, int64_t ldy, hipStream_t st, int relu) {
     if (int rc = check_level_delta(p, d, "conv111_forward")) return rc;
     if (Cin <= 0 || Cout <= 0 || S <= 0) return fail(APRNET_ERR_INVALID_ARGUMENT, "conv111_forward: empty channel / stencil count");
     APRNET_HIP_CHECK(hipSetDevice(p->device));
     // 32 outputs per thread when the layer has more than 16: the input is then read once per 32 output channels
     for (const Segment& sg : segments(p, d, S)) {
         const T* ws = w + (int64_t)sg.stencil * Cout * Cin;
-        if (try_conv111_mfma<T>(x, ldx, Cin, ws, Cin, 1, bias, y, ldy, Cout, sg.begin, sg.end, st)) continue;
+        if (try_conv111_mfma<T>(x, ldx, Cin, ws, Cin, 1, bias, y, ldy, Cout, sg.begin, sg.end, st, relu)) continue;
         if (Cout > 16) {
             dim3 grid((unsigned)((sg.end - sg.begin + TB1 - 1) / TB1), (unsigned)((Cout + 31) / 32));
             hipLaunchKernelGGL((conv111_kernel<T, 32>), grid, dim3(TB1), 0, st, x, ldx, Cin, ws, Cin, 1, bias, y, ldy, Cout,
-                               sg.begin, sg.end);
+                               sg.begin, sg.end, relu);
         } else {
             dim3 grid((unsigned)((sg.end - sg.begin + TB1 - 1) / TB1), 1u);
             hipLaunchKernelGGL((conv111_kernel<T, 16>), grid, dim3(TB1), 0, st, x, ldx, Cin, ws, Cin, 1, bias, y, ldy, Cout,
-                               sg.begin, sg.end);
+                               sg.begin, sg.end, relu);
         }
     }
     APRNET_LAUNCH_CHECK("conv111_kernel");
@@ -223,7 +231,7 @@ int conv111_bwd(const aprnet_plan* p, int d, const T* x, int64_t ldx, int Cin, c
         // grad_x[ci][i] = sum_co w[co][ci] * gy[co][i]: the same kernel with the weight strides swapped
         if (!try_conv111_mfma<T>(gy, ldy, Cout, ws, 1, Cin, (const T*)nullptr, gx, ldgx, Cin, sg.begin, sg.end, st))
             hipLaunchKernelGGL((conv111_kernel<T, OB>), grid, dim3(TB1), 0, st, gy, ldy, Cout, ws, 1, Cin, (const T*)nullptr, gx, ldgx, Cin,
-                               sg.begin, sg.end);
+                               sg.begin, sg.end, 0);
         const int64_t n = sg.end - sg.begin;
         dim3 g2((unsigned)std::min<int64_t>((n + TB1 * 8 - 1) / (TB1 * 8), 256), (unsigned)((Cout + 7) / 8), (unsigned)((Cin + 7) / 8));
         hipLaunchKernelGGL(conv111_dw_kernel<T>, g2, dim3(TB1), 0, st, x, ldx, Cin, gy, ldy, Cout,
@@ -234,15 +242,29 @@ int conv111_bwd(const aprnet_plan* p, int d, const T* x, int64_t ldx, int Cin, c
 }
 
 int conv111_fwd_bf16(const aprnet_plan* p, int d, const bf16_t* x, int64_t ldx, int Cin, const float* w, int S, int Cout,
-                     const float* bias, bf16_t* y, int64_t ldy, hipStream_t st) {
+                     const float* bias, bf16_t* y, int64_t ldy, hipStream_t st, int relu) {
     if (int rc = check_level_delta(p, d, "conv111_forward")) return rc;
     if (Cin <= 0 || Cout <= 0 || S <= 0) return fail(APRNET_ERR_INVALID_ARGUMENT, "conv111_forward: empty channel / stencil count");
     APRNET_HIP_CHECK(hipSetDevice(p->device));
     for (const Segment& sg : segments(p, d, S))
-        if (!launch_conv111_mfma<bf16_t>(x, ldx, Cin, w + (int64_t)sg.stencil * Cout * Cin, Cin, 1, bias, y, ldy, Cout, sg.begin, sg.end, st))
+        if (!launch_conv111_mfma<bf16_t>(x, ldx, Cin, w + (int64_t)sg.stencil * Cout * Cin, Cin, 1, bias, y, ldy, Cout, sg.begin, sg.end, st, relu))
             return fail(APRNET_ERR_UNSUPPORTED, "conv111_forward: more than 128 input channels with bfloat16 features");
     APRNET_LAUNCH_CHECK("conv111_mfma_kernel");
     return 0;
+}
+
+// 1x1x1 forward with the optional clamp at zero, for the fused entry points
+int conv111_fwd_relu(const aprnet_plan* p, int d, const float* x, int64_t ldx, int Cin, const float* w, int S, int Cout,
+                     const float* bias, float* y, int64_t ldy, hipStream_t st, int relu) {
+    return conv111_fwd<float>(p, d, x, ldx, Cin, w, S, Cout, bias, y, ldy, st, relu);
+}
+int conv111_fwd_relu(const aprnet_plan* p, int d, const double* x, int64_t ldx, int Cin, const double* w, int S, int Cout,
+                     const double* bias, double* y, int64_t ldy, hipStream_t st, int relu) {
+    return conv111_fwd<double>(p, d, x, ldx, Cin, w, S, Cout, bias, y, ldy, st, relu);
+}
+int conv111_fwd_relu(const aprnet_plan* p, int d, const bf16_t* x, int64_t ldx, int Cin, const float* w, int S, int Cout,
+                     const float* bias, bf16_t* y, int64_t ldy, hipStream_t st, int relu) {
+    return conv111_fwd_bf16(p, d, x, ldx, Cin, w, S, Cout, bias, y, ldy, st, relu);
 }
 
 }  // namespace aprnet
@@ -251,12 +273,12 @@ using namespace aprnet;
 extern "C" {
 int aprnet_conv111_fwd_bf16(const aprnet_plan* p, int d, const uint16_t* x, int64_t ldx, int Cin, const float* w, int S,
                             int Cout, const float* bias, uint16_t* y, int64_t ldy, void* st) {
-    return conv111_fwd_bf16(p, d, (const bf16_t*)x, ldx, Cin, w, S, Cout, bias, (bf16_t*)y, ldy, (hipStream_t)st);
+    return conv111_fwd_bf16(p, d, (const bf16_t*)x, ldx, Cin, w, S, Cout, bias, (bf16_t*)y, ldy, (hipStream_t)st, 0);
 }
 #define CONV111_API(T, SFX)                                                                                        \
     int aprnet_conv111_fwd_##SFX(const aprnet_plan* p, int d, const T* x, int64_t ldx, int Cin, const T* w, int S,  \
                                  int Cout, const T* bias, T* y, int64_t ldy, void* st) {                            \
-        return conv111_fwd<T>(p, d, x, ldx, Cin, w, S, Cout, bias, y, ldy, (hipStream_t)st); }                      \
+        return conv111_fwd<T>(p, d, x, ldx, Cin, w, S, Cout, bias, y, ldy, (hipStream_t)st, 0); }                      \
     int aprnet_conv111_bwd_##SFX(const aprnet_plan* p, int d, const T* x, int64_t ldx, int Cin, const T* w, int S,  \
                                  int Cout, const T* gy, int64_t ldy, T* gx, int64_t ldgx, T* gw, void* st) {        \
         return conv111_bwd<T>(p, d, x, ldx, Cin, w, S, Cout, gy, ldy, gx, ldgx, gw, (hipStream_t)st); }

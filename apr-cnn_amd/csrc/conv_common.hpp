@@ -26,6 +26,9 @@ struct ConvArgs {
     AccessDev apr, tree;
     const ConvTile* tiles;
     const T* x; int64_t ldx; int Cin;
+    // forward only: channels c_split .. Cin - 1 of the input come from a second tensor (x2 null: all from x), and
+    // the result can be clamped at zero after the bias
+    const T* x2; int64_t ldx2; int c_split; int relu;
     const typename Num<T>::acc* w; int S_exp; int Cout;     // [S_exp][Cout][Cin][K]; fp32 for bfloat16 features
     const typename Num<T>::acc* bias;                       // [Cout] or null
     T* y; int64_t ldy;
@@ -424,7 +427,10 @@ __device__ __forceinline__ void load_values(const ConvArgs<T>& a, int ci0, int n
     __amdgpu_buffer_rsrc_t rx[CIB], rt[CIB];
 #pragma unroll
     for (int c = 0; c < CIB; ++c) {
-        rx[c] = plane_rsrc<T>(a.x, a.ldx, ci0 + c, a.Cin, a.x_count);
+        const int ch = ci0 + c;
+        const bool second = a.x2 != nullptr && ch >= a.c_split;
+        rx[c] = second ? plane_rsrc<T>(a.x2, a.ldx2, ch - a.c_split, a.Cin - a.c_split, a.x_count)
+                       : plane_rsrc<T>(a.x, a.ldx, ch, a.Cin, a.x_count);
         rt[c] = plane_rsrc<T>(a.tree_data, a.ldt, ci0 + c, tree_items ? a.Cin : 0, a.t_count);
     }
 #pragma unroll

@@ -186,7 +186,9 @@ __device__ __forceinline__ void mfma16_window(const ConvArgs<T>& a, int co0, int
 #pragma unroll
                 for (int r = 0; r < 4; ++r) {
                     const int cl = h * 16 + 4 * (lane >> 4) + r;
-                    if (co0 + cl < a.Cout) a.y[(int64_t)(co0 + cl) * a.ldy + o] = Num<T>::st(acc[j][h][r] + bias_l[cl]);
+                    float v = acc[j][h][r] + bias_l[cl];
+                    if (a.relu) v = v < 0.f ? 0.f : v;
+                    if (co0 + cl < a.Cout) a.y[(int64_t)(co0 + cl) * a.ldy + o] = Num<T>::st(v);
                 }
         } else {
             const bool to_tree = (sh.col_pos[col] & COL_TREE) != 0;
@@ -414,7 +416,9 @@ __device__ __forceinline__ void mfma_bf16_window(const ConvArgs<bf16_t>& a, int 
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
                 const int cl = h * 16 + 4 * (lane >> 4) + r;
-                if (co0 + cl < a.Cout) a.y[(int64_t)(co0 + cl) * a.ldy + o] = float_to_bf16(acc[j][h][r] + bias_l[cl]);
+                float v = acc[j][h][r] + bias_l[cl];
+                if (a.relu) v = v < 0.f ? 0.f : v;
+                if (co0 + cl < a.Cout) a.y[(int64_t)(co0 + cl) * a.ldy + o] = float_to_bf16(v);
             }
     }
 }

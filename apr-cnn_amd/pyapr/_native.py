@@ -100,6 +100,9 @@ def hip():
         getattr(lib, f"aprnet_sample_particles_bwd_{t}").argtypes = [vp, i32, vp, i64, i32, vp, i64, vp]
     # bfloat16 features: forward operators of the network, backward of pool / upsample / tree fill
     lib.aprnet_conv_fwd_bf16.argtypes = [vp, i32, i32, i32, i32, vp, i64, i32, vp, i32, i32, vp, vp, i64, vp, i64, vp]
+    for t in ("f32", "f64", "bf16"):      # ..., tree_ws, ld_tree, const aprnet_conv_fusion*, stream
+        getattr(lib, f"aprnet_conv_fwd_fused_{t}").argtypes = [vp, i32, i32, i32, i32, vp, i64, i32, vp, i32, i32, vp, vp, i64,
+                                                                vp, i64, vp, vp]
     lib.aprnet_conv111_fwd_bf16.argtypes = [vp, i32, vp, i64, i32, vp, i32, i32, vp, vp, i64, vp]
     lib.aprnet_fill_tree_mean_bf16.argtypes = [vp, i32, vp, i64, i32, vp, i64, vp]
     lib.aprnet_fill_tree_mean_bwd_bf16.argtypes = [vp, i32, vp, i64, i32, vp, i64, vp]

@@ -124,12 +124,26 @@ def restrict_kernel_backward(grad_weights, num_stencils):
 
 
 # ---------------------------------------------------------------------------------------- convolution
-def conv_forward(aprs, x, weights, level_delta, bias=None):
+class _Fusion(C.Structure):
+    """aprnet_conv_fusion of the C ABI."""
+    _fields_ = [("x2", C.c_void_p), ("ldx2", C.c_int64), ("C2", C.c_int32), ("relu", C.c_int32)]
+
+
+def conv_forward(aprs, x, weights, level_delta, bias=None, relu=False, x2=None):
     """conv333_forward / conv111_forward (wrap_conv_gpu.hpp:32-66, 170-193) for any supported stencil.
     weights: [S_exp, Cout, Cin, kz, kx, ky] (for 1x1x1: [S, Cout, Cin, 1, 1, 1], not expanded).
-    bias ([Cout], optional) is added inside the kernel instead of in a separate pass over the output."""
+    bias ([Cout], optional) is added inside the kernel instead of in a separate pass over the output.
+    relu: the result is clamped at zero in the kernel (the ReLU of BasicBlock, unet_parts.py:17-26).
+    x2 ([B, C2, N], optional): the kernel reads its channels after those of x, which stands for
+    conv(torch.cat([x, x2], dim=1)) (unet_parts.py:82) without writing the concatenated tensor."""
     _check_input(x, "input")
     _check_input(weights, "weights")
+    c2 = 0
+    if x2 is not None:
+        _check_input(x2, "second input")
+        if x2.dtype != x.dtype or x2.size(0) != x.size(0) or x2.size(2) != x.size(2):
+            raise ValueError("the second input must match the first in dtype, batch size and particle count")
+        c2 = x2.size(1)
     if x.dtype == torch.bfloat16:
         # bfloat16 is the storage type of the features only: weights and bias are used in fp32
         weights = weights.float()
@@ -141,9 +155,13 @@ def conv_forward(aprs, x, weights, level_delta, bias=None):
         if bias.dtype != weights.dtype or bias.numel() != weights.size(1):
             raise ValueError("bias must hold one value per output channel, in the dtype of the weights")
     bptr = _ptr(bias) if bias is not None else None
-    if x.size(1) != weights.size(2):
+    if x.size(1) + c2 != weights.size(2):
         raise ValueError("convolve: input tensor shape does not match weights tensor!")   # conv.hpp:63-66
     s_exp, cout, cin, kz, kx, ky = weights.shape
+    c1 = cin - c2
+    fused = relu or x2 is not None
+    if x2 is not None and (kz, kx, ky) == (1, 1, 1):
+        raise ValueError("the 1x1x1 convolution takes a single input")
     B, _, N = x.shape
     d = _deltas(level_delta, len(aprs))
     sizes = [number_particles(a, d[b]) for b, a in enumerate(aprs)]
@@ -155,12 +173,22 @@ def conv_forward(aprs, x, weights, level_delta, bias=None):
         # the reference adds the bias to the whole padded tensor (conv.py:101): tails hold 0 + bias
         for b, nb in enumerate(sizes):
             if nb < N:
-                out[b, :, nb:] = bias.view(-1, 1)
+                out[b, :, nb:] = (bias.clamp(min=0) if relu else bias).view(-1, 1)
     plans = _plans(aprs, x.device)
     sfx = _sfx(x, bf16=True)
     with torch.cuda.device(x.device):
         st = _stream()
-        if (kz, kx, ky) == (1, 1, 1):
+        if fused:
+            ld_tree = max(max(tree_parts(a, d[b]) for b, a in enumerate(aprs)), 1)
+            tree_ws = torch.empty((cin, ld_tree), dtype=x.dtype, device=x.device)
+            fn = getattr(_lib(), "aprnet_conv_fwd_fused_" + sfx)
+            for b in range(B):
+                fu = _Fusion(_ptr(x2[b]) if x2 is not None else None, N, c2, 1 if relu else 0)
+                rc = fn(plans[b], d[b], kz, kx, ky, _ptr(x[b]), N, c1, _ptr(weights), s_exp, cout, bptr, _ptr(out[b]), N,
+                        _ptr(tree_ws), ld_tree, C.byref(fu), st)
+                if rc:
+                    _raise(rc, "conv_forward failed")
+        elif (kz, kx, ky) == (1, 1, 1):
             fn = getattr(_lib(), "aprnet_conv111_fwd_" + sfx)
             for b in range(B):
                 rc = fn(plans[b], d[b], _ptr(x[b]), N, cin, _ptr(weights), s_exp, cout, bptr, _ptr(out[b]), N, st)

@@ -67,6 +67,22 @@ class ConvFunction(Function):
         return grad_input, grad_w, grad_bias, None, None, None
 
 
+def conv_inference(inputs, weights, bias, aprs, level_deltas, layout, relu=False, inputs2=None):
+    """ConvFunction.forward without the autograd record, with the two fusions the kernel offers: the ReLU that
+    follows the convolution in BasicBlock (unet_parts.py:17-26, norm folded away) and a second input tensor in
+    place of torch.cat([inputs, inputs2], dim=1) (unet_parts.py:82).  For inference under torch.no_grad()."""
+    w = _to_device_layout(weights.detach(), layout).contiguous()
+    if inputs.dtype == torch.bfloat16:
+        w = w.float()
+    ksize = tuple(w.shape[3:])
+    if ksize not in SUPPORTED_KERNELS:
+        raise ValueError(f"unsupported kernel size {ksize}")
+    if ksize != (1, 1, 1):
+        w = _ops.restrict_kernel_forward(w, max(a.level_max() - a.level_min() + 1 for a in aprs))
+    return _ops.conv_forward(aprs, inputs.contiguous(), w, level_deltas, None if bias is None else bias.detach().contiguous(),
+                             relu=relu, x2=None if inputs2 is None else inputs2.contiguous())
+
+
 class MaxPoolFunction(Function):
     @staticmethod
     def forward(ctx, inputs, aprs, level_deltas, increment_level_deltas, pad_value):

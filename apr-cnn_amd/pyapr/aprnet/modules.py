@@ -11,7 +11,7 @@ import torch
 from torch import nn
 from torch.nn import init
 
-from .functional import (ConvFunction, MaxPoolFunction, UpSampleConstFunction, ReconstructFunction,
+from .functional import (ConvFunction, conv_inference, MaxPoolFunction, UpSampleConstFunction, ReconstructFunction,
                          SampleParticlesFunction, CPU_LAYOUT, CUDA_LAYOUT, SUPPORTED_KERNELS)
 
 
@@ -48,6 +48,13 @@ class APRConv(nn.Module):
 
     def forward(self, input_features, aprs, level_deltas):
         return ConvFunction.apply(input_features, self.weight, self.bias, aprs, level_deltas, self.weight_layout)
+
+    def forward_fused(self, input_features, aprs, level_deltas, relu=False, second_input=None):
+        """Inference-only forward (no autograd record): optionally clamps the result at zero inside the kernel and
+        reads ``second_input`` as the channels that follow those of ``input_features``, i.e.
+        relu(self(torch.cat([input_features, second_input], 1))) in one pass."""
+        return conv_inference(input_features, self.weight, self.bias, aprs, level_deltas, self.weight_layout,
+                              relu=relu, inputs2=second_input)
 
 
 class MaxPool(nn.Module):

@@ -94,6 +94,17 @@ int aprnet_channel_sum_work_elems(int C);
 int aprnet_channel_sum_f32(const float* x, int64_t ld, int C, int64_t n, float* out, int accumulate, float* work, void* stream);
 int aprnet_channel_sum_f64(const double* x, int64_t ld, int C, int64_t n, double* out, int accumulate, double* work, void* stream);
 
+/* Optional parts of aprnet_conv_fwd_fused_*.  They fuse what the reference network does in separate passes around
+ * a convolution: torch.cat of the skip connection and the upsampled features before the first convolution of a
+ * decoder stage (unet_parts.py:82), and the ReLU that follows a convolution whose norm has been folded into it
+ * (BasicBlock, unet_parts.py:17-26). */
+typedef struct aprnet_conv_fusion {
+    const void* x2;   /* second input [C2][ldx2], element type of x: its channels follow the Cin channels of x in   */
+    int64_t ldx2;     /* the contraction, i.e. w has Cin + C2 input channels; NULL / 0 for a single input           */
+    int32_t C2;
+    int32_t relu;     /* nonzero: y = max(conv + bias, 0) */
+} aprnet_conv_fusion;
+
 #define APRNET_DECL(T, SFX)                                                                                          \
     /* helpers::fill_tree_mean (helpers.hpp:156-252): tree[c][t] for all tree nodes of level < Lc. */               \
     int aprnet_fill_tree_mean_##SFX(const aprnet_plan*, int level_delta, const T* x, int64_t ldx, int C,            \
@@ -110,6 +121,13 @@ int aprnet_channel_sum_f64(const double* x, int64_t ld, int C, int64_t n, double
     int aprnet_conv_fwd_##SFX(const aprnet_plan*, int level_delta, int kz, int kx, int ky,                          \
                               const T* x, int64_t ldx, int Cin, const T* w, int S_exp, int Cout, const T* bias,     \
                               T* y, int64_t ldy, T* tree_ws, int64_t ld_tree, void* stream);                        \
+    /* The same with the optional fused parts (fusion may be NULL).  With a second input tree_ws is                 \
+     * [Cin + C2][ld_tree].  (kz,kx,ky) = (1,1,1) is accepted too (w [S][Cout][Cin], no second input, tree_ws       \
+     * unused): Convolution<1,1,1>::forward followed by the ReLU. */                                                \
+    int aprnet_conv_fwd_fused_##SFX(const aprnet_plan*, int level_delta, int kz, int kx, int ky,                    \
+                                    const T* x, int64_t ldx, int Cin, const T* w, int S_exp, int Cout,              \
+                                    const T* bias, T* y, int64_t ldy, T* tree_ws, int64_t ld_tree,                  \
+                                    const aprnet_conv_fusion* fusion, void* stream);                                \
     /* Convolution<kz,kx,ky>::backward (conv.hpp:261-481), CUDA twin conv333_backward.  grad_x is OVERWRITTEN,      \
      * grad_w [S_exp][Cout][Cin][k] is ACCUMULATED into (zero it before the first batch item, as                    \
      * torch::zeros_like does in conv.hpp:270).  tree_ws / grad_tree_ws: [Cin][ld_tree] scratch each. */            \
@@ -167,6 +185,9 @@ APRNET_DECL(double, f64)
 int aprnet_conv_fwd_bf16(const aprnet_plan*, int level_delta, int kz, int kx, int ky, const uint16_t* x, int64_t ldx, int Cin,
                          const float* w, int S_exp, int Cout, const float* bias, uint16_t* y, int64_t ldy,
                          uint16_t* tree_ws, int64_t ld_tree, void* stream);          /* not 5x5x5 */
+int aprnet_conv_fwd_fused_bf16(const aprnet_plan*, int level_delta, int kz, int kx, int ky, const uint16_t* x, int64_t ldx,
+                               int Cin, const float* w, int S_exp, int Cout, const float* bias, uint16_t* y, int64_t ldy,
+                               uint16_t* tree_ws, int64_t ld_tree, const aprnet_conv_fusion* fusion, void* stream);
 int aprnet_conv111_fwd_bf16(const aprnet_plan*, int level_delta, const uint16_t* x, int64_t ldx, int Cin, const float* w,
                             int S, int Cout, const float* bias, uint16_t* y, int64_t ldy, void* stream);
 int aprnet_fill_tree_mean_bf16(const aprnet_plan*, int level_delta, const uint16_t* x, int64_t ldx, int C, uint16_t* tree,

@@ -452,3 +452,54 @@ def test_conv111_backward_bf16_is_refused():
     wd = w.permute(1, 2, 0, 3, 4, 5).contiguous().to(DEV)
     with pytest.raises(TypeError):
         _ops.conv_backward(aprs, x.to(torch.bfloat16).to(DEV), wd, x.to(torch.bfloat16).to(DEV), ld)
+
+
+# ------------------------------------------------------------------------- fused forward (ReLU, second input)
+@pytest.mark.parametrize("path", [0, 1], ids=["mfma", "valu"])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64, torch.bfloat16], ids=["f32", "f64", "bf16"])
+@pytest.mark.parametrize("ksize,c1,c2,cout", [((3, 3, 3), 16, 16, 16), ((3, 3, 3), 5, 6, 33), ((1, 5, 5), 7, 3, 20),
+                                              ((5, 5, 5), 3, 2, 4)], ids=lambda v: KID(v) if isinstance(v, tuple) else str(v))
+def test_conv_forward_fused_relu_and_second_input(ksize, c1, c2, cout, dtype, path):
+    """aprnet_conv_fwd_fused_*: relu(conv(cat([x, x2])) + bias) in one kernel against the oracle's convolution of the
+    concatenated tensor followed by bias and ReLU (unet_parts.py:17-26, 82).  Unequal batch items: the padded
+    tails must hold relu(bias) as they would after the reference's separate passes."""
+    if dtype == torch.bfloat16 and (ksize == (5, 5, 5) or path == 1):
+        pytest.skip("bfloat16 features: matrix-core stencils only")
+    bt = [("3d_b", 1), ("3d_c", 0)]
+    cdt = torch.float32 if dtype == torch.bfloat16 else dtype
+    x, aprs, ld, w_exp = _conv_case(bt, ksize, 2, c1 + c2, cout, cdt)
+    if dtype == torch.bfloat16:
+        x = x.to(torch.bfloat16).float()
+    g = torch.Generator().manual_seed(5)
+    bias = torch.randn(cout, dtype=cdt, generator=g)
+    ref = torch.relu(oracle.conv_forward(aprs, x, w_exp, ld) + bias.view(1, -1, 1))
+    xa, xb = x[:, :c1].contiguous().to(dtype).to(DEV), x[:, c1:].contiguous().to(dtype).to(DEV)
+    wd = w_exp.permute(1, 2, 0, 3, 4, 5).contiguous().to(DEV)
+    lib = _native.hip()
+    assert lib.aprnet_set_conv_path(path) == 0
+    try:
+        got = _ops.conv_forward(aprs, xa, wd, ld, bias.to(DEV), relu=True, x2=xb)
+        plain = _ops.conv_forward(aprs, torch.cat([xa, xb], 1), wd, ld, bias.to(DEV))
+    finally:
+        lib.aprnet_set_conv_path(0)
+    if dtype == torch.bfloat16:
+        close_bf16(got, ref)
+    else:
+        close(got, ref, dtype)
+        # same kernel, same order of operations: the fusion changes nothing but the clamp
+        assert torch.equal(got, torch.relu(plain))
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64, torch.bfloat16], ids=["f32", "f64", "bf16"])
+def test_conv111_forward_fused_relu(dtype):
+    cdt = torch.float32 if dtype == torch.bfloat16 else dtype
+    x, aprs, ld, w = _conv_case([("3d_b", 1), ("3d_c", 0)], (1, 1, 1), 3, 20, 9, cdt)
+    if dtype == torch.bfloat16:
+        x = x.to(torch.bfloat16).float()
+    bias = torch.linspace(-1, 1, 9, dtype=cdt)
+    ref = torch.relu(oracle.conv_forward(aprs, x, w, ld) + bias.view(1, -1, 1))
+    wd = w.permute(1, 2, 0, 3, 4, 5).contiguous().to(DEV)
+    got = _ops.conv_forward(aprs, x.to(dtype).to(DEV), wd, ld, bias.to(DEV), relu=True)
+    close_bf16(got, ref) if dtype == torch.bfloat16 else close(got, ref, dtype)
+    with pytest.raises(ValueError):
+        _ops.conv_forward(aprs, x[:, :10].contiguous().to(dtype).to(DEV), wd, ld, x2=x[:, 10:].contiguous().to(dtype).to(DEV))
