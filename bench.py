@@ -99,9 +99,18 @@ def other_ops(apr, x, dev):
     nt = _ops.tree_parts(apr, 0)
     res = []
 
+    # what a plain device-to-device copy of the same tensor reaches on this GPU: the practical ceiling that the
+    # memory-bound operators are also priced against
+    dst = torch.empty_like(x)
+    ms = _time(lambda: dst.copy_(x))
+    copy_gbs = 2 * x.numel() * e / ms / 1e6
+    res.append({"op": "copy_d2d", "ms": ms, "algorithmic_GB": 2 * x.numel() * e / 1e9, "GBps": copy_gbs,
+                "hbm_frac": copy_gbs / PEAK_HBM_GBS, "note": "torch copy of the input features, read + write"})
+    del dst
+
     def line(op, ms, nbytes, note):
         res.append({"op": op, "ms": ms, "algorithmic_GB": nbytes / 1e9, "GBps": nbytes / ms / 1e6,
-                    "hbm_frac": nbytes / ms / 1e6 / PEAK_HBM_GBS, "note": note})
+                    "hbm_frac": nbytes / ms / 1e6 / PEAK_HBM_GBS, "copy_frac": nbytes / ms / 1e6 / copy_gbs, "note": note})
 
     with torch.no_grad():
         pooled, idx = _ops.maxpool_forward([apr], x, ld0, 0.0)
