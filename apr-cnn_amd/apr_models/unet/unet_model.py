@@ -60,7 +60,14 @@ def fold_norms(model):
     w' = w * gamma / sqrt(var + eps) per output channel, bias' = beta - mean * gamma / sqrt(var + eps).
     The conv gains a bias parameter and the norm becomes nn.Identity.  GroupNorm depends on the input
     and cannot be folded; models meant for folded inference are built with norm='batch'."""
+    from .hybrid_unet_parts import PixelBasicBlock
     for m in model.modules():
+        if isinstance(m, PixelBasicBlock) and isinstance(m.norm, nn.BatchNorm3d):      # dense stages of the hybrid net
+            bn, conv = m.norm, m.conv
+            scale = bn.weight / torch.sqrt(bn.running_var + bn.eps)
+            conv.weight.mul_(scale.view(-1, 1, 1, 1, 1))                               # [Cout, Cin, kz, kx, ky]
+            conv.bias = nn.Parameter((bn.bias - bn.running_mean * scale).clone())
+            m.norm = nn.Identity()
         if isinstance(m, BasicBlock) and isinstance(m.norm, nn.BatchNorm1d):
             bn, conv = m.norm, m.conv
             scale = bn.weight / torch.sqrt(bn.running_var + bn.eps)

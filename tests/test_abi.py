@@ -90,3 +90,24 @@ def test_apr_state_roundtrip():
     for a, b in ((apr.iterator(), back.iterator()), (apr.tree_iterator(), back.tree_iterator())):
         assert np.array_equal(a.level_xz_vec, b.level_xz_vec) and np.array_equal(a.xz_end_vec, b.xz_end_vec)
         assert np.array_equal(a.y_vec, b.y_vec) and a.level_min() == b.level_min() and a.level_max() == b.level_max()
+
+
+def test_model_parameter_names_mirror_reference():
+    """state_dict keys of the networks are those of the reference's module trees (unet_parts.py:6-83,
+    hybrid_unet_parts.py:9-128, unet_model.py / hybrid_model.py), so checkpoints are interchangeable."""
+    from apr_models.unet import APRUNet, HybridAPRUNet
+    keys = set(APRUNet(1, 2, depth=1, n_filters_base=4).state_dict())
+    assert {"encoder.0.blocks.0.conv.weight", "encoder.0.blocks.1.norm.weight", "encoder.1.conv.blocks.0.conv.weight",
+            "decoder.0.reduce_ch.conv.weight", "decoder.0.conv.blocks.1.norm.bias", "head.weight", "head.bias"} <= keys
+    hyb = HybridAPRUNet(1, 2, depth=3, apr_depth=1, n_filters_base=4)
+    keys = set(hyb.state_dict())
+    assert {"encoder.1.conv.blocks.0.conv.weight",            # DownConv (particles)
+            "encoder.2.conv.blocks.0.conv.weight",            # TransitionDownConv (dense Conv3d)
+            "encoder.3.conv.blocks.1.norm.weight",            # PixelDownConv
+            "decoder.0.reduce_ch.conv.weight",                # PixelUpConv
+            "decoder.1.reduce_ch.conv.weight", "decoder.1.conv.blocks.0.conv.weight",      # TransitionUpConv
+            "decoder.2.reduce_ch.conv.weight", "head.weight"} <= keys
+    sd = hyb.state_dict()
+    assert sd["encoder.2.conv.blocks.0.conv.weight"].dim() == 5       # nn.Conv3d [Cout, Cin, kz, kx, ky]
+    assert sd["decoder.1.conv.blocks.0.conv.weight"].dim() == 6       # APRConv [S, Cout, Cin, kz, kx, ky]
+    assert tuple(sd["decoder.1.conv.blocks.0.conv.weight"].shape[1:3]) == (8, 16)      # reads skip + upsampled

@@ -92,3 +92,111 @@ def test_unet_forward_bf16_features():
     assert got.dtype == torch.bfloat16 and got.shape == ref.shape
     err = float((got.float().cpu() - ref).abs().max()) / float(ref.abs().max())
     assert err < 2e-2, f"rel err {err:.2e}"
+
+
+# ----------------------------------------------------------------------------------------------- hybrid network
+def reference_forward_hybrid(model, x, aprs):
+    """HybridAPRUNet evaluated with the CPU oracle for every particle operator (and the model's own dense torch
+    blocks, on the CPU) in the order of apr_models/apr_models/unet/hybrid_model.py:123-139."""
+    from apr_models.unet import DownConv, UpConv, TransitionDownConv, TransitionUpConv
+    from oracle_modules import OracleReconstruct, OracleSample
+    ld = torch.zeros(len(aprs), dtype=torch.int32)
+    skips = [_cpu_block(model.encoder[0], x, aprs, ld)]
+    for stage in model.encoder[1:]:
+        if isinstance(stage, DownConv):
+            y = OracleMaxPool.apply(skips[-1], aprs, ld); ld += 1
+            skips.append(_cpu_block(stage.conv, y, aprs, ld))
+        elif isinstance(stage, TransitionDownConv):
+            y = OracleMaxPool.apply(skips[-1], aprs, ld); ld += 1
+            skips.append(stage.conv(OracleReconstruct.apply(y, aprs, ld)))
+        else:
+            skips.append(stage(skips[-1]))
+    y = skips[-1]
+    for i, stage in enumerate(model.decoder):
+        skip = skips[-(i + 2)]
+        if isinstance(stage, UpConv):
+            y = torch.relu(_cpu_conv(stage.reduce_ch.conv, y, aprs, ld))
+            y = OracleUpSample.apply(y, aprs, ld); ld -= 1
+            y = _cpu_block(stage.conv, torch.cat([skip, y], dim=1), aprs, ld)
+        elif isinstance(stage, TransitionUpConv):
+            y = OracleSample.apply(stage.reduce_ch(y), aprs, ld)
+            y = OracleUpSample.apply(y, aprs, ld); ld -= 1
+            y = _cpu_block(stage.conv, torch.cat([skip, y], dim=1), aprs, ld)
+        else:
+            y = stage(y, skip)
+    return _cpu_conv(model.head, y, aprs, ld)
+
+
+@pytest.mark.parametrize("apr_depth", [0, 1, 2])
+def test_hybrid_unet_forward_matches_oracle(apr_depth):
+    """Particle stages above, dense stages below the transition (Reconstruct / SampleParticles), norms folded;
+    odd volume dimensions exercise the padding of the dense decoder."""
+    import copy
+    from apr_models.unet import HybridAPRUNet
+    apr = apr_cases.random_apr((33, 29, 37), 11, density=0.02)
+    torch.manual_seed(0)
+    model = HybridAPRUNet(1, 3, depth=3, apr_depth=apr_depth, n_filters_base=8, n_stencils=2, norm="batch").eval()
+    for m in model.modules():
+        if isinstance(m, (torch.nn.BatchNorm1d, torch.nn.BatchNorm3d)):
+            m.running_mean.uniform_(-0.2, 0.2); m.running_var.uniform_(0.5, 1.5)
+            m.weight.data.uniform_(0.5, 1.5); m.bias.data.uniform_(-0.1, 0.1)
+    fold_norms(model)
+    n = apr.total_number_particles()
+    x = torch.randn(1, 1, n)
+    with torch.no_grad():
+        ref = reference_forward_hybrid(copy.deepcopy(model), x, [apr])
+        got = model.to(DEV)(x.to(DEV), [apr])
+    assert got.shape == ref.shape == (1, 3, n)
+    err = float((got.cpu() - ref).abs().max()) / float(ref.abs().max())
+    assert err < 5e-5, f"rel err {err:.2e}"      # dense convolutions of the two sides differ in summation order too
+
+
+def test_hybrid_unet_training_step_matches_oracle_gradients():
+    """One backward pass through particle and dense stages (GroupNorm, not folded): gradients of the first
+    particle convolution and of a dense convolution against the oracle-composed network's autograd."""
+    import copy
+    from apr_models.unet import HybridAPRUNet
+    apr = apr_cases.random_apr((20, 24, 28), 5, density=0.03)
+    torch.manual_seed(3)
+    model = HybridAPRUNet(2, 2, depth=2, apr_depth=1, n_filters_base=4, n_stencils=1, norm="batch").train()
+    for m in model.modules():                       # batch statistics would differ through the padded tails: eval norms
+        if isinstance(m, (torch.nn.BatchNorm1d, torch.nn.BatchNorm3d)):
+            m.eval()
+    n = apr.total_number_particles()
+    x = torch.randn(1, 2, n)
+    ref_model = copy.deepcopy(model)
+
+    def conv_g(conv, y, aprs, ld):                  # oracle convolution that keeps the graph to the parameters
+        return OracleConv.apply(y, conv.weight.permute(2, 0, 1, 3, 4, 5).contiguous(), conv.bias, aprs, ld)
+
+    def cpu_block_bn(block, y, aprs, ld):           # particle blocks with their (eval) norms, on the oracle
+        for bb in block.blocks:
+            y = torch.relu(bb.norm(conv_g(bb.conv, y, aprs, ld)))
+        return y
+
+    from oracle_modules import OracleReconstruct, OracleSample
+    ld = torch.zeros(1, dtype=torch.int32)
+    e0 = cpu_block_bn(ref_model.encoder[0], x, [apr], ld)
+    y = OracleMaxPool.apply(e0, [apr], ld); ld += 1
+    e1 = cpu_block_bn(ref_model.encoder[1].conv, y, [apr], ld)
+    y = OracleMaxPool.apply(e1, [apr], ld); ld += 1
+    e2 = ref_model.encoder[2].conv(OracleReconstruct.apply(y, [apr], ld))
+    d = ref_model.decoder[0]
+    y = OracleUpSample.apply(OracleSample.apply(d.reduce_ch(e2), [apr], ld), [apr], ld); ld -= 1
+    y = cpu_block_bn(d.conv, torch.cat([e1, y], 1), [apr], ld)
+    d = ref_model.decoder[1]
+    y = torch.relu(d.reduce_ch.norm(conv_g(d.reduce_ch.conv, y, [apr], ld)))
+    y = OracleUpSample.apply(y, [apr], ld); ld -= 1
+    y = cpu_block_bn(d.conv, torch.cat([e0, y], 1), [apr], ld)
+    ref = conv_g(ref_model.head, y, [apr], ld)
+    ref.square().sum().backward()
+
+    model.to(DEV)
+    got = model(x.to(DEV), [apr])
+    got.square().sum().backward()
+    assert float((got.detach().cpu() - ref.detach()).abs().max()) <= 5e-5 * float(ref.detach().abs().max())
+    for name in ["encoder.0.blocks.0.conv.weight", "encoder.2.conv.blocks.0.conv.weight", "decoder.0.conv.blocks.0.conv.weight",
+                 "head.bias"]:
+        g = dict(model.named_parameters())[name].grad.cpu()
+        r = dict(ref_model.named_parameters())[name].grad
+        assert float((g - r).abs().max()) <= 2e-4 * float(r.abs().max()) + 1e-7, name
