@@ -200,3 +200,36 @@ def test_hybrid_unet_training_step_matches_oracle_gradients():
         g = dict(model.named_parameters())[name].grad.cpu()
         r = dict(ref_model.named_parameters())[name].grad
         assert float((g - r).abs().max()) <= 2e-4 * float(r.abs().max()) + 1e-7, name
+
+
+@pytest.mark.parametrize("out_delta,after", [(0, None), (1, 12)])
+def test_stardist_unet_heads_match_oracle(out_delta, after):
+    """APRStardistUNet: probability and ray-distance heads on the particles left at output_level_delta, against the
+    oracle composition (stardist_model.py:113-132)."""
+    from apr_models.unet import APRStardistUNet
+    apr = apr_cases.random_apr((33, 29, 37), 11, density=0.02)
+    torch.manual_seed(2)
+    model = fold_norms(APRStardistUNet(1, 8, depth=2, n_filters_base=8, n_stencils=2, norm="batch",
+                                       output_level_delta=out_delta, net_conv_after_unet=after).eval())
+    x = torch.randn(1, 1, apr.total_number_particles())
+    aprs, ld = [apr], torch.zeros(1, dtype=torch.int32)
+    skips = [_cpu_block(model.encoder[0], x, aprs, ld)]
+    for stage in model.encoder[1:]:
+        y = OracleMaxPool.apply(skips[-1], aprs, ld); ld += 1
+        skips.append(_cpu_block(stage.conv, y, aprs, ld))
+    y = skips[-1]
+    for i, stage in enumerate(model.decoder):
+        y = torch.relu(_cpu_conv(stage.reduce_ch.conv, y, aprs, ld))
+        y = OracleUpSample.apply(y, aprs, ld); ld -= 1
+        y = _cpu_block(stage.conv, torch.cat([skips[-(i + 2)], y], dim=1), aprs, ld)
+    if after is not None:
+        y = _cpu_block(model.conv_after_unet, y, aprs, ld)
+    ref_prob = torch.sigmoid(_cpu_conv(model.output_prob.conv, y, aprs, ld))
+    ref_dist = _cpu_conv(model.output_dist, y, aprs, ld)
+    assert int(ld[0]) == out_delta
+    with torch.no_grad():
+        prob, dist = model.to(DEV)(x.to(DEV), [apr])
+    n_out = oracle.number_parts(apr, out_delta)
+    assert prob.shape == (1, 1, n_out) and dist.shape == (1, 8, n_out)
+    assert float((prob.cpu() - ref_prob).abs().max()) < 2e-5
+    assert float((dist.cpu() - ref_dist).abs().max()) < 2e-5 * float(ref_dist.abs().max())
