@@ -43,7 +43,7 @@ conv_fwd_kernel(const ConvArgs<T> a) {
 
             for (int ci0 = 0; ci0 < a.Cin; ci0 += CIB) {
                 __syncthreads();
-                stage_values<G, T, CIB>(a, ci0, nitem, L < a.Lc, sh, patch);
+                stage_values<G, T, CIB>(a, ci0, nitem, L < a.Lc, sh, patch, std::bool_constant<true>{});
                 __syncthreads();
 #pragma unroll
                 for (int it = 0; it < G::ITER; ++it) {

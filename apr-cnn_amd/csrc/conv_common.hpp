@@ -19,6 +19,8 @@
 #pragma once
 #include "common.hpp"
 
+#include <type_traits>
+
 namespace aprnet {
 
 template <typename T>
@@ -421,16 +423,19 @@ __device__ __forceinline__ void fetch_slots(const Lists& sh, int nitem, ItemRegs
 }
 
 // Issues the value loads of one chunk for the fetched slots.
-template <class G, typename T, int CIB, int NR>
+// FUSE (a tag argument, so that the other template arguments stay deduced): the kernel was built for the fused
+// forward entry points and honours a.x2 / a.c_split; otherwise those fields are not looked at.
+template <class G, typename T, int CIB, int NR, bool FUSE = false>
 __device__ __forceinline__ void load_values(const ConvArgs<T>& a, int ci0, int nitem, bool tree_items,
-                                            ItemRegs<G, T, CIB, NR>& R, int round0 = 0) {
+                                            ItemRegs<G, T, CIB, NR>& R, int round0 = 0, std::bool_constant<FUSE> = {}) {
     __amdgpu_buffer_rsrc_t rx[CIB], rt[CIB];
 #pragma unroll
     for (int c = 0; c < CIB; ++c) {
         const int ch = ci0 + c;
-        const bool second = a.x2 != nullptr && ch >= a.c_split;
-        rx[c] = second ? plane_rsrc<T>(a.x2, a.ldx2, ch - a.c_split, a.Cin - a.c_split, a.x_count)
-                       : plane_rsrc<T>(a.x, a.ldx, ch, a.Cin, a.x_count);
+        if (FUSE && a.x2 != nullptr && ch >= a.c_split)
+            rx[c] = plane_rsrc<T>(a.x2, a.ldx2, ch - a.c_split, a.Cin - a.c_split, a.x_count);
+        else
+            rx[c] = plane_rsrc<T>(a.x, a.ldx, ch, a.Cin, a.x_count);
         rt[c] = plane_rsrc<T>(a.tree_data, a.ldt, ci0 + c, tree_items ? a.Cin : 0, a.t_count);
     }
 #pragma unroll
@@ -450,11 +455,12 @@ __device__ __forceinline__ void load_values(const ConvArgs<T>& a, int ci0, int n
 // Issues the loads of a chunk (no LDS writes: they may run ahead of the consumer of the patch).
 // Thread t owns items t, t + NT, ...; a round k that lies beyond the item count is skipped by a
 // wave-uniform branch (most windows hold fewer items than the block has threads).
-template <class G, typename T, int CIB, int NR, class Lists>
+template <class G, typename T, int CIB, int NR, class Lists, bool FUSE = false>
 __device__ __forceinline__ void load_items(const ConvArgs<T>& a, int ci0, int nitem, bool tree_items,
-                                           const Lists& sh, ItemRegs<G, T, CIB, NR>& R, int round0 = 0) {
+                                           const Lists& sh, ItemRegs<G, T, CIB, NR>& R, int round0 = 0,
+                                           std::bool_constant<FUSE> fuse = {}) {
     fetch_slots<G, T, CIB, NR>(sh, nitem, R, round0);
-    load_values<G, T, CIB, NR>(a, ci0, nitem, tree_items, R, round0);
+    load_values<G, T, CIB, NR>(a, ci0, nitem, tree_items, R, round0, fuse);
 }
 
 template <class G, typename T, int CIB, int NR>
@@ -477,11 +483,12 @@ __device__ __forceinline__ void store_items(const ItemRegs<G, T, CIB, NR>& R, in
 // Gather of one channel chunk into the patch.  Cells that no item covers keep the zeros written once
 // per window (outside the image, or inside a particle two or more levels coarser, which a stencil of
 // half-width <= 2 never reads on a 2:1-balanced APR); covered cells are overwritten by every chunk.
-template <class G, typename T, int CIB>
+template <class G, typename T, int CIB, bool FUSE = false>
 __device__ __forceinline__ void stage_values(const ConvArgs<T>& a, int ci0, int nitem, bool tree_items,
-                                             const ConvShared<G>& sh, typename Num<T>::acc* patch) {
+                                             const ConvShared<G>& sh, typename Num<T>::acc* patch,
+                                             std::bool_constant<FUSE> fuse = {}) {
     ItemRegs<G, T, CIB> R;
-    load_items<G, T, CIB>(a, ci0, nitem, tree_items, sh, R);
+    load_items<G, T, CIB>(a, ci0, nitem, tree_items, sh, R, 0, fuse);
     store_items<G, T, CIB>(R, nitem, patch);
 }
 

@@ -72,7 +72,7 @@ __global__ void pack_weights16_kernel(const float* __restrict__ w, int S_exp, in
 
 // MODE 0: forward, results stored (plus bias).  MODE 1: input gradient, results added atomically to the
 // place each column names (feature gradient, or tree gradient with COL_TREE).
-template <typename T, class G, int CIB, int COH, int NB, int MODE, class Lists>
+template <typename T, class G, int CIB, int COH, int NB, int MODE, bool FUSE, class Lists>
 __device__ __forceinline__ void mfma16_window(const ConvArgs<T>& a, int co0, int nc, int nitem, bool tree_items, int first,
                                               const float4* __restrict__ wl, const Lists& sh,
                                               float* __restrict__ patch, float* __restrict__ Wl,
@@ -117,7 +117,7 @@ __device__ __forceinline__ void mfma16_window(const ConvArgs<T>& a, int co0, int
         const int i = threadIdx.x + k * G::NT;                                                     \
         if (i < W4) reinterpret_cast<float4*>(Wl)[i] = wr[k];                                      \
     }
-    load_items<G, T, CIB>(a, 0, nitem, tree_items, sh, R);
+    load_items<G, T, CIB>(a, 0, nitem, tree_items, sh, R, 0, std::bool_constant<FUSE>{});
     APRNET_LOAD_WEIGHTS(0)
     for (int i = threadIdx.x; i < CIB * G::CH_STRIDE; i += G::NT) patch[i] = 0.f;     // once per window
     for (int ci0 = 0; ci0 < a.Cin; ci0 += CIB) {
@@ -126,7 +126,7 @@ __device__ __forceinline__ void mfma16_window(const ConvArgs<T>& a, int co0, int
         APRNET_STORE_WEIGHTS()
         __syncthreads();
         if (ci0 + CIB < a.Cin) {
-            load_values<G, T, CIB>(a, ci0 + CIB, nitem, tree_items, R);
+            load_values<G, T, CIB>(a, ci0 + CIB, nitem, tree_items, R, 0, std::bool_constant<FUSE>{});
             APRNET_LOAD_WEIGHTS(ci0 / CIB + 1)
         }
         if constexpr (MODE == 1) {
@@ -187,7 +187,7 @@ __device__ __forceinline__ void mfma16_window(const ConvArgs<T>& a, int co0, int
                 for (int r = 0; r < 4; ++r) {
                     const int cl = h * 16 + 4 * (lane >> 4) + r;
                     float v = acc[j][h][r] + bias_l[cl];
-                    if (a.relu) v = v < 0.f ? 0.f : v;
+                    if (FUSE && a.relu) v = v < 0.f ? 0.f : v;
                     if (co0 + cl < a.Cout) a.y[(int64_t)(co0 + cl) * a.ldy + o] = Num<T>::st(v);
                 }
         } else {
@@ -208,7 +208,8 @@ __device__ __forceinline__ void mfma16_window(const ConvArgs<T>& a, int co0, int
 // COH = 16-channel parts of the output block: 1 for layers of at most 16 output channels, 2 otherwise
 // LISTS: the windows of the tile come as precomputed lists from the plan (forward); otherwise the block scans
 // the access arrays itself (input gradient).
-template <typename T, class G, int COH, int MODE, bool LISTS>
+// FUSE: built for the fused forward entry points (second input tensor, clamp at zero)
+template <typename T, class G, int COH, int MODE, bool LISTS, bool FUSE = false>
 __global__ void __launch_bounds__(G::NT)
 __attribute__((amdgpu_waves_per_eu(LISTS ? FWD_WAVES : DX_WAVES, LISTS ? FWD_WAVES : DX_WAVES)))
 conv_mfma16_kernel(const ConvArgs<T> a) {
@@ -241,11 +242,11 @@ conv_mfma16_kernel(const ConvArgs<T> a) {
         const int first = (wave + G::NWAVE - (int)((blockIdx.x + win) % G::NWAVE)) % G::NWAVE;                            \
         const int nb = first < nblk ? (nblk - first + G::NWAVE - 1) / G::NWAVE : 0;                                       \
         switch (__builtin_amdgcn_readfirstlane(nb)) {                                                                     \
-            case 0: mfma16_window<T, G, CIB, COH, 0, MODE>(a, co0, nc, nitem, tree_items, first, wl, LISTS_OBJ, patch, Wl, bias_l); break; \
-            case 1: mfma16_window<T, G, CIB, COH, 1, MODE>(a, co0, nc, nitem, tree_items, first, wl, LISTS_OBJ, patch, Wl, bias_l); break; \
-            case 2: mfma16_window<T, G, CIB, COH, 2, MODE>(a, co0, nc, nitem, tree_items, first, wl, LISTS_OBJ, patch, Wl, bias_l); break; \
-            case 3: mfma16_window<T, G, CIB, COH, 3, MODE>(a, co0, nc, nitem, tree_items, first, wl, LISTS_OBJ, patch, Wl, bias_l); break; \
-            default: mfma16_window<T, G, CIB, COH, 4, MODE>(a, co0, nc, nitem, tree_items, first, wl, LISTS_OBJ, patch, Wl, bias_l); break; \
+            case 0: mfma16_window<T, G, CIB, COH, 0, MODE, FUSE>(a, co0, nc, nitem, tree_items, first, wl, LISTS_OBJ, patch, Wl, bias_l); break; \
+            case 1: mfma16_window<T, G, CIB, COH, 1, MODE, FUSE>(a, co0, nc, nitem, tree_items, first, wl, LISTS_OBJ, patch, Wl, bias_l); break; \
+            case 2: mfma16_window<T, G, CIB, COH, 2, MODE, FUSE>(a, co0, nc, nitem, tree_items, first, wl, LISTS_OBJ, patch, Wl, bias_l); break; \
+            case 3: mfma16_window<T, G, CIB, COH, 3, MODE, FUSE>(a, co0, nc, nitem, tree_items, first, wl, LISTS_OBJ, patch, Wl, bias_l); break; \
+            default: mfma16_window<T, G, CIB, COH, 4, MODE, FUSE>(a, co0, nc, nitem, tree_items, first, wl, LISTS_OBJ, patch, Wl, bias_l); break; \
         }                                                                                                                 \
     }
 
@@ -336,7 +337,7 @@ __device__ __forceinline__ void store_items_bf16(const ItemRegs<G, bf16_t, BF_CI
     }
 }
 
-template <class G, int COH, int NB, class Lists>
+template <class G, int COH, int NB, bool FUSE, class Lists>
 __device__ __forceinline__ void mfma_bf16_window(const ConvArgs<bf16_t>& a, int co0, int nc, int nitem, bool tree_items, int first,
                                                  const uint4* __restrict__ wl, const Lists& sh,
                                                  uint2* __restrict__ patch8, uint2* __restrict__ Wl8,
@@ -374,7 +375,7 @@ __device__ __forceinline__ void mfma_bf16_window(const ConvArgs<bf16_t>& a, int 
         const int i = threadIdx.x + k * G::NT;                                                     \
         if (i < W16) reinterpret_cast<uint4*>(Wl8)[i] = wr[k];                                     \
     }
-    load_items<G, bf16_t, BF_CIB>(a, 0, nitem, tree_items, sh, R);
+    load_items<G, bf16_t, BF_CIB>(a, 0, nitem, tree_items, sh, R, 0, std::bool_constant<FUSE>{});
     APRNET_LOAD_WEIGHTS(0)
     for (int i = threadIdx.x; i < 2 * G::CH_STRIDE; i += G::NT) patch8[i] = make_uint2(0u, 0u);     // once per window
     for (int ci0 = 0; ci0 < a.Cin; ci0 += BF_CIB) {
@@ -384,7 +385,7 @@ __device__ __forceinline__ void mfma_bf16_window(const ConvArgs<bf16_t>& a, int 
         APRNET_STORE_WEIGHTS()
         __syncthreads();
         if (ci0 + BF_CIB < a.Cin) {
-            load_values<G, bf16_t, BF_CIB>(a, ci0 + BF_CIB, nitem, tree_items, R);
+            load_values<G, bf16_t, BF_CIB>(a, ci0 + BF_CIB, nitem, tree_items, R, 0, std::bool_constant<FUSE>{});
             APRNET_LOAD_WEIGHTS(ci0 / BF_CIB + 1)
         }
 #pragma unroll
@@ -417,14 +418,14 @@ __device__ __forceinline__ void mfma_bf16_window(const ConvArgs<bf16_t>& a, int 
             for (int r = 0; r < 4; ++r) {
                 const int cl = h * 16 + 4 * (lane >> 4) + r;
                 float v = acc[j][h][r] + bias_l[cl];
-                if (a.relu) v = v < 0.f ? 0.f : v;
+                if (FUSE && a.relu) v = v < 0.f ? 0.f : v;
                 if (co0 + cl < a.Cout) a.y[(int64_t)(co0 + cl) * a.ldy + o] = float_to_bf16(v);
             }
     }
 }
 
 // The windows of the tile come as precomputed lists from the plan.
-template <class G, int COH>
+template <class G, int COH, bool FUSE = false>
 __global__ void __launch_bounds__(G::NT) __attribute__((amdgpu_waves_per_eu(4, 4)))      // two workgroups per CU
 conv_mfma_bf16_kernel(const ConvArgs<bf16_t> a) {
     constexpr int NBW = 4, NSTEP = bf16_steps<G>();
@@ -458,11 +459,11 @@ conv_mfma_bf16_kernel(const ConvArgs<bf16_t> a) {
         const int first = (wave - (int)blockIdx.x - win) & (G::NWAVE - 1);
         const int nb = first < nblk ? (nblk - first + G::NWAVE - 1) / G::NWAVE : 0;
         switch (__builtin_amdgcn_readfirstlane(nb)) {
-            case 0: mfma_bf16_window<G, COH, 0>(a, co0, nc, nitem, tree_items, first, wl, gl, patch8, Wl8, bias_l); break;
-            case 1: mfma_bf16_window<G, COH, 1>(a, co0, nc, nitem, tree_items, first, wl, gl, patch8, Wl8, bias_l); break;
-            case 2: mfma_bf16_window<G, COH, 2>(a, co0, nc, nitem, tree_items, first, wl, gl, patch8, Wl8, bias_l); break;
-            case 3: mfma_bf16_window<G, COH, 3>(a, co0, nc, nitem, tree_items, first, wl, gl, patch8, Wl8, bias_l); break;
-            default: mfma_bf16_window<G, COH, 4>(a, co0, nc, nitem, tree_items, first, wl, gl, patch8, Wl8, bias_l); break;
+            case 0: mfma_bf16_window<G, COH, 0, FUSE>(a, co0, nc, nitem, tree_items, first, wl, gl, patch8, Wl8, bias_l); break;
+            case 1: mfma_bf16_window<G, COH, 1, FUSE>(a, co0, nc, nitem, tree_items, first, wl, gl, patch8, Wl8, bias_l); break;
+            case 2: mfma_bf16_window<G, COH, 2, FUSE>(a, co0, nc, nitem, tree_items, first, wl, gl, patch8, Wl8, bias_l); break;
+            case 3: mfma_bf16_window<G, COH, 3, FUSE>(a, co0, nc, nitem, tree_items, first, wl, gl, patch8, Wl8, bias_l); break;
+            default: mfma_bf16_window<G, COH, 4, FUSE>(a, co0, nc, nitem, tree_items, first, wl, gl, patch8, Wl8, bias_l); break;
         }
         __syncthreads();        // the next window rewrites the patch
     }
@@ -485,9 +486,16 @@ template <typename T, class G, int MODE>
 static int launch16(const ConvArgs<T>& a, int n_tiles, hipStream_t st) {
     const int coh = conv_coh(a.Cout);
     dim3 grid((unsigned)n_tiles, (unsigned)((a.Cout + 16 * coh - 1) / (16 * coh)));
-    if (MODE == 0 && a.tile_win) {
+    const bool fuse = MODE == 0 && (a.relu || a.x2);
+    if (MODE == 0 && a.tile_win && fuse) {
+        if (coh == 1) hipLaunchKernelGGL((conv_mfma16_kernel<T, G, 1, 0, true, true>), grid, dim3(G::NT), 0, st, a);
+        else hipLaunchKernelGGL((conv_mfma16_kernel<T, G, 2, 0, true, true>), grid, dim3(G::NT), 0, st, a);
+    } else if (MODE == 0 && a.tile_win) {
         if (coh == 1) hipLaunchKernelGGL((conv_mfma16_kernel<T, G, 1, 0, true>), grid, dim3(G::NT), 0, st, a);
         else hipLaunchKernelGGL((conv_mfma16_kernel<T, G, 2, 0, true>), grid, dim3(G::NT), 0, st, a);
+    } else if (fuse) {
+        if (coh == 1) hipLaunchKernelGGL((conv_mfma16_kernel<T, G, 1, 0, false, true>), grid, dim3(G::NT), 0, st, a);
+        else hipLaunchKernelGGL((conv_mfma16_kernel<T, G, 2, 0, false, true>), grid, dim3(G::NT), 0, st, a);
     } else if (coh == 1) hipLaunchKernelGGL((conv_mfma16_kernel<T, G, 1, MODE, false>), grid, dim3(G::NT), 0, st, a);
     else hipLaunchKernelGGL((conv_mfma16_kernel<T, G, 2, MODE, false>), grid, dim3(G::NT), 0, st, a);
     APRNET_LAUNCH_CHECK("conv_mfma16_kernel");
@@ -515,7 +523,10 @@ template <class G>
 static int launch_bf16(const ConvArgs<bf16_t>& a, int n_tiles, hipStream_t st) {
     const int coh = conv_coh(a.Cout);
     dim3 grid((unsigned)n_tiles, (unsigned)((a.Cout + 16 * coh - 1) / (16 * coh)));
-    if (coh == 1) hipLaunchKernelGGL((conv_mfma_bf16_kernel<G, 1>), grid, dim3(G::NT), 0, st, a);
+    if (a.relu || a.x2) {
+        if (coh == 1) hipLaunchKernelGGL((conv_mfma_bf16_kernel<G, 1, true>), grid, dim3(G::NT), 0, st, a);
+        else hipLaunchKernelGGL((conv_mfma_bf16_kernel<G, 2, true>), grid, dim3(G::NT), 0, st, a);
+    } else if (coh == 1) hipLaunchKernelGGL((conv_mfma_bf16_kernel<G, 1>), grid, dim3(G::NT), 0, st, a);
     else hipLaunchKernelGGL((conv_mfma_bf16_kernel<G, 2>), grid, dim3(G::NT), 0, st, a);
     APRNET_LAUNCH_CHECK("conv_mfma_bf16_kernel");
     return 0;
