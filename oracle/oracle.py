@@ -154,6 +154,10 @@ def conv_backward(aprs, x, weights, grad_output, level_deltas):
 def restrict_kernel_forward(weights, num_levels):
     weights = weights.contiguous()
     cin, s, cout, kz, kx, ky = weights.shape
+    if num_levels < s:
+        # kernel.hpp:70-74 copies all given stencils into an output of num_levels entries: out of bounds in the
+        # reference when there are fewer levels than stencils.  Refused here (the product refuses it too).
+        raise ValueError("restrict_kernel_forward: fewer levels than stencils")
     out = torch.zeros(cin, num_levels, cout, kz, kx, ky, dtype=weights.dtype)
     getattr(lib(), "oracle_restrict_fwd_" + _sfx(weights))(_p(weights), _p(out), cin, s, num_levels, cout, kz, kx, ky)
     return out
@@ -162,6 +166,8 @@ def restrict_kernel_forward(weights, num_levels):
 def restrict_kernel_backward(grad_weights, num_stencils):
     grad_weights = grad_weights.contiguous()
     cin, se, cout, kz, kx, ky = grad_weights.shape
+    if se < num_stencils:
+        raise ValueError("restrict_kernel_backward: fewer levels than stencils")
     out = torch.zeros(cin, num_stencils, cout, kz, kx, ky, dtype=grad_weights.dtype)
     getattr(lib(), "oracle_restrict_bwd_" + _sfx(grad_weights))(_p(grad_weights), _p(out), cin, num_stencils, se, cout,
                                                                 kz, kx, ky)

@@ -503,3 +503,59 @@ def test_conv111_forward_fused_relu(dtype):
     close_bf16(got, ref) if dtype == torch.bfloat16 else close(got, ref, dtype)
     with pytest.raises(ValueError):
         _ops.conv_forward(aprs, x[:, :10].contiguous().to(dtype).to(DEV), wd, ld, x2=x[:, 10:].contiguous().to(dtype).to(DEV))
+
+
+# ------------------------------------------------------------------------------- degenerate access structures
+DEGENERATE = {
+    "dense": ((16, 16, 16), 1, 1.0, 0),        # every particle on the finest level, full tree
+    "coarse": ((12, 10, 14), 2, 0.0, 2),       # no cell asks for resolution: a handful of particles on level 1
+    "single": ((1, 1, 1), 3, 1.0, 0),          # one particle, one level, no tree level below it
+    "sliver": ((2, 3, 1), 4, 1.0, 0),
+    "line": ((5, 1, 1), 5, 0.5, 1),
+}
+
+
+@pytest.mark.parametrize("name", list(DEGENERATE))
+def test_degenerate_structures(name):
+    """Structures at the edges of what the access arrays can describe: all operators against the oracle at every
+    level delta they accept (forward and backward of the 3x3x3 convolution on both kernel families, pool with
+    argmax, upsample, tree fill through the convolution)."""
+    shape, seed, dens, drop = DEGENERATE[name]
+    apr = apr_cases.random_apr(shape, seed, dens, drop)
+    lib = _native.hip()
+    for d in range(max(apr.level_max() - 1, 1)):
+        n = oracle.number_parts(apr, d)
+        assert _ops.number_particles(apr, d) == n
+        ld = torch.tensor([d], dtype=torch.int32)
+        g = torch.Generator().manual_seed(7 + d)
+        x = torch.randn(1, 3, n, generator=g)
+        levels = apr.level_max() - apr.level_min() + 1
+        w = torch.randn(3, min(2, levels), 5, 3, 3, 3, generator=g)
+        w_exp = oracle.restrict_kernel_forward(w, levels)
+        wd = w_exp.permute(1, 2, 0, 3, 4, 5).contiguous().to(DEV)
+        ref = oracle.conv_forward([apr], x, w_exp, ld)
+        go = torch.randn(ref.shape, generator=g)
+        ref_gx, ref_gw = oracle.conv_backward([apr], x, w_exp, go, ld)
+        for path in (0, 1):
+            assert lib.aprnet_set_conv_path(path) == 0
+            try:
+                got = _ops.conv_forward([apr], x.to(DEV), wd, ld)
+                gx, gw = _ops.conv_backward([apr], x.to(DEV), wd, go.to(DEV), ld)
+            finally:
+                lib.aprnet_set_conv_path(0)
+            close(got, ref, torch.float32)
+            close(gx, ref_gx, torch.float32)
+            close(gw.permute(2, 0, 1, 3, 4, 5), ref_gw, torch.float32)
+        if apr.level_max() - d - 1 >= apr.level_min():          # there is a level left to pool into
+            rp, ri = oracle.maxpool_forward([apr], x, ld)
+            gp, gi = _ops.maxpool_forward([apr], x.to(DEV), ld, -1e17)
+            assert torch.equal(gp.cpu(), rp) and torch.equal(gi.cpu(), ri)
+            ld1 = ld + 1
+            ru = oracle.upsample_const_forward([apr], rp, ld1)
+            assert torch.equal(_ops.upsample_const_forward([apr], gp, ld1).cpu(), ru)
+    # more stencils than levels: kernel.hpp:70-74 writes out of bounds there; refused on both sides
+    levels = apr.level_max() - apr.level_min() + 1
+    with pytest.raises(ValueError):
+        _ops.restrict_kernel_forward(torch.zeros(levels + 1, 2, 2, 3, 3, 3, device=DEV), levels)
+    with pytest.raises(ValueError):
+        oracle.restrict_kernel_forward(torch.zeros(2, levels + 1, 2, 3, 3, 3), levels)

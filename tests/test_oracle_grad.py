@@ -136,3 +136,14 @@ def test_restrict_kernel_invariants(k):
         ov = torch.tensor([0.5, 1.0, 0.5], dtype=torch.float64)     # overlap of source tap i with the centre cell / step
         expect = torch.einsum("zxy,z,x,y->", src, ov, ov, ov)
         torch.testing.assert_close(we[0, s, 0, 1, 1, 1], expect, rtol=1e-12, atol=1e-12)
+
+
+def test_restrict_kernel_refuses_fewer_levels_than_stencils():
+    """kernel.hpp:70-74 copies every given stencil into an output that holds num_levels of them, which writes out
+    of bounds when num_levels < num_stencils; the restatement raises instead of following it there."""
+    w = torch.zeros(2, 3, 2, 3, 3, 3)
+    with pytest.raises(ValueError):
+        oracle.restrict_kernel_forward(w, 2)
+    with pytest.raises(ValueError):
+        oracle.restrict_kernel_backward(torch.zeros(2, 2, 2, 3, 3, 3), 3)
+    assert tuple(oracle.restrict_kernel_forward(w, 3).shape) == (2, 3, 2, 3, 3, 3)
