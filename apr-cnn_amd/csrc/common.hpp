@@ -116,7 +116,7 @@ int fail(int code, const std::string& msg);
 // non-empty row groups for the convolution at `level_delta` (built on first use, cached in the plan)
 // `halo` > 0 also lists the row groups that lie within that many rows of a non-empty one
 int get_tiles(aprnet_plan* plan, int level_delta, int TZ, int TX, TileList* out, int halo = 0);
-int get_lists(aprnet_plan* plan, int level_delta, int code, const TileList& tl, WinLists* out, hipStream_t st);
+int get_lists(aprnet_plan* plan, int level_delta, int code, const TileList& tl, WinLists* out, hipStream_t st, bool dx = false);
 void free_lists(WinLists& wl);
 // makes plan->d_scratch at least `bytes` large (contents are lost when it grows)
 int plan_scratch(aprnet_plan* plan, size_t bytes, hipStream_t st);

@@ -136,7 +136,7 @@ int launch_conv_mfma(int code, const ConvArgs<float>& a, int n_tiles, hipStream_
 int launch_conv_mfma(int code, const ConvArgs<bf16_t>& a, int n_tiles, hipStream_t st);
 int launch_conv_mfma_bf16(int code, const ConvArgs<bf16_t>& a, int n_tiles, hipStream_t st);
 size_t conv_packed_bf16_bytes(int code, int S_exp, int Cout, int Cin);
-int pack_conv_weights_bf16(int code, const float* w, int S_exp, int Cout, int Cin, void* packed, hipStream_t st);
+int pack_conv_weights_bf16(int code, const float* w, int S_exp, int Cout, int Cin, void* packed, hipStream_t st, bool transposed = false);
 static int g_bf16_math = 1;      // bfloat16 features: 1 = bfloat16 matrix instructions, 0 = fp32 matrix instructions
 int fill_tree_for_conv(const aprnet_plan* p, int d, const bf16_t* x, int64_t ldx, int C, bf16_t* tree, int64_t ldt, hipStream_t st);
 size_t conv_packed_floats(int code, int S_exp, int Cm, int Ck, bool transposed);
@@ -144,17 +144,19 @@ int pack_conv_weights(int code, const float* w, int S_exp, int Cm, int Ck, bool 
 
 static int g_conv_path = 0;      // 0: matrix cores where available, 1: VALU kernels only
 int conv_path() { return g_conv_path; }
+int bf16_math();
 
 static int g_use_lists = 1;      // 1: forward kernels take the window lists of the plan, 0: they scan per call
+int bf16_math() { return g_bf16_math; }
 
 // Points the kernel at the plan's window lists.  When the lists are switched off, or cannot be built (no device
 // memory for them, too many entries), a.tile_win stays null and the kernel scans the access arrays itself.
 template <typename T>
-static int set_lists(aprnet_plan* p, int d, int code, const TileList& tl, ConvArgs<T>& a, hipStream_t st) {
+static int set_lists(aprnet_plan* p, int d, int code, const TileList& tl, ConvArgs<T>& a, hipStream_t st, bool dx = false) {
     a.tile_win = nullptr;
     if (!g_use_lists) return 0;
     WinLists wl;
-    if (get_lists(p, d, code, tl, &wl, st) != 0) { (void)hipGetLastError(); return 0; }
+    if (get_lists(p, d, code, tl, &wl, st, dx) != 0) { (void)hipGetLastError(); return 0; }
     a.tile_win = wl.d_tile_win; a.win = wl.d_win;
     a.l_item_idx = wl.d_item_idx; a.l_item_pos = wl.d_item_pos; a.l_col_idx = wl.d_col_idx; a.l_col_pos = wl.d_col_pos;
     return 0;
@@ -162,6 +164,8 @@ static int set_lists(aprnet_plan* p, int d, int code, const TileList& tl, ConvAr
 
 int set_conv_lists(aprnet_plan* p, int d, int code, const TileList& tl, ConvArgs<float>& a, hipStream_t st) { return set_lists(p, d, code, tl, a, st); }
 int set_conv_lists(aprnet_plan* p, int d, int code, const TileList& tl, ConvArgs<bf16_t>& a, hipStream_t st) { return set_lists(p, d, code, tl, a, st); }
+// the input-gradient lists (tl: the tile list with a halo of one row)
+int set_conv_dx_lists(aprnet_plan* p, int d, int code, const TileList& tl, ConvArgs<bf16_t>& a, hipStream_t st) { return set_lists(p, d, code, tl, a, st, true); }
 
 template <typename T> static int try_mfma(aprnet_plan*, const ConvArgs<T>&, int, int, const TileList&, int, hipStream_t, bool*) { return 0; }
 template <> int try_mfma<float>(aprnet_plan* p, const ConvArgs<float>& a, int code, int d, const TileList& tl, int n_tiles,

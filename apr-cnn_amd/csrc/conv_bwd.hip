@@ -238,6 +238,11 @@ int conv_path();
 // points a at the plan's window lists (conv.hip); leaves a.tile_win null when they are off or unavailable
 int set_conv_lists(aprnet_plan* p, int d, int code, const TileList& tl, ConvArgs<float>& a, hipStream_t st);
 int set_conv_lists(aprnet_plan* p, int d, int code, const TileList& tl, ConvArgs<bf16_t>& a, hipStream_t st);
+int set_conv_dx_lists(aprnet_plan* p, int d, int code, const TileList& tl, ConvArgs<bf16_t>& a, hipStream_t st);
+int launch_conv_dx_mfma_bf16(int code, const ConvArgs<bf16_t>& a, int n_tiles, hipStream_t st);
+size_t conv_packed_bf16_bytes(int code, int S_exp, int Cout, int Cin);
+int pack_conv_weights_bf16(int code, const float* w, int S_exp, int Cout, int Cin, void* packed, hipStream_t st, bool transposed);
+int bf16_math();
 
 template <typename T> static int try_mfma_bwd(aprnet_plan*, const ConvArgs<T>&, const TileList&, int, int, hipStream_t, bool*) { return 0; }
 template <> int try_mfma_bwd<float>(aprnet_plan* p, const ConvArgs<float>& a, const TileList& tl, int code, int d, hipStream_t st, bool* done) {
@@ -339,13 +344,26 @@ int conv_bwd_bf16(const aprnet_plan* cp, int d, int kz, int kx, int ky, const bf
         a.tree_data = tree_ws; a.ldt = ldt; a.Lc = p->lc(d); a.tree_off = p->tree_offset(a.Lc);
         a.x_count = np; a.t_count = nt;
         a.gy = gy; a.ldy = ldy; a.gx = gx32_ws; a.ldgx = ldgx32; a.gtree = gtree_ws; a.ldgt = ldgt; a.gw = gw;
-        if (int rc = plan_scratch(p, conv_packed_floats(code, S_exp, Cin, Cout, true) * sizeof(float), st)) return rc;
-        if (int rc = pack_conv_weights(code, w, S_exp, Cin, Cout, true, (float*)p->d_scratch, st)) return rc;
         ConvArgs<bf16_t> b = a;
         b.tiles = near.d_tiles; b.n_tiles = near.n;
-        b.x = gy; b.ldx = ldy; b.Cin = Cout; b.Cout = Cin; b.w = (const float*)p->d_scratch; b.bias = nullptr;
+        b.x = gy; b.ldx = ldy; b.Cin = Cout; b.Cout = Cin; b.bias = nullptr;
         b.tree_data = nullptr; b.t_count = 0;
-        if (near.n > 0) if (int rc = launch_conv_dx_mfma(code, b, near.n, st)) return rc;
+        // input gradient: bfloat16 products on the input-gradient lists of the plan when they are there, otherwise
+        // (lists off or not buildable, fp32 products asked for) the scanning kernel with fp32 products
+        if (near.n > 0 && bf16_math())
+            if (int rc = set_conv_dx_lists(p, d, code, near, b, st)) return rc;
+        if (near.n > 0 && b.tile_win) {
+            if (int rc = plan_scratch(p, conv_packed_bf16_bytes(code, S_exp, Cin, Cout), st)) return rc;
+            if (int rc = pack_conv_weights_bf16(code, w, S_exp, Cin, Cout, p->d_scratch, st, true)) return rc;
+            b.w = (const float*)p->d_scratch;
+            if (int rc = launch_conv_dx_mfma_bf16(code, b, near.n, st)) return rc;
+        } else if (near.n > 0) {
+            if (int rc = plan_scratch(p, conv_packed_floats(code, S_exp, Cin, Cout, true) * sizeof(float), st)) return rc;
+            if (int rc = pack_conv_weights(code, w, S_exp, Cin, Cout, true, (float*)p->d_scratch, st)) return rc;
+            b.w = (const float*)p->d_scratch;
+            b.tile_win = nullptr;
+            if (int rc = launch_conv_dx_mfma(code, b, near.n, st)) return rc;
+        }
         if (int rc = set_conv_lists(p, d, code, tl, a, st)) return rc;
         if (int rc = launch_conv_dw_mfma(code, a, tl, p->apr.level_min, st)) return rc;
     }

@@ -153,6 +153,7 @@ struct ScanArgs {
     int tree_off, yn, y0;
     bool tree_from_x, out_tree;
     int z0, x0, zn, xn;             // tile origin and level extent (input-gradient scan only)
+    bool pool;                      // input-gradient scan: one pooled column per coarser particle (COL_BOX)
 };
 
 template <class G>
@@ -319,7 +320,7 @@ __device__ __attribute__((noinline)) void scan_window_dx_impl(const ScanArgs a, 
                 const bool rows_full = (BOXZ == 1 || (z | 1) < a.zn) && (x | 1) < a.xn;
                 const bool first_row = (BOXZ == 1 || (z & 1) == 0) && (x & 1) == 0;
                 const bool ina = in && ya >= y0 && ya < y0 + G::TY;
-                const bool pooled = rows_full && yb < yn;
+                const bool pooled = a.pool && rows_full && yb < yn;
                 const bool oa = ina && (!pooled || first_row);
                 const bool ob = in && !pooled && yb >= y0 && yb < y0 + G::TY && yb < yn;
                 const unsigned long long ma = __ballot(oa), mb = __ballot(ob);
@@ -349,11 +350,11 @@ __device__ __attribute__((noinline)) void scan_window_dx_impl(const ScanArgs a, 
 
 template <class G, typename T>
 __device__ __forceinline__ void scan_window_dx(const ConvArgs<T>& a, int L, int z0, int x0, int y0, bool out_tree,
-                                               ConvShared<G>& sh) {
+                                               ConvShared<G>& sh, bool pool = true) {
     ScanArgs s;
     s.apr_y = a.apr.y; s.tree_y = a.tree.y; s.tree_off = (int)a.tree_off; s.yn = a.apr.y_num[L]; s.y0 = y0;
     s.tree_from_x = (L == a.Lc); s.out_tree = out_tree;
-    s.z0 = z0; s.x0 = x0; s.zn = a.apr.z_num[L]; s.xn = a.apr.x_num[L];
+    s.z0 = z0; s.x0 = x0; s.zn = a.apr.z_num[L]; s.xn = a.apr.x_num[L]; s.pool = pool;
     scan_window_dx_impl<G>(s, sh);
 }
 

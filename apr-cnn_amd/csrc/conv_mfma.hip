@@ -295,8 +295,10 @@ constexpr int BF_CIB = 8;
 template <class G> constexpr int bf16_steps() { return (G::K + 1) / 2; }
 
 // packedB[s][cb][q][step][h][lane] (8 bytes each), cb = block of 16 * COH output channels, q = chunk of 8 inputs
+// With `transposed` the image is that of the input gradient's stencil: the channel axes swap roles (Cout then
+// names the input channels of the layer, Cin its output channels) and the taps are reversed.
 __global__ void pack_weights_bf16_kernel(const float* __restrict__ w, int S_exp, int Cout, int Cin, int K, int COH,
-                                         uint2* __restrict__ out) {
+                                         int transposed, uint2* __restrict__ out) {
     const int ncb = (Cout + 16 * COH - 1) / (16 * COH), nq = (Cin + BF_CIB - 1) / BF_CIB, nstep = (K + 1) / 2;
     const int64_t n = (int64_t)S_exp * ncb * nq * nstep * COH * 64;
     for (int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; e < n; e += (int64_t)gridDim.x * blockDim.x) {
@@ -313,7 +315,9 @@ __global__ void pack_weights_bf16_kernel(const float* __restrict__ w, int S_exp,
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
             float f = 0.f;
-            if (t < K && co < Cout && ci0 + j < Cin) f = w[(((int64_t)s * Cout + co) * Cin + ci0 + j) * K + t];
+            if (t < K && co < Cout && ci0 + j < Cin)
+                f = transposed ? w[(((int64_t)s * Cin + ci0 + j) * Cout + co) * K + (K - 1 - t)]
+                               : w[(((int64_t)s * Cout + co) * Cin + ci0 + j) * K + t];
             v[j] = float_to_bf16(f).bits;
         }
         out[e] = make_uint2(v[0] | (v[1] << 16), v[2] | (v[3] << 16));
@@ -337,7 +341,9 @@ __device__ __forceinline__ void store_items_bf16(const ItemRegs<G, bf16_t, BF_CI
     }
 }
 
-template <class G, int COH, int NB, bool FUSE, class Lists>
+// MODE 0: forward.  MODE 1: input gradient (items = output gradient, results added atomically in fp32 to the place
+// each column names, as in the fp32 kernel; no pooled columns).
+template <class G, int COH, int NB, bool FUSE, int MODE, class Lists>
 __device__ __forceinline__ void mfma_bf16_window(const ConvArgs<bf16_t>& a, int co0, int nc, int nitem, bool tree_items, int first,
                                                  const uint4* __restrict__ wl, const Lists& sh,
                                                  uint2* __restrict__ patch8, uint2* __restrict__ Wl8,
@@ -412,20 +418,33 @@ __device__ __forceinline__ void mfma_bf16_window(const ConvArgs<bf16_t>& a, int 
         const int col = ((first + G::NWAVE * j) << 4) + (lane & 15);
         if (col >= nc) continue;
         const int64_t o = sh.col_idx[col];
+        if constexpr (MODE == 0) {
 #pragma unroll
-        for (int h = 0; h < COH; ++h)
+            for (int h = 0; h < COH; ++h)
 #pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                const int cl = h * 16 + 4 * (lane >> 4) + r;
-                float v = acc[j][h][r] + bias_l[cl];
-                if (FUSE && a.relu) v = v < 0.f ? 0.f : v;
-                if (co0 + cl < a.Cout) a.y[(int64_t)(co0 + cl) * a.ldy + o] = float_to_bf16(v);
-            }
+                for (int r = 0; r < 4; ++r) {
+                    const int cl = h * 16 + 4 * (lane >> 4) + r;
+                    float v = acc[j][h][r] + bias_l[cl];
+                    if (FUSE && a.relu) v = v < 0.f ? 0.f : v;
+                    if (co0 + cl < a.Cout) a.y[(int64_t)(co0 + cl) * a.ldy + o] = float_to_bf16(v);
+                }
+        } else {
+            const bool to_tree = (sh.col_pos[col] & COL_TREE) != 0;
+            float* dst = (to_tree ? a.gtree : a.gx) + o;
+            const int64_t ld = to_tree ? a.ldgt : a.ldgx;
+#pragma unroll
+            for (int h = 0; h < COH; ++h)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const int cl = h * 16 + 4 * (lane >> 4) + r;
+                    if (co0 + cl < a.Cout) unsafeAtomicAdd(dst + (int64_t)(co0 + cl) * ld, acc[j][h][r]);
+                }
+        }
     }
 }
 
 // The windows of the tile come as precomputed lists from the plan.
-template <class G, int COH, bool FUSE = false>
+template <class G, int COH, bool FUSE = false, int MODE = 0>
 __global__ void __launch_bounds__(G::NT) __attribute__((amdgpu_waves_per_eu(4, 4)))      // two workgroups per CU
 conv_mfma_bf16_kernel(const ConvArgs<bf16_t> a) {
     constexpr int NBW = 4, NSTEP = bf16_steps<G>();
@@ -444,10 +463,10 @@ conv_mfma_bf16_kernel(const ConvArgs<bf16_t> a) {
     const uint4* __restrict__ wl = reinterpret_cast<const uint4*>(a.w) +
                                    ((int64_t)s_idx * gridDim.y + blockIdx.y) * nq * (NSTEP * COH * 32);
     const int wave = threadIdx.x >> 6;
-    const bool tree_items = L < a.Lc;
+    const bool tree_items = MODE == 0 && L < a.Lc;       // the output gradient has no tree part
 
     if (threadIdx.x < 16 * COH)
-        bias_l[threadIdx.x] = (a.bias && co0 + (int)threadIdx.x < a.Cout) ? a.bias[co0 + threadIdx.x] : 0.f;
+        bias_l[threadIdx.x] = (MODE == 0 && a.bias && co0 + (int)threadIdx.x < a.Cout) ? a.bias[co0 + threadIdx.x] : 0.f;
 
     const int wb = a.tile_win[blockIdx.x], we = a.tile_win[blockIdx.x + 1];
     for (int w = wb; w < we; ++w) {
@@ -459,11 +478,11 @@ conv_mfma_bf16_kernel(const ConvArgs<bf16_t> a) {
         const int first = (wave - (int)blockIdx.x - win) & (G::NWAVE - 1);
         const int nb = first < nblk ? (nblk - first + G::NWAVE - 1) / G::NWAVE : 0;
         switch (__builtin_amdgcn_readfirstlane(nb)) {
-            case 0: mfma_bf16_window<G, COH, 0, FUSE>(a, co0, nc, nitem, tree_items, first, wl, gl, patch8, Wl8, bias_l); break;
-            case 1: mfma_bf16_window<G, COH, 1, FUSE>(a, co0, nc, nitem, tree_items, first, wl, gl, patch8, Wl8, bias_l); break;
-            case 2: mfma_bf16_window<G, COH, 2, FUSE>(a, co0, nc, nitem, tree_items, first, wl, gl, patch8, Wl8, bias_l); break;
-            case 3: mfma_bf16_window<G, COH, 3, FUSE>(a, co0, nc, nitem, tree_items, first, wl, gl, patch8, Wl8, bias_l); break;
-            default: mfma_bf16_window<G, COH, 4, FUSE>(a, co0, nc, nitem, tree_items, first, wl, gl, patch8, Wl8, bias_l); break;
+            case 0: mfma_bf16_window<G, COH, 0, FUSE, MODE>(a, co0, nc, nitem, tree_items, first, wl, gl, patch8, Wl8, bias_l); break;
+            case 1: mfma_bf16_window<G, COH, 1, FUSE, MODE>(a, co0, nc, nitem, tree_items, first, wl, gl, patch8, Wl8, bias_l); break;
+            case 2: mfma_bf16_window<G, COH, 2, FUSE, MODE>(a, co0, nc, nitem, tree_items, first, wl, gl, patch8, Wl8, bias_l); break;
+            case 3: mfma_bf16_window<G, COH, 3, FUSE, MODE>(a, co0, nc, nitem, tree_items, first, wl, gl, patch8, Wl8, bias_l); break;
+            default: mfma_bf16_window<G, COH, 4, FUSE, MODE>(a, co0, nc, nitem, tree_items, first, wl, gl, patch8, Wl8, bias_l); break;
         }
         __syncthreads();        // the next window rewrites the patch
     }
@@ -520,10 +539,13 @@ int launch_conv_mfma(int code, const ConvArgs<bf16_t>& a, int n_tiles, hipStream
 
 // bfloat16 features, bfloat16 contraction (a.w = image of pack_conv_weights_bf16)
 template <class G>
-static int launch_bf16(const ConvArgs<bf16_t>& a, int n_tiles, hipStream_t st) {
+static int launch_bf16(const ConvArgs<bf16_t>& a, int n_tiles, hipStream_t st, bool dx = false) {
     const int coh = conv_coh(a.Cout);
     dim3 grid((unsigned)n_tiles, (unsigned)((a.Cout + 16 * coh - 1) / (16 * coh)));
-    if (a.relu || a.x2) {
+    if (dx) {
+        if (coh == 1) hipLaunchKernelGGL((conv_mfma_bf16_kernel<G, 1, false, 1>), grid, dim3(G::NT), 0, st, a);
+        else hipLaunchKernelGGL((conv_mfma_bf16_kernel<G, 2, false, 1>), grid, dim3(G::NT), 0, st, a);
+    } else if (a.relu || a.x2) {
         if (coh == 1) hipLaunchKernelGGL((conv_mfma_bf16_kernel<G, 1, true>), grid, dim3(G::NT), 0, st, a);
         else hipLaunchKernelGGL((conv_mfma_bf16_kernel<G, 2, true>), grid, dim3(G::NT), 0, st, a);
     } else if (coh == 1) hipLaunchKernelGGL((conv_mfma_bf16_kernel<G, 1>), grid, dim3(G::NT), 0, st, a);
@@ -539,15 +561,26 @@ int launch_conv_mfma_bf16(int code, const ConvArgs<bf16_t>& a, int n_tiles, hipS
     }
     return fail(APRNET_ERR_UNSUPPORTED, "no matrix-core kernel for this stencil");
 }
+// Input gradient with bfloat16 products: a.x / a.Cin describe the output gradient, a.Cout the layer's input channels,
+// a.w the transposed image of pack_conv_weights_bf16, a.tile_win ... the input-gradient lists of the plan.
+int launch_conv_dx_mfma_bf16(int code, const ConvArgs<bf16_t>& a, int n_tiles, hipStream_t st) {
+    switch (code) {
+        case 333: return launch_bf16<M333N>(a, n_tiles, st, true);
+        case 133: return launch_bf16<M133N>(a, n_tiles, st, true);
+        case 155: return launch_bf16<M155N>(a, n_tiles, st, true);
+    }
+    return fail(APRNET_ERR_UNSUPPORTED, "no matrix-core kernel for this stencil");
+}
 size_t conv_packed_bf16_bytes(int code, int S_exp, int Cout, int Cin) {
     const int coh = conv_coh(Cout), nstep = (conv_taps(code) + 1) / 2;
     return (size_t)S_exp * ((Cout + 16 * coh - 1) / (16 * coh)) * ((Cin + BF_CIB - 1) / BF_CIB) * nstep * coh * 64 * sizeof(uint2);
 }
-int pack_conv_weights_bf16(int code, const float* w, int S_exp, int Cout, int Cin, void* packed, hipStream_t st) {
+// Cout / Cin: channels on the M axis of the kernel / contracted channels (transposed: the layer's Cin / Cout)
+int pack_conv_weights_bf16(int code, const float* w, int S_exp, int Cout, int Cin, void* packed, hipStream_t st, bool transposed) {
     const size_t n = conv_packed_bf16_bytes(code, S_exp, Cout, Cin) / sizeof(uint2);
     dim3 grid((unsigned)std::min<size_t>((n + 255) / 256, 2048));
     hipLaunchKernelGGL(pack_weights_bf16_kernel, grid, dim3(256), 0, st, w, S_exp, Cout, Cin, conv_taps(code), conv_coh(Cout),
-                       (uint2*)packed);
+                       transposed ? 1 : 0, (uint2*)packed);
     APRNET_LAUNCH_CHECK("pack_weights_bf16_kernel");
     return 0;
 }

@@ -11,7 +11,9 @@
 
 namespace aprnet {
 
-template <class G>
+// DX: lists of the input gradient (scan_window_dx without pooled columns) over the tiles within one row of an
+// output; windows without an output position are not stored.
+template <class G, bool DX>
 __global__ void __launch_bounds__(G::NT)
 build_lists_kernel(const ConvArgs<float> a, const int pass, int4* __restrict__ tile_counts, const int4* __restrict__ tile_off,
                    int4* __restrict__ win, int* __restrict__ item_idx, unsigned short* __restrict__ item_pos,
@@ -28,10 +30,11 @@ build_lists_kernel(const ConvArgs<float> a, const int pass, int4* __restrict__ t
     open_segments<G, float>(a, L, tile.z0, tile.x0, sh);
     __syncthreads();
     for (int y0 = 0; y0 < yn; y0 += G::TY) {
-        scan_window<G, float>(a, L, y0, out_tree, sh);
+        if constexpr (DX) scan_window_dx<G, float>(a, L, tile.z0, tile.x0, y0, out_tree, sh, false);
+        else scan_window<G, float>(a, L, y0, out_tree, sh);
         __syncthreads();
         const int nc = sh.ncol, nitem = sh.nitem;
-        if (nc > 0) {
+        if (nc > 0 && (!DX || nitem > 0)) {
             if (pass == 1) {
                 // list offsets are unsigned 32-bit numbers stored in the int fields of the header
                 const unsigned ib = (unsigned)off.y + (unsigned)ni, cb = (unsigned)off.z + (unsigned)ncl;
@@ -54,16 +57,20 @@ using L155 = ConvGeom<1, 5, 5, 1, 8, 512>;
 
 template <class G>
 static void launch_build(const ConvArgs<float>& a, int n_tiles, int pass, int4* counts, const int4* offs, const WinLists& wl,
-                         hipStream_t st) {
-    hipLaunchKernelGGL(build_lists_kernel<G>, dim3((unsigned)n_tiles), dim3(G::NT), 0, st, a, pass, counts, offs, wl.d_win,
-                       wl.d_item_idx, wl.d_item_pos, wl.d_col_idx, wl.d_col_pos);
+                         bool dx, hipStream_t st) {
+    if (dx)
+        hipLaunchKernelGGL((build_lists_kernel<G, true>), dim3((unsigned)n_tiles), dim3(G::NT), 0, st, a, pass, counts, offs,
+                           wl.d_win, wl.d_item_idx, wl.d_item_pos, wl.d_col_idx, wl.d_col_pos);
+    else
+        hipLaunchKernelGGL((build_lists_kernel<G, false>), dim3((unsigned)n_tiles), dim3(G::NT), 0, st, a, pass, counts, offs,
+                           wl.d_win, wl.d_item_idx, wl.d_item_pos, wl.d_col_idx, wl.d_col_pos);
 }
 
 static void launch_build_code(int code, const ConvArgs<float>& a, int n_tiles, int pass, int4* counts, const int4* offs,
-                              const WinLists& wl, hipStream_t st) {
-    if (code == 333) launch_build<L333>(a, n_tiles, pass, counts, offs, wl, st);
-    else if (code == 133) launch_build<L133>(a, n_tiles, pass, counts, offs, wl, st);
-    else launch_build<L155>(a, n_tiles, pass, counts, offs, wl, st);
+                              const WinLists& wl, bool dx, hipStream_t st) {
+    if (code == 333) launch_build<L333>(a, n_tiles, pass, counts, offs, wl, dx, st);
+    else if (code == 133) launch_build<L133>(a, n_tiles, pass, counts, offs, wl, dx, st);
+    else launch_build<L155>(a, n_tiles, pass, counts, offs, wl, dx, st);
 }
 
 void free_lists(WinLists& wl) {
@@ -75,8 +82,9 @@ void free_lists(WinLists& wl) {
 
 // Lists of the forward convolution at `level_delta` for stencil `code` (333, 133, 155); `tl` must be the tile list
 // of the same stencil.  Built on first use (synchronises the stream and allocates), then served from the plan.
-int get_lists(aprnet_plan* p, int level_delta, int code, const TileList& tl, WinLists* out, hipStream_t st) {
-    auto key = std::make_pair(level_delta, code);
+// dx: the lists of the input gradient instead; `tl` is then the tile list with a halo of one row.
+int get_lists(aprnet_plan* p, int level_delta, int code, const TileList& tl, WinLists* out, hipStream_t st, bool dx) {
+    auto key = std::make_pair(level_delta, code + (dx ? 1000 : 0));
     auto it = p->lists.find(key);
     if (it != p->lists.end()) {
         *out = it->second;
@@ -90,7 +98,7 @@ int get_lists(aprnet_plan* p, int level_delta, int code, const TileList& tl, Win
         a.apr = p->dapr; a.tree = p->dtree; a.tiles = tl.d_tiles; a.Lc = p->lc(level_delta); a.tree_off = p->tree_offset(a.Lc);
         int4* d_counts = nullptr; int4* d_offs = nullptr;
         APRNET_HIP_CHECK(hipMalloc((void**)&d_counts, (size_t)tl.n * sizeof(int4)));
-        launch_build_code(code, a, tl.n, 0, d_counts, nullptr, wl, st);
+        launch_build_code(code, a, tl.n, 0, d_counts, nullptr, wl, dx, st);
         APRNET_LAUNCH_CHECK("build_lists_kernel (count)");
         std::vector<int4> counts(tl.n), offs(tl.n);
         APRNET_HIP_CHECK(hipStreamSynchronize(st));
@@ -119,7 +127,7 @@ int get_lists(aprnet_plan* p, int level_delta, int code, const TileList& tl, Win
         if (rc) { (void)hipFree(d_counts); if (d_offs) (void)hipFree(d_offs); free_lists(wl); return rc; }
         APRNET_HIP_CHECK(hipMemcpy(d_offs, offs.data(), (size_t)tl.n * sizeof(int4), hipMemcpyHostToDevice));
         APRNET_HIP_CHECK(hipMemcpy(wl.d_tile_win, tile_win.data(), tile_win.size() * sizeof(int), hipMemcpyHostToDevice));
-        launch_build_code(code, a, tl.n, 1, d_counts, d_offs, wl, st);
+        launch_build_code(code, a, tl.n, 1, d_counts, d_offs, wl, dx, st);
         APRNET_LAUNCH_CHECK("build_lists_kernel (fill)");
         APRNET_HIP_CHECK(hipStreamSynchronize(st));
         (void)hipFree(d_counts); (void)hipFree(d_offs);

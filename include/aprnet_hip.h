@@ -180,7 +180,7 @@ APRNET_DECL(double, f64)
  * and bias are passed in fp32; the stencil convolution (3x3x3, 1x3x3, 1x5x5) rounds the weights to bfloat16
  * and multiplies on the bfloat16 matrix cores (aprnet_set_conv_path(3) keeps the weights and the products
  * in fp32).  Forward operators of the APR-UNet, plus the backward passes
- * of pool / upsample / tree fill and of the stencil convolution (fp32 matrix instructions).  Argument meaning as
+ * of pool / upsample / tree fill and of the stencil convolution.  Argument meaning as
  * for the _f32 entry points. */
 int aprnet_conv_fwd_bf16(const aprnet_plan*, int level_delta, int kz, int kx, int ky, const uint16_t* x, int64_t ldx, int Cin,
                          const float* w, int S_exp, int Cout, const float* bias, uint16_t* y, int64_t ldy,
@@ -203,7 +203,9 @@ int aprnet_upsample_fwd_bf16(const aprnet_plan*, int level_delta, const uint16_t
 /* Backward of the stencil convolution with bfloat16 features and output gradient: fp32 weights, fp32 weight
  * gradient (accumulated into gw), fp32 accumulation everywhere; the input gradient is collected in the fp32 work
  * space gx32_ws [Cin][ld_gx32] (ld_gx32 >= aprnet_number_parts) and rounded to bfloat16 into gx at the end.
- * gtree_ws: fp32 [Cin][ld_gtree]. */
+ * gtree_ws: fp32 [Cin][ld_gtree].  The input gradient multiplies on the bfloat16 matrix cores (weights rounded to
+ * bfloat16) from input-gradient lists that the plan builds on first use; with aprnet_set_conv_path(3) or (5) it
+ * runs with fp32 products and scans per call.  The weight gradient always uses fp32 products. */
 int aprnet_conv_bwd_bf16(const aprnet_plan*, int level_delta, int kz, int kx, int ky, const uint16_t* x, int64_t ldx, int Cin,
                          const float* w, int S_exp, int Cout, const uint16_t* gy, int64_t ldy, uint16_t* gx, int64_t ldgx,
                          float* gw, uint16_t* tree_ws, int64_t ld_tree, float* gx32_ws, int64_t ld_gx32, float* gtree_ws,

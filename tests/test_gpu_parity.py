@@ -428,18 +428,27 @@ def test_maxpool_upsample_bf16_bit_exact(bt):
     assert torch.equal(_ops.maxpool_backward(aprs, go.to(DEV), idx, ld).float().cpu(), gref)
 
 
+@pytest.mark.parametrize("math", [2, 3, 5], ids=["bf16math", "fp32math", "nolists"])
 @pytest.mark.parametrize("ksize", [(3, 3, 3), (1, 5, 5)], ids=KID)
-@pytest.mark.parametrize("bt", [[("3d_b", 1), ("3d_c", 0)], [("2d_a", 0), ("2d_b", 1)]], ids=lambda b: "+".join(f"{n}@{d}" for n, d in b))
-def test_conv_backward_bf16(bt, ksize):
+@pytest.mark.parametrize("bt", [[("3d_b", 1), ("3d_c", 0)], [("2d_a", 0), ("2d_b", 1)], [("3d_s", 0), ("3d_t", 1)]],
+                         ids=lambda b: "+".join(f"{n}@{d}" for n, d in b))
+def test_conv_backward_bf16(bt, ksize, math):
     """bfloat16 features and output gradient, fp32 weights and accumulation: gradients against the fp32 oracle on
-    the same (bfloat16-representable) inputs; the input gradient comes back in bfloat16, the weight gradient in fp32."""
+    the same (bfloat16-representable) inputs; the input gradient comes back in bfloat16, the weight gradient in fp32.
+    The input gradient runs on the bfloat16 matrix cores from the plan's input-gradient lists (weights rounded to
+    bfloat16), or with fp32 products when those are asked for or the lists are switched off."""
     cin, cout = 20, 33
     x, aprs, ld, w_exp = _conv_case(bt, ksize, 2, cin, cout, torch.float32)
     xb = x.to(torch.bfloat16)
     g = torch.Generator().manual_seed(12)
     gob = torch.randn(x.size(0), cout, x.size(2), generator=g).to(torch.bfloat16)
     gx_ref, gw_ref = oracle.conv_backward(aprs, xb.float(), w_exp, gob.float(), ld)
-    gx, gw = _ops.conv_backward(aprs, xb.to(DEV), w_exp.permute(1, 2, 0, 3, 4, 5).contiguous().to(DEV), gob.to(DEV), ld)
+    lib = _native.hip()
+    assert lib.aprnet_set_conv_path(math) == 0
+    try:
+        gx, gw = _ops.conv_backward(aprs, xb.to(DEV), w_exp.permute(1, 2, 0, 3, 4, 5).contiguous().to(DEV), gob.to(DEV), ld)
+    finally:
+        lib.aprnet_set_conv_path(2); lib.aprnet_set_conv_path(4)
     close_bf16(gx, gx_ref)
     assert gw.dtype == torch.float32
     # fp32 sums; the mean-filled tree values they read are stored in bfloat16, hence the bfloat16 tolerance
