@@ -69,6 +69,45 @@ def test_forward_is_linear_and_backward_is_its_adjoint(apr):
     assert abs(lhs - rhs_w) <= 1e-5 * ref
 
 
+def test_fused_forward_equals_separate_passes(apr):
+    """relu(conv(cat([x, x2])) + bias) from the fused entry point is bit-equal to the plain kernel on the
+    concatenated tensor followed by a clamp (same products in the same order), fp32 and bfloat16 features."""
+    n, c1, c2, cout = apr.total_number_particles(), 16, 16, 16
+    g = torch.Generator().manual_seed(4)
+    ld = torch.zeros(1, dtype=torch.int32)
+    levels = apr.level_max() - apr.level_min() + 1
+    w = (torch.randn(levels, cout, c1 + c2, 3, 3, 3, generator=g) * 0.1).to(DEV)
+    bias = torch.randn(cout, generator=g).to(DEV)
+    for dtype in (torch.float32, torch.bfloat16):
+        xa = torch.randn(1, c1, n, generator=g).to(dtype).to(DEV)
+        xb = torch.randn(1, c2, n, generator=g).to(dtype).to(DEV)
+        fused = _ops.conv_forward([apr], xa, w, ld, bias, relu=True, x2=xb)
+        plain = _ops.conv_forward([apr], torch.cat([xa, xb], dim=1), w, ld, bias)
+        assert torch.equal(fused, torch.relu(plain))
+        assert float(fused.float().abs().max()) > 0
+
+
+def test_bf16_backward_is_adjoint_of_bf16_forward(apr):
+    """bfloat16 features: <conv(x), gy> against <x, dX> and <w, dW> with the input gradient on the bfloat16 matrix
+    cores; the three inner products agree to the bfloat16 rounding of the stored values (1e-2 of the absolute sum)."""
+    n, cin, cout = apr.total_number_particles(), 16, 24
+    g = torch.Generator().manual_seed(5)
+    ld = torch.zeros(1, dtype=torch.int32)
+    levels = apr.level_max() - apr.level_min() + 1
+    w = (torch.randn(levels, cout, cin, 3, 3, 3, generator=g) * 0.2).to(torch.bfloat16).float().to(DEV)   # exact in bf16
+    x = torch.randn(1, cin, n, generator=g).to(torch.bfloat16).to(DEV)
+    gy = torch.randn(1, cout, n, generator=g).to(torch.bfloat16).to(DEV)
+    y = _ops.conv_forward([apr], x, w, ld)
+    gx, gw = _ops.conv_backward([apr], x, w, gy, ld)
+    assert gx.dtype == torch.bfloat16 and gw.dtype == torch.float32
+    lhs = float((y.double() * gy.double()).sum())
+    rhs_x = float((x.double() * gx.double()).sum())
+    rhs_w = float((w.double() * gw.double()).sum())
+    ref = float((y.double().abs() * gy.double().abs()).sum())
+    assert abs(lhs - rhs_x) <= 1e-2 * ref
+    assert abs(lhs - rhs_w) <= 1e-2 * ref
+
+
 def test_pool_argmax_gathers_and_upsample_round_trip(apr):
     n, c = apr.total_number_particles(), 6
     g = torch.Generator().manual_seed(2)
