@@ -142,6 +142,19 @@ def other_ops(apr, x, dev):
     with torch.no_grad():
         ms = _time(lambda: net(xin, [apr]), iters=3, warmup=1)
     res.append({"op": "apr_unet_fwd", "ms": ms, "note": f"4 levels 16-32-64-128, fp32, {n0} particles, norms folded"})
+    # the same forward captured once into a HIP graph and replayed (no host work between the ~250 launches)
+    with torch.no_grad():
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            net(xin, [apr])
+        torch.cuda.current_stream().wait_stream(side)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            y_graph = net(xin, [apr])
+        ms = _time(graph.replay, iters=3, warmup=1)
+    res.append({"op": "apr_unet_fwd_graph", "ms": ms, "note": "the fp32 forward replayed from a HIP graph"})
+    del graph, y_graph
     # the wide 2-D stencil of configs[4] (1x5x5, 64 -> 64), here on the 3-D benchmark APR, fp32
     conv5 = aprnet.cuda.APRConv(64, 64, nstencils=2, kernel_size=(1, 5, 5)).to(dev)
     x64 = torch.randn(1, 64, x.shape[2], device=dev)

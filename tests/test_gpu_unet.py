@@ -233,3 +233,34 @@ def test_stardist_unet_heads_match_oracle(out_delta, after):
     assert prob.shape == (1, 1, n_out) and dist.shape == (1, 8, n_out)
     assert float((prob.cpu() - ref_prob).abs().max()) < 2e-5
     assert float((dist.cpu() - ref_dist).abs().max()) < 2e-5 * float(ref_dist.abs().max())
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
+def test_unet_forward_replays_from_a_hip_graph(dtype):
+    """After one eager call (which builds the plan's lists) the operators neither allocate, copy nor synchronise, so
+    the whole network forward can be captured into a HIP graph.  Replays with new inputs, interleaved with eager
+    calls and synchronisations, reproduce the eager results bit for bit (the forward is deterministic)."""
+    apr = apr_cases.random_apr((33, 29, 37), 11, density=0.02)
+    torch.manual_seed(0)
+    model = fold_norms(APRUNet(1, 3, depth=3, n_filters_base=16, n_stencils=2, norm="batch").eval()).to(DEV)
+    n = apr.total_number_particles()
+    g = torch.Generator().manual_seed(1)
+    x_static = torch.randn(1, 1, n, generator=g).to(dtype).to(DEV)
+    with torch.no_grad():
+        model(x_static, [apr])                                   # eager warm-up: lists, tile tables, scratch
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            model(x_static, [apr])
+        torch.cuda.current_stream().wait_stream(side)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            y_static = model(x_static, [apr])
+        for k in range(3):
+            x_new = torch.randn(1, 1, n, generator=g).to(dtype).to(DEV)
+            eager = model(x_new, [apr])
+            torch.cuda.synchronize()
+            x_static.copy_(x_new)
+            graph.replay()
+            torch.cuda.synchronize()
+            assert torch.equal(y_static, eager), f"replay {k}"
