@@ -100,6 +100,10 @@ def hip():
         getattr(lib, f"aprnet_sample_particles_bwd_{t}").argtypes = [vp, i32, vp, i64, i32, vp, i64, vp]
     # bfloat16 features: forward operators of the network, backward of pool / upsample / tree fill
     lib.aprnet_conv_fwd_bf16.argtypes = [vp, i32, i32, i32, i32, vp, i64, i32, vp, i32, i32, vp, vp, i64, vp, i64, vp]
+    lib.aprnet_particle_coords.argtypes = [vp, i32, vp, vp]
+    lib.aprnet_sample_image_max_f32.argtypes = [vp, i32, vp, i32, i32, i32, vp, vp]
+    for t in ("u8", "u16", "u32", "u64"):     # plan, d, img, zn, xn, yn, dzs, dxs, dys, n_rays, max_steps, dist, stream
+        getattr(lib, f"aprnet_labels_to_dist_{t}").argtypes = [vp, i32, vp, i32, i32, i32, vp, vp, vp, i32, i32, vp, vp]
     for t in ("f32", "f64", "bf16"):      # ..., tree_ws, ld_tree, const aprnet_conv_fusion*, stream
         getattr(lib, f"aprnet_conv_fwd_fused_{t}").argtypes = [vp, i32, i32, i32, i32, vp, i64, i32, vp, i32, i32, vp, vp, i64,
                                                                 vp, i64, vp, vp]

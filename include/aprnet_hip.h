@@ -214,6 +214,27 @@ int aprnet_channel_sum_bf16(const uint16_t* x, int64_t ld, int C, int64_t n, flo
 int aprnet_upsample_bwd_bf16(const aprnet_plan*, int level_delta, const uint16_t* gy, int64_t ldy, int C, uint16_t* gx,
                              int64_t ldx, void* stream);
 
+/* Label and coordinate utilities of the StarDist networks (pyapr/aprnet/src/utils.hpp:86-333; CPU loops in the
+ * reference, device kernels here).  Particle order = feature order at level_delta.  Images are dense device arrays
+ * [zn][xn][yn] with the dimensions of the APR's finest level.
+ *   particle_coords   get_particle_coords (utils.hpp:222-267): coords [N_d][3] = (z, x, y) cell centres in pixels.
+ *   sample_image_max  sample_image (utils.hpp:270-333): parts [N_d] = maximum of img over each particle's cell.
+ *   labels_to_dist    labels_to_dist_cpp (utils.hpp:86-219): dist [N_d][n_rays], left untouched (caller zeroes it)
+ *                     where the particle's centre carries label 0 or lies outside the image.  dzs / dxs / dys:
+ *                     device arrays [n_rays] of the ray steps.  max_steps bounds the walk along a ray (the
+ *                     reference walks until the ray leaves its object, which never ends for a zero step). */
+int aprnet_particle_coords(const aprnet_plan*, int level_delta, float* coords, void* stream);
+int aprnet_sample_image_max_f32(const aprnet_plan*, int level_delta, const float* img, int zn, int xn, int yn, float* parts,
+                                void* stream);
+int aprnet_labels_to_dist_u8(const aprnet_plan*, int level_delta, const uint8_t* img, int zn, int xn, int yn, const float* dzs,
+                             const float* dxs, const float* dys, int n_rays, int max_steps, float* dist, void* stream);
+int aprnet_labels_to_dist_u16(const aprnet_plan*, int level_delta, const uint16_t* img, int zn, int xn, int yn, const float* dzs,
+                              const float* dxs, const float* dys, int n_rays, int max_steps, float* dist, void* stream);
+int aprnet_labels_to_dist_u32(const aprnet_plan*, int level_delta, const uint32_t* img, int zn, int xn, int yn, const float* dzs,
+                              const float* dxs, const float* dys, int n_rays, int max_steps, float* dist, void* stream);
+int aprnet_labels_to_dist_u64(const aprnet_plan*, int level_delta, const uint64_t* img, int zn, int xn, int yn, const float* dzs,
+                              const float* dxs, const float* dys, int n_rays, int max_steps, float* dist, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

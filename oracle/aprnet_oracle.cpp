@@ -20,6 +20,12 @@
 //   restrict_kernel              the compiled reference (oracle/_ref) + closed-form overlap table
 //   reconstruct / sample         dense view; sample(reconstruct(x)) == x (pyapr/tests/test_aprnet.py:272-285)
 //   every backward               float64 torch.autograd.gradcheck and <Ax,y> == <x,A'y>
+//   particle coords              closed form floor((c + 0.5) * 2^(lmax - l)) through the Python row iterator
+//   sample_image (max pyramid)   max_pool3d(ceil_mode) pyramid of the image read at the particles' cells; how LibAPR's
+//                                downsamplePyramid treats the far faces of odd-sized images is not visible in the
+//                                reference (LibAPR is not vendored): PARITY UNPINNED at those faces
+//   labels_to_dist               cuboid labels with axis and diagonal rays (closed-form distances), label 0 and
+//                                out-of-image centres left untouched
 //
 // One deliberate difference: the reference's patch buffer is never cleared, so cells that no source
 // covers keep stale values (helpers.hpp:358-420); here every gathered row starts from zero.  On a
@@ -558,6 +564,75 @@ void sample_particles(const Acc& apr, const Acc& tree, T* parts, int64_t ldp, in
     }
 }
 
+// ---------------------------------------------------------------------------- StarDist utilities
+// Visits the feature positions at level delta d: particles of levels <= Lc (index = particle index), then the tree
+// nodes of level Lc behind them (utils.hpp:100-104, 170-176).  f(level, z, x, y, feature index).
+template <typename F>
+void for_each_feature(const Acc& apr, const Acc& tree, int d, F f) {
+    const int Lc = apr.lmax() - d;
+    for (int l = apr.lmin(); l <= Lc; ++l)
+        for (int z = 0; z < apr.zn(l); ++z)
+            for (int x = 0; x < apr.xn(l); ++x)
+                for (uint64_t i = apr.beg(l, z, x); i < apr.end(l, z, x); ++i) f(l, z, x, apr.y(i), (int64_t)i);
+    if (d > 0) {
+        const int64_t off = tree_offset(apr, tree, Lc);
+        for (int z = 0; z < tree.zn(Lc); ++z)
+            for (int x = 0; x < tree.xn(Lc); ++x)
+                for (uint64_t i = tree.beg(Lc, z, x); i < tree.end(Lc, z, x); ++i) f(Lc, z, x, tree.y(i), (int64_t)i + off);
+    }
+}
+
+// get_particle_coords, utils.hpp:222-267
+void particle_coords(const Acc& apr, const Acc& tree, int d, float* coords) {
+    const int lmax = apr.lmax();
+    for_each_feature(apr, tree, d, [&](int l, int z, int x, int y, int64_t i) {
+        const double s = std::pow(2.0, lmax - l);
+        coords[3 * i + 0] = (float)std::floor((z + 0.5) * s);
+        coords[3 * i + 1] = (float)std::floor((x + 0.5) * s);
+        coords[3 * i + 2] = (float)std::floor((y + 0.5) * s);
+    });
+}
+
+// sample_image, utils.hpp:270-333: pyramid by maxima, every feature reads the pyramid entry of its cell
+void sample_image_max(const Acc& apr, const Acc& tree, int d, const float* img, int zn, int xn, int yn, float* parts) {
+    const int lmax = apr.lmax();
+    for_each_feature(apr, tree, d, [&](int l, int z, int x, int y, int64_t i) {
+        const int f = 1 << (lmax - l);
+        float m = -INFINITY;
+        bool any = false;
+        for (int zz = z * f; zz < std::min((z + 1) * f, zn); ++zz)
+            for (int xx = x * f; xx < std::min((x + 1) * f, xn); ++xx)
+                for (int yy = y * f; yy < std::min((y + 1) * f, yn); ++yy) { m = std::max(m, img[((int64_t)zz * xn + xx) * yn + yy]); any = true; }
+        parts[i] = any ? m : 0.f;
+    });
+}
+
+// labels_to_dist_cpp, utils.hpp:86-219
+template <typename L>
+void labels_to_dist(const Acc& apr, const Acc& tree, int d, const L* img, int zn, int xn, int yn, const float* dzs,
+                    const float* dxs, const float* dys, int n_rays, int max_steps, float* dist) {
+    const int lmax = apr.lmax();
+    for_each_feature(apr, tree, d, [&](int l, int z, int x, int y, int64_t idx) {
+        const double s = std::pow(2.0, lmax - l);
+        const int i = (int)std::floor((z + 0.5) * s), j = (int)std::floor((x + 0.5) * s), k = (int)std::floor((y + 0.5) * s);
+        if (i >= zn || j >= xn || k >= yn) return;
+        const L value = img[((int64_t)i * xn + j) * yn + k];
+        if (value == 0) return;
+        for (int n = 0; n < n_rays; ++n) {
+            float xx = 0.f, yy = 0.f, zz = 0.f;
+            const float dz = dzs[n], dx = dxs[n], dy = dys[n];
+            for (int step = 0; step < max_steps; ++step) {
+                xx += dx; yy += dy; zz += dz;
+                const long ii = std::lrint((float)i + zz), jj = std::lrint((float)j + xx), kk = std::lrint((float)k + yy);
+                if (ii < 0 || ii >= zn || jj < 0 || jj >= xn || kk < 0 || kk >= yn || value != img[((int64_t)ii * xn + jj) * yn + kk])
+                    break;
+            }
+            zz = (float)std::lrint(zz); xx = (float)std::lrint(xx); yy = (float)std::lrint(yy);
+            dist[idx * n_rays + n] = std::sqrt(xx * xx + yy * yy + zz * zz);
+        }
+    });
+}
+
 template <typename T>
 int conv_fwd_dispatch(int kz, int kx, int ky, const Acc& a, const Acc& t, const T* x, int64_t ldx, int Cin, const T* w,
                       int S, int Cout, T* out, int64_t ldo, int d) {
@@ -641,5 +716,19 @@ void oracle_parent_index(const AccessDesc* a, const AccessDesc* t, int which, in
 
 ORACLE_EXPORT(float, f32)
 ORACLE_EXPORT(double, f64)
+
+void oracle_particle_coords(const AccessDesc* a, const AccessDesc* t, int d, float* coords) { particle_coords(Acc(a), Acc(t), d, coords); }
+void oracle_sample_image_max(const AccessDesc* a, const AccessDesc* t, int d, const float* img, int zn, int xn, int yn, float* parts) {
+    sample_image_max(Acc(a), Acc(t), d, img, zn, xn, yn, parts);
+}
+#define ORACLE_LABELS(T, SFX)                                                                                          \
+    void oracle_labels_to_dist_##SFX(const AccessDesc* a, const AccessDesc* t, int d, const T* img, int zn, int xn, int yn, \
+                                     const float* dzs, const float* dxs, const float* dys, int n_rays, int max_steps,  \
+                                     float* dist) {                                                                    \
+        labels_to_dist<T>(Acc(a), Acc(t), d, img, zn, xn, yn, dzs, dxs, dys, n_rays, max_steps, dist); }
+ORACLE_LABELS(uint8_t, u8)
+ORACLE_LABELS(uint16_t, u16)
+ORACLE_LABELS(uint32_t, u32)
+ORACLE_LABELS(uint64_t, u64)
 
 }  // extern "C"

@@ -280,3 +280,38 @@ def sample_particles_backward(aprs, grad_output, level_deltas):
         fn(a, t, _p(grad_output[b]), _i64(grad_output.size(2)), grad_output.size(1), _p(gimg[b]), _i64(z * xx * y),
            int(level_deltas[b]))
     return gimg
+
+
+# ------------------------------------------------------------------------------------ StarDist utilities
+_LABEL_SFX = {torch.uint8: "u8", torch.uint16: "u16", torch.uint32: "u32", torch.uint64: "u64"}
+
+
+def particle_coords(apr, level_delta):
+    """get_particle_coords (utils.hpp:222-267) -> [N_d, 3] float32 (z, x, y)."""
+    a, t, _k = _descs(apr)
+    out = torch.zeros(number_parts(apr, level_delta), 3, dtype=torch.float32)
+    lib().oracle_particle_coords(a, t, int(level_delta), _p(out))
+    return out
+
+
+def sample_image_max(apr, img, level_delta):
+    """sample_image (utils.hpp:270-333): maximum of the image over every particle's cell -> [N_d] float32."""
+    img = img.contiguous().float()
+    a, t, _k = _descs(apr)
+    out = torch.zeros(number_parts(apr, level_delta), dtype=torch.float32)
+    z, x, y = img.shape
+    lib().oracle_sample_image_max(a, t, int(level_delta), _p(img), int(z), int(x), int(y), _p(out))
+    return out
+
+
+def labels_to_dist(apr, labels, dzs, dxs, dys, level_delta, max_steps=1 << 20):
+    """labels_to_dist_cpp (utils.hpp:86-219) -> [N_d, n_rays] float32."""
+    labels = labels.contiguous()
+    dzs, dxs, dys = (v.contiguous().float() for v in (dzs, dxs, dys))
+    a, t, _k = _descs(apr)
+    out = torch.zeros(number_parts(apr, level_delta), dzs.numel(), dtype=torch.float32)
+    z, x, y = labels.shape
+    getattr(lib(), "oracle_labels_to_dist_" + _LABEL_SFX[labels.dtype])(
+        a, t, int(level_delta), _p(labels), int(z), int(x), int(y), _p(dzs), _p(dxs), _p(dys), int(dzs.numel()), int(max_steps),
+        _p(out))
+    return out

@@ -568,3 +568,52 @@ def test_degenerate_structures(name):
         _ops.restrict_kernel_forward(torch.zeros(levels + 1, 2, 2, 3, 3, 3, device=DEV), levels)
     with pytest.raises(ValueError):
         oracle.restrict_kernel_forward(torch.zeros(2, levels + 1, 2, 3, 3, 3), levels)
+
+
+# ------------------------------------------------------------------------------------ StarDist utilities
+@pytest.mark.parametrize("name", ["3d_c", "3d_s", "2d_a", "1d_a"])
+def test_stardist_utilities_match_oracle(name):
+    """get_particle_coordinates, sample_image (max pyramid) and labels_to_dist on the device against the oracle's
+    restatement of utils.hpp:86-333: bit-exact (integer coordinates, maxima, and the same fp32 ray walk with
+    round-half-even), for numpy and tensor inputs, every label type, integer and fractional ray steps."""
+    from pyapr.aprnet import stardist_utils as su
+    apr = apr_cases.get(name)
+    Z, X, Y = apr.shape()
+    g = torch.Generator().manual_seed(21)
+    img = torch.randn(Z, X, Y, generator=g)
+    blobs = (torch.rand(Z, X, Y, generator=g) * 2.2).floor()            # labels 0, 1, 2 in random patches
+    lab = torch.nn.functional.interpolate(blobs[None, None, ::3, ::3, ::3], size=(Z, X, Y), mode="nearest")[0, 0]
+    rays = torch.tensor([[1, 0, 0], [0, -1, 0], [0, 0, 1], [0.5, 0.5, 0], [-0.7, 0.2, 0.4], [0, 1.5, -1.5], [0.3, 0, 0]],
+                        dtype=torch.float32)
+    if Z == 1:
+        rays[:, 0] = 0
+    if X == 1:
+        rays[:, 1] = 0
+    rays = rays[(rays != 0).any(dim=1)]
+    for d in range(max_delta(apr) + 1):
+        n = oracle.number_parts(apr, d)
+        ref_c = oracle.particle_coords(apr, d)
+        got_c = su.get_particle_coordinates(apr, d)
+        assert isinstance(got_c, np.ndarray) and got_c.shape == (n, 3) and np.array_equal(got_c, ref_c.numpy())
+        assert torch.equal(su.get_particle_coordinates(apr, d, device=DEV).cpu(), ref_c)
+        ref_s = oracle.sample_image_max(apr, img, d)
+        assert np.array_equal(su.sample_image(apr, img.numpy(), d), ref_s.numpy())
+        assert torch.equal(su.sample_image(apr, img.to(DEV), d).cpu(), ref_s)
+        for dt in (torch.uint8, torch.uint16, torch.uint32, torch.uint64):
+            labels = lab.to(torch.int64).to(dt)
+            ref_d = oracle.labels_to_dist(apr, labels, rays[:, 0], rays[:, 1], rays[:, 2], d)
+            got_d = su.labels_to_dist(apr, labels.to(DEV), rays.numpy(), level_delta=d)
+            assert torch.equal(got_d.cpu(), ref_d), dt
+        got_np = su.labels_to_dist(apr, lab.numpy().astype(np.uint16), rays.numpy(), step_factor=(2, 2, 2), level_delta=d)
+        ref_np = oracle.labels_to_dist(apr, lab.to(torch.int64).to(torch.uint16), rays[:, 0] / 2, rays[:, 1] / 2, rays[:, 2] / 2, d)
+        assert isinstance(got_np, np.ndarray) and np.array_equal(got_np, ref_np.numpy())
+    with pytest.raises(ValueError):
+        su.labels_to_dist(apr, np.zeros((Z + 1, X, Y), np.uint16), rays.numpy())
+    with pytest.raises(ValueError):
+        su.labels_to_dist(apr, np.zeros((Z, X, Y), np.uint16), np.zeros((2, 3), np.float32))
+    with pytest.raises(TypeError):
+        su.labels_to_dist(apr, np.zeros((Z, X, Y), np.float32), rays.numpy())
+    with pytest.raises(ImportError):
+        su.get_prob_apr(apr, np.zeros((Z, X, Y), np.uint16))            # stardist is not installed here
+    prob = su.get_prob_apr(apr, lab.numpy().astype(np.uint16), prob_fn=lambda a: (a > 0).astype(np.float32))
+    assert np.array_equal(prob, oracle.sample_image_max(apr, (lab > 0).float(), 0).numpy())

@@ -158,3 +158,65 @@ def test_reconstruct_and_sample(case):
             f = 1 << (lc - int(l))
             cell = im[0, :, z * f:(z + 1) * f, xx * f:(xx + 1) * f, y * f:(y + 1) * f]
             torch.testing.assert_close(s[0, :, idx], cell.mean(dim=(1, 2, 3)), **TOL)
+
+
+# ------------------------------------------------------------------------------------ StarDist utilities
+def test_particle_coords_closed_form(case):
+    """get_particle_coords: centre of every feature's cell in pixels, floor((c + 0.5) * 2^(lmax - l)), in feature
+    order (particles of levels <= Lc, then the tree nodes of level Lc)."""
+    apr, D = case
+    lmax = apr.level_max()
+    for d in range(_max_delta(apr) + 1):
+        got = oracle.particle_coords(apr, d)
+        outs = D.outputs(d)                      # (feature index, level, z, x, y)
+        assert got.shape == (len(outs), 3)
+        for i, l, z, x, y in outs:
+            f = 2 ** (lmax - l)
+            want = [np.floor((c + 0.5) * f) for c in (z, x, y)]
+            assert got[i].tolist() == want
+
+
+def test_sample_image_reads_a_max_pyramid(case):
+    """sample_image: every feature takes the entry of its cell in a pyramid built by maxima.  The pyramid here is
+    F.max_pool3d(kernel 2, ceil_mode=True) applied level by level (partial blocks at the far faces hold the maximum
+    of the pixels that exist)."""
+    apr, D = case
+    lmax = apr.level_max()
+    g = torch.Generator().manual_seed(3)
+    img = torch.randn(*apr.shape(), generator=g)
+    pyr = {lmax: img}
+    for l in range(lmax - 1, -1, -1):
+        pyr[l] = torch.nn.functional.max_pool3d(pyr[l + 1][None, None], 2, ceil_mode=True)[0, 0]
+    for d in range(_max_delta(apr) + 1):
+        got = oracle.sample_image_max(apr, img, d)
+        for i, l, z, x, y in D.outputs(d):
+            assert float(got[i]) == float(pyr[l][z, x, y])
+
+
+def test_labels_to_dist_on_a_cuboid():
+    """labels_to_dist: inside an axis-aligned cuboid label the distance along +-axis rays is the number of steps to
+    the first pixel outside, along a face diagonal sqrt(2) times the smaller of the two; label 0 gives 0."""
+    apr = apr_cases.get("3d_c")                                   # 16 x 16 x 16
+    Z, X, Y = apr.shape()
+    lab = torch.zeros(Z, X, Y, dtype=torch.uint16)
+    z0, z1, x0, x1, y0, y1 = 3, 12, 2, 9, 5, 14
+    lab[z0:z1, x0:x1, y0:y1] = 7
+    lab[0:2, 0:2, 0:2] = 3                                        # a second object, touching the image corner
+    rays = torch.tensor([[1, 0, 0], [-1, 0, 0], [0, 1, 0], [0, -1, 0], [0, 0, 1], [0, 0, -1], [1, 1, 0], [0, -1, -1]],
+                        dtype=torch.float32)
+    for d in (0, 1):
+        dist = oracle.labels_to_dist(apr, lab, rays[:, 0], rays[:, 1], rays[:, 2], d)
+        coords = oracle.particle_coords(apr, d).long()
+        inside = 0
+        for n in range(coords.shape[0]):
+            i, j, k = coords[n].tolist()
+            v = int(lab[i, j, k]) if (i < Z and j < X and k < Y) else 0
+            if v == 0:
+                assert float(dist[n].abs().max()) == 0.0
+                continue
+            b = (z0, z1, x0, x1, y0, y1) if v == 7 else (0, 2, 0, 2, 0, 2)
+            want = [b[1] - i, i - b[0] + 1, b[3] - j, j - b[2] + 1, b[5] - k, k - b[4] + 1,
+                    np.sqrt(2.0) * min(b[1] - i, b[3] - j), np.sqrt(2.0) * min(j - b[2] + 1, k - b[4] + 1)]
+            np.testing.assert_allclose(dist[n].numpy(), np.asarray(want, np.float32), rtol=1e-6)
+            inside += 1
+        assert inside > 0
