@@ -95,7 +95,7 @@ def test_apr_state_roundtrip():
 def test_model_parameter_names_mirror_reference():
     """state_dict keys of the networks are those of the reference's module trees (unet_parts.py:6-83,
     hybrid_unet_parts.py:9-128, unet_model.py / hybrid_model.py), so checkpoints are interchangeable."""
-    from apr_models.unet import APRUNet, HybridAPRUNet
+    from apr_models.unet import APRUNet, HybridAPRUNet, APRStardistUNet, HybridStardistUNet
     keys = set(APRUNet(1, 2, depth=1, n_filters_base=4).state_dict())
     assert {"encoder.0.blocks.0.conv.weight", "encoder.0.blocks.1.norm.weight", "encoder.1.conv.blocks.0.conv.weight",
             "decoder.0.reduce_ch.conv.weight", "decoder.0.conv.blocks.1.norm.bias", "head.weight", "head.bias"} <= keys
@@ -107,6 +107,8 @@ def test_model_parameter_names_mirror_reference():
             "decoder.0.reduce_ch.conv.weight",                # PixelUpConv
             "decoder.1.reduce_ch.conv.weight", "decoder.1.conv.blocks.0.conv.weight",      # TransitionUpConv
             "decoder.2.reduce_ch.conv.weight", "head.weight"} <= keys
+    for net in (APRStardistUNet(1, 4, depth=1, n_filters_base=4), HybridStardistUNet(1, 4, depth=2, apr_depth=1, n_filters_base=4)):
+        assert {"output_prob.conv.weight", "output_dist.weight", "output_dist.bias"} <= set(net.state_dict())
     sd = hyb.state_dict()
     assert sd["encoder.2.conv.blocks.0.conv.weight"].dim() == 5       # nn.Conv3d [Cout, Cin, kz, kx, ky]
     assert sd["decoder.1.conv.blocks.0.conv.weight"].dim() == 6       # APRConv [S, Cout, Cin, kz, kx, ky]

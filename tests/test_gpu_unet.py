@@ -264,3 +264,40 @@ def test_unet_forward_replays_from_a_hip_graph(dtype):
             graph.replay()
             torch.cuda.synchronize()
             assert torch.equal(y_static, eager), f"replay {k}"
+
+
+def test_hybrid_stardist_unet_matches_oracle():
+    """HybridStardistUNet (stardist_hybrid_model.py:24-199): dense stages below the transition, decoder back to the
+    particles at output_level_delta = 1, probability and distance heads there; against the oracle composition."""
+    import copy
+    from apr_models.unet import HybridStardistUNet
+    from oracle_modules import OracleReconstruct, OracleSample
+    apr = apr_cases.random_apr((33, 29, 37), 11, density=0.02)
+    torch.manual_seed(4)
+    model = fold_norms(HybridStardistUNet(1, 6, depth=3, apr_depth=1, n_filters_base=8, n_stencils=2, norm="batch",
+                                          output_level_delta=1, net_conv_after_unet=10).eval())
+    with pytest.raises(ValueError):
+        HybridStardistUNet(1, 6, depth=3, apr_depth=1, output_level_delta=2)
+    ref_model = copy.deepcopy(model)
+    x = torch.randn(1, 1, apr.total_number_particles())
+    aprs, ld = [apr], torch.zeros(1, dtype=torch.int32)
+    with torch.no_grad():
+        e0 = _cpu_block(ref_model.encoder[0], x, aprs, ld)
+        y = OracleMaxPool.apply(e0, aprs, ld); ld += 1
+        e1 = _cpu_block(ref_model.encoder[1].conv, y, aprs, ld)                       # DownConv (particles)
+        y = OracleMaxPool.apply(e1, aprs, ld); ld += 1
+        e2 = ref_model.encoder[2].conv(OracleReconstruct.apply(y, aprs, ld))          # TransitionDownConv
+        e3 = ref_model.encoder[3](e2)                                                 # PixelDownConv
+        y = ref_model.decoder[0](e3, e2)                                              # PixelUpConv
+        d = ref_model.decoder[1]                                                      # TransitionUpConv
+        y = OracleUpSample.apply(OracleSample.apply(d.reduce_ch(y), aprs, ld), aprs, ld); ld -= 1
+        y = _cpu_block(d.conv, torch.cat([e1, y], 1), aprs, ld)
+        y = _cpu_block(ref_model.conv_after_unet, y, aprs, ld)
+        ref_prob = torch.sigmoid(_cpu_conv(ref_model.output_prob.conv, y, aprs, ld))
+        ref_dist = _cpu_conv(ref_model.output_dist, y, aprs, ld)
+        assert int(ld[0]) == 1
+        prob, dist = model.to(DEV)(x.to(DEV), [apr])
+    n1 = oracle.number_parts(apr, 1)
+    assert prob.shape == (1, 1, n1) and dist.shape == (1, 6, n1)
+    assert float((prob.cpu() - ref_prob).abs().max()) < 5e-5
+    assert float((dist.cpu() - ref_dist).abs().max()) < 5e-5 * float(ref_dist.abs().max())
