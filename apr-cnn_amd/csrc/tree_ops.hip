@@ -41,6 +41,32 @@ fill_tree_level_kernel(const int32_t* __restrict__ children, int64_t n_tree, int
         if (c >= C) break;
         const T* xc = x + (int64_t)c * ldx;
         T* tc = tree + (int64_t)c * ldt;
+        // Children 2y and 2y + 1 of one (z, x) row are neighbours in memory when both are particles: one 8-byte load
+        // for the two (4-byte aligned) instead of two 4-byte loads whose lanes each use half of every 8 bytes.
+        A val[8];
+#pragma unroll
+        for (int s = 0; s < 8; s += 2) {
+            const int32_t v0 = ch[s], v1 = ch[s + 1];
+            bool paired = false;
+            if constexpr (sizeof(T) >= 4) {
+                if (v0 >= 0 && v1 == v0 + 1) {
+                    typedef T pair_t __attribute__((ext_vector_type(2), aligned(sizeof(T))));
+                    const pair_t pv = *reinterpret_cast<const pair_t*>(xc + v0);
+                    val[s] = pv[0]; val[s + 1] = pv[1];
+                    paired = true;
+                }
+            }
+            if (!paired) {
+#pragma unroll
+                for (int k2 = 0; k2 < 2; ++k2) {
+                    const int32_t v = k2 ? v1 : v0;
+                    A r = 0;
+                    if (v >= 0) r = Num<T>::ld(xc[v]);
+                    else if (v != NO_CHILD) r = Num<T>::ld(tree_child_from_x ? xc[(int64_t)(~v) + tree_off] : tc[~v]);
+                    val[s + k2] = r;
+                }
+            }
+        }
         A sum = 0;
 #pragma unroll
         for (int pass = 0; pass < 2; ++pass) {
@@ -49,8 +75,7 @@ fill_tree_level_kernel(const int32_t* __restrict__ children, int64_t n_tree, int
             for (int s = 0; s < 8; ++s) {
                 const int32_t v = ch[s];
                 if (v == NO_CHILD) continue;
-                if (want_tree && v < 0) sum += Num<T>::ld(tree_child_from_x ? xc[(int64_t)(~v) + tree_off] : tc[~v]);
-                if (!want_tree && v >= 0) sum += Num<T>::ld(xc[v]);
+                if (want_tree == (v < 0)) sum += val[s];
             }
         }
         tc[t] = Num<T>::st(sum * scale);
