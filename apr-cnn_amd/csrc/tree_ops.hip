@@ -10,11 +10,71 @@ namespace aprnet {
 constexpr int TB = 256;
 constexpr int CPT = 4;          // channels per thread
 
+// Children 2y and 2y + 1 of one (z, x) row are neighbours in memory when both are particles (or both tree nodes)
+// with consecutive indices: one 8-byte access for the two (element-aligned) instead of two 4-byte accesses whose
+// lanes each use half of every 8 bytes (4- and 16-byte pairs for bfloat16 and double).
+template <typename T> struct Pair { T v[2]; };        // alignment of one element
+
+// val[s] = value of child s (0 where there is none); particles from `part`, tree nodes from `tnode[~v]`.
 template <typename T>
-struct ChildView {
-    const int32_t* children;   // [8][n_tree]
-    int64_t n_tree;
-};
+__device__ __forceinline__ void load_children(const int32_t (&ch)[8], const T* part,
+                                              const T* tnode, typename Num<T>::acc (&val)[8]) {
+    typedef typename Num<T>::acc A;
+#pragma unroll
+    for (int s = 0; s < 8; s += 2) {
+        const int32_t v0 = ch[s], v1 = ch[s + 1];
+        bool paired = false;
+        if constexpr (sizeof(T) >= 2) {
+            const bool pp = v0 >= 0 && v1 == v0 + 1;
+            const bool tt = v0 < 0 && v0 != NO_CHILD && v1 == v0 - 1;
+            if (pp || tt) {
+                const T* src = pp ? part + v0 : tnode + ~v0;
+                const Pair<T> pv = *reinterpret_cast<const Pair<T>*>(src);
+                val[s] = Num<T>::ld(pv.v[0]); val[s + 1] = Num<T>::ld(pv.v[1]);
+                paired = true;
+            }
+        }
+        if (!paired) {
+#pragma unroll
+            for (int k2 = 0; k2 < 2; ++k2) {
+                const int32_t v = k2 ? v1 : v0;
+                A r = 0;
+                if (v >= 0) r = Num<T>::ld(part[v]);
+                else if (v != NO_CHILD) r = Num<T>::ld(tnode[~v]);
+                val[s + k2] = r;
+            }
+        }
+    }
+}
+
+// Writes val[s] to child s for every existing child, pairs in one 8-byte store.
+template <typename T>
+__device__ __forceinline__ void store_children(const int32_t (&ch)[8], T* part, T* tnode,
+                                               const T (&val)[8]) {
+#pragma unroll
+    for (int s = 0; s < 8; s += 2) {
+        const int32_t v0 = ch[s], v1 = ch[s + 1];
+        bool paired = false;
+        if constexpr (sizeof(T) >= 2) {
+            const bool pp = v0 >= 0 && v1 == v0 + 1;
+            const bool tt = v0 < 0 && v0 != NO_CHILD && v1 == v0 - 1;
+            if (pp || tt) {
+                Pair<T> pv;
+                pv.v[0] = val[s]; pv.v[1] = val[s + 1];
+                *reinterpret_cast<Pair<T>*>(pp ? part + v0 : tnode + ~v0) = pv;
+                paired = true;
+            }
+        }
+        if (!paired) {
+#pragma unroll
+            for (int k2 = 0; k2 < 2; ++k2) {
+                const int32_t v = k2 ? v1 : v0;
+                if (v >= 0) part[v] = val[s + k2];
+                else if (v != NO_CHILD) tnode[~v] = val[s + k2];
+            }
+        }
+    }
+}
 
 // ---------------------------------------------------------------------------- tree fill (mean)
 // helpers.hpp:156-252.  One launch per tree level, finest first.  `tree_first`: the reference adds
@@ -41,32 +101,8 @@ fill_tree_level_kernel(const int32_t* __restrict__ children, int64_t n_tree, int
         if (c >= C) break;
         const T* xc = x + (int64_t)c * ldx;
         T* tc = tree + (int64_t)c * ldt;
-        // Children 2y and 2y + 1 of one (z, x) row are neighbours in memory when both are particles: one 8-byte load
-        // for the two (4-byte aligned) instead of two 4-byte loads whose lanes each use half of every 8 bytes.
         A val[8];
-#pragma unroll
-        for (int s = 0; s < 8; s += 2) {
-            const int32_t v0 = ch[s], v1 = ch[s + 1];
-            bool paired = false;
-            if constexpr (sizeof(T) >= 4) {
-                if (v0 >= 0 && v1 == v0 + 1) {
-                    typedef T pair_t __attribute__((ext_vector_type(2), aligned(sizeof(T))));
-                    const pair_t pv = *reinterpret_cast<const pair_t*>(xc + v0);
-                    val[s] = pv[0]; val[s + 1] = pv[1];
-                    paired = true;
-                }
-            }
-            if (!paired) {
-#pragma unroll
-                for (int k2 = 0; k2 < 2; ++k2) {
-                    const int32_t v = k2 ? v1 : v0;
-                    A r = 0;
-                    if (v >= 0) r = Num<T>::ld(xc[v]);
-                    else if (v != NO_CHILD) r = Num<T>::ld(tree_child_from_x ? xc[(int64_t)(~v) + tree_off] : tc[~v]);
-                    val[s + k2] = r;
-                }
-            }
-        }
+        load_children<T>(ch, xc, tree_child_from_x ? xc + tree_off : tc, val);
         A sum = 0;
 #pragma unroll
         for (int pass = 0; pass < 2; ++pass) {
@@ -103,13 +139,13 @@ fill_tree_bwd_level_kernel(const int32_t* __restrict__ children, int64_t n_tree,
         T* gxc = gx + (int64_t)c * ldx;
         T* gtc = gtree + (int64_t)c * ldt;
         const A g = Num<T>::ld(gtc[t]) * scale;
+        T* gt_child = tree_child_in_x ? gxc + tree_off : gtc;
+        A val[8];
+        load_children<T>(ch, gxc, gt_child, val);
+        T out[8];
 #pragma unroll
-        for (int s = 0; s < 8; ++s) {
-            const int32_t v = ch[s];
-            if (v == NO_CHILD) continue;
-            T* dst = v >= 0 ? gxc + v : (tree_child_in_x ? gxc + ((int64_t)(~v) + tree_off) : gtc + ~v);
-            *dst = Num<T>::st(Num<T>::ld(*dst) + g);
-        }
+        for (int s = 0; s < 8; ++s) out[s] = Num<T>::st(val[s] + g);
+        store_children<T>(ch, gxc, gt_child, out);
     }
 }
 
@@ -144,19 +180,17 @@ maxpool_fwd_kernel(const int32_t* __restrict__ children, int64_t n_tree, int64_t
         typedef typename Num<T>::acc A;
         A best = (A)(-1e17f);               // initial value of the output, maxpool.hpp:51
         int64_t best_i = 0;
+        A val[8];
+        load_children<T>(ch, xc, xc + in_tree_off, val);
 #pragma unroll
         for (int s = 0; s < 8; ++s) {
             const int32_t v = ch[s];
-            if (v >= 0) { const A val = Num<T>::ld(xc[v]); if (val > best) { best = val; best_i = v; } }
+            if (v >= 0 && val[s] > best) { best = val[s]; best_i = v; }
         }
 #pragma unroll
         for (int s = 0; s < 8; ++s) {
             const int32_t v = ch[s];
-            if (v < 0 && v != NO_CHILD) {
-                const int64_t j = (int64_t)(~v) + in_tree_off;
-                const A val = Num<T>::ld(xc[j]);
-                if (val > best) { best = val; best_i = j; }
-            }
+            if (v < 0 && v != NO_CHILD && val[s] > best) { best = val[s]; best_i = (int64_t)(~v) + in_tree_off; }
         }
         y[(int64_t)c * ldy + i] = Num<T>::st(best);
         arg[(int64_t)c * ldi + i] = best_i;
@@ -192,13 +226,14 @@ maxpool_bwd_kernel(const int32_t* __restrict__ children, int64_t n_tree, int64_t
         T* gxc = gx + (int64_t)c * ldx;
         const T g = gy[(int64_t)c * ldy + i];
         const int64_t m = arg[(int64_t)c * ldi + i];
+        T out[8];
 #pragma unroll
         for (int s = 0; s < 8; ++s) {
             const int32_t v = ch[s];
-            if (v == NO_CHILD) continue;
             const int64_t j = v >= 0 ? (int64_t)v : (int64_t)(~v) + in_tree_off;
-            gxc[j] = (j == m) ? g : Num<T>::st(0);
+            out[s] = (j == m) ? g : Num<T>::st(0);
         }
+        store_children<T>(ch, gxc, gxc + in_tree_off, out);
     }
 }
 
@@ -233,18 +268,17 @@ upsample_kernel(const int32_t* __restrict__ children, int64_t n_tree, int64_t n_
         const T* s_ = src + (int64_t)c * lds;
         T* d_ = dst + (int64_t)c * ldd;
         if (!Backward) {
-            const T v = s_[i];
+            T out[8];
 #pragma unroll
-            for (int s = 0; s < 8; ++s) {
-                if (ch[s] == NO_CHILD) continue;
-                d_[ch[s] >= 0 ? (int64_t)ch[s] : (int64_t)(~ch[s]) + out_tree_off] = v;
-            }
+            for (int s = 0; s < 8; ++s) out[s] = s_[i];
+            store_children<T>(ch, d_, d_ + out_tree_off, out);
         } else {
-            typename Num<T>::acc sum = 0;      // particles first, then tree nodes (upsample.hpp:199-232)
+            typename Num<T>::acc sum = 0, val[8];      // particles first, then tree nodes (upsample.hpp:199-232)
+            load_children<T>(ch, s_, s_ + out_tree_off, val);
 #pragma unroll
-            for (int s = 0; s < 8; ++s) if (ch[s] >= 0) sum += Num<T>::ld(s_[ch[s]]);
+            for (int s = 0; s < 8; ++s) if (ch[s] >= 0) sum += val[s];
 #pragma unroll
-            for (int s = 0; s < 8; ++s) if (ch[s] < 0 && ch[s] != NO_CHILD) sum += Num<T>::ld(s_[(int64_t)(~ch[s]) + out_tree_off]);
+            for (int s = 0; s < 8; ++s) if (ch[s] < 0 && ch[s] != NO_CHILD) sum += val[s];
             d_[i] = Num<T>::st(sum);
         }
     }

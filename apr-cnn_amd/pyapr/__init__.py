@@ -3,8 +3,9 @@
 from .data_containers import APR, APRParameters, LinearIterator, APRPtrVector
 from . import converter
 from . import synthetic
+from . import io
 
-__all__ = ["APR", "APRParameters", "LinearIterator", "APRPtrVector", "converter", "synthetic", "aprnet"]
+__all__ = ["APR", "APRParameters", "LinearIterator", "APRPtrVector", "converter", "synthetic", "io", "aprnet"]
 
 
 def __getattr__(name):

@@ -174,6 +174,28 @@ class APR:
         return (self._org[2], self._org[1], self._org[0], self._params, self._acc.xz_end_vec, self._acc.y_vec,
                 self._tree.xz_end_vec, self._tree.y_vec)
 
+    # pickle support with the reference's state tuple (BindAPR.hpp:67-131); device plans are rebuilt on demand
+    def __getstate__(self):
+        if self._acc is None:
+            raise RuntimeError("Invalid state - APR not initialized")
+        return self.get_state() + (self.name,)
+
+    def __setstate__(self, t):
+        if len(t) not in (8, 9):
+            raise RuntimeError("Error unpickling APR object - invalid state size")
+        other = APR.from_state(t[0:3], t[4], t[5], t[6], t[7], parameters=t[3])
+        self.__dict__.update(other.__dict__)
+        other._plans = {}
+        self.name = t[8] if len(t) == 9 else ""
+
+    def particle_levels(self):
+        """Level of every particle, uint8 (what ParticleData.fill_with_levels writes, used by the collate function of
+        apr_models/utils/dataset.py:147-151)."""
+        out = np.empty(self.total_number_particles(), np.uint8)
+        for level in range(self.level_min(), self.level_max() + 1):
+            out[self._acc.particles_level_begin(level):self._acc.particles_level_end(level)] = level
+        return out
+
     # ------------------------------------------------------------------ reference API
     def __repr__(self):
         return "APR(shape [{}, {}, {}], {} particles)".format(*self._org, self.total_number_particles())
