@@ -6,14 +6,15 @@ import torch
 import torch.nn as nn
 
 from pyapr.aprnet import cuda as aprnet
+from .particle_norm import ParticleBatchNorm, ParticleGroupNorm
 
 
 def _make_norm(kind, channels, num_groups, bn_momentum):
     if kind == "group":
         groups = min(num_groups, channels) if num_groups is not None else channels
-        return nn.GroupNorm(num_groups=groups, num_channels=channels)
+        return ParticleGroupNorm(num_groups=groups, num_channels=channels)
     if kind == "batch":
-        return nn.BatchNorm1d(channels, momentum=bn_momentum)
+        return ParticleBatchNorm(channels, momentum=bn_momentum)
     if kind == "none":          # inference with the normalisation folded into the convolution
         return nn.Identity()
     raise ValueError("norm must be either 'group' or 'batch'")
@@ -38,7 +39,10 @@ class BasicBlock(nn.Module):
             return self.conv.forward_fused(x, aprs, level_deltas, relu=True, second_input=x2)
         if x2 is not None:
             x = torch.cat([x, x2], dim=1)
-        return self.activation(self.norm(self.conv(x, aprs, level_deltas)))
+        y = self.conv(x, aprs, level_deltas)
+        if type(self.activation) is nn.ReLU and isinstance(self.norm, (ParticleBatchNorm, ParticleGroupNorm)):
+            return self.norm(y, relu=True)          # one pass for norm + ReLU
+        return self.activation(self.norm(y))
 
 
 class ConvBlock(nn.Module):

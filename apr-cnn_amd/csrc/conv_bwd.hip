@@ -216,9 +216,11 @@ int fill_tree_bwd_for_conv(const aprnet_plan* p, int d, double* gx, int64_t ldx,
 template <typename T, class GX, int XCIB, class GW, int WCIB, int WCOB>
 static int launch_bwd(ConvArgs<T>& a, hipStream_t st) {
     constexpr int COBLK = 8;
-    dim3 gx((unsigned)a.n_tiles, (unsigned)((a.Cin + XCIB - 1) / XCIB));
-    hipLaunchKernelGGL((conv_bwd_dx_kernel<T, GX, XCIB, COBLK>), gx, dim3(GX::NT), 0, st, a);
-    APRNET_LAUNCH_CHECK("conv_bwd_dx_kernel");
+    if (a.gx) {
+        dim3 gx((unsigned)a.n_tiles, (unsigned)((a.Cin + XCIB - 1) / XCIB));
+        hipLaunchKernelGGL((conv_bwd_dx_kernel<T, GX, XCIB, COBLK>), gx, dim3(GX::NT), 0, st, a);
+        APRNET_LAUNCH_CHECK("conv_bwd_dx_kernel");
+    }
     dim3 gw((unsigned)std::min(a.n_tiles, 512), (unsigned)((a.Cin + WCIB - 1) / WCIB), (unsigned)((a.Cout + WCOB - 1) / WCOB));
     hipLaunchKernelGGL((conv_bwd_dw_kernel<T, GW, WCIB, WCOB>), gw, dim3(GW::NT), 0, st, a);
     APRNET_LAUNCH_CHECK("conv_bwd_dw_kernel");
@@ -250,15 +252,17 @@ template <> int try_mfma_bwd<float>(aprnet_plan* p, const ConvArgs<float>& a, co
     *done = true;
     // input gradient: the forward kernel on the output gradient with the transposed, flipped stencil;
     // every row group within one row of an output takes part
-    TileList near;
-    if (int rc = get_tiles(p, d, code == 333 ? 2 : 1, code == 333 ? 4 : 8, &near, 1)) return rc;
-    if (int rc = plan_scratch(p, conv_packed_floats(code, a.S_exp, a.Cin, a.Cout, true) * sizeof(float), st)) return rc;
-    if (int rc = pack_conv_weights(code, a.w, a.S_exp, a.Cin, a.Cout, true, (float*)p->d_scratch, st)) return rc;
-    ConvArgs<float> b = a;
-    b.tiles = near.d_tiles; b.n_tiles = near.n;
-    b.x = a.gy; b.ldx = a.ldy; b.Cin = a.Cout; b.Cout = a.Cin; b.w = (const float*)p->d_scratch; b.bias = nullptr;
-    b.tree_data = nullptr; b.t_count = 0;
-    if (near.n > 0) if (int rc = launch_conv_dx_mfma(code, b, near.n, st)) return rc;
+    if (a.gx) {
+        TileList near;
+        if (int rc = get_tiles(p, d, code == 333 ? 2 : 1, code == 333 ? 4 : 8, &near, 1)) return rc;
+        if (int rc = plan_scratch(p, conv_packed_floats(code, a.S_exp, a.Cin, a.Cout, true) * sizeof(float), st)) return rc;
+        if (int rc = pack_conv_weights(code, a.w, a.S_exp, a.Cin, a.Cout, true, (float*)p->d_scratch, st)) return rc;
+        ConvArgs<float> b = a;
+        b.tiles = near.d_tiles; b.n_tiles = near.n;
+        b.x = a.gy; b.ldx = a.ldy; b.Cin = a.Cout; b.Cout = a.Cin; b.w = (const float*)p->d_scratch; b.bias = nullptr;
+        b.tree_data = nullptr; b.t_count = 0;
+        if (near.n > 0) if (int rc = launch_conv_dx_mfma(code, b, near.n, st)) return rc;
+    }
     ConvArgs<float> c = a;
     if (int rc = set_conv_lists(p, d, code, tl, c, st)) return rc;
     return launch_conv_dw_mfma(code, c, tl, p->apr.level_min, st);
@@ -276,12 +280,15 @@ int conv_bwd(const aprnet_plan* cp, int d, int kz, int kx, int ky, const T* x, i
     if (code != 333 && code != 133 && code != 155 && code != 555)
         return fail(APRNET_ERR_UNSUPPORTED, "conv_backward: stencil must be 333, 133, 155 or 555");
     const int64_t nt = p->tree_parts(d);
-    if (nt > 0 && (!tree_ws || !gtree_ws || ldt < nt || ldgt < nt))
+    // gx == nullptr: the caller does not need the input gradient (first layer of a network); only gw is computed
+    if (nt > 0 && (!tree_ws || ldt < nt || (gx && (!gtree_ws || ldgt < nt))))
         return fail(APRNET_ERR_INVALID_ARGUMENT, "conv_backward: tree work space too small");
     APRNET_HIP_CHECK(hipSetDevice(p->device));
     if (int rc = fill_tree_for_conv(p, d, x, ldx, Cin, tree_ws, ldt, st)) return rc;
-    fill2d<T>(gx, ldgx, p->number_parts(d), Cin, (T)0, st);
-    fill2d<T>(gtree_ws, ldgt, nt, Cin, (T)0, st);
+    if (gx) {
+        fill2d<T>(gx, ldgx, p->number_parts(d), Cin, (T)0, st);
+        fill2d<T>(gtree_ws, ldgt, nt, Cin, (T)0, st);
+    }
     const bool flat = (kz == 1);
     TileList tl;
     if (int rc = get_tiles(p, d, flat ? 1 : 2, flat ? 8 : 4, &tl)) return rc;
@@ -304,7 +311,7 @@ int conv_bwd(const aprnet_plan* cp, int d, int kz, int kx, int ky, const T* x, i
         }
         if (rc) return rc;
     }
-    return fill_tree_bwd_for_conv(p, d, gx, ldgx, Cin, gtree_ws, ldgt, st);
+    return gx ? fill_tree_bwd_for_conv(p, d, gx, ldgx, Cin, gtree_ws, ldgt, st) : 0;
 }
 
 __global__ void round_to_bf16_kernel(const float* __restrict__ src, int64_t lds, bf16_t* __restrict__ dst, int64_t ldd, int64_t n) {
@@ -327,12 +334,14 @@ int conv_bwd_bf16(const aprnet_plan* cp, int d, int kz, int kx, int ky, const bf
     if (!conv_mfma_supported(code))
         return fail(APRNET_ERR_UNSUPPORTED, "conv_backward: bfloat16 features are supported for the 3x3x3, 1x3x3 and 1x5x5 stencils");
     const int64_t nt = p->tree_parts(d), np = p->number_parts(d);
-    if (!gx32_ws || ldgx32 < np || (nt > 0 && (!tree_ws || !gtree_ws || ldt < nt || ldgt < nt)))
+    if ((gx && (!gx32_ws || ldgx32 < np)) || (nt > 0 && (!tree_ws || ldt < nt || (gx && (!gtree_ws || ldgt < nt)))))
         return fail(APRNET_ERR_INVALID_ARGUMENT, "conv_backward: work space too small");
     APRNET_HIP_CHECK(hipSetDevice(p->device));
     if (int rc = fill_tree_for_conv(p, d, x, ldx, Cin, tree_ws, ldt, st)) return rc;
-    fill2d<float>(gx32_ws, ldgx32, np, Cin, 0.f, st);
-    fill2d<float>(gtree_ws, ldgt, nt, Cin, 0.f, st);
+    if (gx) {
+        fill2d<float>(gx32_ws, ldgx32, np, Cin, 0.f, st);
+        fill2d<float>(gtree_ws, ldgt, nt, Cin, 0.f, st);
+    }
     const bool flat = (kz == 1);
     TileList tl, near;
     if (int rc = get_tiles(p, d, flat ? 1 : 2, flat ? 8 : 4, &tl)) return rc;
@@ -350,6 +359,7 @@ int conv_bwd_bf16(const aprnet_plan* cp, int d, int kz, int kx, int ky, const bf
         b.tree_data = nullptr; b.t_count = 0;
         // input gradient: bfloat16 products on the input-gradient lists of the plan when they are there, otherwise
         // (lists off or not buildable, fp32 products asked for) the scanning kernel with fp32 products
+        if (!gx) near.n = 0;              // no input gradient asked for
         if (near.n > 0 && bf16_math())
             if (int rc = set_conv_dx_lists(p, d, code, near, b, st)) return rc;
         if (near.n > 0 && b.tile_win) {
@@ -367,6 +377,7 @@ int conv_bwd_bf16(const aprnet_plan* cp, int d, int kz, int kx, int ky, const bf
         if (int rc = set_conv_lists(p, d, code, tl, a, st)) return rc;
         if (int rc = launch_conv_dw_mfma(code, a, tl, p->apr.level_min, st)) return rc;
     }
+    if (!gx) return 0;
     if (int rc = fill_tree_bwd_for_conv(p, d, gx32_ws, ldgx32, Cin, gtree_ws, ldgt, st)) return rc;
     if (np > 0) {
         dim3 grid((unsigned)std::min<int64_t>((np + 255) / 256, 4096), (unsigned)Cin);

@@ -30,6 +30,7 @@ using W155M = ConvGeom<1, 5, 5, 1, 8, 512, 69>;
 constexpr int DW_CIB = 4;          // input channels per staged chunk
 constexpr int DW_NCH = 4;          // chunks per block
 constexpr int DW_GB = 256;         // columns of gY staged at a time
+constexpr int DW_KB = 8;          // MFMAs issued back to back between operand phases (16 would spill registers)
 constexpr int DW_GLD = 33;         // words per column of gyl (32 output channels + 1 against bank conflicts)
 
 // Lists of the plan carry patch cells for rows of 64 words; this kernel's rows are RS words apart.
@@ -85,20 +86,23 @@ __device__ __forceinline__ void dw_window(const ConvArgs<T>& a, const Lists& sh,
             for (int b = 0; b < nbatch; ++b) {
                 const float* apb = ap + (b * 64 + 32 * kh) * DW_GLD;
                 // Three separate phases, kept apart by scheduling barriers: operand addresses (one LDS read of the
-                // column's cell and one vector add each), then all operand reads, then 16 MFMAs back to back.  A
+                // column's cell and one vector add each), then the operand reads, then DW_KB MFMAs back to back.  A
                 // vector instruction between two fp32 MFMAs costs a pipeline switch each time.
                 const int* cp = cpl + b * 64 + 32 * hi + 16 * kh;      // lanes of the upper half take column k + 32
-                int addr[16];
 #pragma unroll
-                for (int k = 0; k < 16; ++k) addr[k] = bl + cp[k];
-                __builtin_amdgcn_sched_barrier(0);
-                float av[16], bv[16];
+                for (int h = 0; h < 16; h += DW_KB) {
+                    int addr[DW_KB];
 #pragma unroll
-                for (int k = 0; k < 16; ++k) { av[k] = apb[2 * k * DW_GLD]; bv[k] = patch[addr[k]]; }
-                __builtin_amdgcn_sched_barrier(0);
+                    for (int k = 0; k < DW_KB; ++k) addr[k] = bl + cp[h + k];
+                    __builtin_amdgcn_sched_barrier(0);
+                    float av[DW_KB], bv[DW_KB];
 #pragma unroll
-                for (int k = 0; k < 16; ++k) acc[q] = __builtin_amdgcn_mfma_f32_32x32x2f32(av[k], bv[k], acc[q], 0, 0, 0);
-                __builtin_amdgcn_sched_barrier(0);
+                    for (int k = 0; k < DW_KB; ++k) { av[k] = apb[2 * (h + k) * DW_GLD]; bv[k] = patch[addr[k]]; }
+                    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                    for (int k = 0; k < DW_KB; ++k) acc[q] = __builtin_amdgcn_mfma_f32_32x32x2f32(av[k], bv[k], acc[q], 0, 0, 0);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
             }
         }
         __syncthreads();            // gyl is rewritten by the next group, the patch by the next window
@@ -188,9 +192,13 @@ static int launch_dw(const ConvArgs<T>& a0, const TileList& tl, int level_min, h
         ConvArgs<T> a = a0;
         a.tiles = tl.d_tiles + tl.level_begin[l_hi]; a.n_tiles = n;
         if (a.tile_win) a.tile_win += tl.level_begin[l_hi];
-        dim3 grid((unsigned)std::min(n, 512), (unsigned)((a.Cin + DW_CIB * DW_NCH - 1) / (DW_CIB * DW_NCH)),
-                  (unsigned)((a.Cout + 31) / 32));
-        if (a.tile_win) hipLaunchKernelGGL((conv_dw_mfma_kernel<T, G, DW_CIB, DW_NCH, true>), grid, dim3(G::NT), 0, st, a, s);
+        // a narrow input (the first layer of a network) fits one chunk: no staging and products of empty chunks
+        const int nch = a.Cin <= DW_CIB ? 1 : DW_NCH;
+        dim3 grid((unsigned)std::min(n, 512), (unsigned)((a.Cin + DW_CIB * nch - 1) / (DW_CIB * nch)), (unsigned)((a.Cout + 31) / 32));
+        if (nch == 1) {
+            if (a.tile_win) hipLaunchKernelGGL((conv_dw_mfma_kernel<T, G, DW_CIB, 1, true>), grid, dim3(G::NT), 0, st, a, s);
+            else hipLaunchKernelGGL((conv_dw_mfma_kernel<T, G, DW_CIB, 1, false>), grid, dim3(G::NT), 0, st, a, s);
+        } else if (a.tile_win) hipLaunchKernelGGL((conv_dw_mfma_kernel<T, G, DW_CIB, DW_NCH, true>), grid, dim3(G::NT), 0, st, a, s);
         else hipLaunchKernelGGL((conv_dw_mfma_kernel<T, G, DW_CIB, DW_NCH, false>), grid, dim3(G::NT), 0, st, a, s);
         APRNET_LAUNCH_CHECK("conv_dw_mfma_kernel");
     }

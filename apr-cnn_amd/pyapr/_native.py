@@ -104,6 +104,13 @@ def hip():
     lib.aprnet_sample_image_max_f32.argtypes = [vp, i32, vp, i32, i32, i32, vp, vp]
     for t in ("u8", "u16", "u32", "u64"):     # plan, d, img, zn, xn, yn, dzs, dxs, dys, n_rays, max_steps, dist, stream
         getattr(lib, f"aprnet_labels_to_dist_{t}").argtypes = [vp, i32, vp, i32, i32, i32, vp, vp, vp, i32, i32, vp, vp]
+    lib.aprnet_norm_work_elems.argtypes = [i64]
+    lib.aprnet_norm_work_elems.restype = i64
+    for t in ("f32", "bf16"):
+        getattr(lib, f"aprnet_row_moments_{t}").argtypes = [vp, i64, i64, i64, vp, vp, vp, vp]
+        getattr(lib, f"aprnet_norm_apply_{t}").argtypes = [vp, i64, i64, i64, vp, vp, vp, i32, vp, i64, vp]
+        getattr(lib, f"aprnet_norm_bwd_sums_{t}").argtypes = [vp, i64, vp, i64, vp, i64, i64, i64, vp, vp, vp, vp, vp, vp]
+        getattr(lib, f"aprnet_norm_bwd_apply_{t}").argtypes = [vp, i64, vp, i64, vp, i64, i64, i64, vp, vp, vp, vp, vp, vp, i64, vp]
     for t in ("f32", "f64", "bf16"):      # ..., tree_ws, ld_tree, const aprnet_conv_fusion*, stream
         getattr(lib, f"aprnet_conv_fwd_fused_{t}").argtypes = [vp, i32, i32, i32, i32, vp, i64, i32, vp, i32, i32, vp, vp, i64,
                                                                 vp, i64, vp, vp]

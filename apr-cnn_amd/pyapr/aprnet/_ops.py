@@ -224,8 +224,92 @@ def channel_sum(x):
     return out
 
 
-def conv_backward(aprs, x, weights, grad_output, level_delta):
-    """conv333_backward / conv111_backward (wrap_conv_gpu.hpp:87-133, 216-246) -> [grad_input, grad_weights]."""
+# ---------------------------------------------------------------------------- normalisation over the particle axis
+def _norm_sfx(x, name):
+    _check_input(x, name)
+    if x.dtype not in (torch.float32, torch.bfloat16) or x.dim() != 3:
+        raise TypeError(f"{name}: [batch, channels, particles] float32 or bfloat16 tensor expected")
+    return "f32" if x.dtype == torch.float32 else "bf16"
+
+
+def _norm_work(rows, device):
+    return torch.empty(_lib().aprnet_norm_work_elems(rows), dtype=torch.float32, device=device)
+
+
+def _rowvec(v, rows, name):
+    if v.dtype != torch.float32 or v.numel() != rows or not v.is_cuda or not v.is_contiguous():
+        raise ValueError(f"{name}: contiguous float32 GPU tensor with one value per (batch item, channel) expected")
+    return v
+
+
+def row_moments(x):
+    """[B, C, N] -> (mean, m2) float64 [B, C]: mean and sum of squared deviations of every row."""
+    sfx = _norm_sfx(x, "input")
+    B, Cn, N = x.shape
+    mean = torch.empty(B, Cn, dtype=torch.float64, device=x.device)
+    m2 = torch.empty_like(mean)
+    with torch.cuda.device(x.device):
+        rc = getattr(_lib(), "aprnet_row_moments_" + sfx)(_ptr(x), N, B * Cn, N, _ptr(mean), _ptr(m2),
+                                                          _ptr(_norm_work(B * Cn, x.device)), _stream())
+    if rc:
+        _raise(rc, "row_moments failed")
+    return mean, m2
+
+
+def norm_apply(x, mean, scale, shift, relu):
+    """y = (x - mean) * scale + shift per row (float32 [B, C] coefficients), then ReLU if asked."""
+    sfx = _norm_sfx(x, "input")
+    B, Cn, N = x.shape
+    y = torch.empty_like(x)
+    with torch.cuda.device(x.device):
+        rc = getattr(_lib(), "aprnet_norm_apply_" + sfx)(_ptr(x), N, B * Cn, N, _ptr(_rowvec(mean, B * Cn, "mean")),
+                                                         _ptr(_rowvec(scale, B * Cn, "scale")), _ptr(_rowvec(shift, B * Cn, "shift")),
+                                                         1 if relu else 0, _ptr(y), N, _stream())
+    if rc:
+        _raise(rc, "norm_apply failed")
+    return y
+
+
+def norm_backward_sums(gy, x, y, mean, rstd):
+    """-> (sum g, sum g * xhat) float64 [B, C];  g = gy masked by y > 0 when the forward output y is given."""
+    sfx = _norm_sfx(x, "input")
+    _check_input(gy, "grad_output")
+    if gy.dtype != x.dtype or gy.shape != x.shape or (y is not None and (y.dtype != x.dtype or y.shape != x.shape or not y.is_contiguous())):
+        raise ValueError("norm_backward_sums: grad_output / output must match the input in type and shape")
+    B, Cn, N = x.shape
+    s_g = torch.empty(B, Cn, dtype=torch.float64, device=x.device)
+    s_gx = torch.empty_like(s_g)
+    with torch.cuda.device(x.device):
+        rc = getattr(_lib(), "aprnet_norm_bwd_sums_" + sfx)(_ptr(gy), N, _ptr(x), N, None if y is None else _ptr(y), N, B * Cn, N,
+                                                            _ptr(_rowvec(mean, B * Cn, "mean")), _ptr(_rowvec(rstd, B * Cn, "rstd")),
+                                                            _ptr(s_g), _ptr(s_gx), _ptr(_norm_work(B * Cn, x.device)), _stream())
+    if rc:
+        _raise(rc, "norm_backward_sums failed")
+    return s_g, s_gx
+
+
+def norm_backward_apply(gy, x, y, mean, rstd, a, b, c):
+    """gx = a * g + b * xhat + c per row."""
+    sfx = _norm_sfx(x, "input")
+    _check_input(gy, "grad_output")
+    if gy.dtype != x.dtype or gy.shape != x.shape or (y is not None and (y.dtype != x.dtype or y.shape != x.shape or not y.is_contiguous())):
+        raise ValueError("norm_backward_apply: grad_output / output must match the input in type and shape")
+    B, Cn, N = x.shape
+    gx = torch.empty_like(x)
+    rows = B * Cn
+    with torch.cuda.device(x.device):
+        rc = getattr(_lib(), "aprnet_norm_bwd_apply_" + sfx)(_ptr(gy), N, _ptr(x), N, None if y is None else _ptr(y), N, rows, N,
+                                                             _ptr(_rowvec(mean, rows, "mean")), _ptr(_rowvec(rstd, rows, "rstd")),
+                                                             _ptr(_rowvec(a, rows, "a")), _ptr(_rowvec(b, rows, "b")),
+                                                             _ptr(_rowvec(c, rows, "c")), _ptr(gx), N, _stream())
+    if rc:
+        _raise(rc, "norm_backward_apply failed")
+    return gx
+
+
+def conv_backward(aprs, x, weights, grad_output, level_delta, need_input_grad=True):
+    """conv333_backward / conv111_backward (wrap_conv_gpu.hpp:87-133, 216-246) -> [grad_input, grad_weights].
+    ``need_input_grad=False`` (stencil convolutions): the input gradient is not computed, grad_input is None."""
     _check_input(x, "input")
     _check_input(weights, "weights")
     _check_input(grad_output, "grad_output")
@@ -233,8 +317,11 @@ def conv_backward(aprs, x, weights, grad_output, level_delta):
     B, _, N = x.shape
     d = _deltas(level_delta, len(aprs))
     sizes = [number_particles(a, d[b]) for b, a in enumerate(aprs)]
-    gx = torch.empty_like(x)
-    _zero_tails(gx, sizes)
+    skip_gx = not need_input_grad and (kz, kx, ky) != (1, 1, 1)
+    gx = None if skip_gx else torch.empty_like(x)
+    if gx is not None:
+        _zero_tails(gx, sizes)
+    gxp = (lambda b: None) if skip_gx else (lambda b: _ptr(gx[b]))
     plans = _plans(aprs, x.device)
     if x.dtype == torch.bfloat16:
         # bfloat16 features and output gradient; weights and their gradient in fp32, fp32 accumulation
@@ -244,14 +331,15 @@ def conv_backward(aprs, x, weights, grad_output, level_delta):
         gw = torch.zeros_like(weights)
         ld_tree = max(max(tree_parts(a, d[b]) for b, a in enumerate(aprs)), 1)
         tree_ws = torch.empty((cin, ld_tree), dtype=x.dtype, device=x.device)
-        gtree_ws = torch.empty((cin, ld_tree), dtype=torch.float32, device=x.device)
-        gx32_ws = torch.empty((cin, N), dtype=torch.float32, device=x.device)
+        gtree_ws = None if skip_gx else torch.empty((cin, ld_tree), dtype=torch.float32, device=x.device)
+        gx32_ws = None if skip_gx else torch.empty((cin, N), dtype=torch.float32, device=x.device)
         with torch.cuda.device(x.device):
             st = _stream()
             for b in range(B):
                 rc = _lib().aprnet_conv_bwd_bf16(plans[b], d[b], kz, kx, ky, _ptr(x[b]), N, cin, _ptr(weights), s_exp, cout,
-                                                 _ptr(grad_output[b]), grad_output.size(2), _ptr(gx[b]), N, _ptr(gw),
-                                                 _ptr(tree_ws), ld_tree, _ptr(gx32_ws), N, _ptr(gtree_ws), ld_tree, st)
+                                                 _ptr(grad_output[b]), grad_output.size(2), gxp(b), N, _ptr(gw),
+                                                 _ptr(tree_ws), ld_tree, None if skip_gx else _ptr(gx32_ws), N,
+                                                 None if skip_gx else _ptr(gtree_ws), ld_tree, st)
                 if rc:
                     _raise(rc, "conv_backward failed")
         return [gx, gw]
@@ -269,12 +357,12 @@ def conv_backward(aprs, x, weights, grad_output, level_delta):
         else:
             ld_tree = max(max(tree_parts(a, d[b]) for b, a in enumerate(aprs)), 1)
             tree_ws = torch.empty((cin, ld_tree), dtype=x.dtype, device=x.device)
-            gtree_ws = torch.empty((cin, ld_tree), dtype=x.dtype, device=x.device)
+            gtree_ws = None if skip_gx else torch.empty((cin, ld_tree), dtype=x.dtype, device=x.device)
             fn = getattr(_lib(), "aprnet_conv_bwd_" + sfx)
             for b in range(B):
                 rc = fn(plans[b], d[b], kz, kx, ky, _ptr(x[b]), N, cin, _ptr(weights), s_exp, cout,
-                        _ptr(grad_output[b]), grad_output.size(2), _ptr(gx[b]), N, _ptr(gw),
-                        _ptr(tree_ws), ld_tree, _ptr(gtree_ws), ld_tree, st)
+                        _ptr(grad_output[b]), grad_output.size(2), gxp(b), N, _ptr(gw),
+                        _ptr(tree_ws), ld_tree, None if skip_gx else _ptr(gtree_ws), ld_tree, st)
                 if rc:
                     _raise(rc, "conv_backward failed")
     return [gx, gw]

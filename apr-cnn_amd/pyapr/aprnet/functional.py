@@ -57,7 +57,8 @@ class ConvFunction(Function):
     def backward(ctx, grad_output):
         inputs, w_exp, bias, level_deltas = ctx.saved_tensors
         grad_output = grad_output.contiguous()
-        grad_input, grad_w = _ops.conv_backward(ctx.aprs, inputs, w_exp, grad_output, level_deltas)
+        grad_input, grad_w = _ops.conv_backward(ctx.aprs, inputs, w_exp, grad_output, level_deltas,
+                                                need_input_grad=ctx.needs_input_grad[0])
         grad_bias = None if bias is None else _ops.channel_sum(grad_output)
         if ctx.expand:
             grad_w = _ops.restrict_kernel_backward(grad_w, ctx.num_stencils)
@@ -81,6 +82,76 @@ def conv_inference(inputs, weights, bias, aprs, level_deltas, layout, relu=False
         w = _ops.restrict_kernel_forward(w, max(a.level_max() - a.level_min() + 1 for a in aprs))
     return _ops.conv_forward(aprs, inputs.contiguous(), w, level_deltas, None if bias is None else bias.detach().contiguous(),
                              relu=relu, x2=None if inputs2 is None else inputs2.contiguous())
+
+
+class NormFunction(Function):
+    """Normalisation over the particle axis (+ optional ReLU) of a [B, C, N] tensor with the arithmetic of
+    torch.nn.BatchNorm1d (``kind='batch'``: one set of statistics per channel, taken over batch and particles) and
+    torch.nn.GroupNorm (``kind='group'``: one per batch item and group), as BasicBlock applies them
+    (apr_models/unet/unet_parts.py:17-26).  ``stats`` = (mean[C], var[C]) normalises with given statistics (BatchNorm in
+    eval mode) instead of those of the input.  Returns ``(y, mean, var)``: the statistics used (biased variance), per
+    channel for 'batch' and [B, groups] for 'group'."""
+
+    @staticmethod
+    def forward(ctx, x, weight, bias, kind, groups, eps, relu, stats):
+        B, Cn, N = x.shape
+        x = x.contiguous()
+        if stats is None:
+            mean_r, m2_r = _ops.row_moments(x)                      # float64 [B, C]
+            if kind == "batch":
+                k, mr, m2 = B, mean_r.t(), m2_r.t()                 # [C, B]
+            else:
+                k = Cn // groups
+                mr, m2 = mean_r.view(B, groups, k), m2_r.view(B, groups, k)
+            set_mean = mr.mean(-1)
+            set_var = (m2.sum(-1) + N * (mr - set_mean.unsqueeze(-1)).square().sum(-1)) / (k * N)
+        else:
+            set_mean, set_var = stats[0].double(), stats[1].double()
+
+        def to_rows(v):
+            if kind == "batch":
+                return v.unsqueeze(0).expand(B, Cn)
+            return v.unsqueeze(-1).expand(B, groups, Cn // groups).reshape(B, Cn)
+        rstd = to_rows((set_var + eps).rsqrt())
+        gamma = torch.ones(Cn, dtype=torch.float64, device=x.device) if weight is None else weight.detach().double()
+        beta = torch.zeros(Cn, dtype=torch.float64, device=x.device) if bias is None else bias.detach().double()
+        mean32 = to_rows(set_mean).float().contiguous()
+        rstd32 = rstd.float().contiguous()
+        y = _ops.norm_apply(x, mean32, (gamma.unsqueeze(0) * rstd).float().contiguous(),
+                            beta.unsqueeze(0).expand(B, Cn).float().contiguous(), relu)
+        ctx.save_for_backward(x, y if relu else None, mean32, rstd32, weight)
+        ctx.cfg = (kind, groups, stats is None, None if weight is None else weight.dtype, None if bias is None else bias.dtype)
+        ctx.mark_non_differentiable(set_mean, set_var)
+        return y, set_mean, set_var
+
+    @staticmethod
+    def backward(ctx, grad_y, _gm, _gv):
+        x, y, mean32, rstd32, weight = ctx.saved_tensors
+        kind, groups, own_stats, w_dtype, b_dtype = ctx.cfg
+        B, Cn, N = x.shape
+        grad_y = grad_y.contiguous()
+        s_g, s_gx = _ops.norm_backward_sums(grad_y, x, y, mean32, rstd32)          # float64 [B, C]
+        grad_w = s_gx.sum(0).to(w_dtype) if w_dtype is not None and ctx.needs_input_grad[1] else None
+        grad_b = s_g.sum(0).to(b_dtype) if b_dtype is not None and ctx.needs_input_grad[2] else None
+        grad_x = None
+        if ctx.needs_input_grad[0]:
+            gamma = torch.ones(Cn, dtype=torch.float64, device=x.device) if weight is None else weight.detach().double()
+            rstd = rstd32.double()
+            a = gamma.unsqueeze(0) * rstd
+            if own_stats:       # the statistics depend on the input: subtract the set means of g and g * xhat
+                g1, g2 = gamma * s_g, gamma * s_gx
+                if kind == "batch":
+                    G1, G2 = (g1.sum(0) / (B * N)).expand(B, Cn), (g2.sum(0) / (B * N)).expand(B, Cn)
+                else:
+                    k = Cn // groups
+                    G1 = (g1.view(B, groups, k).sum(-1, keepdim=True) / (k * N)).expand(B, groups, k).reshape(B, Cn)
+                    G2 = (g2.view(B, groups, k).sum(-1, keepdim=True) / (k * N)).expand(B, groups, k).reshape(B, Cn)
+                b, c = -rstd * G2, -rstd * G1
+            else:
+                b = c = torch.zeros_like(a)
+            grad_x = _ops.norm_backward_apply(grad_y, x, y, mean32, rstd32, a.float().contiguous(), b.float().contiguous(),
+                                              c.float().contiguous())
+        return grad_x, grad_w, grad_b, None, None, None, None, None
 
 
 class MaxPoolFunction(Function):

@@ -155,6 +155,19 @@ def other_ops(apr, x, dev):
         ms = _time(graph.replay, iters=3, warmup=1)
     res.append({"op": "apr_unet_fwd_graph", "ms": ms, "note": "the fp32 forward replayed from a HIP graph"})
     del graph, y_graph
+    # one training step of the same architecture (unfolded BatchNorm in training mode): forward, loss, backward
+    torch.manual_seed(0)
+    tnet = APRUNet(1, 3, depth=3, n_filters_base=16, n_stencils=2, norm="batch").to(dev).train()
+    target = torch.randn(1, 3, xin.shape[2], device=dev)
+
+    def train_step():
+        for p_ in tnet.parameters():
+            p_.grad = None
+        torch.nn.functional.mse_loss(tnet(xin, [apr]), target).backward()
+    ms = _time(train_step, iters=2, warmup=1)
+    res.append({"op": "apr_unet_train_step", "ms": ms, "particles_per_s": n0 / ms * 1e3,
+                "note": "forward + backward of the 4-level network, fp32, BatchNorm in training mode, MSE loss, no optimizer"})
+    del tnet, target
     # the wide 2-D stencil of configs[4] (1x5x5, 64 -> 64), here on the 3-D benchmark APR, fp32
     conv5 = aprnet.cuda.APRConv(64, 64, nstencils=2, kernel_size=(1, 5, 5)).to(dev)
     x64 = torch.randn(1, 64, x.shape[2], device=dev)

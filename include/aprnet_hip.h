@@ -130,7 +130,9 @@ typedef struct aprnet_conv_fusion {
                                     const aprnet_conv_fusion* fusion, void* stream);                                \
     /* Convolution<kz,kx,ky>::backward (conv.hpp:261-481), CUDA twin conv333_backward.  grad_x is OVERWRITTEN,      \
      * grad_w [S_exp][Cout][Cin][k] is ACCUMULATED into (zero it before the first batch item, as                    \
-     * torch::zeros_like does in conv.hpp:270).  tree_ws / grad_tree_ws: [Cin][ld_tree] scratch each. */            \
+     * torch::zeros_like does in conv.hpp:270).  tree_ws / grad_tree_ws: [Cin][ld_tree] scratch each.               \
+     * grad_x may be NULL (no counterpart in the reference: the first layer of a network needs no input gradient):  \
+     * then only grad_w is computed and grad_tree_ws is not used. */                                                \
     int aprnet_conv_bwd_##SFX(const aprnet_plan*, int level_delta, int kz, int kx, int ky,                          \
                               const T* x, int64_t ldx, int Cin, const T* w, int S_exp, int Cout,                    \
                               const T* grad_y, int64_t ldy, T* grad_x, int64_t ldgx, T* grad_w,                     \
@@ -205,7 +207,8 @@ int aprnet_upsample_fwd_bf16(const aprnet_plan*, int level_delta, const uint16_t
  * space gx32_ws [Cin][ld_gx32] (ld_gx32 >= aprnet_number_parts) and rounded to bfloat16 into gx at the end.
  * gtree_ws: fp32 [Cin][ld_gtree].  The input gradient multiplies on the bfloat16 matrix cores (weights rounded to
  * bfloat16) from input-gradient lists that the plan builds on first use; with aprnet_set_conv_path(3) or (5) it
- * runs with fp32 products and scans per call.  The weight gradient always uses fp32 products. */
+ * runs with fp32 products and scans per call.  The weight gradient always uses fp32 products.  gx may be NULL:
+ * then only gw is computed and gx32_ws / gtree_ws are not used. */
 int aprnet_conv_bwd_bf16(const aprnet_plan*, int level_delta, int kz, int kx, int ky, const uint16_t* x, int64_t ldx, int Cin,
                          const float* w, int S_exp, int Cout, const uint16_t* gy, int64_t ldy, uint16_t* gx, int64_t ldgx,
                          float* gw, uint16_t* tree_ws, int64_t ld_tree, float* gx32_ws, int64_t ld_gx32, float* gtree_ws,
@@ -234,6 +237,38 @@ int aprnet_labels_to_dist_u32(const aprnet_plan*, int level_delta, const uint32_
                               const float* dxs, const float* dys, int n_rays, int max_steps, float* dist, void* stream);
 int aprnet_labels_to_dist_u64(const aprnet_plan*, int level_delta, const uint64_t* img, int zn, int xn, int yn, const float* dzs,
                               const float* dxs, const float* dys, int n_rays, int max_steps, float* dist, void* stream);
+
+/* Normalisation over the particle axis and the ReLU after it: the torch.nn.BatchNorm1d / torch.nn.GroupNorm +
+ * activation that follow every convolution of the networks (apr_models/unet/unet_parts.py:17-26; library calls on
+ * [batch, channels, particles] tensors in the reference, MIOpen / ATen kernels on a GPU).  The kernels work on
+ * rows: row r = one (batch item, channel) line of n elements at x + r * ldx.  The caller joins the per-row results
+ * into per-channel (BatchNorm) or per-group (GroupNorm) statistics - a few values per row - and passes per-row
+ * coefficients back.  rows <= 65535, n > 0.  work: aprnet_norm_work_elems(rows) floats of scratch.
+ *   row_moments     mean[r], m2[r] = mean and sum of squared deviations of row r (fp64 results).
+ *   norm_apply      y = (x - mean[r]) * scale[r] + shift[r], then max(., 0) if relu != 0.
+ *   norm_bwd_sums   sum_g[r] = sum g, sum_gx[r] = sum g * xhat with xhat = (x - mean[r]) * rstd[r] and
+ *                   g = gy, or gy where y > 0 and 0 elsewhere when y (the forward output) is given.
+ *   norm_bwd_apply  gx = a[r] * g + b[r] * xhat + c[r].
+ * Sums are taken in a fixed order (fp32 per thread and block, fp64 across blocks): results repeat bit for bit. */
+int64_t aprnet_norm_work_elems(int64_t rows);
+int aprnet_row_moments_f32(const float* x, int64_t ldx, int64_t rows, int64_t n, double* mean, double* m2, float* work, void* stream);
+int aprnet_row_moments_bf16(const uint16_t* x, int64_t ldx, int64_t rows, int64_t n, double* mean, double* m2, float* work, void* stream);
+int aprnet_norm_apply_f32(const float* x, int64_t ldx, int64_t rows, int64_t n, const float* mean, const float* scale,
+                          const float* shift, int relu, float* y, int64_t ldy, void* stream);
+int aprnet_norm_apply_bf16(const uint16_t* x, int64_t ldx, int64_t rows, int64_t n, const float* mean, const float* scale,
+                           const float* shift, int relu, uint16_t* y, int64_t ldy, void* stream);
+int aprnet_norm_bwd_sums_f32(const float* gy, int64_t ldg, const float* x, int64_t ldx, const float* y, int64_t ldy, int64_t rows,
+                             int64_t n, const float* mean, const float* rstd, double* sum_g, double* sum_gx, float* work,
+                             void* stream);
+int aprnet_norm_bwd_sums_bf16(const uint16_t* gy, int64_t ldg, const uint16_t* x, int64_t ldx, const uint16_t* y, int64_t ldy,
+                              int64_t rows, int64_t n, const float* mean, const float* rstd, double* sum_g, double* sum_gx,
+                              float* work, void* stream);
+int aprnet_norm_bwd_apply_f32(const float* gy, int64_t ldg, const float* x, int64_t ldx, const float* y, int64_t ldy, int64_t rows,
+                              int64_t n, const float* mean, const float* rstd, const float* a, const float* b, const float* c,
+                              float* gx, int64_t ldo, void* stream);
+int aprnet_norm_bwd_apply_bf16(const uint16_t* gy, int64_t ldg, const uint16_t* x, int64_t ldx, const uint16_t* y, int64_t ldy,
+                               int64_t rows, int64_t n, const float* mean, const float* rstd, const float* a, const float* b,
+                               const float* c, uint16_t* gx, int64_t ldo, void* stream);
 
 #ifdef __cplusplus
 }

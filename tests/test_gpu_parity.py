@@ -244,6 +244,34 @@ def test_conv333_backward_channel_shapes(cin, cout, path):
 
 
 @pytest.mark.parametrize("path", [0, 1], ids=["mfma", "valu"])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
+@pytest.mark.parametrize("cin,cout", [(1, 16), (5, 4), (18, 33)])
+def test_conv_backward_weights_only(cin, cout, dtype, path):
+    """need_input_grad=False (what autograd asks of the first layer of a network): no input gradient, the same weight
+    gradient; channel counts that leave whole input-channel chunks of the weight-gradient kernel empty."""
+    if dtype == torch.bfloat16 and path == 1:
+        pytest.skip("bfloat16 features run on the matrix-core kernels only")
+    x, aprs, ld, w_exp = _conv_case([("3d_s", 0), ("3d_t", 1)], (3, 3, 3), 2, cin, cout, torch.float32)
+    g = torch.Generator().manual_seed(9)
+    go = torch.randn(x.size(0), cout, x.size(2), generator=g)
+    if dtype == torch.bfloat16:
+        x, go = x.to(dtype).float(), go.to(dtype).float()          # the oracle sees the rounded values
+    _, gw_ref = oracle.conv_backward(aprs, x, w_exp, go, ld)
+    wd = w_exp.permute(1, 2, 0, 3, 4, 5).contiguous().to(DEV)
+    lib = _native.hip()
+    assert lib.aprnet_set_conv_path(path) == 0
+    try:
+        gx, gw = _ops.conv_backward(aprs, x.to(DEV).to(dtype), wd, go.to(DEV).to(dtype), ld, need_input_grad=False)
+    finally:
+        lib.aprnet_set_conv_path(0)
+    assert gx is None
+    if dtype == torch.bfloat16:      # the mean-filled tree values that the sums read are stored in bfloat16
+        assert float((gw.permute(2, 0, 1, 3, 4, 5).cpu() - gw_ref).abs().max()) <= 1e-2 * float(gw_ref.abs().max())
+    else:
+        close(gw.permute(2, 0, 1, 3, 4, 5), gw_ref, torch.float32)
+
+
+@pytest.mark.parametrize("path", [0, 1], ids=["mfma", "valu"])
 @pytest.mark.parametrize("ksize", [(1, 3, 3), (1, 5, 5)], ids=KID)
 @pytest.mark.parametrize("bt", [[("2d_a", 0), ("2d_b", 1)], [("3d_s", 0)]], ids=lambda b: "+".join(f"{n}@{d}" for n, d in b))
 def test_conv_flat_stencils_wide_channels(bt, ksize, path):

@@ -9,6 +9,7 @@ import apr_cases
 from oracle import oracle
 from oracle_modules import OracleConv, OracleMaxPool, OracleUpSample
 from apr_models.unet import APRUNet, fold_norms
+from pyapr.aprnet import _ops
 
 pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
@@ -301,3 +302,83 @@ def test_hybrid_stardist_unet_matches_oracle():
     assert prob.shape == (1, 1, n1) and dist.shape == (1, 6, n1)
     assert float((prob.cpu() - ref_prob).abs().max()) < 5e-5
     assert float((dist.cpu() - ref_dist).abs().max()) < 5e-5 * float(ref_dist.abs().max())
+
+
+# ---------------------------------------------------------------------------- normalisation over the particle axis
+def _norm_pair(kind, C, groups, dtype, seed):
+    from apr_models.unet.particle_norm import ParticleBatchNorm, ParticleGroupNorm
+    torch.manual_seed(seed)
+    if kind == "batch":
+        mine, ref = ParticleBatchNorm(C, momentum=0.1), torch.nn.BatchNorm1d(C, momentum=0.1)
+    else:
+        mine, ref = ParticleGroupNorm(groups, C), torch.nn.GroupNorm(groups, C)
+    with torch.no_grad():
+        mine.weight.copy_(torch.randn(C) * 0.5 + 1.0)
+        mine.bias.copy_(torch.randn(C))
+    ref.load_state_dict(mine.state_dict())            # interchangeable state
+    return mine.to(DEV), ref.double()
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("kind,C,groups", [("batch", 6, 1), ("group", 6, 6), ("group", 8, 2), ("group", 5, 1)])
+@pytest.mark.parametrize("B,N", [(1, 4099), (3, 1021), (2, 3)])
+@pytest.mark.parametrize("relu", [False, True])
+def test_particle_norm_matches_torch(kind, C, groups, B, N, relu):
+    """Forward, input / weight / bias gradients and running statistics of the streaming-kernel norms against the
+    torch modules the reference uses (float64 on the CPU).  Tolerance 1e-5 relative to the tensor's largest entry."""
+    mine, ref = _norm_pair(kind, C, groups, torch.float32, 7)
+    g = torch.Generator().manual_seed(B * 1000 + N)
+    x = torch.randn(B, C, N, generator=g) * 3.0 + 10.0            # a mean well away from zero
+    go = torch.randn(B, C, N, generator=g)
+    for step in range(2):                                          # two steps: running statistics accumulate
+        xm = x.to(DEV).requires_grad_(True)
+        xr = x.double().requires_grad_(True)
+        ym = mine(xm, relu=relu)
+        yr = ref(xr)
+        if relu:
+            yr = torch.relu(yr)
+        ym.backward(go.to(DEV)); yr.backward(go.double())
+
+        def close(a, b, tol=1e-5):
+            a, b = a.detach().double().cpu(), b.detach().double()
+            assert a.shape == b.shape
+            assert (a - b).abs().max().item() <= tol * max(b.abs().max().item(), 1.0), (a - b).abs().max().item()
+        close(ym, yr); close(xm.grad, xr.grad)
+        close(mine.weight.grad, ref.weight.grad, 2e-5); close(mine.bias.grad, ref.bias.grad, 2e-5)
+        if kind == "batch":
+            close(mine.running_mean, ref.running_mean); close(mine.running_var, ref.running_var)
+            assert int(mine.num_batches_tracked) == int(ref.num_batches_tracked) == step + 1
+        mine.zero_grad(); ref.zero_grad()
+    if kind == "batch":                                            # eval mode: running statistics, no batch terms
+        mine.eval(); ref.eval()
+        xm = x.to(DEV).requires_grad_(True); xr = x.double().requires_grad_(True)
+        ym, yr = mine(xm, relu=relu), ref(xr)
+        if relu:
+            yr = torch.relu(yr)
+        ym.backward(go.to(DEV)); yr.backward(go.double())
+        close(ym, yr); close(xm.grad, xr.grad); close(mine.weight.grad, ref.weight.grad, 2e-5)
+
+
+@pytest.mark.gpu
+def test_particle_norm_bf16_and_repeatability():
+    mine, ref = _norm_pair("group", 8, 4, torch.bfloat16, 3)
+    x = (torch.randn(2, 8, 2050) * 2 + 1).to(torch.bfloat16)
+    go = torch.randn(2, 8, 2050).to(torch.bfloat16)
+    xm = x.to(DEV).requires_grad_(True); xr = x.double().requires_grad_(True)
+    ym = mine(xm, relu=True); yr = torch.relu(ref(xr))
+    ym.backward(go.to(DEV)); yr.backward(go.double())
+    assert ym.dtype == torch.bfloat16 and xm.grad.dtype == torch.bfloat16
+    assert (ym.double().cpu() - yr).abs().max() <= 2e-2 * yr.abs().max()
+    assert (xm.grad.double().cpu() - xr.grad).abs().max() <= 2e-2 * xr.grad.abs().max()
+    # fixed summation order: bit-identical on repetition
+    x32 = torch.randn(1, 4, 100003, device=DEV)
+    a = _ops.row_moments(x32); b = _ops.row_moments(x32)
+    assert torch.equal(a[0], b[0]) and torch.equal(a[1], b[1])
+    # closed forms: a constant row has m2 = 0 and mean = the constant; a ramp 0..n-1 has mean (n-1)/2, m2 = n(n^2-1)/12
+    n = 4097
+    rows = torch.stack([torch.full((n,), 3.25), torch.arange(n, dtype=torch.float32)]).unsqueeze(0).to(DEV).contiguous()
+    mean, m2 = _ops.row_moments(rows)
+    assert mean[0, 0].item() == 3.25 and m2[0, 0].item() == 0.0
+    assert abs(mean[0, 1].item() - (n - 1) / 2) < 1e-6 * n and abs(m2[0, 1].item() / (n * (n * n - 1) / 12) - 1) < 1e-6
+    with pytest.raises(ValueError):
+        _ops.norm_apply(x32, torch.zeros(3, device=DEV), torch.zeros(4, device=DEV), torch.zeros(4, device=DEV), False)
