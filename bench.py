@@ -227,7 +227,7 @@ def main():
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU; --gpus N with N > 1 is not supported "
-                 "(the path shards by batch item or by z-slabs, see DESIGN.md)")
+                 "(the path would shard by batch item, or by z-slabs with a one-row halo per level)")
 
     import torch
     from pyapr import aprnet, _native
