@@ -137,21 +137,22 @@ bool try_conv111_mfma<float>(const float* src, int64_t lds, int Csrc, const floa
 template <typename T>
 __global__ void __launch_bounds__(TB1)
 conv111_dw_kernel(const T* __restrict__ x, int64_t ldx, int Cin, const T* __restrict__ gy, int64_t ldy, int Cout,
-                  T* __restrict__ gw, int64_t begin, int64_t end) {
+                  typename Num<T>::acc* __restrict__ gw, int64_t begin, int64_t end) {
+    typedef typename Num<T>::acc A;          // bfloat16 features: fp32 products, sums and weight gradient
     constexpr int B = 8;
-    __shared__ T red[TB1 / 64][B * B];
+    __shared__ A red[TB1 / 64][B * B];
     const int co0 = blockIdx.y * B, ci0 = blockIdx.z * B;
-    T acc[B][B];
+    A acc[B][B];
 #pragma unroll
     for (int a = 0; a < B; ++a)
 #pragma unroll
         for (int b = 0; b < B; ++b) acc[a][b] = 0;
     for (int64_t i = begin + (int64_t)blockIdx.x * TB1 + threadIdx.x; i < end; i += (int64_t)gridDim.x * TB1) {
-        T g[B], v[B];
+        A g[B], v[B];
 #pragma unroll
-        for (int a = 0; a < B; ++a) g[a] = co0 + a < Cout ? gy[(int64_t)(co0 + a) * ldy + i] : (T)0;
+        for (int a = 0; a < B; ++a) g[a] = co0 + a < Cout ? Num<T>::ld(gy[(int64_t)(co0 + a) * ldy + i]) : (A)0;
 #pragma unroll
-        for (int b = 0; b < B; ++b) v[b] = ci0 + b < Cin ? x[(int64_t)(ci0 + b) * ldx + i] : (T)0;
+        for (int b = 0; b < B; ++b) v[b] = ci0 + b < Cin ? Num<T>::ld(x[(int64_t)(ci0 + b) * ldx + i]) : (A)0;
 #pragma unroll
         for (int a = 0; a < B; ++a)
 #pragma unroll
@@ -162,14 +163,14 @@ conv111_dw_kernel(const T* __restrict__ x, int64_t ldx, int Cin, const T* __rest
     for (int a = 0; a < B; ++a)
 #pragma unroll
         for (int b = 0; b < B; ++b) {
-            T s = acc[a][b];
+            A s = acc[a][b];
 #pragma unroll
             for (int off = 32; off > 0; off >>= 1) s += __shfl_down(s, off);
             if (lane == 0) red[wave][a * B + b] = s;
         }
     __syncthreads();
     if (threadIdx.x < B * B) {
-        T s = 0;
+        A s = 0;
 #pragma unroll
         for (int wv = 0; wv < TB1 / 64; ++wv) s += red[wv][threadIdx.x];
         const int a = threadIdx.x / B, b = threadIdx.x % B;
@@ -253,6 +254,26 @@ int conv111_fwd_bf16(const aprnet_plan* p, int d, const bf16_t* x, int64_t ldx, 
     return 0;
 }
 
+// bfloat16 features and output gradient, fp32 weights and weight gradient (accumulated into gw), fp32 accumulation
+int conv111_bwd_bf16(const aprnet_plan* p, int d, const bf16_t* x, int64_t ldx, int Cin, const float* w, int S, int Cout,
+                     const bf16_t* gy, int64_t ldy, bf16_t* gx, int64_t ldgx, float* gw, hipStream_t st) {
+    if (int rc = check_level_delta(p, d, "conv111_backward")) return rc;
+    if (Cin <= 0 || Cout <= 0 || S <= 0) return fail(APRNET_ERR_INVALID_ARGUMENT, "conv111_backward: empty channel / stencil count");
+    APRNET_HIP_CHECK(hipSetDevice(p->device));
+    for (const Segment& sg : segments(p, d, S)) {
+        const float* ws = w + (int64_t)sg.stencil * Cout * Cin;
+        // grad_x[ci][i] = sum_co w[co][ci] * gy[co][i]: the forward kernel with the weight strides swapped
+        if (!launch_conv111_mfma<bf16_t>(gy, ldy, Cout, ws, 1, Cin, nullptr, gx, ldgx, Cin, sg.begin, sg.end, st))
+            return fail(APRNET_ERR_UNSUPPORTED, "conv111_backward: bfloat16 features support at most 128 output channels");
+        const int64_t n = sg.end - sg.begin;
+        dim3 g2((unsigned)std::min<int64_t>((n + TB1 * 8 - 1) / (TB1 * 8), 256), (unsigned)((Cout + 7) / 8), (unsigned)((Cin + 7) / 8));
+        hipLaunchKernelGGL(conv111_dw_kernel<bf16_t>, g2, dim3(TB1), 0, st, x, ldx, Cin, gy, ldy, Cout,
+                           gw + (int64_t)sg.stencil * Cout * Cin, sg.begin, sg.end);
+    }
+    APRNET_LAUNCH_CHECK("conv111 backward kernels");
+    return 0;
+}
+
 // 1x1x1 forward with the optional clamp at zero, for the fused entry points
 int conv111_fwd_relu(const aprnet_plan* p, int d, const float* x, int64_t ldx, int Cin, const float* w, int S, int Cout,
                      const float* bias, float* y, int64_t ldy, hipStream_t st, int relu) {
@@ -271,6 +292,10 @@ int conv111_fwd_relu(const aprnet_plan* p, int d, const bf16_t* x, int64_t ldx, 
 
 using namespace aprnet;
 extern "C" {
+int aprnet_conv111_bwd_bf16(const aprnet_plan* p, int d, const uint16_t* x, int64_t ldx, int Cin, const float* w, int S, int Cout,
+                            const uint16_t* gy, int64_t ldy, uint16_t* gx, int64_t ldgx, float* gw, void* st) {
+    return conv111_bwd_bf16(p, d, (const bf16_t*)x, ldx, Cin, w, S, Cout, (const bf16_t*)gy, ldy, (bf16_t*)gx, ldgx, gw, (hipStream_t)st);
+}
 int aprnet_conv111_fwd_bf16(const aprnet_plan* p, int d, const uint16_t* x, int64_t ldx, int Cin, const float* w, int S,
                             int Cout, const float* bias, uint16_t* y, int64_t ldy, void* st) {
     return conv111_fwd_bf16(p, d, (const bf16_t*)x, ldx, Cin, w, S, Cout, bias, (bf16_t*)y, ldy, (hipStream_t)st, 0);

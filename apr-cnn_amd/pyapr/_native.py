@@ -115,6 +115,7 @@ def hip():
         getattr(lib, f"aprnet_conv_fwd_fused_{t}").argtypes = [vp, i32, i32, i32, i32, vp, i64, i32, vp, i32, i32, vp, vp, i64,
                                                                 vp, i64, vp, vp]
     lib.aprnet_conv111_fwd_bf16.argtypes = [vp, i32, vp, i64, i32, vp, i32, i32, vp, vp, i64, vp]
+    lib.aprnet_conv111_bwd_bf16.argtypes = [vp, i32, vp, i64, i32, vp, i32, i32, vp, i64, vp, i64, vp, vp]
     lib.aprnet_fill_tree_mean_bf16.argtypes = [vp, i32, vp, i64, i32, vp, i64, vp]
     lib.aprnet_fill_tree_mean_bwd_bf16.argtypes = [vp, i32, vp, i64, i32, vp, i64, vp]
     lib.aprnet_maxpool_fwd_bf16.argtypes = [vp, i32, vp, i64, i32, vp, i64, vp, i64, vp]

@@ -325,10 +325,19 @@ def conv_backward(aprs, x, weights, grad_output, level_delta, need_input_grad=Tr
     plans = _plans(aprs, x.device)
     if x.dtype == torch.bfloat16:
         # bfloat16 features and output gradient; weights and their gradient in fp32, fp32 accumulation
-        if (kz, kx, ky) == (1, 1, 1) or grad_output.dtype != torch.bfloat16:
-            raise TypeError("bfloat16 backward exists for the stencil convolutions with a bfloat16 output gradient")
+        if grad_output.dtype != torch.bfloat16:
+            raise TypeError("bfloat16 features need a bfloat16 output gradient")
         weights = weights.float()
         gw = torch.zeros_like(weights)
+        if (kz, kx, ky) == (1, 1, 1):
+            with torch.cuda.device(x.device):
+                st = _stream()
+                for b in range(B):
+                    rc = _lib().aprnet_conv111_bwd_bf16(plans[b], d[b], _ptr(x[b]), N, cin, _ptr(weights), s_exp, cout,
+                                                        _ptr(grad_output[b]), grad_output.size(2), _ptr(gx[b]), N, _ptr(gw), st)
+                    if rc:
+                        _raise(rc, "conv111_backward failed")
+            return [gx, gw]
         ld_tree = max(max(tree_parts(a, d[b]) for b, a in enumerate(aprs)), 1)
         tree_ws = torch.empty((cin, ld_tree), dtype=x.dtype, device=x.device)
         gtree_ws = None if skip_gx else torch.empty((cin, ld_tree), dtype=torch.float32, device=x.device)

@@ -192,6 +192,11 @@ int aprnet_conv_fwd_fused_bf16(const aprnet_plan*, int level_delta, int kz, int 
                                uint16_t* tree_ws, int64_t ld_tree, const aprnet_conv_fusion* fusion, void* stream);
 int aprnet_conv111_fwd_bf16(const aprnet_plan*, int level_delta, const uint16_t* x, int64_t ldx, int Cin, const float* w,
                             int S, int Cout, const float* bias, uint16_t* y, int64_t ldy, void* stream);
+/* Convolution<1,1,1>::backward with bfloat16 features and output gradient: fp32 weights, fp32 weight gradient
+ * (accumulated into gw), fp32 accumulation; gx overwritten.  At most 128 output channels. */
+int aprnet_conv111_bwd_bf16(const aprnet_plan*, int level_delta, const uint16_t* x, int64_t ldx, int Cin, const float* w,
+                            int S, int Cout, const uint16_t* gy, int64_t ldy, uint16_t* gx, int64_t ldgx, float* gw,
+                            void* stream);
 int aprnet_fill_tree_mean_bf16(const aprnet_plan*, int level_delta, const uint16_t* x, int64_t ldx, int C, uint16_t* tree,
                                int64_t ld_tree, void* stream);
 int aprnet_fill_tree_mean_bwd_bf16(const aprnet_plan*, int level_delta, uint16_t* gx, int64_t ldx, int C, uint16_t* gtree,

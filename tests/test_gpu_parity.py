@@ -484,11 +484,21 @@ def test_conv_backward_bf16(bt, ksize, math):
     assert float((gwc - gw_ref).abs().max()) <= 1e-2 * float(gw_ref.abs().max())
 
 
-def test_conv111_backward_bf16_is_refused():
-    x, aprs, ld, w = _conv_case([("3d_a", 0)], (1, 1, 1), 1, 2, 2, torch.float32)
-    wd = w.permute(1, 2, 0, 3, 4, 5).contiguous().to(DEV)
+@pytest.mark.parametrize("cin,cout,S", [(20, 9, 3), (3, 40, 1), (64, 3, 2)])
+def test_conv111_backward_bf16(cin, cout, S):
+    """1x1x1 backward with bfloat16 features and output gradient: fp32 weights, weight gradient and accumulation;
+    against the fp32 oracle on the same (bfloat16-representable) inputs."""
+    x, aprs, ld, w = _conv_case([("3d_b", 1), ("3d_c", 0)], (1, 1, 1), S, cin, cout, torch.float32)
+    xb = x.to(torch.bfloat16)
+    g = torch.Generator().manual_seed(13)
+    gob = torch.randn(x.size(0), cout, x.size(2), generator=g).to(torch.bfloat16)
+    gx_ref, gw_ref = oracle.conv_backward(aprs, xb.float(), w, gob.float(), ld)
+    gx, gw = _ops.conv_backward(aprs, xb.to(DEV), w.permute(1, 2, 0, 3, 4, 5).contiguous().to(DEV), gob.to(DEV), ld)
+    close_bf16(gx, gx_ref)
+    assert gw.dtype == torch.float32
+    close(gw.permute(2, 0, 1, 3, 4, 5), gw_ref, torch.float32)        # fp32 products of exact inputs, fp32 sums
     with pytest.raises(TypeError):
-        _ops.conv_backward(aprs, x.to(torch.bfloat16).to(DEV), wd, x.to(torch.bfloat16).to(DEV), ld)
+        _ops.conv_backward(aprs, xb.to(DEV), w.permute(1, 2, 0, 3, 4, 5).contiguous().to(DEV), gob.float().to(DEV), ld)
 
 
 # ------------------------------------------------------------------------- fused forward (ReLU, second input)
