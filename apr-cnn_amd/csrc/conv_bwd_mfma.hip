@@ -22,6 +22,7 @@
 namespace aprnet {
 
 typedef float floatx16 __attribute__((ext_vector_type(16)));
+int bf16_math();       // conv.hip: bfloat16 features multiply on the bfloat16 matrix instructions (default) or in fp32
 
 // row strides that put the tap offsets of one B read into different banks: 67 for 3-wide, 69 for 5-wide rows
 using W333M = ConvGeom<3, 3, 3, 2, 4, 512, 67>;
@@ -106,6 +107,158 @@ __device__ __forceinline__ void dw_window(const ConvArgs<T>& a, const Lists& sh,
             }
         }
         __syncthreads();            // gyl is rewritten by the next group, the patch by the next window
+    }
+}
+
+// ---------------------------------------------------------------------------------------------------------
+// bfloat16 features and output gradient: the same contraction on v_mfma_f32_32x32x16_bf16 (16 columns per
+// instruction, fp32 accumulation).  Both operands are bfloat16 values as loaded, so the products are the exact
+// ones the fp32 kernel forms; only the order of the fp32 sums differs.
+//     A: lane l supplies gY[co = l%32] of columns 8*(l/32) .. +7 of a group of 16: one 16-byte read from
+//        gyl16[co][column] (rows DW_LDG16 apart)
+//     B: lane l supplies patch16[ci][cell(column) + off(t = l%32)] of the same 8 columns: 8 two-byte reads
+// An instruction does the work of eight of the fp32 ones, so the loop is bound by its LDS reads.
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+constexpr int DW_LDG16 = DW_GB + 8;            // 16-byte aligned rows, 4 banks apart
+
+template <class G, int CIB, int NCH, bool LISTS, class Lists>
+__device__ __forceinline__ void dw_window_bf16(const ConvArgs<bf16_t>& a, const Lists& sh, int nc, int nitem, bool tree_items,
+                                               int cig0, int co0, int bl, int kh, int hi, int wave, int lane,
+                                               unsigned short* __restrict__ patch, unsigned short* __restrict__ gyl,
+                                               int* __restrict__ cpl, floatx16 (&acc)[NCH]) {
+    for (int i = threadIdx.x; i < CIB * G::CH_STRIDE / 2; i += G::NT) reinterpret_cast<unsigned*>(patch)[i] = 0u;   // once per window
+    ItemRegs<G, bf16_t, CIB> R;
+    fetch_slots<G, bf16_t, CIB>(sh, nitem, R);
+    if constexpr (LISTS) {
+#pragma unroll
+        for (int k = 0; k < ItemRegs<G, bf16_t, CIB>::IPT; ++k)
+            if (R.pos[k] != 0xffffu) R.pos[k] = (unsigned short)restride<G>(R.pos[k]);
+    }
+    load_values<G, bf16_t, CIB>(a, cig0, nitem, tree_items, R);
+    for (int g0 = 0; g0 < nc; g0 += DW_GB) {
+        const int ng = min(DW_GB, nc - g0), nbatch = (ng + 63) >> 6;
+        for (int b = 0; b < nbatch; ++b) {
+            const int c = b * 64 + lane;
+            const int64_t idx = c < ng ? sh.col_idx[g0 + c] : -1;
+            if (wave == 0) {
+                int pb = G::TAP0;
+                if (c < ng) pb = LISTS ? (int)restride<G>(sh.col_pos[g0 + c]) : (int)sh.col_pos[g0 + c];
+                cpl[c] = pb;
+            }
+#pragma unroll
+            for (int k = 0; k < 32 / G::NWAVE; ++k) {
+                const int co = wave + k * G::NWAVE;
+                unsigned short v = 0;
+                if (idx >= 0 && co0 + co < a.Cout) v = a.gy[(int64_t)(co0 + co) * a.ldy + idx].bits;
+                gyl[co * DW_LDG16 + c] = v;
+            }
+        }
+#pragma unroll
+        for (int q = 0; q < NCH; ++q) {
+            __syncthreads();        // previous chunk's reads of the patch are done / gyl is written
+#pragma unroll
+            for (int k = 0; k < ItemRegs<G, bf16_t, CIB>::IPT; ++k) {
+                if (k * G::NT >= nitem) break;       // wave-uniform
+                if (R.pos[k] == 0xffffu) continue;
+                unsigned short* cell = patch + (R.pos[k] & ITEM_CELL);
+#pragma unroll
+                for (int c = 0; c < CIB; ++c) {
+                    const unsigned short v = (unsigned short)R.v[k][c];
+                    cell[c * G::CH_STRIDE] = v;
+                    if (R.pos[k] & ITEM_PAIR) cell[c * G::CH_STRIDE + 1] = v;
+                }
+            }
+            __syncthreads();
+            if (q + 1 < NCH) load_values<G, bf16_t, CIB>(a, cig0 + (q + 1) * CIB, nitem, tree_items, R);
+            else if (g0 + DW_GB < nc) load_values<G, bf16_t, CIB>(a, cig0, nitem, tree_items, R);     // next group starts over
+#pragma unroll 1
+            for (int b = 0; b < nbatch; ++b) {
+#pragma unroll
+                for (int s = 0; s < 2; ++s) {
+                    const int c0 = b * 64 + 32 * kh + 16 * s;           // first of this instruction's 16 columns
+                    if (c0 >= ng) break;                                // wave-uniform: nothing but padding left
+                    const int4 ca = *reinterpret_cast<const int4*>(cpl + c0 + 8 * hi);
+                    const int4 cb = *reinterpret_cast<const int4*>(cpl + c0 + 8 * hi + 4);
+                    const int cell[8] = {ca.x, ca.y, ca.z, ca.w, cb.x, cb.y, cb.z, cb.w};
+                    unsigned w[4];
+#pragma unroll
+                    for (int j = 0; j < 4; ++j)
+                        w[j] = (unsigned)patch[bl + cell[2 * j]] | ((unsigned)patch[bl + cell[2 * j + 1]] << 16);
+                    const uint4 av = *reinterpret_cast<const uint4*>(gyl + (lane & 31) * DW_LDG16 + c0 + 8 * hi);
+                    const uint4 bv = make_uint4(w[0], w[1], w[2], w[3]);
+                    acc[q] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, av), __builtin_bit_cast(bf16x8, bv),
+                                                                     acc[q], 0, 0, 0);
+                }
+            }
+        }
+        __syncthreads();            // gyl is rewritten by the next group, the patch by the next window
+    }
+}
+
+template <class G, int CIB, int NCH, bool LISTS>
+__global__ void __launch_bounds__(G::NT) __attribute__((amdgpu_waves_per_eu(4, 4)))
+conv_dw_bf16_kernel(const ConvArgs<bf16_t> a, const int s_idx) {
+    static_assert(G::NWAVE == 8 && CIB == 4, "wave w owns input channel w%4 and column half w/4");
+    static_assert(G::CH_STRIDE % 2 == 0 && DW_LDG16 % 8 == 0, "dword fill of the patch, 16-byte rows of gyl");
+    __shared__ __attribute__((aligned(16))) unsigned short patch[CIB * G::CH_STRIDE];
+    __shared__ __attribute__((aligned(16))) unsigned short gyl[32 * DW_LDG16];
+    __shared__ __attribute__((aligned(16))) int cpl[DW_GB];
+
+    const int cig0 = blockIdx.y * (CIB * NCH), co0 = blockIdx.z * 32;
+    const int lane = lane_id();
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int cil = wave & 3, kh = wave >> 2;
+    const int t = lane & 31, hi = lane >> 5;
+    const int tt = t < G::K ? t : 0;
+    const int toff = ((tt / (G::KX * G::KY)) * G::RX + (tt / G::KY) % G::KX) * G::RS + (tt % G::KY);
+    const int bl = cil * G::CH_STRIDE - G::TAP0 + toff;       // B operand: + cell of the column
+
+    floatx16 acc[NCH];
+#pragma unroll
+    for (int q = 0; q < NCH; ++q)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[q][r] = 0.f;
+
+    for (int ti = blockIdx.x; ti < a.n_tiles; ti += gridDim.x) {
+        const ConvTile tile = a.tiles[ti];
+        const int L = tile.level;
+        const bool tree_items = L < a.Lc;
+        if constexpr (LISTS) {
+            const int wb = a.tile_win[ti], we = a.tile_win[ti + 1];
+            for (int w = wb; w < we; ++w) {
+                const int4 hd = a.win[w];
+                const int nitem = __builtin_amdgcn_readfirstlane(hd.y), nc = __builtin_amdgcn_readfirstlane(hd.w);
+                const WindowLists gl{a.l_item_idx + (unsigned)hd.x, a.l_item_pos + (unsigned)hd.x, a.l_col_idx + (unsigned)hd.z,
+                                     a.l_col_pos + (unsigned)hd.z};
+                dw_window_bf16<G, CIB, NCH, true>(a, gl, nc, nitem, tree_items, cig0, co0, bl, kh, hi, wave, lane, patch, gyl, cpl, acc);
+            }
+        } else {
+            __shared__ ConvShared<G> sh;
+            const int yn = a.apr.y_num[L];
+            const bool out_tree = (L == a.Lc) && (L < a.apr.level_max);
+            __syncthreads();
+            open_segments<G, bf16_t>(a, L, tile.z0, tile.x0, sh);
+            __syncthreads();
+            for (int y0 = 0; y0 < yn; y0 += G::TY) {
+                scan_window<G, bf16_t>(a, L, y0, out_tree, sh);
+                __syncthreads();
+                const int nc = __builtin_amdgcn_readfirstlane(sh.ncol), nitem = __builtin_amdgcn_readfirstlane(sh.nitem);
+                if (nc > 0) dw_window_bf16<G, CIB, NCH, false>(a, sh, nc, nitem, tree_items, cig0, co0, bl, kh, hi, wave, lane, patch, gyl, cpl, acc);
+                __syncthreads();
+                close_window<G>(sh);
+                __syncthreads();
+            }
+        }
+    }
+#pragma unroll
+    for (int q = 0; q < NCH; ++q) {
+        const int ci = cig0 + q * CIB + cil;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const int co = co0 + 8 * (r >> 2) + 4 * hi + (r & 3);
+            if (t < G::K && ci < a.Cin && co < a.Cout && acc[q][r] != 0.f)
+                unsafeAtomicAdd(a.gw + (((int64_t)s_idx * a.Cout + co) * a.Cin + ci) * G::K + t, acc[q][r]);
+        }
     }
 }
 
@@ -195,6 +348,17 @@ static int launch_dw(const ConvArgs<T>& a0, const TileList& tl, int level_min, h
         // a narrow input (the first layer of a network) fits one chunk: no staging and products of empty chunks
         const int nch = a.Cin <= DW_CIB ? 1 : DW_NCH;
         dim3 grid((unsigned)std::min(n, 512), (unsigned)((a.Cin + DW_CIB * nch - 1) / (DW_CIB * nch)), (unsigned)((a.Cout + 31) / 32));
+        if constexpr (std::is_same<T, bf16_t>::value) {
+            if (bf16_math()) {      // bfloat16 matrix instructions; the fp32 ones below when those are asked for
+                if (nch == 1) {
+                    if (a.tile_win) hipLaunchKernelGGL((conv_dw_bf16_kernel<G, DW_CIB, 1, true>), grid, dim3(G::NT), 0, st, a, s);
+                    else hipLaunchKernelGGL((conv_dw_bf16_kernel<G, DW_CIB, 1, false>), grid, dim3(G::NT), 0, st, a, s);
+                } else if (a.tile_win) hipLaunchKernelGGL((conv_dw_bf16_kernel<G, DW_CIB, DW_NCH, true>), grid, dim3(G::NT), 0, st, a, s);
+                else hipLaunchKernelGGL((conv_dw_bf16_kernel<G, DW_CIB, DW_NCH, false>), grid, dim3(G::NT), 0, st, a, s);
+                APRNET_LAUNCH_CHECK("conv_dw_bf16_kernel");
+                continue;
+            }
+        }
         if (nch == 1) {
             if (a.tile_win) hipLaunchKernelGGL((conv_dw_mfma_kernel<T, G, DW_CIB, 1, true>), grid, dim3(G::NT), 0, st, a, s);
             else hipLaunchKernelGGL((conv_dw_mfma_kernel<T, G, DW_CIB, 1, false>), grid, dim3(G::NT), 0, st, a, s);

@@ -200,8 +200,8 @@ def other_ops(apr, x, dev):
     go5b = torch.randn_like(y5b)
     ms = _time(lambda: torch.autograd.grad(y5b, (x64b, conv5b.weight), go5b, retain_graph=True), iters=2, warmup=1)
     res.append({"op": "conv155_bwd_bf16", "ms": ms, "particles_per_s": n0 / ms * 1e3,
-                "note": "1x5x5 64->64 backward, bfloat16 features and gradients: input gradient on the bfloat16 matrix cores, "
-                        "weight gradient with fp32 products, fp32 accumulation"})
+                "note": "1x5x5 64->64 backward, bfloat16 features and gradients: input and weight gradient on the bfloat16 "
+                        "matrix cores, fp32 accumulation"})
     del y5b, go5b, x64b, conv5b
     with torch.no_grad():
         xinb = xin.to(torch.bfloat16)

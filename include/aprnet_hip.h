@@ -212,7 +212,8 @@ int aprnet_upsample_fwd_bf16(const aprnet_plan*, int level_delta, const uint16_t
  * space gx32_ws [Cin][ld_gx32] (ld_gx32 >= aprnet_number_parts) and rounded to bfloat16 into gx at the end.
  * gtree_ws: fp32 [Cin][ld_gtree].  The input gradient multiplies on the bfloat16 matrix cores (weights rounded to
  * bfloat16) from input-gradient lists that the plan builds on first use; with aprnet_set_conv_path(3) or (5) it
- * runs with fp32 products and scans per call.  The weight gradient always uses fp32 products.  gx may be NULL:
+ * runs with fp32 products and scans per call.  The weight gradient multiplies on the bfloat16 matrix cores as well
+ * (both operands are bfloat16 as stored, so the products are exact), or with fp32 instructions under path 3.  gx may be NULL:
  * then only gw is computed and gx32_ws / gtree_ws are not used. */
 int aprnet_conv_bwd_bf16(const aprnet_plan*, int level_delta, int kz, int kx, int ky, const uint16_t* x, int64_t ldx, int Cin,
                          const float* w, int S_exp, int Cout, const uint16_t* gy, int64_t ldy, uint16_t* gx, int64_t ldgx,
