@@ -131,6 +131,37 @@ def test_pool_argmax_gathers_and_upsample_round_trip(apr):
     torch.testing.assert_close(gi.double().sum(dim=2), go.double().sum(dim=2), rtol=1e-9, atol=1e-6)
 
 
+@pytest.mark.parametrize("kind", ["batch", "group"])
+def test_particle_norm_at_full_size(apr, kind):
+    """The streaming norm kernels on 16 x 23 M elements: the normalised rows have mean 0 and variance 1 in float64,
+    outputs and input gradients agree with torch's own GPU modules (a different implementation and summation order)
+    to 1e-5 / 1e-4 of the tensors' scale, and the input gradient is orthogonal to the constant and to the normalised
+    input, as the derivative of a normalisation must be."""
+    from apr_models.unet.particle_norm import ParticleBatchNorm, ParticleGroupNorm
+    n, c = apr.total_number_particles(), 16
+    g = torch.Generator().manual_seed(4)
+    x = (torch.randn(1, c, n, generator=g) * 2.5 + 7.0).to(DEV).requires_grad_(True)
+    go = torch.randn(1, c, n, generator=g).to(DEV)
+    if kind == "batch":
+        mine, ref = ParticleBatchNorm(c).to(DEV), torch.nn.BatchNorm1d(c).to(DEV)
+    else:
+        mine, ref = ParticleGroupNorm(c, c).to(DEV), torch.nn.GroupNorm(c, c).to(DEV)
+    y = mine(x)
+    yd = y.detach().double()
+    assert float(yd.mean(dim=2).abs().max()) < 1e-5 and float((yd.var(dim=2, unbiased=False) - 1).abs().max()) < 1e-4
+    y.backward(go)
+    gx = x.grad.detach().clone()
+    x.grad = None
+    yr = ref(x)
+    yr.backward(go)
+    assert float((y.detach() - yr.detach()).abs().max()) <= 1e-5 * float(yr.detach().abs().max())
+    assert float((gx - x.grad).abs().max()) <= 1e-4 * float(x.grad.abs().max())
+    gxd = gx.double()
+    scale = float(gxd.abs().sum(dim=2).max())
+    assert float(gxd.sum(dim=2).abs().max()) <= 1e-5 * scale
+    assert float((gxd * yd).sum(dim=2).abs().max()) <= 1e-5 * scale * float(yd.abs().max())
+
+
 def test_centre_crop_against_oracle():
     """The benchmark's CPU-baseline sample (128x256x256 crop, 3 M particles) through both implementations."""
     apr = build_workload("blobs512", crop=(128, 256, 256))
