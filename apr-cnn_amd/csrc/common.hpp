@@ -97,6 +97,8 @@ struct aprnet_plan {
     std::map<std::tuple<int, int, int, int>, aprnet::TileList> tiles;   // (level_delta, TZ, TX, halo) -> row groups
     void* d_scratch = nullptr; size_t scratch_bytes = 0;          // re-laid-out weights of the call in flight
     std::map<std::pair<int, int>, aprnet::WinLists> lists;        // (level_delta, stencil code) -> window lists
+    // second stream of the convolution backward (weight gradient next to input gradient), with its fork / join events
+    hipStream_t side = nullptr; hipEvent_t ev_fork = nullptr, ev_join = nullptr;
 
     int lc(int level_delta) const { return apr.level_max - level_delta; }
     int64_t number_parts(int level_delta) const {

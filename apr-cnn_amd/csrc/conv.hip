@@ -148,6 +148,8 @@ int bf16_math();
 
 static int g_use_lists = 1;      // 1: forward kernels take the window lists of the plan, 0: they scan per call
 int bf16_math() { return g_bf16_math; }
+static int g_bwd_overlap = 1;    // backward: weight gradient on a second stream next to the input gradient
+int backward_overlap() { return g_bwd_overlap; }
 
 // Points the kernel at the plan's window lists.  When the lists are switched off, or cannot be built (no device
 // memory for them, too many entries), a.tile_win stays null and the kernel scans the access arrays itself.
@@ -331,6 +333,7 @@ int aprnet_conv_fwd_fused_f64(const aprnet_plan* p, int d, int kz, int kx, int k
 int aprnet_set_conv_path(int path) {
     if (path == 2 || path == 3) { g_bf16_math = path == 2; return 0; }
     if (path == 4 || path == 5) { g_use_lists = path == 4; return 0; }
+    if (path == 6 || path == 7) { g_bwd_overlap = path == 6; return 0; }
     if (path != 0 && path != 1)
         return fail(APRNET_ERR_INVALID_ARGUMENT, "set_conv_path: 0 (auto), 1 (VALU only), 2 / 3 (bfloat16 features: bfloat16 / fp32 "
                                                  "matrix math), 4 / 5 (forward: window lists of the plan / scan per call)");

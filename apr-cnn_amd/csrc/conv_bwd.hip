@@ -247,12 +247,20 @@ int pack_conv_weights_bf16(int code, const float* w, int S_exp, int Cout, int Ci
 int bf16_math();
 
 template <typename T> static int try_mfma_bwd(aprnet_plan*, const ConvArgs<T>&, const TileList&, int, int, hipStream_t, bool*) { return 0; }
+static int fork_side(aprnet_plan* p, hipStream_t st, hipStream_t* side);
+static int join_side(aprnet_plan* p, hipStream_t st, hipStream_t side);
 template <> int try_mfma_bwd<float>(aprnet_plan* p, const ConvArgs<float>& a, const TileList& tl, int code, int d, hipStream_t st, bool* done) {
     if (conv_path() == 1 || !conv_mfma_supported(code)) return 0;
     *done = true;
-    // input gradient: the forward kernel on the output gradient with the transposed, flipped stencil;
-    // every row group within one row of an output takes part
+    // weight gradient on the side stream (when there is an input gradient to run next to)
+    ConvArgs<float> c = a;
+    if (int rc = set_conv_lists(p, d, code, tl, c, st)) return rc;
+    hipStream_t side = st;
+    if (a.gx) if (int rc = fork_side(p, st, &side)) return rc;
+    if (int rc = launch_conv_dw_mfma(code, c, tl, p->apr.level_min, side)) return rc;
     if (a.gx) {
+        // input gradient: the forward kernel on the output gradient with the transposed, flipped stencil;
+        // every row group within one row of an output takes part
         TileList near;
         if (int rc = get_tiles(p, d, code == 333 ? 2 : 1, code == 333 ? 4 : 8, &near, 1)) return rc;
         if (int rc = plan_scratch(p, conv_packed_floats(code, a.S_exp, a.Cin, a.Cout, true) * sizeof(float), st)) return rc;
@@ -263,9 +271,32 @@ template <> int try_mfma_bwd<float>(aprnet_plan* p, const ConvArgs<float>& a, co
         b.tree_data = nullptr; b.t_count = 0;
         if (near.n > 0) if (int rc = launch_conv_dx_mfma(code, b, near.n, st)) return rc;
     }
-    ConvArgs<float> c = a;
-    if (int rc = set_conv_lists(p, d, code, tl, c, st)) return rc;
-    return launch_conv_dw_mfma(code, c, tl, p->apr.level_min, st);
+    return join_side(p, st, side);
+}
+
+// Fork / join around the two halves of the backward pass: what follows fork() on the returned stream runs next to
+// the caller's stream `st` until join().  Both kernels are bound by their matrix phases and the barriers between
+// them at about half of the matrix peak, and read the same output gradient; side by side they fill each other's
+// gaps.  Default priority, event based, so a caller may capture it into a graph.
+int backward_overlap();
+static int fork_side(aprnet_plan* p, hipStream_t st, hipStream_t* side) {
+    *side = st;
+    if (!backward_overlap()) return 0;
+    if (!p->side) {
+        APRNET_HIP_CHECK(hipStreamCreateWithFlags(&p->side, hipStreamNonBlocking));
+        APRNET_HIP_CHECK(hipEventCreateWithFlags(&p->ev_fork, hipEventDisableTiming));
+        APRNET_HIP_CHECK(hipEventCreateWithFlags(&p->ev_join, hipEventDisableTiming));
+    }
+    APRNET_HIP_CHECK(hipEventRecord(p->ev_fork, st));
+    APRNET_HIP_CHECK(hipStreamWaitEvent(p->side, p->ev_fork, 0));
+    *side = p->side;
+    return 0;
+}
+static int join_side(aprnet_plan* p, hipStream_t st, hipStream_t side) {
+    if (side == st) return 0;
+    APRNET_HIP_CHECK(hipEventRecord(p->ev_join, side));
+    APRNET_HIP_CHECK(hipStreamWaitEvent(st, p->ev_join, 0));
+    return 0;
 }
 
 template <typename T>
@@ -360,6 +391,11 @@ int conv_bwd_bf16(const aprnet_plan* cp, int d, int kz, int kx, int ky, const bf
         // input gradient: bfloat16 products on the input-gradient lists of the plan when they are there, otherwise
         // (lists off or not buildable, fp32 products asked for) the scanning kernel with fp32 products
         if (!gx) near.n = 0;              // no input gradient asked for
+        // weight gradient on the side stream, next to the input gradient
+        if (int rc = set_conv_lists(p, d, code, tl, a, st)) return rc;
+        hipStream_t side = st;
+        if (near.n > 0) if (int rc = fork_side(p, st, &side)) return rc;
+        if (int rc = launch_conv_dw_mfma(code, a, tl, p->apr.level_min, side)) return rc;
         if (near.n > 0 && bf16_math())
             if (int rc = set_conv_dx_lists(p, d, code, near, b, st)) return rc;
         if (near.n > 0 && b.tile_win) {
@@ -374,8 +410,7 @@ int conv_bwd_bf16(const aprnet_plan* cp, int d, int kz, int kx, int ky, const bf
             b.tile_win = nullptr;
             if (int rc = launch_conv_dx_mfma(code, b, near.n, st)) return rc;
         }
-        if (int rc = set_conv_lists(p, d, code, tl, a, st)) return rc;
-        if (int rc = launch_conv_dw_mfma(code, a, tl, p->apr.level_min, st)) return rc;
+        if (int rc = join_side(p, st, side)) return rc;
     }
     if (!gx) return 0;
     if (int rc = fill_tree_bwd_for_conv(p, d, gx32_ws, ldgx32, Cin, gtree_ws, ldgt, st)) return rc;

@@ -202,6 +202,9 @@ void aprnet_plan_destroy(aprnet_plan* p) {
     for (auto& kv : p->tiles) if (kv.second.d_tiles) (void)hipFree(kv.second.d_tiles);
     if (p->d_scratch) (void)hipFree(p->d_scratch);
     for (auto& kv : p->lists) free_lists(kv.second);
+    if (p->side) { (void)hipStreamSynchronize(p->side); (void)hipStreamDestroy(p->side); }
+    if (p->ev_fork) (void)hipEventDestroy(p->ev_fork);
+    if (p->ev_join) (void)hipEventDestroy(p->ev_join);
     delete p;
 }
 

@@ -82,8 +82,10 @@ int aprnet_profile_enable(int on);
  * Independently, for bfloat16 features: 2 = bfloat16 matrix instructions (default), 3 = fp32 matrix
  * instructions; and for the forward matrix-core kernels: 4 = take the window lists that the plan builds on first
  * use and keeps (about 20 bytes of device memory per particle and level delta; default), 5 = scan the access arrays
- * in every call (also the fallback when the lists cannot be allocated).  All are HIP kernels; the switch exists so
- * that tests can cover them and memory-bound callers can do without the lists. */
+ * in every call (also the fallback when the lists cannot be allocated); and for the backward matrix-core kernels:
+ * 6 = the weight gradient runs on a second stream of the plan next to the input gradient, forked from and joined
+ * to the caller's stream with events (default), 7 = both on the caller's stream.  All are HIP kernels; the switch
+ * exists so that tests can cover them and memory-bound callers can do without the lists. */
 int aprnet_set_conv_path(int path);
 float aprnet_profile_last_ms(void);
 

@@ -243,6 +243,33 @@ def test_conv333_backward_channel_shapes(cin, cout, path):
     close(gw.permute(2, 0, 1, 3, 4, 5), gw_ref, torch.float32)
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
+def test_conv_backward_on_one_stream(dtype):
+    """The backward pass with the weight gradient on the caller's stream (path 7) instead of the plan's second stream
+    (default): same gradients, and the switch is accepted both ways."""
+    cin, cout = 20, 33
+    x, aprs, ld, w_exp = _conv_case([("3d_s", 0), ("3d_t", 1)], (3, 3, 3), 2, cin, cout, torch.float32)
+    g = torch.Generator().manual_seed(21)
+    go = torch.randn(x.size(0), cout, x.size(2), generator=g)
+    if dtype == torch.bfloat16:
+        x, go = x.to(dtype).float(), go.to(dtype).float()
+    gx_ref, gw_ref = oracle.conv_backward(aprs, x, w_exp, go, ld)
+    wd = w_exp.permute(1, 2, 0, 3, 4, 5).contiguous().to(DEV)
+    lib = _native.hip()
+    for path in (7, 6):
+        assert lib.aprnet_set_conv_path(path) == 0
+        try:
+            gx, gw = _ops.conv_backward(aprs, x.to(DEV).to(dtype), wd, go.to(DEV).to(dtype), ld)
+        finally:
+            lib.aprnet_set_conv_path(6)
+        if dtype == torch.bfloat16:
+            close_bf16(gx, gx_ref)
+            assert float((gw.permute(2, 0, 1, 3, 4, 5).cpu() - gw_ref).abs().max()) <= 1e-2 * float(gw_ref.abs().max())
+        else:
+            close(gx, gx_ref, dtype)
+            close(gw.permute(2, 0, 1, 3, 4, 5), gw_ref, dtype)
+
+
 @pytest.mark.parametrize("path", [0, 1], ids=["mfma", "valu"])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
 @pytest.mark.parametrize("cin,cout", [(1, 16), (5, 4), (18, 33)])
