@@ -21,9 +21,19 @@ def _cpu_conv(conv, x, aprs, ld):
     return OracleConv.apply(x, w, b, aprs, ld)
 
 
+def _cpu_norm(norm, x):
+    """The block's norm evaluated by torch on the CPU (a CPU copy of the module; nn.Identity when folded away)."""
+    import copy
+    return copy.deepcopy(norm).cpu()(x)
+
+
+def _cpu_basic(bb, x, aprs, ld):
+    return torch.relu(_cpu_norm(bb.norm, _cpu_conv(bb.conv, x, aprs, ld)))
+
+
 def _cpu_block(block, x, aprs, ld):
     for bb in block.blocks:
-        x = torch.relu(_cpu_conv(bb.conv, x, aprs, ld))
+        x = _cpu_basic(bb, x, aprs, ld)
     return x
 
 
@@ -36,7 +46,7 @@ def reference_forward(model, x, aprs):
         skips.append(_cpu_block(stage.conv, y, aprs, ld))
     y = skips[-1]
     for i, stage in enumerate(model.decoder):
-        y = torch.relu(_cpu_conv(stage.reduce_ch.conv, y, aprs, ld))
+        y = _cpu_basic(stage.reduce_ch, y, aprs, ld)
         y = OracleUpSample.apply(y, aprs, ld)
         ld -= 1
         y = _cpu_block(stage.conv, torch.cat([skips[-(i + 2)], y], dim=1), aprs, ld)
@@ -63,6 +73,32 @@ def test_unet_forward_matches_oracle(shape, seed):
     assert got.shape == ref.shape == (1, 3, n)
     err = float((got.cpu() - ref).abs().max()) / float(ref.abs().max())
     assert err < 2e-5, f"rel err {err:.2e}"      # 18 fp32 layers deep; single ops agree to 1e-5
+
+
+@pytest.mark.parametrize("norm,train", [("group", False), ("batch", True), ("batch", False)])
+def test_unet_forward_with_norm_layers_matches_oracle(norm, train):
+    """The network as the reference builds it (GroupNorm with one group per channel by default, or BatchNorm1d in
+    training / eval mode, nothing folded) on a batch of two APRs of different sizes: convolutions, norms over the padded
+    particle axis, pool and upsample on the GPU against the same composition on the CPU (oracle operators, torch norms)."""
+    aprs = [apr_cases.random_apr((24, 40, 36), 5, density=0.05), apr_cases.random_apr((20, 33, 28), 6, density=0.04)]
+    n = max(a.total_number_particles() for a in aprs)
+    torch.manual_seed(3)
+    model = APRUNet(1, 2, depth=2, n_filters_base=8, n_stencils=2, norm=norm)
+    with torch.no_grad():
+        for m in model.modules():
+            if isinstance(m, (torch.nn.BatchNorm1d, torch.nn.GroupNorm)):
+                m.weight.uniform_(0.5, 1.5); m.bias.uniform_(-0.5, 0.5)
+            if isinstance(m, torch.nn.BatchNorm1d):
+                m.running_mean.uniform_(-0.2, 0.2); m.running_var.uniform_(0.5, 2.0)
+    model.train(train)
+    x = torch.randn(2, 1, n)
+    for b, a in enumerate(aprs):
+        x[b, :, a.total_number_particles():] = 0
+    with torch.no_grad():
+        ref = reference_forward(model, x, aprs)
+        got = model.to(DEV)(x.to(DEV), aprs)
+    err = float((got.cpu() - ref).abs().max()) / float(ref.abs().max())
+    assert err < 2e-5, f"rel err {err:.2e}"
 
 
 def test_fold_norms_equals_eval_batchnorm():
