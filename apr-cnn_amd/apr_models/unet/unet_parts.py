@@ -37,9 +37,12 @@ class BasicBlock(nn.Module):
         if (not torch.is_grad_enabled() and isinstance(self.norm, nn.Identity) and type(self.activation) is nn.ReLU
                 and x.is_cuda):
             return self.conv.forward_fused(x, aprs, level_deltas, relu=True, second_input=x2)
-        if x2 is not None:
-            x = torch.cat([x, x2], dim=1)
-        y = self.conv(x, aprs, level_deltas)
+        if x2 is not None and not torch.is_grad_enabled() and x.is_cuda:
+            y = self.conv.forward_fused(x, aprs, level_deltas, relu=False, second_input=x2)      # no concatenated copy
+        else:
+            if x2 is not None:
+                x = torch.cat([x, x2], dim=1)
+            y = self.conv(x, aprs, level_deltas)
         if type(self.activation) is nn.ReLU and isinstance(self.norm, (ParticleBatchNorm, ParticleGroupNorm)):
             return self.norm(y, relu=True)          # one pass for norm + ReLU
         return self.activation(self.norm(y))

@@ -155,6 +155,13 @@ def other_ops(apr, x, dev):
         ms = _time(graph.replay, iters=3, warmup=1)
     res.append({"op": "apr_unet_fwd_graph", "ms": ms, "note": "the fp32 forward replayed from a HIP graph"})
     del graph, y_graph
+    # the reference's default configuration: GroupNorm with one group per channel, which cannot be folded away
+    torch.manual_seed(0)
+    gnet = APRUNet(1, 3, depth=3, n_filters_base=16, n_stencils=2, norm="group").eval().to(dev)
+    with torch.no_grad():
+        ms = _time(lambda: gnet(xin, [apr]), iters=3, warmup=1)
+    res.append({"op": "apr_unet_fwd_groupnorm", "ms": ms, "note": "same architecture with GroupNorm layers (norm + ReLU in one pass of the streaming norm kernels)"})
+    del gnet
     # one training step of the same architecture (unfolded BatchNorm in training mode): forward, loss, backward
     torch.manual_seed(0)
     tnet = APRUNet(1, 3, depth=3, n_filters_base=16, n_stencils=2, norm="batch").to(dev).train()
