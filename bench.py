@@ -129,6 +129,18 @@ def other_ops(apr, x, dev):
         w1 = torch.randn(1, C, C, 1, 1, 1, device=dev) * 0.1
         ms = _time(lambda: _ops.conv_forward([apr], x, w1, ld0))
         line("conv111_fwd", ms, e * 2 * C * n0, f"{C}->{C}")
+    # BatchNorm1d + ReLU over the particle axis in training mode (statistics of the batch), forward and backward
+    from apr_models.unet.particle_norm import ParticleBatchNorm
+    bn = ParticleBatchNorm(C).to(dev).train()
+    with torch.no_grad():
+        ms = _time(lambda: bn(x, relu=True))
+    line("norm_relu_fwd", ms, e * 3 * C * n0, f"C={C}: one pass for the moments, one read + one write to normalise")
+    xn = x.detach().clone().requires_grad_(True)
+    yn = bn(xn, relu=True)
+    gn = torch.randn_like(yn)
+    ms = _time(lambda: torch.autograd.grad(yn, xn, gn, retain_graph=True))
+    line("norm_relu_bwd", ms, e * 7 * C * n0, "gradient, input and output read twice (sums, then result), one write")
+    del xn, yn, gn, bn
     conv = aprnet.cuda.APRConv(C, C, nstencils=2).to(dev)
     xg = x.clone().requires_grad_(True)
     y = conv(xg, [apr], ld0)
