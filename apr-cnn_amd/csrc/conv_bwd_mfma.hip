@@ -111,6 +111,159 @@ __device__ __forceinline__ void dw_window(const ConvArgs<T>& a, const Lists& sh,
 }
 
 // ---------------------------------------------------------------------------------------------------------
+// Layers of at most 16 output channels (the finest stages of the networks): the 32-row instruction above would
+// multiply 16 rows of zeros.  Here D is 16 output channels x 16 taps on v_mfma_f32_16x16x4_f32, two tap tiles per
+// input channel (taps 0-15 and 16-31), four columns per instruction:
+//     A: lane l supplies gY[co = l%16] of column l/16 of the four            (gyl16[column][co], 17 words per column:
+//                                                                              conflict-free writes by column, reads
+//                                                                              with a few two-way conflicts)
+//     B: lane l supplies patch[ci][cell(column l/16) + off(t = l%16 + 16 * tile)]
+// Twice the columns per matrix-pipe cycle of the 32x32x2 form for such layers; same staging, same work split
+// (wave w: input channel w%4 of each chunk, half w/4 of every 64 columns).
+typedef float floatx4d __attribute__((ext_vector_type(4)));
+constexpr int DW_GLD16 = 17;
+
+template <typename T, class G, int CIB, int NCH, bool LISTS, class Lists>
+__device__ __forceinline__ void dw_window16(const ConvArgs<T>& a, const Lists& sh, int nc, int nitem, bool tree_items,
+                                            int cig0, const int (&bl)[2], int kh, int wave, int lane,
+                                            float* __restrict__ patch, float* __restrict__ gyl, int* __restrict__ cpl,
+                                            floatx4d (&acc)[NCH][2]) {
+    for (int i = threadIdx.x; i < CIB * G::CH_STRIDE; i += G::NT) patch[i] = 0.f;     // once per window
+    ItemRegs<G, T, CIB> R;
+    fetch_slots<G, T, CIB>(sh, nitem, R);
+    if constexpr (LISTS) {
+#pragma unroll
+        for (int k = 0; k < ItemRegs<G, T, CIB>::IPT; ++k)
+            if (R.pos[k] != 0xffffu) R.pos[k] = (unsigned short)restride<G>(R.pos[k]);
+    }
+    load_values<G, T, CIB>(a, cig0, nitem, tree_items, R);
+    const int q4 = lane >> 4;                                   // which of the four columns of an instruction
+    const float* ap = gyl + q4 * DW_GLD16 + (lane & 15);
+    for (int g0 = 0; g0 < nc; g0 += DW_GB) {
+        const int ng = min(DW_GB, nc - g0), nbatch = (ng + 63) >> 6;
+        for (int b = 0; b < nbatch; ++b) {
+            const int c = b * 64 + lane;
+            const int64_t idx = c < ng ? sh.col_idx[g0 + c] : -1;
+            if (wave == 0) {
+                int pb = G::TAP0;
+                if (c < ng) pb = LISTS ? (int)restride<G>(sh.col_pos[g0 + c]) : (int)sh.col_pos[g0 + c];
+                cpl[c] = pb;
+            }
+#pragma unroll
+            for (int k = 0; k < 16 / G::NWAVE; ++k) {
+                const int co = wave + k * G::NWAVE;
+                float v = 0.f;
+                if (idx >= 0 && co < a.Cout) v = Num<T>::ld(a.gy[(int64_t)co * a.ldy + idx]);
+                gyl[c * DW_GLD16 + co] = v;
+            }
+        }
+#pragma unroll
+        for (int q = 0; q < NCH; ++q) {
+            __syncthreads();        // previous chunk's reads of the patch are done / gyl is written
+            store_items<G, T, CIB>(R, nitem, patch);
+            __syncthreads();
+            if (q + 1 < NCH) load_values<G, T, CIB>(a, cig0 + (q + 1) * CIB, nitem, tree_items, R);
+            else if (g0 + DW_GB < nc) load_values<G, T, CIB>(a, cig0, nitem, tree_items, R);     // next group starts over
+#pragma unroll 1
+            for (int b = 0; b < nbatch; ++b) {
+                const int c0 = b * 64 + 32 * kh;                 // this wave's 32 columns of the batch
+                if (c0 >= ng) break;                             // wave-uniform: nothing but padding left
+                const int* cp = cpl + c0 + q4;
+                const float* apb = ap + c0 * DW_GLD16;
+                int cell[8];
+#pragma unroll
+                for (int k = 0; k < 8; ++k) cell[k] = cp[4 * k];
+                __builtin_amdgcn_sched_barrier(0);
+                float av[8], b0[8], b1[8];
+#pragma unroll
+                for (int k = 0; k < 8; ++k) { av[k] = apb[4 * k * DW_GLD16]; b0[k] = patch[bl[0] + cell[k]]; b1[k] = patch[bl[1] + cell[k]]; }
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int k = 0; k < 8; ++k) {
+                    acc[q][0] = __builtin_amdgcn_mfma_f32_16x16x4f32(av[k], b0[k], acc[q][0], 0, 0, 0);
+                    acc[q][1] = __builtin_amdgcn_mfma_f32_16x16x4f32(av[k], b1[k], acc[q][1], 0, 0, 0);
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        }
+        __syncthreads();            // gyl is rewritten by the next group, the patch by the next window
+    }
+}
+
+template <typename T, class G, int CIB, int NCH, bool LISTS>
+__global__ void __launch_bounds__(G::NT) __attribute__((amdgpu_waves_per_eu(4, 4)))
+conv_dw16_mfma_kernel(const ConvArgs<T> a, const int s_idx) {
+    static_assert(G::NWAVE == 8 && CIB == 4, "wave w owns input channel w%4 and column half w/4");
+    __shared__ float patch[CIB * G::CH_STRIDE];
+    __shared__ float gyl[DW_GB * DW_GLD16];
+    __shared__ int cpl[DW_GB];
+
+    const int cig0 = blockIdx.y * (CIB * NCH);
+    const int lane = lane_id();
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int cil = wave & 3, kh = wave >> 2;
+    int bl[2];
+#pragma unroll
+    for (int tile = 0; tile < 2; ++tile) {
+        const int t = (lane & 15) + 16 * tile;
+        const int tt = t < G::K ? t : 0;
+        const int toff = ((tt / (G::KX * G::KY)) * G::RX + (tt / G::KY) % G::KX) * G::RS + (tt % G::KY);
+        bl[tile] = cil * G::CH_STRIDE - G::TAP0 + toff;       // B operand: + cell of the column
+    }
+    floatx4d acc[NCH][2];
+#pragma unroll
+    for (int q = 0; q < NCH; ++q)
+#pragma unroll
+        for (int tile = 0; tile < 2; ++tile)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) acc[q][tile][r] = 0.f;
+
+    for (int ti = blockIdx.x; ti < a.n_tiles; ti += gridDim.x) {
+        const ConvTile tile = a.tiles[ti];
+        const int L = tile.level;
+        const bool tree_items = L < a.Lc;
+        if constexpr (LISTS) {
+            const int wb = a.tile_win[ti], we = a.tile_win[ti + 1];
+            for (int w = wb; w < we; ++w) {
+                const int4 hd = a.win[w];
+                const int nitem = __builtin_amdgcn_readfirstlane(hd.y), nc = __builtin_amdgcn_readfirstlane(hd.w);
+                const WindowLists gl{a.l_item_idx + (unsigned)hd.x, a.l_item_pos + (unsigned)hd.x, a.l_col_idx + (unsigned)hd.z,
+                                     a.l_col_pos + (unsigned)hd.z};
+                dw_window16<T, G, CIB, NCH, true>(a, gl, nc, nitem, tree_items, cig0, bl, kh, wave, lane, patch, gyl, cpl, acc);
+            }
+        } else {
+            __shared__ ConvShared<G> sh;
+            const int yn = a.apr.y_num[L];
+            const bool out_tree = (L == a.Lc) && (L < a.apr.level_max);
+            __syncthreads();
+            open_segments<G, T>(a, L, tile.z0, tile.x0, sh);
+            __syncthreads();
+            for (int y0 = 0; y0 < yn; y0 += G::TY) {
+                scan_window<G, T>(a, L, y0, out_tree, sh);
+                __syncthreads();
+                const int nc = __builtin_amdgcn_readfirstlane(sh.ncol), nitem = __builtin_amdgcn_readfirstlane(sh.nitem);
+                if (nc > 0) dw_window16<T, G, CIB, NCH, false>(a, sh, nc, nitem, tree_items, cig0, bl, kh, wave, lane, patch, gyl, cpl, acc);
+                __syncthreads();
+                close_window<G>(sh);
+                __syncthreads();
+            }
+        }
+    }
+#pragma unroll
+    for (int q = 0; q < NCH; ++q) {
+        const int ci = cig0 + q * CIB + cil;
+#pragma unroll
+        for (int tile = 0; tile < 2; ++tile)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int co = 4 * (lane >> 4) + r, t = (lane & 15) + 16 * tile;
+                if (t < G::K && ci < a.Cin && co < a.Cout && acc[q][tile][r] != 0.f)
+                    unsafeAtomicAdd(a.gw + (((int64_t)s_idx * a.Cout + co) * a.Cin + ci) * G::K + t, acc[q][tile][r]);
+            }
+    }
+}
+
+// ---------------------------------------------------------------------------------------------------------
 // bfloat16 features and output gradient: the same contraction on v_mfma_f32_32x32x16_bf16 (16 columns per
 // instruction, fp32 accumulation).  Both operands are bfloat16 values as loaded, so the products are the exact
 // ones the fp32 kernel forms; only the order of the fp32 sums differs.
@@ -358,6 +511,15 @@ static int launch_dw(const ConvArgs<T>& a0, const TileList& tl, int level_min, h
                 APRNET_LAUNCH_CHECK("conv_dw_bf16_kernel");
                 continue;
             }
+        }
+        if (a.Cout <= 16) {         // 16-row form
+            if (nch == 1) {
+                if (a.tile_win) hipLaunchKernelGGL((conv_dw16_mfma_kernel<T, G, DW_CIB, 1, true>), grid, dim3(G::NT), 0, st, a, s);
+                else hipLaunchKernelGGL((conv_dw16_mfma_kernel<T, G, DW_CIB, 1, false>), grid, dim3(G::NT), 0, st, a, s);
+            } else if (a.tile_win) hipLaunchKernelGGL((conv_dw16_mfma_kernel<T, G, DW_CIB, DW_NCH, true>), grid, dim3(G::NT), 0, st, a, s);
+            else hipLaunchKernelGGL((conv_dw16_mfma_kernel<T, G, DW_CIB, DW_NCH, false>), grid, dim3(G::NT), 0, st, a, s);
+            APRNET_LAUNCH_CHECK("conv_dw16_mfma_kernel");
+            continue;
         }
         if (nch == 1) {
             if (a.tile_win) hipLaunchKernelGGL((conv_dw_mfma_kernel<T, G, DW_CIB, 1, true>), grid, dim3(G::NT), 0, st, a, s);
