@@ -270,14 +270,15 @@ def test_conv_backward_on_one_stream(dtype):
             close(gw.permute(2, 0, 1, 3, 4, 5), gw_ref, dtype)
 
 
-@pytest.mark.parametrize("path", [0, 1], ids=["mfma", "valu"])
+@pytest.mark.parametrize("path", [0, 1, 3], ids=["mfma", "valu", "fp32math"])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
 @pytest.mark.parametrize("cin,cout", [(1, 16), (5, 4), (18, 33)])
 def test_conv_backward_weights_only(cin, cout, dtype, path):
     """need_input_grad=False (what autograd asks of the first layer of a network): no input gradient, the same weight
-    gradient; channel counts that leave whole input-channel chunks of the weight-gradient kernel empty."""
-    if dtype == torch.bfloat16 and path == 1:
-        pytest.skip("bfloat16 features run on the matrix-core kernels only")
+    gradient; channel counts that leave whole input-channel chunks of the weight-gradient kernel empty and that take
+    its 16-row and 32-row forms.  bfloat16 features: with bfloat16 and (path 3) with fp32 matrix instructions."""
+    if (dtype == torch.bfloat16 and path == 1) or (dtype == torch.float32 and path == 3):
+        pytest.skip("bfloat16 features run on the matrix-core kernels only; path 3 concerns bfloat16 features")
     x, aprs, ld, w_exp = _conv_case([("3d_s", 0), ("3d_t", 1)], (3, 3, 3), 2, cin, cout, torch.float32)
     g = torch.Generator().manual_seed(9)
     go = torch.randn(x.size(0), cout, x.size(2), generator=g)
@@ -290,7 +291,7 @@ def test_conv_backward_weights_only(cin, cout, dtype, path):
     try:
         gx, gw = _ops.conv_backward(aprs, x.to(DEV).to(dtype), wd, go.to(DEV).to(dtype), ld, need_input_grad=False)
     finally:
-        lib.aprnet_set_conv_path(0)
+        lib.aprnet_set_conv_path(0); lib.aprnet_set_conv_path(2)
     assert gx is None
     if dtype == torch.bfloat16:      # the mean-filled tree values that the sums read are stored in bfloat16
         assert float((gw.permute(2, 0, 1, 3, 4, 5).cpu() - gw_ref).abs().max()) <= 1e-2 * float(gw_ref.abs().max())
