@@ -34,8 +34,8 @@ class ParticleBatchNorm(nn.BatchNorm1d):
         if self.training and self.track_running_stats and self.running_mean is not None:
             n = x.shape[0] * x.shape[2]
             with torch.no_grad():
-                self.running_mean.mul_(1 - factor).add_(mean.to(self.running_mean.dtype), alpha=factor)
-                self.running_var.mul_(1 - factor).add_((var * (n / max(n - 1, 1))).to(self.running_var.dtype), alpha=factor)
+                self.running_mean.lerp_(mean.to(self.running_mean.dtype), factor)
+                self.running_var.lerp_((var * (n / max(n - 1, 1))).to(self.running_var.dtype), factor)
         return y
 
 

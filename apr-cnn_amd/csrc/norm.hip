@@ -2,8 +2,9 @@
 // activation of BasicBlock (apr_models/unet/unet_parts.py:17-26) on [batch, channels, particles] tensors.
 //
 // Both norms are "statistics over sets of rows": a row is one (batch, channel) line of the tensor; BatchNorm joins
-// the rows of one channel over the batch, GroupNorm the rows of one group.  The kernels here work per row and are
-// HBM-bound streams; joining the (tiny) per-row results into per-set results is left to the caller.
+// the rows of one channel over the batch, GroupNorm the rows of one group.  The streaming kernels work per row and
+// are HBM-bound; two one-launch kernels (norm_coeffs_fwd / norm_coeffs_bwd) join the per-row results into per-set
+// statistics and hand back per-row coefficients, so that a layer costs four launches each way.
 //
 //   forward   row_moments : mean and sum of squared deviations per row               reads x once
 //             norm_apply  : y = (x - mean) * scale + shift, optional ReLU            reads x, writes y
@@ -201,6 +202,84 @@ norm_bwd_apply_kernel(const T* __restrict__ gy, int64_t ldg, const T* __restrict
     }
 }
 
+// ---------------------------------------------------------------------------- joining rows into sets
+// One thread per row r = b * C + c.  The rows that share statistics with it ("its set") are the rows of channel c
+// over the batch (groups == 0: BatchNorm) or the C / groups rows of its group in batch item b (GroupNorm); every
+// thread joins its own set (a few to a few hundred values), which keeps the whole join in one tiny launch.
+struct SetOf {
+    int first, stride, count;       // member j is row first + j * stride
+};
+__device__ __forceinline__ SetOf set_of(int r, int B, int C, int groups) {
+    if (groups == 0) return SetOf{r % C, C, B};
+    const int k = C / groups;
+    return SetOf{(r / k) * k, 1, k};
+}
+
+// Per-row coefficients of the forward pass from the per-row moments (or from given statistics per channel).
+__global__ void norm_coeffs_fwd_kernel(int B, int C, int groups, double n, double eps, const double* __restrict__ row_mean,
+                                       const double* __restrict__ row_m2, const float* __restrict__ given_mean,
+                                       const float* __restrict__ given_var, const float* __restrict__ gamma,
+                                       const float* __restrict__ beta, float* __restrict__ mean32, float* __restrict__ rstd32,
+                                       float* __restrict__ scale32, float* __restrict__ shift32, float* __restrict__ set_mean,
+                                       float* __restrict__ set_var) {
+    const int r = blockIdx.x * blockDim.x + threadIdx.x;
+    if (r >= B * C) return;
+    const int c = r % C;
+    double mean, var;
+    if (given_mean) {
+        mean = given_mean[c]; var = given_var[c];
+    } else {
+        const SetOf s = set_of(r, B, C, groups);
+        double sm = 0;
+        for (int j = 0; j < s.count; ++j) sm += row_mean[s.first + j * s.stride];
+        mean = sm / s.count;
+        double m2 = 0;
+        for (int j = 0; j < s.count; ++j) {
+            const double d = row_mean[s.first + j * s.stride] - mean;
+            m2 += row_m2[s.first + j * s.stride] + n * d * d;
+        }
+        var = m2 / (n * s.count);
+        if (r == s.first) {             // the set's first row reports the statistics
+            const int si = groups == 0 ? c : r / (C / groups);
+            set_mean[si] = (float)mean; set_var[si] = (float)var;
+        }
+    }
+    const double rstd = 1.0 / sqrt(var + eps);
+    mean32[r] = (float)mean; rstd32[r] = (float)rstd;
+    scale32[r] = (float)((gamma ? (double)gamma[c] : 1.0) * rstd);
+    shift32[r] = beta ? beta[c] : 0.f;
+}
+
+// Per-row coefficients of gx = a * g + b * xhat + c from the per-row sums, and the parameter gradients.
+__global__ void norm_coeffs_bwd_kernel(int B, int C, int groups, double n, int own_stats, const double* __restrict__ sum_g,
+                                       const double* __restrict__ sum_gx, const float* __restrict__ gamma,
+                                       const float* __restrict__ rstd32, float* __restrict__ ca, float* __restrict__ cb,
+                                       float* __restrict__ cc, float* __restrict__ grad_gamma, float* __restrict__ grad_beta) {
+    const int r = blockIdx.x * blockDim.x + threadIdx.x;
+    if (r >= B * C) return;
+    const int c = r % C;
+    const double rs = rstd32[r];
+    double g1 = 0, g2 = 0;
+    if (own_stats) {                    // the statistics depend on the input: set means of gamma * g and gamma * g * xhat
+        const SetOf s = set_of(r, B, C, groups);
+        for (int j = 0; j < s.count; ++j) {
+            const int m = s.first + j * s.stride;
+            const double gm = gamma ? (double)gamma[m % C] : 1.0;
+            g1 += gm * sum_g[m]; g2 += gm * sum_gx[m];
+        }
+        g1 /= n * s.count; g2 /= n * s.count;
+    }
+    ca[r] = (float)((gamma ? (double)gamma[c] : 1.0) * rs);
+    cb[r] = (float)(-rs * g2);
+    cc[r] = (float)(-rs * g1);
+    if (r < C && (grad_gamma || grad_beta)) {       // sums over the batch for channel c = r
+        double sg = 0, sgx = 0;
+        for (int b = 0; b < B; ++b) { sg += sum_g[b * C + r]; sgx += sum_gx[b * C + r]; }
+        if (grad_gamma) grad_gamma[r] = (float)sgx;
+        if (grad_beta) grad_beta[r] = (float)sg;
+    }
+}
+
 // ---------------------------------------------------------------------------- host side
 static int check_rows(const char* what, int64_t rows, int64_t n) {
     if (rows < 0 || rows > 65535) return fail(APRNET_ERR_INVALID_ARGUMENT, what);      // rows ride on gridDim.y
@@ -267,10 +346,40 @@ int norm_bwd_apply(const T* gy, int64_t ldg, const T* x, int64_t ldx, const T* y
     return 0;
 }
 
+static int check_sets(const char* what, int B, int C, int groups, int64_t n) {
+    if (B <= 0 || C <= 0 || n <= 0 || (int64_t)B * C > 65535 || groups < 0 || (groups > 0 && C % groups != 0))
+        return fail(APRNET_ERR_INVALID_ARGUMENT, what);
+    return 0;
+}
+
 }  // namespace aprnet
 
 using namespace aprnet;
 extern "C" {
+int aprnet_norm_coeffs_fwd(int B, int C, int groups, int64_t n, double eps, const double* row_mean, const double* row_m2,
+                           const float* given_mean, const float* given_var, const float* gamma, const float* beta,
+                           float* mean32, float* rstd32, float* scale32, float* shift32, float* set_mean, float* set_var,
+                           void* st) {
+    if (int rc = check_sets("norm_coeffs_fwd: B, C, n positive, B * C <= 65535, groups dividing C", B, C, groups, n)) return rc;
+    const bool given = given_mean && given_var;
+    if (!mean32 || !rstd32 || !scale32 || !shift32 || (!given && (!row_mean || !row_m2 || !set_mean || !set_var)))
+        return fail(APRNET_ERR_INVALID_ARGUMENT, "norm_coeffs_fwd: null argument");
+    hipLaunchKernelGGL(norm_coeffs_fwd_kernel, dim3((unsigned)((B * C + 127) / 128)), dim3(128), 0, (hipStream_t)st, B, C, groups,
+                       (double)n, eps, row_mean, row_m2, given ? given_mean : nullptr, given ? given_var : nullptr, gamma, beta,
+                       mean32, rstd32, scale32, shift32, set_mean, set_var);
+    APRNET_LAUNCH_CHECK("norm_coeffs_fwd_kernel");
+    return 0;
+}
+int aprnet_norm_coeffs_bwd(int B, int C, int groups, int64_t n, int own_stats, const double* sum_g, const double* sum_gx,
+                           const float* gamma, const float* rstd32, float* a, float* b, float* c, float* grad_gamma,
+                           float* grad_beta, void* st) {
+    if (int rc = check_sets("norm_coeffs_bwd: B, C, n positive, B * C <= 65535, groups dividing C", B, C, groups, n)) return rc;
+    if (!sum_g || !sum_gx || !rstd32 || !a || !b || !c) return fail(APRNET_ERR_INVALID_ARGUMENT, "norm_coeffs_bwd: null argument");
+    hipLaunchKernelGGL(norm_coeffs_bwd_kernel, dim3((unsigned)((B * C + 127) / 128)), dim3(128), 0, (hipStream_t)st, B, C, groups,
+                       (double)n, own_stats, sum_g, sum_gx, gamma, rstd32, a, b, c, grad_gamma, grad_beta);
+    APRNET_LAUNCH_CHECK("norm_coeffs_bwd_kernel");
+    return 0;
+}
 int64_t aprnet_norm_work_elems(int64_t rows) { return std::max<int64_t>(rows, 1) * NORM_BLOCKS * 2; }
 #define NORM_API(T, CT, SFX)                                                                                            \
     int aprnet_row_moments_##SFX(const CT* x, int64_t ldx, int64_t rows, int64_t n, double* mean, double* m2, float* work, \

@@ -104,6 +104,9 @@ def hip():
     lib.aprnet_sample_image_max_f32.argtypes = [vp, i32, vp, i32, i32, i32, vp, vp]
     for t in ("u8", "u16", "u32", "u64"):     # plan, d, img, zn, xn, yn, dzs, dxs, dys, n_rays, max_steps, dist, stream
         getattr(lib, f"aprnet_labels_to_dist_{t}").argtypes = [vp, i32, vp, i32, i32, i32, vp, vp, vp, i32, i32, vp, vp]
+    f64 = C.c_double
+    lib.aprnet_norm_coeffs_fwd.argtypes = [i32, i32, i32, i64, f64, vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, vp]
+    lib.aprnet_norm_coeffs_bwd.argtypes = [i32, i32, i32, i64, i32, vp, vp, vp, vp, vp, vp, vp, vp, vp, vp]
     lib.aprnet_norm_work_elems.argtypes = [i64]
     lib.aprnet_norm_work_elems.restype = i64
     for t in ("f32", "bf16"):

@@ -256,6 +256,58 @@ def row_moments(x):
     return mean, m2
 
 
+def _f32_or_none(v, n, name):
+    if v is None:
+        return None
+    v = v.detach()
+    if v.dtype != torch.float32 or not v.is_contiguous():
+        v = v.float().contiguous()
+    if v.numel() != n or not v.is_cuda:
+        raise ValueError(f"{name}: GPU tensor with {n} entries expected")
+    return v
+
+
+def _optr(v):
+    return None if v is None else _ptr(v)
+
+
+def norm_coeffs_forward(shape, groups, eps, row_mean, row_m2, given, gamma, beta, device):
+    """The join of the forward pass in one launch.  shape = (B, C, N); groups = 0 for BatchNorm.  Either the row
+    moments or ``given`` = (mean[C], var[C]).  -> (mean32, rstd32, scale32, shift32 [B, C]; set_mean, set_var float32,
+    [C] or [B, groups], None with given statistics)."""
+    B, Cn, N = shape
+    out = [torch.empty(B, Cn, dtype=torch.float32, device=device) for _ in range(4)]
+    gm, gv = (None, None) if given is None else (_f32_or_none(given[0], Cn, "mean"), _f32_or_none(given[1], Cn, "var"))
+    sets = None
+    if given is None:
+        sets = [torch.empty(Cn if groups == 0 else (B, groups), dtype=torch.float32, device=device) for _ in range(2)]
+    gamma, beta = _f32_or_none(gamma, Cn, "weight"), _f32_or_none(beta, Cn, "bias")
+    with torch.cuda.device(device):
+        rc = _lib().aprnet_norm_coeffs_fwd(B, Cn, groups, N, float(eps), _optr(row_mean), _optr(row_m2), _optr(gm), _optr(gv),
+                                           _optr(gamma), _optr(beta), *[_ptr(t) for t in out],
+                                           _optr(sets[0] if sets else None), _optr(sets[1] if sets else None), _stream())
+    if rc:
+        _raise(rc, "norm_coeffs_forward failed")
+    return (*out, *(sets or (None, None)))
+
+
+def norm_coeffs_backward(shape, groups, own_stats, sum_g, sum_gx, gamma, rstd32, want_gamma, want_beta):
+    """The join of the backward pass in one launch -> (a, b, c [B, C] float32, grad_gamma, grad_beta [C] float32 or None)."""
+    B, Cn, N = shape
+    dev = sum_g.device
+    a, b, c = (torch.empty(B, Cn, dtype=torch.float32, device=dev) for _ in range(3))
+    gg = torch.empty(Cn, dtype=torch.float32, device=dev) if want_gamma else None
+    gb = torch.empty(Cn, dtype=torch.float32, device=dev) if want_beta else None
+    gamma = _f32_or_none(gamma, Cn, "weight")
+    with torch.cuda.device(dev):
+        rc = _lib().aprnet_norm_coeffs_bwd(B, Cn, groups, N, 1 if own_stats else 0, _ptr(sum_g), _ptr(sum_gx), _optr(gamma),
+                                           _ptr(_rowvec(rstd32, B * Cn, "rstd")), _ptr(a), _ptr(b), _ptr(c), _optr(gg), _optr(gb),
+                                           _stream())
+    if rc:
+        _raise(rc, "norm_coeffs_backward failed")
+    return a, b, c, gg, gb
+
+
 def norm_apply(x, mean, scale, shift, relu):
     """y = (x - mean) * scale + shift per row (float32 [B, C] coefficients), then ReLU if asked."""
     sfx = _norm_sfx(x, "input")

@@ -89,68 +89,40 @@ class NormFunction(Function):
     torch.nn.BatchNorm1d (``kind='batch'``: one set of statistics per channel, taken over batch and particles) and
     torch.nn.GroupNorm (``kind='group'``: one per batch item and group), as BasicBlock applies them
     (apr_models/unet/unet_parts.py:17-26).  ``stats`` = (mean[C], var[C]) normalises with given statistics (BatchNorm in
-    eval mode) instead of those of the input.  Returns ``(y, mean, var)``: the statistics used (biased variance), per
-    channel for 'batch' and [B, groups] for 'group'."""
+    eval mode) instead of those of the input.  Returns ``(y, mean, var)``: the statistics used (biased variance, float32),
+    per channel for 'batch' and [B, groups] for 'group'.  Four launches each way: row moments (two), the join, apply."""
 
     @staticmethod
     def forward(ctx, x, weight, bias, kind, groups, eps, relu, stats):
-        B, Cn, N = x.shape
         x = x.contiguous()
+        g = 0 if kind == "batch" else int(groups)
+        row_mean = row_m2 = None
         if stats is None:
-            mean_r, m2_r = _ops.row_moments(x)                      # float64 [B, C]
-            if kind == "batch":
-                k, mr, m2 = B, mean_r.t(), m2_r.t()                 # [C, B]
-            else:
-                k = Cn // groups
-                mr, m2 = mean_r.view(B, groups, k), m2_r.view(B, groups, k)
-            set_mean = mr.mean(-1)
-            set_var = (m2.sum(-1) + N * (mr - set_mean.unsqueeze(-1)).square().sum(-1)) / (k * N)
-        else:
-            set_mean, set_var = stats[0].double(), stats[1].double()
-
-        def to_rows(v):
-            if kind == "batch":
-                return v.unsqueeze(0).expand(B, Cn)
-            return v.unsqueeze(-1).expand(B, groups, Cn // groups).reshape(B, Cn)
-        rstd = to_rows((set_var + eps).rsqrt())
-        gamma = torch.ones(Cn, dtype=torch.float64, device=x.device) if weight is None else weight.detach().double()
-        beta = torch.zeros(Cn, dtype=torch.float64, device=x.device) if bias is None else bias.detach().double()
-        mean32 = to_rows(set_mean).float().contiguous()
-        rstd32 = rstd.float().contiguous()
-        y = _ops.norm_apply(x, mean32, (gamma.unsqueeze(0) * rstd).float().contiguous(),
-                            beta.unsqueeze(0).expand(B, Cn).float().contiguous(), relu)
+            row_mean, row_m2 = _ops.row_moments(x)                  # float64 [B, C]
+        mean32, rstd32, scale32, shift32, set_mean, set_var = _ops.norm_coeffs_forward(
+            tuple(x.shape), g, eps, row_mean, row_m2, stats, weight, bias, x.device)
+        y = _ops.norm_apply(x, mean32, scale32, shift32, relu)
+        if stats is not None:
+            set_mean, set_var = stats[0].detach().float(), stats[1].detach().float()
         ctx.save_for_backward(x, y if relu else None, mean32, rstd32, weight)
-        ctx.cfg = (kind, groups, stats is None, None if weight is None else weight.dtype, None if bias is None else bias.dtype)
+        ctx.cfg = (g, stats is None, None if weight is None else weight.dtype, None if bias is None else bias.dtype)
         ctx.mark_non_differentiable(set_mean, set_var)
         return y, set_mean, set_var
 
     @staticmethod
     def backward(ctx, grad_y, _gm, _gv):
         x, y, mean32, rstd32, weight = ctx.saved_tensors
-        kind, groups, own_stats, w_dtype, b_dtype = ctx.cfg
-        B, Cn, N = x.shape
+        g, own_stats, w_dtype, b_dtype = ctx.cfg
         grad_y = grad_y.contiguous()
         s_g, s_gx = _ops.norm_backward_sums(grad_y, x, y, mean32, rstd32)          # float64 [B, C]
-        grad_w = s_gx.sum(0).to(w_dtype) if w_dtype is not None and ctx.needs_input_grad[1] else None
-        grad_b = s_g.sum(0).to(b_dtype) if b_dtype is not None and ctx.needs_input_grad[2] else None
-        grad_x = None
-        if ctx.needs_input_grad[0]:
-            gamma = torch.ones(Cn, dtype=torch.float64, device=x.device) if weight is None else weight.detach().double()
-            rstd = rstd32.double()
-            a = gamma.unsqueeze(0) * rstd
-            if own_stats:       # the statistics depend on the input: subtract the set means of g and g * xhat
-                g1, g2 = gamma * s_g, gamma * s_gx
-                if kind == "batch":
-                    G1, G2 = (g1.sum(0) / (B * N)).expand(B, Cn), (g2.sum(0) / (B * N)).expand(B, Cn)
-                else:
-                    k = Cn // groups
-                    G1 = (g1.view(B, groups, k).sum(-1, keepdim=True) / (k * N)).expand(B, groups, k).reshape(B, Cn)
-                    G2 = (g2.view(B, groups, k).sum(-1, keepdim=True) / (k * N)).expand(B, groups, k).reshape(B, Cn)
-                b, c = -rstd * G2, -rstd * G1
-            else:
-                b = c = torch.zeros_like(a)
-            grad_x = _ops.norm_backward_apply(grad_y, x, y, mean32, rstd32, a.float().contiguous(), b.float().contiguous(),
-                                              c.float().contiguous())
+        want_w = w_dtype is not None and ctx.needs_input_grad[1]
+        want_b = b_dtype is not None and ctx.needs_input_grad[2]
+        a, b, c, grad_w, grad_b = _ops.norm_coeffs_backward(tuple(x.shape), g, own_stats, s_g, s_gx, weight, rstd32, want_w, want_b)
+        grad_x = _ops.norm_backward_apply(grad_y, x, y, mean32, rstd32, a, b, c) if ctx.needs_input_grad[0] else None
+        if grad_w is not None and grad_w.dtype != w_dtype:
+            grad_w = grad_w.to(w_dtype)
+        if grad_b is not None and grad_b.dtype != b_dtype:
+            grad_b = grad_b.to(b_dtype)
         return grad_x, grad_w, grad_b, None, None, None, None, None
 
 

@@ -187,6 +187,21 @@ def other_ops(apr, x, dev):
     res.append({"op": "apr_unet_train_step", "ms": ms, "particles_per_s": n0 / ms * 1e3,
                 "note": "forward + backward of the 4-level network, fp32, BatchNorm in training mode, MSE loss, no optimizer"})
     del tnet, target
+    # the same step on an APR of the size training crops have (64 x 128 x 128 centre crop): bound by the host, ~850 launches
+    small = build_workload("blobs512", crop=(64, 128, 128))
+    ns = small.total_number_particles()
+    torch.manual_seed(0)
+    snet = APRUNet(1, 3, depth=3, n_filters_base=16, n_stencils=2, norm="batch").to(dev).train()
+    xs, ts = torch.randn(1, 1, ns, device=dev), torch.randn(1, 3, ns, device=dev)
+
+    def small_step():
+        for p_ in snet.parameters():
+            p_.grad = None
+        torch.nn.functional.mse_loss(snet(xs, [small]), ts).backward()
+    ms = _time(small_step, iters=10, warmup=3)
+    res.append({"op": "apr_unet_train_step_small", "ms": ms, "particles_per_s": ns / ms * 1e3,
+                "note": f"the same training step on a 64x128x128 crop, {ns} particles: host-bound (Python operator wrappers, ~850 launches)"})
+    del snet, xs, ts, small
     # the wide 2-D stencil of configs[4] (1x5x5, 64 -> 64), here on the 3-D benchmark APR, fp32
     conv5 = aprnet.cuda.APRConv(64, 64, nstencils=2, kernel_size=(1, 5, 5)).to(dev)
     x64 = torch.randn(1, 64, x.shape[2], device=dev)

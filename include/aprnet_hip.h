@@ -249,9 +249,9 @@ int aprnet_labels_to_dist_u64(const aprnet_plan*, int level_delta, const uint64_
 /* Normalisation over the particle axis and the ReLU after it: the torch.nn.BatchNorm1d / torch.nn.GroupNorm +
  * activation that follow every convolution of the networks (apr_models/unet/unet_parts.py:17-26; library calls on
  * [batch, channels, particles] tensors in the reference, MIOpen / ATen kernels on a GPU).  The kernels work on
- * rows: row r = one (batch item, channel) line of n elements at x + r * ldx.  The caller joins the per-row results
- * into per-channel (BatchNorm) or per-group (GroupNorm) statistics - a few values per row - and passes per-row
- * coefficients back.  rows <= 65535, n > 0.  work: aprnet_norm_work_elems(rows) floats of scratch.
+ * rows: row r = one (batch item, channel) line of n elements at x + r * ldx.  The per-row results are joined into
+ * per-channel (BatchNorm) or per-group (GroupNorm) statistics - a few values per row - by aprnet_norm_coeffs_*,
+ * which hand per-row coefficients back.  rows <= 65535, n > 0.  work: aprnet_norm_work_elems(rows) floats of scratch.
  *   row_moments     mean[r], m2[r] = mean and sum of squared deviations of row r (fp64 results).
  *   norm_apply      y = (x - mean[r]) * scale[r] + shift[r], then max(., 0) if relu != 0.
  *   norm_bwd_sums   sum_g[r] = sum g, sum_gx[r] = sum g * xhat with xhat = (x - mean[r]) * rstd[r] and
@@ -259,6 +259,21 @@ int aprnet_labels_to_dist_u64(const aprnet_plan*, int level_delta, const uint64_
  *   norm_bwd_apply  gx = a[r] * g + b[r] * xhat + c[r].
  * Sums are taken in a fixed order (fp32 per thread and block, fp64 across blocks): results repeat bit for bit. */
 int64_t aprnet_norm_work_elems(int64_t rows);
+/* The join between the row kernels, one launch each way (the arithmetic of torch.nn.BatchNorm1d when groups == 0 -
+ * a channel's rows over the batch share statistics - and of torch.nn.GroupNorm(groups, C) otherwise; biased
+ * variance).  Arrays are [B * C] per row unless noted; gamma / beta [C] or NULL.
+ *   coeffs_fwd  from row_mean / row_m2 (row_moments), or from given_mean / given_var [C] (BatchNorm in eval mode)
+ *               when those are not NULL: mean32, rstd32, scale32 = gamma * rstd, shift32 = beta for norm_apply, and
+ *               the statistics used, set_mean / set_var ([C], or [B * groups]; not written with given statistics).
+ *   coeffs_bwd  from the sums of norm_bwd_sums: a, b, c for norm_bwd_apply (b = c = 0 when own_stats == 0, i.e. the
+ *               statistics did not depend on the input) and grad_gamma / grad_beta [C] (each may be NULL). */
+int aprnet_norm_coeffs_fwd(int B, int C, int groups, int64_t n, double eps, const double* row_mean, const double* row_m2,
+                           const float* given_mean, const float* given_var, const float* gamma, const float* beta,
+                           float* mean32, float* rstd32, float* scale32, float* shift32, float* set_mean, float* set_var,
+                           void* stream);
+int aprnet_norm_coeffs_bwd(int B, int C, int groups, int64_t n, int own_stats, const double* sum_g, const double* sum_gx,
+                           const float* gamma, const float* rstd32, float* a, float* b, float* c, float* grad_gamma,
+                           float* grad_beta, void* stream);
 int aprnet_row_moments_f32(const float* x, int64_t ldx, int64_t rows, int64_t n, double* mean, double* m2, float* work, void* stream);
 int aprnet_row_moments_bf16(const uint16_t* x, int64_t ldx, int64_t rows, int64_t n, double* mean, double* m2, float* work, void* stream);
 int aprnet_norm_apply_f32(const float* x, int64_t ldx, int64_t rows, int64_t n, const float* mean, const float* scale,
