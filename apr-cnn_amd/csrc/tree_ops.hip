@@ -82,12 +82,9 @@ __device__ __forceinline__ void store_children(const int32_t (&ch)[8], T* part, 
 // particles before tree nodes for coarser parents (:201-250); the same order is kept so the fp32
 // sums agree to the last bit.
 template <typename T>
-__global__ void __launch_bounds__(TB)
-fill_tree_level_kernel(const int32_t* __restrict__ children, int64_t n_tree, int64_t t_begin, int64_t t_end,
-                       const T* __restrict__ x, int64_t ldx, int C, T* __restrict__ tree, int64_t ldt,
-                       int64_t tree_off, int tree_child_from_x, int tree_first) {
-    const int64_t t = t_begin + (int64_t)blockIdx.x * TB + threadIdx.x;
-    if (t >= t_end) return;
+__device__ __forceinline__ void fill_node(const int32_t* children, int64_t n_tree, int64_t t, const T* x, int64_t ldx,
+                                          int C, T* tree, int64_t ldt, int64_t tree_off, int tree_child_from_x,
+                                          int tree_first, int cg) {
     int32_t ch[8];
     int cnt = 0;
 #pragma unroll
@@ -97,7 +94,7 @@ fill_tree_level_kernel(const int32_t* __restrict__ children, int64_t n_tree, int
     const A scale = (A)(1.0f / (float)max(cnt, 1));
 #pragma unroll
     for (int k = 0; k < CPT; ++k) {
-        const int c = blockIdx.y * CPT + k;
+        const int c = cg * CPT + k;
         if (c >= C) break;
         const T* xc = x + (int64_t)c * ldx;
         T* tc = tree + (int64_t)c * ldt;
@@ -118,14 +115,38 @@ fill_tree_level_kernel(const int32_t* __restrict__ children, int64_t n_tree, int
     }
 }
 
-// helpers.hpp:255-350, parent-driven: every child has exactly one parent, so no write conflicts.
 template <typename T>
 __global__ void __launch_bounds__(TB)
-fill_tree_bwd_level_kernel(const int32_t* __restrict__ children, int64_t n_tree, int64_t t_begin, int64_t t_end,
-                           T* __restrict__ gx, int64_t ldx, int C, T* __restrict__ gtree, int64_t ldt,
-                           int64_t tree_off, int tree_child_in_x) {
+fill_tree_level_kernel(const int32_t* __restrict__ children, int64_t n_tree, int64_t t_begin, int64_t t_end,
+                       const T* __restrict__ x, int64_t ldx, int C, T* __restrict__ tree, int64_t ldt,
+                       int64_t tree_off, int tree_child_from_x, int tree_first) {
     const int64_t t = t_begin + (int64_t)blockIdx.x * TB + threadIdx.x;
-    if (t >= t_end) return;
+    if (t < t_end) fill_node<T>(children, n_tree, t, x, ldx, C, tree, ldt, tree_off, tree_child_from_x, tree_first, blockIdx.y);
+}
+
+// The coarse levels of the tree hold a few nodes each: one launch walks them all, finest first, one workgroup per
+// group of CPT channels (a level's parents read only values of the same channels, so a workgroup barrier between
+// levels is enough).  Tree children come from the tree itself (none of these levels sits directly under the features),
+// particle children from the feature vector as always.
+constexpr int MAX_COARSE = 12;
+struct CoarseLevels { int n; int64_t begin[MAX_COARSE], end[MAX_COARSE]; };
+constexpr int64_t COARSE_NODES = 2048;      // levels are merged while they hold at most this many nodes together
+
+template <typename T>
+__global__ void __launch_bounds__(TB)
+fill_tree_coarse_kernel(const int32_t* __restrict__ children, int64_t n_tree, const CoarseLevels lv, const T* x, int64_t ldx,
+                        int C, T* tree, int64_t ldt) {
+    for (int i = 0; i < lv.n; ++i) {
+        for (int64_t t = lv.begin[i] + threadIdx.x; t < lv.end[i]; t += TB)
+            fill_node<T>(children, n_tree, t, x, ldx, C, tree, ldt, 0, 0, 0, blockIdx.x);
+        __syncthreads();
+    }
+}
+
+// helpers.hpp:255-350, parent-driven: every child has exactly one parent, so no write conflicts.
+template <typename T>
+__device__ __forceinline__ void fill_node_bwd(const int32_t* children, int64_t n_tree, int64_t t, T* gx, int64_t ldx,
+                                              int C, T* gtree, int64_t ldt, int64_t tree_off, int tree_child_in_x, int cg) {
     int32_t ch[8];
     int cnt = 0;
 #pragma unroll
@@ -134,7 +155,7 @@ fill_tree_bwd_level_kernel(const int32_t* __restrict__ children, int64_t n_tree,
     const A scale = (A)(1.0f / (float)max(cnt, 1));
 #pragma unroll
     for (int k = 0; k < CPT; ++k) {
-        const int c = blockIdx.y * CPT + k;
+        const int c = cg * CPT + k;
         if (c >= C) break;
         T* gxc = gx + (int64_t)c * ldx;
         T* gtc = gtree + (int64_t)c * ldt;
@@ -146,6 +167,27 @@ fill_tree_bwd_level_kernel(const int32_t* __restrict__ children, int64_t n_tree,
 #pragma unroll
         for (int s = 0; s < 8; ++s) out[s] = Num<T>::st(val[s] + g);
         store_children<T>(ch, gxc, gt_child, out);
+    }
+}
+
+template <typename T>
+__global__ void __launch_bounds__(TB)
+fill_tree_bwd_level_kernel(const int32_t* __restrict__ children, int64_t n_tree, int64_t t_begin, int64_t t_end,
+                           T* __restrict__ gx, int64_t ldx, int C, T* __restrict__ gtree, int64_t ldt,
+                           int64_t tree_off, int tree_child_in_x) {
+    const int64_t t = t_begin + (int64_t)blockIdx.x * TB + threadIdx.x;
+    if (t < t_end) fill_node_bwd<T>(children, n_tree, t, gx, ldx, C, gtree, ldt, tree_off, tree_child_in_x, blockIdx.y);
+}
+
+// the coarse levels in one launch, coarsest first (a parent's share must have arrived before it is handed down)
+template <typename T>
+__global__ void __launch_bounds__(TB)
+fill_tree_bwd_coarse_kernel(const int32_t* __restrict__ children, int64_t n_tree, const CoarseLevels lv, T* gx, int64_t ldx,
+                            int C, T* gtree, int64_t ldt) {
+    for (int i = 0; i < lv.n; ++i) {
+        for (int64_t t = lv.begin[i] + threadIdx.x; t < lv.end[i]; t += TB)
+            fill_node_bwd<T>(children, n_tree, t, gx, ldx, C, gtree, ldt, 0, 0, blockIdx.x);
+        __syncthreads();
     }
 }
 
@@ -285,13 +327,29 @@ upsample_kernel(const int32_t* __restrict__ children, int64_t n_tree, int64_t n_
 }
 
 // ---------------------------------------------------------------------------- host launchers
+// Highest level l <= l_top - 1 such that levels level_min .. l hold at most COARSE_NODES nodes together (and are
+// at most MAX_COARSE levels); level_min - 1 when there is none.  The level directly under the features (l_top when
+// it is Lc - 1) is never merged: its children are read from the feature vector.
+static int coarse_levels_end(const aprnet_plan* p, int l_top) {
+    int64_t nodes = 0;
+    int l = p->tree.level_min - 1;
+    while (l + 1 < l_top && l + 1 - p->tree.level_min < MAX_COARSE) {
+        nodes += p->tree.level_end(l + 1) - p->tree.level_begin(l + 1);
+        if (nodes > COARSE_NODES) break;
+        ++l;
+    }
+    return l;
+}
+
 template <typename T>
 int fill_tree_mean(const aprnet_plan* p, int d, const T* x, int64_t ldx, int C, T* tree, int64_t ldt, hipStream_t st) {
     if (int rc = check_level_delta(p, d, "fill_tree_mean")) return rc;
     if (C <= 0) return 0;
     const int Lc = p->lc(d);
     if (ldt < p->tree_parts(d)) return fail(APRNET_ERR_INVALID_ARGUMENT, "fill_tree_mean: tree work space too small");
-    for (int l = std::min(Lc - 1, p->tree.level_max); l >= p->tree.level_min; --l) {
+    const int l_top = std::min(Lc - 1, p->tree.level_max);
+    const int l_coarse = coarse_levels_end(p, l_top);            // levels level_min .. l_coarse go in one launch
+    for (int l = l_top; l > l_coarse; --l) {
         const int64_t b = p->tree.level_begin(l), e = p->tree.level_end(l);
         if (e <= b) continue;
         dim3 grid((unsigned)((e - b + TB - 1) / TB), (unsigned)((C + CPT - 1) / CPT));
@@ -299,7 +357,13 @@ int fill_tree_mean(const aprnet_plan* p, int d, const T* x, int64_t ldx, int C, 
         hipLaunchKernelGGL(fill_tree_level_kernel<T>, grid, dim3(TB), 0, st, p->d_children, p->n_tree, b, e, x, ldx, C,
                            tree, ldt, from_x ? p->tree_offset(Lc) : 0, from_x, from_x);
     }
-    APRNET_LAUNCH_CHECK("fill_tree_level_kernel");
+    CoarseLevels lv{};
+    for (int l = l_coarse; l >= p->tree.level_min; --l)
+        if (p->tree.level_end(l) > p->tree.level_begin(l)) { lv.begin[lv.n] = p->tree.level_begin(l); lv.end[lv.n] = p->tree.level_end(l); ++lv.n; }
+    if (lv.n > 0)
+        hipLaunchKernelGGL(fill_tree_coarse_kernel<T>, dim3((unsigned)((C + CPT - 1) / CPT)), dim3(TB), 0, st, p->d_children, p->n_tree,
+                           lv, x, ldx, C, tree, ldt);
+    APRNET_LAUNCH_CHECK("fill_tree kernels");
     return 0;
 }
 
@@ -308,7 +372,15 @@ int fill_tree_mean_bwd(const aprnet_plan* p, int d, T* gx, int64_t ldx, int C, T
     if (int rc = check_level_delta(p, d, "fill_tree_mean_bwd")) return rc;
     if (C <= 0) return 0;
     const int Lc = p->lc(d);
-    for (int l = p->tree.level_min; l <= std::min(Lc - 1, p->tree.level_max); ++l) {
+    const int l_top = std::min(Lc - 1, p->tree.level_max);
+    const int l_coarse = coarse_levels_end(p, l_top);
+    CoarseLevels lv{};
+    for (int l = p->tree.level_min; l <= l_coarse; ++l)
+        if (p->tree.level_end(l) > p->tree.level_begin(l)) { lv.begin[lv.n] = p->tree.level_begin(l); lv.end[lv.n] = p->tree.level_end(l); ++lv.n; }
+    if (lv.n > 0)
+        hipLaunchKernelGGL(fill_tree_bwd_coarse_kernel<T>, dim3((unsigned)((C + CPT - 1) / CPT)), dim3(TB), 0, st, p->d_children,
+                           p->n_tree, lv, gx, ldx, C, gtree, ldt);
+    for (int l = std::max(l_coarse + 1, p->tree.level_min); l <= l_top; ++l) {
         const int64_t b = p->tree.level_begin(l), e = p->tree.level_end(l);
         if (e <= b) continue;
         dim3 grid((unsigned)((e - b + TB - 1) / TB), (unsigned)((C + CPT - 1) / CPT));
