@@ -52,15 +52,17 @@ __global__ void pack_weights16_kernel(const float* __restrict__ w, int S_exp, in
                                       int transposed, float* __restrict__ out) {
     const int Cout = transposed ? Ck : Cm, Cin = transposed ? Cm : Ck;
     const int ncb = (Cm + 16 * COH - 1) / (16 * COH), nq = (Ck + CIB - 1) / CIB;
-    const int64_t n = (int64_t)S_exp * ncb * nq * K * COH * CIB * 16;
-    for (int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; e < n; e += (int64_t)gridDim.x * blockDim.x) {
-        int64_t r = e;
-        const int co = (int)(r % 16); r /= 16;
-        const int c = (int)(r % CIB); r /= CIB;
-        const int h = (int)(r % COH); r /= COH;
-        const int t = (int)(r % K); r /= K;
-        const int q = (int)(r % nq); r /= nq;
-        const int cb = (int)(r % ncb); r /= ncb;
+    // 32-bit index arithmetic (the host checks that the image has fewer than 2^31 elements): 64-bit divisions made
+    // this tiny kernel take longer than the convolution of a coarse level
+    const unsigned n = (unsigned)S_exp * ncb * nq * K * COH * CIB * 16;
+    for (unsigned e = blockIdx.x * blockDim.x + threadIdx.x; e < n; e += gridDim.x * blockDim.x) {
+        unsigned r = e;
+        const int co = (int)(r % 16u); r /= 16u;
+        const int c = (int)(r % (unsigned)CIB); r /= (unsigned)CIB;
+        const int h = (int)(r % (unsigned)COH); r /= (unsigned)COH;
+        const int t = (int)(r % (unsigned)K); r /= (unsigned)K;
+        const int q = (int)(r % (unsigned)nq); r /= (unsigned)nq;
+        const int cb = (int)(r % (unsigned)ncb); r /= (unsigned)ncb;
         const int s = (int)r;
         const int ck = q * CIB + c, cm = (cb * COH + h) * 16 + co;
         float v = 0.f;
@@ -606,6 +608,7 @@ size_t conv_packed_floats(int code, int S_exp, int Cm, int Ck, bool transposed) 
 
 int pack_conv_weights(int code, const float* w, int S_exp, int Cm, int Ck, bool transposed, float* packed, hipStream_t st) {
     const size_t n = conv_packed_floats(code, S_exp, Cm, Ck, transposed);
+    if (n >= ((size_t)1 << 31)) return fail(APRNET_ERR_UNSUPPORTED, "packed weight image of 2^31 elements or more");
     dim3 grid((unsigned)std::min<size_t>((n + 255) / 256, 2048));
     hipLaunchKernelGGL(pack_weights16_kernel, grid, dim3(256), 0, st, w, S_exp, Cm, Ck, conv_taps(code), transposed ? DX_CIB : FWD_CIB, conv_coh(Cm),
                        transposed ? 1 : 0, packed);
