@@ -303,6 +303,66 @@ def test_unet_forward_replays_from_a_hip_graph(dtype):
             assert torch.equal(y_static, eager), f"replay {k}"
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
+def test_unet_training_step_replays_from_a_hip_graph(dtype):
+    """Forward, loss and backward of the network in training mode (BatchNorm statistics of the batch, running
+    statistics updated) captured into one HIP graph: the backward operators fork the weight gradient onto the
+    plan's second stream and join it again, clear their work space with fill kernels and neither allocate outside
+    torch's allocator nor synchronise.  Every replay, with new inputs and with eager steps and synchronisations in
+    between, gives the loss, the parameter gradients and the running statistics of the same step run eagerly
+    (to the 1e-4 that the order of the atomic additions of the gradients leaves open; 2e-2 with bfloat16 features)."""
+    import copy
+    apr = apr_cases.random_apr((33, 29, 37), 11, density=0.02)
+    torch.manual_seed(0)
+    model = APRUNet(1, 3, depth=3, n_filters_base=8, n_stencils=2, norm="batch").to(DEV).train()
+    ref = copy.deepcopy(model)
+    n = apr.total_number_particles()
+    g = torch.Generator().manual_seed(1)
+    x_static = torch.randn(1, 1, n, generator=g).to(dtype).to(DEV)
+    t_static = torch.randn(1, 3, n, generator=g).to(DEV)
+
+    def step(m, x, t):
+        for p in m.parameters():
+            p.grad = None
+        loss = torch.nn.functional.mse_loss(m(x, [apr]).float(), t)
+        loss.backward()
+        return loss
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for _ in range(2):                                       # eager warm-up: lists, tile tables, scratch
+            step(model, x_static, t_static)
+            step(ref, x_static, t_static)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    for p in model.parameters():
+        p.grad = None
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        loss_static = step(model, x_static, t_static)
+    tol = 2e-2 if dtype == torch.bfloat16 else 1e-4
+    for k in range(3):
+        x_new = torch.randn(1, 1, n, generator=g).to(dtype).to(DEV)
+        t_new = torch.randn(1, 3, n, generator=g).to(DEV)
+        loss_eager = step(ref, x_new, t_new)
+        torch.cuda.synchronize()
+        x_static.copy_(x_new)
+        t_static.copy_(t_new)
+        graph.replay()
+        torch.cuda.synchronize()
+        assert abs(float(loss_static) - float(loss_eager)) <= tol * abs(float(loss_eager)), f"replay {k}"
+        scale = max(float(q.grad.abs().max()) for q in ref.parameters())
+        for (name, p), q in zip(model.named_parameters(), ref.parameters()):
+            assert p.grad is not None and torch.isfinite(p.grad).all(), name
+            # a convolution's bias in front of a norm layer has a zero gradient up to rounding: absolute term
+            bound = tol * float(q.grad.abs().max()) + 0.02 * tol * scale
+            assert float((p.grad - q.grad).abs().max()) <= bound, f"replay {k}: {name}"
+        for (name, b), c in zip(model.named_buffers(), ref.named_buffers()):
+            assert name == c[0]
+            assert torch.allclose(b.float(), c[1].float(), rtol=tol, atol=tol * 1e-2), f"replay {k}: {name}"
+
+
 def test_hybrid_stardist_unet_matches_oracle():
     """HybridStardistUNet (stardist_hybrid_model.py:24-199): dense stages below the transition, decoder back to the
     particles at output_level_delta = 1, probability and distance heads there; against the oracle composition."""
