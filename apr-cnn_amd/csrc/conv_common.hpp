@@ -443,12 +443,21 @@ __device__ __forceinline__ void load_values(const ConvArgs<T>& a, int ci0, int n
     for (int k = 0; k < NR; ++k) {
         if ((round0 + k) * G::NT >= nitem) break;       // wave-uniform
         const bool from_tree = (R.pos[k] & ITEM_TREE) != 0 && R.pos[k] != 0xffffu;
-        const unsigned offx = from_tree ? BUF_OOB : R.off[k], offt = from_tree ? R.off[k] : BUF_OOB;
-#pragma unroll
-        for (int c = 0; c < CIB; ++c) R.v[k][c] = RawLoad<T>::ld(rx[c], offx);
         if (tree_items) {      // tile-uniform: only levels below the current maximum read the mean-filled tree
+            // Each lane loads from the one tensor its item lives in, under its own half of the execution mask, into
+            // the same registers: no second set of registers and no wait between the two groups of loads (combining
+            // two full loads per channel made the compiler wait for every tree load before it issued the next).
+            if (from_tree) {
 #pragma unroll
-            for (int c = 0; c < CIB; ++c) R.v[k][c] |= RawLoad<T>::ld(rt[c], offt);     // one of the two returned zero
+                for (int c = 0; c < CIB; ++c) R.v[k][c] = RawLoad<T>::ld(rt[c], R.off[k]);
+                asm volatile("" ::: "memory");       // keeps the two branches from being merged into one load with a per-lane descriptor
+            } else {
+#pragma unroll
+                for (int c = 0; c < CIB; ++c) R.v[k][c] = RawLoad<T>::ld(rx[c], R.off[k]);
+            }
+        } else {
+#pragma unroll
+            for (int c = 0; c < CIB; ++c) R.v[k][c] = RawLoad<T>::ld(rx[c], R.off[k]);
         }
     }
 }
