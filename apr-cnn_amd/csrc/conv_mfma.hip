@@ -165,18 +165,26 @@ __device__ __forceinline__ void mfma16_window(const ConvArgs<T>& a, int co0, int
             }
         }
         __builtin_amdgcn_s_setprio(0);
+        // The B operand of the next block is read before the matrix instructions of this one are issued, so that a
+        // wave alone in its matrix phase does not sit out an LDS round trip per pair of instructions.
+        if constexpr (NB > 0) {
+            float bvn = lpatch[bbase[0] + tap_offset<G>(0)];
 #pragma unroll
-        for (int t = 0; t < G::K; ++t) {
+            for (int t = 0; t < G::K; ++t) {
 #pragma unroll
-            for (int sb = 0; sb < NSUB; ++sb) {
-                float av[COH];
+                for (int sb = 0; sb < NSUB; ++sb) {
+                    float av[COH];
 #pragma unroll
-                for (int h = 0; h < COH; ++h) av[h] = ap[((t * COH + h) * NSUB + sb) * 64];
+                    for (int h = 0; h < COH; ++h) av[h] = ap[((t * COH + h) * NSUB + sb) * 64];
 #pragma unroll
-                for (int j = 0; j < NB; ++j) {
-                    const float bv = lpatch[bbase[j] + 4 * sb * G::CH_STRIDE + tap_offset<G>(t)];
+                    for (int j = 0; j < NB; ++j) {
+                        const float bv = bvn;
+                        if (j + 1 < NB) bvn = lpatch[bbase[j + 1] + 4 * sb * G::CH_STRIDE + tap_offset<G>(t)];
+                        else if (sb + 1 < NSUB) bvn = lpatch[bbase[0] + 4 * (sb + 1) * G::CH_STRIDE + tap_offset<G>(t)];
+                        else if (t + 1 < G::K) bvn = lpatch[bbase[0] + tap_offset<G>(t + 1 < G::K ? t + 1 : t)];
 #pragma unroll
-                    for (int h = 0; h < COH; ++h) acc[j][h] = __builtin_amdgcn_mfma_f32_16x16x4f32(av[h], bv, acc[j][h], 0, 0, 0);
+                        for (int h = 0; h < COH; ++h) acc[j][h] = __builtin_amdgcn_mfma_f32_16x16x4f32(av[h], bv, acc[j][h], 0, 0, 0);
+                    }
                 }
             }
         }
