@@ -33,7 +33,7 @@ PEAK_HBM_GBS = 8000.0
 # profiler passes, scaled by what the same counters read for a device-to-device copy of known size
 # (profiles/conv333_fwd_32x32_f32_blobs512_hbm_traffic.txt).  Counters cannot be read from inside this
 # script; the figure is only reported when the workload is the one it was measured on.
-MEASURED_TRAFFIC_BYTES = {23245996: 30.90e9 + 4.21e9}
+MEASURED_TRAFFIC_BYTES = {23245996: 30.18e9 + 4.10e9}
 
 
 def build_workload(name, crop=None):
