@@ -200,8 +200,23 @@ def other_ops(apr, x, dev):
         torch.nn.functional.mse_loss(snet(xs, [small]), ts).backward()
     ms = _time(small_step, iters=10, warmup=3)
     res.append({"op": "apr_unet_train_step_small", "ms": ms, "particles_per_s": ns / ms * 1e3,
-                "note": f"the same training step on a 64x128x128 crop, {ns} particles: host-bound (Python operator wrappers, ~850 launches)"})
-    del snet, xs, ts, small
+                "note": f"the same training step on a 64x128x128 crop, {ns} particles, ~590 short launches on two streams"})
+    # the same step captured once into a HIP graph (forward, loss, backward) and replayed
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        small_step()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    for p_ in snet.parameters():
+        p_.grad = None
+    sgraph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(sgraph):
+        torch.nn.functional.mse_loss(snet(xs, [small]), ts).backward()
+    ms = _time(sgraph.replay, iters=10, warmup=3)
+    res.append({"op": "apr_unet_train_step_small_graph", "ms": ms, "particles_per_s": ns / ms * 1e3,
+                "note": "that step replayed from a HIP graph: no host work between the launches"})
+    del sgraph, snet, xs, ts, small
     # the wide 2-D stencil of configs[4] (1x5x5, 64 -> 64), here on the 3-D benchmark APR, fp32
     conv5 = aprnet.cuda.APRConv(64, 64, nstencils=2, kernel_size=(1, 5, 5)).to(dev)
     x64 = torch.randn(1, 64, x.shape[2], device=dev)
