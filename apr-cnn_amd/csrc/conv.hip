@@ -137,7 +137,10 @@ int launch_conv_mfma(int code, const ConvArgs<bf16_t>& a, int n_tiles, hipStream
 int launch_conv_mfma_bf16(int code, const ConvArgs<bf16_t>& a, int n_tiles, hipStream_t st);
 size_t conv_packed_bf16_bytes(int code, int S_exp, int Cout, int Cin);
 int pack_conv_weights_bf16(int code, const float* w, int S_exp, int Cout, int Cin, void* packed, hipStream_t st, bool transposed = false);
+int interleave8_bf16(const bf16_t* x, int64_t ldx, const bf16_t* x2, int64_t ldx2, int c_split, int C, int64_t count, bf16_t* out,
+                     hipStream_t st);
 static int g_bf16_math = 1;      // bfloat16 features: 1 = bfloat16 matrix instructions, 0 = fp32 matrix instructions
+static int g_bf16_regroup = 1;   // bfloat16 forward: 1 = stage from a copy of the input regrouped by 8 channels, 0 = from the channel planes
 int fill_tree_for_conv(const aprnet_plan* p, int d, const bf16_t* x, int64_t ldx, int C, bf16_t* tree, int64_t ldt, hipStream_t st);
 size_t conv_packed_floats(int code, int S_exp, int Cm, int Ck, bool transposed);
 int pack_conv_weights(int code, const float* w, int S_exp, int Cm, int Ck, bool transposed, float* packed, hipStream_t st);
@@ -269,9 +272,22 @@ int conv_fwd_bf16(const aprnet_plan* cp, int d, int kz, int kx, int ky, const bf
     ConvArgs<bf16_t> a{};
     if (int rc = set_lists(p, d, code, tl, a, st)) return rc;
     const bool bf16_math = g_bf16_math && a.tile_win;      // the bfloat16 contraction exists with window lists only
+    const int64_t n_x = p->number_parts(d), n_t = p->tree_parts(d);
     if (bf16_math) {
-        if (int rc = plan_scratch(p, conv_packed_bf16_bytes(code, S_exp, Cout, Cin), st)) return rc;
+        // The input regrouped as [Cin / 8][count][8] behind the packed weights in the plan's scratch buffer, when its
+        // 16-byte items stay addressable with 32-bit offsets and the copy stays below 32 GiB.
+        const size_t wbytes = (conv_packed_bf16_bytes(code, S_exp, Cout, Cin) + 255) / 256 * 256;
+        const size_t ng = (size_t)(Cin + 7) / 8, ibytes = ng * (size_t)(n_x + n_t) * 16;
+        const bool regroup = g_bf16_regroup && n_x < (1ll << 28) && n_t < (1ll << 28) && ibytes <= ((size_t)32 << 30);
+        if (int rc = plan_scratch(p, wbytes + (regroup ? ibytes : 0), st)) return rc;
         if (int rc = pack_conv_weights_bf16(code, w, S_exp, Cout, Cin, p->d_scratch, st)) return rc;
+        if (regroup) {
+            bf16_t* xi = (bf16_t*)((char*)p->d_scratch + wbytes);
+            bf16_t* ti = xi + ng * (size_t)n_x * 8;
+            if (int rc = interleave8_bf16(x, ldx, fu.x2, fu.ldx2, C1, Cin, n_x, xi, st)) return rc;
+            if (int rc = interleave8_bf16(tree_ws, ldt, nullptr, 0, Cin, Cin, n_t, ti, st)) return rc;
+            a.xi = xi; a.ti = ti;
+        }
     } else {
         if (int rc = plan_scratch(p, conv_packed_floats(code, S_exp, Cout, Cin, false) * sizeof(float), st)) return rc;
         if (int rc = pack_conv_weights(code, w, S_exp, Cout, Cin, false, (float*)p->d_scratch, st)) return rc;
@@ -334,9 +350,11 @@ int aprnet_set_conv_path(int path) {
     if (path == 2 || path == 3) { g_bf16_math = path == 2; return 0; }
     if (path == 4 || path == 5) { g_use_lists = path == 4; return 0; }
     if (path == 6 || path == 7) { g_bwd_overlap = path == 6; return 0; }
+    if (path == 8 || path == 9) { g_bf16_regroup = path == 8; return 0; }
     if (path != 0 && path != 1)
         return fail(APRNET_ERR_INVALID_ARGUMENT, "set_conv_path: 0 (auto), 1 (VALU only), 2 / 3 (bfloat16 features: bfloat16 / fp32 "
-                                                 "matrix math), 4 / 5 (forward: window lists of the plan / scan per call)");
+                                                 "matrix math), 4 / 5 (forward: window lists of the plan / scan per call), 6 / 7 (backward on two streams / one), "
+                                                 "8 / 9 (bfloat16 forward: regrouped copy of the input / channel planes)");
     g_conv_path = path;
     return 0;
 }

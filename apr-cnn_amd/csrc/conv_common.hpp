@@ -37,6 +37,9 @@ struct ConvArgs {
     const T* tree_data; int64_t ldt;
     int Lc; int64_t tree_off;                  // tree_offset(Lc)
     int64_t x_count, t_count;                  // valid elements per channel plane of x / tree_data
+    // bfloat16 forward only: the input (both tensors) and the tree values regrouped as [Cin / 8][count][8], one
+    // 16-byte load per item and group of 8 channels (null: the kernel reads the channel planes)
+    const T* xi; const T* ti;
     // backward only
     // gradients are accumulated in the computation type (fp32 for bfloat16 features)
     const T* gy; typename Num<T>::acc* gx; int64_t ldgx; typename Num<T>::acc* gtree; int64_t ldgt;

@@ -358,9 +358,83 @@ __device__ __forceinline__ void store_items_bf16(const ItemRegs<G, bf16_t, BF_CI
     }
 }
 
+// ---- regrouped input: [Cin / 8][count][8] bfloat16 -----------------------------------------------------------
+// A sparse row inside a window holds few particles, so a gather of one 2-byte channel value per lane touches
+// about twenty cache lines per wave and the kernel waits for memory two thirds of the time.  With the 8 channels
+// of a group next to each other an item is ONE 16-byte load per round of staging instead of eight 2-byte loads
+// through eight descriptors: an eighth of the load instructions, a quarter of the value registers, two
+// descriptors instead of sixteen.  The regrouping is one streaming pass over the input (interleave8_kernel).
+typedef int intx4 __attribute__((ext_vector_type(4)));
+template <class G, int IPT>
+struct ItemRegs16 { intx4 v[IPT]; unsigned off[IPT]; unsigned short pos[IPT]; };
+
+template <class G, int IPT, class Lists>
+__device__ __forceinline__ void fetch_slots16(const Lists& sh, int nitem, ItemRegs16<G, IPT>& R) {
+#pragma unroll
+    for (int k = 0; k < IPT; ++k) {
+        R.pos[k] = 0xffffu; R.off[k] = BUF_OOB;
+        if (k * G::NT >= nitem) continue;               // wave-uniform
+        const int it = threadIdx.x + k * G::NT;
+        if (it < nitem) { R.pos[k] = sh.item_pos[it]; R.off[k] = (unsigned)sh.item_idx[it] * 16u; }
+    }
+}
+template <class G, int IPT>
+__device__ __forceinline__ void load_values16(const ConvArgs<bf16_t>& a, int ci0, int nitem, bool tree_items, ItemRegs16<G, IPT>& R) {
+    const int q = ci0 / BF_CIB;
+    const __amdgpu_buffer_rsrc_t rx = __builtin_amdgcn_make_buffer_rsrc(const_cast<bf16_t*>(a.xi + (int64_t)q * a.x_count * BF_CIB), 0,
+                                                                        (int)(a.x_count * 16), 0x00020000);
+    const __amdgpu_buffer_rsrc_t rt = __builtin_amdgcn_make_buffer_rsrc(const_cast<bf16_t*>(a.ti + (int64_t)q * a.t_count * BF_CIB), 0,
+                                                                        tree_items ? (int)(a.t_count * 16) : 0, 0x00020000);
+#pragma unroll
+    for (int k = 0; k < IPT; ++k) {
+        if (k * G::NT >= nitem) break;                  // wave-uniform
+        const bool from_tree = (R.pos[k] & ITEM_TREE) != 0 && R.pos[k] != 0xffffu;
+        if (tree_items) {
+            if (from_tree) {
+                R.v[k] = __builtin_amdgcn_raw_buffer_load_b128(rt, (int)R.off[k], 0, 0);
+                asm volatile("" ::: "memory");          // keeps the two branches from being merged into one load with a per-lane descriptor
+            } else {
+                R.v[k] = __builtin_amdgcn_raw_buffer_load_b128(rx, (int)R.off[k], 0, 0);
+            }
+        } else {
+            R.v[k] = __builtin_amdgcn_raw_buffer_load_b128(rx, (int)R.off[k], 0, 0);
+        }
+    }
+}
+template <class G, int IPT>
+__device__ __forceinline__ void store_items16(const ItemRegs16<G, IPT>& R, int nitem, uint2* __restrict__ patch8) {
+#pragma unroll
+    for (int k = 0; k < IPT; ++k) {
+        if (k * G::NT >= nitem) break;                  // wave-uniform
+        if (R.pos[k] == 0xffffu) continue;
+        uint2* cell = patch8 + (R.pos[k] & ITEM_CELL);
+        const uint2 v0 = make_uint2((unsigned)R.v[k][0], (unsigned)R.v[k][1]), v1 = make_uint2((unsigned)R.v[k][2], (unsigned)R.v[k][3]);
+        cell[0] = v0; cell[G::CH_STRIDE] = v1;
+        if (R.pos[k] & ITEM_PAIR) { cell[1] = v0; cell[G::CH_STRIDE + 1] = v1; }
+    }
+}
+
+// out[q][i][c] = channel 8 q + c of element i; channels from c_split on come from x2 (null: all from x), channels
+// past C read as zeros.  One thread per (element, group): eight 2-byte reads along the planes, one 16-byte write.
+__global__ void interleave8_kernel(const bf16_t* __restrict__ x, int64_t ldx, const bf16_t* __restrict__ x2, int64_t ldx2, int c_split,
+                                   int C, int64_t count, bf16_t* __restrict__ out) {
+    const int q = blockIdx.y;
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < count; i += (int64_t)gridDim.x * blockDim.x) {
+        unsigned v[BF_CIB];
+#pragma unroll
+        for (int c = 0; c < BF_CIB; ++c) {
+            const int ch = q * BF_CIB + c;
+            v[c] = 0u;
+            if (ch < C) v[c] = (x2 != nullptr && ch >= c_split) ? x2[(int64_t)(ch - c_split) * ldx2 + i].bits : x[(int64_t)ch * ldx + i].bits;
+        }
+        reinterpret_cast<uint4*>(out)[(int64_t)q * count + i] = make_uint4(v[0] | (v[1] << 16), v[2] | (v[3] << 16), v[4] | (v[5] << 16), v[6] | (v[7] << 16));
+    }
+}
+
 // MODE 0: forward.  MODE 1: input gradient (items = output gradient, results added atomically in fp32 to the place
 // each column names, as in the fp32 kernel; no pooled columns).
-template <class G, int COH, int NB, bool FUSE, int MODE, class Lists>
+// IL: the input comes regrouped (a.xi, a.ti), see above
+template <class G, int COH, int NB, bool FUSE, int MODE, bool IL, class Lists>
 __device__ __forceinline__ void mfma_bf16_window(const ConvArgs<bf16_t>& a, int co0, int nc, int nitem, bool tree_items, int first,
                                                  const uint4* __restrict__ wl, const Lists& sh,
                                                  uint2* __restrict__ patch8, uint2* __restrict__ Wl8,
@@ -386,7 +460,7 @@ __device__ __forceinline__ void mfma_bf16_window(const ConvArgs<bf16_t>& a, int 
 
     constexpr int W16 = NSTEP * COH * 32;                        // 16-byte elements of a weight chunk
     constexpr int WPT = (W16 + G::NT - 1) / G::NT;
-    ItemRegs<G, bf16_t, BF_CIB> R;
+    typename std::conditional<IL, ItemRegs16<G, ItemRegs<G, bf16_t, BF_CIB>::IPT>, ItemRegs<G, bf16_t, BF_CIB>>::type R;
     uint4 wr[WPT];
 #define APRNET_LOAD_WEIGHTS(q)                                                                     \
     _Pragma("unroll") for (int k = 0; k < WPT; ++k) {                                              \
@@ -398,17 +472,19 @@ __device__ __forceinline__ void mfma_bf16_window(const ConvArgs<bf16_t>& a, int 
         const int i = threadIdx.x + k * G::NT;                                                     \
         if (i < W16) reinterpret_cast<uint4*>(Wl8)[i] = wr[k];                                     \
     }
-    load_items<G, bf16_t, BF_CIB>(a, 0, nitem, tree_items, sh, R, 0, std::bool_constant<FUSE>{});
+    if constexpr (IL) { fetch_slots16<G>(sh, nitem, R); load_values16<G>(a, 0, nitem, tree_items, R); }
+    else load_items<G, bf16_t, BF_CIB>(a, 0, nitem, tree_items, sh, R, 0, std::bool_constant<FUSE>{});
     APRNET_LOAD_WEIGHTS(0)
     for (int i = threadIdx.x; i < 2 * G::CH_STRIDE; i += G::NT) patch8[i] = make_uint2(0u, 0u);     // once per window
     for (int ci0 = 0; ci0 < a.Cin; ci0 += BF_CIB) {
         __syncthreads();
         // items -> patch: two 8-byte cells (channel groups) per item, four bfloat16 each
-        store_items_bf16<G>(R, nitem, patch8);
+        if constexpr (IL) store_items16<G>(R, nitem, patch8); else store_items_bf16<G>(R, nitem, patch8);
         APRNET_STORE_WEIGHTS()
         __syncthreads();
         if (ci0 + BF_CIB < a.Cin) {
-            load_values<G, bf16_t, BF_CIB>(a, ci0 + BF_CIB, nitem, tree_items, R, 0, std::bool_constant<FUSE>{});
+            if constexpr (IL) load_values16<G>(a, ci0 + BF_CIB, nitem, tree_items, R);
+            else load_values<G, bf16_t, BF_CIB>(a, ci0 + BF_CIB, nitem, tree_items, R, 0, std::bool_constant<FUSE>{});
             APRNET_LOAD_WEIGHTS(ci0 / BF_CIB + 1)
         }
 #pragma unroll
@@ -461,7 +537,7 @@ __device__ __forceinline__ void mfma_bf16_window(const ConvArgs<bf16_t>& a, int 
 }
 
 // The windows of the tile come as precomputed lists from the plan.
-template <class G, int COH, bool FUSE = false, int MODE = 0>
+template <class G, int COH, bool FUSE = false, int MODE = 0, bool IL = false>
 __global__ void __launch_bounds__(G::NT) __attribute__((amdgpu_waves_per_eu(4, 4)))      // two workgroups per CU
 conv_mfma_bf16_kernel(const ConvArgs<bf16_t> a) {
     constexpr int NBW = 4, NSTEP = bf16_steps<G>();
@@ -495,11 +571,11 @@ conv_mfma_bf16_kernel(const ConvArgs<bf16_t> a) {
         const int first = (wave - (int)blockIdx.x - win) & (G::NWAVE - 1);
         const int nb = first < nblk ? (nblk - first + G::NWAVE - 1) / G::NWAVE : 0;
         switch (__builtin_amdgcn_readfirstlane(nb)) {
-            case 0: mfma_bf16_window<G, COH, 0, FUSE, MODE>(a, co0, nc, nitem, tree_items, first, wl, gl, patch8, Wl8, bias_l); break;
-            case 1: mfma_bf16_window<G, COH, 1, FUSE, MODE>(a, co0, nc, nitem, tree_items, first, wl, gl, patch8, Wl8, bias_l); break;
-            case 2: mfma_bf16_window<G, COH, 2, FUSE, MODE>(a, co0, nc, nitem, tree_items, first, wl, gl, patch8, Wl8, bias_l); break;
-            case 3: mfma_bf16_window<G, COH, 3, FUSE, MODE>(a, co0, nc, nitem, tree_items, first, wl, gl, patch8, Wl8, bias_l); break;
-            default: mfma_bf16_window<G, COH, 4, FUSE, MODE>(a, co0, nc, nitem, tree_items, first, wl, gl, patch8, Wl8, bias_l); break;
+            case 0: mfma_bf16_window<G, COH, 0, FUSE, MODE, IL>(a, co0, nc, nitem, tree_items, first, wl, gl, patch8, Wl8, bias_l); break;
+            case 1: mfma_bf16_window<G, COH, 1, FUSE, MODE, IL>(a, co0, nc, nitem, tree_items, first, wl, gl, patch8, Wl8, bias_l); break;
+            case 2: mfma_bf16_window<G, COH, 2, FUSE, MODE, IL>(a, co0, nc, nitem, tree_items, first, wl, gl, patch8, Wl8, bias_l); break;
+            case 3: mfma_bf16_window<G, COH, 3, FUSE, MODE, IL>(a, co0, nc, nitem, tree_items, first, wl, gl, patch8, Wl8, bias_l); break;
+            default: mfma_bf16_window<G, COH, 4, FUSE, MODE, IL>(a, co0, nc, nitem, tree_items, first, wl, gl, patch8, Wl8, bias_l); break;
         }
         __syncthreads();        // the next window rewrites the patch
     }
@@ -562,6 +638,12 @@ static int launch_bf16(const ConvArgs<bf16_t>& a, int n_tiles, hipStream_t st, b
     if (dx) {
         if (coh == 1) hipLaunchKernelGGL((conv_mfma_bf16_kernel<G, 1, false, 1>), grid, dim3(G::NT), 0, st, a);
         else hipLaunchKernelGGL((conv_mfma_bf16_kernel<G, 2, false, 1>), grid, dim3(G::NT), 0, st, a);
+    } else if (a.xi != nullptr) {          // regrouped input (the second tensor is already part of it)
+        if (a.relu) {
+            if (coh == 1) hipLaunchKernelGGL((conv_mfma_bf16_kernel<G, 1, true, 0, true>), grid, dim3(G::NT), 0, st, a);
+            else hipLaunchKernelGGL((conv_mfma_bf16_kernel<G, 2, true, 0, true>), grid, dim3(G::NT), 0, st, a);
+        } else if (coh == 1) hipLaunchKernelGGL((conv_mfma_bf16_kernel<G, 1, false, 0, true>), grid, dim3(G::NT), 0, st, a);
+        else hipLaunchKernelGGL((conv_mfma_bf16_kernel<G, 2, false, 0, true>), grid, dim3(G::NT), 0, st, a);
     } else if (a.relu || a.x2) {
         if (coh == 1) hipLaunchKernelGGL((conv_mfma_bf16_kernel<G, 1, true>), grid, dim3(G::NT), 0, st, a);
         else hipLaunchKernelGGL((conv_mfma_bf16_kernel<G, 2, true>), grid, dim3(G::NT), 0, st, a);
@@ -587,6 +669,15 @@ int launch_conv_dx_mfma_bf16(int code, const ConvArgs<bf16_t>& a, int n_tiles, h
         case 155: return launch_bf16<M155N>(a, n_tiles, st, true);
     }
     return fail(APRNET_ERR_UNSUPPORTED, "no matrix-core kernel for this stencil");
+}
+// x (and x2 from channel c_split on) -> out[(C + 7) / 8][count][8]
+int interleave8_bf16(const bf16_t* x, int64_t ldx, const bf16_t* x2, int64_t ldx2, int c_split, int C, int64_t count, bf16_t* out,
+                     hipStream_t st) {
+    if (count <= 0 || C <= 0) return 0;
+    dim3 grid((unsigned)std::min<int64_t>((count + 255) / 256, 1 << 20), (unsigned)((C + BF_CIB - 1) / BF_CIB));
+    hipLaunchKernelGGL(interleave8_kernel, grid, dim3(256), 0, st, x, ldx, x2, ldx2, c_split, C, count, out);
+    APRNET_LAUNCH_CHECK("interleave8_kernel");
+    return 0;
 }
 size_t conv_packed_bf16_bytes(int code, int S_exp, int Cout, int Cin) {
     const int coh = conv_coh(Cout), nstep = (conv_taps(code) + 1) / 2;

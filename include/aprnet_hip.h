@@ -84,7 +84,10 @@ int aprnet_profile_enable(int on);
  * use and keeps (about 20 bytes of device memory per particle and level delta; default), 5 = scan the access arrays
  * in every call (also the fallback when the lists cannot be allocated); and for the backward matrix-core kernels:
  * 6 = the weight gradient runs on a second stream of the plan next to the input gradient, forked from and joined
- * to the caller's stream with events (default), 7 = both on the caller's stream.  All are HIP kernels; the switch
+ * to the caller's stream with events (default), 7 = both on the caller's stream; and for the bfloat16 forward
+ * kernel: 8 = stage from a copy of the input regrouped as [Cin / 8][particles][8] in the plan's scratch buffer, one
+ * 16-byte load per item and 8 channels (default; 16 bytes per particle and 8 channels of device memory, made by one
+ * streaming pass per call), 9 = gather from the channel planes.  All are HIP kernels; the switch
  * exists so that tests can cover them and memory-bound callers can do without the lists. */
 int aprnet_set_conv_path(int path);
 float aprnet_profile_last_ms(void);
