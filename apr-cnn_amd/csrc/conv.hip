@@ -148,9 +148,11 @@ int pack_conv_weights(int code, const float* w, int S_exp, int Cm, int Ck, bool 
 static int g_conv_path = 0;      // 0: matrix cores where available, 1: VALU kernels only
 int conv_path() { return g_conv_path; }
 int bf16_math();
+int bf16_regroup();
 
 static int g_use_lists = 1;      // 1: forward kernels take the window lists of the plan, 0: they scan per call
 int bf16_math() { return g_bf16_math; }
+int bf16_regroup() { return g_bf16_regroup; }
 static int g_bwd_overlap = 1;    // backward: weight gradient on a second stream next to the input gradient
 int backward_overlap() { return g_bwd_overlap; }
 
@@ -278,7 +280,7 @@ int conv_fwd_bf16(const aprnet_plan* cp, int d, int kz, int kx, int ky, const bf
         // 16-byte items stay addressable with 32-bit offsets and the copy stays below 32 GiB.
         const size_t wbytes = (conv_packed_bf16_bytes(code, S_exp, Cout, Cin) + 255) / 256 * 256;
         const size_t ng = (size_t)(Cin + 7) / 8, ibytes = ng * (size_t)(n_x + n_t) * 16;
-        const bool regroup = g_bf16_regroup && n_x < (1ll << 28) && n_t < (1ll << 28) && ibytes <= ((size_t)32 << 30);
+        const bool regroup = bf16_regroup() && n_x < (1ll << 28) && n_t < (1ll << 28) && ibytes <= ((size_t)32 << 30);
         if (int rc = plan_scratch(p, wbytes + (regroup ? ibytes : 0), st)) return rc;
         if (int rc = pack_conv_weights_bf16(code, w, S_exp, Cout, Cin, p->d_scratch, st)) return rc;
         if (regroup) {

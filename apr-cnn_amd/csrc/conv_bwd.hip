@@ -244,6 +244,9 @@ int set_conv_dx_lists(aprnet_plan* p, int d, int code, const TileList& tl, ConvA
 int launch_conv_dx_mfma_bf16(int code, const ConvArgs<bf16_t>& a, int n_tiles, hipStream_t st);
 size_t conv_packed_bf16_bytes(int code, int S_exp, int Cout, int Cin);
 int pack_conv_weights_bf16(int code, const float* w, int S_exp, int Cout, int Cin, void* packed, hipStream_t st, bool transposed);
+int interleave8_bf16(const bf16_t* x, int64_t ldx, const bf16_t* x2, int64_t ldx2, int c_split, int C, int64_t count, bf16_t* out,
+                     hipStream_t st);
+int bf16_regroup();
 int bf16_math();
 
 template <typename T> static int try_mfma_bwd(aprnet_plan*, const ConvArgs<T>&, const TileList&, int, int, hipStream_t, bool*) { return 0; }
@@ -399,8 +402,17 @@ int conv_bwd_bf16(const aprnet_plan* cp, int d, int kz, int kx, int ky, const bf
         if (near.n > 0 && bf16_math())
             if (int rc = set_conv_dx_lists(p, d, code, near, b, st)) return rc;
         if (near.n > 0 && b.tile_win) {
-            if (int rc = plan_scratch(p, conv_packed_bf16_bytes(code, S_exp, Cin, Cout), st)) return rc;
+            // the output gradient regrouped as [Cout / 8][particles][8] behind the packed weights, as in the forward pass
+            const size_t wbytes = (conv_packed_bf16_bytes(code, S_exp, Cin, Cout) + 255) / 256 * 256;
+            const size_t ng = (size_t)(Cout + 7) / 8, ibytes = ng * (size_t)np * 16;
+            const bool regroup = bf16_regroup() && np < (1ll << 28) && ibytes <= ((size_t)32 << 30);
+            if (int rc = plan_scratch(p, wbytes + (regroup ? ibytes : 0), st)) return rc;
             if (int rc = pack_conv_weights_bf16(code, w, S_exp, Cin, Cout, p->d_scratch, st, true)) return rc;
+            if (regroup) {
+                bf16_t* gyi = (bf16_t*)((char*)p->d_scratch + wbytes);
+                if (int rc = interleave8_bf16(gy, ldy, nullptr, 0, Cout, Cout, np, gyi, st)) return rc;
+                b.xi = gyi; b.ti = nullptr;
+            }
             b.w = (const float*)p->d_scratch;
             if (int rc = launch_conv_dx_mfma_bf16(code, b, near.n, st)) return rc;
         } else if (near.n > 0) {

@@ -635,7 +635,10 @@ template <class G>
 static int launch_bf16(const ConvArgs<bf16_t>& a, int n_tiles, hipStream_t st, bool dx = false) {
     const int coh = conv_coh(a.Cout);
     dim3 grid((unsigned)n_tiles, (unsigned)((a.Cout + 16 * coh - 1) / (16 * coh)));
-    if (dx) {
+    if (dx && a.xi != nullptr) {           // regrouped output gradient
+        if (coh == 1) hipLaunchKernelGGL((conv_mfma_bf16_kernel<G, 1, false, 1, true>), grid, dim3(G::NT), 0, st, a);
+        else hipLaunchKernelGGL((conv_mfma_bf16_kernel<G, 2, false, 1, true>), grid, dim3(G::NT), 0, st, a);
+    } else if (dx) {
         if (coh == 1) hipLaunchKernelGGL((conv_mfma_bf16_kernel<G, 1, false, 1>), grid, dim3(G::NT), 0, st, a);
         else hipLaunchKernelGGL((conv_mfma_bf16_kernel<G, 2, false, 1>), grid, dim3(G::NT), 0, st, a);
     } else if (a.xi != nullptr) {          // regrouped input (the second tensor is already part of it)
