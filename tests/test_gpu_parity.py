@@ -565,6 +565,44 @@ def test_conv_forward_fused_relu_and_second_input(ksize, c1, c2, cout, dtype, pa
         assert torch.equal(got, torch.relu(plain))
 
 
+@pytest.mark.parametrize("ksize,c1,c2,cout", [((3, 3, 3), 16, 16, 16), ((3, 3, 3), 5, 6, 33), ((1, 5, 5), 7, 3, 20),
+                                              ((1, 3, 3), 1, 0, 8)], ids=lambda v: KID(v) if isinstance(v, tuple) else str(v))
+def test_conv_bf16_regrouped_input_equals_channel_planes(ksize, c1, c2, cout):
+    """bfloat16 stencil convolutions stage from a copy of the input regrouped as [Cin / 8][particles][8]
+    (aprnet_set_conv_path(8), the default) or gather from the channel planes (9).  Same values, same products, same
+    order of accumulation: the forward results (with and without a second input tensor and the clamp) are
+    bit-identical, and so is the oracle check; the backward's input gradient (fp32 atomics) agrees to rounding."""
+    bt = [("3d_b", 1), ("3d_c", 0)]
+    x, aprs, ld, w_exp = _conv_case(bt, ksize, 2, c1 + c2, cout, torch.float32)
+    x = x.to(torch.bfloat16)
+    g = torch.Generator().manual_seed(7)
+    bias = torch.randn(cout, generator=g)
+    ref = torch.relu(oracle.conv_forward(aprs, x.float(), w_exp, ld) + bias.view(1, -1, 1))
+    xa = x[:, :c1].contiguous().to(DEV)
+    xb = x[:, c1:].contiguous().to(DEV) if c2 else None
+    wd = w_exp.permute(1, 2, 0, 3, 4, 5).contiguous().to(DEV)
+    go = torch.randn(x.shape[0], cout, x.shape[2], generator=g).to(torch.bfloat16).to(DEV)
+    lib = _native.hip()
+    res = {}
+    try:
+        for path in (8, 9):
+            assert lib.aprnet_set_conv_path(path) == 0
+            fused = _ops.conv_forward(aprs, xa, wd, ld, bias.to(DEV), relu=True, x2=xb)
+            plain = _ops.conv_forward(aprs, x.to(DEV), wd, ld, bias.to(DEV))
+            gx, gw = _ops.conv_backward(aprs, x.to(DEV), wd, go, ld)
+            torch.cuda.synchronize()
+            res[path] = (fused, plain, gx, gw)
+    finally:
+        lib.aprnet_set_conv_path(8)
+    close_bf16(res[8][0], ref)
+    assert torch.equal(res[8][0], res[9][0]) and torch.equal(res[8][1], res[9][1])
+    assert torch.equal(res[8][0], torch.relu(res[8][1]))
+    scale = float(res[9][2].float().abs().max())
+    assert float((res[8][2].float() - res[9][2].float()).abs().max()) <= 1e-2 * scale      # one bfloat16 rounding step
+    assert float((res[8][3] - res[9][3]).abs().max()) <= 1e-5 * float(res[9][3].abs().max())
+    assert lib.aprnet_set_conv_path(10) != 0
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float64, torch.bfloat16], ids=["f32", "f64", "bf16"])
 def test_conv111_forward_fused_relu(dtype):
     cdt = torch.float32 if dtype == torch.bfloat16 else dtype
