@@ -96,6 +96,10 @@ struct aprnet_plan {
     int64_t n_tree = 0, n_apr = 0;
     std::map<std::tuple<int, int, int, int>, aprnet::TileList> tiles;   // (level_delta, TZ, TX, halo) -> row groups
     void* d_scratch = nullptr; size_t scratch_bytes = 0;          // re-laid-out weights of the call in flight
+    bool scratch_in_graph = false;                                // the buffer was handed out while its stream was capturing
+    std::vector<void*> retired;                                   // outgrown buffers that a captured graph may address: freed at destroy
+    hipStream_t scratch_stream = nullptr;                         // stream of the last call that used the buffer
+    bool scratch_stream_valid = false, scratch_stream_capturing = false;
     std::map<std::pair<int, int>, aprnet::WinLists> lists;        // (level_delta, stencil code) -> window lists
     // second stream of the convolution backward (weight gradient next to input gradient), with its fork / join events
     hipStream_t side = nullptr; hipEvent_t ev_fork = nullptr, ev_join = nullptr;
@@ -117,10 +121,17 @@ void set_error(const std::string& msg);
 int fail(int code, const std::string& msg);
 // non-empty row groups for the convolution at `level_delta` (built on first use, cached in the plan)
 // `halo` > 0 also lists the row groups that lie within that many rows of a non-empty one
-int get_tiles(aprnet_plan* plan, int level_delta, int TZ, int TX, TileList* out, int halo = 0);
+// (allocates and copies on first use: refused with APRNET_ERR_UNSUPPORTED while `st` is capturing)
+int get_tiles(aprnet_plan* plan, int level_delta, int TZ, int TX, TileList* out, hipStream_t st, int halo = 0);
+// true while `st` records into a graph (allocation, synchronous copies and stream synchronisation are not allowed then)
+bool stream_is_capturing(hipStream_t st);
 int get_lists(aprnet_plan* plan, int level_delta, int code, const TileList& tl, WinLists* out, hipStream_t st, bool dx = false);
 void free_lists(WinLists& wl);
-// makes plan->d_scratch at least `bytes` large (contents are lost when it grows)
+// Makes plan->d_scratch at least `bytes` large for a call on `st` (contents are lost when it grows).  A buffer that a
+// captured graph may address is never freed before the plan is destroyed; growth while `st` is capturing is refused
+// with APRNET_ERR_UNSUPPORTED (reserve first: aprnet_plan_reserve, or run the call once outside the capture).  A call on
+// another stream than the previous one first waits for that stream, so that two streams cannot overwrite each other's
+// packed weights (under capture the caller must have ordered the streams, as for any input of the graph).
 int plan_scratch(aprnet_plan* plan, size_t bytes, hipStream_t st);
 
 #define APRNET_HIP_CHECK(expr)                                                                                  \

@@ -228,7 +228,7 @@ int conv_fwd(const aprnet_plan* cp, int d, int kz, int kx, int ky, const T* x, i
         if (int rc = fill_tree_for_conv(p, d, fu.x2, fu.ldx2, fu.C2, tree_ws + (int64_t)C1 * ldt, ldt, st)) return rc;
     const bool flat = (kz == 1);
     TileList tl;
-    if (int rc = get_tiles(p, d, flat ? 1 : 2, flat ? 8 : 4, &tl)) return rc;
+    if (int rc = get_tiles(p, d, flat ? 1 : 2, flat ? 8 : 4, &tl, st)) return rc;
     if (tl.n == 0) return 0;
     ConvArgs<T> a{};
     a.apr = p->dapr; a.tree = p->dtree; a.tiles = tl.d_tiles;
@@ -269,7 +269,7 @@ int conv_fwd_bf16(const aprnet_plan* cp, int d, int kz, int kx, int ky, const bf
     if (fu.C2 > 0)
         if (int rc = fill_tree_for_conv(p, d, fu.x2, fu.ldx2, fu.C2, tree_ws + (int64_t)C1 * ldt, ldt, st)) return rc;
     TileList tl;
-    if (int rc = get_tiles(p, d, kz == 1 ? 1 : 2, kz == 1 ? 8 : 4, &tl)) return rc;
+    if (int rc = get_tiles(p, d, kz == 1 ? 1 : 2, kz == 1 ? 8 : 4, &tl, st)) return rc;
     if (tl.n == 0) return 0;
     ConvArgs<bf16_t> a{};
     if (int rc = set_lists(p, d, code, tl, a, st)) return rc;

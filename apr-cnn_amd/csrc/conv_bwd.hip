@@ -252,21 +252,33 @@ int bf16_math();
 template <typename T> static int try_mfma_bwd(aprnet_plan*, const ConvArgs<T>&, const TileList&, int, int, hipStream_t, bool*) { return 0; }
 static int fork_side(aprnet_plan* p, hipStream_t st, hipStream_t* side);
 static int join_side(aprnet_plan* p, hipStream_t st, hipStream_t side);
+// Joins the side stream on every way out of a backward call, also the failing ones: the caller's stream must not run
+// ahead of a weight-gradient kernel that still reads the caller's tensors, and a capture must not end with an open fork.
+struct SideJoin {
+    aprnet_plan* p; hipStream_t st, side; bool open = true;
+    SideJoin(aprnet_plan* p_, hipStream_t st_, hipStream_t side_) : p(p_), st(st_), side(side_) {}
+    int join() { open = false; return join_side(p, st, side); }
+    ~SideJoin() { if (open) (void)join_side(p, st, side); }
+};
 template <> int try_mfma_bwd<float>(aprnet_plan* p, const ConvArgs<float>& a, const TileList& tl, int code, int d, hipStream_t st, bool* done) {
     if (conv_path() == 1 || !conv_mfma_supported(code)) return 0;
     *done = true;
     // weight gradient on the side stream (when there is an input gradient to run next to)
     ConvArgs<float> c = a;
     if (int rc = set_conv_lists(p, d, code, tl, c, st)) return rc;
+    // everything that can allocate or fail on the host comes before the fork
+    TileList near;
+    if (a.gx) {
+        if (int rc = get_tiles(p, d, code == 333 ? 2 : 1, code == 333 ? 4 : 8, &near, st, 1)) return rc;
+        if (int rc = plan_scratch(p, conv_packed_floats(code, a.S_exp, a.Cin, a.Cout, true) * sizeof(float), st)) return rc;
+    }
     hipStream_t side = st;
     if (a.gx) if (int rc = fork_side(p, st, &side)) return rc;
+    SideJoin guard(p, st, side);
     if (int rc = launch_conv_dw_mfma(code, c, tl, p->apr.level_min, side)) return rc;
     if (a.gx) {
         // input gradient: the forward kernel on the output gradient with the transposed, flipped stencil;
         // every row group within one row of an output takes part
-        TileList near;
-        if (int rc = get_tiles(p, d, code == 333 ? 2 : 1, code == 333 ? 4 : 8, &near, 1)) return rc;
-        if (int rc = plan_scratch(p, conv_packed_floats(code, a.S_exp, a.Cin, a.Cout, true) * sizeof(float), st)) return rc;
         if (int rc = pack_conv_weights(code, a.w, a.S_exp, a.Cin, a.Cout, true, (float*)p->d_scratch, st)) return rc;
         ConvArgs<float> b = a;
         b.tiles = near.d_tiles; b.n_tiles = near.n;
@@ -274,7 +286,7 @@ template <> int try_mfma_bwd<float>(aprnet_plan* p, const ConvArgs<float>& a, co
         b.tree_data = nullptr; b.t_count = 0;
         if (near.n > 0) if (int rc = launch_conv_dx_mfma(code, b, near.n, st)) return rc;
     }
-    return join_side(p, st, side);
+    return guard.join();
 }
 
 // Fork / join around the two halves of the backward pass: what follows fork() on the returned stream runs next to
@@ -325,7 +337,7 @@ int conv_bwd(const aprnet_plan* cp, int d, int kz, int kx, int ky, const T* x, i
     }
     const bool flat = (kz == 1);
     TileList tl;
-    if (int rc = get_tiles(p, d, flat ? 1 : 2, flat ? 8 : 4, &tl)) return rc;
+    if (int rc = get_tiles(p, d, flat ? 1 : 2, flat ? 8 : 4, &tl, st)) return rc;
     if (tl.n > 0) {
         ConvArgs<T> a{};
         a.apr = p->dapr; a.tree = p->dtree; a.tiles = tl.d_tiles; a.n_tiles = tl.n;
@@ -378,8 +390,8 @@ int conv_bwd_bf16(const aprnet_plan* cp, int d, int kz, int kx, int ky, const bf
     }
     const bool flat = (kz == 1);
     TileList tl, near;
-    if (int rc = get_tiles(p, d, flat ? 1 : 2, flat ? 8 : 4, &tl)) return rc;
-    if (int rc = get_tiles(p, d, flat ? 1 : 2, flat ? 8 : 4, &near, 1)) return rc;
+    if (int rc = get_tiles(p, d, flat ? 1 : 2, flat ? 8 : 4, &tl, st)) return rc;
+    if (int rc = get_tiles(p, d, flat ? 1 : 2, flat ? 8 : 4, &near, st, 1)) return rc;
     if (tl.n > 0) {
         ConvArgs<bf16_t> a{};
         a.apr = p->dapr; a.tree = p->dtree; a.tiles = tl.d_tiles; a.n_tiles = tl.n;
@@ -396,17 +408,22 @@ int conv_bwd_bf16(const aprnet_plan* cp, int d, int kz, int kx, int ky, const bf
         if (!gx) near.n = 0;              // no input gradient asked for
         // weight gradient on the side stream, next to the input gradient
         if (int rc = set_conv_lists(p, d, code, tl, a, st)) return rc;
-        hipStream_t side = st;
-        if (near.n > 0) if (int rc = fork_side(p, st, &side)) return rc;
-        if (int rc = launch_conv_dw_mfma(code, a, tl, p->apr.level_min, side)) return rc;
+        // everything that can allocate or fail on the host comes before the fork
         if (near.n > 0 && bf16_math())
             if (int rc = set_conv_dx_lists(p, d, code, near, b, st)) return rc;
+        const size_t wbytes = (conv_packed_bf16_bytes(code, S_exp, Cin, Cout) + 255) / 256 * 256;
+        const size_t ng = (size_t)(Cout + 7) / 8, ibytes = ng * (size_t)np * 16;
+        const bool regroup = bf16_regroup() && np < (1ll << 28) && ibytes <= ((size_t)32 << 30);
+        if (near.n > 0) {
+            const size_t need = b.tile_win ? wbytes + (regroup ? ibytes : 0) : conv_packed_floats(code, S_exp, Cin, Cout, true) * sizeof(float);
+            if (int rc = plan_scratch(p, need, st)) return rc;
+        }
+        hipStream_t side = st;
+        if (near.n > 0) if (int rc = fork_side(p, st, &side)) return rc;
+        SideJoin guard(p, st, side);
+        if (int rc = launch_conv_dw_mfma(code, a, tl, p->apr.level_min, side)) return rc;
         if (near.n > 0 && b.tile_win) {
             // the output gradient regrouped as [Cout / 8][particles][8] behind the packed weights, as in the forward pass
-            const size_t wbytes = (conv_packed_bf16_bytes(code, S_exp, Cin, Cout) + 255) / 256 * 256;
-            const size_t ng = (size_t)(Cout + 7) / 8, ibytes = ng * (size_t)np * 16;
-            const bool regroup = bf16_regroup() && np < (1ll << 28) && ibytes <= ((size_t)32 << 30);
-            if (int rc = plan_scratch(p, wbytes + (regroup ? ibytes : 0), st)) return rc;
             if (int rc = pack_conv_weights_bf16(code, w, S_exp, Cin, Cout, p->d_scratch, st, true)) return rc;
             if (regroup) {
                 bf16_t* gyi = (bf16_t*)((char*)p->d_scratch + wbytes);
@@ -416,13 +433,12 @@ int conv_bwd_bf16(const aprnet_plan* cp, int d, int kz, int kx, int ky, const bf
             b.w = (const float*)p->d_scratch;
             if (int rc = launch_conv_dx_mfma_bf16(code, b, near.n, st)) return rc;
         } else if (near.n > 0) {
-            if (int rc = plan_scratch(p, conv_packed_floats(code, S_exp, Cin, Cout, true) * sizeof(float), st)) return rc;
             if (int rc = pack_conv_weights(code, w, S_exp, Cin, Cout, true, (float*)p->d_scratch, st)) return rc;
             b.w = (const float*)p->d_scratch;
             b.tile_win = nullptr;
             if (int rc = launch_conv_dx_mfma(code, b, near.n, st)) return rc;
         }
-        if (int rc = join_side(p, st, side)) return rc;
+        if (int rc = guard.join()) return rc;
     }
     if (!gx) return 0;
     if (int rc = fill_tree_bwd_for_conv(p, d, gx32_ws, ldgx32, Cin, gtree_ws, ldgt, st)) return rc;

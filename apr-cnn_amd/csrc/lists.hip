@@ -90,6 +90,9 @@ int get_lists(aprnet_plan* p, int level_delta, int code, const TileList& tl, Win
         *out = it->second;
         return it->second.unavailable ? fail(APRNET_ERR_UNSUPPORTED, "window lists are not available for this plan") : 0;
     }
+    if (stream_is_capturing(st))
+        return fail(APRNET_ERR_UNSUPPORTED, "window lists are built on the first call at a level delta (allocates and synchronises): "
+                                            "run it once before capturing the stream");
     WinLists wl{};
     WinLists none{}; none.unavailable = true;
     p->lists[key] = none;             // replaced below when the build succeeds

@@ -13,6 +13,16 @@ static thread_local std::string g_last_error;
 void set_error(const std::string& msg) { g_last_error = msg; }
 int fail(int code, const std::string& msg) { g_last_error = msg; return code; }
 
+template <class F>
+static void parallel_for(int n, F f, int serial_below = 64) {
+    const int nt = std::max(1u, std::min(16u, std::thread::hardware_concurrency()));
+    if (n < serial_below || nt == 1) { for (int i = 0; i < n; ++i) f(i); return; }
+    std::vector<std::thread> th;
+    for (int t = 0; t < nt; ++t)
+        th.emplace_back([=]() { for (int i = t; i < n; i += nt) f(i); });
+    for (auto& t : th) t.join();
+}
+
 static int copy_access(const aprnet_access_desc* d, HostAccess& h, int lmax_all) {
     if (!d || !d->z_num || !d->x_num || !d->y_num || !d->level_xz_vec || !d->xz_end_vec)
         return fail(APRNET_ERR_INVALID_ARGUMENT, "plan_create: null access array");
@@ -32,6 +42,41 @@ static int copy_access(const aprnet_access_desc* d, HostAccess& h, int lmax_all)
     // (conv entry points check the element size of the call, check_plane_size)
     if (d->n_particles >= (1ull << 30))
         return fail(APRNET_ERR_UNSUPPORTED, "plan_create: 2^30 or more particles per access");
+    if (d->n_particles && !d->y_vec) return fail(APRNET_ERR_INVALID_ARGUMENT, "plan_create: null y_vec with particles present");
+    // The arrays may come from a file: everything the kernels index with is checked here once, so that a damaged
+    // state is an error code and not an out-of-range access on the GPU.
+    for (int l = 0; l <= lmax_all; ++l)
+        if (h.z_num[l] < 1 || h.x_num[l] < 1 || h.y_num[l] < 1 || h.y_num[l] > 65536)
+            return fail(APRNET_ERR_INVALID_ARGUMENT, "plan_create: level dimensions must lie in 1..65536 (y) and be positive");
+    if (h.level_xz[d->level_min] < 1) return fail(APRNET_ERR_INVALID_ARGUMENT, "plan_create: level_xz_vec must leave the leading sentinel row");
+    for (int l = d->level_min; l <= d->level_max; ++l)
+        if (h.level_xz[l + 1] < h.level_xz[l] || h.level_xz[l + 1] - h.level_xz[l] != (uint64_t)h.z_num[l] * (uint64_t)h.x_num[l])
+            return fail(APRNET_ERR_INVALID_ARGUMENT, "plan_create: level_xz_vec does not match z_num * x_num of level " + std::to_string(l));
+    std::vector<int> bad_level(d->level_max + 1, 0);
+    for (int l = d->level_min; l <= d->level_max; ++l) {
+        const uint64_t r0 = h.level_xz[l], r1 = h.level_xz[l + 1];
+        const int yn = h.y_num[l];
+        const uint64_t* xz = h.xz_end.data();
+        const uint16_t* yv = d->y_vec;
+        const uint64_t n = d->n_particles;
+        std::vector<int> bad(16, 0);
+        parallel_for(16, [&](int t) {
+            for (uint64_t r = r0 + (uint64_t)t; r < r1; r += 16) {
+                const uint64_t b = xz[r - 1], e = xz[r];
+                if (e < b || e > n) { bad[t] = 1; return; }
+                for (uint64_t i = b; i < e; ++i)
+                    if ((int)yv[i] >= yn || (i > b && yv[i] <= yv[i - 1])) { bad[t] = 2; return; }
+            }
+        }, 1);
+        for (int t = 0; t < 16; ++t) bad_level[l] = std::max(bad_level[l], bad[t]);
+        if (bad_level[l] == 1)
+            return fail(APRNET_ERR_INVALID_ARGUMENT, "plan_create: xz_end_vec must be non-decreasing and end within n_particles (level " + std::to_string(l) + ")");
+        if (bad_level[l] == 2)
+            return fail(APRNET_ERR_INVALID_ARGUMENT, "plan_create: y_vec must ascend strictly within a row and stay below y_num (level " + std::to_string(l) + ")");
+    }
+    // rows below level_min (none by construction of level_xz_vec) and the sentinel hold no particles
+    if (h.xz_end[h.level_xz[d->level_min] - 1] != 0)
+        return fail(APRNET_ERR_INVALID_ARGUMENT, "plan_create: rows before level_min must be empty");
     if (d->n_particles) h.y.assign(d->y_vec, d->y_vec + d->n_particles);
     return 0;
 }
@@ -45,15 +90,6 @@ static void fill_dev(const HostAccess& h, AccessDev& d, const void* xz, const vo
     for (int l = h.level_max + 2; l <= MAX_LEVELS; ++l) d.level_xz[l] = h.level_xz[h.level_max + 1];
 }
 
-template <class F>
-static void parallel_for(int n, F f) {
-    const int nt = std::max(1u, std::min(16u, std::thread::hardware_concurrency()));
-    if (n < 64 || nt == 1) { for (int i = 0; i < n; ++i) f(i); return; }
-    std::vector<std::thread> th;
-    for (int t = 0; t < nt; ++t)
-        th.emplace_back([=]() { for (int i = t; i < n; i += nt) f(i); });
-    for (auto& t : th) t.join();
-}
 
 // children[s][t], s = 4*dz + 2*dx + dy: the merge walk of helpers.hpp:185-194 done once, from the
 // parents' side, for particles and for tree nodes.
@@ -101,19 +137,41 @@ static void build_children(const HostAccess& apr, const HostAccess& tree, std::v
     }
 }
 
+bool stream_is_capturing(hipStream_t st) {
+    hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(st, &cs) != hipSuccess) { (void)hipGetLastError(); return false; }
+    return cs != hipStreamCaptureStatusNone;
+}
+
 int plan_scratch(aprnet_plan* p, size_t bytes, hipStream_t st) {
-    if (bytes <= p->scratch_bytes) return 0;
-    if (p->d_scratch) { APRNET_HIP_CHECK(hipStreamSynchronize(st)); APRNET_HIP_CHECK(hipFree(p->d_scratch)); }
-    p->d_scratch = nullptr; p->scratch_bytes = 0;
-    APRNET_HIP_CHECK(hipMalloc(&p->d_scratch, bytes));
-    p->scratch_bytes = bytes;
+    const bool capturing = stream_is_capturing(st);
+    // a second stream takes the buffer over only after the first is done with it
+    if (p->scratch_stream_valid && p->scratch_stream != st && !p->scratch_stream_capturing && !capturing)
+        if (hipStreamSynchronize(p->scratch_stream) != hipSuccess) (void)hipGetLastError();     // a destroyed stream has no work left
+    p->scratch_stream = st; p->scratch_stream_valid = true; p->scratch_stream_capturing = capturing;
+    if (bytes > p->scratch_bytes) {
+        if (capturing)
+            return fail(APRNET_ERR_UNSUPPORTED, "the plan's scratch buffer would have to grow while the stream is capturing: call "
+                                                "aprnet_plan_reserve, or run this call once, before the capture");
+        if (p->d_scratch) {
+            if (p->scratch_in_graph) p->retired.push_back(p->d_scratch);     // a graph may replay into it: keep it until destroy
+            else { APRNET_HIP_CHECK(hipStreamSynchronize(st)); APRNET_HIP_CHECK(hipFree(p->d_scratch)); }
+        }
+        p->d_scratch = nullptr; p->scratch_bytes = 0; p->scratch_in_graph = false;
+        APRNET_HIP_CHECK(hipMalloc(&p->d_scratch, bytes));
+        p->scratch_bytes = bytes;
+    }
+    if (capturing) p->scratch_in_graph = true;
     return 0;
 }
 
-int get_tiles(aprnet_plan* plan, int level_delta, int TZ, int TX, TileList* out, int halo) {
+int get_tiles(aprnet_plan* plan, int level_delta, int TZ, int TX, TileList* out, hipStream_t st, int halo) {
     auto key = std::make_tuple(level_delta, TZ, TX, halo);
     auto it = plan->tiles.find(key);
     if (it != plan->tiles.end()) { *out = it->second; return 0; }
+    if (stream_is_capturing(st))
+        return fail(APRNET_ERR_UNSUPPORTED, "the first convolution at a level delta builds the plan's tile lists (allocates and "
+                                            "copies): run it once before capturing the stream");
     const HostAccess& apr = plan->apr; const HostAccess& tree = plan->tree;
     const int Lc = plan->lc(level_delta);
     std::vector<ConvTile> tiles;
@@ -171,11 +229,14 @@ int aprnet_plan_create(const aprnet_access_desc* apr, const aprnet_access_desc* 
     if (!rc) rc = copy_access(tree, p->tree, lmax_all);
     if (rc) { delete p; return rc; }
     p->n_apr = (int64_t)p->apr.n; p->n_tree = (int64_t)p->tree.n;
-    // per row y must ascend strictly: the staging code relies on it
+    // copy_access has checked that y ascends strictly per row: build_children and the staging code rely on it
     std::vector<int32_t> children;
     build_children(p->apr, p->tree, children);
 
-    APRNET_HIP_CHECK(hipSetDevice(device));
+    if (hipError_t e = hipSetDevice(device); e != hipSuccess) {
+        delete p;
+        return fail(APRNET_ERR_HIP, std::string("hipSetDevice: ") + hipGetErrorString(e));
+    }
     auto upload = [&](void** dst, const void* src, size_t bytes) -> int {
         APRNET_HIP_CHECK(hipMalloc(dst, std::max<size_t>(bytes, 16)));
         if (bytes) APRNET_HIP_CHECK(hipMemcpy(*dst, src, bytes, hipMemcpyHostToDevice));
@@ -201,6 +262,7 @@ void aprnet_plan_destroy(aprnet_plan* p) {
         if (q) (void)hipFree(q);
     for (auto& kv : p->tiles) if (kv.second.d_tiles) (void)hipFree(kv.second.d_tiles);
     if (p->d_scratch) (void)hipFree(p->d_scratch);
+    for (void* q : p->retired) (void)hipFree(q);
     for (auto& kv : p->lists) free_lists(kv.second);
     if (p->side) { (void)hipStreamSynchronize(p->side); (void)hipStreamDestroy(p->side); }
     if (p->ev_fork) (void)hipEventDestroy(p->ev_fork);
@@ -211,6 +273,12 @@ void aprnet_plan_destroy(aprnet_plan* p) {
 int64_t aprnet_number_parts(const aprnet_plan* p, int level_delta) { return p ? p->number_parts(level_delta) : -1; }
 int64_t aprnet_tree_offset(const aprnet_plan* p, int level) { return p ? p->tree_offset(level) : 0; }
 int64_t aprnet_tree_parts(const aprnet_plan* p, int level_delta) { return p ? p->tree_parts(level_delta) : -1; }
+
+int aprnet_plan_reserve(aprnet_plan* p, int64_t bytes, void* stream) {
+    if (!p || bytes < 0) return fail(APRNET_ERR_INVALID_ARGUMENT, "plan_reserve: null plan or negative size");
+    APRNET_HIP_CHECK(hipSetDevice(p->device));
+    return plan_scratch(p, (size_t)bytes, (hipStream_t)stream);
+}
 
 int aprnet_plan_children(const aprnet_plan* p, int32_t* out_host) {
     if (!p || !out_host) return fail(APRNET_ERR_INVALID_ARGUMENT, "plan_children: null argument");

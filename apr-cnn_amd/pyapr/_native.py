@@ -74,6 +74,7 @@ def hip():
         getattr(lib, fn).restype = i64
         getattr(lib, fn).argtypes = [vp, i32]
     lib.aprnet_plan_children.argtypes = [vp, vp]
+    lib.aprnet_plan_reserve.argtypes = [vp, i64, vp]
     lib.aprnet_profile_enable.argtypes = [i32]
     lib.aprnet_set_conv_path.argtypes = [i32]
     lib.aprnet_profile_last_ms.restype = C.c_float

@@ -42,12 +42,13 @@ typedef enum aprnet_status {
  * All pointers are host pointers; the arrays are copied. */
 typedef struct aprnet_access_desc {
     int32_t level_min, level_max;
-    const int32_t* z_num;            /* [level_max+1], indexed by level */
+    const int32_t* z_num;            /* indexed by level; [L+1] entries with L = level_max of the APR's own access */
+                                     /* (also in the tree's descriptor, whose level_max is L-1)                */
     const int32_t* x_num;
     const int32_t* y_num;
     const uint64_t* level_xz_vec;    /* [level_max+2] */
     const uint64_t* xz_end_vec;      /* [n_rows] with leading sentinel 0 */
-    const uint16_t* y_vec;           /* [n_particles] */
+    const uint16_t* y_vec;           /* [n_particles]; per row strictly ascending and < y_num of the row's level */
     uint64_t n_rows;
     uint64_t n_particles;
 } aprnet_access_desc;
@@ -56,9 +57,19 @@ typedef struct aprnet_plan aprnet_plan;
 
 const char* aprnet_last_error(void);
 
-/* Replaces APR::init_cuda() + gpuAPRHelper()/gpuTreeHelper() (wrap_conv_gpu.hpp:25-26). */
+/* Replaces APR::init_cuda() + gpuAPRHelper()/gpuTreeHelper() (wrap_conv_gpu.hpp:25-26).  The arrays are validated on
+ * the host (row table non-decreasing and within n_particles, level_xz_vec consistent with z_num * x_num, y strictly
+ * ascending per row and below y_num): APRNET_ERR_INVALID_ARGUMENT names the first violation. */
 int aprnet_plan_create(const aprnet_access_desc* apr, const aprnet_access_desc* tree, int device, aprnet_plan** out);
 void aprnet_plan_destroy(aprnet_plan* plan);
+
+/* No counterpart in the reference.  The convolutions keep re-laid-out weights (and, for bfloat16 features, a regrouped
+ * copy of their input) in one scratch buffer of the plan that grows to the largest call seen.  Growth allocates, so it is
+ * refused with APRNET_ERR_UNSUPPORTED while `stream` is capturing into a graph, and so is the first convolution at a
+ * level delta (it builds the plan's tile and window lists).  Call this - or run the network once - before a capture;
+ * a buffer that a captured graph may address is kept until aprnet_plan_destroy.  Calls that share a plan use one
+ * stream at a time: a call on another stream first waits for the previous one. */
+int aprnet_plan_reserve(aprnet_plan* plan, int64_t bytes, void* stream);
 
 /* helpers::number_parts (helpers.hpp:86-101); also number_parts_after_pooling/_upsampling with d±1. */
 int64_t aprnet_number_parts(const aprnet_plan* plan, int level_delta);

@@ -113,3 +113,51 @@ def test_model_parameter_names_mirror_reference():
     assert sd["encoder.2.conv.blocks.0.conv.weight"].dim() == 5       # nn.Conv3d [Cout, Cin, kz, kx, ky]
     assert sd["decoder.1.conv.blocks.0.conv.weight"].dim() == 6       # APRConv [S, Cout, Cin, kz, kx, ky]
     assert tuple(sd["decoder.1.conv.blocks.0.conv.weight"].shape[1:3]) == (8, 16)      # reads skip + upsampled
+
+
+def test_plan_create_refuses_damaged_access_arrays():
+    """Access arrays read from a file are validated on the host before any device work: a damaged state is
+    APRNET_ERR_INVALID_ARGUMENT (-1) with a message naming the violation, not an out-of-range access on the GPU.
+    Runs without a GPU: validation comes before the first HIP call."""
+    import ctypes as C
+    import numpy as np
+    import apr_cases
+    from pyapr import APR, _native
+    lib = _native.hip()
+    good = apr_cases.get("3d_a")
+    oy, ox, oz, _params, xz, y, txz, ty = good.get_state()
+
+    def create(xz_, y_, txz_, ty_, drop_y=False):
+        apr = APR.from_state((oy, ox, oz), np.array(xz_), np.array(y_), np.array(txz_), np.array(ty_))
+        a, t = apr._desc(apr.iterator()), apr._desc(apr.tree_iterator())
+        if drop_y:
+            a.y_vec = None
+        h = C.c_void_p()
+        rc = lib.aprnet_plan_create(C.byref(a), C.byref(t), 0, C.byref(h))
+        msg = lib.aprnet_last_error().decode()
+        if rc == 0:
+            lib.aprnet_plan_destroy(h)
+        return rc, msg
+
+    # a row with two or more particles, to break the order inside it
+    rows = np.flatnonzero(np.diff(xz.astype(np.int64)) >= 2)
+    b = int(xz[rows[0]])
+    y_swapped = y.copy(); y_swapped[b], y_swapped[b + 1] = y[b + 1], y[b]
+    rc, msg = create(xz, y_swapped, txz, ty)
+    assert rc == -1 and "ascend" in msg
+    y_big = y.copy(); y_big[b + 1] = 65535
+    rc, msg = create(xz, y_big, txz, ty)
+    assert rc == -1 and "y_num" in msg
+    xz_bad = xz.copy(); xz_bad[rows[0] + 1] = xz_bad[rows[0]] - 1 if xz_bad[rows[0]] > 0 else xz_bad[-1] + 5
+    rc, msg = create(xz_bad, y, txz, ty)
+    assert rc == -1 and ("xz_end_vec" in msg or "y_vec" in msg)       # a moved row end also mis-slices y
+    xz_over = xz.copy(); xz_over[len(xz) // 2] = xz[-1] + 7
+    rc, msg = create(xz_over, y, txz, ty)
+    assert rc == -1 and "xz_end_vec" in msg
+    ty_bad = ty.copy()
+    trows = np.flatnonzero(np.diff(txz.astype(np.int64)) >= 2)
+    tb = int(txz[trows[0]]); ty_bad[tb + 1] = ty_bad[tb]
+    rc, msg = create(xz, y, txz, ty_bad)
+    assert rc == -1 and "ascend" in msg
+    rc, msg = create(xz, y, txz, ty, drop_y=True)
+    assert rc == -1 and "y_vec" in msg
