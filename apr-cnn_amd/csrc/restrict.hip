@@ -4,6 +4,8 @@
 // element, gather form in both directions, so the result is deterministic.
 #include "common.hpp"
 
+#include <mutex>
+
 namespace aprnet {
 
 __device__ __forceinline__ float overlap1(int o, int i, int k, int step) {
@@ -150,10 +152,46 @@ int channel_sum(const T* x, int64_t ld, int C, int64_t n, typename Num<T>::acc* 
     return 0;
 }
 
+// ---------------------------------------------------------------------------- bias gradient without a work-space argument
+// The block partials of channel_sum live in a device array of this library instead of caller memory, for callers that
+// cannot allocate (under stream capture, in serving loops).  Every GPU holds its own copy of the array at its own
+// address; host code only ever uses the address that hipGetSymbolAddress returned on that GPU, never the array's name.
+constexpr int CS_STATIC_MAX_C = 1024;
+constexpr int CS_MAX_DEVICES = 64;
+static __device__ __align__(256) float cs_static_scratch[CS_STATIC_MAX_C * CS_BLOCKS];     // 1 MiB per GPU
+static float* g_cs_static_ptr[CS_MAX_DEVICES] = {};
+static std::mutex g_cs_static_mutex;
+
+static int cs_static_scratch_ptr(float** out) {
+    int dev = -1;
+    APRNET_HIP_CHECK(hipGetDevice(&dev));
+    if (dev < 0 || dev >= CS_MAX_DEVICES) return fail(APRNET_ERR_UNSUPPORTED, "channel_sum_static: device index beyond 63");
+    std::lock_guard<std::mutex> lock(g_cs_static_mutex);
+    if (!g_cs_static_ptr[dev]) {
+        float* ptr = nullptr;
+        APRNET_HIP_CHECK(hipGetSymbolAddress((void**)&ptr, HIP_SYMBOL(cs_static_scratch)));
+        if (!ptr) return fail(APRNET_ERR_HIP, "channel_sum_static: the scratch array has no address on this device");
+        g_cs_static_ptr[dev] = ptr;
+    }
+    *out = g_cs_static_ptr[dev];
+    return 0;
+}
+
 }  // namespace aprnet
 
 using namespace aprnet;
 extern "C" {
+int aprnet_channel_sum_static_max_channels(void) { return CS_STATIC_MAX_C; }
+int aprnet_channel_sum_static_f32(const float* x, int64_t ld, int C, int64_t n, float* out, int accumulate, void* st) {
+    if (C > CS_STATIC_MAX_C)
+        return fail(APRNET_ERR_UNSUPPORTED, "channel_sum_static: at most " + std::to_string(CS_STATIC_MAX_C) +
+                                            " channels per call (" + std::to_string(C) + " given); use aprnet_channel_sum_f32 with a work space");
+    if (C <= 0) return 0;
+    float* work = nullptr;
+    if (int rc = cs_static_scratch_ptr(&work)) return rc;
+    // the partial kernel writes every slot it later reads (C * CS_BLOCKS values): nothing of an earlier call survives
+    return channel_sum<float>(x, ld, C, n, out, accumulate, work, (hipStream_t)st);
+}
 int aprnet_channel_sum_work_elems(int C) { return C * CS_BLOCKS; }
 int aprnet_channel_sum_f32(const float* x, int64_t ld, int C, int64_t n, float* out, int accumulate, float* work, void* st) {
     return channel_sum<float>(x, ld, C, n, out, accumulate, work, (hipStream_t)st);

@@ -110,6 +110,15 @@ int aprnet_channel_sum_work_elems(int C);
 int aprnet_channel_sum_f32(const float* x, int64_t ld, int C, int64_t n, float* out, int accumulate, float* work, void* stream);
 int aprnet_channel_sum_f64(const double* x, int64_t ld, int C, int64_t n, double* out, int accumulate, double* work, void* stream);
 
+/* No counterpart in the reference: aprnet_channel_sum_f32 for callers that cannot allocate device memory (code under
+ * HIP graph capture, serving loops, harnesses that forbid hipMalloc).  The block partials that the other entry point
+ * keeps in the caller's `work` live in a 1 MiB device array of this library (one copy per GPU, held until the
+ * process ends); the call allocates nothing and frees nothing.  The current device must be the one x and out live on.
+ * At most aprnet_channel_sum_static_max_channels() (1024) channels per call: APRNET_ERR_UNSUPPORTED beyond.  All calls
+ * on one GPU share the array: calls that overlap on one GPU (two streams) race and must be ordered by the caller. */
+int aprnet_channel_sum_static_max_channels(void);
+int aprnet_channel_sum_static_f32(const float* x, int64_t ld, int C, int64_t n, float* out, int accumulate, void* stream);
+
 /* Optional parts of aprnet_conv_fwd_fused_*.  They fuse what the reference network does in separate passes around
  * a convolution: torch.cat of the skip connection and the upsampled features before the first convolution of a
  * decoder stage (unet_parts.py:82), and the ReLU that follows a convolution whose norm has been folded into it
