@@ -48,9 +48,13 @@ class APRUNet(nn.Module):
         skips = [self.encoder[0](x, aprs, level_deltas)]
         for stage in self.encoder[1:]:
             skips.append(stage(skips[-1], aprs, level_deltas))
-        y = skips[-1]
-        for i, stage in enumerate(self.decoder):
-            y = stage(y, skips[-(i + 2)], aprs, level_deltas)
+        # every skip tensor is dropped as soon as its decoder stage has read it: at inference the peak working set is
+        # then one stage's inputs and output, not the whole encoder
+        y = skips.pop()
+        for stage in self.decoder:
+            skip = skips.pop()
+            y = stage(y, skip, aprs, level_deltas)
+            del skip
         return self.head(y, aprs, level_deltas)
 
 

@@ -1,19 +1,29 @@
 #!/usr/bin/env python3
-"""Benchmark of the hot path on one MI355X: APRConv 3x3x3 forward, Cin = Cout = 32, fp32, on the APR of the
-seeded 512 x 512 x 256 blob volume (BASELINE.json configs[1]).
+"""Benchmark of the hot path on one MI355X.
 
-  python bench.py [--gpus 1] [--steps K] [--warmup W]
+  python bench.py [--gpus 1] [--steps K] [--warmup W] [--config NAME]
 
-A step is one `aprnet.cuda.APRConv.forward` on device-resident features: weight expansion
-(restrict kernel), tree fill of the 32 input channels and the convolution kernel (bias fused into its store).
-Prints ONE JSON line.  `value` = particles/s of the whole step; `roofline` prices the convolution
-kernel alone (its duration is measured with HIP events recorded around the launch on its own stream,
-see aprnet_profile_enable in include/aprnet_hip.h); `cpu_baseline` times the CPU oracle (a restatement
-of the reference's OpenMP code) on a centre crop of the same volume.
+Default (the line the headline metric is quoted on): APRConv 3x3x3 forward, Cin = Cout = 32, fp32, on the APR of
+the seeded 512 x 512 x 256 blob volume (BASELINE.json configs[1], ``--config blobs512``), plus the forward latency
+of the 4-level APR-UNet on the same APR in ``extra``.  The other BASELINE configurations are selected by name and
+print one JSON line each, with the measured particle count per level:
+
+  spheres128   configs[0]  APRConv 3x3x3 1 -> 16 fp32 forward with bias on the 128^3 volume          (HBM-bound)
+  blobs512     configs[1]  APRConv 3x3x3 32 -> 32 fp32 forward (+ --chain: conv -> ReLU -> pool -> upsample, fwd + bwd)
+  nuclei2048   configs[2]  tree fill + APRConv 3x3x3 16 -> 16 fp32 forward on the 2048 x 2048 x 512 volume
+  nuclei1024   configs[3]  4-level APR-UNet forward, fp32 and bfloat16 features, on the 1024^3 volume
+  spots16k     configs[4]  APRConv 1x5x5 64 -> 64, bfloat16 features, forward + backward, 16384^2 image
+
+A step is one pass of the configuration's operator(s) over device-resident features.  ``value`` is particles/s of
+the whole step (latency in ms for the network); ``roofline`` prices the dominant kernel alone (its duration is
+measured with HIP events recorded around the launch on its own stream, see aprnet_profile_enable in
+include/aprnet_hip.h); ``cpu_baseline`` times the CPU oracle (a restatement of the reference's OpenMP code) on a
+bounded sample of the same workload: one warm-up run, then the median of five, with one thread and with all cores.
 """
 import argparse
 import json
 import os
+import statistics
 import sys
 import time
 
@@ -22,54 +32,107 @@ for _p in (ROOT, os.path.join(ROOT, "apr-cnn_amd")):
     if _p not in sys.path:
         sys.path.insert(0, _p)
 
-CIN = COUT = 32
-K_TAPS = 27
-FLOP_PER_PARTICLE = 2 * K_TAPS * CIN * COUT          # 55 296
-BYTES_PER_PARTICLE = 4 * (CIN + COUT) + 2            # features in + out, y_vec
 PEAK_FP32_MATRIX_TFLOPS = 157.3
 PEAK_BF16_MATRIX_TFLOPS = 2500.0
 PEAK_HBM_GBS = 8000.0
-# HBM-side bytes of one launch of the convolution kernel on this workload: FETCH_SIZE + WRITE_SIZE of two
+# HBM-side bytes of one launch of the convolution kernel on the default workload: FETCH_SIZE + WRITE_SIZE of two
 # profiler passes, scaled by what the same counters read for a device-to-device copy of known size
-# (profiles/conv333_fwd_32x32_f32_blobs512_hbm_traffic.txt).  Counters cannot be read from inside this
-# script; the figure is only reported when the workload is the one it was measured on.
-MEASURED_TRAFFIC_BYTES = {23245996: 30.18e9 + 4.10e9}
+# (profiles/conv333_fwd_32x32_f32_blobs512_hbm_traffic.txt).  Counters cannot be read from inside this script: the
+# figure is a constant taken from that profile and only reported when the workload is the one it was measured on.
+PROFILED_TRAFFIC_BYTES = {23245996: 30.18e9 + 4.10e9}
 
 
-def build_workload(name, crop=None):
+# ------------------------------------------------------------------------------------------------ workloads
+def build_volume(name):
+    from pyapr.synthetic import CONFIGS, synth_volume
+    shape, kind, n, axes, amp, bg, iso, _rel = CONFIGS[name]
+    return synth_volume(shape, 0, kind, n, axes, amp, bg, iso)
+
+
+def centre_crop(img, crop):
     import numpy as np
-    from pyapr.synthetic import CONFIGS, synth_volume, pipeline_parameters
+    sl = []
+    for s, c in zip(img.shape, crop):
+        c = min(c, s)
+        a = (s - c) // 2
+        sl.append(slice(a, a + c))
+    return np.ascontiguousarray(img[tuple(sl)])
+
+
+def build_workload(name, crop=None, img=None, with_parts=False):
+    """APR of a named configuration (optionally of a centre crop of its volume)."""
+    from pyapr.synthetic import CONFIGS, pipeline_parameters
     from pyapr.converter import get_apr
-    shape, kind, n, axes, amp, bg, iso, rel = CONFIGS[name]
-    img = synth_volume(shape, 0, kind, n, axes, amp, bg, iso)
+    if img is None:
+        img = build_volume(name)
     if crop is not None:
-        z, x, y = (s // 2 for s in shape)
-        cz, cx, cy = (c // 2 for c in crop)
-        img = np.ascontiguousarray(img[z - cz:z + cz, x - cx:x + cx, y - cy:y + cy])
-    apr, _parts = get_apr(img, params=pipeline_parameters(rel))
-    return apr
+        img = centre_crop(img, crop)
+    apr, parts = get_apr(img, params=pipeline_parameters(CONFIGS[name][7]))
+    return (apr, parts) if with_parts else apr
 
 
-def cpu_baseline(nstencils):
-    """CPU oracle (port of pyapr/aprnet/src/conv.hpp + helpers.hpp, OpenMP over z) on a 128 x 256 x 256 centre
-    crop of the benchmark volume, same layer shape; a few seconds to tens of seconds of CPU work."""
+def level_counts(apr):
+    it, tr = apr.iterator(), apr.tree_iterator()
+    out = {"particles": {}, "tree_nodes": {}}
+    for l in range(it.level_min(), it.level_max() + 1):
+        out["particles"][str(l)] = it.particles_level_end(l) - it.particles_level_begin(l)
+    for l in range(tr.level_min(), tr.level_max() + 1):
+        out["tree_nodes"][str(l)] = tr.particles_level_end(l) - tr.particles_level_begin(l)
+    return out
+
+
+def host_cores():
+    return int(os.environ.get("OMP_NUM_THREADS", 0)) or len(os.sched_getaffinity(0))
+
+
+def cpu_model():
+    try:
+        for line in open("/proc/cpuinfo"):
+            if line.startswith("model name"):
+                return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
+
+
+def cpu_baseline_conv(apr, cin, cout, ksize, nstencils, sample, budget_s=25.0):
+    """The CPU oracle (port of pyapr/aprnet/src/conv.hpp + helpers.hpp, OpenMP over z) on `apr`: weight expansion +
+    convolution forward, output allocation excluded.  1 warm-up + median of five, with one thread and with all cores.
+    When one single-thread run is longer than a fifth of the budget, fewer runs are taken and the line says so."""
     import torch
     from oracle import oracle
-    crop = (128, 256, 256)
-    apr = build_workload("blobs512", crop=crop)
     n = apr.total_number_particles()
     g = torch.Generator().manual_seed(1)
-    x = torch.randn(1, CIN, n, generator=g)
-    w = torch.randn(CIN, nstencils, COUT, 3, 3, 3, generator=g) * 0.1
+    x = torch.randn(1, cin, n, generator=g)
+    w = torch.randn(cin, nstencils, cout, *ksize, generator=g) * 0.1
     ld = torch.zeros(1, dtype=torch.int32)
-    t0 = time.perf_counter()
-    w_exp = oracle.restrict_kernel_forward(w, apr.level_max() - apr.level_min() + 1)
-    oracle.conv_forward([apr], x, w_exp, ld)
-    dt = time.perf_counter() - t0
-    cores = int(os.environ.get("OMP_NUM_THREADS", 0)) or len(os.sched_getaffinity(0))
-    return {"value": n / dt, "unit": "particles/s", "cores": cores, "kind": "port",
-            "sample": f"centre crop {crop[0]}x{crop[1]}x{crop[2]} of the 256x512x512 volume, {n} particles, "
-                      f"conv 3x3x3 {CIN}->{COUT} fp32, 1 run, {dt:.1f} s"}
+    levels = apr.level_max() - apr.level_min() + 1
+
+    def run():
+        oracle.conv_forward([apr], x, oracle.restrict_kernel_forward(w, levels), ld)
+
+    cores = host_cores()
+    res = {}
+    for threads in (cores, 1):
+        before = oracle.set_threads(threads)
+        t0 = time.perf_counter()
+        run()                                       # warm-up, also sizes the number of timed runs
+        first = time.perf_counter() - t0
+        runs = 5 if first * 6 < budget_s else (3 if first * 4 < budget_s else 1)
+        ts = []
+        for _ in range(runs):
+            t0 = time.perf_counter()
+            run()
+            ts.append(time.perf_counter() - t0)
+        oracle.set_threads(before)
+        res[threads] = (statistics.median(ts), runs)
+    t_all, r_all = res[cores]
+    t_one, r_one = res[1]
+    return {"value": n / t_all, "unit": "particles/s", "cores": cores, "kind": "port",
+            "value_1_thread": n / t_one, "cpu": cpu_model(),
+            "sample": f"{sample}, {n} particles, conv {ksize[0]}x{ksize[1]}x{ksize[2]} {cin}->{cout} fp32 forward incl. weight "
+                      f"expansion; 1 warm-up + median of {r_all} runs on {cores} threads ({t_all:.2f} s each), "
+                      f"median of {r_one} on 1 thread ({t_one:.2f} s each)"}
 
 
 def _time(fn, iters=10, warmup=2):
@@ -86,6 +149,356 @@ def _time(fn, iters=10, warmup=2):
     return a.elapsed_time(b) / iters
 
 
+def _steps(fn, steps, warmup):
+    """The timed region of the contract: W untimed steps, then exactly K steps between two synchronisations."""
+    import torch
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        fn()
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t0) / steps
+
+
+def _kernel_ms(lib, fn, repeats):
+    """Average duration of the convolution kernel inside fn(): HIP events around its launch, on its stream."""
+    lib.aprnet_profile_enable(1)
+    kms = []
+    for _ in range(repeats):
+        fn()
+        kms.append(float(lib.aprnet_profile_last_ms()))
+    lib.aprnet_profile_enable(0)
+    return sum(kms) / len(kms)
+
+
+def make_unet(dev):
+    import torch
+    from apr_models.unet import APRUNet, fold_norms
+    torch.manual_seed(0)
+    net = APRUNet(1, 3, depth=3, n_filters_base=16, n_stencils=2, norm="batch")
+    for m in net.modules():                          # He initialisation of the convolution weights, seed 0
+        if hasattr(m, "weight") and getattr(m, "weight") is not None and m.weight.dim() == 6:
+            fan_in = m.weight.shape[2] * m.weight.shape[3] * m.weight.shape[4] * m.weight.shape[5]
+            torch.nn.init.normal_(m.weight, 0.0, (2.0 / fan_in) ** 0.5)
+    return fold_norms(net.eval()).to(dev)
+
+
+def base_line(metric, value, unit, args, ms_per_step, dtype, config, higher=True):
+    return {"metric": metric, "value": value, "unit": unit, "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+            "ms_per_step": ms_per_step, "higher_is_better": higher, "scaling": "weak", "vs_baseline": None,
+            "dtype": dtype, "data": "synthetic", "config": config}
+
+
+def mfma_roofline(flop, kernel_ms, peak, kernel, hbm_bytes, traffic=None):
+    tflops = flop / (kernel_ms * 1e-3) / 1e12
+    gbs = hbm_bytes / (kernel_ms * 1e-3) / 1e9
+    return {"bound": "mfma", "achieved": tflops, "peak": peak, "unit": "TFLOP/s", "frac": tflops / peak,
+            "traffic": traffic, "traffic_source": "constant from the committed profiler summary, not read in this run" if traffic else None,
+            "kernel": kernel, "kernel_ms": kernel_ms, "hbm_achieved_GBs": gbs, "hbm_frac": gbs / PEAK_HBM_GBS}
+
+
+def hbm_roofline(nbytes, kernel_ms, kernel, flop=None):
+    gbs = nbytes / (kernel_ms * 1e-3) / 1e9
+    out = {"bound": "hbm", "achieved": gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": gbs / PEAK_HBM_GBS, "traffic": None,
+           "kernel": kernel, "kernel_ms": kernel_ms}
+    if flop is not None:
+        out["fp32_TFLOPs"] = flop / (kernel_ms * 1e-3) / 1e12
+    return out
+
+
+# ------------------------------------------------------------------------------------------------ configs
+def run_blobs512(args, dev, lib):
+    """configs[1]: the 32 -> 32 layer (headline metric) and the APR-UNet forward latency on the same APR."""
+    import torch
+    from pyapr import aprnet
+    CIN = COUT = 32
+    flop_pp, bytes_pp = 2 * 27 * CIN * COUT, 4 * (CIN + COUT) + 2
+    nstencils = 2
+    t0 = time.perf_counter()
+    img = build_volume("blobs512")
+    apr = build_workload("blobs512", img=img)
+    t_build = time.perf_counter() - t0
+    t0 = time.perf_counter()
+    apr.init_cuda()
+    t_plan = time.perf_counter() - t0
+    n = apr.total_number_particles()
+    bf16 = args.features == "bf16"
+    torch.manual_seed(0)
+    x = torch.randn(1, CIN, n, device=dev)
+    if bf16:
+        x = x.to(torch.bfloat16)
+    conv = aprnet.cuda.APRConv(CIN, COUT, nstencils=nstencils, kernel_size=(3, 3, 3), bias=True).to(dev)
+    ld = torch.zeros(1, dtype=torch.int32)
+    with torch.no_grad():
+        sec = _steps(lambda: conv(x, [apr], ld), args.steps, args.warmup)
+        kernel_ms = _kernel_ms(lib, lambda: conv(x, [apr], ld), args.steps)
+        y = conv(x, [apr], ld)
+    assert torch.isfinite(y.float()).all()
+    del y
+    e = 2 if bf16 else 4
+    out = base_line("APRConv 3x3x3 fwd particles/s (Cin=Cout=32) + APR-UNet fwd latency, 1 GPU", n / sec, "particles/s", args,
+                    sec * 1e3, "bf16" if bf16 else "f32",
+                    {"workload": f"APRConv 3x3x3 32->32 {'bf16' if bf16 else 'fp32'} forward (restrict + tree fill + conv + bias), batch 1, "
+                                 "APR of the seeded 512x512x256 volume with 2000 ellipsoidal blobs (configs[1]); extra: 4-level "
+                                 "APR-UNet forward on the same APR",
+                     "n_particles": n, "levels": level_counts(apr), "nstencils": nstencils, "level_max": apr.level_max(),
+                     "apr_build_s": round(t_build, 2), "plan_create_s": round(t_plan, 2)})
+    out["roofline"] = mfma_roofline(flop_pp * n, kernel_ms, PEAK_BF16_MATRIX_TFLOPS if bf16 else PEAK_FP32_MATRIX_TFLOPS,
+                                    "conv_mfma_bf16_kernel" if bf16 else "conv_mfma16_kernel",
+                                    (e * (CIN + COUT) + 2) * n, None if bf16 else PROFILED_TRAFFIC_BYTES.get(n))
+    # second half of the metric: forward latency of the 4-level network (16-32-64-128, norms folded) on this APR
+    net = make_unet(dev)
+    xin = x[:, :1].float().contiguous()
+    extra = {"n_particles": n}
+    with torch.no_grad():
+        extra["apr_unet_fwd_ms_f32"] = _time(lambda: net(xin, [apr]), iters=5, warmup=2)
+        xinb = xin.to(torch.bfloat16)
+        extra["apr_unet_fwd_ms_bf16"] = _time(lambda: net(xinb, [apr]), iters=5, warmup=2)
+        # the narrow first layer of the network (1 -> 16 with bias and ReLU folded in): bound by HBM, 68 bytes per particle
+        first = net.encoder[0].blocks[0].conv
+        k1 = _kernel_ms(lib, lambda: first.forward_fused(xin, [apr], ld, relu=True), 5)
+        extra["conv333_1to16_kernel_ms"] = k1
+        extra["conv333_1to16_hbm_frac"] = 68 * n / (k1 * 1e-3) / 1e9 / PEAK_HBM_GBS
+    out["extra"] = extra
+    if args.calibrate_copy:
+        torch.empty_like(x).copy_(x)
+        torch.cuda.synchronize()
+        print(json.dumps({"calibration_copy_bytes_read": x.numel() * e, "calibration_copy_bytes_written": x.numel() * e}),
+              file=sys.stderr, flush=True)
+    if args.chain:
+        print(json.dumps(chain_step(apr, x.float(), dev)), file=sys.stderr, flush=True)
+    if args.ops:
+        for line in other_ops(apr, x.float() if bf16 else x, dev):
+            print(json.dumps(line), file=sys.stderr, flush=True)
+    if not args.no_cpu_baseline:
+        crop = (128, 256, 256)
+        out["cpu_baseline"] = cpu_baseline_conv(build_workload("blobs512", crop=crop, img=img), CIN, COUT, (3, 3, 3), nstencils,
+                                                f"centre crop {crop[0]}x{crop[1]}x{crop[2]} of the 256x512x512 volume")
+    return out
+
+
+def chain_step(apr, x, dev):
+    """configs[1] in full: APRConv(32 -> 32) -> ReLU -> MaxPool -> UpSampleConst, forward + backward (dX, dW)."""
+    import torch
+    from pyapr import aprnet
+    C = x.shape[1]
+    conv = aprnet.cuda.APRConv(C, C, nstencils=2).to(dev)
+    pool, up = aprnet.cuda.MaxPool(), aprnet.cuda.UpSampleConst()
+    xg = x.clone().requires_grad_(True)
+    n = x.shape[2]
+
+    def step():
+        ld = torch.zeros(1, dtype=torch.int32)
+        xg.grad = None
+        conv.weight.grad = None
+        u = up(pool(torch.relu(conv(xg, [apr], ld)), [apr], ld), [apr], ld)
+        u.backward(torch.ones_like(u))
+    ms = _time(step, iters=3, warmup=1)
+    return {"op": "chain_conv_relu_pool_upsample_fwd_bwd", "ms": ms, "particles_per_s": n / ms * 1e3,
+            "note": f"configs[1] chain, {C}->{C} fp32, forward + backward (grad input, grad weight)"}
+
+
+def spheres128_inputs():
+    """configs[0]: the APR of the 128^3 sphere volume, its sampled intensities as the one input channel, and the
+    seeded layer (weights N(0, 0.1), seed 0, one stencil, bias)."""
+    import torch
+    apr, parts = build_workload("spheres128", with_parts=True)
+    x = (torch.from_numpy(parts).float() / 1000.0).view(1, 1, -1).contiguous()
+    g = torch.Generator().manual_seed(0)
+    w = torch.randn(1, 16, 1, 3, 3, 3, generator=g) * 0.1           # device layout [S, Cout, Cin, kz, kx, ky]
+    b = torch.randn(16, generator=g) * 0.1
+    return apr, x, w, b
+
+
+def run_spheres128(args, dev, lib):
+    import torch
+    from pyapr.aprnet import _ops
+    apr, x, w, b = spheres128_inputs()
+    apr.init_cuda()
+    n = apr.total_number_particles()
+    levels = apr.level_max() - apr.level_min() + 1
+    xd, wd, bd = x.to(dev), w.to(dev), b.to(dev)
+    ld = torch.zeros(1, dtype=torch.int32)
+
+    def step():
+        return _ops.conv_forward([apr], xd, _ops.restrict_kernel_forward(wd, levels), ld, bias=bd)
+    with torch.no_grad():
+        sec = _steps(step, args.steps, args.warmup)
+        kernel_ms = _kernel_ms(lib, step, args.steps)
+        y = step()
+    out = base_line("APRConv 3x3x3 fwd particles/s (Cin=1, Cout=16)", n / sec, "particles/s", args, sec * 1e3, "f32",
+                    {"workload": "APRConv 3x3x3 1->16 fp32 forward with bias, batch 1, APR of the seeded 128^3 volume with 200 Gaussian "
+                                 "spheres (configs[0]); the launch is too small to fill the GPU: the same layer shape on the "
+                                 "23 M-particle APR is in the default line's extra",
+                     "n_particles": n, "levels": level_counts(apr), "nstencils": 1, "level_max": apr.level_max()})
+    out["roofline"] = hbm_roofline(68 * n, kernel_ms, "forward convolution kernel of the 1->16 layer", flop=864 * n)
+    # cross-machine golden check of this configuration (tests/golden/spheres128_conv_1to16.json)
+    gold = os.path.join(ROOT, "tests", "golden", "spheres128_conv_1to16.json")
+    if os.path.exists(gold):
+        ref = json.load(open(gold))
+        yc = y[0].cpu().double()
+        scale = max(abs(v) for v in ref["abs_max"])
+        ok = ref["n_particles"] == n
+        for c in range(16):
+            ok = ok and abs(float(yc[c].sum()) - ref["sum"][c]) <= 1e-5 * scale * n
+            ok = ok and max(abs(a - r) for a, r in zip(yc[c, :64].tolist(), ref["first64"][c])) <= 1e-5 * scale
+            ok = ok and max(abs(a - r) for a, r in zip(yc[c, -64:].tolist(), ref["last64"][c])) <= 1e-5 * scale
+        out["config"]["golden_check"] = "ok" if ok else "MISMATCH"
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline_conv(apr, 1, 16, (3, 3, 3), 1, "the whole configuration (128^3 volume)")
+    return out
+
+
+def _largest_apr(name, img, limit=(1 << 30) - 1):
+    """The APR of the whole volume when it stays within the particle limit of a plan, otherwise of the largest
+    centre crop (halving z, then x, then y) that does.  -> (apr, description)."""
+    import numpy as np
+    crop = list(img.shape)
+    axis = 0
+    while True:
+        apr = build_workload(name, crop=tuple(crop) if tuple(crop) != img.shape else None, img=img)
+        if apr.total_number_particles() <= limit:
+            desc = "whole volume" if tuple(crop) == img.shape else f"centre crop {crop[0]}x{crop[1]}x{crop[2]} (the whole volume exceeds 2^30 particles)"
+            return apr, desc
+        while crop[axis % 3] <= 1:
+            axis += 1
+        crop[axis % 3] //= 2
+        axis += 1
+
+
+def run_nuclei2048(args, dev, lib):
+    """configs[2]: bottom-up tree fill, then a 3x3x3 convolution that reads tree parents, 16 channels fp32."""
+    import torch
+    from pyapr import aprnet
+    from pyapr.aprnet import _ops
+    C = 16
+    t0 = time.perf_counter()
+    img = build_volume("nuclei2048")
+    apr, what = _largest_apr("nuclei2048", img)
+    t_build = time.perf_counter() - t0
+    apr.init_cuda()
+    n, nt = apr.total_number_particles(), _ops.tree_parts(apr, 0)
+    print(f"# nuclei2048: {n} particles ({what}), {nt} tree nodes, built in {t_build:.0f} s", file=sys.stderr, flush=True)
+    torch.manual_seed(0)
+    x = torch.randn(1, C, n, device=dev)
+    conv = aprnet.cuda.APRConv(C, C, nstencils=2).to(dev)
+    ld = torch.zeros(1, dtype=torch.int32)
+    with torch.no_grad():
+        sec = _steps(lambda: conv(x, [apr], ld), args.steps, args.warmup)
+        kernel_ms = _kernel_ms(lib, lambda: conv(x, [apr], ld), min(args.steps, 5))
+        tree = torch.empty(C, max(nt, 1), device=dev)
+        plan, st = apr.plan(0), torch.cuda.current_stream().cuda_stream
+        fill_ms = _time(lambda: lib.aprnet_fill_tree_mean_f32(plan, 0, x.data_ptr(), n, C, tree.data_ptr(), tree.shape[1], st), iters=5)
+    out = base_line("tree fill + APRConv 3x3x3 fwd particles/s (16 ch fp32)", n / sec, "particles/s", args, sec * 1e3, "f32",
+                    {"workload": f"tree fill (mean of children) + APRConv 3x3x3 16->16 fp32 forward reading tree parents, batch 1, APR of the "
+                                 f"seeded 2048x2048x512 nuclei volume (configs[2]), {what}",
+                     "n_particles": n, "tree_nodes": nt, "levels": level_counts(apr), "apr_build_s": round(t_build, 1)})
+    out["roofline"] = mfma_roofline(2 * 27 * C * C * n, kernel_ms, PEAK_FP32_MATRIX_TFLOPS, "conv_mfma16_kernel", (8 * C + 2) * n)
+    fill_bytes = 4 * C * (n + 2 * nt)
+    out["extra"] = {"fill_tree_mean_ms": fill_ms, "fill_tree_mean_GBs": fill_bytes / fill_ms / 1e6,
+                    "fill_tree_mean_hbm_frac": fill_bytes / fill_ms / 1e6 / PEAK_HBM_GBS,
+                    "fill_tree_mean_algorithmic_bytes": fill_bytes}
+    if not args.no_cpu_baseline:
+        crop = (128, 256, 256)
+        out["cpu_baseline"] = cpu_baseline_conv(build_workload("nuclei2048", crop=crop, img=img), C, C, (3, 3, 3), 2,
+                                                f"centre crop {crop[0]}x{crop[1]}x{crop[2]} of the 512x2048x2048 volume")
+    return out
+
+
+def run_nuclei1024(args, dev, lib):
+    """configs[3]: forward of the 4-level APR-UNet (16-32-64-128, norms folded, He init seed 0), fp32 and bfloat16."""
+    import torch
+    t0 = time.perf_counter()
+    img = build_volume("nuclei1024")
+    apr, what = _largest_apr("nuclei1024", img)
+    t_build = time.perf_counter() - t0
+    apr.init_cuda()
+    n = apr.total_number_particles()
+    print(f"# nuclei1024: {n} particles ({what}), built in {t_build:.0f} s", file=sys.stderr, flush=True)
+    parts = torch.randn(1, 1, n, device=dev)
+    net = make_unet(dev)
+    res = {}
+    with torch.no_grad():
+        for name, xin in (("bf16", parts.to(torch.bfloat16)), ("f32", parts)):
+            try:
+                torch.cuda.reset_peak_memory_stats()
+                sec = _steps(lambda: net(xin, [apr]), max(1, min(args.steps, 3)), 1)
+                y = net(xin, [apr])
+                assert torch.isfinite(y.float()).all()
+                res[name] = {"ms": sec * 1e3, "peak_device_GB": torch.cuda.max_memory_allocated() / 1e9}
+                del y
+            except RuntimeError as e:           # torch.OutOfMemoryError, or a failed allocation inside the library
+                res[name] = {"ms": None, "error": str(e).split("\n")[0][:200]}
+            torch.cuda.empty_cache()
+            print(f"# nuclei1024 {name}: {res[name]}", file=sys.stderr, flush=True)
+    ms = res["bf16"]["ms"] or res["f32"]["ms"]
+    out = base_line("APR-UNet fwd latency (ms), 4 levels 16-32-64-128", ms, "ms", args, ms, "bf16",
+                    {"workload": f"APR-UNet forward, 4 levels 16-32-64-128, two 3x3x3 convolutions + ReLU per level, norms folded, 1x1x1 head "
+                                 f"to 3 classes, batch 1, APR of the seeded 1024^3 nuclei volume (configs[3]), {what}",
+                     "n_particles": n, "levels": level_counts(apr), "apr_build_s": round(t_build, 1)}, higher=False)
+    out["steps"] = max(1, min(args.steps, 3))
+    out["warmup"] = 1
+    out["extra"] = {"apr_unet_fwd_bf16": res["bf16"], "apr_unet_fwd_f32": res["f32"],
+                    "particles_per_s_bf16": n / res["bf16"]["ms"] * 1e3 if res["bf16"]["ms"] else None}
+    out["roofline"] = None
+    return out
+
+
+def run_spots16k(args, dev, lib):
+    """configs[4]: APRConv 1x5x5 64 -> 64, bfloat16 features with fp32 accumulation, forward + backward."""
+    import torch
+    from pyapr import aprnet
+    C = 64
+    t0 = time.perf_counter()
+    img = build_volume("spots16k")
+    apr = build_workload("spots16k", img=img)
+    t_build = time.perf_counter() - t0
+    apr.init_cuda()
+    n = apr.total_number_particles()
+    print(f"# spots16k: {n} particles, built in {t_build:.0f} s", file=sys.stderr, flush=True)
+    conv = aprnet.cuda.APRConv(C, C, nstencils=2, kernel_size=(1, 5, 5)).to(dev)
+    ld = torch.zeros(1, dtype=torch.int32)
+    x = torch.randn(1, C, n, device=dev).to(torch.bfloat16)
+    steps = max(1, min(args.steps, 5))
+    with torch.no_grad():
+        sec = _steps(lambda: conv(x, [apr], ld), steps, 1)
+        kernel_ms = _kernel_ms(lib, lambda: conv(x, [apr], ld), 3)
+    extra = {"fwd_ms": sec * 1e3, "fwd_peak_device_GB": torch.cuda.max_memory_allocated() / 1e9}
+    # the backward of the layer at full size needs the features, two gradients and an fp32 gradient work space at
+    # 64 channels: run when it fits, otherwise on the 4096^2 corner of the same image
+    try:
+        xg = x.requires_grad_(True)
+        y = conv(xg, [apr], ld)
+        go = torch.randn_like(y)
+        extra["bwd_ms"] = _time(lambda: torch.autograd.grad(y, (xg, conv.weight), go, retain_graph=True), iters=2, warmup=1)
+        extra["bwd_sample"] = "whole image"
+        del y, go
+    except RuntimeError:                        # out of device memory
+        xg = y = go = None
+        torch.cuda.empty_cache()
+        small = build_workload("spots16k", crop=(1, 4096, 4096), img=img)
+        ns = small.total_number_particles()
+        xs = torch.randn(1, C, ns, device=dev).to(torch.bfloat16).requires_grad_(True)
+        ys = conv(xs, [small], ld)
+        gs = torch.randn_like(ys)
+        extra["bwd_ms"] = _time(lambda: torch.autograd.grad(ys, (xs, conv.weight), gs, retain_graph=True), iters=2, warmup=1)
+        extra["bwd_sample"] = f"centre crop 4096x4096 ({ns} particles): the whole image's backward does not fit the device"
+    out = base_line("APRConv 1x5x5 fwd particles/s (Cin=Cout=64, bf16)", n / sec, "particles/s", args, sec * 1e3, "bf16",
+                    {"workload": "APRConv 1x5x5 64->64 forward, bfloat16 features, fp32 accumulation, batch 1, APR of the seeded 16384^2 "
+                                 "image with 1M Gaussian spots (configs[4]); backward in extra",
+                     "n_particles": n, "levels": level_counts(apr), "apr_build_s": round(t_build, 1)})
+    out["steps"], out["warmup"] = steps, 1
+    out["roofline"] = mfma_roofline(2 * 25 * C * C * n, kernel_ms, PEAK_BF16_MATRIX_TFLOPS, "conv_mfma_bf16_kernel", (2 * 2 * C + 2) * n)
+    out["extra"] = extra
+    if not args.no_cpu_baseline:
+        crop = (1, 2048, 2048)
+        out["cpu_baseline"] = cpu_baseline_conv(build_workload("spots16k", crop=crop, img=img), C, C, (1, 5, 5), 2,
+                                                "centre crop 2048x2048 of the 16384^2 image")
+    return out
+
+
 def other_ops(apr, x, dev):
     """Memory-bound operators at 32 channels on the same APR, priced against the HBM roofline with their
     algorithmic bytes, the backward pass of the convolution, and the 4-level APR-UNet forward."""
@@ -99,19 +512,32 @@ def other_ops(apr, x, dev):
     nt = _ops.tree_parts(apr, 0)
     res = []
 
-    # what a plain device-to-device copy of the same tensor reaches on this GPU: the practical ceiling that the
-    # memory-bound operators are also priced against
+    # Two reference rates for the memory-bound operators: a plain device-to-device copy of the same tensor, and the
+    # best streaming rate this library itself reaches on it (the norm kernels: mostly reads, 16 bytes per lane).
     dst = torch.empty_like(x)
     ms = _time(lambda: dst.copy_(x))
     copy_gbs = 2 * x.numel() * e / ms / 1e6
     res.append({"op": "copy_d2d", "ms": ms, "algorithmic_GB": 2 * x.numel() * e / 1e9, "GBps": copy_gbs,
                 "hbm_frac": copy_gbs / PEAK_HBM_GBS, "note": "torch copy of the input features, read + write"})
     del dst
+    from apr_models.unet.particle_norm import ParticleBatchNorm
+    bn = ParticleBatchNorm(C).to(dev).train()
+    with torch.no_grad():
+        ms_nf = _time(lambda: bn(x, relu=True))
+    xn = x.detach().clone().requires_grad_(True)
+    yn = bn(xn, relu=True)
+    gn = torch.randn_like(yn)
+    ms_nb = _time(lambda: torch.autograd.grad(yn, xn, gn, retain_graph=True))
+    del xn, yn, gn, bn
+    stream_gbs = max(copy_gbs, e * 3 * C * n0 / ms_nf / 1e6, e * 7 * C * n0 / ms_nb / 1e6)
 
     def line(op, ms, nbytes, note):
         res.append({"op": op, "ms": ms, "algorithmic_GB": nbytes / 1e9, "GBps": nbytes / ms / 1e6,
-                    "hbm_frac": nbytes / ms / 1e6 / PEAK_HBM_GBS, "copy_frac": nbytes / ms / 1e6 / copy_gbs, "note": note})
+                    "hbm_frac": nbytes / ms / 1e6 / PEAK_HBM_GBS, "copy_frac": nbytes / ms / 1e6 / copy_gbs,
+                    "stream_frac": nbytes / ms / 1e6 / stream_gbs, "note": note})
 
+    line("norm_relu_fwd", ms_nf, e * 3 * C * n0, f"C={C}: one pass for the moments, one read + one write to normalise")
+    line("norm_relu_bwd", ms_nb, e * 7 * C * n0, "gradient, input and output read twice (sums, then result), one write")
     with torch.no_grad():
         pooled, idx = _ops.maxpool_forward([apr], x, ld0, 0.0)
         ms = _time(lambda: _ops.maxpool_forward([apr], x, ld0, 0.0))
@@ -129,24 +555,14 @@ def other_ops(apr, x, dev):
         w1 = torch.randn(1, C, C, 1, 1, 1, device=dev) * 0.1
         ms = _time(lambda: _ops.conv_forward([apr], x, w1, ld0))
         line("conv111_fwd", ms, e * 2 * C * n0, f"{C}->{C}")
-    # BatchNorm1d + ReLU over the particle axis in training mode (statistics of the batch), forward and backward
-    from apr_models.unet.particle_norm import ParticleBatchNorm
-    bn = ParticleBatchNorm(C).to(dev).train()
-    with torch.no_grad():
-        ms = _time(lambda: bn(x, relu=True))
-    line("norm_relu_fwd", ms, e * 3 * C * n0, f"C={C}: one pass for the moments, one read + one write to normalise")
-    xn = x.detach().clone().requires_grad_(True)
-    yn = bn(xn, relu=True)
-    gn = torch.randn_like(yn)
-    ms = _time(lambda: torch.autograd.grad(yn, xn, gn, retain_graph=True))
-    line("norm_relu_bwd", ms, e * 7 * C * n0, "gradient, input and output read twice (sums, then result), one write")
-    del xn, yn, gn, bn
     conv = aprnet.cuda.APRConv(C, C, nstencils=2).to(dev)
     xg = x.clone().requires_grad_(True)
     y = conv(xg, [apr], ld0)
     go = torch.randn_like(y)
     ms = _time(lambda: torch.autograd.grad(y, (xg, conv.weight), go, retain_graph=True), iters=3, warmup=1)
-    res.append({"op": "conv333_bwd", "ms": ms, "particles_per_s": n0 / ms * 1e3, "note": f"{C}->{C} grad_input + grad_weight"})
+    fl = 2 * 2 * 27 * C * C * n0
+    res.append({"op": "conv333_bwd", "ms": ms, "particles_per_s": n0 / ms * 1e3, "TFLOPs": fl / ms / 1e9,
+                "mfma_frac": fl / ms / 1e9 / PEAK_FP32_MATRIX_TFLOPS, "note": f"{C}->{C} grad_input + grad_weight"})
     del y, go, xg
     torch.manual_seed(0)
     net = fold_norms(APRUNet(1, 3, depth=3, n_filters_base=16, n_stencils=2, norm="batch").eval()).to(dev)
@@ -270,98 +686,39 @@ def other_ops(apr, x, dev):
     return res
 
 
+RUNNERS = {"spheres128": run_spheres128, "blobs512": run_blobs512, "nuclei2048": run_nuclei2048,
+           "nuclei1024": run_nuclei1024, "spots16k": run_spots16k}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--config", choices=sorted(RUNNERS), default="blobs512",
+                    help="BASELINE configuration to run (default: the one the headline metric is quoted on)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--features", choices=["f32", "bf16"], default="f32",
-                    help="element type of the feature tensors; bf16 runs the bfloat16 matrix-core kernel "
+                    help="blobs512: element type of the feature tensors; bf16 runs the bfloat16 matrix-core kernel "
                          "(the headline figure is the f32 one)")
     ap.add_argument("--calibrate-copy", action="store_true",
-                    help="run one device-to-device copy of the input features (a kernel of known traffic, "
+                    help="blobs512: run one device-to-device copy of the input features (a kernel of known traffic, "
                          "used to scale the FETCH_SIZE / WRITE_SIZE counters of a profiler run)")
     ap.add_argument("--ops", action="store_true",
-                    help="also time the memory-bound operators and the APR-UNet forward (extra JSON lines on stderr)")
+                    help="blobs512: also time the memory-bound operators, the backward pass and the networks (extra JSON lines on stderr)")
+    ap.add_argument("--chain", action="store_true",
+                    help="blobs512: also time the conv -> ReLU -> pool -> upsample chain of configs[1], forward + backward (stderr)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU; --gpus N with N > 1 is not supported "
                  "(the path would shard by batch item, or by z-slabs with a one-row halo per level)")
 
     import torch
-    from pyapr import aprnet, _native
+    from pyapr import _native
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
-
-    nstencils = 2
-    t0 = time.perf_counter()
-    apr = build_workload("blobs512")
-    t_build = time.perf_counter() - t0
-    t0 = time.perf_counter()
-    apr.init_cuda()
-    t_plan = time.perf_counter() - t0
-    n = apr.total_number_particles()
-
-    torch.manual_seed(0)
-    x = torch.randn(1, CIN, n, device=dev)
-    if args.features == "bf16":
-        x = x.to(torch.bfloat16)
-    conv = aprnet.cuda.APRConv(CIN, COUT, nstencils=nstencils, kernel_size=(3, 3, 3), bias=True).to(dev)
-    ld = torch.zeros(1, dtype=torch.int32)
-    lib = _native.hip()
-
-    with torch.no_grad():
-        for _ in range(args.warmup):
-            y = conv(x, [apr], ld)
-        torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        for _ in range(args.steps):
-            y = conv(x, [apr], ld)
-        torch.cuda.synchronize()
-        dt = time.perf_counter() - t0
-
-        # duration of the convolution kernel alone: HIP events around its launch, on its stream
-        lib.aprnet_profile_enable(1)
-        kms = []
-        for _ in range(args.steps):
-            y = conv(x, [apr], ld)
-            kms.append(float(lib.aprnet_profile_last_ms()))
-        lib.aprnet_profile_enable(0)
-    kernel_ms = sum(kms) / len(kms)
-    assert torch.isfinite(y.float()).all()
-    bf16 = args.features == "bf16"
-
-    ms_per_step = dt / args.steps * 1e3
-    value = n / (dt / args.steps)
-    tflops = FLOP_PER_PARTICLE * n / (kernel_ms * 1e-3) / 1e12
-    gbs = (BYTES_PER_PARTICLE if args.features == "f32" else BYTES_PER_PARTICLE // 2 + 1) * n / (kernel_ms * 1e-3) / 1e9
-    out = {
-        "metric": "APRConv 3x3x3 fwd particles/s (Cin=Cout=32)",
-        "value": value, "unit": "particles/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "bf16" if bf16 else "f32", "data": "synthetic",
-        "config": {"workload": f"APRConv 3x3x3 32->32 {'bf16' if bf16 else 'fp32'} forward (restrict + tree fill + conv + bias), batch 1, "
-                               "APR of the seeded 512x512x256 volume with 2000 ellipsoidal blobs (configs[1])",
-                   "n_particles": n, "nstencils": nstencils, "level_max": apr.level_max(),
-                   "apr_build_s": round(t_build, 2), "plan_create_s": round(t_plan, 2)},
-        "roofline": {"bound": "mfma", "achieved": tflops, "peak": PEAK_BF16_MATRIX_TFLOPS if bf16 else PEAK_FP32_MATRIX_TFLOPS,
-                     "unit": "TFLOP/s", "frac": tflops / (PEAK_BF16_MATRIX_TFLOPS if bf16 else PEAK_FP32_MATRIX_TFLOPS),
-                     "traffic": None if bf16 else MEASURED_TRAFFIC_BYTES.get(n),
-                     "kernel": "conv_mfma_bf16_kernel" if bf16 else "conv_mfma16_kernel", "kernel_ms": kernel_ms,
-                     "hbm_achieved_GBs": gbs, "hbm_frac": gbs / PEAK_HBM_GBS},
-    }
-    if args.calibrate_copy:
-        torch.empty_like(x).copy_(x)
-        torch.cuda.synchronize()
-        print(json.dumps({"calibration_copy_bytes_read": x.numel() * 4, "calibration_copy_bytes_written": x.numel() * 4}),
-              file=sys.stderr, flush=True)
-    if args.ops:
-        for line in other_ops(apr, x, dev):
-            print(json.dumps(line), file=sys.stderr, flush=True)
-    if not args.no_cpu_baseline:
-        out["cpu_baseline"] = cpu_baseline(nstencils)
+    out = RUNNERS[args.config](args, dev, _native.hip())
     print(json.dumps(out), flush=True)
 
 

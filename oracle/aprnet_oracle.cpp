@@ -664,6 +664,9 @@ int conv_bwd_dispatch(int kz, int kx, int ky, const Acc& a, const Acc& t, const 
 
 extern "C" {
 
+// thread count of the OpenMP regions (the CPU baseline is timed with one thread and with all cores)
+int oracle_set_threads(int n) { const int before = omp_get_max_threads(); if (n > 0) omp_set_num_threads(n); return before; }
+
 int64_t oracle_number_parts(const AccessDesc* a, const AccessDesc* t, int d) { return number_parts(Acc(a), Acc(t), d); }
 int64_t oracle_tree_offset(const AccessDesc* a, const AccessDesc* t, int level) { return tree_offset(Acc(a), Acc(t), level); }
 

@@ -47,6 +47,11 @@ def lib():
     return _LIB
 
 
+def set_threads(n):
+    """Sets the OpenMP thread count of the oracle; returns the previous maximum."""
+    return int(lib().oracle_set_threads(int(n)))
+
+
 def _desc(it):
     d = _Desc()
     d.level_min, d.level_max = it.level_min(), it.level_max()

@@ -102,3 +102,22 @@ def test_hip_path_matches_the_frozen_vectors(vec, tag):
         img = _ops.reconstruct_forward([apr], x, ld)
         assert np.array_equal(img.cpu().numpy(), vec[f"{tag}/reconstruct/y"])
         _close(_ops.sample_particles_forward([apr], img, ld), vec[f"{tag}/sample_particles/y"], tol)
+
+
+def test_spheres128_golden_summary_matches_the_oracle():
+    """BASELINE configs[0] on the CPU: the builder reproduces the committed particle counts per level and the oracle
+    reproduces the committed per-channel sums and first / last 64 output values (the cross-machine check)."""
+    import json
+    import os
+    import sys
+    here = os.path.dirname(os.path.abspath(__file__))
+    sys.path.insert(0, os.path.join(here, "golden"))
+    import make_spheres128
+    gold = json.load(open(os.path.join(here, "golden", "spheres128_conv_1to16.json")))
+    now = make_spheres128.summary(*make_spheres128.oracle_output())
+    assert now["n_particles"] == gold["n_particles"] and now["levels"] == gold["levels"]
+    scale = max(gold["abs_max"])
+    for c in range(16):
+        assert abs(now["sum"][c] - gold["sum"][c]) <= 1e-6 * scale * gold["n_particles"] ** 0.5
+        assert max(abs(a - b) for a, b in zip(now["first64"][c], gold["first64"][c])) <= 1e-6 * scale
+        assert max(abs(a - b) for a, b in zip(now["last64"][c], gold["last64"][c])) <= 1e-6 * scale
