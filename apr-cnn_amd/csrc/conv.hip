@@ -155,6 +155,8 @@ int bf16_math() { return g_bf16_math; }
 int bf16_regroup() { return g_bf16_regroup; }
 static int g_bwd_overlap = 1;    // backward: weight gradient on a second stream next to the input gradient
 int backward_overlap() { return g_bwd_overlap; }
+static int g_bwd_deterministic = 1;   // backward: weight gradient summed in a fixed order (partial sums per workgroup) instead of atomics
+int bwd_deterministic() { return g_bwd_deterministic; }
 
 // Points the kernel at the plan's window lists.  When the lists are switched off, or cannot be built (no device
 // memory for them, too many entries), a.tile_win stays null and the kernel scans the access arrays itself.
@@ -353,10 +355,12 @@ int aprnet_set_conv_path(int path) {
     if (path == 4 || path == 5) { g_use_lists = path == 4; return 0; }
     if (path == 6 || path == 7) { g_bwd_overlap = path == 6; return 0; }
     if (path == 8 || path == 9) { g_bf16_regroup = path == 8; return 0; }
+    if (path == 10 || path == 11) { g_bwd_deterministic = path == 10; return 0; }
     if (path != 0 && path != 1)
         return fail(APRNET_ERR_INVALID_ARGUMENT, "set_conv_path: 0 (auto), 1 (VALU only), 2 / 3 (bfloat16 features: bfloat16 / fp32 "
                                                  "matrix math), 4 / 5 (forward: window lists of the plan / scan per call), 6 / 7 (backward on two streams / one), "
-                                                 "8 / 9 (bfloat16 forward: regrouped copy of the input / channel planes)");
+                                                 "8 / 9 (bfloat16 forward: regrouped copy of the input / channel planes), 10 / 11 (weight gradient: "
+                                                 "fixed-order partial sums / atomic additions)");
     g_conv_path = path;
     return 0;
 }

@@ -248,6 +248,17 @@ int interleave8_bf16(const bf16_t* x, int64_t ldx, const bf16_t* x2, int64_t ldx
                      hipStream_t st);
 int bf16_regroup();
 int bf16_math();
+int bwd_deterministic();
+int conv_dw_partial_blocks(int code, int Cout, int Cin);
+size_t conv_dw_partial_bytes(int code, int Cout, int Cin);
+// Points the weight-gradient kernels at their partial-sum slots, `off` bytes into the plan's scratch buffer (behind
+// whatever the input gradient keeps there: the two run side by side).
+template <typename T>
+static void set_dw_partials(aprnet_plan* p, size_t off, int code, ConvArgs<T>& a) {
+    a.gw_part = (float*)((char*)p->d_scratch + off);
+    a.gw_part_ld = (int64_t)a.Cout * a.Cin * (code == 333 ? 27 : code == 133 ? 9 : 25);
+    a.gw_part_blocks = conv_dw_partial_blocks(code, a.Cout, a.Cin);
+}
 
 template <typename T> static int try_mfma_bwd(aprnet_plan*, const ConvArgs<T>&, const TileList&, int, int, hipStream_t, bool*) { return 0; }
 static int fork_side(aprnet_plan* p, hipStream_t st, hipStream_t* side);
@@ -268,10 +279,11 @@ template <> int try_mfma_bwd<float>(aprnet_plan* p, const ConvArgs<float>& a, co
     if (int rc = set_conv_lists(p, d, code, tl, c, st)) return rc;
     // everything that can allocate or fail on the host comes before the fork
     TileList near;
-    if (a.gx) {
-        if (int rc = get_tiles(p, d, code == 333 ? 2 : 1, code == 333 ? 4 : 8, &near, st, 1)) return rc;
-        if (int rc = plan_scratch(p, conv_packed_floats(code, a.S_exp, a.Cin, a.Cout, true) * sizeof(float), st)) return rc;
-    }
+    if (a.gx) if (int rc = get_tiles(p, d, code == 333 ? 2 : 1, code == 333 ? 4 : 8, &near, st, 1)) return rc;
+    const size_t wbytes = a.gx ? (conv_packed_floats(code, a.S_exp, a.Cin, a.Cout, true) * sizeof(float) + 255) / 256 * 256 : 0;
+    const size_t pbytes = bwd_deterministic() ? conv_dw_partial_bytes(code, a.Cout, a.Cin) : 0;
+    if (wbytes + pbytes) if (int rc = plan_scratch(p, wbytes + pbytes, st)) return rc;
+    if (pbytes) set_dw_partials(p, wbytes, code, c);
     hipStream_t side = st;
     if (a.gx) if (int rc = fork_side(p, st, &side)) return rc;
     SideJoin guard(p, st, side);
@@ -414,10 +426,12 @@ int conv_bwd_bf16(const aprnet_plan* cp, int d, int kz, int kx, int ky, const bf
         const size_t wbytes = (conv_packed_bf16_bytes(code, S_exp, Cin, Cout) + 255) / 256 * 256;
         const size_t ng = (size_t)(Cout + 7) / 8, ibytes = ng * (size_t)np * 16;
         const bool regroup = bf16_regroup() && np < (1ll << 28) && ibytes <= ((size_t)32 << 30);
-        if (near.n > 0) {
-            const size_t need = b.tile_win ? wbytes + (regroup ? ibytes : 0) : conv_packed_floats(code, S_exp, Cin, Cout, true) * sizeof(float);
-            if (int rc = plan_scratch(p, need, st)) return rc;
-        }
+        size_t need = 0;
+        if (near.n > 0) need = b.tile_win ? wbytes + (regroup ? ibytes : 0) : conv_packed_floats(code, S_exp, Cin, Cout, true) * sizeof(float);
+        need = (need + 255) / 256 * 256;
+        const size_t pbytes = bwd_deterministic() ? conv_dw_partial_bytes(code, Cout, Cin) : 0;
+        if (need + pbytes) if (int rc = plan_scratch(p, need + pbytes, st)) return rc;
+        if (pbytes) set_dw_partials(p, need, code, a);
         hipStream_t side = st;
         if (near.n > 0) if (int rc = fork_side(p, st, &side)) return rc;
         SideJoin guard(p, st, side);

@@ -257,8 +257,11 @@ conv_dw16_mfma_kernel(const ConvArgs<T> a, const int s_idx) {
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
                 const int co = 4 * (lane >> 4) + r, t = (lane & 15) + 16 * tile;
-                if (t < G::K && ci < a.Cin && co < a.Cout && acc[q][tile][r] != 0.f)
-                    unsafeAtomicAdd(a.gw + (((int64_t)s_idx * a.Cout + co) * a.Cin + ci) * G::K + t, acc[q][tile][r]);
+                if (t < G::K && ci < a.Cin && co < a.Cout) {
+                    const int64_t e = ((int64_t)co * a.Cin + ci) * G::K + t;
+                    if (a.gw_part) a.gw_part[(int64_t)(2 * blockIdx.x + kh) * a.gw_part_ld + e] = acc[q][tile][r];
+                    else if (acc[q][tile][r] != 0.f) unsafeAtomicAdd(a.gw + (int64_t)s_idx * a.Cout * a.Cin * G::K + e, acc[q][tile][r]);
+                }
             }
     }
 }
@@ -409,8 +412,11 @@ conv_dw_bf16_kernel(const ConvArgs<bf16_t> a, const int s_idx) {
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
             const int co = co0 + 8 * (r >> 2) + 4 * hi + (r & 3);
-            if (t < G::K && ci < a.Cin && co < a.Cout && acc[q][r] != 0.f)
-                unsafeAtomicAdd(a.gw + (((int64_t)s_idx * a.Cout + co) * a.Cin + ci) * G::K + t, acc[q][r]);
+            if (t < G::K && ci < a.Cin && co < a.Cout) {
+                const int64_t e = ((int64_t)co * a.Cin + ci) * G::K + t;
+                if (a.gw_part) a.gw_part[(int64_t)(2 * blockIdx.x + kh) * a.gw_part_ld + e] = acc[q][r];
+                else if (acc[q][r] != 0.f) unsafeAtomicAdd(a.gw + (int64_t)s_idx * a.Cout * a.Cin * G::K + e, acc[q][r]);
+            }
         }
     }
 }
@@ -478,10 +484,39 @@ conv_dw_mfma_kernel(const ConvArgs<T> a, const int s_idx) {
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
             const int co = co0 + 8 * (r >> 2) + 4 * hi + (r & 3);
-            if (t < G::K && ci < a.Cin && co < a.Cout && acc[q][r] != 0.f)
-                unsafeAtomicAdd(a.gw + (((int64_t)s_idx * a.Cout + co) * a.Cin + ci) * G::K + t, acc[q][r]);
+            if (t < G::K && ci < a.Cin && co < a.Cout) {
+                const int64_t e = ((int64_t)co * a.Cin + ci) * G::K + t;
+                if (a.gw_part) a.gw_part[(int64_t)(2 * blockIdx.x + kh) * a.gw_part_ld + e] = acc[q][r];
+                else if (acc[q][r] != 0.f) unsafeAtomicAdd(a.gw + (int64_t)s_idx * a.Cout * a.Cin * G::K + e, acc[q][r]);
+            }
         }
     }
+}
+
+// gw[e] += sum of part[slot][e] over the slots, in slot order: one thread per element, coalesced over e.
+__global__ void dw_reduce_kernel(const float* __restrict__ part, int64_t ld, int slots, int64_t n, float* __restrict__ gw) {
+    for (int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; e < n; e += (int64_t)gridDim.x * blockDim.x) {
+        float s0 = 0.f, s1 = 0.f, s2 = 0.f, s3 = 0.f;
+        int k = 0;
+        for (; k + 3 < slots; k += 4) {
+            s0 += part[(int64_t)k * ld + e]; s1 += part[(int64_t)(k + 1) * ld + e];
+            s2 += part[(int64_t)(k + 2) * ld + e]; s3 += part[(int64_t)(k + 3) * ld + e];
+        }
+        for (; k < slots; ++k) s0 += part[(int64_t)k * ld + e];
+        gw[e] += (s0 + s1) + (s2 + s3);
+    }
+}
+
+// Workgroups of one weight-gradient launch when its partial sums go to a buffer: at most 512, fewer for very wide
+// layers so that the buffer (two slots per workgroup) stays within 512 MiB.
+int conv_dw_partial_blocks(int code, int Cout, int Cin) {
+    const int64_t e = (int64_t)Cout * Cin * (code == 333 ? 27 : code == 133 ? 9 : 25);
+    const int64_t cap = ((int64_t)512 << 20) / (8 * e);
+    return (int)std::max<int64_t>(16, std::min<int64_t>(512, cap));
+}
+size_t conv_dw_partial_bytes(int code, int Cout, int Cin) {
+    const int64_t e = (int64_t)Cout * Cin * (code == 333 ? 27 : code == 133 ? 9 : 25);
+    return (size_t)(2 * conv_dw_partial_blocks(code, Cout, Cin)) * e * sizeof(float);
 }
 
 // Weight gradient; a.gw is accumulated into (the caller zeroes it).
@@ -500,7 +535,17 @@ static int launch_dw(const ConvArgs<T>& a0, const TileList& tl, int level_min, h
         if (a.tile_win) a.tile_win += tl.level_begin[l_hi];
         // a narrow input (the first layer of a network) fits one chunk: no staging and products of empty chunks
         const int nch = a.Cin <= DW_CIB ? 1 : DW_NCH;
-        dim3 grid((unsigned)std::min(n, 512), (unsigned)((a.Cin + DW_CIB * nch - 1) / (DW_CIB * nch)), (unsigned)((a.Cout + 31) / 32));
+        const int gmax = a.gw_part ? a.gw_part_blocks : 512;
+        dim3 grid((unsigned)std::min(n, gmax), (unsigned)((a.Cin + DW_CIB * nch - 1) / (DW_CIB * nch)), (unsigned)((a.Cout + 31) / 32));
+        const int64_t n_el = (int64_t)a.Cout * a.Cin * G::K;
+        // the partial sums of this launch, added up in slot order (every slot of the grid is written in full)
+        auto reduce = [&]() -> int {
+            if (!a.gw_part) return 0;
+            hipLaunchKernelGGL(dw_reduce_kernel, dim3((unsigned)std::min<int64_t>((n_el + 255) / 256, 2048)), dim3(256), 0, st,
+                               (const float*)a.gw_part, a.gw_part_ld, 2 * (int)grid.x, n_el, (float*)a.gw + (int64_t)s * n_el);
+            APRNET_LAUNCH_CHECK("dw_reduce_kernel");
+            return 0;
+        };
         if constexpr (std::is_same<T, bf16_t>::value) {
             if (bf16_math()) {      // bfloat16 matrix instructions; the fp32 ones below when those are asked for
                 if (nch == 1) {
@@ -509,6 +554,7 @@ static int launch_dw(const ConvArgs<T>& a0, const TileList& tl, int level_min, h
                 } else if (a.tile_win) hipLaunchKernelGGL((conv_dw_bf16_kernel<G, DW_CIB, DW_NCH, true>), grid, dim3(G::NT), 0, st, a, s);
                 else hipLaunchKernelGGL((conv_dw_bf16_kernel<G, DW_CIB, DW_NCH, false>), grid, dim3(G::NT), 0, st, a, s);
                 APRNET_LAUNCH_CHECK("conv_dw_bf16_kernel");
+                if (int rc = reduce()) return rc;
                 continue;
             }
         }
@@ -519,6 +565,7 @@ static int launch_dw(const ConvArgs<T>& a0, const TileList& tl, int level_min, h
             } else if (a.tile_win) hipLaunchKernelGGL((conv_dw16_mfma_kernel<T, G, DW_CIB, DW_NCH, true>), grid, dim3(G::NT), 0, st, a, s);
             else hipLaunchKernelGGL((conv_dw16_mfma_kernel<T, G, DW_CIB, DW_NCH, false>), grid, dim3(G::NT), 0, st, a, s);
             APRNET_LAUNCH_CHECK("conv_dw16_mfma_kernel");
+            if (int rc = reduce()) return rc;
             continue;
         }
         if (nch == 1) {
@@ -527,6 +574,7 @@ static int launch_dw(const ConvArgs<T>& a0, const TileList& tl, int level_min, h
         } else if (a.tile_win) hipLaunchKernelGGL((conv_dw_mfma_kernel<T, G, DW_CIB, DW_NCH, true>), grid, dim3(G::NT), 0, st, a, s);
         else hipLaunchKernelGGL((conv_dw_mfma_kernel<T, G, DW_CIB, DW_NCH, false>), grid, dim3(G::NT), 0, st, a, s);
         APRNET_LAUNCH_CHECK("conv_dw_mfma_kernel");
+        if (int rc = reduce()) return rc;
     }
     return 0;
 }

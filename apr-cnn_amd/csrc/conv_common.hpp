@@ -44,6 +44,10 @@ struct ConvArgs {
     // gradients are accumulated in the computation type (fp32 for bfloat16 features)
     const T* gy; typename Num<T>::acc* gx; int64_t ldgx; typename Num<T>::acc* gtree; int64_t ldgt;
     typename Num<T>::acc* gw; int n_tiles;
+    // Weight gradient without atomics: every persistent workgroup writes the sums of its tiles to two slots (one per
+    // half of the columns) of gw_part [2 * gw_part_blocks][gw_part_ld], which a second kernel adds up in slot order and
+    // adds to gw, so the result does not depend on scheduling (null: atomic additions to gw).
+    typename Num<T>::acc* gw_part; int64_t gw_part_ld; int gw_part_blocks;
     // window lists built once per APR and kept in the plan (kernels that do not scan)
     const int* tile_win;                       // [n_tiles + 1] first stored window of every tile
     const int4* win;                           // per stored window: {first item, items, first column, columns}; the two

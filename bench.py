@@ -81,6 +81,11 @@ def level_counts(apr):
     return out
 
 
+def say(msg):
+    """Progress line on stderr (long configurations would otherwise be silent for minutes)."""
+    print("# " + msg, file=sys.stderr, flush=True)
+
+
 def host_cores():
     return int(os.environ.get("OMP_NUM_THREADS", 0)) or len(os.sched_getaffinity(0))
 
@@ -115,24 +120,25 @@ def cpu_baseline_conv(apr, cin, cout, ksize, nstencils, sample, budget_s=25.0):
     res = {}
     for threads in (cores, 1):
         before = oracle.set_threads(threads)
+        say(f"cpu baseline: {n} particles on {threads} thread(s)")
         t0 = time.perf_counter()
         run()                                       # warm-up, also sizes the number of timed runs
         first = time.perf_counter() - t0
-        runs = 5 if first * 6 < budget_s else (3 if first * 4 < budget_s else 1)
+        runs = 5 if first * 6 < budget_s else (3 if first * 4 < budget_s else (1 if first * 2 < budget_s else 0))
         ts = []
         for _ in range(runs):
             t0 = time.perf_counter()
             run()
             ts.append(time.perf_counter() - t0)
         oracle.set_threads(before)
-        res[threads] = (statistics.median(ts), runs)
+        # a run too long for the budget is its own (un-warmed) measurement
+        res[threads] = (statistics.median(ts), f"1 warm-up + median of {runs}") if runs else (first, "one run without warm-up")
     t_all, r_all = res[cores]
     t_one, r_one = res[1]
     return {"value": n / t_all, "unit": "particles/s", "cores": cores, "kind": "port",
             "value_1_thread": n / t_one, "cpu": cpu_model(),
             "sample": f"{sample}, {n} particles, conv {ksize[0]}x{ksize[1]}x{ksize[2]} {cin}->{cout} fp32 forward incl. weight "
-                      f"expansion; 1 warm-up + median of {r_all} runs on {cores} threads ({t_all:.2f} s each), "
-                      f"median of {r_one} on 1 thread ({t_one:.2f} s each)"}
+                      f"expansion; {cores} threads: {r_all}, {t_all:.2f} s per run; 1 thread: {r_one}, {t_one:.2f} s per run"}
 
 
 def _time(fn, iters=10, warmup=2):
@@ -352,6 +358,7 @@ def run_spheres128(args, dev, lib):
 
 
 def _largest_apr(name, img, limit=(1 << 30) - 1):
+    say(f"{name}: volume {img.shape} synthesised, building the APR")
     """The APR of the whole volume when it stays within the particle limit of a plan, otherwise of the largest
     centre crop (halving z, then x, then y) that does.  -> (apr, description)."""
     import numpy as np
@@ -375,12 +382,13 @@ def run_nuclei2048(args, dev, lib):
     from pyapr.aprnet import _ops
     C = 16
     t0 = time.perf_counter()
+    say("nuclei2048: synthesising the 512x2048x2048 volume")
     img = build_volume("nuclei2048")
     apr, what = _largest_apr("nuclei2048", img)
     t_build = time.perf_counter() - t0
     apr.init_cuda()
     n, nt = apr.total_number_particles(), _ops.tree_parts(apr, 0)
-    print(f"# nuclei2048: {n} particles ({what}), {nt} tree nodes, built in {t_build:.0f} s", file=sys.stderr, flush=True)
+    say(f"nuclei2048: {n} particles ({what}), {nt} tree nodes, built in {t_build:.0f} s")
     torch.manual_seed(0)
     x = torch.randn(1, C, n, device=dev)
     conv = aprnet.cuda.APRConv(C, C, nstencils=2).to(dev)
@@ -411,12 +419,13 @@ def run_nuclei1024(args, dev, lib):
     """configs[3]: forward of the 4-level APR-UNet (16-32-64-128, norms folded, He init seed 0), fp32 and bfloat16."""
     import torch
     t0 = time.perf_counter()
+    say("nuclei1024: synthesising the 1024^3 volume")
     img = build_volume("nuclei1024")
     apr, what = _largest_apr("nuclei1024", img)
     t_build = time.perf_counter() - t0
     apr.init_cuda()
     n = apr.total_number_particles()
-    print(f"# nuclei1024: {n} particles ({what}), built in {t_build:.0f} s", file=sys.stderr, flush=True)
+    say(f"nuclei1024: {n} particles ({what}), built in {t_build:.0f} s")
     parts = torch.randn(1, 1, n, device=dev)
     net = make_unet(dev)
     res = {}
@@ -432,7 +441,7 @@ def run_nuclei1024(args, dev, lib):
             except RuntimeError as e:           # torch.OutOfMemoryError, or a failed allocation inside the library
                 res[name] = {"ms": None, "error": str(e).split("\n")[0][:200]}
             torch.cuda.empty_cache()
-            print(f"# nuclei1024 {name}: {res[name]}", file=sys.stderr, flush=True)
+            say(f"nuclei1024 {name}: {res[name]}")
     ms = res["bf16"]["ms"] or res["f32"]["ms"]
     out = base_line("APR-UNet fwd latency (ms), 4 levels 16-32-64-128", ms, "ms", args, ms, "bf16",
                     {"workload": f"APR-UNet forward, 4 levels 16-32-64-128, two 3x3x3 convolutions + ReLU per level, norms folded, 1x1x1 head "
@@ -457,7 +466,7 @@ def run_spots16k(args, dev, lib):
     t_build = time.perf_counter() - t0
     apr.init_cuda()
     n = apr.total_number_particles()
-    print(f"# spots16k: {n} particles, built in {t_build:.0f} s", file=sys.stderr, flush=True)
+    say(f"spots16k: {n} particles, built in {t_build:.0f} s")
     conv = aprnet.cuda.APRConv(C, C, nstencils=2, kernel_size=(1, 5, 5)).to(dev)
     ld = torch.zeros(1, dtype=torch.int32)
     x = torch.randn(1, C, n, device=dev).to(torch.bfloat16)
@@ -466,6 +475,7 @@ def run_spots16k(args, dev, lib):
         sec = _steps(lambda: conv(x, [apr], ld), steps, 1)
         kernel_ms = _kernel_ms(lib, lambda: conv(x, [apr], ld), 3)
     extra = {"fwd_ms": sec * 1e3, "fwd_peak_device_GB": torch.cuda.max_memory_allocated() / 1e9}
+    say(f"spots16k forward: {sec * 1e3:.1f} ms per step, kernel {kernel_ms:.1f} ms")
     # the backward of the layer at full size needs the features, two gradients and an fp32 gradient work space at
     # 64 channels: run when it fits, otherwise on the 4096^2 corner of the same image
     try:
@@ -474,10 +484,12 @@ def run_spots16k(args, dev, lib):
         go = torch.randn_like(y)
         extra["bwd_ms"] = _time(lambda: torch.autograd.grad(y, (xg, conv.weight), go, retain_graph=True), iters=2, warmup=1)
         extra["bwd_sample"] = "whole image"
+        say(f"spots16k backward (whole image): {extra['bwd_ms']:.1f} ms")
         del y, go
     except RuntimeError:                        # out of device memory
         xg = y = go = None
         torch.cuda.empty_cache()
+        say("spots16k backward does not fit at full size: 4096^2 crop")
         small = build_workload("spots16k", crop=(1, 4096, 4096), img=img)
         ns = small.total_number_particles()
         xs = torch.randn(1, C, ns, device=dev).to(torch.bfloat16).requires_grad_(True)
@@ -493,9 +505,9 @@ def run_spots16k(args, dev, lib):
     out["roofline"] = mfma_roofline(2 * 25 * C * C * n, kernel_ms, PEAK_BF16_MATRIX_TFLOPS, "conv_mfma_bf16_kernel", (2 * 2 * C + 2) * n)
     out["extra"] = extra
     if not args.no_cpu_baseline:
-        crop = (1, 2048, 2048)
+        crop = (1, 1024, 1024)
         out["cpu_baseline"] = cpu_baseline_conv(build_workload("spots16k", crop=crop, img=img), C, C, (1, 5, 5), 2,
-                                                "centre crop 2048x2048 of the 16384^2 image")
+                                                "centre crop 1024x1024 of the 16384^2 image")
     return out
 
 
@@ -713,9 +725,19 @@ def main():
         sys.exit("bench.py: this build runs on one GPU; --gpus N with N > 1 is not supported "
                  "(the path would shard by batch item, or by z-slabs with a one-row halo per level)")
 
+    import threading
     import torch
     from pyapr import _native
     assert torch.cuda.is_available(), "bench.py needs a GPU"
+    if args.config != "blobs512":
+        # the large configurations spend minutes in native host code (volume synthesis, APR build, CPU baseline)
+        t_start = time.perf_counter()
+
+        def heartbeat():
+            while True:
+                time.sleep(60)
+                say(f"{args.config}: working, {time.perf_counter() - t_start:.0f} s")
+        threading.Thread(target=heartbeat, daemon=True).start()
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
     out = RUNNERS[args.config](args, dev, _native.hip())

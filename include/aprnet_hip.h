@@ -98,7 +98,10 @@ int aprnet_profile_enable(int on);
  * to the caller's stream with events (default), 7 = both on the caller's stream; and for the bfloat16 forward
  * kernel: 8 = stage from a copy of the input regrouped as [Cin / 8][particles][8] in the plan's scratch buffer, one
  * 16-byte load per item and 8 channels (default; 16 bytes per particle and 8 channels of device memory, made by one
- * streaming pass per call), 9 = gather from the channel planes.  All are HIP kernels; the switch
+ * streaming pass per call), 9 = gather from the channel planes; and for the weight gradient of the matrix-core
+ * kernels: 10 = every workgroup writes the sums of its tiles to its own slots of the plan's scratch buffer and a second
+ * kernel adds the slots in a fixed order (default: the gradient repeats bit for bit from run to run; at most 512 MiB
+ * of scratch), 11 = atomic additions.  All are HIP kernels; the switch
  * exists so that tests can cover them and memory-bound callers can do without the lists. */
 int aprnet_set_conv_path(int path);
 float aprnet_profile_last_ms(void);

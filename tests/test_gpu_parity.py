@@ -600,7 +600,7 @@ def test_conv_bf16_regrouped_input_equals_channel_planes(ksize, c1, c2, cout):
     scale = float(res[9][2].float().abs().max())
     assert float((res[8][2].float() - res[9][2].float()).abs().max()) <= 1e-2 * scale      # one bfloat16 rounding step
     assert float((res[8][3] - res[9][3]).abs().max()) <= 1e-5 * float(res[9][3].abs().max())
-    assert lib.aprnet_set_conv_path(10) != 0
+    assert lib.aprnet_set_conv_path(12) != 0
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float64, torch.bfloat16], ids=["f32", "f64", "bf16"])
