@@ -85,6 +85,17 @@ struct WinLists {
     bool unavailable = false;                   // building them failed once (no memory, too many entries): do not retry
 };
 
+// Particles that stick out of a far face of the next finer level, with the (output, tap) pairs that read them
+// (faces.hip); device arrays owned by the plan.
+struct FaceLists {
+    int n_part = 0;
+    int* d_part_idx = nullptr;                  // [n_part] index of the particle in the input gradient
+    int* d_part_level = nullptr;                // [n_part] level of the outputs that read it (its own level + 1)
+    int* d_pair_begin = nullptr;                // [n_part + 1]
+    int* d_pair_out = nullptr;                  // [pairs] index into the output gradient
+    unsigned char* d_pair_tap = nullptr;        // [pairs]
+};
+
 }  // namespace aprnet
 
 struct aprnet_plan {
@@ -101,6 +112,7 @@ struct aprnet_plan {
     hipStream_t scratch_stream = nullptr;                         // stream of the last call that used the buffer
     bool scratch_stream_valid = false, scratch_stream_capturing = false;
     std::map<std::pair<int, int>, aprnet::WinLists> lists;        // (level_delta, stencil code) -> window lists
+    std::map<std::pair<int, int>, aprnet::FaceLists> faces;       // (level_delta, stencil code) -> far-face particles
     // second stream of the convolution backward (weight gradient next to input gradient), with its fork / join events
     hipStream_t side = nullptr; hipEvent_t ev_fork = nullptr, ev_join = nullptr;
 
@@ -127,6 +139,8 @@ int get_tiles(aprnet_plan* plan, int level_delta, int TZ, int TX, TileList* out,
 bool stream_is_capturing(hipStream_t st);
 int get_lists(aprnet_plan* plan, int level_delta, int code, const TileList& tl, WinLists* out, hipStream_t st, bool dx = false);
 void free_lists(WinLists& wl);
+int get_face_lists(aprnet_plan* plan, int level_delta, int code, FaceLists* out, hipStream_t st);
+void free_face_lists(FaceLists& fl);
 // Makes plan->d_scratch at least `bytes` large for a call on `st` (contents are lost when it grows).  A buffer that a
 // captured graph may address is never freed before the plan is destroyed; growth while `st` is capturing is refused
 // with APRNET_ERR_UNSUPPORTED (reserve first: aprnet_plan_reserve, or run the call once outside the capture).  A call on

@@ -249,6 +249,8 @@ int interleave8_bf16(const bf16_t* x, int64_t ldx, const bf16_t* x2, int64_t ldx
 int bf16_regroup();
 int bf16_math();
 int bwd_deterministic();
+int launch_face_dx(const FaceLists& fl, const float* gy, int64_t ldy, const float* w, int S_exp, int Cout, int Cin, int K, int Lc,
+                   float* gx, int64_t ldgx, hipStream_t st);
 int conv_dw_partial_blocks(int code, int Cout, int Cin);
 size_t conv_dw_partial_bytes(int code, int Cout, int Cin);
 // Points the weight-gradient kernels at their partial-sum slots, `off` bytes into the plan's scratch buffer (behind
@@ -279,7 +281,10 @@ template <> int try_mfma_bwd<float>(aprnet_plan* p, const ConvArgs<float>& a, co
     if (int rc = set_conv_lists(p, d, code, tl, c, st)) return rc;
     // everything that can allocate or fail on the host comes before the fork
     TileList near;
+    FaceLists faces;
+    const bool split_faces = a.gx && bwd_deterministic();
     if (a.gx) if (int rc = get_tiles(p, d, code == 333 ? 2 : 1, code == 333 ? 4 : 8, &near, st, 1)) return rc;
+    if (split_faces) if (int rc = get_face_lists(p, d, code, &faces, st)) return rc;
     const size_t wbytes = a.gx ? (conv_packed_floats(code, a.S_exp, a.Cin, a.Cout, true) * sizeof(float) + 255) / 256 * 256 : 0;
     const size_t pbytes = bwd_deterministic() ? conv_dw_partial_bytes(code, a.Cout, a.Cin) : 0;
     if (wbytes + pbytes) if (int rc = plan_scratch(p, wbytes + pbytes, st)) return rc;
@@ -296,7 +301,12 @@ template <> int try_mfma_bwd<float>(aprnet_plan* p, const ConvArgs<float>& a, co
         b.tiles = near.d_tiles; b.n_tiles = near.n;
         b.x = a.gy; b.ldx = a.ldy; b.Cin = a.Cout; b.Cout = a.Cin; b.w = (const float*)p->d_scratch; b.bias = nullptr;
         b.tree_data = nullptr; b.t_count = 0;
+        b.dx_skip_faces = split_faces ? 1 : 0;
         if (near.n > 0) if (int rc = launch_conv_dx_mfma(code, b, near.n, st)) return rc;
+        // coarser particles with cells outside their finer level: summed pair by pair in list order
+        if (split_faces)
+            if (int rc = launch_face_dx(faces, a.gy, a.ldy, a.w, a.S_exp, a.Cout, a.Cin, code == 333 ? 27 : code == 133 ? 9 : 25, a.Lc,
+                                        a.gx, a.ldgx, st)) return rc;
     }
     return guard.join();
 }

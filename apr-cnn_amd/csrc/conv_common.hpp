@@ -48,6 +48,9 @@ struct ConvArgs {
     // half of the columns) of gw_part [2 * gw_part_blocks][gw_part_ld], which a second kernel adds up in slot order and
     // adds to gw, so the result does not depend on scheduling (null: atomic additions to gw).
     typename Num<T>::acc* gw_part; int64_t gw_part_ld; int gw_part_blocks;
+    // input-gradient scan: leave out the coarser particles that stick out of a far face of the level (some of the
+    // cells they would cover do not exist); a separate kernel adds their gradient (faces.hip)
+    int dx_skip_faces;
     // window lists built once per APR and kept in the plan (kernels that do not scan)
     const int* tile_win;                       // [n_tiles + 1] first stored window of every tile
     const int4* win;                           // per stored window: {first item, items, first column, columns}; the two
@@ -161,6 +164,7 @@ struct ScanArgs {
     bool tree_from_x, out_tree;
     int z0, x0, zn, xn;             // tile origin and level extent (input-gradient scan only)
     bool pool;                      // input-gradient scan: one pooled column per coarser particle (COL_BOX)
+    bool skip_faces;                // input-gradient scan: no columns for coarser particles with cells outside the level
 };
 
 template <class G>
@@ -328,8 +332,9 @@ __device__ __attribute__((noinline)) void scan_window_dx_impl(const ScanArgs a, 
                 const bool first_row = (BOXZ == 1 || (z & 1) == 0) && (x & 1) == 0;
                 const bool ina = in && ya >= y0 && ya < y0 + G::TY;
                 const bool pooled = a.pool && rows_full && yb < yn;
-                const bool oa = ina && (!pooled || first_row);
-                const bool ob = in && !pooled && yb >= y0 && yb < y0 + G::TY && yb < yn;
+                const bool keep = pooled || !a.skip_faces;
+                const bool oa = ina && keep && (!pooled || first_row);
+                const bool ob = in && keep && !pooled && yb >= y0 && yb < y0 + G::TY && yb < yn;
                 const unsigned long long ma = __ballot(oa), mb = __ballot(ob);
                 if (ma | mb) {
                     int base = 0;
@@ -362,6 +367,7 @@ __device__ __forceinline__ void scan_window_dx(const ConvArgs<T>& a, int L, int 
     s.apr_y = a.apr.y; s.tree_y = a.tree.y; s.tree_off = (int)a.tree_off; s.yn = a.apr.y_num[L]; s.y0 = y0;
     s.tree_from_x = (L == a.Lc); s.out_tree = out_tree;
     s.z0 = z0; s.x0 = x0; s.zn = a.apr.z_num[L]; s.xn = a.apr.x_num[L]; s.pool = pool;
+    s.skip_faces = pool && a.dx_skip_faces != 0;
     scan_window_dx_impl<G>(s, sh);
 }
 
