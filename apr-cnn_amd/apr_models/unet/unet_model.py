@@ -53,7 +53,21 @@ class APRUNet(nn.Module):
         y = skips.pop()
         for stage in self.decoder:
             skip = skips.pop()
-            y = stage(y, skip, aprs, level_deltas)
+            if torch.is_grad_enabled():
+                y = stage(y, skip, aprs, level_deltas)
+            else:
+                # UpConv.forward (unet_parts.py:78-83) unrolled here, so that the skip tensor and the upsampled tensor
+                # are released as soon as the first convolution of the stage has read them (inside stage.forward the
+                # caller's references would keep both alive until the whole stage returns)
+                y = stage.upsample(stage.reduce_ch(y, aprs, level_deltas), aprs, level_deltas)
+                blocks = stage.conv.blocks
+                out = blocks[0](skip, aprs, level_deltas, y)
+                y = None
+                skip = None
+                for block in blocks[1:]:
+                    out = block(out, aprs, level_deltas)
+                y = out
+                del out
             del skip
         return self.head(y, aprs, level_deltas)
 

@@ -83,6 +83,8 @@ struct WinLists {
     int* d_col_idx = nullptr; unsigned short* d_col_pos = nullptr;
     int n_win = 0; int64_t n_items = 0, n_cols = 0;
     bool unavailable = false;                   // building them failed once (no memory, too many entries): do not retry
+    // the levels that have windows, in window order (finest first): first window and level of each
+    int n_lv = 0; int lv_first[MAX_LEVELS] = {}; int lv_level[MAX_LEVELS] = {};
 };
 
 // Particles that stick out of a far face of the next finer level, with the (output, tap) pairs that read them

@@ -145,6 +145,12 @@ int fill_tree_for_conv(const aprnet_plan* p, int d, const bf16_t* x, int64_t ldx
 size_t conv_packed_floats(int code, int S_exp, int Cm, int Ck, bool transposed);
 int pack_conv_weights(int code, const float* w, int S_exp, int Cm, int Ck, bool transposed, float* packed, hipStream_t st);
 
+bool conv_narrow_supported(int code, int Cin);
+size_t conv_narrow_packed_floats(int code, int S_exp, int Cout, int Cin);
+int pack_conv_weights_narrow(int code, const float* w, int S_exp, int Cout, int Cin, float* packed, hipStream_t st);
+int launch_conv_narrow(int code, const ConvArgs<float>& a, const WinLists& wl, hipStream_t st);
+int launch_conv_narrow(int code, const ConvArgs<bf16_t>& a, const WinLists& wl, hipStream_t st);
+static int g_narrow = 1;         // layers of 1 to 3 input channels: 1 = the bandwidth-shaped kernel (conv_narrow.hip), 0 = the general one
 static int g_conv_path = 0;      // 0: matrix cores where available, 1: VALU kernels only
 int conv_path() { return g_conv_path; }
 int bf16_math();
@@ -176,10 +182,31 @@ int set_conv_lists(aprnet_plan* p, int d, int code, const TileList& tl, ConvArgs
 // the input-gradient lists (tl: the tile list with a halo of one row)
 int set_conv_dx_lists(aprnet_plan* p, int d, int code, const TileList& tl, ConvArgs<bf16_t>& a, hipStream_t st) { return set_lists(p, d, code, tl, a, st, true); }
 
+// Channel-aware dispatch: a layer with 1 to 3 input channels is bound by memory (4 (Cin + Cout) bytes for 2 K Cin Cout
+// flops per particle) and goes to the pipelined kernel of conv_narrow.hip, which needs the plan's window lists and a
+// single input tensor.  *done tells whether the layer was taken.
+template <typename T>
+static int try_narrow(aprnet_plan* p, const ConvArgs<T>& a, int code, int d, const TileList& tl, hipStream_t st, bool* done) {
+    if (!g_narrow || g_conv_path == 1 || !g_use_lists || a.x2 != nullptr || !conv_narrow_supported(code, a.Cin)) return 0;
+    WinLists wl;
+    if (get_lists(p, d, code, tl, &wl, st) != 0) { (void)hipGetLastError(); return 0; }
+    *done = true;
+    if (int rc = plan_scratch(p, conv_narrow_packed_floats(code, a.S_exp, a.Cout, a.Cin) * sizeof(float), st)) return rc;
+    if (int rc = pack_conv_weights_narrow(code, (const float*)a.w, a.S_exp, a.Cout, a.Cin, (float*)p->d_scratch, st)) return rc;
+    ConvArgs<T> b = a;
+    b.w = (const float*)p->d_scratch;
+    b.tile_win = wl.d_tile_win; b.win = wl.d_win;
+    b.l_item_idx = wl.d_item_idx; b.l_item_pos = wl.d_item_pos; b.l_col_idx = wl.d_col_idx; b.l_col_pos = wl.d_col_pos;
+    TimedLaunch timed(st);
+    return launch_conv_narrow(code, b, wl, st);
+}
+
 template <typename T> static int try_mfma(aprnet_plan*, const ConvArgs<T>&, int, int, const TileList&, int, hipStream_t, bool*) { return 0; }
 template <> int try_mfma<float>(aprnet_plan* p, const ConvArgs<float>& a, int code, int d, const TileList& tl, int n_tiles,
                                 hipStream_t st, bool* done) {
     if (g_conv_path == 1 || !conv_mfma_supported(code)) return 0;
+    if (int rc = try_narrow<float>(p, a, code, d, tl, st, done)) return rc;
+    if (*done) return 0;
     *done = true;
     // plan-owned scratch for the re-laid-out weights, grown on demand
     if (int rc = plan_scratch(p, conv_packed_floats(code, a.S_exp, a.Cout, a.Cin, false) * sizeof(float), st)) return rc;
@@ -274,6 +301,17 @@ int conv_fwd_bf16(const aprnet_plan* cp, int d, int kz, int kx, int ky, const bf
     if (int rc = get_tiles(p, d, kz == 1 ? 1 : 2, kz == 1 ? 8 : 4, &tl, st)) return rc;
     if (tl.n == 0) return 0;
     ConvArgs<bf16_t> a{};
+    if (conv_narrow_supported(code, Cin) && fu.C2 == 0) {
+        // a narrow first layer: fp32 products of the bfloat16 features on the pipelined kernel
+        ConvArgs<bf16_t> n{};
+        n.apr = p->dapr; n.tree = p->dtree; n.tiles = tl.d_tiles;
+        n.x = x; n.ldx = ldx; n.Cin = Cin; n.w = w; n.S_exp = S_exp; n.Cout = Cout; n.bias = bias; n.relu = fu.relu;
+        n.y = y; n.ldy = ldy; n.tree_data = tree_ws; n.ldt = ldt; n.Lc = p->lc(d); n.tree_off = p->tree_offset(n.Lc);
+        n.x_count = p->number_parts(d); n.t_count = p->tree_parts(d);
+        bool done = false;
+        if (int rc = try_narrow<bf16_t>(p, n, code, d, tl, st, &done)) return rc;
+        if (done) return 0;
+    }
     if (int rc = set_lists(p, d, code, tl, a, st)) return rc;
     const bool bf16_math = g_bf16_math && a.tile_win;      // the bfloat16 contraction exists with window lists only
     const int64_t n_x = p->number_parts(d), n_t = p->tree_parts(d);
@@ -356,11 +394,12 @@ int aprnet_set_conv_path(int path) {
     if (path == 6 || path == 7) { g_bwd_overlap = path == 6; return 0; }
     if (path == 8 || path == 9) { g_bf16_regroup = path == 8; return 0; }
     if (path == 10 || path == 11) { g_bwd_deterministic = path == 10; return 0; }
+    if (path == 12 || path == 13) { g_narrow = path == 12; return 0; }
     if (path != 0 && path != 1)
         return fail(APRNET_ERR_INVALID_ARGUMENT, "set_conv_path: 0 (auto), 1 (VALU only), 2 / 3 (bfloat16 features: bfloat16 / fp32 "
                                                  "matrix math), 4 / 5 (forward: window lists of the plan / scan per call), 6 / 7 (backward on two streams / one), "
                                                  "8 / 9 (bfloat16 forward: regrouped copy of the input / channel planes), 10 / 11 (weight gradient: "
-                                                 "fixed-order partial sums / atomic additions)");
+                                                 "fixed-order partial sums / atomic additions), 12 / 13 (1 to 3 input channels: pipelined kernel / general kernel)");
     g_conv_path = path;
     return 0;
 }

@@ -119,6 +119,11 @@ int get_lists(aprnet_plan* p, int level_delta, int code, const TileList& tl, Win
             return fail(APRNET_ERR_UNSUPPORTED, "window lists: more than 2^32 entries");
         }
         wl.n_win = (int)nw; wl.n_items = ni; wl.n_cols = nc;
+        for (int l = MAX_LEVELS; l >= 0; --l) {        // tiles are sorted finest level first
+            if (tl.level_count[l] <= 0) continue;
+            const int fw = tile_win[tl.level_begin[l]], lw = tile_win[tl.level_begin[l] + tl.level_count[l]];
+            if (lw > fw) { wl.lv_first[wl.n_lv] = fw; wl.lv_level[wl.n_lv] = l; ++wl.n_lv; }
+        }
         auto alloc = [&](void** q, size_t bytes) -> int { APRNET_HIP_CHECK(hipMalloc(q, std::max<size_t>(bytes, 16))); return 0; };
         int rc = alloc((void**)&d_offs, (size_t)tl.n * sizeof(int4));
         if (!rc) rc = alloc((void**)&wl.d_tile_win, tile_win.size() * sizeof(int));

@@ -339,7 +339,7 @@ def run_spheres128(args, dev, lib):
                                  "spheres (configs[0]); the launch is too small to fill the GPU: the same layer shape on the "
                                  "23 M-particle APR is in the default line's extra",
                      "n_particles": n, "levels": level_counts(apr), "nstencils": 1, "level_max": apr.level_max()})
-    out["roofline"] = hbm_roofline(68 * n, kernel_ms, "forward convolution kernel of the 1->16 layer", flop=864 * n)
+    out["roofline"] = hbm_roofline(68 * n, kernel_ms, "conv_narrow_kernel", flop=864 * n)
     # cross-machine golden check of this configuration (tests/golden/spheres128_conv_1to16.json)
     gold = os.path.join(ROOT, "tests", "golden", "spheres128_conv_1to16.json")
     if os.path.exists(gold):

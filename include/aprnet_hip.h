@@ -101,7 +101,9 @@ int aprnet_profile_enable(int on);
  * streaming pass per call), 9 = gather from the channel planes; and for the weight gradient of the matrix-core
  * kernels: 10 = every workgroup writes the sums of its tiles to its own slots of the plan's scratch buffer and a second
  * kernel adds the slots in a fixed order (default: the gradient repeats bit for bit from run to run; at most 512 MiB
- * of scratch), 11 = atomic additions.  All are HIP kernels; the switch
+ * of scratch), 11 = atomic additions; and for forward layers of 1 to 3 input channels (bound by memory, not by the
+ * contraction): 12 = the pipelined kernel with the (tap, channel) axis flattened (default), 13 = the general kernel.
+ * All are HIP kernels; the switch
  * exists so that tests can cover them and memory-bound callers can do without the lists. */
 int aprnet_set_conv_path(int path);
 float aprnet_profile_last_ms(void);

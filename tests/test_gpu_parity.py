@@ -600,7 +600,7 @@ def test_conv_bf16_regrouped_input_equals_channel_planes(ksize, c1, c2, cout):
     scale = float(res[9][2].float().abs().max())
     assert float((res[8][2].float() - res[9][2].float()).abs().max()) <= 1e-2 * scale      # one bfloat16 rounding step
     assert float((res[8][3] - res[9][3]).abs().max()) <= 1e-5 * float(res[9][3].abs().max())
-    assert lib.aprnet_set_conv_path(12) != 0
+    assert lib.aprnet_set_conv_path(99) != 0
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float64, torch.bfloat16], ids=["f32", "f64", "bf16"])
@@ -751,3 +751,39 @@ def test_conv_backward_fp32_repeats_bit_for_bit_on_odd_sizes(bt, ksize):
         lib.aprnet_set_conv_path(10)
     close(gx_a, gx_ref, torch.float32)
     close(gw_a.permute(2, 0, 1, 3, 4, 5), gw_ref, torch.float32)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
+@pytest.mark.parametrize("ksize", [(3, 3, 3), (1, 3, 3), (1, 5, 5)], ids=KID)
+@pytest.mark.parametrize("cin,cout", [(1, 16), (1, 32), (2, 5), (3, 24), (2, 40)])
+def test_conv_forward_narrow_input(cin, cout, ksize, dtype):
+    """Layers of 1 to 3 input channels run on the pipelined kernel with the (tap, channel) axis flattened: against the
+    oracle (batch of two APRs at different level deltas, bias, ReLU fused for one of the two runs), against the general
+    matrix-core kernel (path 13), and bit-identical from run to run."""
+    bt = [("3d_s", 0), ("3d_t", 1)] if ksize[0] == 3 else [("2d_t", 0), ("2d_s", 1), ("3d_s", 0)]
+    x, aprs, ld, w_exp = _conv_case(bt, ksize, 2, cin, cout, torch.float32)
+    g = torch.Generator().manual_seed(41)
+    bias = torch.randn(cout, generator=g)
+    xd = x.to(dtype).to(DEV)
+    wd = w_exp.permute(1, 2, 0, 3, 4, 5).contiguous().to(DEV)
+    ref = oracle.conv_forward(aprs, xd.float().cpu(), w_exp, ld) + bias.view(1, -1, 1)
+    for b, a in enumerate(aprs):                     # the oracle leaves padding slots at zero, the modules add the bias there
+        ref[b, :, oracle.number_parts(a, int(ld[b])):] = bias.view(-1, 1)
+    lib = _native.hip()
+    got = _ops.conv_forward(aprs, xd, wd, ld, bias=bias.to(DEV))
+    again = _ops.conv_forward(aprs, xd, wd, ld, bias=bias.to(DEV))
+    fused = _ops.conv_forward(aprs, xd, wd, ld, bias=bias.to(DEV), relu=True)
+    assert lib.aprnet_set_conv_path(13) == 0
+    try:
+        general = _ops.conv_forward(aprs, xd, wd, ld, bias=bias.to(DEV))
+    finally:
+        lib.aprnet_set_conv_path(12)
+    assert torch.equal(got, again)
+    if dtype == torch.float32:
+        close(got, ref, dtype)
+        close(general, ref, dtype)
+        assert torch.equal(fused, torch.relu(got))
+    else:
+        close_bf16(got, ref)
+        close_bf16(general, ref)
+        assert torch.equal(fused, torch.relu(got))
