@@ -2,6 +2,7 @@
 """Builds the native libraries in-tree:
      libaprnet_hip.so  HIP operators for gfx950 (hipcc, one translation unit per .hip file)
      libaprcore.so     host-only APR builder (g++ / OpenMP)
+     ../_pyaprwrapper.<abi>.so   pybind11 module with the reference's native function names over the C ABI (g++, torch headers)
 Usage: python build.py [--force]"""
 import os
 import subprocess
@@ -44,7 +45,30 @@ def build(force=False, verbose=True):
         run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", "libaprnet_hip.so", *objs])
     if force or _newer("libaprcore.so", ["aprcore.cpp"]):
         run(["g++", "-O3", "-march=x86-64-v3", "-fopenmp", "-shared", "-fPIC", "-std=c++17", "-o", "libaprcore.so", "aprcore.cpp"])
+    build_binding(force=force, verbose=verbose)
     return os.path.join(HERE, "libaprnet_hip.so"), os.path.join(HERE, "libaprcore.so")
+
+
+def build_binding(force=False, verbose=True):
+    """pybind/pyaprwrapper.cpp -> apr-cnn_amd/_pyaprwrapper.<abi>.so, linked against libaprnet_hip.so (found through an
+    $ORIGIN rpath) and the torch libraries of this interpreter."""
+    import sysconfig
+    import torch
+    tdir = os.path.dirname(torch.__file__)
+    src = os.path.join(HERE, "pybind", "pyaprwrapper.cpp")
+    out = os.path.join(os.path.dirname(HERE), "_pyaprwrapper" + sysconfig.get_config_var("EXT_SUFFIX"))
+    if not (force or _newer(out, [src, os.path.join(HERE, "..", "..", "include", "aprnet_hip.h")])):
+        return out
+    cmd = ["g++", "-O2", "-std=c++17", "-shared", "-fPIC", "-D__HIP_PLATFORM_AMD__", "-DUSE_ROCM",
+           "-DTORCH_EXTENSION_NAME=_pyaprwrapper", "-D_GLIBCXX_USE_CXX11_ABI=%d" % int(torch._C._GLIBCXX_USE_CXX11_ABI),
+           "-I" + os.path.join(tdir, "include"), "-I" + os.path.join(tdir, "include", "torch", "csrc", "api", "include"),
+           "-I/opt/rocm/include", "-I" + sysconfig.get_paths()["include"], src, "-o", out,
+           "-L" + HERE, "-laprnet_hip", "-L" + os.path.join(tdir, "lib"), "-ltorch", "-ltorch_cpu", "-ltorch_python", "-lc10",
+           "-lc10_hip", "-ltorch_hip", "-L/opt/rocm/lib", "-lamdhip64", "-Wl,-rpath,$ORIGIN/csrc", "-Wl,-rpath," + os.path.join(tdir, "lib")]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    subprocess.check_call(cmd)
+    return out
 
 
 if __name__ == "__main__":

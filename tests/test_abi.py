@@ -161,3 +161,28 @@ def test_plan_create_refuses_damaged_access_arrays():
     assert rc == -1 and "ascend" in msg
     rc, msg = create(xz, y, txz, ty, drop_y=True)
     assert rc == -1 and "y_vec" in msg
+
+
+def test_compiled_binding_exposes_the_reference_names():
+    """The pybind11 module builds in-tree, imports without a GPU and registers the native function names of
+    wrappers/pythonBind.cpp:144-182, wrap_conv.hpp:12-49, wrap_pool.hpp:14-15, wrap_upsample.hpp:14-15 and
+    utils.hpp:340-380 (the operator part)."""
+    import _pyaprwrapper
+    m = _pyaprwrapper.aprnet
+    cuda = ["maxpool_forward_cuda", "maxpool_backward_cuda", "conv111_forward", "conv111_backward", "conv333_forward",
+            "conv333_backward", "upsample_const_forward", "upsample_const_backward", "restrict_kernel333_forward",
+            "restrict_kernel333_backward", "reconstruct_forward", "reconstruct_backward", "sample_particles_forward",
+            "sample_particles_backward"]
+    conv = [f"convolve{k}_{d}" for k in ("111", "333", "133", "555", "155") for d in ("forward", "backward")]
+    conv += [f"restrict_kernel{k}_{d}" for k in ("333", "133", "555", "155") for d in ("forward", "backward")]
+    for mod, names in ((m.cuda, cuda), (m.conv, conv), (m.pool, ["maxpool_forward", "maxpool_backward"]),
+                       (m.upsample, ["upsample_const_forward", "upsample_const_backward"]),
+                       (m.utils, ["number_particles", "number_parts", "number_particles_after_pooling",
+                                  "number_particles_after_upsampling"])):
+        missing = [n for n in names if not hasattr(mod, n)]
+        assert not missing, missing
+    import apr_cases
+    apr = apr_cases.get("3d_a")
+    assert m.utils.number_particles(apr, 0) == apr.total_number_particles()
+    with pytest.raises(RuntimeError, match="CUDA tensor"):          # CHECK_INPUT, cuda/src/common.hpp:14-16
+        m.cuda.conv333_forward([apr], torch.zeros(1, 1, 4), torch.zeros(1, 1, 1, 3, 3, 3), torch.zeros(1, dtype=torch.int32))
