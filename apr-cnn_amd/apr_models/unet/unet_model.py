@@ -14,6 +14,7 @@ class APRUNet(nn.Module):
                  channels_per_group=None, norm="group"):
         super().__init__()
         self.in_channels, self.out_channels, self.depth = in_channels, out_channels, depth
+        self.use_grouped = True         # inference with bfloat16 features: keep tensors grouped by eight channels between layers
         self.num_groups = self.channels_per_group = None
         if num_groups is None and channels_per_group is None:
             self.num_groups = n_filters_base
@@ -42,9 +43,63 @@ class APRUNet(nn.Module):
                                        num_groups=groups(widths[i]), **common))
         self.head = aprnet.APRConv(widths[0], out_channels, nstencils=stencils[0], kernel_size=(1, 1, 1))
 
+    def _grouped_ok(self, x, aprs):
+        """Inference with bfloat16 features and every norm folded away runs on tensors grouped by eight channels
+        (pyapr.aprnet.grouped): same arithmetic as the plane operators, no regrouping pass per convolution."""
+        from pyapr.aprnet import grouped
+        if torch.is_grad_enabled() or not x.is_cuda or x.dtype != torch.bfloat16 or x.size(1) > 3 or not self.use_grouped:
+            return False
+        blocks = [b for m in self.modules() if isinstance(m, ConvBlock) for b in m.blocks] + [st.reduce_ch for st in self.decoder]
+        for b in blocks:
+            if not isinstance(b.norm, nn.Identity) or type(b.activation) is not nn.ReLU:
+                return False
+            if tuple(b.conv.weight.shape[3:]) not in ((3, 3, 3), (1, 3, 3), (1, 5, 5), (1, 1, 1)) or b.conv.weight.shape[1] % 8:
+                return False
+        return grouped.supported(aprs, [])
+
+    def _forward_grouped(self, x, aprs, level_deltas):
+        from pyapr.aprnet import grouped as g8
+        from pyapr.aprnet import _ops
+        levels = max(a.level_max() - a.level_min() + 1 for a in aprs)
+
+        def conv(bb, inp, second=None):
+            w = bb.conv.weight.detach().float()
+            bias = None if bb.conv.bias is None else bb.conv.bias.detach()
+            if tuple(w.shape[3:]) == (1, 1, 1):
+                return g8.conv111_forward(aprs, inp, w, level_deltas, bias, relu=True)
+            return g8.conv_forward(aprs, inp, _ops.restrict_kernel_forward(w.contiguous(), levels), level_deltas, bias, relu=True, x2=second)
+
+        def block(cb, inp, second=None):
+            for i, bb in enumerate(cb.blocks):
+                inp = conv(bb, inp, second if i == 0 else None)
+            return inp
+
+        skips = [block(self.encoder[0], x.contiguous())]
+        for stage in self.encoder[1:]:
+            pooled = g8.maxpool_forward(aprs, skips[-1], level_deltas)
+            level_deltas += 1
+            skips.append(block(stage.conv, pooled))
+            del pooled
+        y = skips.pop()
+        for stage in self.decoder:
+            skip = skips.pop()
+            y = g8.upsample_const_forward(aprs, conv(stage.reduce_ch, y), level_deltas)
+            level_deltas -= 1
+            out = conv(stage.conv.blocks[0], skip, y)
+            y = skip = None
+            for bb in stage.conv.blocks[1:]:
+                out = conv(bb, out)
+            y = out
+            del out
+        hw = self.head.weight.detach().float()
+        hb = None if self.head.bias is None else self.head.bias.detach()
+        return g8.conv111_forward(aprs, y, hw, level_deltas, hb, relu=False, grouped_output=False)
+
     def forward(self, x, aprs, level_deltas=None):
         if level_deltas is None:
             level_deltas = torch.zeros(len(aprs), dtype=torch.int32, device=torch.device("cpu"))
+        if self._grouped_ok(x, aprs):
+            return self._forward_grouped(x, aprs, level_deltas)
         skips = [self.encoder[0](x, aprs, level_deltas)]
         for stage in self.encoder[1:]:
             skips.append(stage(skips[-1], aprs, level_deltas))

@@ -328,7 +328,7 @@ int conv_fwd_bf16(const aprnet_plan* cp, int d, int kz, int kx, int ky, const bf
             bf16_t* ti = xi + ng * (size_t)n_x * 8;
             if (int rc = interleave8_bf16(x, ldx, fu.x2, fu.ldx2, C1, Cin, n_x, xi, st)) return rc;
             if (int rc = interleave8_bf16(tree_ws, ldt, nullptr, 0, Cin, Cin, n_t, ti, st)) return rc;
-            a.xi = xi; a.ti = ti;
+            a.xi = xi; a.ti = ti; a.xi_ld = n_x; a.ti_ld = n_t;
         }
     } else {
         if (int rc = plan_scratch(p, conv_packed_floats(code, S_exp, Cout, Cin, false) * sizeof(float), st)) return rc;
@@ -341,6 +341,59 @@ int conv_fwd_bf16(const aprnet_plan* cp, int d, int kz, int kx, int ky, const bf
     a.x_count = p->number_parts(d); a.t_count = p->tree_parts(d);
     TimedLaunch timed(st);
     return bf16_math ? launch_conv_mfma_bf16(code, a, tl.n, st) : launch_conv_mfma(code, a, tl.n, st);
+}
+
+// bfloat16 features with a layout per tensor: planes [C][ld] or groups of eight channels [C / 8][ld][8] (grouped.hip).
+//   grouped input   Cin (and the channels of a second input) multiples of 8; tree_ws is grouped too; the kernel stages
+//                   straight from the tensors, no regrouping pass
+//   planes input    1 to 3 channels (the first layer of a network) on the pipelined kernel
+//   grouped output  Cout a multiple of 8
+int fill_tree_mean_g8(const aprnet_plan* p, int d, const bf16_t* x, int64_t ldx, int C, bf16_t* tree, int64_t ldt, hipStream_t st);
+int conv_fwd_bf16_layout(const aprnet_plan* cp, int d, int kz, int kx, int ky, const bf16_t* x, int64_t ldx, int C1, int x_g8, const float* w,
+                         int S_exp, int Cout, const float* bias, bf16_t* y, int64_t ldy, int y_g8, bf16_t* tree_ws, int64_t ldt,
+                         hipStream_t st, const Fusion<bf16_t>& fu) {
+    aprnet_plan* p = const_cast<aprnet_plan*>(cp);
+    if (int rc = check_level_delta(p, d, "conv_forward")) return rc;
+    if (int rc = check_plane_size(p, d, 16, "conv_forward")) return rc;          // 16-byte items, 32-bit offsets
+    const int Cin = C1 + fu.C2;
+    if (C1 <= 0 || Cout <= 0 || S_exp <= 0) return fail(APRNET_ERR_INVALID_ARGUMENT, "conv_forward: empty channel / stencil count");
+    const int code = kz * 100 + kx * 10 + ky;
+    if (!conv_mfma_supported(code))
+        return fail(APRNET_ERR_UNSUPPORTED, "conv_forward: bfloat16 features are supported for the 3x3x3, 1x3x3 and 1x5x5 stencils");
+    if (y_g8 && Cout % 8) return fail(APRNET_ERR_INVALID_ARGUMENT, "conv_forward: a grouped output holds a multiple of eight channels");
+    if (x_g8 && (C1 % 8 || fu.C2 % 8)) return fail(APRNET_ERR_INVALID_ARGUMENT, "conv_forward: grouped inputs hold multiples of eight channels");
+    if (!x_g8 && (fu.C2 > 0 || !conv_narrow_supported(code, Cin)))
+        return fail(APRNET_ERR_UNSUPPORTED, "conv_forward: a planes input with a grouped output is taken for 1 to 3 channels only");
+    const int64_t nt = p->tree_parts(d);
+    if (nt > 0 && (!tree_ws || ldt < nt)) return fail(APRNET_ERR_INVALID_ARGUMENT, "conv_forward: tree work space too small");
+    APRNET_HIP_CHECK(hipSetDevice(p->device));
+    TileList tl;
+    if (int rc = get_tiles(p, d, kz == 1 ? 1 : 2, kz == 1 ? 8 : 4, &tl, st)) return rc;
+    ConvArgs<bf16_t> a{};
+    a.apr = p->dapr; a.tree = p->dtree; a.tiles = tl.d_tiles;
+    a.x = x; a.ldx = ldx; a.Cin = Cin; a.w = w; a.S_exp = S_exp; a.Cout = Cout; a.bias = bias; a.relu = fu.relu;
+    a.y = y; a.ldy = ldy; a.y_g8 = y_g8; a.tree_data = tree_ws; a.ldt = ldt; a.Lc = p->lc(d); a.tree_off = p->tree_offset(a.Lc);
+    a.x_count = p->number_parts(d); a.t_count = nt; a.c_split = C1;
+    if (!x_g8) {
+        if (int rc = fill_tree_for_conv(p, d, x, ldx, C1, tree_ws, ldt, st)) return rc;
+        if (tl.n == 0) return 0;
+        bool done = false;
+        if (int rc = try_narrow<bf16_t>(p, a, code, d, tl, st, &done)) return rc;
+        return done ? 0 : fail(APRNET_ERR_UNSUPPORTED, "conv_forward: the window lists of the plan are not available");
+    }
+    if (int rc = fill_tree_mean_g8(p, d, x, ldx, C1, tree_ws, ldt, st)) return rc;
+    if (fu.C2 > 0)
+        if (int rc = fill_tree_mean_g8(p, d, fu.x2, fu.ldx2, fu.C2, tree_ws + (int64_t)(C1 / 8) * ldt * 8, ldt, st)) return rc;
+    if (tl.n == 0) return 0;
+    if (int rc = set_lists(p, d, code, tl, a, st)) return rc;
+    if (!a.tile_win) return fail(APRNET_ERR_UNSUPPORTED, "conv_forward: the window lists of the plan are not available");
+    if (int rc = plan_scratch(p, conv_packed_bf16_bytes(code, S_exp, Cout, Cin), st)) return rc;
+    if (int rc = pack_conv_weights_bf16(code, w, S_exp, Cout, Cin, p->d_scratch, st)) return rc;
+    a.w = (const float*)p->d_scratch;
+    a.xi = x; a.xi_ld = ldx; a.xi2 = fu.C2 > 0 ? fu.x2 : nullptr; a.xi2_ld = fu.ldx2; a.ti = tree_ws; a.ti_ld = ldt;
+    a.x = nullptr; a.x2 = nullptr; a.tree_data = nullptr;
+    TimedLaunch timed(st);
+    return launch_conv_mfma_bf16(code, a, tl.n, st);
 }
 
 int conv111_fwd_relu(const aprnet_plan*, int, const float*, int64_t, int, const float*, int, int, const float*, float*, int64_t, hipStream_t, int);
@@ -371,6 +424,14 @@ int aprnet_conv_fwd_fused_bf16(const aprnet_plan* p, int d, int kz, int kx, int 
     APRNET_FUSED_111(bf16_t)
     return conv_fwd_bf16(p, d, kz, kx, ky, (const bf16_t*)x, ldx, Cin, w, S_exp, Cout, bias, (bf16_t*)y, ldy, (bf16_t*)tree_ws,
                          ldt, (hipStream_t)st, fu);
+}
+int aprnet_conv_fwd_fused_bf16l(const aprnet_plan* p, int d, int kz, int kx, int ky, const uint16_t* x, int64_t ldx, int Cin, int x_grouped,
+                                const float* w, int S_exp, int Cout, const float* bias, uint16_t* y, int64_t ldy, int y_grouped,
+                                uint16_t* tree_ws, int64_t ldt, const aprnet_conv_fusion* fusion, void* st) {
+    Fusion<bf16_t> fu;
+    if (int rc = read_fusion(fusion, &fu)) return rc;
+    return conv_fwd_bf16_layout(p, d, kz, kx, ky, (const bf16_t*)x, ldx, Cin, x_grouped, w, S_exp, Cout, bias, (bf16_t*)y, ldy, y_grouped,
+                                (bf16_t*)tree_ws, ldt, (hipStream_t)st, fu);
 }
 int aprnet_conv_fwd_fused_f32(const aprnet_plan* p, int d, int kz, int kx, int ky, const float* x, int64_t ldx, int Cin,
                               const float* w, int S_exp, int Cout, const float* bias, float* y, int64_t ldy, float* tree_ws,

@@ -452,7 +452,7 @@ int conv_bwd_bf16(const aprnet_plan* cp, int d, int kz, int kx, int ky, const bf
             if (regroup) {
                 bf16_t* gyi = (bf16_t*)((char*)p->d_scratch + wbytes);
                 if (int rc = interleave8_bf16(gy, ldy, nullptr, 0, Cout, Cout, np, gyi, st)) return rc;
-                b.xi = gyi; b.ti = nullptr;
+                b.xi = gyi; b.ti = nullptr; b.xi_ld = np; b.ti_ld = 0;
             }
             b.w = (const float*)p->d_scratch;
             if (int rc = launch_conv_dx_mfma_bf16(code, b, near.n, st)) return rc;

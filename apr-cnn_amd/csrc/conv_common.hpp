@@ -40,6 +40,9 @@ struct ConvArgs {
     // bfloat16 forward only: the input (both tensors) and the tree values regrouped as [Cin / 8][count][8], one
     // 16-byte load per item and group of 8 channels (null: the kernel reads the channel planes)
     const T* xi; const T* ti;
+    int64_t xi_ld, ti_ld;                      // particles between two groups of xi / ti
+    const T* xi2; int64_t xi2_ld;              // grouped second input: groups from c_split / 8 on (null: all groups in xi)
+    int y_g8;                                  // bfloat16 forward: the output is grouped too, [Cout / 8][ldy][8]
     // backward only
     // gradients are accumulated in the computation type (fp32 for bfloat16 features)
     const T* gy; typename Num<T>::acc* gx; int64_t ldgx; typename Num<T>::acc* gtree; int64_t ldgt;
@@ -424,14 +427,37 @@ struct ItemRegs {
 // Which items this thread stages, and where they go: read once per window from the lists (LDS or global).
 template <class G, typename T, int CIB, int NR, class Lists>
 __device__ __forceinline__ void fetch_slots(const Lists& sh, int nitem, ItemRegs<G, T, CIB, NR>& R, int round0 = 0) {
+    if constexpr (std::is_same<Lists, WindowLists>::value) {
+        // Lists in global memory: every round is an unconditional buffer load (lanes past the window's items read
+        // zero) and nothing is done with the results before all rounds are issued.  A load under a per-lane branch
+        // whose result is scaled inside the branch waits for memory there: one round trip per round.
+        const __amdgpu_buffer_rsrc_t ri = __builtin_amdgcn_make_buffer_rsrc(const_cast<int*>(sh.item_idx), 0, nitem * 4, 0x00020000);
+        const __amdgpu_buffer_rsrc_t rp = __builtin_amdgcn_make_buffer_rsrc(const_cast<unsigned short*>(sh.item_pos), 0, nitem * 2, 0x00020000);
+        int idx[NR], pos[NR];
 #pragma unroll
-    for (int k = 0; k < NR; ++k) {
-        R.pos[k] = 0xffffu; R.off[k] = BUF_OOB;
-        if ((round0 + k) * G::NT >= nitem) continue;    // wave-uniform
-        const int it = threadIdx.x + (round0 + k) * G::NT;
-        if (it < nitem) {
-            R.pos[k] = sh.item_pos[it];
-            R.off[k] = (unsigned)sh.item_idx[it] * (unsigned)sizeof(T);
+        for (int k = 0; k < NR; ++k) {
+            idx[k] = 0; pos[k] = 0;
+            if ((round0 + k) * G::NT >= nitem) continue;    // wave-uniform
+            const int it = threadIdx.x + (round0 + k) * G::NT;
+            idx[k] = __builtin_amdgcn_raw_buffer_load_b32(ri, it * 4, 0, 0);
+            pos[k] = (int)__builtin_amdgcn_raw_buffer_load_b16(rp, it * 2, 0, 0);
+        }
+#pragma unroll
+        for (int k = 0; k < NR; ++k) {
+            const bool valid = (int)threadIdx.x + (round0 + k) * G::NT < nitem;
+            R.pos[k] = valid ? (unsigned short)pos[k] : (unsigned short)0xffffu;
+            R.off[k] = valid ? (unsigned)idx[k] * (unsigned)sizeof(T) : BUF_OOB;
+        }
+    } else {
+#pragma unroll
+        for (int k = 0; k < NR; ++k) {
+            R.pos[k] = 0xffffu; R.off[k] = BUF_OOB;
+            if ((round0 + k) * G::NT >= nitem) continue;    // wave-uniform
+            const int it = threadIdx.x + (round0 + k) * G::NT;
+            if (it < nitem) {
+                R.pos[k] = sh.item_pos[it];
+                R.off[k] = (unsigned)sh.item_idx[it] * (unsigned)sizeof(T);
+            }
         }
     }
 }

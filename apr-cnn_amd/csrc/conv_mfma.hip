@@ -370,20 +370,32 @@ struct ItemRegs16 { intx4 v[IPT]; unsigned off[IPT]; unsigned short pos[IPT]; };
 
 template <class G, int IPT, class Lists>
 __device__ __forceinline__ void fetch_slots16(const Lists& sh, int nitem, ItemRegs16<G, IPT>& R) {
+    // unconditional buffer loads, results touched only after every round is issued (see fetch_slots)
+    const __amdgpu_buffer_rsrc_t ri = __builtin_amdgcn_make_buffer_rsrc(const_cast<int*>(sh.item_idx), 0, nitem * 4, 0x00020000);
+    const __amdgpu_buffer_rsrc_t rp = __builtin_amdgcn_make_buffer_rsrc(const_cast<unsigned short*>(sh.item_pos), 0, nitem * 2, 0x00020000);
+    int idx[IPT], pos[IPT];
 #pragma unroll
     for (int k = 0; k < IPT; ++k) {
-        R.pos[k] = 0xffffu; R.off[k] = BUF_OOB;
+        idx[k] = 0; pos[k] = 0;
         if (k * G::NT >= nitem) continue;               // wave-uniform
         const int it = threadIdx.x + k * G::NT;
-        if (it < nitem) { R.pos[k] = sh.item_pos[it]; R.off[k] = (unsigned)sh.item_idx[it] * 16u; }
+        idx[k] = __builtin_amdgcn_raw_buffer_load_b32(ri, it * 4, 0, 0);
+        pos[k] = (int)__builtin_amdgcn_raw_buffer_load_b16(rp, it * 2, 0, 0);
+    }
+#pragma unroll
+    for (int k = 0; k < IPT; ++k) {
+        const bool valid = (int)threadIdx.x + k * G::NT < nitem;
+        R.pos[k] = valid ? (unsigned short)pos[k] : (unsigned short)0xffffu;
+        R.off[k] = valid ? (unsigned)idx[k] * 16u : BUF_OOB;
     }
 }
 template <class G, int IPT>
 __device__ __forceinline__ void load_values16(const ConvArgs<bf16_t>& a, int ci0, int nitem, bool tree_items, ItemRegs16<G, IPT>& R) {
     const int q = ci0 / BF_CIB;
-    const __amdgpu_buffer_rsrc_t rx = __builtin_amdgcn_make_buffer_rsrc(const_cast<bf16_t*>(a.xi + (int64_t)q * a.x_count * BF_CIB), 0,
-                                                                        (int)(a.x_count * 16), 0x00020000);
-    const __amdgpu_buffer_rsrc_t rt = __builtin_amdgcn_make_buffer_rsrc(const_cast<bf16_t*>(a.ti + (int64_t)q * a.t_count * BF_CIB), 0,
+    const int q1 = a.c_split / BF_CIB;          // groups of the first tensor when there is a second one
+    const bf16_t* xg = (a.xi2 != nullptr && q >= q1) ? a.xi2 + (int64_t)(q - q1) * a.xi2_ld * BF_CIB : a.xi + (int64_t)q * a.xi_ld * BF_CIB;
+    const __amdgpu_buffer_rsrc_t rx = __builtin_amdgcn_make_buffer_rsrc(const_cast<bf16_t*>(xg), 0, (int)(a.x_count * 16), 0x00020000);
+    const __amdgpu_buffer_rsrc_t rt = __builtin_amdgcn_make_buffer_rsrc(const_cast<bf16_t*>(a.ti + (int64_t)q * a.ti_ld * BF_CIB), 0,
                                                                         tree_items ? (int)(a.t_count * 16) : 0, 0x00020000);
 #pragma unroll
     for (int k = 0; k < IPT; ++k) {
@@ -512,6 +524,24 @@ __device__ __forceinline__ void mfma_bf16_window(const ConvArgs<bf16_t>& a, int 
         if (col >= nc) continue;
         const int64_t o = sh.col_idx[col];
         if constexpr (MODE == 0) {
+            if (IL && a.y_g8) {
+                // grouped output: the lane's four channels of a part are half of a 16-byte group
+#pragma unroll
+                for (int h = 0; h < COH; ++h) {
+                    const int c4 = co0 + h * 16 + 4 * (lane >> 4);
+                    float v[4];
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) {
+                        v[r] = acc[j][h][r] + bias_l[h * 16 + 4 * (lane >> 4) + r];
+                        if (FUSE && a.relu) v[r] = v[r] < 0.f ? 0.f : v[r];
+                    }
+                    if (c4 < a.Cout)
+                        *reinterpret_cast<uint2*>(a.y + (((int64_t)(c4 >> 3) * a.ldy + o) << 3) + (c4 & 4)) =
+                            make_uint2((unsigned)float_to_bf16(v[0]).bits | ((unsigned)float_to_bf16(v[1]).bits << 16),
+                                       (unsigned)float_to_bf16(v[2]).bits | ((unsigned)float_to_bf16(v[3]).bits << 16));
+                }
+                continue;
+            }
 #pragma unroll
             for (int h = 0; h < COH; ++h)
 #pragma unroll

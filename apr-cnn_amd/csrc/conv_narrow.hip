@@ -176,6 +176,25 @@ conv_narrow_kernel(const ConvArgs<T> a, const NarrowArgs na) {
             if (((first + G::NWAVE * j) << 4) >= nc) break;          // wave-uniform: no such block
             if (col >= nc) continue;
             const int64_t o = c.idx[j];
+            if constexpr (std::is_same<T, bf16_t>::value) {
+                if (a.y_g8) {          // grouped output [Cout / 8][ldy][8]: the lane's four channels are half of a 16-byte group
+#pragma unroll
+                    for (int h = 0; h < COH; ++h) {
+                        const int c4 = co0 + h * 16 + 4 * (lane >> 4);
+                        float v[4];
+#pragma unroll
+                        for (int r = 0; r < 4; ++r) {
+                            v[r] = acc[j][h][r] + bias_l[h * 16 + 4 * (lane >> 4) + r];
+                            if (a.relu) v[r] = v[r] < 0.f ? 0.f : v[r];
+                        }
+                        if (c4 < a.Cout)
+                            *reinterpret_cast<uint2*>(a.y + (((int64_t)(c4 >> 3) * a.ldy + o) << 3) + (c4 & 4)) =
+                                make_uint2((unsigned)float_to_bf16(v[0]).bits | ((unsigned)float_to_bf16(v[1]).bits << 16),
+                                           (unsigned)float_to_bf16(v[2]).bits | ((unsigned)float_to_bf16(v[3]).bits << 16));
+                    }
+                    continue;
+                }
+            }
 #pragma unroll
             for (int h = 0; h < COH; ++h)
 #pragma unroll

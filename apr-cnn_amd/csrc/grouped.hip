@@ -1,0 +1,322 @@
+// bfloat16 features grouped by eight channels: [C / 8][ld][8], the eight channels of a particle in one 16-byte word.
+//
+// The reference keeps channel planes [C][N] (conv.hpp:68).  On planes every operator of this library gathers one
+// 2-byte value per channel and particle; grouped, a particle's eight channels come with one 16-byte access, which
+// is what the bfloat16 convolution stages from anyway.  A network whose layers hand each other grouped tensors
+// converts at its two ends only (regroup / ungroup below) and needs neither the per-call regrouping pass of the
+// convolution nor two-byte stores in its epilogue.  The operators here are those of a network's forward pass:
+// tree fill (for the convolution), max pool (values only: the argmax serves the backward pass), constant
+// upsampling and the 1x1x1 convolution.  Arithmetic and summation order are those of the plane kernels
+// (tree_ops.hip, conv111.hip), so results are bit-identical to theirs.
+#include "common.hpp"
+
+namespace aprnet {
+
+constexpr int GTB = 256;
+
+__device__ __forceinline__ void unpack8(const uint4 v, float (&f)[8]) {
+    const unsigned w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        f[2 * k] = __builtin_bit_cast(float, w[k] << 16);
+        f[2 * k + 1] = __builtin_bit_cast(float, w[k] & 0xffff0000u);
+    }
+}
+__device__ __forceinline__ uint4 pack8(const float (&f)[8]) {
+    unsigned w[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) w[k] = (unsigned)float_to_bf16(f[2 * k]).bits | ((unsigned)float_to_bf16(f[2 * k + 1]).bits << 16);
+    return make_uint4(w[0], w[1], w[2], w[3]);
+}
+__device__ __forceinline__ const uint4* g8_at(const bf16_t* base, int64_t ld, int q, int64_t i) {
+    return reinterpret_cast<const uint4*>(base) + (int64_t)q * ld + i;
+}
+__device__ __forceinline__ uint4* g8_at(bf16_t* base, int64_t ld, int q, int64_t i) {
+    return reinterpret_cast<uint4*>(base) + (int64_t)q * ld + i;
+}
+
+// ---------------------------------------------------------------------------- planes <-> groups
+// out[q][i][c] = x[8 q + c][i]; channels past C read as zeros
+__global__ void regroup8_kernel(const bf16_t* __restrict__ x, int64_t ldx, int C, int64_t n, bf16_t* __restrict__ out, int64_t ldo) {
+    const int q = blockIdx.y;
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x) {
+        unsigned v[8];
+#pragma unroll
+        for (int c = 0; c < 8; ++c) v[c] = (8 * q + c < C) ? x[(int64_t)(8 * q + c) * ldx + i].bits : 0u;
+        *g8_at(out, ldo, q, i) = make_uint4(v[0] | (v[1] << 16), v[2] | (v[3] << 16), v[4] | (v[5] << 16), v[6] | (v[7] << 16));
+    }
+}
+__global__ void ungroup8_kernel(const bf16_t* __restrict__ xg, int64_t ldg, int C, int64_t n, bf16_t* __restrict__ out, int64_t ldo) {
+    const int q = blockIdx.y;
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x) {
+        const uint4 v = *g8_at(xg, ldg, q, i);
+        const unsigned w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+        for (int c = 0; c < 8; ++c)
+            if (8 * q + c < C) out[(int64_t)(8 * q + c) * ldo + i].bits = (unsigned short)(c & 1 ? w[c >> 1] >> 16 : w[c >> 1] & 0xffffu);
+    }
+}
+
+// ---------------------------------------------------------------------------- tree fill (mean of children)
+// fill_node of tree_ops.hip for eight channels at once: same pass order (downsampled particles before particles
+// under the features, particles before tree nodes elsewhere), same fp32 sums.
+__device__ __forceinline__ void fill_node_g8(const int32_t* children, int64_t n_tree, int64_t t, const bf16_t* x, int64_t ldx,
+                                             bf16_t* tree, int64_t ldt, int64_t tree_off, int tree_child_from_x, int tree_first, int q) {
+    int32_t ch[8];
+    int cnt = 0;
+#pragma unroll
+    for (int s = 0; s < 8; ++s) { ch[s] = children[(int64_t)s * n_tree + t]; cnt += ch[s] != NO_CHILD; }
+    const float scale = 1.0f / (float)max(cnt, 1);
+    uint4 raw[8];
+#pragma unroll
+    for (int s = 0; s < 8; ++s) {
+        const int32_t v = ch[s];
+        raw[s] = make_uint4(0u, 0u, 0u, 0u);
+        if (v >= 0) raw[s] = *g8_at(x, ldx, q, v);
+        else if (v != NO_CHILD) raw[s] = tree_child_from_x ? *g8_at(x, ldx, q, tree_off + ~v) : *g8_at((const bf16_t*)tree, ldt, q, ~v);
+    }
+    float sum[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int pass = 0; pass < 2; ++pass) {
+        const bool want_tree = (pass == 0) == (tree_first != 0);
+#pragma unroll
+        for (int s = 0; s < 8; ++s) {
+            const int32_t v = ch[s];
+            if (v == NO_CHILD || want_tree != (v < 0)) continue;
+            float f[8];
+            unpack8(raw[s], f);
+#pragma unroll
+            for (int c = 0; c < 8; ++c) sum[c] += f[c];
+        }
+    }
+#pragma unroll
+    for (int c = 0; c < 8; ++c) sum[c] *= scale;
+    *g8_at(tree, ldt, q, t) = pack8(sum);
+}
+
+__global__ void __launch_bounds__(GTB)
+fill_tree_level_g8_kernel(const int32_t* __restrict__ children, int64_t n_tree, int64_t t_begin, int64_t t_end, const bf16_t* __restrict__ x,
+                          int64_t ldx, bf16_t* __restrict__ tree, int64_t ldt, int64_t tree_off, int from_x) {
+    const int64_t t = t_begin + (int64_t)blockIdx.x * GTB + threadIdx.x;
+    if (t < t_end) fill_node_g8(children, n_tree, t, x, ldx, tree, ldt, tree_off, from_x, from_x, blockIdx.y);
+}
+
+constexpr int G_MAX_COARSE = 12;
+struct GCoarse { int n; int64_t begin[G_MAX_COARSE], end[G_MAX_COARSE]; };
+
+// the coarse levels in one launch, finest first, one workgroup per channel group (see fill_tree_coarse_kernel)
+__global__ void __launch_bounds__(GTB)
+fill_tree_coarse_g8_kernel(const int32_t* __restrict__ children, int64_t n_tree, const GCoarse lv, const bf16_t* x, int64_t ldx,
+                           bf16_t* tree, int64_t ldt) {
+    for (int i = 0; i < lv.n; ++i) {
+        for (int64_t t = lv.begin[i] + threadIdx.x; t < lv.end[i]; t += GTB)
+            fill_node_g8(children, n_tree, t, x, ldx, tree, ldt, 0, 0, 0, blockIdx.x);
+        __syncthreads();
+    }
+}
+
+int fill_tree_mean_g8(const aprnet_plan* p, int d, const bf16_t* x, int64_t ldx, int C, bf16_t* tree, int64_t ldt, hipStream_t st) {
+    if (C <= 0) return 0;
+    if (C % 8) return fail(APRNET_ERR_INVALID_ARGUMENT, "grouped features hold a multiple of eight channels");
+    const int Lc = p->lc(d), G = C / 8;
+    if (ldt < p->tree_parts(d)) return fail(APRNET_ERR_INVALID_ARGUMENT, "fill_tree_mean: tree work space too small");
+    const int l_top = std::min(Lc - 1, p->tree.level_max);
+    // levels level_min .. l_coarse (at most 2048 nodes together, never the level under the features) go in one launch
+    int64_t nodes = 0;
+    int l_coarse = p->tree.level_min - 1;
+    while (l_coarse + 1 < l_top && l_coarse + 1 - p->tree.level_min < G_MAX_COARSE) {
+        nodes += p->tree.level_end(l_coarse + 1) - p->tree.level_begin(l_coarse + 1);
+        if (nodes > 2048) break;
+        ++l_coarse;
+    }
+    for (int l = l_top; l > l_coarse; --l) {
+        const int64_t b = p->tree.level_begin(l), e = p->tree.level_end(l);
+        if (e <= b) continue;
+        const int from_x = (l + 1 == Lc);
+        hipLaunchKernelGGL(fill_tree_level_g8_kernel, dim3((unsigned)((e - b + GTB - 1) / GTB), (unsigned)G), dim3(GTB), 0, st, p->d_children,
+                           p->n_tree, b, e, x, ldx, tree, ldt, from_x ? p->tree_offset(Lc) : 0, from_x);
+    }
+    GCoarse lv{};
+    for (int l = l_coarse; l >= p->tree.level_min; --l)
+        if (p->tree.level_end(l) > p->tree.level_begin(l)) { lv.begin[lv.n] = p->tree.level_begin(l); lv.end[lv.n] = p->tree.level_end(l); ++lv.n; }
+    if (lv.n > 0)
+        hipLaunchKernelGGL(fill_tree_coarse_g8_kernel, dim3((unsigned)G), dim3(GTB), 0, st, p->d_children, p->n_tree, lv, x, ldx, tree, ldt);
+    APRNET_LAUNCH_CHECK("fill_tree g8 kernels");
+    return 0;
+}
+
+// ---------------------------------------------------------------------------- max pool (values), upsample
+// maxpool_fwd_kernel of tree_ops.hip without the argmax plane: candidate order (dz, dx, dy), particles before
+// downsampled particles, strict >, start value -1e17 (maxpool.hpp:51, 88-143).
+__global__ void __launch_bounds__(GTB)
+maxpool_g8_kernel(const int32_t* __restrict__ children, int64_t n_tree, int64_t n_copy, int64_t n_out, int64_t t_begin,
+                  const bf16_t* __restrict__ x, int64_t ldx, bf16_t* __restrict__ y, int64_t ldy, int64_t in_tree_off) {
+    const int64_t i = (int64_t)blockIdx.x * GTB + threadIdx.x;
+    const int q = blockIdx.y;
+    if (i >= n_out) return;
+    if (i < n_copy) { *g8_at(y, ldy, q, i) = *g8_at(x, ldx, q, i); return; }
+    const int64_t t = t_begin + (i - n_copy);
+    float best[8];
+#pragma unroll
+    for (int c = 0; c < 8; ++c) best[c] = -1e17f;
+#pragma unroll
+    for (int pass = 0; pass < 2; ++pass)
+#pragma unroll
+        for (int s = 0; s < 8; ++s) {
+            const int32_t v = children[(int64_t)s * n_tree + t];
+            if (v == NO_CHILD || (pass == 0) != (v >= 0)) continue;
+            float f[8];
+            unpack8(*g8_at(x, ldx, q, v >= 0 ? (int64_t)v : in_tree_off + ~v), f);
+#pragma unroll
+            for (int c = 0; c < 8; ++c) if (f[c] > best[c]) best[c] = f[c];
+        }
+    *g8_at(y, ldy, q, i) = pack8(best);
+}
+
+// upsample_kernel of tree_ops.hip, forward: a downsampled particle's value goes to each of its children
+__global__ void __launch_bounds__(GTB)
+upsample_g8_kernel(const int32_t* __restrict__ children, int64_t n_tree, int64_t n_copy, int64_t n_in, int64_t t_begin,
+                   const bf16_t* __restrict__ src, int64_t lds, bf16_t* __restrict__ dst, int64_t ldd, int64_t out_tree_off) {
+    const int64_t i = (int64_t)blockIdx.x * GTB + threadIdx.x;
+    const int q = blockIdx.y;
+    if (i >= n_in) return;
+    const uint4 v = *g8_at(src, lds, q, i);
+    if (i < n_copy) { *g8_at(dst, ldd, q, i) = v; return; }
+    const int64_t t = t_begin + (i - n_copy);
+#pragma unroll
+    for (int s = 0; s < 8; ++s) {
+        const int32_t c = children[(int64_t)s * n_tree + t];
+        if (c >= 0) *g8_at(dst, ldd, q, c) = v;
+        else if (c != NO_CHILD) *g8_at(dst, ldd, q, out_tree_off + ~c) = v;
+    }
+}
+
+// ---------------------------------------------------------------------------- 1x1x1 convolution
+// out[co][i] = bias[co] + sum_ci w[s][co][ci] x[ci][i], s constant over a range of particles (conv.hpp:199-256).
+// One thread per (particle, group of eight outputs): the input groups come with 16-byte loads, the 8 x Cin weights of
+// the output group sit in LDS and are read as broadcasts.  Bound by memory for the layers it serves (channel
+// reductions of the decoder, the head).  OUT_G8: grouped output, otherwise channel planes (the head of a network).
+constexpr int C111_MAX_CIN = 256;
+
+template <bool OUT_G8>
+__global__ void __launch_bounds__(GTB)
+conv111_g8_kernel(const bf16_t* __restrict__ x, int64_t ldx, int Cin, const float* __restrict__ w, int Cout, const float* __restrict__ bias,
+                  int relu, bf16_t* __restrict__ y, int64_t ldy, int64_t begin, int64_t end) {
+    __shared__ __attribute__((aligned(16))) float wl[C111_MAX_CIN * 8];        // [ci][co8]
+    const int og = blockIdx.y, nq = Cin / 8;
+    for (int e = threadIdx.x; e < Cin * 8; e += GTB) {
+        const int ci = e >> 3, co = og * 8 + (e & 7);
+        wl[e] = co < Cout ? w[(int64_t)co * Cin + ci] : 0.f;
+    }
+    __syncthreads();
+    const int64_t i = begin + (int64_t)blockIdx.x * GTB + threadIdx.x;
+    if (i >= end) return;
+    float acc[8];
+#pragma unroll
+    for (int c = 0; c < 8; ++c) acc[c] = 0.f;
+    for (int q = 0; q < nq; ++q) {
+        float f[8];
+        unpack8(*g8_at(x, ldx, q, i), f);
+#pragma unroll
+        for (int k = 0; k < 8; ++k) {
+            const float4 w0 = *reinterpret_cast<const float4*>(wl + (q * 8 + k) * 8), w1 = *reinterpret_cast<const float4*>(wl + (q * 8 + k) * 8 + 4);
+            acc[0] += w0.x * f[k]; acc[1] += w0.y * f[k]; acc[2] += w0.z * f[k]; acc[3] += w0.w * f[k];
+            acc[4] += w1.x * f[k]; acc[5] += w1.y * f[k]; acc[6] += w1.z * f[k]; acc[7] += w1.w * f[k];
+        }
+    }
+#pragma unroll
+    for (int c = 0; c < 8; ++c) {
+        const int co = og * 8 + c;
+        if (bias && co < Cout) acc[c] += bias[co];
+        if (relu) acc[c] = acc[c] < 0.f ? 0.f : acc[c];
+    }
+    if constexpr (OUT_G8) *g8_at(y, ldy, og, i) = pack8(acc);
+    else {
+#pragma unroll
+        for (int c = 0; c < 8; ++c)
+            if (og * 8 + c < Cout) y[(int64_t)(og * 8 + c) * ldy + i] = float_to_bf16(acc[c]);
+    }
+}
+
+}  // namespace aprnet
+
+using namespace aprnet;
+extern "C" {
+
+int aprnet_regroup8_bf16(const uint16_t* x, int64_t ldx, int C, int64_t n, uint16_t* out, int64_t ldo, void* st) {
+    if (C <= 0 || n <= 0) return 0;
+    if (!x || !out || ldo < n || ldx < n) return fail(APRNET_ERR_INVALID_ARGUMENT, "regroup8: null pointer or row shorter than n");
+    dim3 grid((unsigned)std::min<int64_t>((n + 255) / 256, 1 << 20), (unsigned)((C + 7) / 8));
+    hipLaunchKernelGGL(regroup8_kernel, grid, dim3(256), 0, (hipStream_t)st, (const bf16_t*)x, ldx, C, n, (bf16_t*)out, ldo);
+    APRNET_LAUNCH_CHECK("regroup8_kernel");
+    return 0;
+}
+int aprnet_ungroup8_bf16(const uint16_t* xg, int64_t ldg, int C, int64_t n, uint16_t* out, int64_t ldo, void* st) {
+    if (C <= 0 || n <= 0) return 0;
+    if (!xg || !out || ldo < n || ldg < n) return fail(APRNET_ERR_INVALID_ARGUMENT, "ungroup8: null pointer or row shorter than n");
+    dim3 grid((unsigned)std::min<int64_t>((n + 255) / 256, 1 << 20), (unsigned)((C + 7) / 8));
+    hipLaunchKernelGGL(ungroup8_kernel, grid, dim3(256), 0, (hipStream_t)st, (const bf16_t*)xg, ldg, C, n, (bf16_t*)out, ldo);
+    APRNET_LAUNCH_CHECK("ungroup8_kernel");
+    return 0;
+}
+int aprnet_fill_tree_mean_bf16g(const aprnet_plan* p, int d, const uint16_t* x, int64_t ldx, int C, uint16_t* tree, int64_t ldt, void* st) {
+    if (int rc = check_level_delta(p, d, "fill_tree_mean")) return rc;
+    APRNET_HIP_CHECK(hipSetDevice(p->device));
+    return fill_tree_mean_g8(p, d, (const bf16_t*)x, ldx, C, (bf16_t*)tree, ldt, (hipStream_t)st);
+}
+int aprnet_maxpool_fwd_bf16g(const aprnet_plan* p, int d, const uint16_t* x, int64_t ldx, int C, uint16_t* y, int64_t ldy, void* st) {
+    if (int rc = check_level_delta(p, d, "maxpool_forward")) return rc;
+    if (C % 8) return fail(APRNET_ERR_INVALID_ARGUMENT, "grouped features hold a multiple of eight channels");
+    const int Lc = p->lc(d);
+    if (Lc - 1 < p->tree.level_min) return fail(APRNET_ERR_LEVEL_DELTA, "maxpool_forward: nothing left to pool");
+    const int64_t n_out = p->number_parts(d + 1), n_copy = p->apr.level_end(Lc - 1);
+    if (C <= 0 || n_out <= 0) return 0;
+    if (ldy < n_out || ldx < p->number_parts(d)) return fail(APRNET_ERR_INVALID_ARGUMENT, "maxpool_forward: row shorter than the particle count");
+    APRNET_HIP_CHECK(hipSetDevice(p->device));
+    hipLaunchKernelGGL(maxpool_g8_kernel, dim3((unsigned)((n_out + GTB - 1) / GTB), (unsigned)(C / 8)), dim3(GTB), 0, (hipStream_t)st,
+                       p->d_children, p->n_tree, n_copy, n_out, p->tree.level_begin(Lc - 1), (const bf16_t*)x, ldx, (bf16_t*)y, ldy,
+                       p->tree_offset(Lc));
+    APRNET_LAUNCH_CHECK("maxpool_g8_kernel");
+    return 0;
+}
+int aprnet_upsample_fwd_bf16g(const aprnet_plan* p, int d, const uint16_t* x, int64_t ldx, int C, uint16_t* y, int64_t ldy, void* st) {
+    if (int rc = check_level_delta(p, d, "upsample_const_forward")) return rc;
+    if (d <= 0) return fail(APRNET_ERR_INVALID_ARGUMENT, "UpSampleConst is only implemented for downsampled particles (level_delta > 0)");
+    if (C % 8) return fail(APRNET_ERR_INVALID_ARGUMENT, "grouped features hold a multiple of eight channels");
+    const int Lc = p->lc(d);
+    const int64_t n_in = p->number_parts(d), n_copy = p->apr.level_end(Lc);
+    if (C <= 0 || n_in <= 0) return 0;
+    if (ldx < n_in || ldy < p->number_parts(d - 1)) return fail(APRNET_ERR_INVALID_ARGUMENT, "upsample_const_forward: row shorter than the particle count");
+    APRNET_HIP_CHECK(hipSetDevice(p->device));
+    hipLaunchKernelGGL(upsample_g8_kernel, dim3((unsigned)((n_in + GTB - 1) / GTB), (unsigned)(C / 8)), dim3(GTB), 0, (hipStream_t)st,
+                       p->d_children, p->n_tree, n_copy, n_in, p->tree.level_begin(Lc), (const bf16_t*)x, ldx, (bf16_t*)y, ldy,
+                       p->tree_offset(Lc + 1));
+    APRNET_LAUNCH_CHECK("upsample_g8_kernel");
+    return 0;
+}
+int aprnet_conv111_fwd_bf16g(const aprnet_plan* p, int d, const uint16_t* x, int64_t ldx, int Cin, const float* w, int S, int Cout,
+                             const float* bias, int relu, uint16_t* y, int64_t ldy, int y_grouped, void* st) {
+    if (int rc = check_level_delta(p, d, "conv111_forward")) return rc;
+    if (Cin <= 0 || Cout <= 0 || S <= 0) return fail(APRNET_ERR_INVALID_ARGUMENT, "conv111_forward: empty channel / stencil count");
+    if (Cin % 8 || Cin > C111_MAX_CIN || (y_grouped && Cout % 8))
+        return fail(APRNET_ERR_UNSUPPORTED, "conv111_forward (grouped): channel counts must be multiples of eight, at most 256 inputs");
+    APRNET_HIP_CHECK(hipSetDevice(p->device));
+    const int Lc = p->lc(d);
+    // particles of levels that share a stencil are contiguous: stencil s serves level Lc - s (the downsampled
+    // particles sit behind level Lc and take stencil 0 with it), the last stencil every coarser level as well
+    for (int s = 0; s < S; ++s) {
+        const int l_hi = Lc - s, l_lo = (s == S - 1) ? p->apr.level_min : l_hi;
+        if (l_hi < p->apr.level_min) break;
+        int64_t b = p->apr.level_begin(std::max(l_lo, p->apr.level_min)), e = p->apr.level_end(l_hi);
+        if (s == 0) e = p->number_parts(d);
+        if (e <= b) continue;
+        dim3 grid((unsigned)((e - b + GTB - 1) / GTB), (unsigned)((Cout + 7) / 8));
+        const float* ws = w + (int64_t)s * Cout * Cin;
+        if (y_grouped) hipLaunchKernelGGL(conv111_g8_kernel<true>, grid, dim3(GTB), 0, (hipStream_t)st, (const bf16_t*)x, ldx, Cin, ws, Cout, bias, relu, (bf16_t*)y, ldy, b, e);
+        else hipLaunchKernelGGL(conv111_g8_kernel<false>, grid, dim3(GTB), 0, (hipStream_t)st, (const bf16_t*)x, ldx, Cin, ws, Cout, bias, relu, (bf16_t*)y, ldy, b, e);
+    }
+    APRNET_LAUNCH_CHECK("conv111_g8_kernel");
+    return 0;
+}
+
+}  // extern "C"

@@ -131,5 +131,14 @@ def hip():
     lib.aprnet_channel_sum_bf16.argtypes = [vp, i64, i32, i64, vp, i32, vp, vp]
     lib.aprnet_conv_bwd_bf16.argtypes = [vp, i32, i32, i32, i32, vp, i64, i32, vp, i32, i32, vp, i64, vp, i64, vp,
                                          vp, i64, vp, i64, vp, i64, vp]
+    # bfloat16 features grouped by eight channels
+    lib.aprnet_regroup8_bf16.argtypes = [vp, i64, i32, i64, vp, i64, vp]
+    lib.aprnet_ungroup8_bf16.argtypes = [vp, i64, i32, i64, vp, i64, vp]
+    lib.aprnet_fill_tree_mean_bf16g.argtypes = [vp, i32, vp, i64, i32, vp, i64, vp]
+    lib.aprnet_maxpool_fwd_bf16g.argtypes = [vp, i32, vp, i64, i32, vp, i64, vp]
+    lib.aprnet_upsample_fwd_bf16g.argtypes = [vp, i32, vp, i64, i32, vp, i64, vp]
+    lib.aprnet_conv111_fwd_bf16g.argtypes = [vp, i32, vp, i64, i32, vp, i32, i32, vp, i32, vp, i64, i32, vp]
+    lib.aprnet_conv_fwd_fused_bf16l.argtypes = [vp, i32, i32, i32, i32, vp, i64, i32, i32, vp, i32, i32, vp, vp, i64, i32,
+                                                vp, i64, vp, vp]
     _hip = lib
     return lib

@@ -230,23 +230,36 @@ def run_blobs512(args, dev, lib):
     apr.init_cuda()
     t_plan = time.perf_counter() - t0
     n = apr.total_number_particles()
-    bf16 = args.features == "bf16"
+    bf16 = args.features in ("bf16", "bf16g")
     torch.manual_seed(0)
     x = torch.randn(1, CIN, n, device=dev)
     if bf16:
         x = x.to(torch.bfloat16)
     conv = aprnet.cuda.APRConv(CIN, COUT, nstencils=nstencils, kernel_size=(3, 3, 3), bias=True).to(dev)
     ld = torch.zeros(1, dtype=torch.int32)
+    if args.features == "bf16g":
+        # the same layer between two layers of a network that keeps its tensors grouped by eight channels
+        from pyapr.aprnet import _ops, grouped
+        xg = grouped.regroup(x)
+        levels = apr.level_max() - apr.level_min() + 1
+
+        def step():
+            return grouped.conv_forward([apr], xg, _ops.restrict_kernel_forward(conv.weight.detach(), levels), ld, conv.bias.detach())
+    else:
+        def step():
+            return conv(x, [apr], ld)
     with torch.no_grad():
-        sec = _steps(lambda: conv(x, [apr], ld), args.steps, args.warmup)
-        kernel_ms = _kernel_ms(lib, lambda: conv(x, [apr], ld), args.steps)
-        y = conv(x, [apr], ld)
+        sec = _steps(step, args.steps, args.warmup)
+        kernel_ms = _kernel_ms(lib, step, args.steps)
+        y = step()
+    y = y.data if args.features == "bf16g" else y
     assert torch.isfinite(y.float()).all()
     del y
     e = 2 if bf16 else 4
     out = base_line("APRConv 3x3x3 fwd particles/s (Cin=Cout=32) + APR-UNet fwd latency, 1 GPU", n / sec, "particles/s", args,
                     sec * 1e3, "bf16" if bf16 else "f32",
-                    {"workload": f"APRConv 3x3x3 32->32 {'bf16' if bf16 else 'fp32'} forward (restrict + tree fill + conv + bias), batch 1, "
+                    {"workload": f"APRConv 3x3x3 32->32 {'bf16' if bf16 else 'fp32'} forward (restrict + tree fill + conv + bias"
+                                 f"{', input and output grouped by eight channels' if args.features == 'bf16g' else ''}), batch 1, "
                                  "APR of the seeded 512x512x256 volume with 2000 ellipsoidal blobs (configs[1]); extra: 4-level "
                                  "APR-UNet forward on the same APR",
                      "n_particles": n, "levels": level_counts(apr), "nstencils": nstencils, "level_max": apr.level_max(),
@@ -254,6 +267,8 @@ def run_blobs512(args, dev, lib):
     out["roofline"] = mfma_roofline(flop_pp * n, kernel_ms, PEAK_BF16_MATRIX_TFLOPS if bf16 else PEAK_FP32_MATRIX_TFLOPS,
                                     "conv_mfma_bf16_kernel" if bf16 else "conv_mfma16_kernel",
                                     (e * (CIN + COUT) + 2) * n, None if bf16 else PROFILED_TRAFFIC_BYTES.get(n))
+    if args.no_extra:                      # profiler runs: the convolution step only
+        return out
     # second half of the metric: forward latency of the 4-level network (16-32-64-128, norms folded) on this APR
     net = make_unet(dev)
     xin = x[:, :1].float().contiguous()
@@ -710,8 +725,11 @@ def main():
     ap.add_argument("--config", choices=sorted(RUNNERS), default="blobs512",
                     help="BASELINE configuration to run (default: the one the headline metric is quoted on)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--features", choices=["f32", "bf16"], default="f32",
-                    help="blobs512: element type of the feature tensors; bf16 runs the bfloat16 matrix-core kernel "
+    ap.add_argument("--no-extra", action="store_true",
+                    help="blobs512: only the convolution step (no APR-UNet latency, no CPU baseline): for profiler runs")
+    ap.add_argument("--features", choices=["f32", "bf16", "bf16g"], default="f32",
+                    help="blobs512: element type of the feature tensors; bf16 runs the bfloat16 matrix-core kernel on channel "
+                         "planes, bf16g on tensors grouped by eight channels, as a network keeps them between its layers "
                          "(the headline figure is the f32 one)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="blobs512: run one device-to-device copy of the input features (a kernel of known traffic, "

@@ -253,6 +253,33 @@ int aprnet_channel_sum_bf16(const uint16_t* x, int64_t ld, int C, int64_t n, flo
 int aprnet_upsample_bwd_bf16(const aprnet_plan*, int level_delta, const uint16_t* gy, int64_t ldy, int C, uint16_t* gx,
                              int64_t ldx, void* stream);
 
+/* bfloat16 features grouped by eight channels: [C / 8][ld][8], the eight channels of a particle in one 16-byte word
+ * (no counterpart in the reference, whose tensors are channel planes, conv.hpp:68).  A network's forward pass that
+ * hands grouped tensors from layer to layer converts at its two ends only; the convolution then stages straight from
+ * its input (no regrouping pass per call) and stores 8 bytes per lane instead of four 2-byte values.  Results are
+ * bit-identical to the plane entry points (same arithmetic, same summation order).  C, Cin and Cout of grouped
+ * tensors are multiples of 8; ld counts particles between two groups; at most 2^28 - 1 particles.
+ *   regroup8 / ungroup8     planes [C][ldx] <-> groups [C / 8][ldo][8] (channels past C read as zeros)
+ *   fill_tree_mean_bf16g    helpers::fill_tree_mean on grouped features, tree [C / 8][ld_tree][8]
+ *   maxpool_fwd_bf16g       MaxPool::forward, values only (the argmax serves the backward pass)
+ *   upsample_fwd_bf16g      UpSampleConst::forward
+ *   conv111_fwd_bf16g       Convolution<1,1,1>::forward with bias and optional ReLU; y grouped (y_grouped != 0) or planes
+ *   conv_fwd_fused_bf16l    aprnet_conv_fwd_fused_bf16 with a layout per tensor: x (and fusion->x2) grouped, or planes
+ *                           of 1 to 3 channels; y grouped or planes; tree_ws has the layout of x */
+int aprnet_regroup8_bf16(const uint16_t* x, int64_t ldx, int C, int64_t n, uint16_t* out, int64_t ldo, void* stream);
+int aprnet_ungroup8_bf16(const uint16_t* xg, int64_t ldg, int C, int64_t n, uint16_t* out, int64_t ldo, void* stream);
+int aprnet_fill_tree_mean_bf16g(const aprnet_plan*, int level_delta, const uint16_t* x, int64_t ldx, int C, uint16_t* tree,
+                                int64_t ld_tree, void* stream);
+int aprnet_maxpool_fwd_bf16g(const aprnet_plan*, int level_delta, const uint16_t* x, int64_t ldx, int C, uint16_t* y, int64_t ldy,
+                             void* stream);
+int aprnet_upsample_fwd_bf16g(const aprnet_plan*, int level_delta, const uint16_t* x, int64_t ldx, int C, uint16_t* y, int64_t ldy,
+                              void* stream);
+int aprnet_conv111_fwd_bf16g(const aprnet_plan*, int level_delta, const uint16_t* x, int64_t ldx, int Cin, const float* w, int S,
+                             int Cout, const float* bias, int relu, uint16_t* y, int64_t ldy, int y_grouped, void* stream);
+int aprnet_conv_fwd_fused_bf16l(const aprnet_plan*, int level_delta, int kz, int kx, int ky, const uint16_t* x, int64_t ldx, int Cin,
+                                int x_grouped, const float* w, int S_exp, int Cout, const float* bias, uint16_t* y, int64_t ldy,
+                                int y_grouped, uint16_t* tree_ws, int64_t ld_tree, const aprnet_conv_fusion* fusion, void* stream);
+
 /* Label and coordinate utilities of the StarDist networks (pyapr/aprnet/src/utils.hpp:86-333; CPU loops in the
  * reference, device kernels here).  Particle order = feature order at level_delta.  Images are dense device arrays
  * [zn][xn][yn] with the dimensions of the APR's finest level.

@@ -1,0 +1,120 @@
+"""bfloat16 features grouped by eight channels ([B, C / 8, N, 8]): every grouped operator against its plane twin
+(bit-identical where the arithmetic and its order are the same, which is everywhere but the 1x1x1 convolution) and
+the grouped network forward against the fp32 oracle."""
+import pytest
+import torch
+
+import apr_cases
+from oracle import oracle
+from pyapr import _native
+from pyapr.aprnet import _ops, grouped as g8
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def _batch(c, seed=0):
+    aprs = [apr_cases.get("3d_s"), apr_cases.get("3d_t")]
+    ld = torch.tensor([0, 1], dtype=torch.int32)
+    sizes = [oracle.number_parts(a, int(d)) for a, d in zip(aprs, ld)]
+    g = torch.Generator().manual_seed(seed)
+    x = torch.randn(2, c, max(sizes), generator=g).to(torch.bfloat16)
+    for i, n in enumerate(sizes):
+        x[i, :, n:] = 0
+    return aprs, ld, x.to(DEV), g
+
+
+def test_regroup_roundtrip_and_padding():
+    _, _, x, _ = _batch(24)
+    g = g8.regroup(x)
+    assert g.data.shape == (2, 3, x.shape[2], 8) and g.channels == 24
+    assert torch.equal(g8.ungroup(g), x)
+    assert torch.equal(g.data[:, 1, :, 3], x[:, 11, :])
+    odd = x[:, :13].contiguous()                       # 13 channels: the last group is padded with zeros
+    go = g8.regroup(odd)
+    assert go.channels == 16 and torch.equal(g8.ungroup(go, 13), odd) and float(go.data[:, 1, :, 5:].abs().max()) == 0
+
+
+def test_tree_fill_pool_upsample_equal_the_plane_kernels():
+    aprs, ld, x, _ = _batch(16, seed=1)
+    g = g8.regroup(x)
+    lib = _native.hip()
+    st = torch.cuda.current_stream().cuda_stream
+    for b, apr in enumerate(aprs):
+        d = int(ld[b])
+        nt = _ops.tree_parts(apr, d)
+        n = x.shape[2]
+        tp = torch.zeros(16, nt, dtype=torch.bfloat16, device=DEV)
+        tg = torch.zeros(2, nt, 8, dtype=torch.bfloat16, device=DEV)
+        assert lib.aprnet_fill_tree_mean_bf16(apr.plan(0), d, x[b].data_ptr(), n, 16, tp.data_ptr(), nt, st) == 0
+        assert lib.aprnet_fill_tree_mean_bf16g(apr.plan(0), d, g.data[b].data_ptr(), n, 16, tg.data_ptr(), nt, st) == 0
+        assert torch.equal(tg.permute(0, 2, 1).reshape(16, nt), tp)
+    pooled = g8.maxpool_forward(aprs, g, ld)
+    ref, _ = _ops.maxpool_forward(aprs, x, ld, 0.0)
+    assert torch.equal(g8.ungroup(pooled), ref)
+    up = g8.upsample_const_forward(aprs, pooled, ld + 1)
+    assert torch.equal(g8.ungroup(up), _ops.upsample_const_forward(aprs, ref, ld + 1))
+
+
+@pytest.mark.parametrize("ksize", [(3, 3, 3), (1, 5, 5)], ids=["333", "155"])
+@pytest.mark.parametrize("c1,c2,cout", [(16, 0, 16), (8, 24, 40), (32, 0, 8)])
+def test_grouped_convolution_equals_the_plane_kernel(c1, c2, cout, ksize):
+    """Grouped input (with and without a second input), grouped and plane output, bias and ReLU: bit-identical to the
+    fused plane entry point, which stages the same values from a regrouped copy."""
+    aprs, ld, x, g = _batch(c1 + c2, seed=2)
+    levels = max(a.level_max() - a.level_min() + 1 for a in aprs)
+    w = (torch.randn(levels, cout, c1 + c2, *ksize, generator=g) * 0.1).to(DEV)
+    bias = torch.randn(cout, generator=g).to(DEV)
+    xa, xb = x[:, :c1].contiguous(), (x[:, c1:].contiguous() if c2 else None)
+    ref = _ops.conv_forward(aprs, xa, w, ld, bias, relu=True, x2=xb)
+    got = g8.conv_forward(aprs, g8.regroup(xa), w, ld, bias, relu=True, x2=g8.regroup(xb) if c2 else None)
+    assert torch.equal(g8.ungroup(got), ref)
+    planes = g8.conv_forward(aprs, g8.regroup(xa), w, ld, bias, relu=False, x2=g8.regroup(xb) if c2 else None, grouped_output=False)
+    assert torch.equal(planes, _ops.conv_forward(aprs, xa, w, ld, bias, x2=xb))
+
+
+@pytest.mark.parametrize("cin", [1, 3])
+def test_first_layer_planes_in_grouped_out(cin):
+    aprs, ld, x, g = _batch(cin, seed=3)
+    levels = max(a.level_max() - a.level_min() + 1 for a in aprs)
+    w = (torch.randn(levels, 16, cin, 3, 3, 3, generator=g) * 0.2).to(DEV)
+    bias = torch.randn(16, generator=g).to(DEV)
+    got = g8.conv_forward(aprs, x, w, ld, bias, relu=True)
+    assert torch.equal(g8.ungroup(got), _ops.conv_forward(aprs, x, w, ld, bias, relu=True))
+
+
+@pytest.mark.parametrize("cin,cout,grouped_out", [(16, 8, True), (64, 32, True), (16, 3, False)])
+def test_grouped_conv111_against_oracle(cin, cout, grouped_out):
+    aprs, ld, x, g = _batch(cin, seed=4)
+    w = torch.randn(2, cout, cin, 1, 1, 1, generator=g) * 0.2
+    bias = torch.randn(cout, generator=g)
+    ref = oracle.conv_forward(aprs, x.float().cpu(), w.permute(2, 0, 1, 3, 4, 5).contiguous(), ld) + bias.view(1, -1, 1)
+    got = g8.conv111_forward(aprs, g8.regroup(x), w.to(DEV), ld, bias.to(DEV), relu=False, grouped_output=grouped_out)
+    got = g8.ungroup(got) if grouped_out else got
+    for b, a in enumerate(aprs):
+        n = oracle.number_parts(a, int(ld[b]))
+        err = float((got[b, :, :n].float().cpu() - ref[b, :, :n]).abs().max())
+        assert err <= 1e-2 * float(ref.abs().max())
+
+
+def test_unet_grouped_forward_against_oracle_and_plane_path():
+    """The 4-level network with bfloat16 features: the grouped path (default for inference with folded norms) against
+    the fp32 oracle composition (2e-2 of the output scale) and against the plane path of the same build (the two differ
+    only in the summation order of the 1x1x1 convolutions)."""
+    from bench import make_unet
+    from test_gpu_unet import reference_forward
+    apr = apr_cases.random_apr((33, 29, 37), 11, density=0.02)
+    n = apr.total_number_particles()
+    x = torch.randn(1, 1, n, generator=torch.Generator().manual_seed(5)).to(torch.bfloat16)
+    model = make_unet("cpu")
+    with torch.no_grad():
+        ref = reference_forward(model, x.float(), [apr])
+        model = model.to(DEV)
+        assert model._grouped_ok(x.to(DEV), [apr])
+        got = model(x.to(DEV), [apr])
+        model.use_grouped = False
+        planes = model(x.to(DEV), [apr])
+    assert got.shape == planes.shape == (1, 3, n) and got.dtype == torch.bfloat16
+    scale = float(ref.abs().max())
+    assert float((got.float().cpu() - ref).abs().max()) <= 2e-2 * scale
+    assert float((got.float() - planes.float()).abs().max()) <= 1e-2 * scale
