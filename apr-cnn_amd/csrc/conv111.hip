@@ -48,6 +48,10 @@ conv111_kernel(const T* __restrict__ src, int64_t lds, int Csrc, const T* __rest
 // whole kernel) and  B: lane l -> src[c = 2p + l/32][i0 + l%32]  (two coalesced 128-byte rows per load), so
 // the kernel streams the input once per 32 output channels and is bound by HBM.
 typedef float floatx16_111 __attribute__((ext_vector_type(16)));
+template <typename T> struct Pair111 { T v[2]; };        // two neighbours, alignment of one element
+template <int BYTES> struct PairBits111;
+template <> struct PairBits111<4> { typedef uint32_t type __attribute__((aligned(2))); };
+template <> struct PairBits111<8> { typedef uint32_t type __attribute__((ext_vector_type(2), aligned(4))); };
 
 // T = storage type of the features (float, or bfloat16 with fp32 weights, bias and arithmetic)
 template <typename T, int KP>      // KP = channel pairs held in registers (ceil(Csrc / 2) <= KP)
@@ -72,6 +76,42 @@ conv111_mfma_kernel(const T* __restrict__ src, int64_t lds, int Csrc, const floa
     const int64_t nwave = (int64_t)gridDim.x * (TB1 / 64);
     const int64_t wave = (int64_t)blockIdx.x * (TB1 / 64) + (threadIdx.x >> 6);
     for (int64_t i0 = begin + wave * 64; i0 < end; i0 += nwave * 64) {
+        if (i0 + 64 <= end) {
+            // whole block of 64 positions: lane `col` takes the neighbours i0 + 2 col and i0 + 2 col + 1 as one
+            // (element-aligned) pair, so a half-wave reads and writes 32 pairs in a row per channel
+            typedef typename PairBits111<2 * sizeof(T)>::type B;
+            const int64_t ip = i0 + 2 * col;
+            float va[KP], vb[KP];
+#pragma unroll
+            for (int p = 0; p < KP; ++p) {
+                const int c = 2 * p + hi;
+                if (c < Csrc) {
+                    // (one vector value each way: a struct of two elements is split into two half-width accesses again)
+                    const Pair111<T> pv = __builtin_bit_cast(Pair111<T>, *reinterpret_cast<const B*>(src + (int64_t)c * lds + ip));
+                    va[p] = Num<T>::ld(pv.v[0]); vb[p] = Num<T>::ld(pv.v[1]);
+                } else { va[p] = 0.f; vb[p] = 0.f; }
+            }
+            floatx16_111 acca, accb;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) { acca[r] = bs[r]; accb[r] = bs[r]; }
+#pragma unroll
+            for (int p = 0; p < KP; ++p) {
+                acca = __builtin_amdgcn_mfma_f32_32x32x2f32(aw[p], va[p], acca, 0, 0, 0);
+                accb = __builtin_amdgcn_mfma_f32_32x32x2f32(aw[p], vb[p], accb, 0, 0, 0);
+            }
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int o = o0 + 8 * (r >> 2) + 4 * hi + (r & 3);
+                if (o < Cdst) {
+                    float ya = acca[r], yb = accb[r];
+                    if (relu) { ya = ya < 0.f ? 0.f : ya; yb = yb < 0.f ? 0.f : yb; }
+                    Pair111<T> pv;
+                    pv.v[0] = Num<T>::st(ya); pv.v[1] = Num<T>::st(yb);
+                    *reinterpret_cast<B*>(dst + (int64_t)o * ldd + ip) = __builtin_bit_cast(B, pv);
+                }
+            }
+            continue;
+        }
         const int64_t ia = i0 + col, ib = i0 + 32 + col;
         float va[KP], vb[KP];
 #pragma unroll

@@ -1,77 +1,116 @@
 // Child-table operators: bottom-up tree fill (mean of children), max-pool with argmax, constant
 // upsampling, and their backward passes.  All are HBM-bound gathers/scatters: one thread per
-// (tree node, group of CPT channels), tree nodes of one level are contiguous, so every access is
+// (tree node, group of `cpt` channels), tree nodes of one level are contiguous, so every access is
 // coalesced along the node index and the eight child slots are read from slot-major planes, once for
-// the CPT channels of the thread (the index traffic would otherwise equal the data traffic).
+// the channels of the thread.  The slots are 32 bytes per node: against 8 x 4 bytes of fp32 data per node and channel
+// they cost 1/cpt of the data traffic on top, so cpt is as large as the launch allows (channels_per_thread).
 #include "common.hpp"
 
 namespace aprnet {
 
 constexpr int TB = 256;
-constexpr int CPT = 4;          // channels per thread
+constexpr int CPT_COARSE = 4;   // channels per workgroup of the coarse-level kernels
+constexpr int NB = 4;           // channels of one batch: all loads of a batch are issued before its first store
 
-// Children 2y and 2y + 1 of one (z, x) row are neighbours in memory when both are particles (or both tree nodes)
-// with consecutive indices: one 8-byte access for the two (element-aligned) instead of two 4-byte accesses whose
-// lanes each use half of every 8 bytes (4- and 16-byte pairs for bfloat16 and double).
-template <typename T> struct Pair { T v[2]; };        // alignment of one element
+// Channels per thread of a launch over n nodes: up to 16 (32 for 2-byte features), halved while fewer than 2^20
+// threads would remain (the chip holds 2^19 threads at a time).
+static int channels_per_thread(int64_t n, int C, size_t elem_bytes) {
+    int cpt = elem_bytes <= 2 ? 32 : 16;
+    while (cpt > NB && n * ((C + cpt - 1) / cpt) < ((int64_t)1 << 20)) cpt >>= 1;
+    return cpt;
+}
 
-// val[s] = value of child s (0 where there is none); particles from `part`, tree nodes from `tnode[~v]`.
-template <typename T>
-__device__ __forceinline__ void load_children(const int32_t (&ch)[8], const T* part,
-                                              const T* tnode, typename Num<T>::acc (&val)[8]) {
-    typedef typename Num<T>::acc A;
+// Walks the channels [c_begin, c_end) of a thread in batches of NB with two buffers: the loads of batch b + 1 are
+// issued BEFORE the stores of batch b, so that waiting for those loads (memory operations complete in issue order)
+// does not wait for the stores, and a thread has up to two batches of loads in flight.  The empty asm statements only
+// pin that order for the compiler, which otherwise sinks the loads of a channel below the stores of the one before.
+#define APRNET_ORDER() __asm__ volatile("" ::: "memory")
+template <int NBT, typename Buf, typename Load, typename Use>
+__device__ __forceinline__ void channel_pipeline(int c_begin, int c_end, Load load, Use use) {
+    Buf a, b;
+    load(c_begin, a);
+    APRNET_ORDER();
+    for (int c = c_begin; c < c_end; c += 2 * NBT) {
+        if (c + NBT < c_end) load(c + NBT, b);
+        APRNET_ORDER();
+        use(c, a);
+        APRNET_ORDER();
+        if (c + NBT >= c_end) break;
+        if (c + 2 * NBT < c_end) load(c + 2 * NBT, a);
+        APRNET_ORDER();
+        use(c + NBT, b);
+        APRNET_ORDER();
+    }
+}
+// Kernels that mostly store need less in flight than kernels that mostly load: two channels per batch.
+#ifndef APRNET_NBS
+#define APRNET_NBS 2
+#endif
+constexpr int NBS = APRNET_NBS;
+template <typename A, int NBT = NB> struct KidVals { A v[NBT][8]; };
+template <typename T, int NBT = NB> struct RowVals { T v[NBT]; };
+
+// The eight child slots of one tree node, decoded once per thread.  Every load that follows is unconditional (a
+// missing child reads element 0 of the particle plane and its value is dropped): a load under a per-lane branch
+// makes the compiler wait for memory inside the branch, which serialises the eight children of every channel.
+struct Kids {
+    int32_t off[8];                 // index among the particles (>= 0 in the table) or among the tree nodes (~v)
+    uint32_t tree_mask, has_mask;   // bit s: child s is a tree node / exists
+    __device__ __forceinline__ void read(const int32_t* __restrict__ children, int64_t n_tree, int64_t t) {
+        int32_t v[8];
 #pragma unroll
-    for (int s = 0; s < 8; s += 2) {
-        const int32_t v0 = ch[s], v1 = ch[s + 1];
-        bool paired = false;
-        if constexpr (sizeof(T) >= 2) {
-            const bool pp = v0 >= 0 && v1 == v0 + 1;
-            const bool tt = v0 < 0 && v0 != NO_CHILD && v1 == v0 - 1;
-            if (pp || tt) {
-                const T* src = pp ? part + v0 : tnode + ~v0;
-                const Pair<T> pv = *reinterpret_cast<const Pair<T>*>(src);
-                val[s] = Num<T>::ld(pv.v[0]); val[s + 1] = Num<T>::ld(pv.v[1]);
-                paired = true;
-            }
-        }
-        if (!paired) {
+        for (int s = 0; s < 8; ++s) v[s] = children[(int64_t)s * n_tree + t];
+        tree_mask = has_mask = 0;
 #pragma unroll
-            for (int k2 = 0; k2 < 2; ++k2) {
-                const int32_t v = k2 ? v1 : v0;
-                A r = 0;
-                if (v >= 0) r = Num<T>::ld(part[v]);
-                else if (v != NO_CHILD) r = Num<T>::ld(tnode[~v]);
-                val[s + k2] = r;
-            }
+        for (int s = 0; s < 8; ++s) {
+            const bool has = v[s] != NO_CHILD, tr = has && v[s] < 0;
+            off[s] = has ? (tr ? ~v[s] : v[s]) : 0;
+            has_mask |= (uint32_t)has << s;
+            tree_mask |= (uint32_t)tr << s;
         }
+    }
+    __device__ __forceinline__ bool has(int s) const { return (has_mask >> s) & 1u; }
+    __device__ __forceinline__ bool tree(int s) const { return (tree_mask >> s) & 1u; }
+    __device__ __forceinline__ int count() const { return __popc(has_mask); }
+    template <typename T> __device__ __forceinline__ T* ptr(int s, T* part, T* tnode) const { return (tree(s) ? tnode : part) + off[s]; }
+};
+
+// val[k][s] = value of child s in channel c + k, k < NBT (channels past c_end repeat the last one; the caller drops them)
+template <typename T, int NBT = NB>
+__device__ __forceinline__ void load_children(const Kids& kd, const T* part, int64_t ldp, const T* tnode, int64_t ldt,
+                                              int c, int c_end, KidVals<typename Num<T>::acc, NBT>& val) {
+#pragma unroll
+    for (int k = 0; k < NBT; ++k) {
+        const int cc = min(c + k, c_end - 1);
+        const T* pb = part + (int64_t)cc * ldp;
+        const T* tb = tnode + (int64_t)cc * ldt;
+#pragma unroll
+        for (int s = 0; s < 8; ++s) val.v[k][s] = Num<T>::ld(*kd.ptr(s, pb, tb));
     }
 }
 
-// Writes val[s] to child s for every existing child, pairs in one 8-byte store.
+// Children 2y and 2y + 1 of one (z, x) row are neighbours in memory when both are particles (or both tree nodes)
+// with consecutive indices: one 8-byte store for the two (element-aligned) instead of two 4-byte stores (4- and
+// 16-byte pairs for bfloat16 and double).  Stores need no wait, so these branches cost nothing.
+// (The pair goes out as ONE vector value: a struct of two elements is split into two stores again, each of which
+// fills only every other element of the lines it touches.)
+template <typename T> struct Pair { T v[2]; };
+template <int BYTES> struct PairBits;
+template <> struct PairBits<4> { typedef uint32_t type __attribute__((aligned(2))); };
+template <> struct PairBits<8> { typedef uint32_t type __attribute__((ext_vector_type(2), aligned(4))); };
+template <> struct PairBits<16> { typedef uint32_t type __attribute__((ext_vector_type(4), aligned(8))); };
 template <typename T>
-__device__ __forceinline__ void store_children(const int32_t (&ch)[8], T* part, T* tnode,
-                                               const T (&val)[8]) {
+__device__ __forceinline__ void store_children(const Kids& kd, T* part, T* tnode, const T (&val)[8]) {
 #pragma unroll
     for (int s = 0; s < 8; s += 2) {
-        const int32_t v0 = ch[s], v1 = ch[s + 1];
-        bool paired = false;
-        if constexpr (sizeof(T) >= 2) {
-            const bool pp = v0 >= 0 && v1 == v0 + 1;
-            const bool tt = v0 < 0 && v0 != NO_CHILD && v1 == v0 - 1;
-            if (pp || tt) {
-                Pair<T> pv;
-                pv.v[0] = val[s]; pv.v[1] = val[s + 1];
-                *reinterpret_cast<Pair<T>*>(pp ? part + v0 : tnode + ~v0) = pv;
-                paired = true;
-            }
-        }
-        if (!paired) {
-#pragma unroll
-            for (int k2 = 0; k2 < 2; ++k2) {
-                const int32_t v = k2 ? v1 : v0;
-                if (v >= 0) part[v] = val[s + k2];
-                else if (v != NO_CHILD) tnode[~v] = val[s + k2];
-            }
+        if (kd.has(s) && kd.has(s + 1) && kd.tree(s) == kd.tree(s + 1) && kd.off[s + 1] == kd.off[s] + 1) {
+            typedef typename PairBits<2 * sizeof(T)>::type B;
+            Pair<T> pv;
+            pv.v[0] = val[s]; pv.v[1] = val[s + 1];
+            *reinterpret_cast<B*>(kd.ptr(s, part, tnode)) = __builtin_bit_cast(B, pv);
+        } else {
+            if (kd.has(s)) *kd.ptr(s, part, tnode) = val[s];
+            if (kd.has(s + 1)) *kd.ptr(s + 1, part, tnode) = val[s + 1];
         }
     }
 }
@@ -84,48 +123,46 @@ __device__ __forceinline__ void store_children(const int32_t (&ch)[8], T* part, 
 template <typename T>
 __device__ __forceinline__ void fill_node(const int32_t* children, int64_t n_tree, int64_t t, const T* x, int64_t ldx,
                                           int C, T* tree, int64_t ldt, int64_t tree_off, int tree_child_from_x,
-                                          int tree_first, int cg) {
-    int32_t ch[8];
-    int cnt = 0;
-#pragma unroll
-    for (int s = 0; s < 8; ++s) { ch[s] = children[(int64_t)s * n_tree + t]; cnt += ch[s] != NO_CHILD; }
+                                          int tree_first, int c_begin, int cpt) {
+    Kids kd;
+    kd.read(children, n_tree, t);
     // 1/cnt is a power of two (cnt = product of 1-or-2 per dimension, helpers.hpp:133-153)
     typedef typename Num<T>::acc A;
-    const A scale = (A)(1.0f / (float)max(cnt, 1));
+    const A scale = (A)(1.0f / (float)max(kd.count(), 1));
+    const int c_end = min(C, c_begin + cpt);
+    // tree children: a window of the feature planes (parents directly under the features) or the tree planes
+    const T* tn = tree_child_from_x ? x + tree_off : tree;
+    const int64_t ldn = tree_child_from_x ? ldx : ldt;
+    channel_pipeline<NB, KidVals<A>>(c_begin, c_end,
+        [&](int c, KidVals<A>& val) { load_children<T>(kd, x, ldx, tn, ldn, c, c_end, val); },
+        [&](int c, const KidVals<A>& val) {
 #pragma unroll
-    for (int k = 0; k < CPT; ++k) {
-        const int c = cg * CPT + k;
-        if (c >= C) break;
-        const T* xc = x + (int64_t)c * ldx;
-        T* tc = tree + (int64_t)c * ldt;
-        A val[8];
-        load_children<T>(ch, xc, tree_child_from_x ? xc + tree_off : tc, val);
-        A sum = 0;
+            for (int k = 0; k < NB; ++k) {
+                if (c + k >= c_end) break;
+                A sum = 0;
 #pragma unroll
-        for (int pass = 0; pass < 2; ++pass) {
-            const bool want_tree = (pass == 0) == (tree_first != 0);
+                for (int pass = 0; pass < 2; ++pass) {
+                    const bool want_tree = (pass == 0) == (tree_first != 0);
 #pragma unroll
-            for (int s = 0; s < 8; ++s) {
-                const int32_t v = ch[s];
-                if (v == NO_CHILD) continue;
-                if (want_tree == (v < 0)) sum += val[s];
+                    for (int s = 0; s < 8; ++s)
+                        if (kd.has(s) && want_tree == kd.tree(s)) sum += val.v[k][s];
+                }
+                tree[(int64_t)(c + k) * ldt + t] = Num<T>::st(sum * scale);
             }
-        }
-        tc[t] = Num<T>::st(sum * scale);
-    }
+        });
 }
 
 template <typename T>
 __global__ void __launch_bounds__(TB)
 fill_tree_level_kernel(const int32_t* __restrict__ children, int64_t n_tree, int64_t t_begin, int64_t t_end,
                        const T* __restrict__ x, int64_t ldx, int C, T* __restrict__ tree, int64_t ldt,
-                       int64_t tree_off, int tree_child_from_x, int tree_first) {
+                       int64_t tree_off, int tree_child_from_x, int tree_first, int cpt) {
     const int64_t t = t_begin + (int64_t)blockIdx.x * TB + threadIdx.x;
-    if (t < t_end) fill_node<T>(children, n_tree, t, x, ldx, C, tree, ldt, tree_off, tree_child_from_x, tree_first, blockIdx.y);
+    if (t < t_end) fill_node<T>(children, n_tree, t, x, ldx, C, tree, ldt, tree_off, tree_child_from_x, tree_first, blockIdx.y * cpt, cpt);
 }
 
 // The coarse levels of the tree hold a few nodes each: one launch walks them all, finest first, one workgroup per
-// group of CPT channels (a level's parents read only values of the same channels, so a workgroup barrier between
+// group of CPT_COARSE channels (a level's parents read only values of the same channels, so a workgroup barrier between
 // levels is enough).  Tree children come from the tree itself (none of these levels sits directly under the features),
 // particle children from the feature vector as always.
 constexpr int MAX_COARSE = 12;
@@ -138,7 +175,7 @@ fill_tree_coarse_kernel(const int32_t* __restrict__ children, int64_t n_tree, co
                         int C, T* tree, int64_t ldt) {
     for (int i = 0; i < lv.n; ++i) {
         for (int64_t t = lv.begin[i] + threadIdx.x; t < lv.end[i]; t += TB)
-            fill_node<T>(children, n_tree, t, x, ldx, C, tree, ldt, 0, 0, 0, blockIdx.x);
+            fill_node<T>(children, n_tree, t, x, ldx, C, tree, ldt, 0, 0, 0, blockIdx.x * CPT_COARSE, CPT_COARSE);
         __syncthreads();
     }
 }
@@ -146,37 +183,41 @@ fill_tree_coarse_kernel(const int32_t* __restrict__ children, int64_t n_tree, co
 // helpers.hpp:255-350, parent-driven: every child has exactly one parent, so no write conflicts.
 template <typename T>
 __device__ __forceinline__ void fill_node_bwd(const int32_t* children, int64_t n_tree, int64_t t, T* gx, int64_t ldx,
-                                              int C, T* gtree, int64_t ldt, int64_t tree_off, int tree_child_in_x, int cg) {
-    int32_t ch[8];
-    int cnt = 0;
-#pragma unroll
-    for (int s = 0; s < 8; ++s) { ch[s] = children[(int64_t)s * n_tree + t]; cnt += ch[s] != NO_CHILD; }
+                                              int C, T* gtree, int64_t ldt, int64_t tree_off, int tree_child_in_x,
+                                              int c_begin, int cpt) {
+    Kids kd;
+    kd.read(children, n_tree, t);
     typedef typename Num<T>::acc A;
-    const A scale = (A)(1.0f / (float)max(cnt, 1));
+    const A scale = (A)(1.0f / (float)max(kd.count(), 1));
+    const int c_end = min(C, c_begin + cpt);
+    T* tn = tree_child_in_x ? gx + tree_off : gtree;
+    const int64_t ldn = tree_child_in_x ? ldx : ldt;
+    struct Buf { A g[NBS]; KidVals<A, NBS> val; };
+    channel_pipeline<NBS, Buf>(c_begin, c_end,
+        [&](int c, Buf& b) {
 #pragma unroll
-    for (int k = 0; k < CPT; ++k) {
-        const int c = cg * CPT + k;
-        if (c >= C) break;
-        T* gxc = gx + (int64_t)c * ldx;
-        T* gtc = gtree + (int64_t)c * ldt;
-        const A g = Num<T>::ld(gtc[t]) * scale;
-        T* gt_child = tree_child_in_x ? gxc + tree_off : gtc;
-        A val[8];
-        load_children<T>(ch, gxc, gt_child, val);
-        T out[8];
+            for (int k = 0; k < NBS; ++k) b.g[k] = Num<T>::ld(gtree[(int64_t)min(c + k, c_end - 1) * ldt + t]);
+            load_children<T, NBS>(kd, (const T*)gx, ldx, (const T*)tn, ldn, c, c_end, b.val);
+        },
+        [&](int c, const Buf& b) {
 #pragma unroll
-        for (int s = 0; s < 8; ++s) out[s] = Num<T>::st(val[s] + g);
-        store_children<T>(ch, gxc, gt_child, out);
-    }
+            for (int k = 0; k < NBS; ++k) {
+                if (c + k >= c_end) break;
+                T out[8];
+#pragma unroll
+                for (int s = 0; s < 8; ++s) out[s] = Num<T>::st(b.val.v[k][s] + b.g[k] * scale);
+                store_children<T>(kd, gx + (int64_t)(c + k) * ldx, tn + (int64_t)(c + k) * ldn, out);
+            }
+        });
 }
 
 template <typename T>
 __global__ void __launch_bounds__(TB)
 fill_tree_bwd_level_kernel(const int32_t* __restrict__ children, int64_t n_tree, int64_t t_begin, int64_t t_end,
-                           T* __restrict__ gx, int64_t ldx, int C, T* __restrict__ gtree, int64_t ldt,
-                           int64_t tree_off, int tree_child_in_x) {
+                           T* gx, int64_t ldx, int C, T* gtree, int64_t ldt,
+                           int64_t tree_off, int tree_child_in_x, int cpt) {
     const int64_t t = t_begin + (int64_t)blockIdx.x * TB + threadIdx.x;
-    if (t < t_end) fill_node_bwd<T>(children, n_tree, t, gx, ldx, C, gtree, ldt, tree_off, tree_child_in_x, blockIdx.y);
+    if (t < t_end) fill_node_bwd<T>(children, n_tree, t, gx, ldx, C, gtree, ldt, tree_off, tree_child_in_x, blockIdx.y * cpt, cpt);
 }
 
 // the coarse levels in one launch, coarsest first (a parent's share must have arrived before it is handed down)
@@ -186,7 +227,7 @@ fill_tree_bwd_coarse_kernel(const int32_t* __restrict__ children, int64_t n_tree
                             int C, T* gtree, int64_t ldt) {
     for (int i = 0; i < lv.n; ++i) {
         for (int64_t t = lv.begin[i] + threadIdx.x; t < lv.end[i]; t += TB)
-            fill_node_bwd<T>(children, n_tree, t, gx, ldx, C, gtree, ldt, 0, 0, blockIdx.x);
+            fill_node_bwd<T>(children, n_tree, t, gx, ldx, C, gtree, ldt, 0, 0, blockIdx.x * CPT_COARSE, CPT_COARSE);
         __syncthreads();
     }
 }
@@ -198,45 +239,44 @@ template <typename T>
 __global__ void __launch_bounds__(TB)
 maxpool_fwd_kernel(const int32_t* __restrict__ children, int64_t n_tree, int64_t n_copy, int64_t n_out,
                    int64_t t_begin, const T* __restrict__ x, int64_t ldx, int C, T* __restrict__ y, int64_t ldy,
-                   int64_t* __restrict__ arg, int64_t ldi, int64_t in_tree_off) {
+                   int64_t* __restrict__ arg, int64_t ldi, int64_t in_tree_off, int cpt) {
     const int64_t i = (int64_t)blockIdx.x * TB + threadIdx.x;
     if (i >= n_out) return;
+    const int c_begin = blockIdx.y * cpt, c_end = min(C, c_begin + cpt);
     if (i < n_copy) {
+        channel_pipeline<NB, RowVals<T>>(c_begin, c_end,
+            [&](int c, RowVals<T>& r) {
 #pragma unroll
-        for (int k = 0; k < CPT; ++k) {
-            const int c = blockIdx.y * CPT + k;
-            if (c >= C) break;
-            y[(int64_t)c * ldy + i] = x[(int64_t)c * ldx + i]; arg[(int64_t)c * ldi + i] = 0;
-        }
+                for (int k = 0; k < NB; ++k) r.v[k] = x[(int64_t)min(c + k, c_end - 1) * ldx + i];
+            },
+            [&](int c, const RowVals<T>& r) {
+#pragma unroll
+                for (int k = 0; k < NB; ++k)
+                    if (c + k < c_end) { y[(int64_t)(c + k) * ldy + i] = r.v[k]; arg[(int64_t)(c + k) * ldi + i] = 0; }
+            });
         return;
     }
-    const int64_t t = t_begin + (i - n_copy);
-    int32_t ch[8];
+    Kids kd;
+    kd.read(children, n_tree, t_begin + (i - n_copy));
+    typedef typename Num<T>::acc A;
+    channel_pipeline<NB, KidVals<A>>(c_begin, c_end,
+        [&](int c, KidVals<A>& val) { load_children<T>(kd, x, ldx, x + in_tree_off, ldx, c, c_end, val); },
+        [&](int c, const KidVals<A>& val) {
 #pragma unroll
-    for (int s = 0; s < 8; ++s) ch[s] = children[(int64_t)s * n_tree + t];
+            for (int k = 0; k < NB; ++k) {
+                if (c + k >= c_end) break;
+                A best = (A)(-1e17f);               // initial value of the output, maxpool.hpp:51
+                int64_t best_i = 0;
 #pragma unroll
-    for (int k = 0; k < CPT; ++k) {
-        const int c = blockIdx.y * CPT + k;
-        if (c >= C) break;
-        const T* xc = x + (int64_t)c * ldx;
-        typedef typename Num<T>::acc A;
-        A best = (A)(-1e17f);               // initial value of the output, maxpool.hpp:51
-        int64_t best_i = 0;
-        A val[8];
-        load_children<T>(ch, xc, xc + in_tree_off, val);
+                for (int s = 0; s < 8; ++s)
+                    if (kd.has(s) && !kd.tree(s) && val.v[k][s] > best) { best = val.v[k][s]; best_i = kd.off[s]; }
 #pragma unroll
-        for (int s = 0; s < 8; ++s) {
-            const int32_t v = ch[s];
-            if (v >= 0 && val[s] > best) { best = val[s]; best_i = v; }
-        }
-#pragma unroll
-        for (int s = 0; s < 8; ++s) {
-            const int32_t v = ch[s];
-            if (v < 0 && v != NO_CHILD && val[s] > best) { best = val[s]; best_i = (int64_t)(~v) + in_tree_off; }
-        }
-        y[(int64_t)c * ldy + i] = Num<T>::st(best);
-        arg[(int64_t)c * ldi + i] = best_i;
-    }
+                for (int s = 0; s < 8; ++s)
+                    if (kd.tree(s) && val.v[k][s] > best) { best = val.v[k][s]; best_i = (int64_t)kd.off[s] + in_tree_off; }
+                y[(int64_t)(c + k) * ldy + i] = Num<T>::st(best);
+                arg[(int64_t)(c + k) * ldi + i] = best_i;
+            }
+        });
 }
 
 // maxpool.hpp:170-230 without the zero-fill pass: every input position of level Lc has exactly one
@@ -245,85 +285,137 @@ template <typename T>
 __global__ void __launch_bounds__(TB)
 maxpool_bwd_kernel(const int32_t* __restrict__ children, int64_t n_tree, int64_t n_copy, int64_t n_out,
                    int64_t t_begin, const T* __restrict__ gy, int64_t ldy, int C, T* __restrict__ gx, int64_t ldx,
-                   const int64_t* __restrict__ arg, int64_t ldi, int64_t in_tree_off) {
+                   const int64_t* __restrict__ arg, int64_t ldi, int64_t in_tree_off, int cpt) {
     const int64_t i = (int64_t)blockIdx.x * TB + threadIdx.x;
     if (i >= n_out) return;
+    const int c_begin = blockIdx.y * cpt, c_end = min(C, c_begin + cpt);
     if (i < n_copy) {
+        channel_pipeline<NB, RowVals<T>>(c_begin, c_end,
+            [&](int c, RowVals<T>& r) {
 #pragma unroll
-        for (int k = 0; k < CPT; ++k) {
-            const int c = blockIdx.y * CPT + k;
-            if (c >= C) break;
-            gx[(int64_t)c * ldx + i] = gy[(int64_t)c * ldy + i];
-        }
+                for (int k = 0; k < NB; ++k) r.v[k] = gy[(int64_t)min(c + k, c_end - 1) * ldy + i];
+            },
+            [&](int c, const RowVals<T>& r) {
+#pragma unroll
+                for (int k = 0; k < NB; ++k)
+                    if (c + k < c_end) { gx[(int64_t)(c + k) * ldx + i] = r.v[k]; }
+            });
         return;
     }
-    const int64_t t = t_begin + (i - n_copy);
-    int32_t ch[8];
+    Kids kd;
+    kd.read(children, n_tree, t_begin + (i - n_copy));
+    struct Buf { T g[NBS]; int64_t m[NBS]; };
+    channel_pipeline<NBS, Buf>(c_begin, c_end,
+        [&](int c, Buf& b) {
 #pragma unroll
-    for (int s = 0; s < 8; ++s) ch[s] = children[(int64_t)s * n_tree + t];
+            for (int k = 0; k < NBS; ++k) {
+                const int cc = min(c + k, c_end - 1);
+                b.g[k] = gy[(int64_t)cc * ldy + i];
+                b.m[k] = arg[(int64_t)cc * ldi + i];
+            }
+        },
+        [&](int c, const Buf& b) {
 #pragma unroll
-    for (int k = 0; k < CPT; ++k) {
-        const int c = blockIdx.y * CPT + k;
-        if (c >= C) break;
-        T* gxc = gx + (int64_t)c * ldx;
-        const T g = gy[(int64_t)c * ldy + i];
-        const int64_t m = arg[(int64_t)c * ldi + i];
-        T out[8];
+            for (int k = 0; k < NBS; ++k) {
+                if (c + k >= c_end) break;
+                T* gxc = gx + (int64_t)(c + k) * ldx;
+                T out[8];
 #pragma unroll
-        for (int s = 0; s < 8; ++s) {
-            const int32_t v = ch[s];
-            const int64_t j = v >= 0 ? (int64_t)v : (int64_t)(~v) + in_tree_off;
-            out[s] = (j == m) ? g : Num<T>::st(0);
-        }
-        store_children<T>(ch, gxc, gxc + in_tree_off, out);
-    }
+                for (int s = 0; s < 8; ++s) {
+                    const int64_t j = (int64_t)kd.off[s] + (kd.tree(s) ? in_tree_off : 0);
+                    out[s] = (j == b.m[k]) ? b.g[k] : Num<T>::st(0);
+                }
+                store_children<T>(kd, gxc, gxc + in_tree_off, out);
+            }
+        });
 }
 
 // ---------------------------------------------------------------------------- upsample (constant)
-// upsample.hpp:72-141.  Input slot i < n_copy: copy.  Otherwise downsampled particle = tree node t of
-// level Lc: its value goes to every child (particle of level Lc+1, or tree node of level Lc+1).
-template <typename T, bool Backward>
+// Backward of upsample.hpp:72-141 (upsample.hpp:199-232).  Gradient slot i < n_copy: copy.  Otherwise downsampled
+// particle = tree node t of level Lc: the sum of its children's gradients, particles first, then tree nodes.
+template <typename T>
 __global__ void __launch_bounds__(TB)
-upsample_kernel(const int32_t* __restrict__ children, int64_t n_tree, int64_t n_copy, int64_t n_in,
-                int64_t t_begin, const T* __restrict__ src, int64_t lds, int C, T* __restrict__ dst, int64_t ldd,
-                int64_t out_tree_off) {
+upsample_bwd_kernel(const int32_t* __restrict__ children, int64_t n_tree, int64_t n_copy, int64_t n_in,
+                    int64_t t_begin, const T* __restrict__ src, int64_t lds, int C, T* __restrict__ dst, int64_t ldd,
+                    int64_t out_tree_off, int cpt) {
     const int64_t i = (int64_t)blockIdx.x * TB + threadIdx.x;
     if (i >= n_in) return;
-    // forward: src = input at d, dst = output at d-1.  backward: src = grad_output, dst = grad_input.
+    const int c_begin = blockIdx.y * cpt, c_end = min(C, c_begin + cpt);
     if (i < n_copy) {
+        channel_pipeline<NB, RowVals<T>>(c_begin, c_end,
+            [&](int c, RowVals<T>& r) {
 #pragma unroll
-        for (int k = 0; k < CPT; ++k) {
-            const int c = blockIdx.y * CPT + k;
-            if (c >= C) break;
-            dst[(int64_t)c * ldd + i] = src[(int64_t)c * lds + i];
-        }
+                for (int k = 0; k < NB; ++k) r.v[k] = src[(int64_t)min(c + k, c_end - 1) * lds + i];
+            },
+            [&](int c, const RowVals<T>& r) {
+#pragma unroll
+                for (int k = 0; k < NB; ++k)
+                    if (c + k < c_end) { dst[(int64_t)(c + k) * ldd + i] = r.v[k]; }
+            });
         return;
     }
-    const int64_t t = t_begin + (i - n_copy);
-    int32_t ch[8];
+    Kids kd;
+    kd.read(children, n_tree, t_begin + (i - n_copy));
+    typedef typename Num<T>::acc A;
+    channel_pipeline<NB, KidVals<A>>(c_begin, c_end,
+        [&](int c, KidVals<A>& val) { load_children<T>(kd, src, lds, src + out_tree_off, lds, c, c_end, val); },
+        [&](int c, const KidVals<A>& val) {
 #pragma unroll
-    for (int s = 0; s < 8; ++s) ch[s] = children[(int64_t)s * n_tree + t];
+            for (int k = 0; k < NB; ++k) {
+                if (c + k >= c_end) break;
+                A sum = 0;
 #pragma unroll
-    for (int k = 0; k < CPT; ++k) {
-        const int c = blockIdx.y * CPT + k;
-        if (c >= C) break;
-        const T* s_ = src + (int64_t)c * lds;
-        T* d_ = dst + (int64_t)c * ldd;
-        if (!Backward) {
-            T out[8];
+                for (int s = 0; s < 8; ++s) if (kd.has(s) && !kd.tree(s)) sum += val.v[k][s];
 #pragma unroll
-            for (int s = 0; s < 8; ++s) out[s] = s_[i];
-            store_children<T>(ch, d_, d_ + out_tree_off, out);
-        } else {
-            typename Num<T>::acc sum = 0, val[8];      // particles first, then tree nodes (upsample.hpp:199-232)
-            load_children<T>(ch, s_, s_ + out_tree_off, val);
+                for (int s = 0; s < 8; ++s) if (kd.tree(s)) sum += val.v[k][s];
+                dst[(int64_t)(c + k) * ldd + i] = Num<T>::st(sum);
+            }
+        });
+}
+
+// upsample.hpp:72-141.  Input slot i < n_copy: copy.  Otherwise downsampled particle = tree node t of level Lc: its
+// value goes to every child (particle of level Lc + 1, or tree node of level Lc + 1).
+// (A child-driven form -- one thread per 16 bytes of consecutive outputs, the source index from a parent table -- writes
+// perfectly coalesced lines but was no faster: each parent value is then fetched by up to four XCDs.)
+template <typename T>
+__global__ void __launch_bounds__(TB)
+upsample_fwd_kernel(const int32_t* __restrict__ children, int64_t n_tree, int64_t n_copy, int64_t n_in,
+                    int64_t t_begin, const T* __restrict__ src, int64_t lds, int C, T* __restrict__ dst, int64_t ldd,
+                    int64_t out_tree_off, int cpt) {
+    const int64_t i = (int64_t)blockIdx.x * TB + threadIdx.x;
+    if (i >= n_in) return;
+    const int c_begin = blockIdx.y * cpt, c_end = min(C, c_begin + cpt);
+    if (i < n_copy) {
+        channel_pipeline<NB, RowVals<T>>(c_begin, c_end,
+            [&](int c, RowVals<T>& r) {
 #pragma unroll
-            for (int s = 0; s < 8; ++s) if (ch[s] >= 0) sum += val[s];
+                for (int k = 0; k < NB; ++k) r.v[k] = src[(int64_t)min(c + k, c_end - 1) * lds + i];
+            },
+            [&](int c, const RowVals<T>& r) {
 #pragma unroll
-            for (int s = 0; s < 8; ++s) if (ch[s] < 0 && ch[s] != NO_CHILD) sum += val[s];
-            d_[i] = Num<T>::st(sum);
-        }
+                for (int k = 0; k < NB; ++k)
+                    if (c + k < c_end) { dst[(int64_t)(c + k) * ldd + i] = r.v[k]; }
+            });
+        return;
     }
+    Kids kd;
+    kd.read(children, n_tree, t_begin + (i - n_copy));
+    channel_pipeline<NBS, RowVals<T, NBS>>(c_begin, c_end,
+        [&](int c, RowVals<T, NBS>& r) {
+#pragma unroll
+            for (int k = 0; k < NBS; ++k) r.v[k] = src[(int64_t)min(c + k, c_end - 1) * lds + i];
+        },
+        [&](int c, const RowVals<T, NBS>& r) {
+#pragma unroll
+            for (int k = 0; k < NBS; ++k) {
+                if (c + k >= c_end) break;
+                T* d_ = dst + (int64_t)(c + k) * ldd;
+                T out[8];
+#pragma unroll
+                for (int s = 0; s < 8; ++s) out[s] = r.v[k];
+                store_children<T>(kd, d_, d_ + out_tree_off, out);
+            }
+        });
 }
 
 // ---------------------------------------------------------------------------- host launchers
@@ -352,16 +444,17 @@ int fill_tree_mean(const aprnet_plan* p, int d, const T* x, int64_t ldx, int C, 
     for (int l = l_top; l > l_coarse; --l) {
         const int64_t b = p->tree.level_begin(l), e = p->tree.level_end(l);
         if (e <= b) continue;
-        dim3 grid((unsigned)((e - b + TB - 1) / TB), (unsigned)((C + CPT - 1) / CPT));
+        const int cpt = channels_per_thread(e - b, C, sizeof(T));
+        dim3 grid((unsigned)((e - b + TB - 1) / TB), (unsigned)((C + cpt - 1) / cpt));
         const int from_x = (l + 1 == Lc);
         hipLaunchKernelGGL(fill_tree_level_kernel<T>, grid, dim3(TB), 0, st, p->d_children, p->n_tree, b, e, x, ldx, C,
-                           tree, ldt, from_x ? p->tree_offset(Lc) : 0, from_x, from_x);
+                           tree, ldt, from_x ? p->tree_offset(Lc) : 0, from_x, from_x, cpt);
     }
     CoarseLevels lv{};
     for (int l = l_coarse; l >= p->tree.level_min; --l)
         if (p->tree.level_end(l) > p->tree.level_begin(l)) { lv.begin[lv.n] = p->tree.level_begin(l); lv.end[lv.n] = p->tree.level_end(l); ++lv.n; }
     if (lv.n > 0)
-        hipLaunchKernelGGL(fill_tree_coarse_kernel<T>, dim3((unsigned)((C + CPT - 1) / CPT)), dim3(TB), 0, st, p->d_children, p->n_tree,
+        hipLaunchKernelGGL(fill_tree_coarse_kernel<T>, dim3((unsigned)((C + CPT_COARSE - 1) / CPT_COARSE)), dim3(TB), 0, st, p->d_children, p->n_tree,
                            lv, x, ldx, C, tree, ldt);
     APRNET_LAUNCH_CHECK("fill_tree kernels");
     return 0;
@@ -378,15 +471,16 @@ int fill_tree_mean_bwd(const aprnet_plan* p, int d, T* gx, int64_t ldx, int C, T
     for (int l = p->tree.level_min; l <= l_coarse; ++l)
         if (p->tree.level_end(l) > p->tree.level_begin(l)) { lv.begin[lv.n] = p->tree.level_begin(l); lv.end[lv.n] = p->tree.level_end(l); ++lv.n; }
     if (lv.n > 0)
-        hipLaunchKernelGGL(fill_tree_bwd_coarse_kernel<T>, dim3((unsigned)((C + CPT - 1) / CPT)), dim3(TB), 0, st, p->d_children,
+        hipLaunchKernelGGL(fill_tree_bwd_coarse_kernel<T>, dim3((unsigned)((C + CPT_COARSE - 1) / CPT_COARSE)), dim3(TB), 0, st, p->d_children,
                            p->n_tree, lv, gx, ldx, C, gtree, ldt);
     for (int l = std::max(l_coarse + 1, p->tree.level_min); l <= l_top; ++l) {
         const int64_t b = p->tree.level_begin(l), e = p->tree.level_end(l);
         if (e <= b) continue;
-        dim3 grid((unsigned)((e - b + TB - 1) / TB), (unsigned)((C + CPT - 1) / CPT));
+        const int cpt = channels_per_thread(e - b, C, sizeof(T));
+        dim3 grid((unsigned)((e - b + TB - 1) / TB), (unsigned)((C + cpt - 1) / cpt));
         const int in_x = (l + 1 == Lc);
         hipLaunchKernelGGL(fill_tree_bwd_level_kernel<T>, grid, dim3(TB), 0, st, p->d_children, p->n_tree, b, e, gx, ldx, C,
-                           gtree, ldt, in_x ? p->tree_offset(Lc) : 0, in_x);
+                           gtree, ldt, in_x ? p->tree_offset(Lc) : 0, in_x, cpt);
     }
     APRNET_LAUNCH_CHECK("fill_tree_bwd_level_kernel");
     return 0;
@@ -400,9 +494,10 @@ int maxpool_fwd(const aprnet_plan* p, int d, const T* x, int64_t ldx, int C, T* 
     if (Lc - 1 < p->tree.level_min) return fail(APRNET_ERR_LEVEL_DELTA, "maxpool_forward: nothing left to pool");
     const int64_t n_out = p->number_parts(d + 1), n_copy = p->apr.level_end(Lc - 1);
     if (C <= 0 || n_out <= 0) return 0;
-    dim3 grid((unsigned)((n_out + TB - 1) / TB), (unsigned)((C + CPT - 1) / CPT));
+    const int cpt = channels_per_thread(n_out, C, sizeof(T));
+    dim3 grid((unsigned)((n_out + TB - 1) / TB), (unsigned)((C + cpt - 1) / cpt));
     hipLaunchKernelGGL(maxpool_fwd_kernel<T>, grid, dim3(TB), 0, st, p->d_children, p->n_tree, n_copy, n_out,
-                       p->tree.level_begin(Lc - 1), x, ldx, C, y, ldy, arg, ldi, p->tree_offset(Lc));
+                       p->tree.level_begin(Lc - 1), x, ldx, C, y, ldy, arg, ldi, p->tree_offset(Lc), cpt);
     APRNET_LAUNCH_CHECK("maxpool_fwd_kernel");
     return 0;
 }
@@ -415,9 +510,10 @@ int maxpool_bwd(const aprnet_plan* p, int d, const T* gy, int64_t ldy, int C, T*
     if (Lc - 1 < p->tree.level_min) return fail(APRNET_ERR_LEVEL_DELTA, "maxpool_backward: invalid level delta");
     const int64_t n_out = p->number_parts(d + 1), n_copy = p->apr.level_end(Lc - 1);
     if (C <= 0 || n_out <= 0) return 0;
-    dim3 grid((unsigned)((n_out + TB - 1) / TB), (unsigned)((C + CPT - 1) / CPT));
+    const int cpt = channels_per_thread(n_out, C, sizeof(T));
+    dim3 grid((unsigned)((n_out + TB - 1) / TB), (unsigned)((C + cpt - 1) / cpt));
     hipLaunchKernelGGL(maxpool_bwd_kernel<T>, grid, dim3(TB), 0, st, p->d_children, p->n_tree, n_copy, n_out,
-                       p->tree.level_begin(Lc - 1), gy, ldy, C, gx, ldx, arg, ldi, p->tree_offset(Lc));
+                       p->tree.level_begin(Lc - 1), gy, ldy, C, gx, ldx, arg, ldi, p->tree_offset(Lc), cpt);
     APRNET_LAUNCH_CHECK("maxpool_bwd_kernel");
     return 0;
 }
@@ -431,10 +527,11 @@ int upsample(const aprnet_plan* p, int d, const T* src, int64_t lds, int C, T* d
     const int Lc = p->lc(d);
     const int64_t n_in = p->number_parts(d), n_copy = p->apr.level_end(Lc);
     if (C <= 0 || n_in <= 0) return 0;
-    dim3 grid((unsigned)((n_in + TB - 1) / TB), (unsigned)((C + CPT - 1) / CPT));
-    hipLaunchKernelGGL((upsample_kernel<T, Backward>), grid, dim3(TB), 0, st, p->d_children, p->n_tree, n_copy, n_in,
-                       p->tree.level_begin(Lc), src, lds, C, dst, ldd, p->tree_offset(Lc + 1));
-    APRNET_LAUNCH_CHECK("upsample_kernel");
+    const int cpt = channels_per_thread(n_in, C, sizeof(T));
+    dim3 grid((unsigned)((n_in + TB - 1) / TB), (unsigned)((C + cpt - 1) / cpt));
+    hipLaunchKernelGGL((Backward ? upsample_bwd_kernel<T> : upsample_fwd_kernel<T>), grid, dim3(TB), 0, st, p->d_children, p->n_tree, n_copy, n_in,
+                       p->tree.level_begin(Lc), src, lds, C, dst, ldd, p->tree_offset(Lc + 1), cpt);
+    APRNET_LAUNCH_CHECK("upsample kernel");
     return 0;
 }
 

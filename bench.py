@@ -267,22 +267,21 @@ def run_blobs512(args, dev, lib):
     out["roofline"] = mfma_roofline(flop_pp * n, kernel_ms, PEAK_BF16_MATRIX_TFLOPS if bf16 else PEAK_FP32_MATRIX_TFLOPS,
                                     "conv_mfma_bf16_kernel" if bf16 else "conv_mfma16_kernel",
                                     (e * (CIN + COUT) + 2) * n, None if bf16 else PROFILED_TRAFFIC_BYTES.get(n))
-    if args.no_extra:                      # profiler runs: the convolution step only
-        return out
-    # second half of the metric: forward latency of the 4-level network (16-32-64-128, norms folded) on this APR
-    net = make_unet(dev)
-    xin = x[:, :1].float().contiguous()
-    extra = {"n_particles": n}
-    with torch.no_grad():
-        extra["apr_unet_fwd_ms_f32"] = _time(lambda: net(xin, [apr]), iters=5, warmup=2)
-        xinb = xin.to(torch.bfloat16)
-        extra["apr_unet_fwd_ms_bf16"] = _time(lambda: net(xinb, [apr]), iters=5, warmup=2)
-        # the narrow first layer of the network (1 -> 16 with bias and ReLU folded in): bound by HBM, 68 bytes per particle
-        first = net.encoder[0].blocks[0].conv
-        k1 = _kernel_ms(lib, lambda: first.forward_fused(xin, [apr], ld, relu=True), 5)
-        extra["conv333_1to16_kernel_ms"] = k1
-        extra["conv333_1to16_hbm_frac"] = 68 * n / (k1 * 1e-3) / 1e9 / PEAK_HBM_GBS
-    out["extra"] = extra
+    if not args.no_extra:                  # (profiler runs pass --no-extra: the convolution step only)
+        # second half of the metric: forward latency of the 4-level network (16-32-64-128, norms folded) on this APR
+        net = make_unet(dev)
+        xin = x[:, :1].float().contiguous()
+        extra = {"n_particles": n}
+        with torch.no_grad():
+            extra["apr_unet_fwd_ms_f32"] = _time(lambda: net(xin, [apr]), iters=5, warmup=2)
+            xinb = xin.to(torch.bfloat16)
+            extra["apr_unet_fwd_ms_bf16"] = _time(lambda: net(xinb, [apr]), iters=5, warmup=2)
+            # the narrow first layer of the network (1 -> 16 with bias and ReLU folded in): bound by HBM, 68 bytes per particle
+            first = net.encoder[0].blocks[0].conv
+            k1 = _kernel_ms(lib, lambda: first.forward_fused(xin, [apr], ld, relu=True), 5)
+            extra["conv333_1to16_kernel_ms"] = k1
+            extra["conv333_1to16_hbm_frac"] = 68 * n / (k1 * 1e-3) / 1e9 / PEAK_HBM_GBS
+        out["extra"] = extra
     if args.calibrate_copy:
         torch.empty_like(x).copy_(x)
         torch.cuda.synchronize()
@@ -290,6 +289,9 @@ def run_blobs512(args, dev, lib):
               file=sys.stderr, flush=True)
     if args.chain:
         print(json.dumps(chain_step(apr, x.float(), dev)), file=sys.stderr, flush=True)
+    if args.ops or args.ops_mem:
+        for line in memory_ops(apr, x.float() if bf16 else x, dev):
+            print(json.dumps(line), file=sys.stderr, flush=True)
     if args.ops:
         for line in other_ops(apr, x.float() if bf16 else x, dev):
             print(json.dumps(line), file=sys.stderr, flush=True)
@@ -526,13 +528,12 @@ def run_spots16k(args, dev, lib):
     return out
 
 
-def other_ops(apr, x, dev):
-    """Memory-bound operators at 32 channels on the same APR, priced against the HBM roofline with their
-    algorithmic bytes, the backward pass of the convolution, and the 4-level APR-UNet forward."""
+def memory_ops(apr, x, dev):
+    """Memory-bound operators at 32 channels on the benchmark APR, priced with their algorithmic bytes against the HBM
+    peak (hbm_frac), a device-to-device copy of the same tensor (copy_frac) and the best streaming rate measured
+    here (stream_frac).  fp32 channel planes, bfloat16 channel planes, and bfloat16 grouped by eight channels."""
     import torch
-    from pyapr import aprnet
-    from pyapr.aprnet import _ops
-    from apr_models.unet import APRUNet, fold_norms
+    from pyapr.aprnet import _ops, grouped
     C, e = x.shape[1], 4
     ld0, ld1 = torch.zeros(1, dtype=torch.int32), torch.ones(1, dtype=torch.int32)
     n0, n1 = _ops.number_particles(apr, 0), _ops.number_particles(apr, 1)
@@ -546,6 +547,12 @@ def other_ops(apr, x, dev):
     copy_gbs = 2 * x.numel() * e / ms / 1e6
     res.append({"op": "copy_d2d", "ms": ms, "algorithmic_GB": 2 * x.numel() * e / 1e9, "GBps": copy_gbs,
                 "hbm_frac": copy_gbs / PEAK_HBM_GBS, "note": "torch copy of the input features, read + write"})
+    ms = _time(lambda: dst.fill_(1.0))
+    res.append({"op": "fill", "ms": ms, "algorithmic_GB": x.numel() * e / 1e9, "GBps": x.numel() * e / ms / 1e6,
+                "hbm_frac": x.numel() * e / ms / 1e6 / PEAK_HBM_GBS, "note": "torch fill of a tensor of the same size: writes only"})
+    ms = _time(lambda: torch.sum(x, dim=2))
+    res.append({"op": "row_sum", "ms": ms, "algorithmic_GB": x.numel() * e / 1e9, "GBps": x.numel() * e / ms / 1e6,
+                "hbm_frac": x.numel() * e / ms / 1e6 / PEAK_HBM_GBS, "note": "torch sum over the particles: reads only"})
     del dst
     from apr_models.unet.particle_norm import ParticleBatchNorm
     bn = ParticleBatchNorm(C).to(dev).train()
@@ -565,6 +572,7 @@ def other_ops(apr, x, dev):
 
     line("norm_relu_fwd", ms_nf, e * 3 * C * n0, f"C={C}: one pass for the moments, one read + one write to normalise")
     line("norm_relu_bwd", ms_nb, e * 7 * C * n0, "gradient, input and output read twice (sums, then result), one write")
+    lib, plan, st = _ops._lib(), apr.plan(0), torch.cuda.current_stream().cuda_stream
     with torch.no_grad():
         pooled, idx = _ops.maxpool_forward([apr], x, ld0, 0.0)
         ms = _time(lambda: _ops.maxpool_forward([apr], x, ld0, 0.0))
@@ -576,12 +584,54 @@ def other_ops(apr, x, dev):
         ms = _time(lambda: _ops.upsample_const_backward([apr], x, ld1))
         line("upsample_bwd", ms, e * C * (n1 + n0), "sum of child gradients")
         tree = torch.empty(C, max(nt, 1), device=dev)
-        lib, plan, st = _ops._lib(), apr.plan(0), torch.cuda.current_stream().cuda_stream
         ms = _time(lambda: lib.aprnet_fill_tree_mean_f32(plan, 0, x.data_ptr(), x.shape[2], C, tree.data_ptr(), tree.shape[1], st))
         line("fill_tree_mean", ms, e * C * (n0 + 2 * nt), f"C={C}, {nt} tree nodes")
+        gxt, gtt = torch.zeros_like(x[0]), torch.randn(C, max(nt, 1), device=dev)
+        ms = _time(lambda: lib.aprnet_fill_tree_mean_bwd_f32(plan, 0, gxt.data_ptr(), gxt.shape[1], C, gtt.data_ptr(), gtt.shape[1], st))
+        line("fill_tree_mean_bwd", ms, e * C * (2 * n0 + 3 * nt), "children read and written in place, tree gradient read and written")
+        del gxt, gtt, tree
         w1 = torch.randn(1, C, C, 1, 1, 1, device=dev) * 0.1
         ms = _time(lambda: _ops.conv_forward([apr], x, w1, ld0))
         line("conv111_fwd", ms, e * 2 * C * n0, f"{C}->{C}")
+        # bfloat16 channel planes
+        xb = x.to(torch.bfloat16)
+        pooled_b, idx_b = _ops.maxpool_forward([apr], xb, ld0, 0.0)
+        ms = _time(lambda: _ops.maxpool_forward([apr], xb, ld0, 0.0))
+        line("maxpool_fwd_bf16", ms, 2 * C * n0 + (2 + 8) * C * n1, "bfloat16 planes, int64 argmax")
+        ms = _time(lambda: _ops.upsample_const_forward([apr], pooled_b, ld1))
+        line("upsample_fwd_bf16", ms, 2 * C * (n1 + n0), "bfloat16 planes")
+        ms = _time(lambda: _ops.conv_forward([apr], xb, w1, ld0))
+        line("conv111_fwd_bf16", ms, 2 * 2 * C * n0, f"{C}->{C}, bfloat16 planes")
+        del idx_b, idx
+        # bfloat16 grouped by eight channels (the layout a network keeps between its layers at inference)
+        if grouped.supported([apr], (C,)):
+            xg8 = grouped.regroup(xb)
+            ms = _time(lambda: grouped.regroup(xb))
+            line("regroup8_bf16", ms, 2 * 2 * C * n0, "channel planes -> groups of eight")
+            pg8 = grouped.maxpool_forward([apr], xg8, ld0)
+            ms = _time(lambda: grouped.maxpool_forward([apr], xg8, ld0))
+            line("maxpool_fwd_bf16g", ms, 2 * C * (n0 + n1), "values only (no argmax at inference)")
+            ms = _time(lambda: grouped.upsample_const_forward([apr], pg8, ld1))
+            line("upsample_fwd_bf16g", ms, 2 * C * (n1 + n0), "")
+            ms = _time(lambda: grouped.conv111_forward([apr], xg8, w1, ld0))
+            line("conv111_fwd_bf16g", ms, 2 * 2 * C * n0, f"{C}->{C}, grouped in and out")
+            treeg = torch.empty((C // 8) * max(nt, 1) * 8, dtype=torch.bfloat16, device=dev)
+            ms = _time(lambda: lib.aprnet_fill_tree_mean_bf16g(plan, 0, xg8.data.data_ptr(), n0, C, treeg.data_ptr(), max(nt, 1), st))
+            line("fill_tree_mean_bf16g", ms, 2 * C * (n0 + 2 * nt), "")
+    return res
+
+
+def other_ops(apr, x, dev):
+    """The backward pass of the convolution, the wide 2-D stencil, and the 4-level APR-UNet (forward, HIP graph, training
+    step) on the benchmark APR."""
+    import torch
+    from pyapr import aprnet
+    from pyapr.aprnet import _ops
+    from apr_models.unet import APRUNet, fold_norms
+    C = x.shape[1]
+    ld0 = torch.zeros(1, dtype=torch.int32)
+    n0 = _ops.number_particles(apr, 0)
+    res = []
     conv = aprnet.cuda.APRConv(C, C, nstencils=2).to(dev)
     xg = x.clone().requires_grad_(True)
     y = conv(xg, [apr], ld0)
@@ -680,8 +730,6 @@ def other_ops(apr, x, dev):
         ms = _time(lambda: conv(xb, [apr], ld0), iters=5, warmup=1)
         res.append({"op": "conv333_fwd_bf16", "ms": ms, "particles_per_s": n0 / ms * 1e3,
                     "note": f"{C}->{C}, bfloat16 features and matrix math (fp32 accumulate), whole APRConv.forward"})
-        ms = _time(lambda: _ops.maxpool_forward([apr], xb, ld0, 0.0))
-        line("maxpool_fwd_bf16", ms, 2 * C * n0 + (2 + 8) * C * n1, "bfloat16 values, int64 argmax")
         x64b = torch.randn(1, 64, x.shape[2], device=dev).to(torch.bfloat16)
         conv5b = aprnet.cuda.APRConv(64, 64, nstencils=2, kernel_size=(1, 5, 5)).to(dev)
         ms = _time(lambda: conv5b(x64b, [apr], ld0), iters=3, warmup=1)
@@ -736,6 +784,8 @@ def main():
                          "used to scale the FETCH_SIZE / WRITE_SIZE counters of a profiler run)")
     ap.add_argument("--ops", action="store_true",
                     help="blobs512: also time the memory-bound operators, the backward pass and the networks (extra JSON lines on stderr)")
+    ap.add_argument("--ops-mem", action="store_true",
+                    help="blobs512: also time the memory-bound operators only (fp32, bfloat16 planes, bfloat16 grouped by eight)")
     ap.add_argument("--chain", action="store_true",
                     help="blobs512: also time the conv -> ReLU -> pool -> upsample chain of configs[1], forward + backward (stderr)")
     args = ap.parse_args()
