@@ -41,7 +41,7 @@ def build(force=False, verbose=True):
         subprocess.check_call(cmd)
     with ThreadPoolExecutor(max_workers=min(8, max(1, len(jobs)))) as ex:
         list(ex.map(run, jobs))
-    if force or jobs or not os.path.exists("libaprnet_hip.so"):
+    if force or jobs or _newer("libaprnet_hip.so", objs):
         run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", "libaprnet_hip.so", *objs])
     if force or _newer("libaprcore.so", ["aprcore.cpp"]):
         run(["g++", "-O3", "-march=x86-64-v3", "-fopenmp", "-shared", "-fPIC", "-std=c++17", "-o", "libaprcore.so", "aprcore.cpp"])

@@ -67,13 +67,15 @@ __device__ __forceinline__ void fill_node_g8(const int32_t* children, int64_t n_
 #pragma unroll
     for (int s = 0; s < 8; ++s) { ch[s] = children[(int64_t)s * n_tree + t]; cnt += ch[s] != NO_CHILD; }
     const float scale = 1.0f / (float)max(cnt, 1);
+    // unconditional loads (a missing child reads particle 0 and is skipped below): a load under a per-lane branch
+    // makes the compiler wait for memory inside the branch, one child after the other
     uint4 raw[8];
 #pragma unroll
     for (int s = 0; s < 8; ++s) {
         const int32_t v = ch[s];
-        raw[s] = make_uint4(0u, 0u, 0u, 0u);
-        if (v >= 0) raw[s] = *g8_at(x, ldx, q, v);
-        else if (v != NO_CHILD) raw[s] = tree_child_from_x ? *g8_at(x, ldx, q, tree_off + ~v) : *g8_at((const bf16_t*)tree, ldt, q, ~v);
+        const bool from_tree = v < 0 && v != NO_CHILD && !tree_child_from_x;
+        const int64_t idx = v >= 0 ? (int64_t)v : (v == NO_CHILD ? 0 : (tree_child_from_x ? tree_off + ~v : (int64_t)~v));
+        raw[s] = *g8_at(from_tree ? (const bf16_t*)tree : x, from_tree ? ldt : ldx, q, idx);
     }
     float sum[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 #pragma unroll
@@ -156,6 +158,13 @@ maxpool_g8_kernel(const int32_t* __restrict__ children, int64_t n_tree, int64_t 
     if (i >= n_out) return;
     if (i < n_copy) { *g8_at(y, ldy, q, i) = *g8_at(x, ldx, q, i); return; }
     const int64_t t = t_begin + (i - n_copy);
+    int32_t ch[8];
+#pragma unroll
+    for (int s = 0; s < 8; ++s) ch[s] = children[(int64_t)s * n_tree + t];
+    uint4 raw[8];                         // unconditional loads, as in fill_node_g8
+#pragma unroll
+    for (int s = 0; s < 8; ++s)
+        raw[s] = *g8_at(x, ldx, q, ch[s] >= 0 ? (int64_t)ch[s] : (ch[s] == NO_CHILD ? 0 : in_tree_off + ~ch[s]));
     float best[8];
 #pragma unroll
     for (int c = 0; c < 8; ++c) best[c] = -1e17f;
@@ -163,31 +172,42 @@ maxpool_g8_kernel(const int32_t* __restrict__ children, int64_t n_tree, int64_t 
     for (int pass = 0; pass < 2; ++pass)
 #pragma unroll
         for (int s = 0; s < 8; ++s) {
-            const int32_t v = children[(int64_t)s * n_tree + t];
-            if (v == NO_CHILD || (pass == 0) != (v >= 0)) continue;
+            if (ch[s] == NO_CHILD || (pass == 0) != (ch[s] >= 0)) continue;
             float f[8];
-            unpack8(*g8_at(x, ldx, q, v >= 0 ? (int64_t)v : in_tree_off + ~v), f);
+            unpack8(raw[s], f);
 #pragma unroll
             for (int c = 0; c < 8; ++c) if (f[c] > best[c]) best[c] = f[c];
         }
     *g8_at(y, ldy, q, i) = pack8(best);
 }
 
-// upsample_kernel of tree_ops.hip, forward: a downsampled particle's value goes to each of its children
+// upsample_fwd_kernel of tree_ops.hip: a downsampled particle's value goes to each of its children.  TWO lanes per
+// parent, one for the children with even y and one for those with odd y: children 2y and 2y + 1 of a row are neighbours
+// in memory, so the lanes of a wave write whole lines (one lane per parent would fill every other 16 bytes of them).
 __global__ void __launch_bounds__(GTB)
 upsample_g8_kernel(const int32_t* __restrict__ children, int64_t n_tree, int64_t n_copy, int64_t n_in, int64_t t_begin,
-                   const bf16_t* __restrict__ src, int64_t lds, bf16_t* __restrict__ dst, int64_t ldd, int64_t out_tree_off) {
-    const int64_t i = (int64_t)blockIdx.x * GTB + threadIdx.x;
-    const int q = blockIdx.y;
-    if (i >= n_in) return;
-    const uint4 v = *g8_at(src, lds, q, i);
-    if (i < n_copy) { *g8_at(dst, ldd, q, i) = v; return; }
-    const int64_t t = t_begin + (i - n_copy);
+                   const bf16_t* __restrict__ src, int64_t lds, int G, bf16_t* __restrict__ dst, int64_t ldd, int64_t out_tree_off) {
+    const int64_t j = (int64_t)blockIdx.x * GTB + threadIdx.x;
+    const int64_t n_par = n_in - n_copy;
+    if (j < n_copy) {                     // copied positions: one lane each
+        for (int q = 0; q < G; ++q) *g8_at(dst, ldd, q, j) = *g8_at(src, lds, q, j);
+        return;
+    }
+    const int64_t k = j - n_copy;
+    if (k >= 2 * n_par) return;
+    const int64_t i = n_copy + (k >> 1), t = t_begin + (k >> 1);
+    const int dy = (int)(k & 1);
+    int64_t at[4];                        // the four children with this dy (slot = 2 * (2 dz + dx) + dy); -1: none
 #pragma unroll
-    for (int s = 0; s < 8; ++s) {
-        const int32_t c = children[(int64_t)s * n_tree + t];
-        if (c >= 0) *g8_at(dst, ldd, q, c) = v;
-        else if (c != NO_CHILD) *g8_at(dst, ldd, q, out_tree_off + ~c) = v;
+    for (int p = 0; p < 4; ++p) {
+        const int32_t c = children[(int64_t)(2 * p + dy) * n_tree + t];
+        at[p] = c >= 0 ? (int64_t)c : (c != NO_CHILD ? out_tree_off + ~c : -1);
+    }
+    for (int q = 0; q < G; ++q) {
+        const uint4 v = *g8_at(src, lds, q, i);
+#pragma unroll
+        for (int p = 0; p < 4; ++p)
+            if (at[p] >= 0) *g8_at(dst, ldd, q, at[p]) = v;
     }
 }
 
@@ -197,44 +217,71 @@ upsample_g8_kernel(const int32_t* __restrict__ children, int64_t n_tree, int64_t
 // the output group sit in LDS and are read as broadcasts.  Bound by memory for the layers it serves (channel
 // reductions of the decoder, the head).  OUT_G8: grouped output, otherwise channel planes (the head of a network).
 constexpr int C111_MAX_CIN = 256;
+constexpr int C111_OG = 4;        // output groups (of eight channels) per thread: the input is read once per 32 outputs
 
 template <bool OUT_G8>
 __global__ void __launch_bounds__(GTB)
 conv111_g8_kernel(const bf16_t* __restrict__ x, int64_t ldx, int Cin, const float* __restrict__ w, int Cout, const float* __restrict__ bias,
                   int relu, bf16_t* __restrict__ y, int64_t ldy, int64_t begin, int64_t end) {
-    __shared__ __attribute__((aligned(16))) float wl[C111_MAX_CIN * 8];        // [ci][co8]
-    const int og = blockIdx.y, nq = Cin / 8;
-    for (int e = threadIdx.x; e < Cin * 8; e += GTB) {
-        const int ci = e >> 3, co = og * 8 + (e & 7);
+    extern __shared__ __attribute__((aligned(16))) float wl[];        // [ci][8 * C111_OG]
+    constexpr int NO = 8 * C111_OG;
+    const int o0 = blockIdx.y * NO, nq = Cin / 8;
+    for (int e = threadIdx.x; e < Cin * NO; e += GTB) {
+        const int ci = e / NO, co = o0 + (e % NO);
         wl[e] = co < Cout ? w[(int64_t)co * Cin + ci] : 0.f;
     }
     __syncthreads();
     const int64_t i = begin + (int64_t)blockIdx.x * GTB + threadIdx.x;
     if (i >= end) return;
-    float acc[8];
+    float acc[NO];
 #pragma unroll
-    for (int c = 0; c < 8; ++c) acc[c] = 0.f;
-    for (int q = 0; q < nq; ++q) {
-        float f[8];
-        unpack8(*g8_at(x, ldx, q, i), f);
+    for (int c = 0; c < NO; ++c) acc[c] = 0.f;
+    // input groups four at a time: the next four loads are in flight while these are multiplied
+    uint4 cur[4], nxt[4];
 #pragma unroll
-        for (int k = 0; k < 8; ++k) {
-            const float4 w0 = *reinterpret_cast<const float4*>(wl + (q * 8 + k) * 8), w1 = *reinterpret_cast<const float4*>(wl + (q * 8 + k) * 8 + 4);
-            acc[0] += w0.x * f[k]; acc[1] += w0.y * f[k]; acc[2] += w0.z * f[k]; acc[3] += w0.w * f[k];
-            acc[4] += w1.x * f[k]; acc[5] += w1.y * f[k]; acc[6] += w1.z * f[k]; acc[7] += w1.w * f[k];
+    for (int k = 0; k < 4; ++k) cur[k] = *g8_at(x, ldx, min(k, nq - 1), i);
+    for (int q0 = 0; q0 < nq; q0 += 4) {
+        if (q0 + 4 < nq) {
+#pragma unroll
+            for (int k = 0; k < 4; ++k) nxt[k] = *g8_at(x, ldx, min(q0 + 4 + k, nq - 1), i);
         }
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            if (q0 + k >= nq) break;
+            float f[8];
+            unpack8(cur[k], f);
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                const float* wr = wl + ((q0 + k) * 8 + j) * NO;
+#pragma unroll
+                for (int c4 = 0; c4 < NO; c4 += 4) {
+                    const float4 w4 = *reinterpret_cast<const float4*>(wr + c4);
+                    acc[c4] += w4.x * f[j]; acc[c4 + 1] += w4.y * f[j]; acc[c4 + 2] += w4.z * f[j]; acc[c4 + 3] += w4.w * f[j];
+                }
+            }
+        }
+#pragma unroll
+        for (int k = 0; k < 4; ++k) cur[k] = nxt[k];
     }
 #pragma unroll
-    for (int c = 0; c < 8; ++c) {
-        const int co = og * 8 + c;
+    for (int c = 0; c < NO; ++c) {
+        const int co = o0 + c;
         if (bias && co < Cout) acc[c] += bias[co];
         if (relu) acc[c] = acc[c] < 0.f ? 0.f : acc[c];
     }
-    if constexpr (OUT_G8) *g8_at(y, ldy, og, i) = pack8(acc);
-    else {
 #pragma unroll
-        for (int c = 0; c < 8; ++c)
-            if (og * 8 + c < Cout) y[(int64_t)(og * 8 + c) * ldy + i] = float_to_bf16(acc[c]);
+    for (int g = 0; g < C111_OG; ++g) {
+        if (o0 + 8 * g >= Cout) break;
+        if constexpr (OUT_G8) {
+            float a8[8];
+#pragma unroll
+            for (int c = 0; c < 8; ++c) a8[c] = acc[8 * g + c];
+            *g8_at(y, ldy, blockIdx.y * C111_OG + g, i) = pack8(a8);
+        } else {
+#pragma unroll
+            for (int c = 0; c < 8; ++c)
+                if (o0 + 8 * g + c < Cout) y[(int64_t)(o0 + 8 * g + c) * ldy + i] = float_to_bf16(acc[8 * g + c]);
+        }
     }
 }
 
@@ -288,8 +335,9 @@ int aprnet_upsample_fwd_bf16g(const aprnet_plan* p, int d, const uint16_t* x, in
     if (C <= 0 || n_in <= 0) return 0;
     if (ldx < n_in || ldy < p->number_parts(d - 1)) return fail(APRNET_ERR_INVALID_ARGUMENT, "upsample_const_forward: row shorter than the particle count");
     APRNET_HIP_CHECK(hipSetDevice(p->device));
-    hipLaunchKernelGGL(upsample_g8_kernel, dim3((unsigned)((n_in + GTB - 1) / GTB), (unsigned)(C / 8)), dim3(GTB), 0, (hipStream_t)st,
-                       p->d_children, p->n_tree, n_copy, n_in, p->tree.level_begin(Lc), (const bf16_t*)x, ldx, (bf16_t*)y, ldy,
+    const int64_t n_thr = n_copy + 2 * (n_in - n_copy);
+    hipLaunchKernelGGL(upsample_g8_kernel, dim3((unsigned)((n_thr + GTB - 1) / GTB)), dim3(GTB), 0, (hipStream_t)st,
+                       p->d_children, p->n_tree, n_copy, n_in, p->tree.level_begin(Lc), (const bf16_t*)x, ldx, C / 8, (bf16_t*)y, ldy,
                        p->tree_offset(Lc + 1));
     APRNET_LAUNCH_CHECK("upsample_g8_kernel");
     return 0;
@@ -310,10 +358,11 @@ int aprnet_conv111_fwd_bf16g(const aprnet_plan* p, int d, const uint16_t* x, int
         int64_t b = p->apr.level_begin(std::max(l_lo, p->apr.level_min)), e = p->apr.level_end(l_hi);
         if (s == 0) e = p->number_parts(d);
         if (e <= b) continue;
-        dim3 grid((unsigned)((e - b + GTB - 1) / GTB), (unsigned)((Cout + 7) / 8));
+        dim3 grid((unsigned)((e - b + GTB - 1) / GTB), (unsigned)((Cout + 8 * C111_OG - 1) / (8 * C111_OG)));
+        const size_t lds = (size_t)Cin * 8 * C111_OG * sizeof(float);
         const float* ws = w + (int64_t)s * Cout * Cin;
-        if (y_grouped) hipLaunchKernelGGL(conv111_g8_kernel<true>, grid, dim3(GTB), 0, (hipStream_t)st, (const bf16_t*)x, ldx, Cin, ws, Cout, bias, relu, (bf16_t*)y, ldy, b, e);
-        else hipLaunchKernelGGL(conv111_g8_kernel<false>, grid, dim3(GTB), 0, (hipStream_t)st, (const bf16_t*)x, ldx, Cin, ws, Cout, bias, relu, (bf16_t*)y, ldy, b, e);
+        if (y_grouped) hipLaunchKernelGGL(conv111_g8_kernel<true>, grid, dim3(GTB), lds, (hipStream_t)st, (const bf16_t*)x, ldx, Cin, ws, Cout, bias, relu, (bf16_t*)y, ldy, b, e);
+        else hipLaunchKernelGGL(conv111_g8_kernel<false>, grid, dim3(GTB), lds, (hipStream_t)st, (const bf16_t*)x, ldx, Cin, ws, Cout, bias, relu, (bf16_t*)y, ldy, b, e);
     }
     APRNET_LAUNCH_CHECK("conv111_g8_kernel");
     return 0;

@@ -219,7 +219,7 @@ def run_blobs512(args, dev, lib):
     """configs[1]: the 32 -> 32 layer (headline metric) and the APR-UNet forward latency on the same APR."""
     import torch
     from pyapr import aprnet
-    CIN = COUT = 32
+    CIN, COUT = args.channels
     flop_pp, bytes_pp = 2 * 27 * CIN * COUT, 4 * (CIN + COUT) + 2
     nstencils = 2
     t0 = time.perf_counter()
@@ -256,9 +256,12 @@ def run_blobs512(args, dev, lib):
     assert torch.isfinite(y.float()).all()
     del y
     e = 2 if bf16 else 4
-    out = base_line("APRConv 3x3x3 fwd particles/s (Cin=Cout=32) + APR-UNet fwd latency, 1 GPU", n / sec, "particles/s", args,
+    metric = "APRConv 3x3x3 fwd particles/s (Cin=Cout=32) + APR-UNet fwd latency, 1 GPU"
+    if (CIN, COUT) != (32, 32):
+        metric = f"APRConv 3x3x3 fwd particles/s (Cin={CIN}, Cout={COUT})"
+    out = base_line(metric, n / sec, "particles/s", args,
                     sec * 1e3, "bf16" if bf16 else "f32",
-                    {"workload": f"APRConv 3x3x3 32->32 {'bf16' if bf16 else 'fp32'} forward (restrict + tree fill + conv + bias"
+                    {"workload": f"APRConv 3x3x3 {CIN}->{COUT} {'bf16' if bf16 else 'fp32'} forward (restrict + tree fill + conv + bias"
                                  f"{', input and output grouped by eight channels' if args.features == 'bf16g' else ''}), batch 1, "
                                  "APR of the seeded 512x512x256 volume with 2000 ellipsoidal blobs (configs[1]); extra: 4-level "
                                  "APR-UNet forward on the same APR",
@@ -784,6 +787,8 @@ def main():
                          "used to scale the FETCH_SIZE / WRITE_SIZE counters of a profiler run)")
     ap.add_argument("--ops", action="store_true",
                     help="blobs512: also time the memory-bound operators, the backward pass and the networks (extra JSON lines on stderr)")
+    ap.add_argument("--channels", type=int, nargs=2, default=[32, 32], metavar=("CIN", "COUT"),
+                    help="blobs512: channel counts of the timed layer (default 32 32, the layer the metric is quoted on)")
     ap.add_argument("--ops-mem", action="store_true",
                     help="blobs512: also time the memory-bound operators only (fp32, bfloat16 planes, bfloat16 grouped by eight)")
     ap.add_argument("--chain", action="store_true",
