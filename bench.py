@@ -248,6 +248,29 @@ def run_blobs512(args, dev, lib):
     else:
         def step():
             return conv(x, [apr], ld)
+    e = 2 if bf16 else 4
+    if args.backward:
+        # the backward pass of the same layer (input and weight gradient) as the timed step: the call a profiler run traces
+        if args.features == "bf16g":
+            sys.exit("bench.py: --backward runs on channel planes (--features f32 or bf16)")
+        xg = x.clone().requires_grad_(True)
+        yb = conv(xg, [apr], ld)
+        go = torch.randn_like(yb)
+
+        def bstep():
+            return torch.autograd.grad(yb, (xg, conv.weight, conv.bias), go, retain_graph=True)
+        sec = _steps(bstep, args.steps, args.warmup)
+        out = base_line(f"APRConv 3x3x3 bwd particles/s (Cin={CIN}, Cout={COUT})", n / sec, "particles/s", args, sec * 1e3,
+                        "bf16" if bf16 else "f32",
+                        {"workload": f"APRConv 3x3x3 {CIN}->{COUT} {'bf16' if bf16 else 'fp32'} backward (input, weight and bias gradient, "
+                                     "tree-fill and restriction backward), batch 1, blobs512 APR", "n_particles": n})
+        out["roofline"] = mfma_roofline(2 * flop_pp * n, sec * 1e3, PEAK_BF16_MATRIX_TFLOPS if bf16 else PEAK_FP32_MATRIX_TFLOPS,
+                                        "whole backward call (input-gradient and weight-gradient kernels on two streams)",
+                                        (e * 2 * (CIN + COUT)) * n)
+        if args.calibrate_copy:
+            torch.empty_like(x).copy_(x)
+            torch.cuda.synchronize()
+        return out
     with torch.no_grad():
         sec = _steps(step, args.steps, args.warmup)
         kernel_ms = _kernel_ms(lib, step, args.steps)
@@ -255,7 +278,6 @@ def run_blobs512(args, dev, lib):
     y = y.data if args.features == "bf16g" else y
     assert torch.isfinite(y.float()).all()
     del y
-    e = 2 if bf16 else 4
     metric = "APRConv 3x3x3 fwd particles/s (Cin=Cout=32) + APR-UNet fwd latency, 1 GPU"
     if (CIN, COUT) != (32, 32):
         metric = f"APRConv 3x3x3 fwd particles/s (Cin={CIN}, Cout={COUT})"
@@ -267,9 +289,13 @@ def run_blobs512(args, dev, lib):
                                  "APR-UNet forward on the same APR",
                      "n_particles": n, "levels": level_counts(apr), "nstencils": nstencils, "level_max": apr.level_max(),
                      "apr_build_s": round(t_build, 2), "plan_create_s": round(t_plan, 2)})
-    out["roofline"] = mfma_roofline(flop_pp * n, kernel_ms, PEAK_BF16_MATRIX_TFLOPS if bf16 else PEAK_FP32_MATRIX_TFLOPS,
-                                    "conv_mfma_bf16_kernel" if bf16 else "conv_mfma16_kernel",
-                                    (e * (CIN + COUT) + 2) * n, None if bf16 else PROFILED_TRAFFIC_BYTES.get(n))
+    peak = PEAK_BF16_MATRIX_TFLOPS if bf16 else PEAK_FP32_MATRIX_TFLOPS
+    alg_bytes = (e * (CIN + COUT) + 2) * n
+    if flop_pp / (e * (CIN + COUT) + 2) < peak * 1e12 / (PEAK_HBM_GBS * 1e9):      # fewer flops per byte than the machine: HBM bounds it
+        out["roofline"] = hbm_roofline(alg_bytes, kernel_ms, "conv_narrow_kernel" if CIN <= 3 else "conv kernel", flop_pp * n)
+    else:
+        out["roofline"] = mfma_roofline(flop_pp * n, kernel_ms, peak, "conv_mfma_bf16_kernel" if bf16 else "conv_mfma16_kernel",
+                                        alg_bytes, None if bf16 or (CIN, COUT) != (32, 32) else PROFILED_TRAFFIC_BYTES.get(n))
     if not args.no_extra:                  # (profiler runs pass --no-extra: the convolution step only)
         # second half of the metric: forward latency of the 4-level network (16-32-64-128, norms folded) on this APR
         net = make_unet(dev)
@@ -789,6 +815,8 @@ def main():
                     help="blobs512: also time the memory-bound operators, the backward pass and the networks (extra JSON lines on stderr)")
     ap.add_argument("--channels", type=int, nargs=2, default=[32, 32], metavar=("CIN", "COUT"),
                     help="blobs512: channel counts of the timed layer (default 32 32, the layer the metric is quoted on)")
+    ap.add_argument("--backward", action="store_true",
+                    help="blobs512: time the backward pass of the layer instead of the forward pass")
     ap.add_argument("--ops-mem", action="store_true",
                     help="blobs512: also time the memory-bound operators only (fp32, bfloat16 planes, bfloat16 grouped by eight)")
     ap.add_argument("--chain", action="store_true",
