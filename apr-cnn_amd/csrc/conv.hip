@@ -10,6 +10,8 @@
 // channel is formed first and then added to the running output (helpers.hpp:537-544).
 #include "conv_common.hpp"
 
+#include <atomic>
+
 namespace aprnet {
 
 template <typename T, class G, int CIB, int COB>
@@ -139,8 +141,8 @@ size_t conv_packed_bf16_bytes(int code, int S_exp, int Cout, int Cin);
 int pack_conv_weights_bf16(int code, const float* w, int S_exp, int Cout, int Cin, void* packed, hipStream_t st, bool transposed = false);
 int interleave8_bf16(const bf16_t* x, int64_t ldx, const bf16_t* x2, int64_t ldx2, int c_split, int C, int64_t count, bf16_t* out,
                      hipStream_t st);
-static int g_bf16_math = 1;      // bfloat16 features: 1 = bfloat16 matrix instructions, 0 = fp32 matrix instructions
-static int g_bf16_regroup = 1;   // bfloat16 forward: 1 = stage from a copy of the input regrouped by 8 channels, 0 = from the channel planes
+static std::atomic<int> g_bf16_math{1};      // bfloat16 features: 1 = bfloat16 matrix instructions, 0 = fp32 matrix instructions
+static std::atomic<int> g_bf16_regroup{1};   // bfloat16 forward: 1 = stage from a copy of the input regrouped by 8 channels, 0 = from the channel planes
 int fill_tree_for_conv(const aprnet_plan* p, int d, const bf16_t* x, int64_t ldx, int C, bf16_t* tree, int64_t ldt, hipStream_t st);
 size_t conv_packed_floats(int code, int S_exp, int Cm, int Ck, bool transposed);
 int pack_conv_weights(int code, const float* w, int S_exp, int Cm, int Ck, bool transposed, float* packed, hipStream_t st);
@@ -150,18 +152,18 @@ size_t conv_narrow_packed_floats(int code, int S_exp, int Cout, int Cin);
 int pack_conv_weights_narrow(int code, const float* w, int S_exp, int Cout, int Cin, float* packed, hipStream_t st);
 int launch_conv_narrow(int code, const ConvArgs<float>& a, const WinLists& wl, hipStream_t st);
 int launch_conv_narrow(int code, const ConvArgs<bf16_t>& a, const WinLists& wl, hipStream_t st);
-static int g_narrow = 1;         // layers of 1 to 3 input channels: 1 = the bandwidth-shaped kernel (conv_narrow.hip), 0 = the general one
-static int g_conv_path = 0;      // 0: matrix cores where available, 1: VALU kernels only
+static std::atomic<int> g_narrow{1};         // layers of 1 to 3 input channels: 1 = the bandwidth-shaped kernel (conv_narrow.hip), 0 = the general one
+static std::atomic<int> g_conv_path{0};      // 0: matrix cores where available, 1: VALU kernels only
 int conv_path() { return g_conv_path; }
 int bf16_math();
 int bf16_regroup();
 
-static int g_use_lists = 1;      // 1: forward kernels take the window lists of the plan, 0: they scan per call
+static std::atomic<int> g_use_lists{1};      // 1: forward kernels take the window lists of the plan, 0: they scan per call
 int bf16_math() { return g_bf16_math; }
 int bf16_regroup() { return g_bf16_regroup; }
-static int g_bwd_overlap = 1;    // backward: weight gradient on a second stream next to the input gradient
+static std::atomic<int> g_bwd_overlap{1};    // backward: weight gradient on a second stream next to the input gradient
 int backward_overlap() { return g_bwd_overlap; }
-static int g_bwd_deterministic = 1;   // backward: weight gradient summed in a fixed order (partial sums per workgroup) instead of atomics
+static std::atomic<int> g_bwd_deterministic{1};   // backward: weight gradient summed in a fixed order (partial sums per workgroup) instead of atomics
 int bwd_deterministic() { return g_bwd_deterministic; }
 
 // Points the kernel at the plan's window lists.  When the lists are switched off, or cannot be built (no device

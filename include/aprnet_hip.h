@@ -88,7 +88,10 @@ int aprnet_plan_children(const aprnet_plan* plan, int32_t* out_host);
  * the call's stream; aprnet_profile_last_ms() waits for the last bracket and returns its duration in
  * milliseconds (-1 if none).  Process-wide, not thread-safe; meant for benchmarks. */
 int aprnet_profile_enable(int on);
-/* No counterpart in the reference.  Selects the convolution kernels: 0 = matrix-core (MFMA) kernels where one
+/* No counterpart in the reference.  A knob for TESTS AND MEASUREMENTS, not part of the operator interface: it selects
+ * between kernels that compute the same results, process-wide (atomic flags; a call in flight keeps the choice it read),
+ * so that tests can cover every kernel family and benchmarks can compare them.  Callers of the operators never need it.
+ * Selects the convolution kernels: 0 = matrix-core (MFMA) kernels where one
  * exists for the stencil and element type, VALU kernels otherwise (default); 1 = VALU kernels only.
  * Independently, for bfloat16 features: 2 = bfloat16 matrix instructions (default), 3 = fp32 matrix
  * instructions; and for the forward matrix-core kernels: 4 = take the window lists that the plan builds on first
