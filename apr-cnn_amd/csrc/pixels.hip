@@ -22,20 +22,21 @@ pixel_kernel(const AccessDev acc, int level, int Lc, int64_t idx_off, T* __restr
     const int z0 = z * f, z1 = min(z0 + f, zn), x0 = x * f, x1 = min(x0 + f, xn);
     for (int64_t i = b + threadIdx.x; i < e; i += 64) {
         const int y0 = (int)acc.y[i] * f, y1 = min(y0 + f, yn);
+        typedef typename Num<T>::acc A;     // bfloat16 cells are summed and divided in fp32
         for (int c = 0; c < C; ++c) {
             T* pv = parts + (int64_t)c * ldp + i + idx_off;
             T* im = img + (int64_t)c * ldi;
             if (MODE == RECON_FWD || MODE == SAMPLE_BWD) {
-                const T v = MODE == RECON_FWD ? *pv : *pv / (T)((z1 - z0) * (x1 - x0) * (y1 - y0));
+                const T v = MODE == RECON_FWD ? *pv : Num<T>::st(Num<T>::ld(*pv) / (A)((z1 - z0) * (x1 - x0) * (y1 - y0)));
                 for (int zz = z0; zz < z1; ++zz)
                     for (int xx = x0; xx < x1; ++xx)
                         for (int yy = y0; yy < y1; ++yy) im[((int64_t)zz * xn + xx) * yn + yy] = v;
             } else {
-                T s = 0;
+                A s = 0;
                 for (int zz = z0; zz < z1; ++zz)
                     for (int xx = x0; xx < x1; ++xx)
-                        for (int yy = y0; yy < y1; ++yy) s += im[((int64_t)zz * xn + xx) * yn + yy];
-                *pv = MODE == RECON_BWD ? s : s / (T)((z1 - z0) * (x1 - x0) * (y1 - y0));
+                        for (int yy = y0; yy < y1; ++yy) s += Num<T>::ld(im[((int64_t)zz * xn + xx) * yn + yy]);
+                *pv = Num<T>::st(MODE == RECON_BWD ? s : s / (A)((z1 - z0) * (x1 - x0) * (y1 - y0)));
             }
         }
     }
@@ -75,4 +76,13 @@ extern "C" {
                                           void* st) { return pixel_op<T, SAMPLE_BWD>(p, d, const_cast<T*>(gy), ldy, C, gimg, ldi, (hipStream_t)st); }
 PIXEL_API(float, f32)
 PIXEL_API(double, f64)
+// bfloat16 images and particles (bit patterns in uint16_t): sums and means in fp32, rounded to nearest even on store
+int aprnet_reconstruct_fwd_bf16(const aprnet_plan* p, int d, const uint16_t* x, int64_t ldx, int C, uint16_t* img, int64_t ldi, void* st) {
+    return pixel_op<bf16_t, RECON_FWD>(p, d, (bf16_t*)const_cast<uint16_t*>(x), ldx, C, (bf16_t*)img, ldi, (hipStream_t)st); }
+int aprnet_reconstruct_bwd_bf16(const aprnet_plan* p, int d, const uint16_t* gimg, int64_t ldi, int C, uint16_t* gx, int64_t ldx, void* st) {
+    return pixel_op<bf16_t, RECON_BWD>(p, d, (bf16_t*)gx, ldx, C, (bf16_t*)const_cast<uint16_t*>(gimg), ldi, (hipStream_t)st); }
+int aprnet_sample_particles_fwd_bf16(const aprnet_plan* p, int d, const uint16_t* img, int64_t ldi, int C, uint16_t* y, int64_t ldy, void* st) {
+    return pixel_op<bf16_t, SAMPLE_FWD>(p, d, (bf16_t*)y, ldy, C, (bf16_t*)const_cast<uint16_t*>(img), ldi, (hipStream_t)st); }
+int aprnet_sample_particles_bwd_bf16(const aprnet_plan* p, int d, const uint16_t* gy, int64_t ldy, int C, uint16_t* gimg, int64_t ldi, void* st) {
+    return pixel_op<bf16_t, SAMPLE_BWD>(p, d, (bf16_t*)const_cast<uint16_t*>(gy), ldy, C, (bf16_t*)gimg, ldi, (hipStream_t)st); }
 }

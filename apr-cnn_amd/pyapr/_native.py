@@ -126,6 +126,8 @@ def hip():
     lib.aprnet_maxpool_bwd_bf16.argtypes = [vp, i32, vp, i64, i32, vp, i64, vp, i64, vp]
     lib.aprnet_upsample_fwd_bf16.argtypes = [vp, i32, vp, i64, i32, vp, i64, vp]
     lib.aprnet_upsample_bwd_bf16.argtypes = [vp, i32, vp, i64, i32, vp, i64, vp]
+    for op in ("reconstruct_fwd", "reconstruct_bwd", "sample_particles_fwd", "sample_particles_bwd"):
+        getattr(lib, f"aprnet_{op}_bf16").argtypes = [vp, i32, vp, i64, i32, vp, i64, vp]
     lib.aprnet_channel_sum_work_elems.argtypes = [i32]
     lib.aprnet_channel_sum_static_f32.argtypes = [vp, i64, i32, i64, vp, i32, vp]
     lib.aprnet_channel_sum_bf16.argtypes = [vp, i64, i32, i64, vp, i32, vp, vp]

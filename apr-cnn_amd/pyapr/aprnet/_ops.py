@@ -546,7 +546,7 @@ def reconstruct_forward(aprs, x, level_delta):
     out = torch.zeros((B, Cn, *shape), dtype=x.dtype, device=x.device)
     plane = shape[0] * shape[1] * shape[2]
     plans = _plans(aprs, x.device)
-    fn = getattr(_lib(), "aprnet_reconstruct_fwd_" + _sfx(x))
+    fn = getattr(_lib(), "aprnet_reconstruct_fwd_" + _sfx(x, bf16=True))
     with torch.cuda.device(x.device):
         st = _stream()
         for b in range(B):
@@ -567,7 +567,7 @@ def reconstruct_backward(aprs, grad_output, level_delta):
     _zero_tails(gx, sizes)
     plane = grad_output[0, 0].numel()
     plans = _plans(aprs, grad_output.device)
-    fn = getattr(_lib(), "aprnet_reconstruct_bwd_" + _sfx(grad_output))
+    fn = getattr(_lib(), "aprnet_reconstruct_bwd_" + _sfx(grad_output, bf16=True))
     with torch.cuda.device(grad_output.device):
         st = _stream()
         for b in range(B):
@@ -589,7 +589,7 @@ def sample_particles_forward(aprs, img, level_delta):
     _zero_tails(out, sizes)
     plane = img[0, 0].numel()
     plans = _plans(aprs, img.device)
-    fn = getattr(_lib(), "aprnet_sample_particles_fwd_" + _sfx(img))
+    fn = getattr(_lib(), "aprnet_sample_particles_fwd_" + _sfx(img, bf16=True))
     with torch.cuda.device(img.device):
         st = _stream()
         for b in range(B):
@@ -608,7 +608,7 @@ def sample_particles_backward(aprs, grad_output, level_delta):
     gimg = torch.zeros((B, Cn, *shape), dtype=grad_output.dtype, device=grad_output.device)
     plane = shape[0] * shape[1] * shape[2]
     plans = _plans(aprs, grad_output.device)
-    fn = getattr(_lib(), "aprnet_sample_particles_bwd_" + _sfx(grad_output))
+    fn = getattr(_lib(), "aprnet_sample_particles_bwd_" + _sfx(grad_output, bf16=True))
     with torch.cuda.device(grad_output.device):
         st = _stream()
         for b in range(B):

@@ -240,6 +240,16 @@ int aprnet_maxpool_bwd_bf16(const aprnet_plan*, int level_delta, const uint16_t*
                             int64_t ldx, const int64_t* argmax, int64_t ldi, void* stream);
 int aprnet_upsample_fwd_bf16(const aprnet_plan*, int level_delta, const uint16_t* x, int64_t ldx, int C, uint16_t* y,
                              int64_t ldy, void* stream);
+/* reconstruct / sample_particles with bfloat16 particles and images (cuda/src/reconstruct_gpu.cu:3-127,
+ * sample_particles_gpu.cu:3-246; the reference has no 16-bit path): cell sums and means in fp32. */
+int aprnet_reconstruct_fwd_bf16(const aprnet_plan*, int level_delta, const uint16_t* x, int64_t ldx, int C, uint16_t* img,
+                                int64_t ld_img, void* stream);
+int aprnet_reconstruct_bwd_bf16(const aprnet_plan*, int level_delta, const uint16_t* grad_img, int64_t ld_img, int C, uint16_t* grad_x,
+                                int64_t ldx, void* stream);
+int aprnet_sample_particles_fwd_bf16(const aprnet_plan*, int level_delta, const uint16_t* img, int64_t ld_img, int C, uint16_t* y,
+                                     int64_t ldy, void* stream);
+int aprnet_sample_particles_bwd_bf16(const aprnet_plan*, int level_delta, const uint16_t* grad_y, int64_t ldy, int C, uint16_t* grad_img,
+                                     int64_t ld_img, void* stream);
 /* Backward of the stencil convolution with bfloat16 features and output gradient: fp32 weights, fp32 weight
  * gradient (accumulated into gw), fp32 accumulation everywhere; the input gradient is collected in the fp32 work
  * space gx32_ws [Cin][ld_gx32] (ld_gx32 >= aprnet_number_parts) and rounded to bfloat16 into gx at the end.

@@ -424,6 +424,25 @@ def close_bf16(got, ref):
     assert err <= 1e-2 * scale, f"max abs err {err:.3e} vs scale {scale:.3e}"
 
 
+@pytest.mark.parametrize("bt", [[("3d_a", 0)], [("3d_b", 1)], [("3d_c", 2), ("3d_c", 2)], [("2d_a", 1)]],
+                         ids=lambda b: "+".join(f"{n}@{d}" for n, d in b))
+def test_reconstruct_and_sample_bf16(bt):
+    """bfloat16 particles and images: the piecewise-constant fill copies bit patterns; sums and means are taken in
+    fp32 over bfloat16 inputs and rounded once."""
+    x, aprs, ld = batch(bt, 2, torch.float32)
+    xb = x.to(torch.bfloat16)
+    img = _ops.reconstruct_forward(aprs, xb.to(DEV), ld)
+    assert img.dtype == torch.bfloat16
+    assert torch.equal(img.float().cpu(), oracle.reconstruct_forward(aprs, xb.float(), ld))
+    # SampleParticles(Reconstruct(x)) == x exactly: the mean of equal bfloat16 values is that value
+    assert torch.equal(_ops.sample_particles_forward(aprs, img, ld).cpu(), xb)
+    g = torch.Generator().manual_seed(2)
+    im = torch.randn(img.shape, generator=g).to(torch.bfloat16)
+    close_bf16(_ops.sample_particles_forward(aprs, im.to(DEV), ld), oracle.sample_particles_forward(aprs, im.float(), ld))
+    close_bf16(_ops.reconstruct_backward(aprs, im.to(DEV), ld), oracle.reconstruct_backward(aprs, im.float(), ld))
+    close_bf16(_ops.sample_particles_backward(aprs, xb.to(DEV), ld), oracle.sample_particles_backward(aprs, xb.float(), ld))
+
+
 @pytest.mark.parametrize("math", [2, 3], ids=["bf16math", "fp32math"])
 @pytest.mark.parametrize("cin,cout", [(1, 16), (32, 32), (33, 17)])
 @pytest.mark.parametrize("bt", [[("3d_a", 0)], [("3d_b", 1), ("3d_c", 2)], [("3d_s", 0), ("3d_t", 1)]],
