@@ -17,7 +17,8 @@ namespace aprnet {
 template <typename T, class G, int CIB, int COB>
 __global__ void __launch_bounds__(G::NT)
 conv_fwd_kernel(const ConvArgs<T> a) {
-    __shared__ T patch[CIB * G::CH_STRIDE];
+    typedef typename Num<T>::acc A;          // bfloat16 features: fp32 patch, weights, products and sums
+    __shared__ A patch[CIB * G::CH_STRIDE];
     __shared__ ConvShared<G> sh;
 
     const ConvTile tile = a.tiles[blockIdx.x];
@@ -26,7 +27,7 @@ conv_fwd_kernel(const ConvArgs<T> a) {
     const int yn = a.apr.y_num[L];
     const int s_idx = min(a.S_exp - 1, a.Lc - L);
     const bool out_tree = (L == a.Lc) && (L < a.apr.level_max);
-    const T* __restrict__ wl = a.w + (int64_t)s_idx * a.Cout * a.Cin * G::K;
+    const A* __restrict__ wl = a.w + (int64_t)s_idx * a.Cout * a.Cin * G::K;
 
     open_segments<G, T>(a, L, z0, x0, sh);
     __syncthreads();
@@ -36,7 +37,7 @@ conv_fwd_kernel(const ConvArgs<T> a) {
         __syncthreads();
         const int nc = sh.ncol, nitem = sh.nitem;
         if (nc > 0) {
-            T acc[G::ITER][COB];
+            A acc[G::ITER][COB];
 #pragma unroll
             for (int it = 0; it < G::ITER; ++it)
 #pragma unroll
@@ -51,12 +52,12 @@ conv_fwd_kernel(const ConvArgs<T> a) {
                 for (int it = 0; it < G::ITER; ++it) {
                     const int col = threadIdx.x + it * G::NT;
                     if (col >= nc) continue;
-                    const T* p0 = patch + (int)sh.col_pos[col] - G::TAP0;
+                    const A* p0 = patch + (int)sh.col_pos[col] - G::TAP0;
 #pragma unroll 1
                     for (int c = 0; c < CIB; ++c) {
                         const int ci = ci0 + c;
                         if (ci >= a.Cin) break;
-                        T v[G::K];
+                        A v[G::K];
 #pragma unroll
                         for (int sz = 0; sz < G::KZ; ++sz)
 #pragma unroll
@@ -67,8 +68,8 @@ conv_fwd_kernel(const ConvArgs<T> a) {
 #pragma unroll
                         for (int co = 0; co < COB; ++co) {
                             if (co0 + co >= a.Cout) break;
-                            const T* __restrict__ wp = wl + ((int64_t)(co0 + co) * a.Cin + ci) * G::K;
-                            T res = 0;
+                            const A* __restrict__ wp = wl + ((int64_t)(co0 + co) * a.Cin + ci) * G::K;
+                            A res = 0;
 #pragma unroll
                             for (int t = 0; t < G::K; ++t) res += v[t] * wp[t];
                             acc[it][co] += res;
@@ -84,9 +85,9 @@ conv_fwd_kernel(const ConvArgs<T> a) {
 #pragma unroll
                 for (int co = 0; co < COB; ++co)
                     if (co0 + co < a.Cout) {
-                        T v = acc[it][co] + (a.bias ? a.bias[co0 + co] : (T)0);
-                        if (a.relu) v = v < (T)0 ? (T)0 : v;
-                        a.y[(int64_t)(co0 + co) * a.ldy + o] = v;
+                        A v = acc[it][co] + (a.bias ? a.bias[co0 + co] : (A)0);
+                        if (a.relu) v = v < (A)0 ? (A)0 : v;
+                        a.y[(int64_t)(co0 + co) * a.ldy + o] = Num<T>::st(v);
                     }
             }
         }
@@ -291,8 +292,8 @@ int conv_fwd_bf16(const aprnet_plan* cp, int d, int kz, int kx, int ky, const bf
     const int Cin = C1 + fu.C2;
     if (C1 <= 0 || Cout <= 0 || S_exp <= 0) return fail(APRNET_ERR_INVALID_ARGUMENT, "conv_forward: empty channel / stencil count");
     const int code = kz * 100 + kx * 10 + ky;
-    if (!conv_mfma_supported(code))
-        return fail(APRNET_ERR_UNSUPPORTED, "conv_forward: bfloat16 features are supported for the 3x3x3, 1x3x3 and 1x5x5 stencils");
+    if (!conv_mfma_supported(code) && code != 555)
+        return fail(APRNET_ERR_UNSUPPORTED, "conv_forward: bfloat16 features are supported for the 3x3x3, 1x3x3, 1x5x5 and 5x5x5 stencils");
     const int64_t nt = p->tree_parts(d);
     if (nt > 0 && (!tree_ws || ldt < nt)) return fail(APRNET_ERR_INVALID_ARGUMENT, "conv_forward: tree work space too small");
     APRNET_HIP_CHECK(hipSetDevice(p->device));
@@ -303,6 +304,15 @@ int conv_fwd_bf16(const aprnet_plan* cp, int d, int kz, int kx, int ky, const bf
     if (int rc = get_tiles(p, d, kz == 1 ? 1 : 2, kz == 1 ? 8 : 4, &tl, st)) return rc;
     if (tl.n == 0) return 0;
     ConvArgs<bf16_t> a{};
+    if (code == 555) {
+        // no matrix-core kernel for this stencil: the vector-ALU kernel with fp32 patch, weights and sums
+        a.apr = p->dapr; a.tree = p->dtree; a.tiles = tl.d_tiles;
+        a.x = x; a.ldx = ldx; a.Cin = Cin; a.w = w; a.S_exp = S_exp; a.Cout = Cout; a.bias = bias;
+        a.x2 = fu.x2; a.ldx2 = fu.ldx2; a.c_split = C1; a.relu = fu.relu;
+        a.y = y; a.ldy = ldy; a.tree_data = tree_ws; a.ldt = ldt; a.Lc = p->lc(d); a.tree_off = p->tree_offset(a.Lc);
+        a.x_count = p->number_parts(d); a.t_count = p->tree_parts(d);
+        return launch_fwd<bf16_t, G555, Chunk<float>::c555, 4>(a, tl.n, st);
+    }
     if (conv_narrow_supported(code, Cin) && fu.C2 == 0) {
         // a narrow first layer: fp32 products of the bfloat16 features on the pipelined kernel
         ConvArgs<bf16_t> n{};

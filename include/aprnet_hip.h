@@ -214,12 +214,13 @@ APRNET_DECL(double, f64)
  * Values are widened to fp32 on load, accumulated in fp32 and rounded to nearest even on store.  Weights
  * and bias are passed in fp32; the stencil convolution (3x3x3, 1x3x3, 1x5x5) rounds the weights to bfloat16
  * and multiplies on the bfloat16 matrix cores (aprnet_set_conv_path(3) keeps the weights and the products
- * in fp32).  Forward operators of the APR-UNet, plus the backward passes
+ * in fp32; the 5x5x5 stencil has no matrix-core kernel and multiplies in fp32 on the vector-ALU kernel, forward
+ * only).  Forward operators of the APR-UNet, plus the backward passes
  * of pool / upsample / tree fill and of the stencil convolution.  Argument meaning as
  * for the _f32 entry points. */
 int aprnet_conv_fwd_bf16(const aprnet_plan*, int level_delta, int kz, int kx, int ky, const uint16_t* x, int64_t ldx, int Cin,
                          const float* w, int S_exp, int Cout, const float* bias, uint16_t* y, int64_t ldy,
-                         uint16_t* tree_ws, int64_t ld_tree, void* stream);          /* not 5x5x5 */
+                         uint16_t* tree_ws, int64_t ld_tree, void* stream);          /* 5x5x5: fp32 products on the vector-ALU kernel */
 int aprnet_conv_fwd_fused_bf16(const aprnet_plan*, int level_delta, int kz, int kx, int ky, const uint16_t* x, int64_t ldx,
                                int Cin, const float* w, int S_exp, int Cout, const float* bias, uint16_t* y, int64_t ldy,
                                uint16_t* tree_ws, int64_t ld_tree, const aprnet_conv_fusion* fusion, void* stream);
