@@ -39,6 +39,67 @@ template <class G> __device__ __forceinline__ unsigned restride(unsigned pos) {
     return (pos & ~ITEM_CELL) | (((pos & ITEM_CELL) >> 6) * G::RS + (pos & 63u));
 }
 
+// Output gradient of one group of up to DW_GB columns -> LDS (through `put`), and the patch cell of every column of the
+// group -> cpl.  Wave w takes output channels co0 + w, co0 + w + NWAVE, ... (NCO of them) of 64 columns per batch.
+// The loads come in two rounds for the whole group -- column indices and cells of all batches (unconditional buffer
+// loads, lanes past the group read zero), then the gradient values, those of batch b + 1 issued before the LDS stores
+// of batch b -- instead of five dependent round trips per batch: a load under `c < ng`, or under `idx >= 0`, followed
+// by its use makes the compiler wait for memory on the spot.
+template <typename T, class G, int NCO, bool LISTS, class Lists, class Put>
+__device__ __forceinline__ void stage_gy_group(const ConvArgs<T>& a, const Lists& sh, int g0, int ng, int co0, int co_end, int wave,
+                                               int lane, int* __restrict__ cpl, Put put) {
+    constexpr int NBM = DW_GB / 64;
+    const int nbatch = (ng + 63) >> 6;
+    int idx[NBM], pos[NBM];
+    if constexpr (LISTS) {
+        const __amdgpu_buffer_rsrc_t ri = __builtin_amdgcn_make_buffer_rsrc(const_cast<int*>(sh.col_idx + g0), 0, ng * 4, 0x00020000);
+        const __amdgpu_buffer_rsrc_t rp = __builtin_amdgcn_make_buffer_rsrc(const_cast<unsigned short*>(sh.col_pos + g0), 0, ng * 2, 0x00020000);
+#pragma unroll
+        for (int b = 0; b < NBM; ++b) {
+            idx[b] = __builtin_amdgcn_raw_buffer_load_b32(ri, (b * 64 + lane) * 4, 0, 0);
+            pos[b] = (int)__builtin_amdgcn_raw_buffer_load_b16(rp, (b * 64 + lane) * 2, 0, 0);
+        }
+    } else {
+#pragma unroll
+        for (int b = 0; b < NBM; ++b) {
+            const int c = b * 64 + lane;
+            idx[b] = c < ng ? sh.col_idx[g0 + c] : 0;
+            pos[b] = c < ng ? (int)sh.col_pos[g0 + c] : 0;
+        }
+    }
+    if (wave == 0) {        // patch cell of every column of the group, as a word offset
+#pragma unroll
+        for (int b = 0; b < NBM; ++b) {
+            if (b >= nbatch) break;
+            const int c = b * 64 + lane;
+            cpl[c] = c < ng ? (LISTS ? (int)restride<G>((unsigned)pos[b]) : pos[b]) : G::TAP0;
+        }
+    }
+    T cur[NCO], nxt[NCO];
+    auto load = [&](int b, T (&v)[NCO]) {
+#pragma unroll
+        for (int k = 0; k < NCO; ++k) {
+            const int co = co0 + wave + k * G::NWAVE;
+            // (a lane past the group reads element 0 of the plane; its value is replaced by zero below)
+            v[k] = a.gy[(int64_t)min(co, co_end - 1) * a.ldy + idx[b]];
+        }
+    };
+    load(0, cur);
+#pragma unroll
+    for (int b = 0; b < NBM; ++b) {
+        if (b >= nbatch) break;
+        if (b + 1 < nbatch) load(b + 1 < NBM ? b + 1 : b, nxt);
+        const int c = b * 64 + lane;
+#pragma unroll
+        for (int k = 0; k < NCO; ++k) {
+            const int co = wave + k * G::NWAVE;
+            put(b, c, co, cur[k], c < ng && co0 + co < co_end);
+        }
+#pragma unroll
+        for (int k = 0; k < NCO; ++k) cur[k] = nxt[k];
+    }
+}
+
 // One window: its output gradient goes to gyl in groups of DW_GB columns; per group the four channel chunks of
 // the block are staged one after the other (the loads of the next chunk are issued before the matrix phase of
 // the current one) and contracted with the group's columns.
@@ -59,23 +120,11 @@ __device__ __forceinline__ void dw_window(const ConvArgs<T>& a, const Lists& sh,
     for (int g0 = 0; g0 < nc; g0 += DW_GB) {
         const int ng = min(DW_GB, nc - g0), nbatch = (ng + 63) >> 6;
         // output gradient of this group of columns -> gyl; a wave reads 64 columns of one channel
-        for (int b = 0; b < nbatch; ++b) {
-            const int c = b * 64 + lane;
-            const int64_t idx = c < ng ? sh.col_idx[g0 + c] : -1;
-            const int slot = b * 64 + 2 * (lane & 31) + (lane >> 5);
-            if (wave == 0) {        // patch cell of every column of the group, as a word offset
-                int pb = G::TAP0;
-                if (c < ng) pb = LISTS ? (int)restride<G>(sh.col_pos[g0 + c]) : (int)sh.col_pos[g0 + c];
-                cpl[c] = pb;
-            }
-#pragma unroll
-            for (int k = 0; k < 32 / G::NWAVE; ++k) {
-                const int co = wave + k * G::NWAVE;
-                float v = 0.f;
-                if (idx >= 0 && co0 + co < a.Cout) v = Num<T>::ld(a.gy[(int64_t)(co0 + co) * a.ldy + idx]);
-                gyl[slot * DW_GLD + co] = v;
-            }
-        }
+        stage_gy_group<T, G, 32 / G::NWAVE, LISTS>(a, sh, g0, ng, co0, a.Cout, wave, lane, cpl,
+            [&](int b, int, int co, T v, bool valid) {
+                const int slot = b * 64 + 2 * (lane & 31) + (lane >> 5);
+                gyl[slot * DW_GLD + co] = valid ? Num<T>::ld(v) : 0.f;
+            });
 #pragma unroll
         for (int q = 0; q < NCH; ++q) {
             __syncthreads();        // previous chunk's reads of the patch are done / gyl is written
@@ -141,22 +190,8 @@ __device__ __forceinline__ void dw_window16(const ConvArgs<T>& a, const Lists& s
     const float* ap = gyl + q4 * DW_GLD16 + (lane & 15);
     for (int g0 = 0; g0 < nc; g0 += DW_GB) {
         const int ng = min(DW_GB, nc - g0), nbatch = (ng + 63) >> 6;
-        for (int b = 0; b < nbatch; ++b) {
-            const int c = b * 64 + lane;
-            const int64_t idx = c < ng ? sh.col_idx[g0 + c] : -1;
-            if (wave == 0) {
-                int pb = G::TAP0;
-                if (c < ng) pb = LISTS ? (int)restride<G>(sh.col_pos[g0 + c]) : (int)sh.col_pos[g0 + c];
-                cpl[c] = pb;
-            }
-#pragma unroll
-            for (int k = 0; k < 16 / G::NWAVE; ++k) {
-                const int co = wave + k * G::NWAVE;
-                float v = 0.f;
-                if (idx >= 0 && co < a.Cout) v = Num<T>::ld(a.gy[(int64_t)co * a.ldy + idx]);
-                gyl[c * DW_GLD16 + co] = v;
-            }
-        }
+        stage_gy_group<T, G, 16 / G::NWAVE, LISTS>(a, sh, g0, ng, 0, a.Cout, wave, lane, cpl,
+            [&](int, int c, int co, T v, bool valid) { gyl[c * DW_GLD16 + co] = valid ? Num<T>::ld(v) : 0.f; });
 #pragma unroll
         for (int q = 0; q < NCH; ++q) {
             __syncthreads();        // previous chunk's reads of the patch are done / gyl is written
@@ -293,22 +328,8 @@ __device__ __forceinline__ void dw_window_bf16(const ConvArgs<bf16_t>& a, const 
     load_values<G, bf16_t, CIB>(a, cig0, nitem, tree_items, R);
     for (int g0 = 0; g0 < nc; g0 += DW_GB) {
         const int ng = min(DW_GB, nc - g0), nbatch = (ng + 63) >> 6;
-        for (int b = 0; b < nbatch; ++b) {
-            const int c = b * 64 + lane;
-            const int64_t idx = c < ng ? sh.col_idx[g0 + c] : -1;
-            if (wave == 0) {
-                int pb = G::TAP0;
-                if (c < ng) pb = LISTS ? (int)restride<G>(sh.col_pos[g0 + c]) : (int)sh.col_pos[g0 + c];
-                cpl[c] = pb;
-            }
-#pragma unroll
-            for (int k = 0; k < 32 / G::NWAVE; ++k) {
-                const int co = wave + k * G::NWAVE;
-                unsigned short v = 0;
-                if (idx >= 0 && co0 + co < a.Cout) v = a.gy[(int64_t)(co0 + co) * a.ldy + idx].bits;
-                gyl[co * DW_LDG16 + c] = v;
-            }
-        }
+        stage_gy_group<bf16_t, G, 32 / G::NWAVE, LISTS>(a, sh, g0, ng, co0, a.Cout, wave, lane, cpl,
+            [&](int, int c, int co, bf16_t v, bool valid) { gyl[co * DW_LDG16 + c] = valid ? v.bits : (unsigned short)0; });
 #pragma unroll
         for (int q = 0; q < NCH; ++q) {
             __syncthreads();        // previous chunk's reads of the patch are done / gyl is written
