@@ -134,6 +134,11 @@ class StarDistDataset(Dataset):
 
         dist = prob = None
         if self.labels:
+            # The label targets are computed on the GPU (the reference has CPU loops, utils.hpp:86-333): a DataLoader
+            # worker process has no usable GPU context (CUDA cannot be re-initialised after fork, and every spawned
+            # worker would open a context of its own), so this data set is for num_workers = 0.
+            if torch.utils.data.get_worker_info() is not None:
+                raise RuntimeError("StarDistDataset computes its label targets on the GPU: use DataLoader(num_workers=0)")
             label_image = imread(self._label_path(data_path))
             if window is not None:
                 label_image = np.ascontiguousarray(label_image[window])

@@ -165,6 +165,20 @@ def test_stardist_dataset_without_labels(tmp_path, capsys):
     assert dist is None and prob is None and parts.shape[0] == apr.total_number_particles()
 
 
+def test_stardist_dataset_with_labels_refuses_loader_workers(tmp_path, monkeypatch):
+    """The label targets are computed on the GPU, which a DataLoader worker process cannot use: a clear error
+    instead of 'Cannot re-initialize CUDA in forked subprocess' (the reference's CPU loops work in workers)."""
+    (tmp_path / "img").mkdir(); (tmp_path / "lab").mkdir()
+    img = (np.random.default_rng(0).random((6, 12, 12)) * 1000).astype(np.uint16)
+    np.save(tmp_path / "img" / "v0.npy", img)
+    np.save(tmp_path / "lab" / "v0_seg.npy", np.zeros(img.shape, np.uint16))
+    rays = np.array([[1, 0, 0]], np.float32)
+    ds = StarDistDataset(rays, str(tmp_path / "img"), str(tmp_path / "lab"), label_tag="_seg", pixels=True, file_ext="*.npy")
+    monkeypatch.setattr(torch.utils.data, "get_worker_info", lambda: object())
+    with pytest.raises(RuntimeError, match="num_workers=0"):
+        ds[0]
+
+
 @pytest.mark.gpu
 def test_stardist_dataset_targets_from_images(tmp_path):
     """pixels=True: image -> APR on the fly, targets from the device kernels; checked against the oracle."""
