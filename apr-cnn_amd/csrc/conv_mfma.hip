@@ -298,25 +298,30 @@ conv_mfma16_kernel(const ConvArgs<T> a) {
 }
 
 // ---------------------------------------------------------------------------------------------------------
-// bfloat16 contraction (forward, bfloat16 features): v_mfma_f32_16x16x16_bf16, fp32 accumulation.
-// The 16 k of one instruction are 2 taps x 8 input channels: lane group g = l/16 supplies four consecutive
-// bfloat16 (8 bytes) of tap 2*step + g/2, channels 4*(g%2) .. +3 of the 8-channel chunk.
-//     patch8[cg][cell]   8 bytes = 4 channels of channel group cg (0, 1) at one cell
-//     Wl8[step][h][lane] 8 bytes = the A operand of that lane (weights rounded to bfloat16 when packed)
-// Channels of the two groups are CH_STRIDE (= 16 mod 32) cells apart, so the lanes of a half wave read
-// 32 different 8-byte bank pairs.  Same lists, same D layout and epilogue as the fp32 kernel; a window needs a
-// quarter of the channel chunks and 1/8 of the matrix instructions.
-typedef short bf16x4 __attribute__((ext_vector_type(4)));
+// bfloat16 contraction (forward, bfloat16 features): v_mfma_f32_16x16x32_bf16 (gfx950), fp32 accumulation.
+// The 32 k of one instruction are 4 taps x 8 input channels: lane group g = l/16 supplies the eight bfloat16
+// (16 bytes) of tap 4*step + g, the whole 8-channel chunk of one patch cell.
+//     patch16[cell]        16 bytes = the 8 channels of the chunk at one cell
+//     Wl16[step][h][lane]  16 bytes = the A operand of that lane (weights rounded to bfloat16 when packed)
+// The sixteen lanes of a group read sixteen consecutive cells (256 bytes, every LDS bank once).  Same lists, same D
+// layout and epilogue as the fp32 kernel; a window needs a quarter of the channel chunks and 1/16 of the matrix
+// instructions.  (The K = 16 form of older parts runs at half the rate here: 16 cycles for 8192 flop.)
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 constexpr int BF_CIB = 8;
 
-template <class G> constexpr int bf16_steps() { return (G::K + 1) / 2; }
+template <class G> constexpr int bf16_steps() { return (G::K + 3) / 4; }
+// word offset of tap t's cell from the column's first tap; taps past the stencil (zero weights) re-read tap 0
+template <class G> __device__ __forceinline__ int tap_offset_rt(int t) {
+    if (t >= G::K) t = 0;
+    return ((t / (G::KX * G::KY)) * G::RX + (t / G::KY) % G::KX) * G::RS + t % G::KY;
+}
 
-// packedB[s][cb][q][step][h][lane] (8 bytes each), cb = block of 16 * COH output channels, q = chunk of 8 inputs
+// packedB[s][cb][q][step][h][lane] (16 bytes each), cb = block of 16 * COH output channels, q = chunk of 8 inputs
 // With `transposed` the image is that of the input gradient's stencil: the channel axes swap roles (Cout then
 // names the input channels of the layer, Cin its output channels) and the taps are reversed.
 __global__ void pack_weights_bf16_kernel(const float* __restrict__ w, int S_exp, int Cout, int Cin, int K, int COH,
-                                         int transposed, uint2* __restrict__ out) {
-    const int ncb = (Cout + 16 * COH - 1) / (16 * COH), nq = (Cin + BF_CIB - 1) / BF_CIB, nstep = (K + 1) / 2;
+                                         int transposed, uint4* __restrict__ out) {
+    const int ncb = (Cout + 16 * COH - 1) / (16 * COH), nq = (Cin + BF_CIB - 1) / BF_CIB, nstep = (K + 3) / 4;
     const int64_t n = (int64_t)S_exp * ncb * nq * nstep * COH * 64;
     for (int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; e < n; e += (int64_t)gridDim.x * blockDim.x) {
         int64_t r = e;
@@ -327,34 +332,31 @@ __global__ void pack_weights_bf16_kernel(const float* __restrict__ w, int S_exp,
         const int cb = (int)(r % ncb); r /= ncb;
         const int s = (int)r;
         const int g = lane >> 4, co = (cb * COH + h) * 16 + (lane & 15);
-        const int t = 2 * step + (g >> 1), ci0 = q * BF_CIB + 4 * (g & 1);
-        unsigned v[4];
+        const int t = 4 * step + g, ci0 = q * BF_CIB;
+        unsigned v[8];
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
+        for (int j = 0; j < 8; ++j) {
             float f = 0.f;
             if (t < K && co < Cout && ci0 + j < Cin)
                 f = transposed ? w[(((int64_t)s * Cin + ci0 + j) * Cout + co) * K + (K - 1 - t)]
                                : w[(((int64_t)s * Cout + co) * Cin + ci0 + j) * K + t];
             v[j] = float_to_bf16(f).bits;
         }
-        out[e] = make_uint2(v[0] | (v[1] << 16), v[2] | (v[3] << 16));
+        out[e] = make_uint4(v[0] | (v[1] << 16), v[2] | (v[3] << 16), v[4] | (v[5] << 16), v[6] | (v[7] << 16));
     }
 }
 
 template <class G>
-__device__ __forceinline__ void store_items_bf16(const ItemRegs<G, bf16_t, BF_CIB>& R, int nitem, uint2* __restrict__ patch8) {
+__device__ __forceinline__ void store_items_bf16(const ItemRegs<G, bf16_t, BF_CIB>& R, int nitem, uint4* __restrict__ patch16) {
 #pragma unroll
     for (int k = 0; k < ItemRegs<G, bf16_t, BF_CIB>::IPT; ++k) {
         if (k * G::NT >= nitem) break;                  // wave-uniform
         if (R.pos[k] == 0xffffu) continue;
-        uint2* cell = patch8 + (R.pos[k] & ITEM_CELL);
-#pragma unroll
-        for (int cg = 0; cg < 2; ++cg) {
-            const uint2 v = make_uint2((unsigned)R.v[k][4 * cg] | ((unsigned)R.v[k][4 * cg + 1] << 16),
-                                       (unsigned)R.v[k][4 * cg + 2] | ((unsigned)R.v[k][4 * cg + 3] << 16));
-            cell[cg * G::CH_STRIDE] = v;
-            if (R.pos[k] & ITEM_PAIR) cell[cg * G::CH_STRIDE + 1] = v;
-        }
+        uint4* cell = patch16 + (R.pos[k] & ITEM_CELL);
+        const uint4 v = make_uint4((unsigned)R.v[k][0] | ((unsigned)R.v[k][1] << 16), (unsigned)R.v[k][2] | ((unsigned)R.v[k][3] << 16),
+                                   (unsigned)R.v[k][4] | ((unsigned)R.v[k][5] << 16), (unsigned)R.v[k][6] | ((unsigned)R.v[k][7] << 16));
+        cell[0] = v;
+        if (R.pos[k] & ITEM_PAIR) cell[1] = v;
     }
 }
 
@@ -414,15 +416,15 @@ __device__ __forceinline__ void load_values16(const ConvArgs<bf16_t>& a, int ci0
     }
 }
 template <class G, int IPT>
-__device__ __forceinline__ void store_items16(const ItemRegs16<G, IPT>& R, int nitem, uint2* __restrict__ patch8) {
+__device__ __forceinline__ void store_items16(const ItemRegs16<G, IPT>& R, int nitem, uint4* __restrict__ patch16) {
 #pragma unroll
     for (int k = 0; k < IPT; ++k) {
         if (k * G::NT >= nitem) break;                  // wave-uniform
         if (R.pos[k] == 0xffffu) continue;
-        uint2* cell = patch8 + (R.pos[k] & ITEM_CELL);
-        const uint2 v0 = make_uint2((unsigned)R.v[k][0], (unsigned)R.v[k][1]), v1 = make_uint2((unsigned)R.v[k][2], (unsigned)R.v[k][3]);
-        cell[0] = v0; cell[G::CH_STRIDE] = v1;
-        if (R.pos[k] & ITEM_PAIR) { cell[1] = v0; cell[G::CH_STRIDE + 1] = v1; }
+        uint4* cell = patch16 + (R.pos[k] & ITEM_CELL);
+        const uint4 v = make_uint4((unsigned)R.v[k][0], (unsigned)R.v[k][1], (unsigned)R.v[k][2], (unsigned)R.v[k][3]);
+        cell[0] = v;
+        if (R.pos[k] & ITEM_PAIR) cell[1] = v;
     }
 }
 
@@ -449,18 +451,21 @@ __global__ void interleave8_kernel(const bf16_t* __restrict__ x, int64_t ldx, co
 template <class G, int COH, int NB, bool FUSE, int MODE, bool IL, class Lists>
 __device__ __forceinline__ void mfma_bf16_window(const ConvArgs<bf16_t>& a, int co0, int nc, int nitem, bool tree_items, int first,
                                                  const uint4* __restrict__ wl, const Lists& sh,
-                                                 uint2* __restrict__ patch8, uint2* __restrict__ Wl8,
+                                                 uint4* __restrict__ patch16, uint4* __restrict__ Wl16,
                                                  const float* __restrict__ bias_l) {
     constexpr int NSTEP = bf16_steps<G>();
     const int lane = lane_id();
-    const bool second_tap = lane >= 32;
+    // cell offset of this lane group's tap in every step (tap 4 * step + lane / 16)
+    int toff[NSTEP];
+#pragma unroll
+    for (int st = 0; st < NSTEP; ++st) toff[st] = tap_offset_rt<G>(4 * st + (lane >> 4));
     constexpr int NBA = NB > 0 ? NB : 1;
     int bbase[NBA];
 #pragma unroll
     for (int j = 0; j < NB; ++j) {
         const int col = ((first + G::NWAVE * j) << 4) + (lane & 15);
         const int pos = col < nc ? (int)(sh.col_pos[col] & COL_CELL) - G::TAP0 : 0;
-        bbase[j] = pos + ((lane >> 4) & 1) * G::CH_STRIDE;
+        bbase[j] = pos;
     }
     floatx4 acc[NBA][COH];
 #pragma unroll
@@ -470,7 +475,7 @@ __device__ __forceinline__ void mfma_bf16_window(const ConvArgs<bf16_t>& a, int 
 #pragma unroll
             for (int r = 0; r < 4; ++r) acc[j][h][r] = 0.f;
 
-    constexpr int W16 = NSTEP * COH * 32;                        // 16-byte elements of a weight chunk
+    constexpr int W16 = NSTEP * COH * 64;                        // 16-byte elements of a weight chunk
     constexpr int WPT = (W16 + G::NT - 1) / G::NT;
     typename std::conditional<IL, ItemRegs16<G, ItemRegs<G, bf16_t, BF_CIB>::IPT>, ItemRegs<G, bf16_t, BF_CIB>>::type R;
     uint4 wr[WPT];
@@ -482,16 +487,16 @@ __device__ __forceinline__ void mfma_bf16_window(const ConvArgs<bf16_t>& a, int 
 #define APRNET_STORE_WEIGHTS()                                                                     \
     _Pragma("unroll") for (int k = 0; k < WPT; ++k) {                                              \
         const int i = threadIdx.x + k * G::NT;                                                     \
-        if (i < W16) reinterpret_cast<uint4*>(Wl8)[i] = wr[k];                                     \
+        if (i < W16) Wl16[i] = wr[k];                                                              \
     }
     if constexpr (IL) { fetch_slots16<G>(sh, nitem, R); load_values16<G>(a, 0, nitem, tree_items, R); }
     else load_items<G, bf16_t, BF_CIB>(a, 0, nitem, tree_items, sh, R, 0, std::bool_constant<FUSE>{});
     APRNET_LOAD_WEIGHTS(0)
-    for (int i = threadIdx.x; i < 2 * G::CH_STRIDE; i += G::NT) patch8[i] = make_uint2(0u, 0u);     // once per window
+    for (int i = threadIdx.x; i < G::CH_STRIDE; i += G::NT) patch16[i] = make_uint4(0u, 0u, 0u, 0u);     // once per window
     for (int ci0 = 0; ci0 < a.Cin; ci0 += BF_CIB) {
         __syncthreads();
-        // items -> patch: two 8-byte cells (channel groups) per item, four bfloat16 each
-        if constexpr (IL) store_items16<G>(R, nitem, patch8); else store_items_bf16<G>(R, nitem, patch8);
+        // items -> patch: one 16-byte cell per item, the eight bfloat16 channels of the chunk
+        if constexpr (IL) store_items16<G>(R, nitem, patch16); else store_items_bf16<G>(R, nitem, patch16);
         APRNET_STORE_WEIGHTS()
         __syncthreads();
         if (ci0 + BF_CIB < a.Cin) {
@@ -501,18 +506,14 @@ __device__ __forceinline__ void mfma_bf16_window(const ConvArgs<bf16_t>& a, int 
         }
 #pragma unroll
         for (int st = 0; st < NSTEP; ++st) {
-            constexpr int dummy = 0; (void)dummy;
-            const int offA = tap_offset<G>(2 * st);
-            const int offB = (2 * st + 1 < G::K) ? tap_offset<G>(2 * st + 1) : offA;     // the weights of a missing tap are zero
-            const int off = second_tap ? offB : offA;
-            bf16x4 av[COH];
+            bf16x8 av[COH];
 #pragma unroll
-            for (int h = 0; h < COH; ++h) av[h] = __builtin_bit_cast(bf16x4, Wl8[(st * COH + h) * 64 + lane]);
+            for (int h = 0; h < COH; ++h) av[h] = __builtin_bit_cast(bf16x8, Wl16[(st * COH + h) * 64 + lane]);
 #pragma unroll
             for (int j = 0; j < NB; ++j) {
-                const bf16x4 bv = __builtin_bit_cast(bf16x4, patch8[bbase[j] + off]);
+                const bf16x8 bv = __builtin_bit_cast(bf16x8, patch16[bbase[j] + toff[st]]);
 #pragma unroll
-                for (int h = 0; h < COH; ++h) acc[j][h] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(av[h], bv, acc[j][h], 0, 0, 0);
+                for (int h = 0; h < COH; ++h) acc[j][h] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(av[h], bv, acc[j][h], 0, 0, 0);
             }
         }
     }
@@ -572,9 +573,8 @@ __global__ void __launch_bounds__(G::NT) __attribute__((amdgpu_waves_per_eu(4, 4
 conv_mfma_bf16_kernel(const ConvArgs<bf16_t> a) {
     constexpr int NBW = 4, NSTEP = bf16_steps<G>();
     static_assert((G::MAXCOL + 15) / 16 <= G::NWAVE * NBW, "a window must fit the accumulators of the block");
-    static_assert(G::CH_STRIDE % 32 == 16, "the two channel groups of a half wave must fall on different bank pairs");
-    __shared__ uint2 patch8[2 * G::CH_STRIDE];
-    __shared__ __attribute__((aligned(16))) uint2 Wl8[NSTEP * COH * 64];
+    __shared__ __attribute__((aligned(16))) uint4 patch16[G::CH_STRIDE];
+    __shared__ __attribute__((aligned(16))) uint4 Wl16[NSTEP * COH * 64];
     __shared__ float bias_l[16 * COH];
 
     const ConvTile tile = a.tiles[blockIdx.x];
@@ -584,7 +584,7 @@ conv_mfma_bf16_kernel(const ConvArgs<bf16_t> a) {
     const int nq = (a.Cin + BF_CIB - 1) / BF_CIB;
     // a.w carries the packed bfloat16 image
     const uint4* __restrict__ wl = reinterpret_cast<const uint4*>(a.w) +
-                                   ((int64_t)s_idx * gridDim.y + blockIdx.y) * nq * (NSTEP * COH * 32);
+                                   ((int64_t)s_idx * gridDim.y + blockIdx.y) * nq * (NSTEP * COH * 64);
     const int wave = threadIdx.x >> 6;
     const bool tree_items = MODE == 0 && L < a.Lc;       // the output gradient has no tree part
 
@@ -601,11 +601,11 @@ conv_mfma_bf16_kernel(const ConvArgs<bf16_t> a) {
         const int first = (wave - (int)blockIdx.x - win) & (G::NWAVE - 1);
         const int nb = first < nblk ? (nblk - first + G::NWAVE - 1) / G::NWAVE : 0;
         switch (__builtin_amdgcn_readfirstlane(nb)) {
-            case 0: mfma_bf16_window<G, COH, 0, FUSE, MODE, IL>(a, co0, nc, nitem, tree_items, first, wl, gl, patch8, Wl8, bias_l); break;
-            case 1: mfma_bf16_window<G, COH, 1, FUSE, MODE, IL>(a, co0, nc, nitem, tree_items, first, wl, gl, patch8, Wl8, bias_l); break;
-            case 2: mfma_bf16_window<G, COH, 2, FUSE, MODE, IL>(a, co0, nc, nitem, tree_items, first, wl, gl, patch8, Wl8, bias_l); break;
-            case 3: mfma_bf16_window<G, COH, 3, FUSE, MODE, IL>(a, co0, nc, nitem, tree_items, first, wl, gl, patch8, Wl8, bias_l); break;
-            default: mfma_bf16_window<G, COH, 4, FUSE, MODE, IL>(a, co0, nc, nitem, tree_items, first, wl, gl, patch8, Wl8, bias_l); break;
+            case 0: mfma_bf16_window<G, COH, 0, FUSE, MODE, IL>(a, co0, nc, nitem, tree_items, first, wl, gl, patch16, Wl16, bias_l); break;
+            case 1: mfma_bf16_window<G, COH, 1, FUSE, MODE, IL>(a, co0, nc, nitem, tree_items, first, wl, gl, patch16, Wl16, bias_l); break;
+            case 2: mfma_bf16_window<G, COH, 2, FUSE, MODE, IL>(a, co0, nc, nitem, tree_items, first, wl, gl, patch16, Wl16, bias_l); break;
+            case 3: mfma_bf16_window<G, COH, 3, FUSE, MODE, IL>(a, co0, nc, nitem, tree_items, first, wl, gl, patch16, Wl16, bias_l); break;
+            default: mfma_bf16_window<G, COH, 4, FUSE, MODE, IL>(a, co0, nc, nitem, tree_items, first, wl, gl, patch16, Wl16, bias_l); break;
         }
         __syncthreads();        // the next window rewrites the patch
     }
@@ -713,15 +713,15 @@ int interleave8_bf16(const bf16_t* x, int64_t ldx, const bf16_t* x2, int64_t ldx
     return 0;
 }
 size_t conv_packed_bf16_bytes(int code, int S_exp, int Cout, int Cin) {
-    const int coh = conv_coh(Cout), nstep = (conv_taps(code) + 1) / 2;
-    return (size_t)S_exp * ((Cout + 16 * coh - 1) / (16 * coh)) * ((Cin + BF_CIB - 1) / BF_CIB) * nstep * coh * 64 * sizeof(uint2);
+    const int coh = conv_coh(Cout), nstep = (conv_taps(code) + 3) / 4;
+    return (size_t)S_exp * ((Cout + 16 * coh - 1) / (16 * coh)) * ((Cin + BF_CIB - 1) / BF_CIB) * nstep * coh * 64 * sizeof(uint4);
 }
 // Cout / Cin: channels on the M axis of the kernel / contracted channels (transposed: the layer's Cin / Cout)
 int pack_conv_weights_bf16(int code, const float* w, int S_exp, int Cout, int Cin, void* packed, hipStream_t st, bool transposed) {
-    const size_t n = conv_packed_bf16_bytes(code, S_exp, Cout, Cin) / sizeof(uint2);
+    const size_t n = conv_packed_bf16_bytes(code, S_exp, Cout, Cin) / sizeof(uint4);
     dim3 grid((unsigned)std::min<size_t>((n + 255) / 256, 2048));
     hipLaunchKernelGGL(pack_weights_bf16_kernel, grid, dim3(256), 0, st, w, S_exp, Cout, Cin, conv_taps(code), conv_coh(Cout),
-                       transposed ? 1 : 0, (uint2*)packed);
+                       transposed ? 1 : 0, (uint4*)packed);
     APRNET_LAUNCH_CHECK("pack_weights_bf16_kernel");
     return 0;
 }
