@@ -460,12 +460,25 @@ __device__ __forceinline__ void mfma_bf16_window(const ConvArgs<bf16_t>& a, int 
 #pragma unroll
     for (int st = 0; st < NSTEP; ++st) toff[st] = tap_offset_rt<G>(4 * st + (lane >> 4));
     constexpr int NBA = NB > 0 ? NB : 1;
-    int bbase[NBA];
+    int bbase[NBA], ocol[NBA];
+    if constexpr (IL) {
+        // cell and output index of this lane's columns: unconditional loads (columns past the end read zero) that
+        // travel together with the list loads below instead of taking a round trip each
+        const __amdgpu_buffer_rsrc_t rcp = __builtin_amdgcn_make_buffer_rsrc(const_cast<unsigned short*>(sh.col_pos), 0, nc * 2, 0x00020000);
+        const __amdgpu_buffer_rsrc_t rci = __builtin_amdgcn_make_buffer_rsrc(const_cast<int*>(sh.col_idx), 0, nc * 4, 0x00020000);
 #pragma unroll
-    for (int j = 0; j < NB; ++j) {
-        const int col = ((first + G::NWAVE * j) << 4) + (lane & 15);
-        const int pos = col < nc ? (int)(sh.col_pos[col] & COL_CELL) - G::TAP0 : 0;
-        bbase[j] = pos;
+        for (int j = 0; j < NB; ++j) {
+            const int col = ((first + G::NWAVE * j) << 4) + (lane & 15);
+            bbase[j] = (int)__builtin_amdgcn_raw_buffer_load_b16(rcp, col * 2, 0, 0);
+            ocol[j] = __builtin_amdgcn_raw_buffer_load_b32(rci, col * 4, 0, 0);
+        }
+    } else {
+#pragma unroll
+        for (int j = 0; j < NB; ++j) {
+            const int col = ((first + G::NWAVE * j) << 4) + (lane & 15);
+            const int pos = col < nc ? (int)(sh.col_pos[col] & COL_CELL) - G::TAP0 : 0;
+            bbase[j] = pos;
+        }
     }
     floatx4 acc[NBA][COH];
 #pragma unroll
@@ -489,8 +502,15 @@ __device__ __forceinline__ void mfma_bf16_window(const ConvArgs<bf16_t>& a, int 
         const int i = threadIdx.x + k * G::NT;                                                     \
         if (i < W16) Wl16[i] = wr[k];                                                              \
     }
-    if constexpr (IL) { fetch_slots16<G>(sh, nitem, R); load_values16<G>(a, 0, nitem, tree_items, R); }
-    else load_items<G, bf16_t, BF_CIB>(a, 0, nitem, tree_items, sh, R, 0, std::bool_constant<FUSE>{});
+    if constexpr (IL) {
+        fetch_slots16<G>(sh, nitem, R);
+#pragma unroll
+        for (int j = 0; j < NB; ++j) {
+            const int col = ((first + G::NWAVE * j) << 4) + (lane & 15);
+            bbase[j] = col < nc ? (bbase[j] & (int)COL_CELL) - G::TAP0 : 0;
+        }
+        load_values16<G>(a, 0, nitem, tree_items, R);
+    } else load_items<G, bf16_t, BF_CIB>(a, 0, nitem, tree_items, sh, R, 0, std::bool_constant<FUSE>{});
     APRNET_LOAD_WEIGHTS(0)
     for (int i = threadIdx.x; i < G::CH_STRIDE; i += G::NT) patch16[i] = make_uint4(0u, 0u, 0u, 0u);     // once per window
     for (int ci0 = 0; ci0 < a.Cin; ci0 += BF_CIB) {
@@ -523,7 +543,8 @@ __device__ __forceinline__ void mfma_bf16_window(const ConvArgs<bf16_t>& a, int 
     for (int j = 0; j < NB; ++j) {
         const int col = ((first + G::NWAVE * j) << 4) + (lane & 15);
         if (col >= nc) continue;
-        const int64_t o = sh.col_idx[col];
+        int64_t o;
+        if constexpr (IL) o = ocol[j]; else o = sh.col_idx[col];
         if constexpr (MODE == 0) {
             if (IL && a.y_g8) {
                 // grouped output: the lane's four channels of a part are half of a 16-byte group
@@ -591,12 +612,18 @@ conv_mfma_bf16_kernel(const ConvArgs<bf16_t> a) {
     if (threadIdx.x < 16 * COH)
         bias_l[threadIdx.x] = (MODE == 0 && a.bias && co0 + (int)threadIdx.x < a.Cout) ? a.bias[co0 + threadIdx.x] : 0.f;
 
+    __shared__ int4 hdr[16];                  // headers of sixteen windows: one round trip instead of one per window
     const int wb = a.tile_win[blockIdx.x], we = a.tile_win[blockIdx.x + 1];
     for (int w = wb; w < we; ++w) {
         const int win = w - wb;
-        const int4 hd = a.win[w];
+        if ((win & 15) == 0) {                // every wave is past the previous window's last barrier
+            if (threadIdx.x < 16 && w + (int)threadIdx.x < we) hdr[threadIdx.x] = a.win[w + threadIdx.x];
+            __syncthreads();
+        }
+        const int4 hd = hdr[win & 15];
         const int nitem = __builtin_amdgcn_readfirstlane(hd.y), nc = __builtin_amdgcn_readfirstlane(hd.w);
-        const WindowLists gl{a.l_item_idx + (unsigned)hd.x, a.l_item_pos + (unsigned)hd.x, a.l_col_idx + (unsigned)hd.z, a.l_col_pos + (unsigned)hd.z};
+        const unsigned i0 = (unsigned)__builtin_amdgcn_readfirstlane(hd.x), c0 = (unsigned)__builtin_amdgcn_readfirstlane(hd.z);
+        const WindowLists gl{a.l_item_idx + i0, a.l_item_pos + i0, a.l_col_idx + c0, a.l_col_pos + c0};
         const int nblk = (nc + 15) >> 4;
         const int first = (wave - (int)blockIdx.x - win) & (G::NWAVE - 1);
         const int nb = first < nblk ? (nblk - first + G::NWAVE - 1) / G::NWAVE : 0;
