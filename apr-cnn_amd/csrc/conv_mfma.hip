@@ -21,6 +21,8 @@
 
 namespace aprnet {
 
+typedef int intx4w __attribute__((ext_vector_type(4)));
+
 template <class G>
 __device__ __forceinline__ constexpr int tap_offset(int t) {
     return ((t / (G::KX * G::KY)) * G::RX + (t / G::KY) % G::KX) * G::RS + (t % G::KY);
@@ -109,16 +111,21 @@ __device__ __forceinline__ void mfma16_window(const ConvArgs<T>& a, int co0, int
     constexpr int W4 = KC * 4 * COH;                             // float4 elements of a weight chunk
     constexpr int WPT = (W4 + G::NT - 1) / G::NT;
     ItemRegs<G, T, CIB> R;
-    float4 wr[WPT];
+    // The weights of a chunk come through unconditional buffer loads (lanes past the end read zeros): under a
+    // per-lane branch the compiler waits for every load in flight before it enters the branch, which made each
+    // chunk wait for the feature loads issued just before instead of letting them travel during the matrix phase.
+    intx4w wr[WPT];
 #define APRNET_LOAD_WEIGHTS(q)                                                                     \
-    _Pragma("unroll") for (int k = 0; k < WPT; ++k) {                                              \
-        const int i = threadIdx.x + k * G::NT;                                                     \
-        wr[k] = (i < W4) ? (wl + (int64_t)(q) * W4)[i] : make_float4(0.f, 0.f, 0.f, 0.f);          \
+    {                                                                                              \
+        const __amdgpu_buffer_rsrc_t rw_ = __builtin_amdgcn_make_buffer_rsrc(                      \
+            const_cast<float4*>(wl + (int64_t)(q) * W4), 0, W4 * 16, 0x00020000);                  \
+        _Pragma("unroll") for (int k = 0; k < WPT; ++k)                                            \
+            wr[k] = __builtin_amdgcn_raw_buffer_load_b128(rw_, (int)(threadIdx.x + k * G::NT) * 16, 0, 0); \
     }
 #define APRNET_STORE_WEIGHTS()                                                                     \
     _Pragma("unroll") for (int k = 0; k < WPT; ++k) {                                              \
         const int i = threadIdx.x + k * G::NT;                                                     \
-        if (i < W4) reinterpret_cast<float4*>(Wl)[i] = wr[k];                                      \
+        if (i < W4) reinterpret_cast<intx4w*>(Wl)[i] = wr[k];                                      \
     }
     // Staging runs at a raised wave priority, the matrix loop at the default one: fp32 matrix instructions share the
     // SIMD's vector pipe, and a workgroup that is staging gets back to its own matrix phase sooner when its few
@@ -491,16 +498,18 @@ __device__ __forceinline__ void mfma_bf16_window(const ConvArgs<bf16_t>& a, int 
     constexpr int W16 = NSTEP * COH * 64;                        // 16-byte elements of a weight chunk
     constexpr int WPT = (W16 + G::NT - 1) / G::NT;
     typename std::conditional<IL, ItemRegs16<G, ItemRegs<G, bf16_t, BF_CIB>::IPT>, ItemRegs<G, bf16_t, BF_CIB>>::type R;
-    uint4 wr[WPT];
+    intx4w wr[WPT];                    // unconditional buffer loads, see the fp32 kernel
 #define APRNET_LOAD_WEIGHTS(q)                                                                     \
-    _Pragma("unroll") for (int k = 0; k < WPT; ++k) {                                              \
-        const int i = threadIdx.x + k * G::NT;                                                     \
-        wr[k] = (i < W16) ? (wl + (int64_t)(q) * W16)[i] : make_uint4(0u, 0u, 0u, 0u);             \
+    {                                                                                              \
+        const __amdgpu_buffer_rsrc_t rw_ = __builtin_amdgcn_make_buffer_rsrc(                      \
+            const_cast<uint4*>(wl + (int64_t)(q) * W16), 0, W16 * 16, 0x00020000);                 \
+        _Pragma("unroll") for (int k = 0; k < WPT; ++k)                                            \
+            wr[k] = __builtin_amdgcn_raw_buffer_load_b128(rw_, (int)(threadIdx.x + k * G::NT) * 16, 0, 0); \
     }
 #define APRNET_STORE_WEIGHTS()                                                                     \
     _Pragma("unroll") for (int k = 0; k < WPT; ++k) {                                              \
         const int i = threadIdx.x + k * G::NT;                                                     \
-        if (i < W16) Wl16[i] = wr[k];                                                              \
+        if (i < W16) reinterpret_cast<intx4w*>(Wl16)[i] = wr[k];                                   \
     }
     if constexpr (IL) {
         fetch_slots16<G>(sh, nitem, R);
