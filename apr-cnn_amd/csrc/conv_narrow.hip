@@ -233,7 +233,10 @@ conv_narrow_kernel(const ConvArgs<T> a, const NarrowArgs na) {
         h0 = h1; h1 = h2; h2 = hN; s0 = s1; s1 = sN; cp = c0; c0 = cN; v0 = vN; nc_prev = nc;
         const int nitem = __builtin_amdgcn_readfirstlane(h0[1]);
         nc = __builtin_amdgcn_readfirstlane(h0[3]);
-        // 0. outputs of the previous window
+        // 0. outputs of the previous window.  Everything loaded during the previous iteration is waited for here, by
+        // hand (vmcnt 0, the other counters untouched): left to the compiler the wait lands at the first use of a
+        // loaded value, after these stores, and then includes them (memory operations complete in issue order).
+        __builtin_amdgcn_s_waitcnt(0x0F70);
         if (nc_prev > 0) store_outputs(cp, w - 1, nc_prev);
         // 1. the items of this window -> its patch buffer (zeroed two windows ago)
 #pragma unroll
