@@ -60,13 +60,16 @@ __global__ void pack_weights_narrow_kernel(const float* __restrict__ w, int S_ex
 // two workgroups of eight waves per CU (three, at 80 registers with a few spills, ran slower: 2.0 against 1.25 ms)
 constexpr int NARROW_WAVES = 4;
 struct NarrowArgs {
-    int n_win;                          // stored windows of the plan's lists, finest level first
+    int win0;                           // first window of this launch
+    int n_win;                          // windows of this launch (stored windows of the plan's lists, finest level first)
     int n_lv;                           // levels with windows
     int lv_first[MAX_LEVELS];           // first window of the k-th such level
     int lv_level[MAX_LEVELS];
 };
 
-template <typename T, class G, int CIN, int COH>
+// TREE: the windows may hold items that come from the tree (any level below the finest one of the call); without
+// it the tree loads, a third of a window's load instructions, are not issued at all
+template <typename T, class G, int CIN, int COH, bool TREE>
 __global__ void __launch_bounds__(G::NT) __attribute__((amdgpu_waves_per_eu(NARROW_WAVES, NARROW_WAVES)))
 conv_narrow_kernel(const ConvArgs<T> a, const NarrowArgs na) {
     typedef NarrowShape<G, CIN> NS;
@@ -80,7 +83,7 @@ conv_narrow_kernel(const ConvArgs<T> a, const NarrowArgs na) {
     const int lane = lane_id();
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int co0 = blockIdx.y * 16 * COH;
-    const int wb = (int)((int64_t)na.n_win * blockIdx.x / gridDim.x), we = (int)((int64_t)na.n_win * (blockIdx.x + 1) / gridDim.x);
+    const int wb = na.win0 + (int)((int64_t)na.n_win * blockIdx.x / gridDim.x), we = na.win0 + (int)((int64_t)na.n_win * (blockIdx.x + 1) / gridDim.x);
     if (wb >= we) return;
 
     if (threadIdx.x < 16 * COH)
@@ -96,7 +99,7 @@ conv_narrow_kernel(const ConvArgs<T> a, const NarrowArgs na) {
         loff[q] = (u / G::KY) * G::CH_STRIDE + (u % G::KY) - G::TAP0;
     }
 
-    const __amdgpu_buffer_rsrc_t r_hdr = __builtin_amdgcn_make_buffer_rsrc(const_cast<int4*>(a.win), 0, na.n_win * 16, 0x00020000);
+    const __amdgpu_buffer_rsrc_t r_hdr = __builtin_amdgcn_make_buffer_rsrc(const_cast<int4*>(a.win), 0, (na.win0 + na.n_win) * 16, 0x00020000);
     __amdgpu_buffer_rsrc_t rx[CIN], rt[CIN];
 #pragma unroll
     for (int c = 0; c < CIN; ++c) {
@@ -120,22 +123,35 @@ conv_narrow_kernel(const ConvArgs<T> a, const NarrowArgs na) {
 #pragma unroll
         for (int k = 0; k < IPT; ++k) {
             const int it = threadIdx.x + k * G::NT;
-            s.idx[k] = __builtin_amdgcn_raw_buffer_load_b32(ri, it * 4, 0, 0);
-            s.pos[k] = (int)__builtin_amdgcn_raw_buffer_load_b16(rp, it * 2, 0, 0);
+            if (k == 0 || k * G::NT < nitem) {          // wave-uniform: most windows fill one round
+                s.idx[k] = __builtin_amdgcn_raw_buffer_load_b32(ri, it * 4, 0, 0);
+                s.pos[k] = (int)__builtin_amdgcn_raw_buffer_load_b16(rp, it * 2, 0, 0);
+            } else { s.idx[k] = 0; s.pos[k] = 0; }
         }
     };
     // values of the slots' items: a lane past the window's items reads slot zeros and loads element 0 (unused)
     // (from the plane and from the tree with one of the two offsets out of range; the two are combined when the
     // values are used, not here: an operation on a loaded value makes the wave wait for it)
-    struct Vals { typename RawLoad<T>::raw x[IPT][CIN], t[IPT][CIN]; };
-    auto load_vals = [&](const Slots& s, Vals& v) {
+    struct Vals { typename RawLoad<T>::raw x[IPT][CIN], t[TREE ? IPT : 1][CIN]; };
+    auto load_vals = [&](const intx4n hd, const Slots& s, Vals& v) {
+        const int nitem = __builtin_amdgcn_readfirstlane(hd[1]);
 #pragma unroll
         for (int k = 0; k < IPT; ++k) {
+            if (k > 0 && k * G::NT >= nitem) {              // wave-uniform: a round without items issues no loads
+#pragma unroll
+                for (int c = 0; c < CIN; ++c) { v.x[k][c] = 0; if constexpr (TREE) v.t[k][c] = 0; }
+                continue;
+            }
             const unsigned off = (unsigned)s.idx[k] * (unsigned)sizeof(T);
             const bool from_tree = (s.pos[k] & ITEM_TREE) != 0;
-            const unsigned ox = from_tree ? BUF_OOB : off, ot = from_tree ? off : BUF_OOB;
+            if constexpr (TREE) {
+                const unsigned ox = from_tree ? BUF_OOB : off, ot = from_tree ? off : BUF_OOB;
 #pragma unroll
-            for (int c = 0; c < CIN; ++c) { v.x[k][c] = RawLoad<T>::ld(rx[c], ox); v.t[k][c] = RawLoad<T>::ld(rt[c], ot); }
+                for (int c = 0; c < CIN; ++c) { v.x[k][c] = RawLoad<T>::ld(rx[c], ox); v.t[k][c] = RawLoad<T>::ld(rt[c], ot); }
+            } else {
+#pragma unroll
+                for (int c = 0; c < CIN; ++c) v.x[k][c] = RawLoad<T>::ld(rx[c], off);
+            }
         }
     };
     // the columns this wave computes in window w: block j holds columns 16 * (first + NWAVE j) .. + 15
@@ -149,8 +165,10 @@ conv_narrow_kernel(const ConvArgs<T> a, const NarrowArgs na) {
 #pragma unroll
         for (int j = 0; j < NBW; ++j) {
             const int col = ((first + G::NWAVE * j) << 4) + (lane & 15);
-            c.idx[j] = __builtin_amdgcn_raw_buffer_load_b32(ri, col * 4, 0, 0);
-            c.pos[j] = (int)__builtin_amdgcn_raw_buffer_load_b16(rp, col * 2, 0, 0);
+            if (j == 0 || ((first + G::NWAVE * j) << 4) < nc) {        // wave-uniform: a block the window does not have issues no loads
+                c.idx[j] = __builtin_amdgcn_raw_buffer_load_b32(ri, col * 4, 0, 0);
+                c.pos[j] = (int)__builtin_amdgcn_raw_buffer_load_b16(rp, col * 2, 0, 0);
+            } else { c.idx[j] = 0; c.pos[j] = 0; }
         }
     };
     auto level_of = [&](int w) -> int {
@@ -217,7 +235,7 @@ conv_narrow_kernel(const ConvArgs<T> a, const NarrowArgs na) {
     load_slots(h1, s1);
     load_cols(h1, wb, cN);
     load_slots(h2, sN);
-    load_vals(s1, vN);
+    load_vals(h1, s1, vN);
     int cur_level = level_of(wb);
     stage_weights(cur_level);
     __syncthreads();
@@ -246,13 +264,14 @@ conv_narrow_kernel(const ConvArgs<T> a, const NarrowArgs na) {
             float* cell = buf + ((unsigned)s0.pos[k] & ITEM_CELL);
 #pragma unroll
             for (int c = 0; c < CIN; ++c) {
-                const float v = RawLoad<T>::cast(v0.x[k][c] | v0.t[k][c]);
+                float v;
+                if constexpr (TREE) v = RawLoad<T>::cast(v0.x[k][c] | v0.t[k][c]); else v = RawLoad<T>::cast(v0.x[k][c]);
                 cell[c * G::CH_STRIDE] = v;
                 if (s0.pos[k] & ITEM_PAIR) cell[c * G::CH_STRIDE + 1] = v;
             }
         }
         // 2. loads of the windows ahead: values of w + 1, columns of w + 1, slots of w + 2, header of w + 3
-        load_vals(s1, vN);
+        load_vals(h1, s1, vN);
         load_cols(h1, w + 1, cN);
         load_slots(h2, sN);
         hN = load_header(w + 3);
@@ -348,10 +367,23 @@ static int launch_narrow_cin(const ConvArgs<T>& a, const NarrowArgs& na, hipStre
     // two persistent workgroups per CU; short lists get one workgroup per window
     int dev = 0, cus = 256;
     if (hipGetDevice(&dev) == hipSuccess) (void)hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
-    dim3 grid((unsigned)std::max(1, std::min(na.n_win, 2 * cus)), (unsigned)((a.Cout + 16 * coh - 1) / (16 * coh)));
-    if (coh == 1) hipLaunchKernelGGL((conv_narrow_kernel<T, G, CIN, 1>), grid, dim3(G::NT), 0, st, a, na);
-    else hipLaunchKernelGGL((conv_narrow_kernel<T, G, CIN, 2>), grid, dim3(G::NT), 0, st, a, na);
-    APRNET_LAUNCH_CHECK("conv_narrow_kernel");
+    // the windows of the call's finest level hold no tree items (they come first in the list): their launch skips the tree loads
+    const int n_fine = (na.n_lv > 0 && na.lv_level[0] == a.Lc) ? (na.n_lv > 1 ? na.lv_first[1] : na.n_win) : 0;
+    for (int part = 0; part < 2; ++part) {
+        NarrowArgs nb = na;
+        nb.win0 = part == 0 ? 0 : n_fine;
+        nb.n_win = part == 0 ? n_fine : na.n_win - n_fine;
+        if (nb.n_win <= 0) continue;
+        dim3 grid((unsigned)std::max(1, std::min(nb.n_win, 2 * cus)), (unsigned)((a.Cout + 16 * coh - 1) / (16 * coh)));
+        if (part == 0) {
+            if (coh == 1) hipLaunchKernelGGL((conv_narrow_kernel<T, G, CIN, 1, false>), grid, dim3(G::NT), 0, st, a, nb);
+            else hipLaunchKernelGGL((conv_narrow_kernel<T, G, CIN, 2, false>), grid, dim3(G::NT), 0, st, a, nb);
+        } else {
+            if (coh == 1) hipLaunchKernelGGL((conv_narrow_kernel<T, G, CIN, 1, true>), grid, dim3(G::NT), 0, st, a, nb);
+            else hipLaunchKernelGGL((conv_narrow_kernel<T, G, CIN, 2, true>), grid, dim3(G::NT), 0, st, a, nb);
+        }
+        APRNET_LAUNCH_CHECK("conv_narrow_kernel");
+    }
     return 0;
 }
 template <typename T, class G>
