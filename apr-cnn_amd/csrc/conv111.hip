@@ -55,24 +55,25 @@ template <> struct PairBits111<8> { typedef uint32_t type __attribute__((ext_vec
 
 // T = storage type of the features (float, or bfloat16 with fp32 weights, bias and arithmetic)
 template <typename T, int KP>      // KP = channel pairs held in registers (ceil(Csrc / 2) <= KP)
-__global__ void __launch_bounds__(TB1)
+__global__ void __launch_bounds__(TB1) __attribute__((amdgpu_waves_per_eu(KP <= 16 ? 2 : 1)))
 conv111_mfma_kernel(const T* __restrict__ src, int64_t lds, int Csrc, const float* __restrict__ w, int so, int sc,
                     const float* __restrict__ bias, T* __restrict__ dst, int64_t ldd, int Cdst, int64_t begin,
                     int64_t end, int relu) {
     const int lane = threadIdx.x & 63, hi = lane >> 5, col = lane & 31;
     const int o0 = blockIdx.y * 32;
+    // weights and bias: all loads first, from clamped places, masked afterwards (a load under a per-lane branch is
+    // waited for on the spot: 32 round trips in a row at the start of every block)
     float aw[KP];
+    {
+        const int o = min(o0 + col, Cdst - 1);
 #pragma unroll
-    for (int p = 0; p < KP; ++p) {
-        const int c = 2 * p + hi, o = o0 + col;
-        aw[p] = (c < Csrc && o < Cdst) ? w[(int64_t)o * so + (int64_t)c * sc] : 0.f;
+        for (int p = 0; p < KP; ++p) aw[p] = w[(int64_t)o * so + (int64_t)min(2 * p + hi, Csrc - 1) * sc];
+#pragma unroll
+        for (int p = 0; p < KP; ++p) aw[p] = (2 * p + hi < Csrc && o0 + col < Cdst) ? aw[p] : 0.f;
     }
     float bs[16];
 #pragma unroll
-    for (int r = 0; r < 16; ++r) {
-        const int o = o0 + 8 * (r >> 2) + 4 * hi + (r & 3);
-        bs[r] = (bias && o < Cdst) ? bias[o] : 0.f;
-    }
+    for (int r = 0; r < 16; ++r) bs[r] = bias ? bias[min(o0 + 8 * (r >> 2) + 4 * hi + (r & 3), Cdst - 1)] : 0.f;
     const int64_t nwave = (int64_t)gridDim.x * (TB1 / 64);
     const int64_t wave = (int64_t)blockIdx.x * (TB1 / 64) + (threadIdx.x >> 6);
     for (int64_t i0 = begin + wave * 64; i0 < end; i0 += nwave * 64) {
@@ -81,15 +82,22 @@ conv111_mfma_kernel(const T* __restrict__ src, int64_t lds, int Csrc, const floa
             // (element-aligned) pair, so a half-wave reads and writes 32 pairs in a row per channel
             typedef typename PairBits111<2 * sizeof(T)>::type B;
             const int64_t ip = i0 + 2 * col;
+            // Every channel pair is loaded, none under a branch: the channel depends on the lane's half, and before a
+            // load under a per-lane branch the compiler waits for all loads in flight, which made the channels of a
+            // block sixteen memory round trips in a row.  A pair past the last channel re-reads the last one; its
+            // weights are zero.  (One vector value each way: a struct of two elements is split into two accesses.)
+            B raw[KP];
+#pragma unroll
+            for (int p = 0; p < KP; ++p) {
+                const int c = min(2 * p + hi, Csrc - 1);
+                raw[p] = *reinterpret_cast<const B*>(src + (int64_t)c * lds + ip);
+            }
+            if constexpr (KP <= 32) __builtin_amdgcn_sched_barrier(0);      // all loads in flight before the first matrix instruction
             float va[KP], vb[KP];
 #pragma unroll
             for (int p = 0; p < KP; ++p) {
-                const int c = 2 * p + hi;
-                if (c < Csrc) {
-                    // (one vector value each way: a struct of two elements is split into two half-width accesses again)
-                    const Pair111<T> pv = __builtin_bit_cast(Pair111<T>, *reinterpret_cast<const B*>(src + (int64_t)c * lds + ip));
-                    va[p] = Num<T>::ld(pv.v[0]); vb[p] = Num<T>::ld(pv.v[1]);
-                } else { va[p] = 0.f; vb[p] = 0.f; }
+                const Pair111<T> pv = __builtin_bit_cast(Pair111<T>, raw[p]);
+                va[p] = Num<T>::ld(pv.v[0]); vb[p] = Num<T>::ld(pv.v[1]);
             }
             floatx16_111 acca, accb;
 #pragma unroll
