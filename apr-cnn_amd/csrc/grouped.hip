@@ -285,6 +285,118 @@ conv111_g8_kernel(const bf16_t* __restrict__ x, int64_t ldx, int Cin, const floa
     }
 }
 
+
+// The same operator on the bfloat16 matrix cores, for up to 128 input channels: v_mfma_f32_32x32x16_bf16 contracts
+// 16 input channels of 32 particles with 32 outputs, and its B operand -- lane l supplies channels 8 (l / 32) .. + 7
+// of particle l % 32 -- IS the 16-byte group of that particle: a lane loads group 2 kb + l / 32 and hands it to the
+// instruction untouched.  The fp32 weights are split into a bfloat16 head and a bfloat16 remainder (two instructions
+// per 16 channels, the products summed in fp32), so the result keeps the weights to 2^-16.  The vector-ALU kernel above
+// needs 2 * Cin * Cout / 64 multiply-add instructions per particle and is bound by them from 32 x 32 on; here the layer
+// streams.  A wave takes TILES tiles of 32 particles per round, all their loads in flight before the first product.
+typedef __bf16 bf16x8g __attribute__((ext_vector_type(8)));
+typedef float floatx16g __attribute__((ext_vector_type(16)));
+
+template <bool OUT_G8, int KB, int MB, int TILES>      // KB blocks of 16 input channels, MB blocks of 32 outputs per workgroup
+__global__ void __launch_bounds__(GTB) __attribute__((amdgpu_waves_per_eu(2)))
+conv111_g8_mfma_kernel(const bf16_t* __restrict__ x, int64_t ldx, int Cin, const float* __restrict__ w, int Cout,
+                       const float* __restrict__ bias, int relu, bf16_t* __restrict__ y, int64_t ldy, int64_t begin, int64_t end) {
+    const int lane = threadIdx.x & 63, hi = lane >> 5, col = lane & 31;
+    const int o0 = blockIdx.y * 32 * MB, nq = Cin / 8;
+    // A operands: lane supplies W[o0 + 32 mb + col][16 kb + 8 hi .. + 7], head and remainder
+    bf16x8g ah[MB][KB], al[MB][KB];
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+        for (int kb = 0; kb < KB; ++kb) {
+            const int o = o0 + 32 * mb + col, c0 = 16 * kb + 8 * hi;
+            float f[8];
+#pragma unroll
+            for (int j = 0; j < 8; ++j) f[j] = w[(int64_t)min(o, Cout - 1) * Cin + min(c0 + j, Cin - 1)];
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                const float v = (o < Cout && c0 + j < Cin) ? f[j] : 0.f;
+                const bf16_t h = float_to_bf16(v);
+                const bf16_t l = float_to_bf16(v - bf16_to_float(h));
+                ah[mb][kb][j] = __builtin_bit_cast(__bf16, h.bits);
+                al[mb][kb][j] = __builtin_bit_cast(__bf16, l.bits);
+            }
+        }
+    // the lane's 16 results of a 32 x 32 block are outputs 8 (r / 4) + 4 hi + r % 4 of particle col
+    float bs[MB][16];
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const int o = o0 + 32 * mb + 8 * (r >> 2) + 4 * hi + (r & 3);
+            bs[mb][r] = bias ? bias[min(o, Cout - 1)] : 0.f;
+        }
+    const int64_t nwave = (int64_t)gridDim.x * (GTB / 64);
+    const int64_t wave = (int64_t)blockIdx.x * (GTB / 64) + (threadIdx.x >> 6);
+    for (int64_t i0 = begin + wave * (32 * TILES); i0 < end; i0 += nwave * (32 * TILES)) {
+        uint4 raw[TILES][KB];
+#pragma unroll
+        for (int t = 0; t < TILES; ++t) {
+            const int64_t i = min(i0 + 32 * t + col, end - 1);          // past the end: a particle that exists, never stored
+#pragma unroll
+            for (int kb = 0; kb < KB; ++kb) raw[t][kb] = *g8_at(x, ldx, min(2 * kb + hi, nq - 1), i);     // (a group past the last: zero weights)
+        }
+        __builtin_amdgcn_sched_barrier(0);          // all loads in flight before the first matrix instruction
+#pragma unroll
+        for (int t = 0; t < TILES; ++t) {
+            const int64_t i = i0 + 32 * t + col;
+#pragma unroll
+            for (int mb = 0; mb < MB; ++mb) {
+                floatx16g acc;
+#pragma unroll
+                for (int r = 0; r < 16; ++r) acc[r] = bs[mb][r];
+#pragma unroll
+                for (int kb = 0; kb < KB; ++kb) {
+                    const bf16x8g bv = __builtin_bit_cast(bf16x8g, raw[t][kb]);
+                    acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ah[mb][kb], bv, acc, 0, 0, 0);
+                    acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(al[mb][kb], bv, acc, 0, 0, 0);
+                }
+                if (i >= end) continue;
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    const int oc = o0 + 32 * mb + 8 * g + 4 * hi;        // the lane's four channels of output group g
+                    if (oc >= Cout) continue;
+                    float v[4];
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) { v[j] = acc[4 * g + j]; if (relu) v[j] = v[j] < 0.f ? 0.f : v[j]; }
+                    if constexpr (OUT_G8) {
+                        *reinterpret_cast<uint2*>(y + (((int64_t)(oc >> 3) * ldy + i) << 3) + (oc & 4)) =
+                            make_uint2((unsigned)float_to_bf16(v[0]).bits | ((unsigned)float_to_bf16(v[1]).bits << 16),
+                                       (unsigned)float_to_bf16(v[2]).bits | ((unsigned)float_to_bf16(v[3]).bits << 16));
+                    } else {
+#pragma unroll
+                        for (int j = 0; j < 4; ++j)
+                            if (oc + j < Cout) y[(int64_t)(oc + j) * ldy + i] = float_to_bf16(v[j]);
+                    }
+                }
+            }
+        }
+    }
+}
+
+template <bool OUT_G8>
+static bool launch_conv111_g8_mfma(const bf16_t* x, int64_t ldx, int Cin, const float* w, int Cout, const float* bias, int relu,
+                                   bf16_t* y, int64_t ldy, int64_t b, int64_t e, hipStream_t st) {
+    const int kb = (Cin + 15) / 16;
+    if (kb > 8) return false;
+    const int mb = (Cout > 32 && kb <= 4) ? 2 : 1;
+    const int64_t per_block = (int64_t)(GTB / 64) * 32 * (mb == 2 ? 2 : 4);
+    dim3 grid((unsigned)std::min<int64_t>((e - b + per_block - 1) / per_block, 256 * 16), (unsigned)((Cout + 32 * mb - 1) / (32 * mb)));
+#define APRNET_C111(KB, MB, TILES) hipLaunchKernelGGL((conv111_g8_mfma_kernel<OUT_G8, KB, MB, TILES>), grid, dim3(GTB), 0, st, x, ldx, Cin, w, \
+                                                     Cout, bias, relu, y, ldy, b, e)
+    if (mb == 2) { if (kb <= 1) APRNET_C111(1, 2, 2); else if (kb <= 2) APRNET_C111(2, 2, 2); else APRNET_C111(4, 2, 2); }
+    else if (kb <= 1) APRNET_C111(1, 1, 4);
+    else if (kb <= 2) APRNET_C111(2, 1, 4);
+    else if (kb <= 4) APRNET_C111(4, 1, 4);
+    else APRNET_C111(8, 1, 4);
+#undef APRNET_C111
+    return true;
+}
+
 }  // namespace aprnet
 
 using namespace aprnet;
@@ -361,6 +473,11 @@ int aprnet_conv111_fwd_bf16g(const aprnet_plan* p, int d, const uint16_t* x, int
         dim3 grid((unsigned)((e - b + GTB - 1) / GTB), (unsigned)((Cout + 8 * C111_OG - 1) / (8 * C111_OG)));
         const size_t lds = (size_t)Cin * 8 * C111_OG * sizeof(float);
         const float* ws = w + (int64_t)s * Cout * Cin;
+        if (Cin * Cout >= 16 * 32) {      // from here on the vector-ALU kernel is bound by its multiply-adds
+            const bool done = y_grouped ? launch_conv111_g8_mfma<true>((const bf16_t*)x, ldx, Cin, ws, Cout, bias, relu, (bf16_t*)y, ldy, b, e, (hipStream_t)st)
+                                        : launch_conv111_g8_mfma<false>((const bf16_t*)x, ldx, Cin, ws, Cout, bias, relu, (bf16_t*)y, ldy, b, e, (hipStream_t)st);
+            if (done) continue;
+        }
         if (y_grouped) hipLaunchKernelGGL(conv111_g8_kernel<true>, grid, dim3(GTB), lds, (hipStream_t)st, (const bf16_t*)x, ldx, Cin, ws, Cout, bias, relu, (bf16_t*)y, ldy, b, e);
         else hipLaunchKernelGGL(conv111_g8_kernel<false>, grid, dim3(GTB), lds, (hipStream_t)st, (const bf16_t*)x, ldx, Cin, ws, Cout, bias, relu, (bf16_t*)y, ldy, b, e);
     }
