@@ -83,13 +83,19 @@ def test_first_layer_planes_in_grouped_out(cin):
     assert torch.equal(g8.ungroup(got), _ops.conv_forward(aprs, x, w, ld, bias, relu=True))
 
 
-@pytest.mark.parametrize("cin,cout,grouped_out", [(16, 8, True), (64, 32, True), (16, 3, False)])
-def test_grouped_conv111_against_oracle(cin, cout, grouped_out):
+# small layers run on the vector-ALU kernel, the others on the matrix-core kernel: whole and partial blocks of 16 input
+# channels and of 32 outputs, one and two output blocks per workgroup, 128 inputs, plane output
+@pytest.mark.parametrize("cin,cout,grouped_out,relu", [(16, 8, True, False), (64, 32, True, False), (16, 3, False, False),
+                                                       (24, 40, True, True), (32, 64, True, False), (128, 16, True, True),
+                                                       (48, 19, False, True), (8, 64, True, False)])
+def test_grouped_conv111_against_oracle(cin, cout, grouped_out, relu):
     aprs, ld, x, g = _batch(cin, seed=4)
     w = torch.randn(2, cout, cin, 1, 1, 1, generator=g) * 0.2
     bias = torch.randn(cout, generator=g)
     ref = oracle.conv_forward(aprs, x.float().cpu(), w.permute(2, 0, 1, 3, 4, 5).contiguous(), ld) + bias.view(1, -1, 1)
-    got = g8.conv111_forward(aprs, g8.regroup(x), w.to(DEV), ld, bias.to(DEV), relu=False, grouped_output=grouped_out)
+    if relu:
+        ref = ref.clamp_min(0)
+    got = g8.conv111_forward(aprs, g8.regroup(x), w.to(DEV), ld, bias.to(DEV), relu=relu, grouped_output=grouped_out)
     got = g8.ungroup(got) if grouped_out else got
     for b, a in enumerate(aprs):
         n = oracle.number_parts(a, int(ld[b]))
