@@ -238,7 +238,8 @@ __device__ __forceinline__ void mfma16_window(const ConvArgs<T>& a, int co0, int
 // FUSE: built for the fused forward entry points (second input tensor, clamp at zero)
 template <typename T, class G, int COH, int MODE, bool LISTS, bool FUSE = false>
 __global__ void __launch_bounds__(G::NT)
-__attribute__((amdgpu_waves_per_eu(LISTS ? (COH == 1 ? FWD_WAVES16 : FWD_WAVES) : DX_WAVES, LISTS ? (COH == 1 ? FWD_WAVES16 : FWD_WAVES) : DX_WAVES)))
+__attribute__((amdgpu_waves_per_eu(LISTS ? ((COH == 1 && G::NT <= 512) ? FWD_WAVES16 : FWD_WAVES) : DX_WAVES,
+                                   LISTS ? ((COH == 1 && G::NT <= 512) ? FWD_WAVES16 : FWD_WAVES) : DX_WAVES)))
 conv_mfma16_kernel(const ConvArgs<T> a) {
     constexpr int CIB = LISTS ? FWD_CIB : DX_CIB, NBW = 4;
     static_assert((G::MAXCOL + 15) / 16 <= G::NWAVE * NBW, "a window must fit the accumulators of the block");
@@ -602,7 +603,12 @@ __device__ __forceinline__ void mfma_bf16_window(const ConvArgs<bf16_t>& a, int 
 
 // The windows of the tile come as precomputed lists from the plan.
 template <class G, int COH, bool FUSE = false, int MODE = 0, bool IL = false>
-__global__ void __launch_bounds__(G::NT) __attribute__((amdgpu_waves_per_eu(4, 4)))      // two workgroups per CU
+// Two workgroups per CU (128 registers); the forward pass of layers of at most 16 outputs on regrouped input runs
+// three (80 registers, with spills): a third chain of windows per CU hides more of the memory round trips at the
+// start of every window than the spills cost (16->16 on the 23 M-particle APR 1.40 -> 1.28 ms; four workgroups at 64
+// registers: 2.39 ms; three for 32 outputs: 3.76 against 2.61 ms).
+__global__ void __launch_bounds__(G::NT)
+__attribute__((amdgpu_waves_per_eu((COH == 1 && MODE == 0 && IL) ? 6 : 4, (COH == 1 && MODE == 0 && IL) ? 6 : 4)))
 conv_mfma_bf16_kernel(const ConvArgs<bf16_t> a) {
     constexpr int NBW = 4, NSTEP = bf16_steps<G>();
     static_assert((G::MAXCOL + 15) / 16 <= G::NWAVE * NBW, "a window must fit the accumulators of the block");
