@@ -41,10 +41,9 @@ typedef float floatx4 __attribute__((ext_vector_type(4)));
 // compiled for.  Three workgroups per CU (six waves per SIMD, 80 registers) beat two with chunks of 8: the
 // third group hides more of the latency between the matrix phases than the few spilled registers cost.
 // Forward takes its window lists from the plan; the input gradient scans and keeps its lists in LDS.
+// (Layers of at most 16 outputs fit 64 registers without spilling; four workgroups per CU instead of three make the
+// plain 16->16 layer 2 % faster, 4.29 -> 4.21 ms, and the network, whose 16-output layers are the fused forms, 0.8 % slower.)
 constexpr int FWD_CIB = 4, FWD_WAVES = 6;
-// forward layers of at most 16 outputs hold half the accumulators and fit 64 registers without spilling: four
-// workgroups per CU instead of three (16->16 on the 23 M-particle APR 4.29 -> 4.21 ms)
-constexpr int FWD_WAVES16 = 8;
 constexpr int DX_CIB = 4, DX_WAVES = 6;
 constexpr int STAGE_PRIO = 3;      // wave priority outside the matrix loops
 
@@ -238,8 +237,7 @@ __device__ __forceinline__ void mfma16_window(const ConvArgs<T>& a, int co0, int
 // FUSE: built for the fused forward entry points (second input tensor, clamp at zero)
 template <typename T, class G, int COH, int MODE, bool LISTS, bool FUSE = false>
 __global__ void __launch_bounds__(G::NT)
-__attribute__((amdgpu_waves_per_eu(LISTS ? ((COH == 1 && G::NT <= 512) ? FWD_WAVES16 : FWD_WAVES) : DX_WAVES,
-                                   LISTS ? ((COH == 1 && G::NT <= 512) ? FWD_WAVES16 : FWD_WAVES) : DX_WAVES)))
+__attribute__((amdgpu_waves_per_eu(LISTS ? FWD_WAVES : DX_WAVES, LISTS ? FWD_WAVES : DX_WAVES)))
 conv_mfma16_kernel(const ConvArgs<T> a) {
     constexpr int CIB = LISTS ? FWD_CIB : DX_CIB, NBW = 4;
     static_assert((G::MAXCOL + 15) / 16 <= G::NWAVE * NBW, "a window must fit the accumulators of the block");
