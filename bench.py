@@ -522,6 +522,26 @@ def run_spots16k(args, dev, lib):
         kernel_ms = _kernel_ms(lib, lambda: conv(x, [apr], ld), 3)
     extra = {"fwd_ms": sec * 1e3, "fwd_peak_device_GB": torch.cuda.max_memory_allocated() / 1e9}
     say(f"spots16k forward: {sec * 1e3:.1f} ms per step, kernel {kernel_ms:.1f} ms")
+    # the same layer between two layers of a network that keeps its tensors grouped by eight channels: no regrouping
+    # pass per call, 8-byte output stores instead of 2-byte ones
+    try:
+        from pyapr.aprnet import _ops, grouped
+        xg8 = grouped.regroup(x)
+        levels = apr.level_max() - apr.level_min() + 1
+        with torch.no_grad():
+            gstep = lambda: grouped.conv_forward([apr], xg8, _ops.restrict_kernel_forward(conv.weight.detach(), levels), ld, conv.bias.detach())
+            gsec = _steps(gstep, steps, 1)
+            gk = _kernel_ms(lib, gstep, 3)
+        extra["fwd_grouped_ms"] = gsec * 1e3
+        extra["fwd_grouped_kernel_ms"] = gk
+        extra["fwd_grouped_frac_of_bf16_matrix_peak"] = 2 * 25 * C * C * n / (gk * 1e-3) / 1e12 / PEAK_BF16_MATRIX_TFLOPS
+        say(f"spots16k forward on grouped tensors: {gsec * 1e3:.1f} ms per step, kernel {gk:.1f} ms")
+        del xg8
+        torch.cuda.empty_cache()
+    except RuntimeError as err:                 # out of device memory, or the grouped layout's size limit
+        extra["fwd_grouped_ms"] = None
+        extra["fwd_grouped_note"] = str(err).splitlines()[0][:200]
+        torch.cuda.empty_cache()
     # the backward of the layer at full size needs the features, two gradients and an fp32 gradient work space at
     # 64 channels: run when it fits, otherwise on the 4096^2 corner of the same image
     try:
