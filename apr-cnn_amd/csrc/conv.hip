@@ -153,6 +153,7 @@ size_t conv_narrow_packed_floats(int code, int S_exp, int Cout, int Cin);
 int pack_conv_weights_narrow(int code, const float* w, int S_exp, int Cout, int Cin, float* packed, hipStream_t st);
 int launch_conv_narrow(int code, const ConvArgs<float>& a, const WinLists& wl, hipStream_t st);
 int launch_conv_narrow(int code, const ConvArgs<bf16_t>& a, const WinLists& wl, hipStream_t st);
+static std::atomic<int> g_big_addr{0};       // bfloat16 forward on grouped tensors: 1 = 64-bit addresses also where 32-bit offsets would do
 static std::atomic<int> g_narrow{1};         // layers of 1 to 3 input channels: 1 = the bandwidth-shaped kernel (conv_narrow.hip), 0 = the general one
 static std::atomic<int> g_conv_path{0};      // 0: matrix cores where available, 1: VALU kernels only
 int conv_path() { return g_conv_path; }
@@ -366,7 +367,7 @@ int conv_fwd_bf16_layout(const aprnet_plan* cp, int d, int kz, int kx, int ky, c
                          hipStream_t st, const Fusion<bf16_t>& fu) {
     aprnet_plan* p = const_cast<aprnet_plan*>(cp);
     if (int rc = check_level_delta(p, d, "conv_forward")) return rc;
-    if (int rc = check_plane_size(p, d, 16, "conv_forward")) return rc;          // 16-byte items, 32-bit offsets
+    if (int rc = check_plane_size(p, d, 2, "conv_forward")) return rc;           // the plane input of a first layer: 32-bit offsets
     const int Cin = C1 + fu.C2;
     if (C1 <= 0 || Cout <= 0 || S_exp <= 0) return fail(APRNET_ERR_INVALID_ARGUMENT, "conv_forward: empty channel / stencil count");
     const int code = kz * 100 + kx * 10 + ky;
@@ -404,6 +405,8 @@ int conv_fwd_bf16_layout(const aprnet_plan* cp, int d, int kz, int kx, int ky, c
     a.w = (const float*)p->d_scratch;
     a.xi = x; a.xi_ld = ldx; a.xi2 = fu.C2 > 0 ? fu.x2 : nullptr; a.xi2_ld = fu.ldx2; a.ti = tree_ws; a.ti_ld = ldt;
     a.x = nullptr; a.x2 = nullptr; a.tree_data = nullptr;
+    // 16-byte items: 32-bit byte offsets reach 2^28 elements of a group; beyond, the kernel takes 64-bit addresses
+    a.big = g_big_addr || a.x_count >= (1ll << 28) || a.t_count >= (1ll << 28);
     TimedLaunch timed(st);
     return launch_conv_mfma_bf16(code, a, tl.n, st);
 }
@@ -468,11 +471,13 @@ int aprnet_set_conv_path(int path) {
     if (path == 8 || path == 9) { g_bf16_regroup = path == 8; return 0; }
     if (path == 10 || path == 11) { g_bwd_deterministic = path == 10; return 0; }
     if (path == 12 || path == 13) { g_narrow = path == 12; return 0; }
+    if (path == 14 || path == 15) { g_big_addr = path == 15; return 0; }
     if (path != 0 && path != 1)
         return fail(APRNET_ERR_INVALID_ARGUMENT, "set_conv_path: 0 (auto), 1 (VALU only), 2 / 3 (bfloat16 features: bfloat16 / fp32 "
                                                  "matrix math), 4 / 5 (forward: window lists of the plan / scan per call), 6 / 7 (backward on two streams / one), "
                                                  "8 / 9 (bfloat16 forward: regrouped copy of the input / channel planes), 10 / 11 (weight gradient: "
-                                                 "fixed-order partial sums / atomic additions), 12 / 13 (1 to 3 input channels: pipelined kernel / general kernel)");
+                                                 "fixed-order partial sums / atomic additions), 12 / 13 (1 to 3 input channels: pipelined kernel / general kernel), "
+                                                 "14 / 15 (grouped bfloat16 forward: 32-bit offsets where they suffice / 64-bit addresses always)");
     g_conv_path = path;
     return 0;
 }

@@ -43,6 +43,7 @@ struct ConvArgs {
     int64_t xi_ld, ti_ld;                      // particles between two groups of xi / ti
     const T* xi2; int64_t xi2_ld;              // grouped second input: groups from c_split / 8 on (null: all groups in xi)
     int y_g8;                                  // bfloat16 forward: the output is grouped too, [Cout / 8][ldy][8]
+    int big;                                   // bfloat16 forward on grouped input: 64-bit addresses (2^28 elements and more per group)
     // backward only
     // gradients are accumulated in the computation type (fp32 for bfloat16 features)
     const T* gy; typename Num<T>::acc* gx; int64_t ldgx; typename Num<T>::acc* gtree; int64_t ldgt;

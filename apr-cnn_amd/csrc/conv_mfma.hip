@@ -379,7 +379,9 @@ typedef int intx4 __attribute__((ext_vector_type(4)));
 template <class G, int IPT>
 struct ItemRegs16 { intx4 v[IPT]; unsigned off[IPT]; unsigned short pos[IPT]; };
 
-template <class G, int IPT, class Lists>
+// BIG: tensors of 2^28 elements and more per group, whose 16-byte items lie past 32-bit byte offsets: R.off keeps the
+// element index and the loads take 64-bit addresses (a lane without an item reads element 0; its value is never stored)
+template <class G, int IPT, bool BIG = false, class Lists>
 __device__ __forceinline__ void fetch_slots16(const Lists& sh, int nitem, ItemRegs16<G, IPT>& R) {
     // unconditional buffer loads, results touched only after every round is issued (see fetch_slots)
     const __amdgpu_buffer_rsrc_t ri = __builtin_amdgcn_make_buffer_rsrc(const_cast<int*>(sh.item_idx), 0, nitem * 4, 0x00020000);
@@ -397,14 +399,25 @@ __device__ __forceinline__ void fetch_slots16(const Lists& sh, int nitem, ItemRe
     for (int k = 0; k < IPT; ++k) {
         const bool valid = (int)threadIdx.x + k * G::NT < nitem;
         R.pos[k] = valid ? (unsigned short)pos[k] : (unsigned short)0xffffu;
-        R.off[k] = valid ? (unsigned)idx[k] * 16u : BUF_OOB;
+        R.off[k] = BIG ? (valid ? (unsigned)idx[k] : 0u) : (valid ? (unsigned)idx[k] * 16u : BUF_OOB);
     }
 }
-template <class G, int IPT>
+template <class G, int IPT, bool BIG = false>
 __device__ __forceinline__ void load_values16(const ConvArgs<bf16_t>& a, int ci0, int nitem, bool tree_items, ItemRegs16<G, IPT>& R) {
     const int q = ci0 / BF_CIB;
     const int q1 = a.c_split / BF_CIB;          // groups of the first tensor when there is a second one
     const bf16_t* xg = (a.xi2 != nullptr && q >= q1) ? a.xi2 + (int64_t)(q - q1) * a.xi2_ld * BF_CIB : a.xi + (int64_t)q * a.xi_ld * BF_CIB;
+    if constexpr (BIG) {
+        const bf16_t* tg = a.ti + (int64_t)q * a.ti_ld * BF_CIB;
+#pragma unroll
+        for (int k = 0; k < IPT; ++k) {
+            if (k * G::NT >= nitem) break;                  // wave-uniform
+            const bool from_tree = tree_items && (R.pos[k] & ITEM_TREE) != 0 && R.pos[k] != 0xffffu;
+            const bf16_t* base = from_tree ? tg : xg;       // a select, not a branch
+            R.v[k] = *reinterpret_cast<const intx4*>(base + (uint64_t)R.off[k] * 8u);
+        }
+        return;
+    }
     const __amdgpu_buffer_rsrc_t rx = __builtin_amdgcn_make_buffer_rsrc(const_cast<bf16_t*>(xg), 0, (int)(a.x_count * 16), 0x00020000);
     const __amdgpu_buffer_rsrc_t rt = __builtin_amdgcn_make_buffer_rsrc(const_cast<bf16_t*>(a.ti + (int64_t)q * a.ti_ld * BF_CIB), 0,
                                                                         tree_items ? (int)(a.t_count * 16) : 0, 0x00020000);
@@ -457,7 +470,7 @@ __global__ void interleave8_kernel(const bf16_t* __restrict__ x, int64_t ldx, co
 // MODE 0: forward.  MODE 1: input gradient (items = output gradient, results added atomically in fp32 to the place
 // each column names, as in the fp32 kernel; no pooled columns).
 // IL: the input comes regrouped (a.xi, a.ti), see above
-template <class G, int COH, int NB, bool FUSE, int MODE, bool IL, class Lists>
+template <class G, int COH, int NB, bool FUSE, int MODE, bool IL, bool BIG, class Lists>
 __device__ __forceinline__ void mfma_bf16_window(const ConvArgs<bf16_t>& a, int co0, int nc, int nitem, bool tree_items, int first,
                                                  const uint4* __restrict__ wl, const Lists& sh,
                                                  uint4* __restrict__ patch16, uint4* __restrict__ Wl16,
@@ -514,13 +527,13 @@ __device__ __forceinline__ void mfma_bf16_window(const ConvArgs<bf16_t>& a, int 
         if (i < W16) reinterpret_cast<intx4w*>(Wl16)[i] = wr[k];                                   \
     }
     if constexpr (IL) {
-        fetch_slots16<G>(sh, nitem, R);
+        fetch_slots16<G, ItemRegs<G, bf16_t, BF_CIB>::IPT, BIG>(sh, nitem, R);
 #pragma unroll
         for (int j = 0; j < NB; ++j) {
             const int col = ((first + G::NWAVE * j) << 4) + (lane & 15);
             bbase[j] = col < nc ? (bbase[j] & (int)COL_CELL) - G::TAP0 : 0;
         }
-        load_values16<G>(a, 0, nitem, tree_items, R);
+        load_values16<G, ItemRegs<G, bf16_t, BF_CIB>::IPT, BIG>(a, 0, nitem, tree_items, R);
     } else load_items<G, bf16_t, BF_CIB>(a, 0, nitem, tree_items, sh, R, 0, std::bool_constant<FUSE>{});
     APRNET_LOAD_WEIGHTS(0)
     for (int i = threadIdx.x; i < G::CH_STRIDE; i += G::NT) patch16[i] = make_uint4(0u, 0u, 0u, 0u);     // once per window
@@ -531,7 +544,7 @@ __device__ __forceinline__ void mfma_bf16_window(const ConvArgs<bf16_t>& a, int 
         APRNET_STORE_WEIGHTS()
         __syncthreads();
         if (ci0 + BF_CIB < a.Cin) {
-            if constexpr (IL) load_values16<G>(a, ci0 + BF_CIB, nitem, tree_items, R);
+            if constexpr (IL) load_values16<G, ItemRegs<G, bf16_t, BF_CIB>::IPT, BIG>(a, ci0 + BF_CIB, nitem, tree_items, R);
             else load_values<G, bf16_t, BF_CIB>(a, ci0 + BF_CIB, nitem, tree_items, R, 0, std::bool_constant<FUSE>{});
             APRNET_LOAD_WEIGHTS(ci0 / BF_CIB + 1)
         }
@@ -600,11 +613,11 @@ __device__ __forceinline__ void mfma_bf16_window(const ConvArgs<bf16_t>& a, int 
 }
 
 // The windows of the tile come as precomputed lists from the plan.
-template <class G, int COH, bool FUSE = false, int MODE = 0, bool IL = false>
 // Two workgroups per CU (128 registers); the forward pass of layers of at most 16 outputs on regrouped input runs
 // three (80 registers, with spills): a third chain of windows per CU hides more of the memory round trips at the
 // start of every window than the spills cost (16->16 on the 23 M-particle APR 1.40 -> 1.28 ms; four workgroups at 64
 // registers: 2.39 ms; three for 32 outputs: 3.76 against 2.61 ms).
+template <class G, int COH, bool FUSE = false, int MODE = 0, bool IL = false, bool BIG = false>
 __global__ void __launch_bounds__(G::NT)
 __attribute__((amdgpu_waves_per_eu((COH == 1 && MODE == 0 && IL) ? 6 : 4, (COH == 1 && MODE == 0 && IL) ? 6 : 4)))
 conv_mfma_bf16_kernel(const ConvArgs<bf16_t> a) {
@@ -644,11 +657,11 @@ conv_mfma_bf16_kernel(const ConvArgs<bf16_t> a) {
         const int first = (wave - (int)blockIdx.x - win) & (G::NWAVE - 1);
         const int nb = first < nblk ? (nblk - first + G::NWAVE - 1) / G::NWAVE : 0;
         switch (__builtin_amdgcn_readfirstlane(nb)) {
-            case 0: mfma_bf16_window<G, COH, 0, FUSE, MODE, IL>(a, co0, nc, nitem, tree_items, first, wl, gl, patch16, Wl16, bias_l); break;
-            case 1: mfma_bf16_window<G, COH, 1, FUSE, MODE, IL>(a, co0, nc, nitem, tree_items, first, wl, gl, patch16, Wl16, bias_l); break;
-            case 2: mfma_bf16_window<G, COH, 2, FUSE, MODE, IL>(a, co0, nc, nitem, tree_items, first, wl, gl, patch16, Wl16, bias_l); break;
-            case 3: mfma_bf16_window<G, COH, 3, FUSE, MODE, IL>(a, co0, nc, nitem, tree_items, first, wl, gl, patch16, Wl16, bias_l); break;
-            default: mfma_bf16_window<G, COH, 4, FUSE, MODE, IL>(a, co0, nc, nitem, tree_items, first, wl, gl, patch16, Wl16, bias_l); break;
+            case 0: mfma_bf16_window<G, COH, 0, FUSE, MODE, IL, BIG>(a, co0, nc, nitem, tree_items, first, wl, gl, patch16, Wl16, bias_l); break;
+            case 1: mfma_bf16_window<G, COH, 1, FUSE, MODE, IL, BIG>(a, co0, nc, nitem, tree_items, first, wl, gl, patch16, Wl16, bias_l); break;
+            case 2: mfma_bf16_window<G, COH, 2, FUSE, MODE, IL, BIG>(a, co0, nc, nitem, tree_items, first, wl, gl, patch16, Wl16, bias_l); break;
+            case 3: mfma_bf16_window<G, COH, 3, FUSE, MODE, IL, BIG>(a, co0, nc, nitem, tree_items, first, wl, gl, patch16, Wl16, bias_l); break;
+            default: mfma_bf16_window<G, COH, 4, FUSE, MODE, IL, BIG>(a, co0, nc, nitem, tree_items, first, wl, gl, patch16, Wl16, bias_l); break;
         }
         __syncthreads();        // the next window rewrites the patch
     }
@@ -714,6 +727,12 @@ static int launch_bf16(const ConvArgs<bf16_t>& a, int n_tiles, hipStream_t st, b
     } else if (dx) {
         if (coh == 1) hipLaunchKernelGGL((conv_mfma_bf16_kernel<G, 1, false, 1>), grid, dim3(G::NT), 0, st, a);
         else hipLaunchKernelGGL((conv_mfma_bf16_kernel<G, 2, false, 1>), grid, dim3(G::NT), 0, st, a);
+    } else if (a.xi != nullptr && a.big) {   // regrouped input of 2^28 elements and more per group: 64-bit addresses
+        if (a.relu) {
+            if (coh == 1) hipLaunchKernelGGL((conv_mfma_bf16_kernel<G, 1, true, 0, true, true>), grid, dim3(G::NT), 0, st, a);
+            else hipLaunchKernelGGL((conv_mfma_bf16_kernel<G, 2, true, 0, true, true>), grid, dim3(G::NT), 0, st, a);
+        } else if (coh == 1) hipLaunchKernelGGL((conv_mfma_bf16_kernel<G, 1, false, 0, true, true>), grid, dim3(G::NT), 0, st, a);
+        else hipLaunchKernelGGL((conv_mfma_bf16_kernel<G, 2, false, 0, true, true>), grid, dim3(G::NT), 0, st, a);
     } else if (a.xi != nullptr) {          // regrouped input (the second tensor is already part of it)
         if (a.relu) {
             if (coh == 1) hipLaunchKernelGGL((conv_mfma_bf16_kernel<G, 1, true, 0, true>), grid, dim3(G::NT), 0, st, a);

@@ -3,7 +3,7 @@ keeps between its layers on the GPU (no counterpart in the reference, whose tens
 conv.hpp:68).  A particle's eight channels are one 16-byte word: the convolution stages straight from its input
 instead of from a regrouped copy, pool / upsample / tree fill move 16 bytes per access, and every result is
 bit-identical to the plane operators'.  Inference only (no autograd), channel counts multiples of eight, at most
-2^28 - 1 particles per APR."""
+2^31 - 1 particles per APR (from 2^28 on the convolution addresses its items with 64 bits instead of 32-bit offsets)."""
 import ctypes as C
 
 import torch
@@ -11,7 +11,7 @@ import torch
 from . import _ops
 from ._ops import _check_input, _deltas, _lib, _plans, _ptr, _raise, _stream, number_particles, tree_parts
 
-MAX_PARTICLES = (1 << 28) - 1
+MAX_PARTICLES = (1 << 31) - 1
 
 
 class Grouped:

@@ -105,7 +105,9 @@ int aprnet_profile_enable(int on);
  * kernels: 10 = every workgroup writes the sums of its tiles to its own slots of the plan's scratch buffer and a second
  * kernel adds the slots in a fixed order (default: the gradient repeats bit for bit from run to run; at most 512 MiB
  * of scratch), 11 = atomic additions; and for forward layers of 1 to 3 input channels (bound by memory, not by the
- * contraction): 12 = the pipelined kernel with the (tap, channel) axis flattened (default), 13 = the general kernel.
+ * contraction): 12 = the pipelined kernel with the (tap, channel) axis flattened (default), 13 = the general kernel;
+ * and for the bfloat16 forward kernel on grouped tensors: 14 = 32-bit byte offsets where a group holds fewer than 2^28
+ * elements, 64-bit addresses beyond (default), 15 = 64-bit addresses always.
  * All are HIP kernels; the switch
  * exists so that tests can cover them and memory-bound callers can do without the lists. */
 int aprnet_set_conv_path(int path);

@@ -73,6 +73,28 @@ def test_grouped_convolution_equals_the_plane_kernel(c1, c2, cout, ksize):
     assert torch.equal(planes, _ops.conv_forward(aprs, xa, w, ld, bias, x2=xb))
 
 
+@pytest.mark.parametrize("c1,c2,cout", [(16, 0, 16), (8, 24, 40)])
+def test_grouped_convolution_with_64_bit_addresses(c1, c2, cout):
+    """Tensors of 2^28 particles and more make the kernel address its 16-byte items with 64 bits instead of 32-bit
+    byte offsets; forced here on a small batch (tiles with and without tree items, a second input, lanes without an
+    item): bit-identical to the default."""
+    aprs, ld, x, g = _batch(c1 + c2, seed=6)
+    levels = max(a.level_max() - a.level_min() + 1 for a in aprs)
+    w = (torch.randn(levels, cout, c1 + c2, 3, 3, 3, generator=g) * 0.1).to(DEV)
+    bias = torch.randn(cout, generator=g).to(DEV)
+    xa, xb = g8.regroup(x[:, :c1].contiguous()), (g8.regroup(x[:, c1:].contiguous()) if c2 else None)
+    ref = g8.conv_forward(aprs, xa, w, ld, bias, relu=True, x2=xb)
+    lib = _native.hip()
+    assert lib.aprnet_set_conv_path(15) == 0
+    try:
+        got = g8.conv_forward(aprs, xa, w, ld, bias, relu=True, x2=xb)
+        planes = g8.conv_forward(aprs, xa, w, ld, bias, relu=False, x2=xb, grouped_output=False)
+    finally:
+        assert lib.aprnet_set_conv_path(14) == 0
+    assert torch.equal(got.data, ref.data)
+    assert torch.equal(planes, g8.conv_forward(aprs, xa, w, ld, bias, relu=False, x2=xb, grouped_output=False))
+
+
 @pytest.mark.parametrize("cin", [1, 3])
 def test_first_layer_planes_in_grouped_out(cin):
     aprs, ld, x, g = _batch(cin, seed=3)
