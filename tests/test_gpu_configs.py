@@ -201,6 +201,31 @@ def test_nuclei1024_unet_on_the_quarter_scale_replica_properties():
     assert _rel(yb.float(), y1) <= 2e-2
 
 
+def test_nuclei1024_whole_volume_grouped_path_against_plane_path():
+    """The whole 1024^3 volume (844 M particles): with bfloat16 features the network keeps its tensors grouped by eight
+    channels, and from 2^28 particles on the convolution addresses its 16-byte items with 64 bits.  Checked against the
+    plane path of the same build over the whole particle range (the two differ in the summation order and the weight
+    rounding of the 1x1x1 convolutions: 2e-2 of the output scale, as for the small replicas)."""
+    if torch.cuda.get_device_properties(0).total_memory < 200e9:
+        pytest.skip("needs about 100 GB of device memory")
+    apr, parts = make_config("nuclei1024")
+    n = apr.total_number_particles()
+    assert n >= (1 << 28)
+    x = (torch.from_numpy(parts).float() / 1000.0).view(1, 1, -1).to(DEV).to(torch.bfloat16)
+    model = _unet().to(DEV)
+    with torch.no_grad():
+        model.use_grouped = True
+        yg = model(x, [apr])
+        model.use_grouped = False
+        yp = model(x, [apr])
+    assert yg.shape == (1, 3, n) and yg.dtype == torch.bfloat16
+    scale = float(yp.float().abs().max())
+    assert scale > 0 and torch.isfinite(yg.float()).all()
+    step = 1 << 26
+    worst = max(float((yg[:, :, lo:lo + step].float() - yp[:, :, lo:lo + step].float()).abs().max()) for lo in range(0, n, step))
+    assert worst <= 2e-2 * scale
+
+
 # ------------------------------------------------------------------------------------------------ configs[4]
 def test_spots16k_small_replica_against_oracle():
     """APRConv 1x5x5 64 -> 64 with bfloat16 features on the 256^2 replica of configs[4] (59 k particles): forward,
