@@ -274,7 +274,8 @@ int aprnet_upsample_bwd_bf16(const aprnet_plan*, int level_delta, const uint16_t
  * hands grouped tensors from layer to layer converts at its two ends only; the convolution then stages straight from
  * its input (no regrouping pass per call) and stores 8 bytes per lane instead of four 2-byte values.  Results are
  * bit-identical to the plane entry points (same arithmetic, same summation order).  C, Cin and Cout of grouped
- * tensors are multiples of 8; ld counts particles between two groups; at most 2^28 - 1 particles.
+ * tensors are multiples of 8; ld counts particles between two groups; at most 2^31 - 1 particles (from 2^28 on the
+ * convolution addresses its 16-byte items with 64 bits instead of 32-bit byte offsets).
  *   regroup8 / ungroup8     planes [C][ldx] <-> groups [C / 8][ldo][8] (channels past C read as zeros)
  *   fill_tree_mean_bf16g    helpers::fill_tree_mean on grouped features, tree [C / 8][ld_tree][8]
  *   maxpool_fwd_bf16g       MaxPool::forward, values only (the argmax serves the backward pass)
