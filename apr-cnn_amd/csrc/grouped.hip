@@ -473,7 +473,7 @@ int aprnet_conv111_fwd_bf16g(const aprnet_plan* p, int d, const uint16_t* x, int
         dim3 grid((unsigned)((e - b + GTB - 1) / GTB), (unsigned)((Cout + 8 * C111_OG - 1) / (8 * C111_OG)));
         const size_t lds = (size_t)Cin * 8 * C111_OG * sizeof(float);
         const float* ws = w + (int64_t)s * Cout * Cin;
-        if (Cin * Cout >= 16 * 32) {      // from here on the vector-ALU kernel is bound by its multiply-adds
+        if (Cin >= 16) {      // also the head of a network (16 -> 3, plane output): it streams its input like the wide layers
             const bool done = y_grouped ? launch_conv111_g8_mfma<true>((const bf16_t*)x, ldx, Cin, ws, Cout, bias, relu, (bf16_t*)y, ldy, b, e, (hipStream_t)st)
                                         : launch_conv111_g8_mfma<false>((const bf16_t*)x, ldx, Cin, ws, Cout, bias, relu, (bf16_t*)y, ldy, b, e, (hipStream_t)st);
             if (done) continue;

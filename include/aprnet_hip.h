@@ -281,7 +281,7 @@ int aprnet_upsample_bwd_bf16(const aprnet_plan*, int level_delta, const uint16_t
  *   maxpool_fwd_bf16g       MaxPool::forward, values only (the argmax serves the backward pass)
  *   upsample_fwd_bf16g      UpSampleConst::forward
  *   conv111_fwd_bf16g       Convolution<1,1,1>::forward with bias and optional ReLU; y grouped (y_grouped != 0) or planes
- *                           (the head of a network); at most 256 inputs.  Layers of 16 x 32 channels and more, up to 128
+ *                           (the head of a network); at most 256 inputs.  Layers of 16 to 128
  *                           inputs, multiply on the bfloat16 matrix cores with each fp32 weight split into a bfloat16
  *                           head and remainder (weights kept to 2^-16, sums in fp32); smaller layers multiply in fp32
  *   conv_fwd_fused_bf16l    aprnet_conv_fwd_fused_bf16 with a layout per tensor: x (and fusion->x2) grouped, or planes
