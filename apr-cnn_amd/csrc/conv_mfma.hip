@@ -89,12 +89,22 @@ __device__ __forceinline__ void mfma16_window(const ConvArgs<T>& a, int co0, int
     const int lane = lane_id();
     constexpr int NBA = NB > 0 ? NB : 1;
     int bbase[NBA];
+    constexpr bool LISTED = std::is_same<Lists, WindowLists>::value;
 #pragma unroll
     for (int j = 0; j < NB; ++j) {
         const int col = ((first + G::NWAVE * j) << 4) + (lane & 15);
-        const unsigned cp = col < nc ? (unsigned)sh.col_pos[col] : (unsigned)G::TAP0;
-        // pooled columns of the input gradient read the box-summed patch that follows the patch in LDS
-        bbase[j] = (int)(cp & COL_CELL) - G::TAP0 + (lane >> 4) * G::CH_STRIDE + ((MODE == 1 && (cp & COL_BOX)) ? CIB * G::CH_STRIDE : 0);
+        unsigned cp;
+        if constexpr (LISTED) {
+            // lists in global memory: an unconditional load (columns past the end read zero), so that it travels with the
+            // slot loads below instead of being waited for on the spot, as a load under `col < nc` is
+            const __amdgpu_buffer_rsrc_t rcp = __builtin_amdgcn_make_buffer_rsrc(const_cast<unsigned short*>(sh.col_pos), 0, nc * 2, 0x00020000);
+            cp = (unsigned)__builtin_amdgcn_raw_buffer_load_b16(rcp, col * 2, 0, 0) & 0xffffu;
+            bbase[j] = (int)cp;
+        } else {
+            cp = col < nc ? (unsigned)sh.col_pos[col] : (unsigned)G::TAP0;
+            // pooled columns of the input gradient read the box-summed patch that follows the patch in LDS
+            bbase[j] = (int)(cp & COL_CELL) - G::TAP0 + (lane >> 4) * G::CH_STRIDE + ((MODE == 1 && (cp & COL_BOX)) ? CIB * G::CH_STRIDE : 0);
+        }
     }
     floatx4 acc[NBA][COH];
 #pragma unroll
@@ -134,6 +144,14 @@ __device__ __forceinline__ void mfma16_window(const ConvArgs<T>& a, int co0, int
     // vector instructions are not queued behind the other workgroups' matrix loops (15.0 -> 14.8 ms).
     __builtin_amdgcn_s_setprio(STAGE_PRIO);
     load_items<G, T, CIB>(a, 0, nitem, tree_items, sh, R, 0, std::bool_constant<FUSE>{});
+    if constexpr (LISTED) {
+#pragma unroll
+        for (int j = 0; j < NB; ++j) {
+            const int col = ((first + G::NWAVE * j) << 4) + (lane & 15);
+            const unsigned cp = col < nc ? (unsigned)bbase[j] : (unsigned)G::TAP0;
+            bbase[j] = (int)(cp & COL_CELL) - G::TAP0 + (lane >> 4) * G::CH_STRIDE + ((MODE == 1 && (cp & COL_BOX)) ? CIB * G::CH_STRIDE : 0);
+        }
+    }
     APRNET_LOAD_WEIGHTS(0)
     for (int i = threadIdx.x; i < CIB * G::CH_STRIDE; i += G::NT) patch[i] = 0.f;     // once per window
     for (int ci0 = 0; ci0 < a.Cin; ci0 += CIB) {
@@ -278,12 +296,18 @@ conv_mfma16_kernel(const ConvArgs<T> a) {
 
     if constexpr (LISTS) {
         (void)z0; (void)x0; (void)yn; (void)out_tree;
+        __shared__ int4 hdr[16];              // headers of sixteen windows: one round trip instead of one per window
         const int wb = a.tile_win[blockIdx.x], we = a.tile_win[blockIdx.x + 1];
         for (int w = wb; w < we; ++w) {
             const int win = w - wb;
-            const int4 hd = a.win[w];
+            if ((win & 15) == 0) {            // every wave is past the previous window's last barrier
+                if (threadIdx.x < 16 && w + (int)threadIdx.x < we) hdr[threadIdx.x] = a.win[w + threadIdx.x];
+                __syncthreads();
+            }
+            const int4 hd = hdr[win & 15];
             const int nitem = __builtin_amdgcn_readfirstlane(hd.y), nc = __builtin_amdgcn_readfirstlane(hd.w);
-            const WindowLists gl{a.l_item_idx + (unsigned)hd.x, a.l_item_pos + (unsigned)hd.x, a.l_col_idx + (unsigned)hd.z, a.l_col_pos + (unsigned)hd.z};
+            const unsigned i0 = (unsigned)__builtin_amdgcn_readfirstlane(hd.x), c0 = (unsigned)__builtin_amdgcn_readfirstlane(hd.z);
+            const WindowLists gl{a.l_item_idx + i0, a.l_item_pos + i0, a.l_col_idx + c0, a.l_col_pos + c0};
             APRNET_WINDOW(gl)
             __syncthreads();        // the next window rewrites the patch
         }
