@@ -62,12 +62,23 @@ class APRUNet(nn.Module):
         from pyapr.aprnet import _ops
         levels = max(a.level_max() - a.level_min() + 1 for a in aprs)
 
+        def restricted(weight):
+            # the stencils of the coarser levels (restrict_kernel) change only when the weights do: kept per parameter
+            # and version of its storage, so that inference does not recompute them in every forward pass
+            key = (weight.data_ptr(), weight._version, levels, weight.dtype)
+            cache = self.__dict__.setdefault("_restricted_weights", {})
+            hit = cache.get(id(weight))
+            if hit is None or hit[0] != key:
+                hit = (key, _ops.restrict_kernel_forward(weight.detach().float().contiguous(), levels))
+                cache[id(weight)] = hit
+            return hit[1]
+
         def conv(bb, inp, second=None):
             w = bb.conv.weight.detach().float()
             bias = None if bb.conv.bias is None else bb.conv.bias.detach()
             if tuple(w.shape[3:]) == (1, 1, 1):
                 return g8.conv111_forward(aprs, inp, w, level_deltas, bias, relu=True)
-            return g8.conv_forward(aprs, inp, _ops.restrict_kernel_forward(w.contiguous(), levels), level_deltas, bias, relu=True, x2=second)
+            return g8.conv_forward(aprs, inp, restricted(bb.conv.weight), level_deltas, bias, relu=True, x2=second)
 
         def block(cb, inp, second=None):
             for i, bb in enumerate(cb.blocks):

@@ -146,3 +146,21 @@ def test_unet_grouped_forward_against_oracle_and_plane_path():
     scale = float(ref.abs().max())
     assert float((got.float().cpu() - ref).abs().max()) <= 2e-2 * scale
     assert float((got.float() - planes.float()).abs().max()) <= 1e-2 * scale
+
+
+def test_unet_grouped_forward_follows_weight_updates():
+    """The grouped forward keeps the restricted stencils of a layer until its weights change: an in-place update of a
+    weight tensor must show in the next forward pass."""
+    from bench import make_unet
+    apr = apr_cases.random_apr((20, 24, 22), 3, density=0.05)
+    x = torch.randn(1, 1, apr.total_number_particles(), generator=torch.Generator().manual_seed(7)).to(torch.bfloat16).to(DEV)
+    model = make_unet(DEV)
+    with torch.no_grad():
+        y0 = model(x, [apr]).clone()
+        assert torch.equal(model(x, [apr]), y0)
+        w = model.encoder[0].blocks[0].conv.weight
+        w.mul_(0.5)
+        y1 = model(x, [apr])
+        assert not torch.equal(y1, y0)
+        w.mul_(2.0)
+        assert torch.equal(model(x, [apr]), y0)
