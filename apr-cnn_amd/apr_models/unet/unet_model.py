@@ -45,40 +45,96 @@ class APRUNet(nn.Module):
 
     def _grouped_ok(self, x, aprs):
         """Inference with bfloat16 features and every norm folded away runs on tensors grouped by eight channels
-        (pyapr.aprnet.grouped): same arithmetic as the plane operators, no regrouping pass per convolution."""
+        (pyapr.aprnet.grouped): same arithmetic as the plane operators, no regrouping pass per convolution.
+        Checked before any layer runs: element type, the channel limits of the grouped kernels, and that no
+        submodule carries hooks or non-default level-delta flags (the grouped path calls the operators directly, so
+        hooks on the submodules would not fire); anything else takes the module path."""
         from pyapr.aprnet import grouped
-        if torch.is_grad_enabled() or not x.is_cuda or x.dtype != torch.bfloat16 or x.size(1) > 3 or not self.use_grouped:
+        if torch.is_grad_enabled() or not x.is_cuda or x.dtype != torch.bfloat16 or x.size(1) > 3 \
+                or not getattr(self, "use_grouped", True):
             return False
         blocks = [b for m in self.modules() if isinstance(m, ConvBlock) for b in m.blocks] + [st.reduce_ch for st in self.decoder]
+        limits = grouped.limits()
         for b in blocks:
             if not isinstance(b.norm, nn.Identity) or type(b.activation) is not nn.ReLU:
                 return False
-            if tuple(b.conv.weight.shape[3:]) not in ((3, 3, 3), (1, 3, 3), (1, 5, 5), (1, 1, 1)) or b.conv.weight.shape[1] % 8:
+            s_, cout, cin = b.conv.weight.shape[:3]
+            ks = tuple(b.conv.weight.shape[3:])
+            if ks not in ((3, 3, 3), (1, 3, 3), (1, 5, 5), (1, 1, 1)) or cout % 8:
+                return False
+            if ks == (1, 1, 1) and (cin % 8 or cin > limits["conv111_max_cin"]):
+                return False
+            if ks != (1, 1, 1) and cin > 3 and cin % 8:
+                return False
+        hw = self.head.weight
+        if tuple(hw.shape[3:]) != (1, 1, 1) or hw.shape[2] % 8 or hw.shape[2] > limits["conv111_max_cin"]:
+            return False
+        for m in self.modules():
+            if m is self:
+                continue
+            if m._forward_hooks or m._forward_pre_hooks or m._backward_hooks:
+                return False
+            if getattr(m, "increment_level_deltas", True) is not True or getattr(m, "decrement_level_deltas", True) is not True:
                 return False
         return grouped.supported(aprs, [])
+
+    def prepare_inference(self, aprs=None, levels=None):
+        """Builds the restricted stencils (restrict_kernel) of every stencil convolution once and keeps them on the
+        convolution modules, so that the grouped inference path does not recompute them in every forward pass.
+        ``levels``: number of APR levels the stencils are expanded to (default: taken from ``aprs``).  The kept
+        stencils are dropped by ``train()``, ``load_state_dict()``, ``.to()`` / ``.float()`` ... and
+        ``invalidate_inference_cache()``; call the latter after writing weights in a way autograd does not see
+        (``weight.data.copy_()``, EMA swaps).  Without this call every forward pass restricts its stencils anew."""
+        from pyapr.aprnet import _ops
+        if levels is None:
+            if aprs is None:
+                raise ValueError("prepare_inference needs the APRs or the number of levels")
+            levels = max(a.level_max() - a.level_min() + 1 for a in aprs)
+        self.invalidate_inference_cache()
+        with torch.no_grad():
+            for m in self.modules():
+                if isinstance(m, aprnet.APRConv) and tuple(m.weight.shape[3:]) != (1, 1, 1) and m.weight.is_cuda:
+                    m._inference_stencils = (int(levels), _ops.restrict_kernel_forward(m.weight.detach().float().contiguous(), int(levels)))
+        return self
+
+    def invalidate_inference_cache(self):
+        for m in self.modules():
+            if hasattr(m, "_inference_stencils"):
+                del m._inference_stencils
+        return self
+
+    def train(self, mode=True):
+        if mode:
+            self.invalidate_inference_cache()
+        return super().train(mode)
+
+    def load_state_dict(self, *args, **kwargs):
+        self.invalidate_inference_cache()
+        return super().load_state_dict(*args, **kwargs)
+
+    def _apply(self, fn, *args, **kwargs):
+        self.invalidate_inference_cache()
+        return super()._apply(fn, *args, **kwargs)
 
     def _forward_grouped(self, x, aprs, level_deltas):
         from pyapr.aprnet import grouped as g8
         from pyapr.aprnet import _ops
         levels = max(a.level_max() - a.level_min() + 1 for a in aprs)
 
-        def restricted(weight):
-            # the stencils of the coarser levels (restrict_kernel) change only when the weights do: kept per parameter
-            # and version of its storage, so that inference does not recompute them in every forward pass
-            key = (weight.data_ptr(), weight._version, levels, weight.dtype)
-            cache = self.__dict__.setdefault("_restricted_weights", {})
-            hit = cache.get(id(weight))
-            if hit is None or hit[0] != key:
-                hit = (key, _ops.restrict_kernel_forward(weight.detach().float().contiguous(), levels))
-                cache[id(weight)] = hit
-            return hit[1]
+        def restricted(conv_module):
+            # stencils of the coarser levels: taken from prepare_inference() when it ran for this number of levels,
+            # otherwise computed here (never cached implicitly: a write through weight.data would go unnoticed)
+            kept = getattr(conv_module, "_inference_stencils", None)
+            if kept is not None and kept[0] == levels:
+                return kept[1]
+            return _ops.restrict_kernel_forward(conv_module.weight.detach().float().contiguous(), levels)
 
         def conv(bb, inp, second=None):
             w = bb.conv.weight.detach().float()
             bias = None if bb.conv.bias is None else bb.conv.bias.detach()
             if tuple(w.shape[3:]) == (1, 1, 1):
                 return g8.conv111_forward(aprs, inp, w, level_deltas, bias, relu=True)
-            return g8.conv_forward(aprs, inp, restricted(bb.conv.weight), level_deltas, bias, relu=True, x2=second)
+            return g8.conv_forward(aprs, inp, restricted(bb.conv), level_deltas, bias, relu=True, x2=second)
 
         def block(cb, inp, second=None):
             for i, bb in enumerate(cb.blocks):
@@ -110,7 +166,14 @@ class APRUNet(nn.Module):
         if level_deltas is None:
             level_deltas = torch.zeros(len(aprs), dtype=torch.int32, device=torch.device("cpu"))
         if self._grouped_ok(x, aprs):
-            return self._forward_grouped(x, aprs, level_deltas)
+            from pyapr.aprnet._ops import UnsupportedError
+            saved = level_deltas.clone()
+            try:
+                return self._forward_grouped(x, aprs, level_deltas)
+            except UnsupportedError:
+                # a limit of the grouped kernels that _grouped_ok cannot see (the plan's window lists could not be
+                # built, or were switched off): the plane operators compute the same network
+                level_deltas.copy_(saved)
         skips = [self.encoder[0](x, aprs, level_deltas)]
         for stage in self.encoder[1:]:
             skips.append(stage(skips[-1], aprs, level_deltas))

@@ -111,8 +111,12 @@ struct aprnet_plan {
     void* d_scratch = nullptr; size_t scratch_bytes = 0;          // re-laid-out weights of the call in flight
     bool scratch_in_graph = false;                                // the buffer was handed out while its stream was capturing
     std::vector<void*> retired;                                   // outgrown buffers that a captured graph may address: freed at destroy
-    hipStream_t scratch_stream = nullptr;                         // stream of the last call that used the buffer
-    bool scratch_stream_valid = false, scratch_stream_capturing = false;
+    // Hand-over of the buffer between streams: the last call that used it recorded ev_scratch behind its kernels, and a
+    // call on another stream waits for that event on the device (no host synchronisation).  scratch_stream is kept for
+    // comparison only; it is never passed to a HIP call, so the stream it named may have been destroyed since.
+    hipStream_t scratch_stream = nullptr;
+    hipEvent_t ev_scratch = nullptr;
+    bool scratch_stream_valid = false, scratch_event_recorded = false;
     std::map<std::pair<int, int>, aprnet::WinLists> lists;        // (level_delta, stencil code) -> window lists
     std::map<std::pair<int, int>, aprnet::FaceLists> faces;       // (level_delta, stencil code) -> far-face particles
     // second stream of the convolution backward (weight gradient next to input gradient), with its fork / join events
@@ -149,6 +153,23 @@ void free_face_lists(FaceLists& fl);
 // another stream than the previous one first waits for that stream, so that two streams cannot overwrite each other's
 // packed weights (under capture the caller must have ordered the streams, as for any input of the graph).
 int plan_scratch(aprnet_plan* plan, size_t bytes, hipStream_t st);
+// Records "this call is done with the scratch buffer" on `st` (after the last kernel that reads it was launched).
+void plan_scratch_done(aprnet_plan* plan, hipStream_t st);
+// A call's hold on the scratch buffer: acquire() is plan_scratch(); the destructor records the hand-over event, on every
+// way out of the call.  Declare it before anything that enqueues work at scope exit (the side-stream join), so that
+// its destructor runs last.
+struct ScratchLease {
+    aprnet_plan* plan = nullptr; hipStream_t st = nullptr;
+    int acquire(aprnet_plan* p, size_t bytes, hipStream_t s) {
+        const int rc = plan_scratch(p, bytes, s);
+        if (!rc) { plan = p; st = s; }
+        return rc;
+    }
+    ~ScratchLease() { if (plan) plan_scratch_done(plan, st); }
+    ScratchLease() = default;
+    ScratchLease(const ScratchLease&) = delete;
+    ScratchLease& operator=(const ScratchLease&) = delete;
+};
 
 #define APRNET_HIP_CHECK(expr)                                                                                  \
     do {                                                                                                        \
@@ -168,6 +189,15 @@ int plan_scratch(aprnet_plan* plan, size_t bytes, hipStream_t st);
 inline int check_plane_size(const aprnet_plan* p, int d, size_t elem, const char* who) {
     if ((uint64_t)p->number_parts(d) * elem >= (1ull << 32) || (uint64_t)p->tree_parts(d) * elem >= (1ull << 32))
         return fail(APRNET_ERR_UNSUPPORTED, std::string(who) + ": a channel plane of this element size exceeds 4 GiB");
+    return 0;
+}
+
+// a channel plane (or group) must hold at least the `need` elements the kernels address: a shorter row would turn into
+// an out-of-range device access instead of an error code
+inline int check_rows(int64_t ld, int64_t need, const char* who, const char* what) {
+    if (ld < need)
+        return fail(APRNET_ERR_INVALID_ARGUMENT, std::string(who) + ": " + what + " holds " + std::to_string(ld) +
+                    " elements per channel, the APR has " + std::to_string(need) + " at this level delta");
     return 0;
 }
 

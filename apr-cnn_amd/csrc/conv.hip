@@ -138,8 +138,8 @@ bool conv_mfma_supported(int code);
 int launch_conv_mfma(int code, const ConvArgs<float>& a, int n_tiles, hipStream_t st);
 int launch_conv_mfma(int code, const ConvArgs<bf16_t>& a, int n_tiles, hipStream_t st);
 int launch_conv_mfma_bf16(int code, const ConvArgs<bf16_t>& a, int n_tiles, hipStream_t st);
-size_t conv_packed_bf16_bytes(int code, int S_exp, int Cout, int Cin);
-int pack_conv_weights_bf16(int code, const float* w, int S_exp, int Cout, int Cin, void* packed, hipStream_t st, bool transposed = false);
+size_t conv_packed_bf16_bytes(int code, int S_exp, int Cout, int Cin, bool wide);
+int pack_conv_weights_bf16(int code, const float* w, int S_exp, int Cout, int Cin, void* packed, hipStream_t st, bool transposed, bool wide);
 int interleave8_bf16(const bf16_t* x, int64_t ldx, const bf16_t* x2, int64_t ldx2, int c_split, int C, int64_t count, bf16_t* out,
                      hipStream_t st);
 static std::atomic<int> g_bf16_math{1};      // bfloat16 features: 1 = bfloat16 matrix instructions, 0 = fp32 matrix instructions
@@ -195,7 +195,8 @@ static int try_narrow(aprnet_plan* p, const ConvArgs<T>& a, int code, int d, con
     WinLists wl;
     if (get_lists(p, d, code, tl, &wl, st) != 0) { (void)hipGetLastError(); return 0; }
     *done = true;
-    if (int rc = plan_scratch(p, conv_narrow_packed_floats(code, a.S_exp, a.Cout, a.Cin) * sizeof(float), st)) return rc;
+    ScratchLease lease;
+    if (int rc = lease.acquire(p, conv_narrow_packed_floats(code, a.S_exp, a.Cout, a.Cin) * sizeof(float), st)) return rc;
     if (int rc = pack_conv_weights_narrow(code, (const float*)a.w, a.S_exp, a.Cout, a.Cin, (float*)p->d_scratch, st)) return rc;
     ConvArgs<T> b = a;
     b.w = (const float*)p->d_scratch;
@@ -213,7 +214,8 @@ template <> int try_mfma<float>(aprnet_plan* p, const ConvArgs<float>& a, int co
     if (*done) return 0;
     *done = true;
     // plan-owned scratch for the re-laid-out weights, grown on demand
-    if (int rc = plan_scratch(p, conv_packed_floats(code, a.S_exp, a.Cout, a.Cin, false) * sizeof(float), st)) return rc;
+    ScratchLease lease;
+    if (int rc = lease.acquire(p, conv_packed_floats(code, a.S_exp, a.Cout, a.Cin, false) * sizeof(float), st)) return rc;
     if (int rc = pack_conv_weights(code, a.w, a.S_exp, a.Cout, a.Cin, false, (float*)p->d_scratch, st)) return rc;
     ConvArgs<float> b = a;
     b.w = (const float*)p->d_scratch;
@@ -248,6 +250,9 @@ int conv_fwd(const aprnet_plan* cp, int d, int kz, int kx, int ky, const T* x, i
     aprnet_plan* p = const_cast<aprnet_plan*>(cp);
     if (int rc = check_level_delta(p, d, "conv_forward")) return rc;
     if (int rc = check_plane_size(p, d, sizeof(*x), "conv_forward")) return rc;
+    if (int rc = check_rows(ldx, p->number_parts(d), "conv_forward", "input")) return rc;
+    if (int rc = check_rows(ldy, p->number_parts(d), "conv_forward", "output")) return rc;
+    if (fu.C2 > 0) if (int rc = check_rows(fu.ldx2, p->number_parts(d), "conv_forward", "second input")) return rc;
     const int Cin = C1 + fu.C2;
     if (C1 <= 0 || Cout <= 0 || S_exp <= 0) return fail(APRNET_ERR_INVALID_ARGUMENT, "conv_forward: empty channel / stencil count");
     const int code = kz * 100 + kx * 10 + ky;
@@ -290,6 +295,9 @@ int conv_fwd_bf16(const aprnet_plan* cp, int d, int kz, int kx, int ky, const bf
     aprnet_plan* p = const_cast<aprnet_plan*>(cp);
     if (int rc = check_level_delta(p, d, "conv_forward")) return rc;
     if (int rc = check_plane_size(p, d, sizeof(*x), "conv_forward")) return rc;
+    if (int rc = check_rows(ldx, p->number_parts(d), "conv_forward", "input")) return rc;
+    if (int rc = check_rows(ldy, p->number_parts(d), "conv_forward", "output")) return rc;
+    if (fu.C2 > 0) if (int rc = check_rows(fu.ldx2, p->number_parts(d), "conv_forward", "second input")) return rc;
     const int Cin = C1 + fu.C2;
     if (C1 <= 0 || Cout <= 0 || S_exp <= 0) return fail(APRNET_ERR_INVALID_ARGUMENT, "conv_forward: empty channel / stencil count");
     const int code = kz * 100 + kx * 10 + ky;
@@ -328,14 +336,15 @@ int conv_fwd_bf16(const aprnet_plan* cp, int d, int kz, int kx, int ky, const bf
     if (int rc = set_lists(p, d, code, tl, a, st)) return rc;
     const bool bf16_math = g_bf16_math && a.tile_win;      // the bfloat16 contraction exists with window lists only
     const int64_t n_x = p->number_parts(d), n_t = p->tree_parts(d);
+    ScratchLease lease;
     if (bf16_math) {
         // The input regrouped as [Cin / 8][count][8] behind the packed weights in the plan's scratch buffer, when its
         // 16-byte items stay addressable with 32-bit offsets and the copy stays below 32 GiB.
-        const size_t wbytes = (conv_packed_bf16_bytes(code, S_exp, Cout, Cin) + 255) / 256 * 256;
         const size_t ng = (size_t)(Cin + 7) / 8, ibytes = ng * (size_t)(n_x + n_t) * 16;
         const bool regroup = bf16_regroup() && n_x < (1ll << 28) && n_t < (1ll << 28) && ibytes <= ((size_t)32 << 30);
-        if (int rc = plan_scratch(p, wbytes + (regroup ? ibytes : 0), st)) return rc;
-        if (int rc = pack_conv_weights_bf16(code, w, S_exp, Cout, Cin, p->d_scratch, st)) return rc;
+        const size_t wbytes = (conv_packed_bf16_bytes(code, S_exp, Cout, Cin, regroup) + 255) / 256 * 256;
+        if (int rc = lease.acquire(p, wbytes + (regroup ? ibytes : 0), st)) return rc;
+        if (int rc = pack_conv_weights_bf16(code, w, S_exp, Cout, Cin, p->d_scratch, st, false, regroup)) return rc;
         if (regroup) {
             bf16_t* xi = (bf16_t*)((char*)p->d_scratch + wbytes);
             bf16_t* ti = xi + ng * (size_t)n_x * 8;
@@ -344,7 +353,7 @@ int conv_fwd_bf16(const aprnet_plan* cp, int d, int kz, int kx, int ky, const bf
             a.xi = xi; a.ti = ti; a.xi_ld = n_x; a.ti_ld = n_t;
         }
     } else {
-        if (int rc = plan_scratch(p, conv_packed_floats(code, S_exp, Cout, Cin, false) * sizeof(float), st)) return rc;
+        if (int rc = lease.acquire(p, conv_packed_floats(code, S_exp, Cout, Cin, false) * sizeof(float), st)) return rc;
         if (int rc = pack_conv_weights(code, w, S_exp, Cout, Cin, false, (float*)p->d_scratch, st)) return rc;
     }
     a.apr = p->dapr; a.tree = p->dtree; a.tiles = tl.d_tiles;
@@ -368,6 +377,9 @@ int conv_fwd_bf16_layout(const aprnet_plan* cp, int d, int kz, int kx, int ky, c
     aprnet_plan* p = const_cast<aprnet_plan*>(cp);
     if (int rc = check_level_delta(p, d, "conv_forward")) return rc;
     if (int rc = check_plane_size(p, d, 2, "conv_forward")) return rc;           // the plane input of a first layer: 32-bit offsets
+    if (int rc = check_rows(ldx, p->number_parts(d), "conv_forward", "input")) return rc;
+    if (int rc = check_rows(ldy, p->number_parts(d), "conv_forward", "output")) return rc;
+    if (fu.C2 > 0) if (int rc = check_rows(fu.ldx2, p->number_parts(d), "conv_forward", "second input")) return rc;
     const int Cin = C1 + fu.C2;
     if (C1 <= 0 || Cout <= 0 || S_exp <= 0) return fail(APRNET_ERR_INVALID_ARGUMENT, "conv_forward: empty channel / stencil count");
     const int code = kz * 100 + kx * 10 + ky;
@@ -400,8 +412,9 @@ int conv_fwd_bf16_layout(const aprnet_plan* cp, int d, int kz, int kx, int ky, c
     if (tl.n == 0) return 0;
     if (int rc = set_lists(p, d, code, tl, a, st)) return rc;
     if (!a.tile_win) return fail(APRNET_ERR_UNSUPPORTED, "conv_forward: the window lists of the plan are not available");
-    if (int rc = plan_scratch(p, conv_packed_bf16_bytes(code, S_exp, Cout, Cin), st)) return rc;
-    if (int rc = pack_conv_weights_bf16(code, w, S_exp, Cout, Cin, p->d_scratch, st)) return rc;
+    ScratchLease lease;
+    if (int rc = lease.acquire(p, conv_packed_bf16_bytes(code, S_exp, Cout, Cin, true), st)) return rc;
+    if (int rc = pack_conv_weights_bf16(code, w, S_exp, Cout, Cin, p->d_scratch, st, false, true)) return rc;
     a.w = (const float*)p->d_scratch;
     a.xi = x; a.xi_ld = ldx; a.xi2 = fu.C2 > 0 ? fu.x2 : nullptr; a.xi2_ld = fu.ldx2; a.ti = tree_ws; a.ti_ld = ldt;
     a.x = nullptr; a.x2 = nullptr; a.tree_data = nullptr;

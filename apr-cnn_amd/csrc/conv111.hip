@@ -247,6 +247,8 @@ template <typename T>
 int conv111_fwd(const aprnet_plan* p, int d, const T* x, int64_t ldx, int Cin, const T* w, int S, int Cout,
                 const T* bias, T* y, int64_t ldy, hipStream_t st, int relu) {
     if (int rc = check_level_delta(p, d, "conv111_forward")) return rc;
+    if (int rc = check_rows(ldx, p->number_parts(d), "conv111_forward", "input")) return rc;
+    if (int rc = check_rows(ldy, p->number_parts(d), "conv111_forward", "output")) return rc;
     if (Cin <= 0 || Cout <= 0 || S <= 0) return fail(APRNET_ERR_INVALID_ARGUMENT, "conv111_forward: empty channel / stencil count");
     APRNET_HIP_CHECK(hipSetDevice(p->device));
     // 32 outputs per thread when the layer has more than 16: the input is then read once per 32 output channels
@@ -271,6 +273,9 @@ template <typename T>
 int conv111_bwd(const aprnet_plan* p, int d, const T* x, int64_t ldx, int Cin, const T* w, int S, int Cout, const T* gy,
                 int64_t ldy, T* gx, int64_t ldgx, T* gw, hipStream_t st) {
     if (int rc = check_level_delta(p, d, "conv111_backward")) return rc;
+    if (int rc = check_rows(ldx, p->number_parts(d), "conv111_backward", "input")) return rc;
+    if (int rc = check_rows(ldy, p->number_parts(d), "conv111_backward", "output gradient")) return rc;
+    if (int rc = check_rows(ldgx, p->number_parts(d), "conv111_backward", "input gradient")) return rc;
     if (Cin <= 0 || Cout <= 0 || S <= 0) return fail(APRNET_ERR_INVALID_ARGUMENT, "conv111_backward: empty channel / stencil count");
     APRNET_HIP_CHECK(hipSetDevice(p->device));
     constexpr int OB = 16;
@@ -293,6 +298,8 @@ int conv111_bwd(const aprnet_plan* p, int d, const T* x, int64_t ldx, int Cin, c
 int conv111_fwd_bf16(const aprnet_plan* p, int d, const bf16_t* x, int64_t ldx, int Cin, const float* w, int S, int Cout,
                      const float* bias, bf16_t* y, int64_t ldy, hipStream_t st, int relu) {
     if (int rc = check_level_delta(p, d, "conv111_forward")) return rc;
+    if (int rc = check_rows(ldx, p->number_parts(d), "conv111_forward", "input")) return rc;
+    if (int rc = check_rows(ldy, p->number_parts(d), "conv111_forward", "output")) return rc;
     if (Cin <= 0 || Cout <= 0 || S <= 0) return fail(APRNET_ERR_INVALID_ARGUMENT, "conv111_forward: empty channel / stencil count");
     APRNET_HIP_CHECK(hipSetDevice(p->device));
     for (const Segment& sg : segments(p, d, S))
@@ -306,6 +313,9 @@ int conv111_fwd_bf16(const aprnet_plan* p, int d, const bf16_t* x, int64_t ldx, 
 int conv111_bwd_bf16(const aprnet_plan* p, int d, const bf16_t* x, int64_t ldx, int Cin, const float* w, int S, int Cout,
                      const bf16_t* gy, int64_t ldy, bf16_t* gx, int64_t ldgx, float* gw, hipStream_t st) {
     if (int rc = check_level_delta(p, d, "conv111_backward")) return rc;
+    if (int rc = check_rows(ldx, p->number_parts(d), "conv111_backward", "input")) return rc;
+    if (int rc = check_rows(ldy, p->number_parts(d), "conv111_backward", "output gradient")) return rc;
+    if (int rc = check_rows(ldgx, p->number_parts(d), "conv111_backward", "input gradient")) return rc;
     if (Cin <= 0 || Cout <= 0 || S <= 0) return fail(APRNET_ERR_INVALID_ARGUMENT, "conv111_backward: empty channel / stencil count");
     APRNET_HIP_CHECK(hipSetDevice(p->device));
     for (const Segment& sg : segments(p, d, S)) {

@@ -242,8 +242,8 @@ int set_conv_lists(aprnet_plan* p, int d, int code, const TileList& tl, ConvArgs
 int set_conv_lists(aprnet_plan* p, int d, int code, const TileList& tl, ConvArgs<bf16_t>& a, hipStream_t st);
 int set_conv_dx_lists(aprnet_plan* p, int d, int code, const TileList& tl, ConvArgs<bf16_t>& a, hipStream_t st);
 int launch_conv_dx_mfma_bf16(int code, const ConvArgs<bf16_t>& a, int n_tiles, hipStream_t st);
-size_t conv_packed_bf16_bytes(int code, int S_exp, int Cout, int Cin);
-int pack_conv_weights_bf16(int code, const float* w, int S_exp, int Cout, int Cin, void* packed, hipStream_t st, bool transposed);
+size_t conv_packed_bf16_bytes(int code, int S_exp, int Cout, int Cin, bool wide);
+int pack_conv_weights_bf16(int code, const float* w, int S_exp, int Cout, int Cin, void* packed, hipStream_t st, bool transposed, bool wide);
 int interleave8_bf16(const bf16_t* x, int64_t ldx, const bf16_t* x2, int64_t ldx2, int c_split, int C, int64_t count, bf16_t* out,
                      hipStream_t st);
 int bf16_regroup();
@@ -287,7 +287,8 @@ template <> int try_mfma_bwd<float>(aprnet_plan* p, const ConvArgs<float>& a, co
     if (split_faces) if (int rc = get_face_lists(p, d, code, &faces, st)) return rc;
     const size_t wbytes = a.gx ? (conv_packed_floats(code, a.S_exp, a.Cin, a.Cout, true) * sizeof(float) + 255) / 256 * 256 : 0;
     const size_t pbytes = bwd_deterministic() ? conv_dw_partial_bytes(code, a.Cout, a.Cin) : 0;
-    if (wbytes + pbytes) if (int rc = plan_scratch(p, wbytes + pbytes, st)) return rc;
+    ScratchLease lease;          // before the join guard below: its hand-over event is recorded after the join
+    if (wbytes + pbytes) if (int rc = lease.acquire(p, wbytes + pbytes, st)) return rc;
     if (pbytes) set_dw_partials(p, wbytes, code, c);
     hipStream_t side = st;
     if (a.gx) if (int rc = fork_side(p, st, &side)) return rc;
@@ -343,6 +344,9 @@ int conv_bwd(const aprnet_plan* cp, int d, int kz, int kx, int ky, const T* x, i
     aprnet_plan* p = const_cast<aprnet_plan*>(cp);
     if (int rc = check_level_delta(p, d, "conv_backward")) return rc;
     if (int rc = check_plane_size(p, d, sizeof(*x), "conv_backward")) return rc;
+    if (int rc = check_rows(ldx, p->number_parts(d), "conv_backward", "input")) return rc;
+    if (int rc = check_rows(ldy, p->number_parts(d), "conv_backward", "output gradient")) return rc;
+    if (gx) if (int rc = check_rows(ldgx, p->number_parts(d), "conv_backward", "input gradient")) return rc;
     if (Cin <= 0 || Cout <= 0 || S_exp <= 0) return fail(APRNET_ERR_INVALID_ARGUMENT, "conv_backward: empty channel / stencil count");
     const int code = kz * 100 + kx * 10 + ky;
     if (code != 333 && code != 133 && code != 155 && code != 555)
@@ -397,6 +401,9 @@ int conv_bwd_bf16(const aprnet_plan* cp, int d, int kz, int kx, int ky, const bf
     aprnet_plan* p = const_cast<aprnet_plan*>(cp);
     if (int rc = check_level_delta(p, d, "conv_backward")) return rc;
     if (int rc = check_plane_size(p, d, sizeof(float), "conv_backward")) return rc;
+    if (int rc = check_rows(ldx, p->number_parts(d), "conv_backward", "input")) return rc;
+    if (int rc = check_rows(ldy, p->number_parts(d), "conv_backward", "output gradient")) return rc;
+    if (gx) if (int rc = check_rows(ldgx, p->number_parts(d), "conv_backward", "input gradient")) return rc;
     if (Cin <= 0 || Cout <= 0 || S_exp <= 0) return fail(APRNET_ERR_INVALID_ARGUMENT, "conv_backward: empty channel / stencil count");
     const int code = kz * 100 + kx * 10 + ky;
     if (!conv_mfma_supported(code))
@@ -433,14 +440,15 @@ int conv_bwd_bf16(const aprnet_plan* cp, int d, int kz, int kx, int ky, const bf
         // everything that can allocate or fail on the host comes before the fork
         if (near.n > 0 && bf16_math())
             if (int rc = set_conv_dx_lists(p, d, code, near, b, st)) return rc;
-        const size_t wbytes = (conv_packed_bf16_bytes(code, S_exp, Cin, Cout) + 255) / 256 * 256;
+        const size_t wbytes = (conv_packed_bf16_bytes(code, S_exp, Cin, Cout, false) + 255) / 256 * 256;
         const size_t ng = (size_t)(Cout + 7) / 8, ibytes = ng * (size_t)np * 16;
         const bool regroup = bf16_regroup() && np < (1ll << 28) && ibytes <= ((size_t)32 << 30);
         size_t need = 0;
         if (near.n > 0) need = b.tile_win ? wbytes + (regroup ? ibytes : 0) : conv_packed_floats(code, S_exp, Cin, Cout, true) * sizeof(float);
         need = (need + 255) / 256 * 256;
         const size_t pbytes = bwd_deterministic() ? conv_dw_partial_bytes(code, Cout, Cin) : 0;
-        if (need + pbytes) if (int rc = plan_scratch(p, need + pbytes, st)) return rc;
+        ScratchLease lease;      // before the join guard below: its hand-over event is recorded after the join
+        if (need + pbytes) if (int rc = lease.acquire(p, need + pbytes, st)) return rc;
         if (pbytes) set_dw_partials(p, need, code, a);
         hipStream_t side = st;
         if (near.n > 0) if (int rc = fork_side(p, st, &side)) return rc;
@@ -448,7 +456,7 @@ int conv_bwd_bf16(const aprnet_plan* cp, int d, int kz, int kx, int ky, const bf
         if (int rc = launch_conv_dw_mfma(code, a, tl, p->apr.level_min, side)) return rc;
         if (near.n > 0 && b.tile_win) {
             // the output gradient regrouped as [Cout / 8][particles][8] behind the packed weights, as in the forward pass
-            if (int rc = pack_conv_weights_bf16(code, w, S_exp, Cin, Cout, p->d_scratch, st, true)) return rc;
+            if (int rc = pack_conv_weights_bf16(code, w, S_exp, Cin, Cout, p->d_scratch, st, true, false)) return rc;
             if (regroup) {
                 bf16_t* gyi = (bf16_t*)((char*)p->d_scratch + wbytes);
                 if (int rc = interleave8_bf16(gy, ldy, nullptr, 0, Cout, Cout, np, gyi, st)) return rc;

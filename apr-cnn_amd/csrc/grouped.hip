@@ -420,6 +420,8 @@ int aprnet_ungroup8_bf16(const uint16_t* xg, int64_t ldg, int C, int64_t n, uint
 }
 int aprnet_fill_tree_mean_bf16g(const aprnet_plan* p, int d, const uint16_t* x, int64_t ldx, int C, uint16_t* tree, int64_t ldt, void* st) {
     if (int rc = check_level_delta(p, d, "fill_tree_mean")) return rc;
+    if (int rc = check_rows(ldx, p->number_parts(d), "fill_tree_mean (grouped)", "input")) return rc;
+    if (int rc = check_rows(ldt, p->tree_parts(d), "fill_tree_mean (grouped)", "tree work space")) return rc;
     APRNET_HIP_CHECK(hipSetDevice(p->device));
     return fill_tree_mean_g8(p, d, (const bf16_t*)x, ldx, C, (bf16_t*)tree, ldt, (hipStream_t)st);
 }
@@ -454,12 +456,15 @@ int aprnet_upsample_fwd_bf16g(const aprnet_plan* p, int d, const uint16_t* x, in
     APRNET_LAUNCH_CHECK("upsample_g8_kernel");
     return 0;
 }
+int aprnet_conv111_g8_max_cin(void) { return C111_MAX_CIN; }
 int aprnet_conv111_fwd_bf16g(const aprnet_plan* p, int d, const uint16_t* x, int64_t ldx, int Cin, const float* w, int S, int Cout,
                              const float* bias, int relu, uint16_t* y, int64_t ldy, int y_grouped, void* st) {
     if (int rc = check_level_delta(p, d, "conv111_forward")) return rc;
     if (Cin <= 0 || Cout <= 0 || S <= 0) return fail(APRNET_ERR_INVALID_ARGUMENT, "conv111_forward: empty channel / stencil count");
     if (Cin % 8 || Cin > C111_MAX_CIN || (y_grouped && Cout % 8))
         return fail(APRNET_ERR_UNSUPPORTED, "conv111_forward (grouped): channel counts must be multiples of eight, at most 256 inputs");
+    if (int rc = check_rows(ldx, p->number_parts(d), "conv111_forward (grouped)", "input")) return rc;
+    if (int rc = check_rows(ldy, p->number_parts(d), "conv111_forward (grouped)", "output")) return rc;
     APRNET_HIP_CHECK(hipSetDevice(p->device));
     const int Lc = p->lc(d);
     // particles of levels that share a stencil are contiguous: stencil s serves level Lc - s (the downsampled

@@ -46,8 +46,10 @@ template <typename T, int MODE>
 int pixel_op(const aprnet_plan* p, int d, T* parts, int64_t ldp, int C, T* img, int64_t ldi, hipStream_t st) {
     if (int rc = check_level_delta(p, d, "reconstruct/sample")) return rc;
     if (C <= 0) return 0;
+    if (int rc = check_rows(ldp, p->number_parts(d), "reconstruct/sample", "particle tensor")) return rc;
     APRNET_HIP_CHECK(hipSetDevice(p->device));
     const int Lc = p->lc(d);
+    if (int rc = check_rows(ldi, (int64_t)p->apr.z_num[Lc] * p->apr.x_num[Lc] * p->apr.y_num[Lc], "reconstruct/sample", "image")) return rc;
     for (int l = Lc; l >= p->apr.level_min; --l) {
         if (p->apr.level_end(l) == p->apr.level_begin(l)) continue;
         dim3 grid((unsigned)p->apr.x_num[l], (unsigned)p->apr.z_num[l]);

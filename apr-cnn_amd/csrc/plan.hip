@@ -143,19 +143,36 @@ bool stream_is_capturing(hipStream_t st) {
     return cs != hipStreamCaptureStatusNone;
 }
 
+void plan_scratch_done(aprnet_plan* p, hipStream_t st) {
+    if (stream_is_capturing(st)) { p->scratch_event_recorded = false; return; }   // inside a graph the caller orders its streams
+    if (!p->ev_scratch && hipEventCreateWithFlags(&p->ev_scratch, hipEventDisableTiming) != hipSuccess) {
+        (void)hipGetLastError(); p->ev_scratch = nullptr; p->scratch_event_recorded = false;
+        (void)hipStreamSynchronize(st);          // no event to hand over with: finish the work instead
+        return;
+    }
+    p->scratch_event_recorded = hipEventRecord(p->ev_scratch, st) == hipSuccess;
+    if (!p->scratch_event_recorded) { (void)hipGetLastError(); (void)hipStreamSynchronize(st); }
+}
+
 int plan_scratch(aprnet_plan* p, size_t bytes, hipStream_t st) {
     const bool capturing = stream_is_capturing(st);
-    // a second stream takes the buffer over only after the first is done with it
-    if (p->scratch_stream_valid && p->scratch_stream != st && !p->scratch_stream_capturing && !capturing)
-        if (hipStreamSynchronize(p->scratch_stream) != hipSuccess) (void)hipGetLastError();     // a destroyed stream has no work left
-    p->scratch_stream = st; p->scratch_stream_valid = true; p->scratch_stream_capturing = capturing;
+    // a second stream takes the buffer over only after the first is done with it: a device-side wait for the event
+    // that the previous call recorded behind its kernels
+    if (p->scratch_stream_valid && p->scratch_stream != st && p->scratch_event_recorded && !capturing)
+        APRNET_HIP_CHECK(hipStreamWaitEvent(st, p->ev_scratch, 0));
+    p->scratch_stream = st; p->scratch_stream_valid = true;
     if (bytes > p->scratch_bytes) {
         if (capturing)
             return fail(APRNET_ERR_UNSUPPORTED, "the plan's scratch buffer would have to grow while the stream is capturing: call "
                                                 "aprnet_plan_reserve, or run this call once, before the capture");
         if (p->d_scratch) {
             if (p->scratch_in_graph) p->retired.push_back(p->d_scratch);     // a graph may replay into it: keep it until destroy
-            else { APRNET_HIP_CHECK(hipStreamSynchronize(st)); APRNET_HIP_CHECK(hipFree(p->d_scratch)); }
+            else {
+                // nothing may still read the old buffer: this stream's work, and the last user's (another stream's)
+                APRNET_HIP_CHECK(hipStreamSynchronize(st));
+                if (p->scratch_event_recorded) APRNET_HIP_CHECK(hipEventSynchronize(p->ev_scratch));
+                APRNET_HIP_CHECK(hipFree(p->d_scratch));
+            }
         }
         p->d_scratch = nullptr; p->scratch_bytes = 0; p->scratch_in_graph = false;
         APRNET_HIP_CHECK(hipMalloc(&p->d_scratch, bytes));
@@ -268,6 +285,7 @@ void aprnet_plan_destroy(aprnet_plan* p) {
     if (p->side) { (void)hipStreamSynchronize(p->side); (void)hipStreamDestroy(p->side); }
     if (p->ev_fork) (void)hipEventDestroy(p->ev_fork);
     if (p->ev_join) (void)hipEventDestroy(p->ev_join);
+    if (p->ev_scratch) (void)hipEventDestroy(p->ev_scratch);
     delete p;
 }
 

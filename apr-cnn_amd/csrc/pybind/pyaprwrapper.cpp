@@ -50,6 +50,13 @@ std::vector<const aprnet_plan*> plans_of(const py::sequence& aprs, const Tensor&
     return out;
 }
 
+// one batch item per APR (the reference indexes input[b] for every APR of the list, wrap_conv_gpu.hpp:23-28): a shorter
+// batch is refused here rather than read out of range
+void check_batch(const std::vector<const aprnet_plan*>& plans, const Tensor& t) {
+    if (t.dim() < 1 || (size_t)t.size(0) != plans.size())
+        throw std::invalid_argument("the batch dimension of the tensors must equal the number of APRs");
+}
+
 std::vector<int> deltas_of(const Tensor& level_delta, size_t n) {
     TORCH_CHECK(level_delta.device().is_cpu() && level_delta.scalar_type() == torch::kInt32 && level_delta.dim() == 1,
                 "level_delta must be a 1-D int32 CPU tensor");
@@ -84,6 +91,7 @@ Tensor conv_forward_impl(const py::sequence& aprs, Tensor input, Tensor weights,
     TORCH_CHECK(input.scalar_type() == weights.scalar_type(), "weights must have the dtype of the input");
     c10::DeviceGuard guard(input.device());
     auto plans = plans_of(aprs, input);
+    check_batch(plans, input);
     auto d = deltas_of(level_delta, plans.size());
     const int kz = weights.size(3), kx = weights.size(4), ky = weights.size(5);
     const int64_t B = input.size(0), Cin = input.size(1), N = input.size(2), Cout = weights.size(1), S = weights.size(0);
@@ -112,6 +120,7 @@ std::vector<Tensor> conv_backward_impl(const py::sequence& aprs, Tensor input, T
     CHECK_INPUT(input); CHECK_INPUT(weights); CHECK_INPUT(grad_output);
     c10::DeviceGuard guard(input.device());
     auto plans = plans_of(aprs, input);
+    check_batch(plans, input);
     auto d = deltas_of(level_delta, plans.size());
     const int kz = weights.size(3), kx = weights.size(4), ky = weights.size(5);
     const int64_t Cin = input.size(1), N = input.size(2), Cout = weights.size(1), S = weights.size(0), Ng = grad_output.size(2);
@@ -172,6 +181,7 @@ std::vector<Tensor> maxpool_forward_impl(const py::sequence& aprs, Tensor input,
     CHECK_INPUT(input);
     c10::DeviceGuard guard(input.device());
     auto plans = plans_of(aprs, input);
+    check_batch(plans, input);
     auto d = deltas_of(level_delta, plans.size());
     const int64_t B = input.size(0), C = input.size(1), N = input.size(2), n_out = max_over(plans, d, 1, false);
     auto output = torch::full({B, C, n_out}, pad, input.options());       // maxpool.hpp:51 / wrap_maxpool_gpu.hpp:42
@@ -189,6 +199,7 @@ Tensor maxpool_backward_impl(const py::sequence& aprs, Tensor grad_output, Tenso
     CHECK_INPUT(grad_output); CHECK_INPUT(max_indices);
     c10::DeviceGuard guard(grad_output.device());
     auto plans = plans_of(aprs, grad_output);
+    check_batch(plans, grad_output);
     auto d = deltas_of(level_delta, plans.size());
     const int64_t B = grad_output.size(0), C = grad_output.size(1), n_out = grad_output.size(2), n_in = max_over(plans, d, 0, false);
     auto grad_input = torch::zeros({B, C, n_in}, grad_output.options());
@@ -206,6 +217,7 @@ Tensor upsample_forward_impl(const py::sequence& aprs, Tensor input, Tensor leve
     CHECK_INPUT(input);
     c10::DeviceGuard guard(input.device());
     auto plans = plans_of(aprs, input);
+    check_batch(plans, input);
     auto d = deltas_of(level_delta, plans.size());
     for (int v : d)
         if (v <= 0)      // upsample.hpp:49-54
@@ -224,6 +236,7 @@ Tensor upsample_backward_impl(const py::sequence& aprs, Tensor grad_output, Tens
     CHECK_INPUT(grad_output);
     c10::DeviceGuard guard(grad_output.device());
     auto plans = plans_of(aprs, grad_output);
+    check_batch(plans, grad_output);
     auto d = deltas_of(level_delta, plans.size());
     const int64_t B = grad_output.size(0), C = grad_output.size(1), n_out = grad_output.size(2), n_in = max_over(plans, d, 0, false);
     auto grad_input = torch::zeros({B, C, n_in}, grad_output.options());
@@ -252,6 +265,7 @@ Tensor reconstruct_forward_impl(const py::sequence& aprs, Tensor input, Tensor l
     CHECK_INPUT(input);
     c10::DeviceGuard guard(input.device());
     auto plans = plans_of(aprs, input);
+    check_batch(plans, input);
     auto d = deltas_of(level_delta, plans.size());
     auto shape = dense_shape(aprs, d);
     const int64_t B = input.size(0), C = input.size(1), N = input.size(2), plane = shape[0] * shape[1] * shape[2];
@@ -267,6 +281,7 @@ Tensor reconstruct_backward_impl(const py::sequence& aprs, Tensor grad_output, T
     CHECK_INPUT(grad_output);
     c10::DeviceGuard guard(grad_output.device());
     auto plans = plans_of(aprs, grad_output);
+    check_batch(plans, grad_output);
     auto d = deltas_of(level_delta, plans.size());
     (void)dense_shape(aprs, d);
     const int64_t B = grad_output.size(0), C = grad_output.size(1), n = max_over(plans, d, 0, false);
@@ -283,6 +298,7 @@ Tensor sample_forward_impl(const py::sequence& aprs, Tensor input, Tensor level_
     CHECK_INPUT(input);
     c10::DeviceGuard guard(input.device());
     auto plans = plans_of(aprs, input);
+    check_batch(plans, input);
     auto d = deltas_of(level_delta, plans.size());
     (void)dense_shape(aprs, d);
     const int64_t B = input.size(0), C = input.size(1), n = max_over(plans, d, 0, false), plane = input.size(2) * input.size(3) * input.size(4);
@@ -298,6 +314,7 @@ Tensor sample_backward_impl(const py::sequence& aprs, Tensor grad_output, Tensor
     CHECK_INPUT(grad_output);
     c10::DeviceGuard guard(grad_output.device());
     auto plans = plans_of(aprs, grad_output);
+    check_batch(plans, grad_output);
     auto d = deltas_of(level_delta, plans.size());
     auto shape = dense_shape(aprs, d);
     const int64_t B = grad_output.size(0), C = grad_output.size(1), N = grad_output.size(2), plane = shape[0] * shape[1] * shape[2];

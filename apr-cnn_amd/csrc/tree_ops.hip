@@ -439,6 +439,7 @@ int fill_tree_mean(const aprnet_plan* p, int d, const T* x, int64_t ldx, int C, 
     if (C <= 0) return 0;
     const int Lc = p->lc(d);
     if (ldt < p->tree_parts(d)) return fail(APRNET_ERR_INVALID_ARGUMENT, "fill_tree_mean: tree work space too small");
+    if (int rc = check_rows(ldx, p->number_parts(d), "fill_tree_mean", "input")) return rc;
     const int l_top = std::min(Lc - 1, p->tree.level_max);
     const int l_coarse = coarse_levels_end(p, l_top);            // levels level_min .. l_coarse go in one launch
     for (int l = l_top; l > l_coarse; --l) {
@@ -464,6 +465,8 @@ template <typename T>
 int fill_tree_mean_bwd(const aprnet_plan* p, int d, T* gx, int64_t ldx, int C, T* gtree, int64_t ldt, hipStream_t st) {
     if (int rc = check_level_delta(p, d, "fill_tree_mean_bwd")) return rc;
     if (C <= 0) return 0;
+    if (int rc = check_rows(ldx, p->number_parts(d), "fill_tree_mean_bwd", "input gradient")) return rc;
+    if (int rc = check_rows(ldt, p->tree_parts(d), "fill_tree_mean_bwd", "tree gradient")) return rc;
     const int Lc = p->lc(d);
     const int l_top = std::min(Lc - 1, p->tree.level_max);
     const int l_coarse = coarse_levels_end(p, l_top);
@@ -494,6 +497,9 @@ int maxpool_fwd(const aprnet_plan* p, int d, const T* x, int64_t ldx, int C, T* 
     if (Lc - 1 < p->tree.level_min) return fail(APRNET_ERR_LEVEL_DELTA, "maxpool_forward: nothing left to pool");
     const int64_t n_out = p->number_parts(d + 1), n_copy = p->apr.level_end(Lc - 1);
     if (C <= 0 || n_out <= 0) return 0;
+    if (int rc = check_rows(ldx, p->number_parts(d), "maxpool_forward", "input")) return rc;
+    if (int rc = check_rows(ldy, n_out, "maxpool_forward", "output")) return rc;
+    if (arg) if (int rc = check_rows(ldi, n_out, "maxpool_forward", "index output")) return rc;
     const int cpt = channels_per_thread(n_out, C, sizeof(T));
     dim3 grid((unsigned)((n_out + TB - 1) / TB), (unsigned)((C + cpt - 1) / cpt));
     hipLaunchKernelGGL(maxpool_fwd_kernel<T>, grid, dim3(TB), 0, st, p->d_children, p->n_tree, n_copy, n_out,
@@ -510,6 +516,9 @@ int maxpool_bwd(const aprnet_plan* p, int d, const T* gy, int64_t ldy, int C, T*
     if (Lc - 1 < p->tree.level_min) return fail(APRNET_ERR_LEVEL_DELTA, "maxpool_backward: invalid level delta");
     const int64_t n_out = p->number_parts(d + 1), n_copy = p->apr.level_end(Lc - 1);
     if (C <= 0 || n_out <= 0) return 0;
+    if (int rc = check_rows(ldx, p->number_parts(d), "maxpool_backward", "input gradient")) return rc;
+    if (int rc = check_rows(ldy, n_out, "maxpool_backward", "output gradient")) return rc;
+    if (int rc = check_rows(ldi, n_out, "maxpool_backward", "index input")) return rc;
     const int cpt = channels_per_thread(n_out, C, sizeof(T));
     dim3 grid((unsigned)((n_out + TB - 1) / TB), (unsigned)((C + cpt - 1) / cpt));
     hipLaunchKernelGGL(maxpool_bwd_kernel<T>, grid, dim3(TB), 0, st, p->d_children, p->n_tree, n_copy, n_out,
@@ -527,6 +536,9 @@ int upsample(const aprnet_plan* p, int d, const T* src, int64_t lds, int C, T* d
     const int Lc = p->lc(d);
     const int64_t n_in = p->number_parts(d), n_copy = p->apr.level_end(Lc);
     if (C <= 0 || n_in <= 0) return 0;
+    // forward: src at level delta d, dst at d - 1; backward: src is the gradient at d - 1, dst the gradient at d
+    if (int rc = check_rows(lds, Backward ? p->number_parts(d - 1) : n_in, "upsample_const", Backward ? "output gradient" : "input")) return rc;
+    if (int rc = check_rows(ldd, Backward ? n_in : p->number_parts(d - 1), "upsample_const", Backward ? "input gradient" : "output")) return rc;
     const int cpt = channels_per_thread(n_in, C, sizeof(T));
     dim3 grid((unsigned)((n_in + TB - 1) / TB), (unsigned)((C + cpt - 1) / cpt));
     hipLaunchKernelGGL((Backward ? upsample_bwd_kernel<T> : upsample_fwd_kernel<T>), grid, dim3(TB), 0, st, p->d_children, p->n_tree, n_copy, n_in,

@@ -19,10 +19,17 @@ def _lib():
     return _native.hip()
 
 
+class UnsupportedError(RuntimeError):
+    """APRNET_ERR_UNSUPPORTED: the call is valid but this build has no kernel for it (a size or channel limit, window
+    lists that could not be built).  A RuntimeError, as the reference's TORCH_CHECK failures are."""
+
+
 def _raise(rc, what):
     msg = _lib().aprnet_last_error().decode()
     if rc == -1:
         raise ValueError(msg or what)            # std::invalid_argument -> ValueError (pybind11)
+    if rc == -4:
+        raise UnsupportedError(msg or what)
     raise RuntimeError(msg or what)              # TORCH_CHECK -> RuntimeError
 
 

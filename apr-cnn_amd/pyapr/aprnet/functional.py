@@ -68,10 +68,18 @@ class ConvFunction(Function):
         return grad_input, grad_w, grad_bias, None, None, None
 
 
-def conv_inference(inputs, weights, bias, aprs, level_deltas, layout, relu=False, inputs2=None):
+def conv_inference(inputs, weights, bias, aprs, level_deltas, layout, relu=False, inputs2=None, kept_stencils=None):
     """ConvFunction.forward without the autograd record, with the two fusions the kernel offers: the ReLU that
     follows the convolution in BasicBlock (unet_parts.py:17-26, norm folded away) and a second input tensor in
-    place of torch.cat([inputs, inputs2], dim=1) (unet_parts.py:82).  For inference under torch.no_grad()."""
+    place of torch.cat([inputs, inputs2], dim=1) (unet_parts.py:82).  For inference under torch.no_grad().
+    ``kept_stencils``: (levels, fp32 stencils in the device layout already restricted to that many levels), used when
+    the APRs have that many levels."""
+    levels = max(a.level_max() - a.level_min() + 1 for a in aprs)
+    if (kept_stencils is not None and kept_stencils[0] == levels and inputs.dtype in (torch.float32, torch.bfloat16)
+            and kept_stencils[1].device == inputs.device):
+        return _ops.conv_forward(aprs, inputs.contiguous(), kept_stencils[1], level_deltas,
+                                 None if bias is None else bias.detach().contiguous(),
+                                 relu=relu, x2=None if inputs2 is None else inputs2.contiguous())
     w = _to_device_layout(weights.detach(), layout).contiguous()
     if inputs.dtype == torch.bfloat16:
         w = w.float()
@@ -79,7 +87,7 @@ def conv_inference(inputs, weights, bias, aprs, level_deltas, layout, relu=False
     if ksize not in SUPPORTED_KERNELS:
         raise ValueError(f"unsupported kernel size {ksize}")
     if ksize != (1, 1, 1):
-        w = _ops.restrict_kernel_forward(w, max(a.level_max() - a.level_min() + 1 for a in aprs))
+        w = _ops.restrict_kernel_forward(w, levels)
     return _ops.conv_forward(aprs, inputs.contiguous(), w, level_deltas, None if bias is None else bias.detach().contiguous(),
                              relu=relu, x2=None if inputs2 is None else inputs2.contiguous())
 

@@ -31,6 +31,11 @@ class Grouped:
         return self.data.size(2)
 
 
+def limits():
+    """Channel limits of the grouped kernels, read from the library."""
+    return {"conv111_max_cin": int(_lib().aprnet_conv111_g8_max_cin())}
+
+
 def supported(aprs, channels):
     return all(c % 8 == 0 for c in channels) and all(a.total_number_particles() <= MAX_PARTICLES for a in aprs)
 

@@ -53,8 +53,11 @@ class APRConv(nn.Module):
         """Inference-only forward (no autograd record): optionally clamps the result at zero inside the kernel and
         reads ``second_input`` as the channels that follow those of ``input_features``, i.e.
         relu(self(torch.cat([input_features, second_input], 1))) in one pass."""
+        # stencils kept by a network's prepare_inference() (fp32, device layout); only weights that are fp32 themselves
+        # would be restricted to the same values here
+        kept = getattr(self, "_inference_stencils", None) if self.weight.dtype == torch.float32 else None
         return conv_inference(input_features, self.weight, self.bias, aprs, level_deltas, self.weight_layout,
-                              relu=relu, inputs2=second_input)
+                              relu=relu, inputs2=second_input, kept_stencils=kept)
 
 
 class MaxPool(nn.Module):

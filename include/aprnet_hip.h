@@ -296,6 +296,9 @@ int aprnet_upsample_fwd_bf16g(const aprnet_plan*, int level_delta, const uint16_
                               void* stream);
 int aprnet_conv111_fwd_bf16g(const aprnet_plan*, int level_delta, const uint16_t* x, int64_t ldx, int Cin, const float* w, int S,
                              int Cout, const float* bias, int relu, uint16_t* y, int64_t ldy, int y_grouped, void* stream);
+/* largest Cin that aprnet_conv111_fwd_bf16g takes (256): callers that choose between the grouped and the plane
+ * operators ask before they start a network (no counterpart in the reference) */
+int aprnet_conv111_g8_max_cin(void);
 int aprnet_conv_fwd_fused_bf16l(const aprnet_plan*, int level_delta, int kz, int kx, int ky, const uint16_t* x, int64_t ldx, int Cin,
                                 int x_grouped, const float* w, int S_exp, int Cout, const float* bias, uint16_t* y, int64_t ldy,
                                 int y_grouped, uint16_t* tree_ws, int64_t ld_tree, const aprnet_conv_fusion* fusion, void* stream);

@@ -149,18 +149,102 @@ def test_unet_grouped_forward_against_oracle_and_plane_path():
 
 
 def test_unet_grouped_forward_follows_weight_updates():
-    """The grouped forward keeps the restricted stencils of a layer until its weights change: an in-place update of a
-    weight tensor must show in the next forward pass."""
+    """Without prepare_inference() the grouped forward restricts its stencils in every pass, so every kind of weight
+    update shows in the next forward pass: in place (w.mul_), and through .data (which autograd's version counter
+    does not see).  With prepare_inference() the stencils are kept until they are dropped: by
+    invalidate_inference_cache(), load_state_dict(), train() or a move of the module."""
     from bench import make_unet
     apr = apr_cases.random_apr((20, 24, 22), 3, density=0.05)
     x = torch.randn(1, 1, apr.total_number_particles(), generator=torch.Generator().manual_seed(7)).to(torch.bfloat16).to(DEV)
     model = make_unet(DEV)
+    conv = model.encoder[0].blocks[1].conv
     with torch.no_grad():
+        assert model._grouped_ok(x, [apr])
         y0 = model(x, [apr]).clone()
         assert torch.equal(model(x, [apr]), y0)
-        w = model.encoder[0].blocks[0].conv.weight
+        w = conv.weight
         w.mul_(0.5)
-        y1 = model(x, [apr])
+        y1 = model(x, [apr]).clone()
         assert not torch.equal(y1, y0)
         w.mul_(2.0)
         assert torch.equal(model(x, [apr]), y0)
+        w.data.mul_(0.5)                                   # leaves w._version and w.data_ptr() unchanged
+        assert torch.equal(model(x, [apr]), y1)
+        w.data.mul_(2.0)
+        # kept stencils
+        model.prepare_inference([apr])
+        assert hasattr(conv, "_inference_stencils")
+        assert torch.equal(model(x, [apr]), y0)
+        w.data.mul_(0.5)
+        assert torch.equal(model(x, [apr]), y0)            # stale by contract ...
+        model.invalidate_inference_cache()
+        assert torch.equal(model(x, [apr]), y1)            # ... until invalidated
+        w.data.mul_(2.0)
+        model.prepare_inference([apr])
+        state = {k: v.clone() for k, v in model.state_dict().items()}
+        state["encoder.0.blocks.1.conv.weight"] *= 0.5
+        model.load_state_dict(state)
+        assert not hasattr(conv, "_inference_stencils")
+        assert torch.equal(model(x, [apr]), y1)
+        model.prepare_inference([apr])
+        model.train()
+        assert not hasattr(conv, "_inference_stencils")
+        model.eval()
+        model.prepare_inference(levels=apr.level_max() - apr.level_min() + 1)
+        model.float()
+        assert not hasattr(conv, "_inference_stencils")
+
+
+def test_unet_grouped_limits_fall_back_to_the_plane_path():
+    """A network whose 1x1x1 reduction sees 512 channels is beyond the grouped 1x1x1 kernel (256 inputs): the model
+    must notice before any layer runs and compute the same result on channel planes.  The same when the plan's
+    window lists are switched off (the grouped convolution then reports "unsupported" from inside the forward pass),
+    and when a submodule carries a forward hook, which the grouped path would skip."""
+    from apr_models.unet import APRUNet, fold_norms
+    apr = apr_cases.random_apr((12, 10, 14), 5, density=0.08)
+    x = torch.randn(1, 1, apr.total_number_particles(), generator=torch.Generator().manual_seed(9)).to(torch.bfloat16).to(DEV)
+    torch.manual_seed(3)
+    wide = fold_norms(APRUNet(1, 2, depth=3, n_filters_base=64, n_stencils=1, norm="batch").eval()).to(DEV)
+    assert g8.limits()["conv111_max_cin"] == 256
+    with torch.no_grad():
+        assert not wide._grouped_ok(x, [apr])
+        got = wide(x, [apr])
+        wide.use_grouped = False
+        assert torch.equal(wide(x, [apr]), got)
+    from bench import make_unet
+    model = make_unet(DEV)
+    lib = _native.hip()
+    with torch.no_grad():
+        assert model._grouped_ok(x, [apr])
+        grouped_out = model(x, [apr])
+        model.use_grouped = False
+        planes = model(x, [apr])
+        model.use_grouped = True
+        ld = torch.zeros(1, dtype=torch.int32)
+        assert lib.aprnet_set_conv_path(5) == 0            # no window lists: the grouped convolution refuses
+        try:
+            fallback = model(x, [apr], ld)
+        finally:
+            assert lib.aprnet_set_conv_path(4) == 0
+        assert int(ld[0]) == 0                             # level deltas restored and walked down and up again
+        lib.aprnet_set_conv_path(5)
+        try:
+            model.use_grouped = False
+            planes_nolists = model(x, [apr])
+        finally:
+            lib.aprnet_set_conv_path(4)
+            model.use_grouped = True
+        assert torch.equal(fallback, planes_nolists)
+        scale = float(planes.float().abs().max())
+        assert float((fallback.float() - grouped_out.float()).abs().max()) <= 1e-2 * scale
+        seen = []
+        h = model.encoder[1].pool.register_forward_hook(lambda m, i, o: seen.append(1))
+        assert not model._grouped_ok(x, [apr])
+        assert torch.equal(model(x, [apr]), planes) and seen
+        h.remove()
+        assert model._grouped_ok(x, [apr])
+        model.encoder[1].pool.increment_level_deltas = False
+        assert not model._grouped_ok(x, [apr])
+        model.encoder[1].pool.increment_level_deltas = True
+        del model.use_grouped                              # a whole-model pickle from before the attribute existed
+        assert model._grouped_ok(x, [apr])

@@ -806,3 +806,81 @@ def test_conv_forward_narrow_input(cin, cout, ksize, dtype):
         close_bf16(got, ref)
         close_bf16(general, ref)
         assert torch.equal(fused, torch.relu(got))
+
+
+def _tight(got32, ora32, ref64, terms64, what):
+    """fp32 parity as a claim the arithmetic fixes: the HIP result must be (1) as close to the float64 truth as the
+    reference's own fp32 loop order is, up to a factor of two, and (2) element by element within
+    1e-5 * |truth| + 1e-5 * sum |terms| - the rounding of an fp32 sum is bounded by its terms, so an element that is
+    small because large terms cancel is held to the size of the terms, every other element to rel 1e-5
+    (the reference's check is element-wise too: torch.allclose, pyapr/tests/test_aprnet.py:176-179)."""
+    got, ora = got32.detach().cpu().double(), ora32.double()
+    e_hip, e_ora = float((got - ref64).abs().max()), float((ora - ref64).abs().max())
+    floor = 1e-7 * float(ref64.abs().max())             # both at the last bit of fp32
+    assert e_hip <= 2.0 * e_ora + floor, f"{what}: HIP fp32 is {e_hip:.3e} from float64, the oracle's fp32 {e_ora:.3e}"
+    bound = 1e-5 * ref64.abs() + 1e-5 * terms64
+    worst = float(((got - ref64).abs() - bound).max())
+    assert worst <= 0.0, f"{what}: element-wise bound exceeded by {worst:.3e}"
+
+
+@pytest.mark.parametrize("ksize", [(3, 3, 3), (1, 5, 5)], ids=KID)
+@pytest.mark.parametrize("cin,cout", [(32, 32), (33, 33)])
+def test_conv_fp32_is_as_close_to_float64_as_the_reference_order(cin, cout, ksize):
+    """Forward, input gradient and weight gradient in fp32 against the oracle run in float64 on the same fp32 inputs
+    and the same expanded stencils (so that only the convolution arithmetic differs)."""
+    bt = [("3d_s", 0), ("3d_t", 1)] if ksize[0] == 3 else [("2d_s", 0), ("2d_t", 1)]
+    x, aprs, ld, w_exp = _conv_case(bt, ksize, 2, cin, cout, torch.float32)
+    go = torch.randn(x.size(0), cout, x.size(2), generator=torch.Generator().manual_seed(8))
+    sizes = [oracle.number_parts(a, int(d)) for a, d in zip(aprs, ld)]
+    for i, n in enumerate(sizes):
+        go[i, :, n:] = 0
+    x64, w64, go64 = x.double(), w_exp.double(), go.double()
+    y32, y64 = oracle.conv_forward(aprs, x, w_exp, ld), oracle.conv_forward(aprs, x64, w64, ld)
+    y_terms = oracle.conv_forward(aprs, x64.abs(), w64.abs(), ld)
+    gx32, gw32 = oracle.conv_backward(aprs, x, w_exp, go, ld)
+    gx64, gw64 = oracle.conv_backward(aprs, x64, w64, go64, ld)
+    gx_terms, gw_terms = oracle.conv_backward(aprs, x64.abs(), w64.abs(), go64.abs(), ld)
+    wd = w_exp.permute(1, 2, 0, 3, 4, 5).contiguous().to(DEV)
+    y = _ops.conv_forward(aprs, x.to(DEV), wd, ld)
+    gx, gw = _ops.conv_backward(aprs, x.to(DEV), wd, go.to(DEV), ld)
+    _tight(y, y32, y64, y_terms, "forward")
+    _tight(gx, gx32, gx64, gx_terms, "input gradient")
+    _tight(gw.permute(2, 0, 1, 3, 4, 5), gw32, gw64, gw_terms, "weight gradient")
+
+
+def test_short_rows_are_refused_before_any_launch():
+    """A tensor with fewer elements per channel than the APR has particles at the level delta must come back as
+    APRNET_ERR_INVALID_ARGUMENT (-1) from the C ABI, not as an out-of-range device access."""
+    apr = apr_cases.get("3d_b")
+    apr.init_cuda()
+    lib, plan = _native.hip(), apr.plan(0)
+    n, n1, nt = oracle.number_parts(apr, 0), oracle.number_parts(apr, 1), _ops.tree_parts(apr, 0)
+    x = torch.zeros(4, n, device=DEV)
+    y = torch.zeros(4, n, device=DEV)
+    w = torch.zeros(1, 4, 4, 3, 3, 3, device=DEV)
+    tree = torch.zeros(4, max(nt, 1), device=DEV)
+    idx = torch.zeros(4, n1, dtype=torch.int64, device=DEV)
+    st = torch.cuda.current_stream().cuda_stream
+    p = lambda t: C.c_void_p(t.data_ptr())
+    torch.cuda.synchronize()
+    assert lib.aprnet_conv_fwd_f32(plan, 0, 3, 3, 3, p(x), n - 1, 4, p(w), 1, 4, None, p(y), n, p(tree), max(nt, 1), st) == -1
+    assert lib.aprnet_conv_fwd_f32(plan, 0, 3, 3, 3, p(x), n, 4, p(w), 1, 4, None, p(y), n - 1, p(tree), max(nt, 1), st) == -1
+    assert b"holds" in lib.aprnet_last_error()
+    assert lib.aprnet_conv111_fwd_f32(plan, 0, p(x), n - 1, 4, p(w), 1, 4, None, p(y), n, st) == -1
+    assert lib.aprnet_maxpool_fwd_f32(plan, 0, p(x), n - 1, 4, p(y), n1, p(idx), n1, st) == -1
+    assert lib.aprnet_maxpool_fwd_f32(plan, 0, p(x), n, 4, p(y), n1 - 1, p(idx), n1, st) == -1
+    assert lib.aprnet_maxpool_fwd_f32(plan, 0, p(x), n, 4, p(y), n1, p(idx), n1 - 1, st) == -1
+    assert lib.aprnet_upsample_fwd_f32(plan, 1, p(x), n1 - 1, 4, p(y), n, st) == -1
+    assert lib.aprnet_upsample_fwd_f32(plan, 1, p(x), n1, 4, p(y), n - 1, st) == -1
+    assert lib.aprnet_upsample_bwd_f32(plan, 1, p(x), n - 1, 4, p(y), n1, st) == -1
+    assert lib.aprnet_fill_tree_mean_f32(plan, 0, p(x), n - 1, 4, p(tree), max(nt, 1), st) == -1
+    xg = torch.zeros(1, n, 8, dtype=torch.bfloat16, device=DEV)
+    assert lib.aprnet_conv111_fwd_bf16g(plan, 0, p(xg), n - 1, 8, p(w), 1, 8, None, 0, p(xg), n, 1, st) == -1
+    # the reference-named binding: one batch item per APR
+    import _pyaprwrapper
+    ldt = torch.zeros(1, dtype=torch.int32)
+    with pytest.raises(ValueError, match="batch"):
+        _pyaprwrapper.aprnet.cuda.conv333_forward([apr, apr], x.view(1, 4, n), w, torch.zeros(2, dtype=torch.int32))
+    with pytest.raises(ValueError, match="holds"):
+        _pyaprwrapper.aprnet.cuda.conv333_forward([apr], x.view(1, 4, n)[:, :, :n - 1].contiguous(), w, ldt)
+    torch.cuda.synchronize()
