@@ -138,8 +138,8 @@ bool conv_mfma_supported(int code);
 int launch_conv_mfma(int code, const ConvArgs<float>& a, int n_tiles, hipStream_t st);
 int launch_conv_mfma(int code, const ConvArgs<bf16_t>& a, int n_tiles, hipStream_t st);
 int launch_conv_mfma_bf16(int code, const ConvArgs<bf16_t>& a, int n_tiles, hipStream_t st);
-size_t conv_packed_bf16_bytes(int code, int S_exp, int Cout, int Cin, bool wide);
-int pack_conv_weights_bf16(int code, const float* w, int S_exp, int Cout, int Cin, void* packed, hipStream_t st, bool transposed, bool wide);
+size_t conv_packed_bf16_bytes(int code, int S_exp, int Cout, int Cin);
+int pack_conv_weights_bf16(int code, const float* w, int S_exp, int Cout, int Cin, void* packed, hipStream_t st, bool transposed = false);
 int interleave8_bf16(const bf16_t* x, int64_t ldx, const bf16_t* x2, int64_t ldx2, int c_split, int C, int64_t count, bf16_t* out,
                      hipStream_t st);
 static std::atomic<int> g_bf16_math{1};      // bfloat16 features: 1 = bfloat16 matrix instructions, 0 = fp32 matrix instructions
@@ -340,11 +340,11 @@ int conv_fwd_bf16(const aprnet_plan* cp, int d, int kz, int kx, int ky, const bf
     if (bf16_math) {
         // The input regrouped as [Cin / 8][count][8] behind the packed weights in the plan's scratch buffer, when its
         // 16-byte items stay addressable with 32-bit offsets and the copy stays below 32 GiB.
+        const size_t wbytes = (conv_packed_bf16_bytes(code, S_exp, Cout, Cin) + 255) / 256 * 256;
         const size_t ng = (size_t)(Cin + 7) / 8, ibytes = ng * (size_t)(n_x + n_t) * 16;
         const bool regroup = bf16_regroup() && n_x < (1ll << 28) && n_t < (1ll << 28) && ibytes <= ((size_t)32 << 30);
-        const size_t wbytes = (conv_packed_bf16_bytes(code, S_exp, Cout, Cin, regroup) + 255) / 256 * 256;
         if (int rc = lease.acquire(p, wbytes + (regroup ? ibytes : 0), st)) return rc;
-        if (int rc = pack_conv_weights_bf16(code, w, S_exp, Cout, Cin, p->d_scratch, st, false, regroup)) return rc;
+        if (int rc = pack_conv_weights_bf16(code, w, S_exp, Cout, Cin, p->d_scratch, st)) return rc;
         if (regroup) {
             bf16_t* xi = (bf16_t*)((char*)p->d_scratch + wbytes);
             bf16_t* ti = xi + ng * (size_t)n_x * 8;
@@ -413,8 +413,8 @@ int conv_fwd_bf16_layout(const aprnet_plan* cp, int d, int kz, int kx, int ky, c
     if (int rc = set_lists(p, d, code, tl, a, st)) return rc;
     if (!a.tile_win) return fail(APRNET_ERR_UNSUPPORTED, "conv_forward: the window lists of the plan are not available");
     ScratchLease lease;
-    if (int rc = lease.acquire(p, conv_packed_bf16_bytes(code, S_exp, Cout, Cin, true), st)) return rc;
-    if (int rc = pack_conv_weights_bf16(code, w, S_exp, Cout, Cin, p->d_scratch, st, false, true)) return rc;
+    if (int rc = lease.acquire(p, conv_packed_bf16_bytes(code, S_exp, Cout, Cin), st)) return rc;
+    if (int rc = pack_conv_weights_bf16(code, w, S_exp, Cout, Cin, p->d_scratch, st)) return rc;
     a.w = (const float*)p->d_scratch;
     a.xi = x; a.xi_ld = ldx; a.xi2 = fu.C2 > 0 ? fu.x2 : nullptr; a.xi2_ld = fu.ldx2; a.ti = tree_ws; a.ti_ld = ldt;
     a.x = nullptr; a.x2 = nullptr; a.tree_data = nullptr;

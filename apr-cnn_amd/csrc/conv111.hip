@@ -10,22 +10,24 @@ namespace aprnet {
 constexpr int TB1 = 256;
 
 // dst[o][i] = sum_c W(o, c) * src[c][i],  W(o, c) = w[o * so + c * sc]
+// T = storage type of the features; weights, bias and sums in Num<T>::acc (fp32 for bfloat16 features)
 template <typename T, int OB>
 __global__ void __launch_bounds__(TB1)
-conv111_kernel(const T* __restrict__ src, int64_t lds, int Csrc, const T* __restrict__ w, int so, int sc,
-               const T* __restrict__ bias, T* __restrict__ dst, int64_t ldd, int Cdst, int64_t begin, int64_t end,
+conv111_kernel(const T* __restrict__ src, int64_t lds, int Csrc, const typename Num<T>::acc* __restrict__ w, int so, int sc,
+               const typename Num<T>::acc* __restrict__ bias, T* __restrict__ dst, int64_t ldd, int Cdst, int64_t begin, int64_t end,
                int relu) {
+    typedef typename Num<T>::acc A;
     const int64_t i = begin + (int64_t)blockIdx.x * TB1 + threadIdx.x;
     if (i >= end) return;
     const int o0 = blockIdx.y * OB;
-    T acc[OB];
+    A acc[OB];
 #pragma unroll
     for (int o = 0; o < OB; ++o) acc[o] = 0;
     constexpr int CU = 8;            // input channels loaded together: eight independent loads in flight
     for (int c0 = 0; c0 < Csrc; c0 += CU) {
-        T v[CU];
+        A v[CU];
 #pragma unroll
-        for (int k = 0; k < CU; ++k) v[k] = c0 + k < Csrc ? src[(int64_t)(c0 + k) * lds + i] : (T)0;
+        for (int k = 0; k < CU; ++k) v[k] = c0 + k < Csrc ? Num<T>::ld(src[(int64_t)(c0 + k) * lds + i]) : (A)0;
 #pragma unroll
         for (int k = 0; k < CU; ++k) {
             if (c0 + k >= Csrc) break;
@@ -37,9 +39,9 @@ conv111_kernel(const T* __restrict__ src, int64_t lds, int Csrc, const T* __rest
 #pragma unroll
     for (int o = 0; o < OB; ++o)
         if (o0 + o < Cdst) {
-            T v = acc[o] + (bias ? bias[o0 + o] : (T)0);
-            if (relu) v = v < (T)0 ? (T)0 : v;
-            dst[(int64_t)(o0 + o) * ldd + i] = v;
+            A v = acc[o] + (bias ? bias[o0 + o] : (A)0);
+            if (relu) v = v < (A)0 ? (A)0 : v;
+            dst[(int64_t)(o0 + o) * ldd + i] = Num<T>::st(v);
         }
 }
 
@@ -303,8 +305,12 @@ int conv111_fwd_bf16(const aprnet_plan* p, int d, const bf16_t* x, int64_t ldx, 
     if (Cin <= 0 || Cout <= 0 || S <= 0) return fail(APRNET_ERR_INVALID_ARGUMENT, "conv111_forward: empty channel / stencil count");
     APRNET_HIP_CHECK(hipSetDevice(p->device));
     for (const Segment& sg : segments(p, d, S))
-        if (!launch_conv111_mfma<bf16_t>(x, ldx, Cin, w + (int64_t)sg.stencil * Cout * Cin, Cin, 1, bias, y, ldy, Cout, sg.begin, sg.end, st, relu))
-            return fail(APRNET_ERR_UNSUPPORTED, "conv111_forward: more than 128 input channels with bfloat16 features");
+        if (!launch_conv111_mfma<bf16_t>(x, ldx, Cin, w + (int64_t)sg.stencil * Cout * Cin, Cin, 1, bias, y, ldy, Cout, sg.begin, sg.end, st, relu)) {
+            // more than 128 input channels: the vector-ALU kernel (fp32 sums), 16 outputs per thread
+            dim3 grid((unsigned)((sg.end - sg.begin + TB1 - 1) / TB1), (unsigned)((Cout + 15) / 16));
+            hipLaunchKernelGGL((conv111_kernel<bf16_t, 16>), grid, dim3(TB1), 0, st, x, ldx, Cin, w + (int64_t)sg.stencil * Cout * Cin, Cin, 1,
+                               bias, y, ldy, Cout, sg.begin, sg.end, relu);
+        }
     APRNET_LAUNCH_CHECK("conv111_mfma_kernel");
     return 0;
 }
@@ -321,8 +327,11 @@ int conv111_bwd_bf16(const aprnet_plan* p, int d, const bf16_t* x, int64_t ldx, 
     for (const Segment& sg : segments(p, d, S)) {
         const float* ws = w + (int64_t)sg.stencil * Cout * Cin;
         // grad_x[ci][i] = sum_co w[co][ci] * gy[co][i]: the forward kernel with the weight strides swapped
-        if (!launch_conv111_mfma<bf16_t>(gy, ldy, Cout, ws, 1, Cin, nullptr, gx, ldgx, Cin, sg.begin, sg.end, st))
-            return fail(APRNET_ERR_UNSUPPORTED, "conv111_backward: bfloat16 features support at most 128 output channels");
+        if (!launch_conv111_mfma<bf16_t>(gy, ldy, Cout, ws, 1, Cin, nullptr, gx, ldgx, Cin, sg.begin, sg.end, st)) {
+            dim3 grid((unsigned)((sg.end - sg.begin + TB1 - 1) / TB1), (unsigned)((Cin + 15) / 16));
+            hipLaunchKernelGGL((conv111_kernel<bf16_t, 16>), grid, dim3(TB1), 0, st, gy, ldy, Cout, ws, 1, Cin, (const float*)nullptr, gx, ldgx, Cin,
+                               sg.begin, sg.end, 0);
+        }
         const int64_t n = sg.end - sg.begin;
         dim3 g2((unsigned)std::min<int64_t>((n + TB1 * 8 - 1) / (TB1 * 8), 256), (unsigned)((Cout + 7) / 8), (unsigned)((Cin + 7) / 8));
         hipLaunchKernelGGL(conv111_dw_kernel<bf16_t>, g2, dim3(TB1), 0, st, x, ldx, Cin, gy, ldy, Cout,

@@ -242,8 +242,8 @@ int set_conv_lists(aprnet_plan* p, int d, int code, const TileList& tl, ConvArgs
 int set_conv_lists(aprnet_plan* p, int d, int code, const TileList& tl, ConvArgs<bf16_t>& a, hipStream_t st);
 int set_conv_dx_lists(aprnet_plan* p, int d, int code, const TileList& tl, ConvArgs<bf16_t>& a, hipStream_t st);
 int launch_conv_dx_mfma_bf16(int code, const ConvArgs<bf16_t>& a, int n_tiles, hipStream_t st);
-size_t conv_packed_bf16_bytes(int code, int S_exp, int Cout, int Cin, bool wide);
-int pack_conv_weights_bf16(int code, const float* w, int S_exp, int Cout, int Cin, void* packed, hipStream_t st, bool transposed, bool wide);
+size_t conv_packed_bf16_bytes(int code, int S_exp, int Cout, int Cin);
+int pack_conv_weights_bf16(int code, const float* w, int S_exp, int Cout, int Cin, void* packed, hipStream_t st, bool transposed);
 int interleave8_bf16(const bf16_t* x, int64_t ldx, const bf16_t* x2, int64_t ldx2, int c_split, int C, int64_t count, bf16_t* out,
                      hipStream_t st);
 int bf16_regroup();
@@ -440,7 +440,7 @@ int conv_bwd_bf16(const aprnet_plan* cp, int d, int kz, int kx, int ky, const bf
         // everything that can allocate or fail on the host comes before the fork
         if (near.n > 0 && bf16_math())
             if (int rc = set_conv_dx_lists(p, d, code, near, b, st)) return rc;
-        const size_t wbytes = (conv_packed_bf16_bytes(code, S_exp, Cin, Cout, false) + 255) / 256 * 256;
+        const size_t wbytes = (conv_packed_bf16_bytes(code, S_exp, Cin, Cout) + 255) / 256 * 256;
         const size_t ng = (size_t)(Cout + 7) / 8, ibytes = ng * (size_t)np * 16;
         const bool regroup = bf16_regroup() && np < (1ll << 28) && ibytes <= ((size_t)32 << 30);
         size_t need = 0;
@@ -456,7 +456,7 @@ int conv_bwd_bf16(const aprnet_plan* cp, int d, int kz, int kx, int ky, const bf
         if (int rc = launch_conv_dw_mfma(code, a, tl, p->apr.level_min, side)) return rc;
         if (near.n > 0 && b.tile_win) {
             // the output gradient regrouped as [Cout / 8][particles][8] behind the packed weights, as in the forward pass
-            if (int rc = pack_conv_weights_bf16(code, w, S_exp, Cin, Cout, p->d_scratch, st, true, false)) return rc;
+            if (int rc = pack_conv_weights_bf16(code, w, S_exp, Cin, Cout, p->d_scratch, st, true)) return rc;
             if (regroup) {
                 bf16_t* gyi = (bf16_t*)((char*)p->d_scratch + wbytes);
                 if (int rc = interleave8_bf16(gy, ldy, nullptr, 0, Cout, Cout, np, gyi, st)) return rc;

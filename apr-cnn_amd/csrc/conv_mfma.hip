@@ -702,10 +702,6 @@ using D333N = ConvGeom<3, 3, 3, 2, 4, 768, 64, 16>;
 bool conv_mfma_supported(int code) { return code == 333 || code == 133 || code == 155; }
 static int conv_taps(int code) { return code == 333 ? 27 : code == 133 ? 9 : 25; }
 static int conv_coh(int Cm) { return Cm <= 16 ? 1 : 2; }
-// bfloat16 kernels: `wide` (forward on grouped or regrouped input) lets layers of more than 32 outputs take four
-// 16-channel parts per block, so that a 64-output layer stages its input once instead of twice and reads each B
-// operand once per four matrix instructions
-static int conv_coh_bf16(int Cm, bool wide) { return Cm <= 16 ? 1 : (wide && Cm > 32) ? 4 : 2; }
 
 // a.tile_win set: forward with the window lists of the plan; otherwise the kernel scans (always for the input gradient)
 template <typename T, class G, int MODE>
@@ -747,29 +743,31 @@ int launch_conv_mfma(int code, const ConvArgs<bf16_t>& a, int n_tiles, hipStream
 // bfloat16 features, bfloat16 contraction (a.w = image of pack_conv_weights_bf16)
 template <class G>
 static int launch_bf16(const ConvArgs<bf16_t>& a, int n_tiles, hipStream_t st, bool dx = false) {
-    const bool wide = !dx && a.xi != nullptr;
-    const int coh = conv_coh_bf16(a.Cout, wide);
+    const int coh = conv_coh(a.Cout);
     dim3 grid((unsigned)n_tiles, (unsigned)((a.Cout + 16 * coh - 1) / (16 * coh)));
-#define APRNET_BF16_LAUNCH(...)                                                                                          \
-    do {                                                                                                                 \
-        if (coh == 1) hipLaunchKernelGGL((conv_mfma_bf16_kernel<G, 1, __VA_ARGS__>), grid, dim3(G::NT), 0, st, a);       \
-        else hipLaunchKernelGGL((conv_mfma_bf16_kernel<G, 2, __VA_ARGS__>), grid, dim3(G::NT), 0, st, a);                \
-    } while (0)
-#define APRNET_BF16_LAUNCH_WIDE(...)                                                                                     \
-    do {                                                                                                                 \
-        if (coh == 4) hipLaunchKernelGGL((conv_mfma_bf16_kernel<G, 4, __VA_ARGS__>), grid, dim3(G::NT), 0, st, a);       \
-        else APRNET_BF16_LAUNCH(__VA_ARGS__);                                                                            \
-    } while (0)
-    if (dx && a.xi != nullptr) APRNET_BF16_LAUNCH(false, 1, true);             // regrouped output gradient
-    else if (dx) APRNET_BF16_LAUNCH(false, 1);
-    else if (a.xi != nullptr && a.big) {     // regrouped input of 2^28 elements and more per group: 64-bit addresses
-        if (a.relu) APRNET_BF16_LAUNCH_WIDE(true, 0, true, true); else APRNET_BF16_LAUNCH_WIDE(false, 0, true, true);
-    } else if (a.xi != nullptr) {            // regrouped input (the second tensor is already part of it)
-        if (a.relu) APRNET_BF16_LAUNCH_WIDE(true, 0, true); else APRNET_BF16_LAUNCH_WIDE(false, 0, true);
-    } else if (a.relu || a.x2) APRNET_BF16_LAUNCH(true);
-    else APRNET_BF16_LAUNCH(false);
-#undef APRNET_BF16_LAUNCH
-#undef APRNET_BF16_LAUNCH_WIDE
+    if (dx && a.xi != nullptr) {           // regrouped output gradient
+        if (coh == 1) hipLaunchKernelGGL((conv_mfma_bf16_kernel<G, 1, false, 1, true>), grid, dim3(G::NT), 0, st, a);
+        else hipLaunchKernelGGL((conv_mfma_bf16_kernel<G, 2, false, 1, true>), grid, dim3(G::NT), 0, st, a);
+    } else if (dx) {
+        if (coh == 1) hipLaunchKernelGGL((conv_mfma_bf16_kernel<G, 1, false, 1>), grid, dim3(G::NT), 0, st, a);
+        else hipLaunchKernelGGL((conv_mfma_bf16_kernel<G, 2, false, 1>), grid, dim3(G::NT), 0, st, a);
+    } else if (a.xi != nullptr && a.big) {   // regrouped input of 2^28 elements and more per group: 64-bit addresses
+        if (a.relu) {
+            if (coh == 1) hipLaunchKernelGGL((conv_mfma_bf16_kernel<G, 1, true, 0, true, true>), grid, dim3(G::NT), 0, st, a);
+            else hipLaunchKernelGGL((conv_mfma_bf16_kernel<G, 2, true, 0, true, true>), grid, dim3(G::NT), 0, st, a);
+        } else if (coh == 1) hipLaunchKernelGGL((conv_mfma_bf16_kernel<G, 1, false, 0, true, true>), grid, dim3(G::NT), 0, st, a);
+        else hipLaunchKernelGGL((conv_mfma_bf16_kernel<G, 2, false, 0, true, true>), grid, dim3(G::NT), 0, st, a);
+    } else if (a.xi != nullptr) {          // regrouped input (the second tensor is already part of it)
+        if (a.relu) {
+            if (coh == 1) hipLaunchKernelGGL((conv_mfma_bf16_kernel<G, 1, true, 0, true>), grid, dim3(G::NT), 0, st, a);
+            else hipLaunchKernelGGL((conv_mfma_bf16_kernel<G, 2, true, 0, true>), grid, dim3(G::NT), 0, st, a);
+        } else if (coh == 1) hipLaunchKernelGGL((conv_mfma_bf16_kernel<G, 1, false, 0, true>), grid, dim3(G::NT), 0, st, a);
+        else hipLaunchKernelGGL((conv_mfma_bf16_kernel<G, 2, false, 0, true>), grid, dim3(G::NT), 0, st, a);
+    } else if (a.relu || a.x2) {
+        if (coh == 1) hipLaunchKernelGGL((conv_mfma_bf16_kernel<G, 1, true>), grid, dim3(G::NT), 0, st, a);
+        else hipLaunchKernelGGL((conv_mfma_bf16_kernel<G, 2, true>), grid, dim3(G::NT), 0, st, a);
+    } else if (coh == 1) hipLaunchKernelGGL((conv_mfma_bf16_kernel<G, 1>), grid, dim3(G::NT), 0, st, a);
+    else hipLaunchKernelGGL((conv_mfma_bf16_kernel<G, 2>), grid, dim3(G::NT), 0, st, a);
     APRNET_LAUNCH_CHECK("conv_mfma_bf16_kernel");
     return 0;
 }
@@ -800,16 +798,15 @@ int interleave8_bf16(const bf16_t* x, int64_t ldx, const bf16_t* x2, int64_t ldx
     APRNET_LAUNCH_CHECK("interleave8_kernel");
     return 0;
 }
-// wide: image for the forward kernel on grouped or regrouped input (see conv_coh_bf16)
-size_t conv_packed_bf16_bytes(int code, int S_exp, int Cout, int Cin, bool wide) {
-    const int coh = conv_coh_bf16(Cout, wide), nstep = (conv_taps(code) + 3) / 4;
+size_t conv_packed_bf16_bytes(int code, int S_exp, int Cout, int Cin) {
+    const int coh = conv_coh(Cout), nstep = (conv_taps(code) + 3) / 4;
     return (size_t)S_exp * ((Cout + 16 * coh - 1) / (16 * coh)) * ((Cin + BF_CIB - 1) / BF_CIB) * nstep * coh * 64 * sizeof(uint4);
 }
 // Cout / Cin: channels on the M axis of the kernel / contracted channels (transposed: the layer's Cin / Cout)
-int pack_conv_weights_bf16(int code, const float* w, int S_exp, int Cout, int Cin, void* packed, hipStream_t st, bool transposed, bool wide) {
-    const size_t n = conv_packed_bf16_bytes(code, S_exp, Cout, Cin, wide) / sizeof(uint4);
+int pack_conv_weights_bf16(int code, const float* w, int S_exp, int Cout, int Cin, void* packed, hipStream_t st, bool transposed) {
+    const size_t n = conv_packed_bf16_bytes(code, S_exp, Cout, Cin) / sizeof(uint4);
     dim3 grid((unsigned)std::min<size_t>((n + 255) / 256, 2048));
-    hipLaunchKernelGGL(pack_weights_bf16_kernel, grid, dim3(256), 0, st, w, S_exp, Cout, Cin, conv_taps(code), conv_coh_bf16(Cout, wide),
+    hipLaunchKernelGGL(pack_weights_bf16_kernel, grid, dim3(256), 0, st, w, S_exp, Cout, Cin, conv_taps(code), conv_coh(Cout),
                        transposed ? 1 : 0, (uint4*)packed);
     APRNET_LAUNCH_CHECK("pack_weights_bf16_kernel");
     return 0;

@@ -56,8 +56,8 @@ def test_tree_fill_pool_upsample_equal_the_plane_kernels():
     assert torch.equal(g8.ungroup(up), _ops.upsample_const_forward(aprs, ref, ld + 1))
 
 
-@pytest.mark.parametrize("ksize", [(3, 3, 3), (1, 5, 5)], ids=["333", "155"])
-@pytest.mark.parametrize("c1,c2,cout", [(16, 0, 16), (8, 24, 40), (32, 0, 8)])
+@pytest.mark.parametrize("ksize", [(3, 3, 3), (1, 3, 3), (1, 5, 5)], ids=["333", "133", "155"])
+@pytest.mark.parametrize("c1,c2,cout", [(16, 0, 16), (8, 24, 40), (32, 0, 8), (32, 32, 64), (64, 0, 72), (8, 0, 16)])
 def test_grouped_convolution_equals_the_plane_kernel(c1, c2, cout, ksize):
     """Grouped input (with and without a second input), grouped and plane output, bias and ReLU: bit-identical to the
     fused plane entry point, which stages the same values from a regrouped copy."""
