@@ -11,7 +11,7 @@ from concurrent.futures import ThreadPoolExecutor
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
-HIP_SOURCES = ["plan.hip", "lists.hip", "faces.hip", "tree_ops.hip", "grouped.hip", "conv.hip", "conv_mfma.hip", "conv_narrow.hip", "conv_bwd.hip", "conv_bwd_mfma.hip", "conv111.hip", "restrict.hip", "pixels.hip", "stardist.hip", "norm.hip"]
+HIP_SOURCES = ["plan.hip", "lists.hip", "faces.hip", "need.hip", "tree_ops.hip", "grouped.hip", "conv.hip", "conv_mfma.hip", "conv_narrow.hip", "conv_bwd.hip", "conv_bwd_mfma.hip", "conv111.hip", "restrict.hip", "pixels.hip", "stardist.hip", "norm.hip"]
 HIP_FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fno-gpu-rdc",
              "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
              "-Wno-unused-command-line-argument", "-Wno-unknown-attributes"]

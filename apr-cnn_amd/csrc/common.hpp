@@ -87,6 +87,15 @@ struct WinLists {
     int n_lv = 0; int lv_first[MAX_LEVELS] = {}; int lv_level[MAX_LEVELS] = {};
 };
 
+// Tree nodes whose mean a convolution reads (need.hip): per tree level an ascending list of node indices in `d_nodes`.
+struct NeedLists {
+    int32_t* d_nodes = nullptr;
+    int64_t n_nodes = 0;
+    int64_t off[MAX_LEVELS + 1] = {}, cnt[MAX_LEVELS + 1] = {};   // first entry and count of a level's list
+    bool whole[MAX_LEVELS + 1] = {};                               // the level is needed (almost) entirely: fill it whole
+    bool unavailable = false;                                      // building them failed once: do not retry
+};
+
 // Particles that stick out of a far face of the next finer level, with the (output, tap) pairs that read them
 // (faces.hip); device arrays owned by the plan.
 struct FaceLists {
@@ -119,6 +128,7 @@ struct aprnet_plan {
     bool scratch_stream_valid = false, scratch_event_recorded = false;
     std::map<std::pair<int, int>, aprnet::WinLists> lists;        // (level_delta, stencil code) -> window lists
     std::map<std::pair<int, int>, aprnet::FaceLists> faces;       // (level_delta, stencil code) -> far-face particles
+    std::map<std::pair<int, int>, aprnet::NeedLists> need;        // (level_delta, stencil code) -> tree nodes the convolution reads
     // second stream of the convolution backward (weight gradient next to input gradient), with its fork / join events
     hipStream_t side = nullptr; hipEvent_t ev_fork = nullptr, ev_join = nullptr;
 
@@ -147,6 +157,8 @@ int get_lists(aprnet_plan* plan, int level_delta, int code, const TileList& tl, 
 void free_lists(WinLists& wl);
 int get_face_lists(aprnet_plan* plan, int level_delta, int code, FaceLists* out, hipStream_t st);
 void free_face_lists(FaceLists& fl);
+int get_need_lists(aprnet_plan* plan, int level_delta, int code, const WinLists& wl, NeedLists* out, hipStream_t st);
+void free_need_lists(NeedLists& nl);
 // Makes plan->d_scratch at least `bytes` large for a call on `st` (contents are lost when it grows).  A buffer that a
 // captured graph may address is never freed before the plan is destroyed; growth while `st` is capturing is refused
 // with APRNET_ERR_UNSUPPORTED (reserve first: aprnet_plan_reserve, or run the call once outside the capture).  A call on

@@ -144,7 +144,8 @@ int interleave8_bf16(const bf16_t* x, int64_t ldx, const bf16_t* x2, int64_t ldx
                      hipStream_t st);
 static std::atomic<int> g_bf16_math{1};      // bfloat16 features: 1 = bfloat16 matrix instructions, 0 = fp32 matrix instructions
 static std::atomic<int> g_bf16_regroup{1};   // bfloat16 forward: 1 = stage from a copy of the input regrouped by 8 channels, 0 = from the channel planes
-int fill_tree_for_conv(const aprnet_plan* p, int d, const bf16_t* x, int64_t ldx, int C, bf16_t* tree, int64_t ldt, hipStream_t st);
+int fill_tree_for_conv(const aprnet_plan* p, int d, const bf16_t* x, int64_t ldx, int C, bf16_t* tree, int64_t ldt, hipStream_t st,
+                       const NeedLists* need);
 size_t conv_packed_floats(int code, int S_exp, int Cm, int Ck, bool transposed);
 int pack_conv_weights(int code, const float* w, int S_exp, int Cm, int Ck, bool transposed, float* packed, hipStream_t st);
 
@@ -224,8 +225,22 @@ template <> int try_mfma<float>(aprnet_plan* p, const ConvArgs<float>& a, int co
     return launch_conv_mfma(code, b, n_tiles, st);
 }
 
-int fill_tree_for_conv(const aprnet_plan* p, int d, const float* x, int64_t ldx, int C, float* tree, int64_t ldt, hipStream_t st);
-int fill_tree_for_conv(const aprnet_plan* p, int d, const double* x, int64_t ldx, int C, double* tree, int64_t ldt, hipStream_t st);
+int fill_tree_for_conv(const aprnet_plan* p, int d, const float* x, int64_t ldx, int C, float* tree, int64_t ldt, hipStream_t st,
+                       const NeedLists* need);
+int fill_tree_for_conv(const aprnet_plan* p, int d, const double* x, int64_t ldx, int C, double* tree, int64_t ldt, hipStream_t st,
+                       const NeedLists* need);
+
+// The tree nodes the forward kernels of this stencil read, for a fill that skips the others; null when the restricted
+// fill is switched off or its lists cannot be had (no window lists, first call under stream capture, no memory): the
+// caller then fills every node.  The kernels stage exactly what the window lists name, so either fill gives the same result.
+static std::atomic<int> g_need_fill{1};      // 1: the tree fill before a forward convolution covers the nodes that are read, 0: all nodes
+static const NeedLists* needed_nodes(aprnet_plan* p, int d, int code, const TileList& tl, hipStream_t st, NeedLists* store) {
+    if (!g_need_fill || !g_use_lists || g_conv_path == 1 || !conv_mfma_supported(code) || tl.n == 0) return nullptr;
+    WinLists wl;
+    if (get_lists(p, d, code, tl, &wl, st) != 0) { (void)hipGetLastError(); return nullptr; }
+    if (get_need_lists(p, d, code, wl, store, st) != 0) { (void)hipGetLastError(); return nullptr; }
+    return store;
+}
 
 // Optional parts of the fused forward entry points: a second input tensor whose C2 channels follow the Cin of x
 // in the contraction, and a clamp at zero of the result.
@@ -261,12 +276,14 @@ int conv_fwd(const aprnet_plan* cp, int d, int kz, int kx, int ky, const T* x, i
     const int64_t nt = p->tree_parts(d);
     if (nt > 0 && (!tree_ws || ldt < nt)) return fail(APRNET_ERR_INVALID_ARGUMENT, "conv_forward: tree work space too small");
     APRNET_HIP_CHECK(hipSetDevice(p->device));
-    if (int rc = fill_tree_for_conv(p, d, x, ldx, C1, tree_ws, ldt, st)) return rc;
-    if (fu.C2 > 0)
-        if (int rc = fill_tree_for_conv(p, d, fu.x2, fu.ldx2, fu.C2, tree_ws + (int64_t)C1 * ldt, ldt, st)) return rc;
     const bool flat = (kz == 1);
     TileList tl;
     if (int rc = get_tiles(p, d, flat ? 1 : 2, flat ? 8 : 4, &tl, st)) return rc;
+    NeedLists need_store;
+    const NeedLists* need = sizeof(T) == 4 ? needed_nodes(p, d, code, tl, st, &need_store) : nullptr;
+    if (int rc = fill_tree_for_conv(p, d, x, ldx, C1, tree_ws, ldt, st, need)) return rc;
+    if (fu.C2 > 0)
+        if (int rc = fill_tree_for_conv(p, d, fu.x2, fu.ldx2, fu.C2, tree_ws + (int64_t)C1 * ldt, ldt, st, need)) return rc;
     if (tl.n == 0) return 0;
     ConvArgs<T> a{};
     a.apr = p->dapr; a.tree = p->dtree; a.tiles = tl.d_tiles;
@@ -306,11 +323,13 @@ int conv_fwd_bf16(const aprnet_plan* cp, int d, int kz, int kx, int ky, const bf
     const int64_t nt = p->tree_parts(d);
     if (nt > 0 && (!tree_ws || ldt < nt)) return fail(APRNET_ERR_INVALID_ARGUMENT, "conv_forward: tree work space too small");
     APRNET_HIP_CHECK(hipSetDevice(p->device));
-    if (int rc = fill_tree_for_conv(p, d, x, ldx, C1, tree_ws, ldt, st)) return rc;
-    if (fu.C2 > 0)
-        if (int rc = fill_tree_for_conv(p, d, fu.x2, fu.ldx2, fu.C2, tree_ws + (int64_t)C1 * ldt, ldt, st)) return rc;
     TileList tl;
     if (int rc = get_tiles(p, d, kz == 1 ? 1 : 2, kz == 1 ? 8 : 4, &tl, st)) return rc;
+    NeedLists need_store;
+    const NeedLists* need = needed_nodes(p, d, code, tl, st, &need_store);   // (the regrouped copy below carries the unfilled nodes along unread)
+    if (int rc = fill_tree_for_conv(p, d, x, ldx, C1, tree_ws, ldt, st, need)) return rc;
+    if (fu.C2 > 0)
+        if (int rc = fill_tree_for_conv(p, d, fu.x2, fu.ldx2, fu.C2, tree_ws + (int64_t)C1 * ldt, ldt, st, need)) return rc;
     if (tl.n == 0) return 0;
     ConvArgs<bf16_t> a{};
     if (code == 555) {
@@ -370,7 +389,8 @@ int conv_fwd_bf16(const aprnet_plan* cp, int d, int kz, int kx, int ky, const bf
 //                   straight from the tensors, no regrouping pass
 //   planes input    1 to 3 channels (the first layer of a network) on the pipelined kernel
 //   grouped output  Cout a multiple of 8
-int fill_tree_mean_g8(const aprnet_plan* p, int d, const bf16_t* x, int64_t ldx, int C, bf16_t* tree, int64_t ldt, hipStream_t st);
+int fill_tree_mean_g8(const aprnet_plan* p, int d, const bf16_t* x, int64_t ldx, int C, bf16_t* tree, int64_t ldt, hipStream_t st,
+                      const NeedLists* need);
 int conv_fwd_bf16_layout(const aprnet_plan* cp, int d, int kz, int kx, int ky, const bf16_t* x, int64_t ldx, int C1, int x_g8, const float* w,
                          int S_exp, int Cout, const float* bias, bf16_t* y, int64_t ldy, int y_g8, bf16_t* tree_ws, int64_t ldt,
                          hipStream_t st, const Fusion<bf16_t>& fu) {
@@ -399,16 +419,18 @@ int conv_fwd_bf16_layout(const aprnet_plan* cp, int d, int kz, int kx, int ky, c
     a.x = x; a.ldx = ldx; a.Cin = Cin; a.w = w; a.S_exp = S_exp; a.Cout = Cout; a.bias = bias; a.relu = fu.relu;
     a.y = y; a.ldy = ldy; a.y_g8 = y_g8; a.tree_data = tree_ws; a.ldt = ldt; a.Lc = p->lc(d); a.tree_off = p->tree_offset(a.Lc);
     a.x_count = p->number_parts(d); a.t_count = nt; a.c_split = C1;
+    NeedLists need_store;
+    const NeedLists* need = needed_nodes(p, d, code, tl, st, &need_store);
     if (!x_g8) {
-        if (int rc = fill_tree_for_conv(p, d, x, ldx, C1, tree_ws, ldt, st)) return rc;
+        if (int rc = fill_tree_for_conv(p, d, x, ldx, C1, tree_ws, ldt, st, need)) return rc;
         if (tl.n == 0) return 0;
         bool done = false;
         if (int rc = try_narrow<bf16_t>(p, a, code, d, tl, st, &done)) return rc;
         return done ? 0 : fail(APRNET_ERR_UNSUPPORTED, "conv_forward: the window lists of the plan are not available");
     }
-    if (int rc = fill_tree_mean_g8(p, d, x, ldx, C1, tree_ws, ldt, st)) return rc;
+    if (int rc = fill_tree_mean_g8(p, d, x, ldx, C1, tree_ws, ldt, st, need)) return rc;
     if (fu.C2 > 0)
-        if (int rc = fill_tree_mean_g8(p, d, fu.x2, fu.ldx2, fu.C2, tree_ws + (int64_t)(C1 / 8) * ldt * 8, ldt, st)) return rc;
+        if (int rc = fill_tree_mean_g8(p, d, fu.x2, fu.ldx2, fu.C2, tree_ws + (int64_t)(C1 / 8) * ldt * 8, ldt, st, need)) return rc;
     if (tl.n == 0) return 0;
     if (int rc = set_lists(p, d, code, tl, a, st)) return rc;
     if (!a.tile_win) return fail(APRNET_ERR_UNSUPPORTED, "conv_forward: the window lists of the plan are not available");
@@ -485,12 +507,14 @@ int aprnet_set_conv_path(int path) {
     if (path == 10 || path == 11) { g_bwd_deterministic = path == 10; return 0; }
     if (path == 12 || path == 13) { g_narrow = path == 12; return 0; }
     if (path == 14 || path == 15) { g_big_addr = path == 15; return 0; }
+    if (path == 16 || path == 17) { g_need_fill = path == 16; return 0; }
     if (path != 0 && path != 1)
         return fail(APRNET_ERR_INVALID_ARGUMENT, "set_conv_path: 0 (auto), 1 (VALU only), 2 / 3 (bfloat16 features: bfloat16 / fp32 "
                                                  "matrix math), 4 / 5 (forward: window lists of the plan / scan per call), 6 / 7 (backward on two streams / one), "
                                                  "8 / 9 (bfloat16 forward: regrouped copy of the input / channel planes), 10 / 11 (weight gradient: "
                                                  "fixed-order partial sums / atomic additions), 12 / 13 (1 to 3 input channels: pipelined kernel / general kernel), "
-                                                 "14 / 15 (grouped bfloat16 forward: 32-bit offsets where they suffice / 64-bit addresses always)");
+                                                 "14 / 15 (grouped bfloat16 forward: 32-bit offsets where they suffice / 64-bit addresses always), "
+                                                 "16 / 17 (tree fill before a forward convolution: the nodes it reads / every node)");
     g_conv_path = path;
     return 0;
 }

@@ -208,8 +208,8 @@ using W133 = ConvGeom<1, 3, 3, 1, 8, 256>;
 using W155 = ConvGeom<1, 5, 5, 1, 8, 256>;
 using W555 = ConvGeom<5, 5, 5, 2, 4, 256>;
 
-int fill_tree_for_conv(const aprnet_plan* p, int d, const float* x, int64_t ldx, int C, float* tree, int64_t ldt, hipStream_t st);
-int fill_tree_for_conv(const aprnet_plan* p, int d, const double* x, int64_t ldx, int C, double* tree, int64_t ldt, hipStream_t st);
+int fill_tree_for_conv(const aprnet_plan* p, int d, const float* x, int64_t ldx, int C, float* tree, int64_t ldt, hipStream_t st, const NeedLists* need);
+int fill_tree_for_conv(const aprnet_plan* p, int d, const double* x, int64_t ldx, int C, double* tree, int64_t ldt, hipStream_t st, const NeedLists* need);
 int fill_tree_bwd_for_conv(const aprnet_plan* p, int d, float* gx, int64_t ldx, int C, float* gt, int64_t ldt, hipStream_t st);
 int fill_tree_bwd_for_conv(const aprnet_plan* p, int d, double* gx, int64_t ldx, int C, double* gt, int64_t ldt, hipStream_t st);
 
@@ -233,7 +233,7 @@ int launch_conv_dx_mfma(int code, const ConvArgs<float>& a, int n_tiles, hipStre
 int launch_conv_dw_mfma(int code, const ConvArgs<float>& a, const TileList& tl, int level_min, hipStream_t st);
 int launch_conv_dx_mfma(int code, const ConvArgs<bf16_t>& a, int n_tiles, hipStream_t st);
 int launch_conv_dw_mfma(int code, const ConvArgs<bf16_t>& a, const TileList& tl, int level_min, hipStream_t st);
-int fill_tree_for_conv(const aprnet_plan* p, int d, const bf16_t* x, int64_t ldx, int C, bf16_t* tree, int64_t ldt, hipStream_t st);
+int fill_tree_for_conv(const aprnet_plan* p, int d, const bf16_t* x, int64_t ldx, int C, bf16_t* tree, int64_t ldt, hipStream_t st, const NeedLists* need);
 size_t conv_packed_floats(int code, int S_exp, int Cm, int Ck, bool transposed);
 int pack_conv_weights(int code, const float* w, int S_exp, int Cm, int Ck, bool transposed, float* packed, hipStream_t st);
 int conv_path();
@@ -356,7 +356,7 @@ int conv_bwd(const aprnet_plan* cp, int d, int kz, int kx, int ky, const T* x, i
     if (nt > 0 && (!tree_ws || ldt < nt || (gx && (!gtree_ws || ldgt < nt))))
         return fail(APRNET_ERR_INVALID_ARGUMENT, "conv_backward: tree work space too small");
     APRNET_HIP_CHECK(hipSetDevice(p->device));
-    if (int rc = fill_tree_for_conv(p, d, x, ldx, Cin, tree_ws, ldt, st)) return rc;
+    if (int rc = fill_tree_for_conv(p, d, x, ldx, Cin, tree_ws, ldt, st, nullptr)) return rc;
     if (gx) {
         fill2d<T>(gx, ldgx, p->number_parts(d), Cin, (T)0, st);
         fill2d<T>(gtree_ws, ldgt, nt, Cin, (T)0, st);
@@ -412,7 +412,7 @@ int conv_bwd_bf16(const aprnet_plan* cp, int d, int kz, int kx, int ky, const bf
     if ((gx && (!gx32_ws || ldgx32 < np)) || (nt > 0 && (!tree_ws || ldt < nt || (gx && (!gtree_ws || ldgt < nt)))))
         return fail(APRNET_ERR_INVALID_ARGUMENT, "conv_backward: work space too small");
     APRNET_HIP_CHECK(hipSetDevice(p->device));
-    if (int rc = fill_tree_for_conv(p, d, x, ldx, Cin, tree_ws, ldt, st)) return rc;
+    if (int rc = fill_tree_for_conv(p, d, x, ldx, Cin, tree_ws, ldt, st, nullptr)) return rc;
     if (gx) {
         fill2d<float>(gx32_ws, ldgx32, np, Cin, 0.f, st);
         fill2d<float>(gtree_ws, ldgt, nt, Cin, 0.f, st);

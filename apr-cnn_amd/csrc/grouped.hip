@@ -103,6 +103,13 @@ fill_tree_level_g8_kernel(const int32_t* __restrict__ children, int64_t n_tree, 
     if (t < t_end) fill_node_g8(children, n_tree, t, x, ldx, tree, ldt, tree_off, from_x, from_x, blockIdx.y);
 }
 
+__global__ void __launch_bounds__(GTB)
+fill_tree_list_g8_kernel(const int32_t* __restrict__ children, int64_t n_tree, const int32_t* __restrict__ nodes, int64_t count,
+                         const bf16_t* __restrict__ x, int64_t ldx, bf16_t* __restrict__ tree, int64_t ldt, int64_t tree_off, int from_x) {
+    const int64_t i = (int64_t)blockIdx.x * GTB + threadIdx.x;
+    if (i < count) fill_node_g8(children, n_tree, nodes[i], x, ldx, tree, ldt, tree_off, from_x, from_x, blockIdx.y);
+}
+
 constexpr int G_MAX_COARSE = 12;
 struct GCoarse { int n; int64_t begin[G_MAX_COARSE], end[G_MAX_COARSE]; };
 
@@ -117,8 +124,10 @@ fill_tree_coarse_g8_kernel(const int32_t* __restrict__ children, int64_t n_tree,
     }
 }
 
-int fill_tree_mean_g8(const aprnet_plan* p, int d, const bf16_t* x, int64_t ldx, int C, bf16_t* tree, int64_t ldt, hipStream_t st) {
-    if (C <= 0) return 0;
+// need: fill only the nodes a convolution reads (see need.hip); null: every node
+int fill_tree_mean_g8(const aprnet_plan* p, int d, const bf16_t* x, int64_t ldx, int C, bf16_t* tree, int64_t ldt, hipStream_t st,
+                      const NeedLists* need) {
+    if (C <= 0 || (need && need->n_nodes == 0)) return 0;
     if (C % 8) return fail(APRNET_ERR_INVALID_ARGUMENT, "grouped features hold a multiple of eight channels");
     const int Lc = p->lc(d), G = C / 8;
     if (ldt < p->tree_parts(d)) return fail(APRNET_ERR_INVALID_ARGUMENT, "fill_tree_mean: tree work space too small");
@@ -135,8 +144,14 @@ int fill_tree_mean_g8(const aprnet_plan* p, int d, const bf16_t* x, int64_t ldx,
         const int64_t b = p->tree.level_begin(l), e = p->tree.level_end(l);
         if (e <= b) continue;
         const int from_x = (l + 1 == Lc);
-        hipLaunchKernelGGL(fill_tree_level_g8_kernel, dim3((unsigned)((e - b + GTB - 1) / GTB), (unsigned)G), dim3(GTB), 0, st, p->d_children,
-                           p->n_tree, b, e, x, ldx, tree, ldt, from_x ? p->tree_offset(Lc) : 0, from_x);
+        if (need && need->cnt[l] == 0) continue;
+        if (need && !need->whole[l])
+            hipLaunchKernelGGL(fill_tree_list_g8_kernel, dim3((unsigned)((need->cnt[l] + GTB - 1) / GTB), (unsigned)G), dim3(GTB), 0, st,
+                               p->d_children, p->n_tree, need->d_nodes + need->off[l], need->cnt[l], x, ldx, tree, ldt,
+                               from_x ? p->tree_offset(Lc) : 0, from_x);
+        else
+            hipLaunchKernelGGL(fill_tree_level_g8_kernel, dim3((unsigned)((e - b + GTB - 1) / GTB), (unsigned)G), dim3(GTB), 0, st, p->d_children,
+                               p->n_tree, b, e, x, ldx, tree, ldt, from_x ? p->tree_offset(Lc) : 0, from_x);
     }
     GCoarse lv{};
     for (int l = l_coarse; l >= p->tree.level_min; --l)
@@ -423,7 +438,7 @@ int aprnet_fill_tree_mean_bf16g(const aprnet_plan* p, int d, const uint16_t* x, 
     if (int rc = check_rows(ldx, p->number_parts(d), "fill_tree_mean (grouped)", "input")) return rc;
     if (int rc = check_rows(ldt, p->tree_parts(d), "fill_tree_mean (grouped)", "tree work space")) return rc;
     APRNET_HIP_CHECK(hipSetDevice(p->device));
-    return fill_tree_mean_g8(p, d, (const bf16_t*)x, ldx, C, (bf16_t*)tree, ldt, (hipStream_t)st);
+    return fill_tree_mean_g8(p, d, (const bf16_t*)x, ldx, C, (bf16_t*)tree, ldt, (hipStream_t)st, nullptr);
 }
 int aprnet_maxpool_fwd_bf16g(const aprnet_plan* p, int d, const uint16_t* x, int64_t ldx, int C, uint16_t* y, int64_t ldy, void* st) {
     if (int rc = check_level_delta(p, d, "maxpool_forward")) return rc;

@@ -282,6 +282,7 @@ void aprnet_plan_destroy(aprnet_plan* p) {
     for (void* q : p->retired) (void)hipFree(q);
     for (auto& kv : p->lists) free_lists(kv.second);
     for (auto& kv : p->faces) free_face_lists(kv.second);
+    for (auto& kv : p->need) free_need_lists(kv.second);
     if (p->side) { (void)hipStreamSynchronize(p->side); (void)hipStreamDestroy(p->side); }
     if (p->ev_fork) (void)hipEventDestroy(p->ev_fork);
     if (p->ev_join) (void)hipEventDestroy(p->ev_join);

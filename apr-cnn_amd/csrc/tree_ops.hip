@@ -161,6 +161,16 @@ fill_tree_level_kernel(const int32_t* __restrict__ children, int64_t n_tree, int
     if (t < t_end) fill_node<T>(children, n_tree, t, x, ldx, C, tree, ldt, tree_off, tree_child_from_x, tree_first, blockIdx.y * cpt, cpt);
 }
 
+// the same for the listed nodes only (ascending indices of one level)
+template <typename T>
+__global__ void __launch_bounds__(TB)
+fill_tree_list_kernel(const int32_t* __restrict__ children, int64_t n_tree, const int32_t* __restrict__ nodes, int64_t count,
+                      const T* __restrict__ x, int64_t ldx, int C, T* __restrict__ tree, int64_t ldt,
+                      int64_t tree_off, int tree_child_from_x, int tree_first, int cpt) {
+    const int64_t i = (int64_t)blockIdx.x * TB + threadIdx.x;
+    if (i < count) fill_node<T>(children, n_tree, nodes[i], x, ldx, C, tree, ldt, tree_off, tree_child_from_x, tree_first, blockIdx.y * cpt, cpt);
+}
+
 // The coarse levels of the tree hold a few nodes each: one launch walks them all, finest first, one workgroup per
 // group of CPT_COARSE channels (a level's parents read only values of the same channels, so a workgroup barrier between
 // levels is enough).  Tree children come from the tree itself (none of these levels sits directly under the features),
@@ -461,6 +471,45 @@ int fill_tree_mean(const aprnet_plan* p, int d, const T* x, int64_t ldx, int C, 
     return 0;
 }
 
+// fill_tree_mean for the nodes a convolution reads (`need`, see need.hip): the other nodes of the work space keep
+// whatever they held.  Same arithmetic per node, so the values that are computed are those of the full fill.
+template <typename T>
+int fill_tree_mean_needed(const aprnet_plan* p, int d, const NeedLists& need, const T* x, int64_t ldx, int C, T* tree, int64_t ldt,
+                          hipStream_t st) {
+    if (C <= 0 || need.n_nodes == 0) return 0;
+    const int Lc = p->lc(d);
+    if (ldt < p->tree_parts(d)) return fail(APRNET_ERR_INVALID_ARGUMENT, "fill_tree_mean: tree work space too small");
+    const int l_top = std::min(Lc - 1, p->tree.level_max);
+    const int l_coarse = coarse_levels_end(p, l_top);
+    for (int l = l_top; l > l_coarse; --l) {
+        const int64_t b = p->tree.level_begin(l), e = p->tree.level_end(l);
+        if (e <= b || need.cnt[l] == 0) continue;
+        const int from_x = (l + 1 == Lc);
+        if (need.whole[l]) {
+            const int cpt = channels_per_thread(e - b, C, sizeof(T));
+            dim3 grid((unsigned)((e - b + TB - 1) / TB), (unsigned)((C + cpt - 1) / cpt));
+            hipLaunchKernelGGL(fill_tree_level_kernel<T>, grid, dim3(TB), 0, st, p->d_children, p->n_tree, b, e, x, ldx, C,
+                               tree, ldt, from_x ? p->tree_offset(Lc) : 0, from_x, from_x, cpt);
+        } else {
+            const int cpt = channels_per_thread(need.cnt[l], C, sizeof(T));
+            dim3 grid((unsigned)((need.cnt[l] + TB - 1) / TB), (unsigned)((C + cpt - 1) / cpt));
+            hipLaunchKernelGGL(fill_tree_list_kernel<T>, grid, dim3(TB), 0, st, p->d_children, p->n_tree, need.d_nodes + need.off[l],
+                               need.cnt[l], x, ldx, C, tree, ldt, from_x ? p->tree_offset(Lc) : 0, from_x, from_x, cpt);
+        }
+    }
+    CoarseLevels lv{};
+    bool any = false;
+    for (int l = l_coarse; l >= p->tree.level_min; --l) {
+        if (p->tree.level_end(l) > p->tree.level_begin(l)) { lv.begin[lv.n] = p->tree.level_begin(l); lv.end[lv.n] = p->tree.level_end(l); ++lv.n; }
+        any = any || need.cnt[l] > 0;
+    }
+    if (lv.n > 0 && any)          // the coarse levels (a few thousand nodes together) are filled whole, in one launch
+        hipLaunchKernelGGL(fill_tree_coarse_kernel<T>, dim3((unsigned)((C + CPT_COARSE - 1) / CPT_COARSE)), dim3(TB), 0, st, p->d_children, p->n_tree,
+                           lv, x, ldx, C, tree, ldt);
+    APRNET_LAUNCH_CHECK("fill_tree kernels (needed nodes)");
+    return 0;
+}
+
 template <typename T>
 int fill_tree_mean_bwd(const aprnet_plan* p, int d, T* gx, int64_t ldx, int C, T* gtree, int64_t ldt, hipStream_t st) {
     if (int rc = check_level_delta(p, d, "fill_tree_mean_bwd")) return rc;
@@ -591,14 +640,18 @@ TREE_OPS_BF16(upsample_bwd, (const aprnet_plan* p, int d, const uint16_t* gy, in
 
 namespace aprnet {
 // used by the convolution launchers (conv.hip, conv_bwd.hip)
-int fill_tree_for_conv(const aprnet_plan* p, int d, const float* x, int64_t ldx, int C, float* tree, int64_t ldt, hipStream_t st) {
-    return fill_tree_mean<float>(p, d, x, ldx, C, tree, ldt, st);
+// `need`: fill only the nodes the convolution's window lists read (null: every node)
+int fill_tree_for_conv(const aprnet_plan* p, int d, const float* x, int64_t ldx, int C, float* tree, int64_t ldt, hipStream_t st,
+                       const NeedLists* need) {
+    return need ? fill_tree_mean_needed<float>(p, d, *need, x, ldx, C, tree, ldt, st) : fill_tree_mean<float>(p, d, x, ldx, C, tree, ldt, st);
 }
-int fill_tree_for_conv(const aprnet_plan* p, int d, const double* x, int64_t ldx, int C, double* tree, int64_t ldt, hipStream_t st) {
-    return fill_tree_mean<double>(p, d, x, ldx, C, tree, ldt, st);
+int fill_tree_for_conv(const aprnet_plan* p, int d, const double* x, int64_t ldx, int C, double* tree, int64_t ldt, hipStream_t st,
+                       const NeedLists* need) {
+    return need ? fill_tree_mean_needed<double>(p, d, *need, x, ldx, C, tree, ldt, st) : fill_tree_mean<double>(p, d, x, ldx, C, tree, ldt, st);
 }
-int fill_tree_for_conv(const aprnet_plan* p, int d, const bf16_t* x, int64_t ldx, int C, bf16_t* tree, int64_t ldt, hipStream_t st) {
-    return fill_tree_mean<bf16_t>(p, d, x, ldx, C, tree, ldt, st);
+int fill_tree_for_conv(const aprnet_plan* p, int d, const bf16_t* x, int64_t ldx, int C, bf16_t* tree, int64_t ldt, hipStream_t st,
+                       const NeedLists* need) {
+    return need ? fill_tree_mean_needed<bf16_t>(p, d, *need, x, ldx, C, tree, ldt, st) : fill_tree_mean<bf16_t>(p, d, x, ldx, C, tree, ldt, st);
 }
 int fill_tree_bwd_for_conv(const aprnet_plan* p, int d, float* gx, int64_t ldx, int C, float* gt, int64_t ldt, hipStream_t st) {
     return fill_tree_mean_bwd<float>(p, d, gx, ldx, C, gt, ldt, st);

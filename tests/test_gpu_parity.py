@@ -891,3 +891,45 @@ def test_short_rows_are_refused_before_any_launch():
     with pytest.raises(ValueError, match="holds"):
         _pyaprwrapper.aprnet.cuda.conv333_forward([apr], x.view(1, 4, n)[:, :, :n - 1].contiguous(), w, ldt)
     torch.cuda.synchronize()
+
+
+# ------------------------------------------------------------------------- tree fill restricted to the nodes read
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
+@pytest.mark.parametrize("cin", [2, 8], ids=["narrow", "general"])
+@pytest.mark.parametrize("ksize", [(3, 3, 3), (1, 3, 3), (1, 5, 5)], ids=KID)
+def test_conv_forward_fills_only_the_tree_nodes_it_reads(ksize, cin, dtype):
+    """Before a forward convolution the library fills the mean tree at the nodes the kernel's window lists name (and
+    their descendants), not at every node (aprnet_set_conv_path(16), the default; 17 fills all).  With the work space
+    poisoned beforehand: same bits in the output either way, no NaN reaches it, the filled nodes hold the values of the
+    full fill, and on APRs with resolved interiors some nodes stay untouched (the restriction is in effect)."""
+    lib = _native.hip()
+    sfx = "f32" if dtype == torch.float32 else "bf16"
+    fn = getattr(lib, "aprnet_conv_fwd_" + sfx)
+    untouched = 0
+    for name, d in [("3d_s", 0), ("3d_t", 0), ("3d_a", 0), ("3d_b", 1), ("2d_a", 0), ("2d_t", 1)]:
+        apr = apr_cases.get(name)
+        apr.init_cuda()
+        n, nt = oracle.number_parts(apr, d), max(oracle.tree_parts(apr, d), 1)
+        g = torch.Generator().manual_seed(n)
+        x = torch.randn(cin, n, generator=g).to(dtype).to(DEV)
+        S = apr.level_max() - apr.level_min() + 1
+        w = torch.randn(S, 5, cin, *ksize, generator=g).to(DEV)
+        st = torch.cuda.current_stream().cuda_stream
+        outs, trees = [], []
+        for path in (16, 17):
+            tree = torch.full((cin, nt), float("nan"), dtype=dtype, device=DEV)
+            y = torch.zeros(5, n, dtype=dtype, device=DEV)
+            assert lib.aprnet_set_conv_path(path) == 0
+            try:
+                rc = fn(apr.plan(0), d, *ksize, x.data_ptr(), n, cin, w.data_ptr(), S, 5, None, y.data_ptr(), n, tree.data_ptr(), nt, st)
+            finally:
+                lib.aprnet_set_conv_path(16)
+            assert rc == 0, lib.aprnet_last_error()
+            outs.append(y.cpu()); trees.append(tree.float().cpu())
+        assert not torch.isnan(outs[0]).any() and not torch.isnan(outs[1]).any()
+        assert torch.equal(outs[0], outs[1]), (name, d)
+        filled = ~torch.isnan(trees[0])
+        assert not torch.isnan(trees[1][:, :oracle.tree_parts(apr, d)]).any()
+        assert torch.equal(trees[0][filled], trees[1][filled])
+        untouched += int((~filled).sum())
+    assert untouched > 0
