@@ -13,12 +13,20 @@ namespace aprnet {
 
 // DX: lists of the input gradient (scan_window_dx without pooled columns) over the tiles within one row of an
 // output; windows without an output position are not stored.
+//
+// Forward lists keep the items that some output position of the window can reach through the stencil.  The scan
+// yields every particle and tree node of the staged rows, but a window of a coarser level often holds a handful of
+// output positions next to long runs of tree nodes standing for finely resolved regions: no output reads those, so
+// they are neither staged by the kernels nor needed in the mean-filled tree (need.hip).
 template <class G, bool DX>
 __global__ void __launch_bounds__(G::NT)
 build_lists_kernel(const ConvArgs<float> a, const int pass, int4* __restrict__ tile_counts, const int4* __restrict__ tile_off,
                    int4* __restrict__ win, int* __restrict__ item_idx, unsigned short* __restrict__ item_pos,
                    int* __restrict__ col_idx, unsigned short* __restrict__ col_pos) {
     __shared__ ConvShared<G> sh;
+    __shared__ unsigned char reach[DX ? 4 : G::NROW * G::RS];   // cell -> an output position of its row lies within the y taps
+    __shared__ int kept;
+    static_assert((G::NROW * G::RS) % 4 == 0, "the reach map is cleared with 4-byte stores");
     const ConvTile tile = a.tiles[blockIdx.x];
     const int L = tile.level;
     const int yn = a.apr.y_num[L];
@@ -35,14 +43,54 @@ build_lists_kernel(const ConvArgs<float> a, const int pass, int4* __restrict__ t
         __syncthreads();
         const int nc = sh.ncol, nitem = sh.nitem;
         if (nc > 0 && (!DX || nitem > 0)) {
+            // list offsets are unsigned 32-bit numbers stored in the int fields of the header
+            const unsigned ib = (unsigned)off.y + (unsigned)ni, cb = (unsigned)off.z + (unsigned)ncl;
+            int nkeep = nitem;
+            if constexpr (DX) {
+                if (pass == 1)
+                    for (int i = threadIdx.x; i < nitem; i += G::NT) { item_idx[(size_t)ib + i] = sh.item_idx[i]; item_pos[(size_t)ib + i] = sh.item_pos[i]; }
+            } else {
+                for (int i = threadIdx.x; i < G::NROW * G::RS / 4; i += G::NT) reinterpret_cast<int*>(reach)[i] = 0;
+                if (threadIdx.x == 0) kept = 0;
+                __syncthreads();
+                for (int i = threadIdx.x; i < nc; i += G::NT) {
+                    const int cell = sh.col_pos[i] & COL_CELL, y = cell % G::RS, row = cell - y;
+                    for (int yy = max(y - G::HY, 0); yy <= min(y + G::HY, G::RS - 1); ++yy) reach[row + yy] = 1;
+                }
+                __syncthreads();
+                for (int i0 = 0; i0 < nitem; i0 += G::NT) {
+                    const int i = i0 + (int)threadIdx.x;
+                    bool keep = false;
+                    unsigned pos = 0;
+                    if (i < nitem) {
+                        pos = sh.item_pos[i];
+                        const int cell = pos & 0x0fffu, y = cell % G::RS, r = cell / G::RS, rz = r / G::RX, rx = r - rz * G::RX;
+                        const bool pair = (pos & ITEM_PAIR) != 0 && y + 1 < G::RS;
+                        for (int dz = -G::HZ; dz <= G::HZ; ++dz)
+                            for (int dx = -G::HX; dx <= G::HX; ++dx) {
+                                const int z2 = rz + dz, x2 = rx + dx;
+                                if (z2 < 0 || z2 >= G::RZ || x2 < 0 || x2 >= G::RX) continue;
+                                const int c2 = (z2 * G::RX + x2) * G::RS + y;
+                                keep = keep || reach[c2] != 0 || (pair && reach[c2 + 1] != 0);
+                            }
+                    }
+                    const unsigned long long m = __ballot(keep);
+                    int base = 0;
+                    if (lane_id() == 0 && m) base = atomicAdd(&kept, __popcll(m));
+                    base = __shfl(base, 0);
+                    if (keep && pass == 1) {
+                        const size_t dst = (size_t)ib + base + __popcll(m & ((1ull << lane_id()) - 1ull));
+                        item_idx[dst] = sh.item_idx[i]; item_pos[dst] = (unsigned short)pos;
+                    }
+                }
+                __syncthreads();
+                nkeep = kept;
+            }
             if (pass == 1) {
-                // list offsets are unsigned 32-bit numbers stored in the int fields of the header
-                const unsigned ib = (unsigned)off.y + (unsigned)ni, cb = (unsigned)off.z + (unsigned)ncl;
-                if (threadIdx.x == 0) win[off.x + nwin] = make_int4((int)ib, nitem, (int)cb, nc);
-                for (int i = threadIdx.x; i < nitem; i += G::NT) { item_idx[(size_t)ib + i] = sh.item_idx[i]; item_pos[(size_t)ib + i] = sh.item_pos[i]; }
+                if (threadIdx.x == 0) win[off.x + nwin] = make_int4((int)ib, nkeep, (int)cb, nc);
                 for (int i = threadIdx.x; i < nc; i += G::NT) { col_idx[(size_t)cb + i] = sh.col_idx[i]; col_pos[(size_t)cb + i] = sh.col_pos[i]; }
             }
-            ++nwin; ni += nitem; ncl += nc;
+            ++nwin; ni += nkeep; ncl += nc;
         }
         __syncthreads();
         close_window<G>(sh);
