@@ -183,11 +183,12 @@ bool try_conv111_mfma<float>(const float* src, int64_t lds, int Csrc, const floa
 }
 
 // gw[co][ci] += sum_i gy[co][i] * x[ci][i] over [begin, end): 8x8 register tile per thread, block
-// reduction through LDS, one atomic per (co, ci) and block.
+// reduction through LDS; then one atomic per (co, ci) and block, or - with `part` - the block's sum goes to
+// part[blockIdx.x][co][ci] for conv111_dw_reduce_kernel to add up in a fixed order (same bits on every run).
 template <typename T>
 __global__ void __launch_bounds__(TB1)
 conv111_dw_kernel(const T* __restrict__ x, int64_t ldx, int Cin, const T* __restrict__ gy, int64_t ldy, int Cout,
-                  typename Num<T>::acc* __restrict__ gw, int64_t begin, int64_t end) {
+                  typename Num<T>::acc* __restrict__ gw, typename Num<T>::acc* __restrict__ part, int64_t begin, int64_t end) {
     typedef typename Num<T>::acc A;          // bfloat16 features: fp32 products, sums and weight gradient
     constexpr int B = 8;
     __shared__ A red[TB1 / 64][B * B];
@@ -224,8 +225,45 @@ conv111_dw_kernel(const T* __restrict__ x, int64_t ldx, int Cin, const T* __rest
 #pragma unroll
         for (int wv = 0; wv < TB1 / 64; ++wv) s += red[wv][threadIdx.x];
         const int a = threadIdx.x / B, b = threadIdx.x % B;
-        if (co0 + a < Cout && ci0 + b < Cin) atomicAdd(&gw[(int64_t)(co0 + a) * Cin + (ci0 + b)], s);
+        if (co0 + a < Cout && ci0 + b < Cin) {
+            const int64_t e = (int64_t)(co0 + a) * Cin + (ci0 + b);
+            if (part) part[(int64_t)blockIdx.x * Cout * Cin + e] = s;
+            else atomicAdd(&gw[e], s);
+        }
     }
+}
+
+// gw[e] += part[0][e] + part[1][e] + ... in that order
+template <typename A>
+__global__ void __launch_bounds__(TB1)
+conv111_dw_reduce_kernel(const A* __restrict__ part, int nblocks, int n, A* __restrict__ gw) {
+    const int e = blockIdx.x * TB1 + threadIdx.x;
+    if (e >= n) return;
+    A s = 0;
+    for (int b = 0; b < nblocks; ++b) s += part[(int64_t)b * n + e];
+    gw[e] += s;
+}
+
+int bwd_deterministic();
+
+// the weight gradient of one segment, by partial sums per workgroup (default) or by atomic additions
+template <typename T>
+static int launch_conv111_dw(aprnet_plan* p, const T* x, int64_t ldx, int Cin, const T* gy, int64_t ldy, int Cout,
+                             typename Num<T>::acc* gw, int64_t begin, int64_t end, hipStream_t st) {
+    typedef typename Num<T>::acc A;
+    const int64_t n = end - begin;
+    dim3 g2((unsigned)std::min<int64_t>((n + TB1 * 8 - 1) / (TB1 * 8), 256), (unsigned)((Cout + 7) / 8), (unsigned)((Cin + 7) / 8));
+    if (!bwd_deterministic()) {
+        hipLaunchKernelGGL(conv111_dw_kernel<T>, g2, dim3(TB1), 0, st, x, ldx, Cin, gy, ldy, Cout, gw, (A*)nullptr, begin, end);
+        return 0;
+    }
+    ScratchLease lease;
+    if (int rc = lease.acquire(p, (size_t)g2.x * Cout * Cin * sizeof(A), st)) return rc;
+    A* part = (A*)p->d_scratch;
+    hipLaunchKernelGGL(conv111_dw_kernel<T>, g2, dim3(TB1), 0, st, x, ldx, Cin, gy, ldy, Cout, gw, part, begin, end);
+    hipLaunchKernelGGL(conv111_dw_reduce_kernel<A>, dim3((unsigned)((Cout * Cin + TB1 - 1) / TB1)), dim3(TB1), 0, st, part, (int)g2.x,
+                       Cout * Cin, gw);
+    return 0;
 }
 
 struct Segment { int64_t begin, end; int stencil; };
@@ -288,10 +326,8 @@ int conv111_bwd(const aprnet_plan* p, int d, const T* x, int64_t ldx, int Cin, c
         if (!try_conv111_mfma<T>(gy, ldy, Cout, ws, 1, Cin, (const T*)nullptr, gx, ldgx, Cin, sg.begin, sg.end, st))
             hipLaunchKernelGGL((conv111_kernel<T, OB>), grid, dim3(TB1), 0, st, gy, ldy, Cout, ws, 1, Cin, (const T*)nullptr, gx, ldgx, Cin,
                                sg.begin, sg.end, 0);
-        const int64_t n = sg.end - sg.begin;
-        dim3 g2((unsigned)std::min<int64_t>((n + TB1 * 8 - 1) / (TB1 * 8), 256), (unsigned)((Cout + 7) / 8), (unsigned)((Cin + 7) / 8));
-        hipLaunchKernelGGL(conv111_dw_kernel<T>, g2, dim3(TB1), 0, st, x, ldx, Cin, gy, ldy, Cout,
-                           gw + (int64_t)sg.stencil * Cout * Cin, sg.begin, sg.end);
+        if (int rc = launch_conv111_dw<T>(const_cast<aprnet_plan*>(p), x, ldx, Cin, gy, ldy, Cout, gw + (int64_t)sg.stencil * Cout * Cin,
+                                          sg.begin, sg.end, st)) return rc;
     }
     APRNET_LAUNCH_CHECK("conv111 backward kernels");
     return 0;
@@ -332,10 +368,8 @@ int conv111_bwd_bf16(const aprnet_plan* p, int d, const bf16_t* x, int64_t ldx, 
             hipLaunchKernelGGL((conv111_kernel<bf16_t, 16>), grid, dim3(TB1), 0, st, gy, ldy, Cout, ws, 1, Cin, (const float*)nullptr, gx, ldgx, Cin,
                                sg.begin, sg.end, 0);
         }
-        const int64_t n = sg.end - sg.begin;
-        dim3 g2((unsigned)std::min<int64_t>((n + TB1 * 8 - 1) / (TB1 * 8), 256), (unsigned)((Cout + 7) / 8), (unsigned)((Cin + 7) / 8));
-        hipLaunchKernelGGL(conv111_dw_kernel<bf16_t>, g2, dim3(TB1), 0, st, x, ldx, Cin, gy, ldy, Cout,
-                           gw + (int64_t)sg.stencil * Cout * Cin, sg.begin, sg.end);
+        if (int rc = launch_conv111_dw<bf16_t>(const_cast<aprnet_plan*>(p), x, ldx, Cin, gy, ldy, Cout, gw + (int64_t)sg.stencil * Cout * Cin,
+                                               sg.begin, sg.end, st)) return rc;
     }
     APRNET_LAUNCH_CHECK("conv111 backward kernels");
     return 0;

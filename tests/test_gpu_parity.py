@@ -772,6 +772,39 @@ def test_conv_backward_fp32_repeats_bit_for_bit_on_odd_sizes(bt, ksize):
     close(gw_a.permute(2, 0, 1, 3, 4, 5), gw_ref, torch.float32)
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64, torch.bfloat16], ids=["f32", "f64", "bf16"])
+def test_conv111_backward_repeats_bit_for_bit(dtype):
+    """The 1x1x1 weight gradient is summed from per-workgroup partials in a fixed order (each level range adds to its
+    stencil's slot in turn) and the input gradient has one writer per element: three runs give identical bits, equal
+    within the stated tolerance to the oracle and to the run with atomic additions (aprnet_set_conv_path(11))."""
+    cin, cout = 12, 20
+    cd = torch.float32 if dtype == torch.bfloat16 else dtype
+    x, aprs, ld, w = _conv_case([("3d_t", 0), ("3d_a", 1), ("3d_s", 0)], (1, 1, 1), 2, cin, cout, cd)
+    g = torch.Generator().manual_seed(33)
+    go = torch.randn(x.size(0), cout, x.size(2), dtype=cd, generator=g)
+    if dtype == torch.bfloat16:
+        x, go = x.to(dtype).float(), go.to(dtype).float()          # the oracle sees the rounded values
+    gx_ref, gw_ref = oracle.conv_backward(aprs, x, w, go, ld)
+    wd = w.permute(1, 2, 0, 3, 4, 5).contiguous().to(DEV)
+    xd, god = x.to(dtype).to(DEV), go.to(dtype).to(DEV)
+    runs = [_ops.conv_backward(aprs, xd, wd, god, ld) for _ in range(3)]
+    for gx, gw in runs[1:]:
+        assert torch.equal(gx, runs[0][0]) and torch.equal(gw, runs[0][1])
+    lib = _native.hip()
+    assert lib.aprnet_set_conv_path(11) == 0
+    try:
+        gx_a, gw_a = _ops.conv_backward(aprs, xd, wd, god, ld)
+    finally:
+        lib.aprnet_set_conv_path(10)
+    assert torch.equal(gx_a, runs[0][0])
+    for gw in (runs[0][1], gw_a):
+        close(gw.permute(2, 0, 1, 3, 4, 5), gw_ref, cd)
+    if dtype == torch.bfloat16:
+        close_bf16(runs[0][0], gx_ref)
+    else:
+        close(runs[0][0], gx_ref, dtype)
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
 @pytest.mark.parametrize("ksize", [(3, 3, 3), (1, 3, 3), (1, 5, 5)], ids=KID)
 @pytest.mark.parametrize("cin,cout", [(1, 16), (1, 32), (2, 5), (3, 24), (2, 40)])
