@@ -498,13 +498,9 @@ template <class G, int COH, int NB, bool FUSE, int MODE, bool IL, bool BIG, clas
 __device__ __forceinline__ void mfma_bf16_window(const ConvArgs<bf16_t>& a, int co0, int nc, int nitem, bool tree_items, int first,
                                                  const uint4* __restrict__ wl, const Lists& sh,
                                                  uint4* __restrict__ patch16, uint4* __restrict__ Wl16,
-                                                 const float* __restrict__ bias_l) {
+                                                 const float* __restrict__ bias_l, const int* __restrict__ toff_l) {
     constexpr int NSTEP = bf16_steps<G>();
     const int lane = lane_id();
-    // cell offset of this lane group's tap in every step (tap 4 * step + lane / 16)
-    int toff[NSTEP];
-#pragma unroll
-    for (int st = 0; st < NSTEP; ++st) toff[st] = tap_offset_rt<G>(4 * st + (lane >> 4));
     constexpr int NBA = NB > 0 ? NB : 1;
     int bbase[NBA], ocol[NBA];
     if constexpr (IL) {
@@ -577,9 +573,10 @@ __device__ __forceinline__ void mfma_bf16_window(const ConvArgs<bf16_t>& a, int 
             bf16x8 av[COH];
 #pragma unroll
             for (int h = 0; h < COH; ++h) av[h] = __builtin_bit_cast(bf16x8, Wl16[(st * COH + h) * 64 + lane]);
+            const int toff = toff_l[st * 4 + (lane >> 4)];       // cell offset of this lane group's tap (4 * step + lane / 16)
 #pragma unroll
             for (int j = 0; j < NB; ++j) {
-                const bf16x8 bv = __builtin_bit_cast(bf16x8, patch16[bbase[j] + toff[st]]);
+                const bf16x8 bv = __builtin_bit_cast(bf16x8, patch16[bbase[j] + toff]);
 #pragma unroll
                 for (int h = 0; h < COH; ++h) acc[j][h] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(av[h], bv, acc[j][h], 0, 0, 0);
             }
@@ -666,6 +663,10 @@ conv_mfma_bf16_kernel(const ConvArgs<bf16_t> a) {
         bias_l[threadIdx.x] = (MODE == 0 && a.bias && co0 + (int)threadIdx.x < a.Cout) ? a.bias[co0 + threadIdx.x] : 0.f;
 
     __shared__ int4 hdr[16];                  // headers of sixteen windows: one round trip instead of one per window
+    // tap offsets per step and lane group: a table in LDS costs one read per step and saves the registers of a
+    // per-lane copy through the whole kernel (the 16-output form no longer spills inside its matrix phase)
+    __shared__ int toff_l[NSTEP * 4];
+    if (threadIdx.x < NSTEP * 4) toff_l[threadIdx.x] = tap_offset_rt<G>(threadIdx.x);
     const int wb = a.tile_win[blockIdx.x], we = a.tile_win[blockIdx.x + 1];
     for (int w = wb; w < we; ++w) {
         const int win = w - wb;
@@ -681,11 +682,11 @@ conv_mfma_bf16_kernel(const ConvArgs<bf16_t> a) {
         const int first = (wave - (int)blockIdx.x - win) & (G::NWAVE - 1);
         const int nb = first < nblk ? (nblk - first + G::NWAVE - 1) / G::NWAVE : 0;
         switch (__builtin_amdgcn_readfirstlane(nb)) {
-            case 0: mfma_bf16_window<G, COH, 0, FUSE, MODE, IL, BIG>(a, co0, nc, nitem, tree_items, first, wl, gl, patch16, Wl16, bias_l); break;
-            case 1: mfma_bf16_window<G, COH, 1, FUSE, MODE, IL, BIG>(a, co0, nc, nitem, tree_items, first, wl, gl, patch16, Wl16, bias_l); break;
-            case 2: mfma_bf16_window<G, COH, 2, FUSE, MODE, IL, BIG>(a, co0, nc, nitem, tree_items, first, wl, gl, patch16, Wl16, bias_l); break;
-            case 3: mfma_bf16_window<G, COH, 3, FUSE, MODE, IL, BIG>(a, co0, nc, nitem, tree_items, first, wl, gl, patch16, Wl16, bias_l); break;
-            default: mfma_bf16_window<G, COH, 4, FUSE, MODE, IL, BIG>(a, co0, nc, nitem, tree_items, first, wl, gl, patch16, Wl16, bias_l); break;
+            case 0: mfma_bf16_window<G, COH, 0, FUSE, MODE, IL, BIG>(a, co0, nc, nitem, tree_items, first, wl, gl, patch16, Wl16, bias_l, toff_l); break;
+            case 1: mfma_bf16_window<G, COH, 1, FUSE, MODE, IL, BIG>(a, co0, nc, nitem, tree_items, first, wl, gl, patch16, Wl16, bias_l, toff_l); break;
+            case 2: mfma_bf16_window<G, COH, 2, FUSE, MODE, IL, BIG>(a, co0, nc, nitem, tree_items, first, wl, gl, patch16, Wl16, bias_l, toff_l); break;
+            case 3: mfma_bf16_window<G, COH, 3, FUSE, MODE, IL, BIG>(a, co0, nc, nitem, tree_items, first, wl, gl, patch16, Wl16, bias_l, toff_l); break;
+            default: mfma_bf16_window<G, COH, 4, FUSE, MODE, IL, BIG>(a, co0, nc, nitem, tree_items, first, wl, gl, patch16, Wl16, bias_l, toff_l); break;
         }
         __syncthreads();        // the next window rewrites the patch
     }
