@@ -435,11 +435,15 @@ __device__ __forceinline__ void fetch_slots(const Lists& sh, int nitem, ItemRegs
         const __amdgpu_buffer_rsrc_t ri = __builtin_amdgcn_make_buffer_rsrc(const_cast<int*>(sh.item_idx), 0, nitem * 4, 0x00020000);
         const __amdgpu_buffer_rsrc_t rp = __builtin_amdgcn_make_buffer_rsrc(const_cast<unsigned short*>(sh.item_pos), 0, nitem * 2, 0x00020000);
         int idx[NR], pos[NR];
+        // the list offsets are formed from this copy of the thread index on every call: kept across the window loop
+        // they are spilled, and a reload from scratch before a list load makes that load wait for the one before it
+        int tid = threadIdx.x;
+        asm volatile("" : "+v"(tid));
 #pragma unroll
         for (int k = 0; k < NR; ++k) {
             idx[k] = 0; pos[k] = 0;
             if ((round0 + k) * G::NT >= nitem) continue;    // wave-uniform
-            const int it = threadIdx.x + (round0 + k) * G::NT;
+            const int it = tid + (round0 + k) * G::NT;
             idx[k] = __builtin_amdgcn_raw_buffer_load_b32(ri, it * 4, 0, 0);
             pos[k] = (int)__builtin_amdgcn_raw_buffer_load_b16(rp, it * 2, 0, 0);
         }

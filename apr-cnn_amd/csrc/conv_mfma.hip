@@ -411,11 +411,13 @@ __device__ __forceinline__ void fetch_slots16(const Lists& sh, int nitem, ItemRe
     const __amdgpu_buffer_rsrc_t ri = __builtin_amdgcn_make_buffer_rsrc(const_cast<int*>(sh.item_idx), 0, nitem * 4, 0x00020000);
     const __amdgpu_buffer_rsrc_t rp = __builtin_amdgcn_make_buffer_rsrc(const_cast<unsigned short*>(sh.item_pos), 0, nitem * 2, 0x00020000);
     int idx[IPT], pos[IPT];
+    int tid = threadIdx.x;
+    asm volatile("" : "+v"(tid));                       // offsets formed per call, not kept (and spilled) across the window loop
 #pragma unroll
     for (int k = 0; k < IPT; ++k) {
         idx[k] = 0; pos[k] = 0;
         if (k * G::NT >= nitem) continue;               // wave-uniform
-        const int it = threadIdx.x + k * G::NT;
+        const int it = tid + k * G::NT;
         idx[k] = __builtin_amdgcn_raw_buffer_load_b32(ri, it * 4, 0, 0);
         pos[k] = (int)__builtin_amdgcn_raw_buffer_load_b16(rp, it * 2, 0, 0);
     }
