@@ -11,6 +11,7 @@
 #include "conv_common.hpp"
 
 #include <atomic>
+#include <cstdlib>
 
 namespace aprnet {
 
@@ -500,6 +501,12 @@ int aprnet_conv_fwd_fused_f64(const aprnet_plan* p, int d, int kz, int kx, int k
     return conv_fwd<double>(p, d, kz, kx, ky, x, ldx, Cin, w, S_exp, Cout, bias, y, ldy, tree_ws, ldt, (hipStream_t)st, fu);
 }
 int aprnet_set_conv_path(int path) {
+    // process-wide, so a caller that is not a test or a measurement has no business here: the switch answers only in a
+    // process that asked for it through its environment before the first call
+    static const bool testing = [] { const char* e = getenv("APRNET_TESTING"); return e && e[0] && !(e[0] == '0' && !e[1]); }();
+    if (!testing)
+        return fail(APRNET_ERR_UNSUPPORTED, "set_conv_path: the kernel-selection switch is for tests and measurements; "
+                                            "it answers only when the process runs with APRNET_TESTING=1 in its environment");
     if (path == 2 || path == 3) { g_bf16_math = path == 2; return 0; }
     if (path == 4 || path == 5) { g_use_lists = path == 4; return 0; }
     if (path == 6 || path == 7) { g_bwd_overlap = path == 6; return 0; }

@@ -90,7 +90,9 @@ int aprnet_plan_children(const aprnet_plan* plan, int32_t* out_host);
 int aprnet_profile_enable(int on);
 /* No counterpart in the reference.  A knob for TESTS AND MEASUREMENTS, not part of the operator interface: it selects
  * between kernels that compute the same results, process-wide (atomic flags; a call in flight keeps the choice it read),
- * so that tests can cover every kernel family and benchmarks can compare them.  Callers of the operators never need it.
+ * so that tests can cover every kernel family and benchmarks can compare them.  Callers of the operators never need it,
+ * and it answers only in a process started with APRNET_TESTING=1 in its environment (read once, at the first call);
+ * everywhere else it returns APRNET_ERR_UNSUPPORTED and changes nothing.
  * Selects the convolution kernels: 0 = matrix-core (MFMA) kernels where one
  * exists for the stencil and element type, VALU kernels otherwise (default); 1 = VALU kernels only.
  * Independently, for bfloat16 features: 2 = bfloat16 matrix instructions (default), 3 = fp32 matrix
@@ -107,7 +109,9 @@ int aprnet_profile_enable(int on);
  * of scratch), 11 = atomic additions; and for forward layers of 1 to 3 input channels (bound by memory, not by the
  * contraction): 12 = the pipelined kernel with the (tap, channel) axis flattened (default), 13 = the general kernel;
  * and for the bfloat16 forward kernel on grouped tensors: 14 = 32-bit byte offsets where a group holds fewer than 2^28
- * elements, 64-bit addresses beyond (default), 15 = 64-bit addresses always.
+ * elements, 64-bit addresses beyond (default), 15 = 64-bit addresses always; and for the tree fill that precedes a
+ * forward stencil convolution: 16 = fill the nodes that the kernel's window lists read, and their descendants (default;
+ * the node lists are built with the window lists and kept in the plan, 4 bytes per needed node), 17 = fill every node.
  * All are HIP kernels; the switch
  * exists so that tests can cover them and memory-bound callers can do without the lists. */
 int aprnet_set_conv_path(int path);

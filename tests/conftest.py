@@ -3,6 +3,9 @@ import sys
 
 import pytest
 
+# the kernel-selection switch of the library (aprnet_set_conv_path) answers only in a process that asks for it
+os.environ.setdefault("APRNET_TESTING", "1")
+
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 for p in (ROOT, os.path.join(ROOT, "apr-cnn_amd"), os.path.join(ROOT, "tests")):
     if p not in sys.path:

@@ -186,3 +186,25 @@ def test_compiled_binding_exposes_the_reference_names():
     assert m.utils.number_particles(apr, 0) == apr.total_number_particles()
     with pytest.raises(RuntimeError, match="CUDA tensor"):          # CHECK_INPUT, cuda/src/common.hpp:14-16
         m.cuda.conv333_forward([apr], torch.zeros(1, 1, 4), torch.zeros(1, 1, 1, 3, 3, 3), torch.zeros(1, dtype=torch.int32))
+
+
+def test_kernel_selection_switch_answers_only_in_a_testing_process():
+    """aprnet_set_conv_path is process-wide, so it is shut unless the process asked for it: without APRNET_TESTING=1
+    in the environment every value is refused (and nothing changes), with it the documented values are taken and
+    unknown ones are refused.  Checked in fresh processes, because the flag is read once."""
+    import subprocess
+    import sys
+    code = ("import ctypes, sys; lib = ctypes.CDLL(sys.argv[1]); "
+            "print(lib.aprnet_set_conv_path(1), lib.aprnet_set_conv_path(0), lib.aprnet_set_conv_path(17), "
+            "lib.aprnet_set_conv_path(16), lib.aprnet_set_conv_path(99))")
+    def run(env_value):
+        env = {k: v for k, v in os.environ.items() if k != "APRNET_TESTING"}
+        if env_value is not None:
+            env["APRNET_TESTING"] = env_value
+        out = subprocess.run([sys.executable, "-c", code, LIB], env=env, capture_output=True, text=True, timeout=120)
+        assert out.returncode == 0, out.stderr
+        return [int(v) for v in out.stdout.split()]
+    for off in (None, "0", ""):
+        assert all(rc != 0 for rc in run(off))
+    on = run("1")
+    assert on[:4] == [0, 0, 0, 0] and on[4] != 0
