@@ -13,7 +13,12 @@
  *    device memory.  All other pointers are DEVICE pointers owned by the caller.
  *  - Operators work on ONE batch item: features are `C` channel planes of `n` particles, plane `c`
  *    starting at `base + c*ld` (ld in elements).  The reference's batch loop
- *    (conv.hpp:99, wrap_conv_gpu.hpp:23-28) stays on the caller's side.
+ *    (conv.hpp:99, wrap_conv_gpu.hpp:23-28) stays on the caller's side.  Every `ld` is checked against the
+ *    number of elements the operator touches per channel at its level delta (aprnet_number_parts, the tree
+ *    size, the image size) before anything is launched: a shorter row is APRNET_ERR_INVALID_ARGUMENT with
+ *    both numbers in the message, as the reference refuses tensors whose shape does not match (conv.hpp:63-66).
+ *  - Work-space contents: the stencil convolutions fill the mean tree in `tree_ws` only at the nodes their
+ *    kernels read (the others keep what the buffer held); callers must not rely on it afterwards.
  *  - `level_delta` d is the number of finest levels pooled away (helpers.hpp:86-117);
  *    Lc = level_max - d.  A feature vector at d holds aprnet_number_parts(plan, d) values.
  *  - No function allocates caller-visible memory; work space is passed in.  Kernels are enqueued
