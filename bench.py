@@ -42,7 +42,7 @@ PEAK_HBM_GBS = 8000.0
 # profiler passes, scaled by what the same counters read for a device-to-device copy of known size
 # (profiles/conv333_fwd_32x32_f32_blobs512_hbm_traffic.txt).  Counters cannot be read from inside this script: the
 # figure is a constant taken from that profile and only reported when the workload is the one it was measured on.
-PROFILED_TRAFFIC_BYTES = {23245996: 29.62e9 + 4.01e9}
+PROFILED_TRAFFIC_BYTES = {23245996: 27.18e9 + 3.91e9}
 
 
 # ------------------------------------------------------------------------------------------------ workloads
