@@ -1,8 +1,9 @@
-"""BASELINE configs[2] and configs[4] at their full size (360 M and 246 M particles), where the CPU oracle cannot be
-the checker: properties that hold at any size and that a wrong index, a dropped window or a 32-bit overflow at these
-particle counts would break.  (configs[0] and configs[1] run at full size in test_gpu_configs.py / test_gpu_fullsize.py,
-configs[3] in test_gpu_configs.py; scaled replicas of every configuration are compared with the oracle there.)
-Needs a device with about 200 GB of free memory; skipped otherwise."""
+"""BASELINE configs[2], configs[3] and configs[4] at their full size (360 M, 844 M and 246 M particles).  At 16 to 64
+channels the CPU oracle cannot be the checker there: properties that hold at any size and that a wrong index, a
+dropped window or a 32-bit overflow at these particle counts would break.  With 1 to 8 channels it can: configs[3] is
+compared with it on every particle, for the forward kernel families, the tree operators and the gradients.
+(configs[0] and configs[1] run at full size in test_gpu_configs.py / test_gpu_fullsize.py; scaled replicas of every
+configuration are compared with the oracle there.)  Needs a device with about 200 GB of free memory; skipped otherwise."""
 import pytest
 import torch
 
@@ -96,3 +97,91 @@ def test_spots16k_whole_image_identity_adjoint_and_grouped_equals_planes():
     gx, gw = _ops.conv_backward([apr], x, w, gy, ld)
     assert abs(lhs - _dot(x, gx)) <= 1e-2 * ref
     assert abs(lhs - float((w.double() * gw.double()).sum())) <= 1e-2 * ref
+
+
+def test_nuclei1024_whole_volume_conv_matches_the_oracle():
+    """configs[3], whole 1024^3 volume (844 M particles): with few channels the CPU oracle finishes in seconds at this
+    size too, so the three forward kernel families are compared with it on EVERY particle of the full-size APR -
+    the pipelined kernel for narrow inputs (1 -> 4, fp32), the general matrix-core kernel (4 -> 4, fp32; rel 1e-5 of the
+    output scale, the tolerance of the parity tests) and the bfloat16 kernel on grouped tensors in its 64-bit-address
+    form, which only APRs of 2^28 particles and more take (8 -> 8; every stored value within 1e-2 of the scale of the
+    fp32 result on the same bfloat16 inputs)."""
+    from oracle import oracle
+    _need(70)
+    apr, _ = make_config("nuclei1024")
+    apr.init_cuda()
+    n = apr.total_number_particles()
+    assert n >= 1 << 28
+    levels = apr.level_max() - apr.level_min() + 1
+    ld = torch.zeros(1, dtype=torch.int32)
+    g = torch.Generator(device=DEV).manual_seed(11)
+    gw = torch.Generator().manual_seed(12)
+
+    def compare(got, ref, tol):
+        for c in range(ref.shape[1]):                     # one channel at a time: no second copy of the tensors
+            scale = max(float(ref[0, c].abs().max()), 1e-30)
+            err = float((got[0, c].float() - ref[0, c]).abs().max())
+            assert err <= tol * scale, f"channel {c}: max abs err {err:.3e} vs scale {scale:.3e}"
+
+    x = torch.empty(1, 4, n, device=DEV).normal_(generator=g)
+    xc = x.cpu()
+    for cin, cout in ((1, 4), (4, 4)):
+        w = torch.randn(cin, levels, cout, 3, 3, 3, generator=gw) * 0.2          # oracle layout, one stencil per level
+        got = _ops.conv_forward([apr], x[:, :cin].contiguous(), w.permute(1, 2, 0, 3, 4, 5).contiguous().to(DEV), ld).cpu()
+        ref = oracle.conv_forward([apr], xc[:, :cin].contiguous(), w, ld)
+        compare(got, ref, 1e-5)
+        del got, ref
+    del x, xc
+    torch.cuda.empty_cache()
+    xb = torch.empty(1, 8, n, device=DEV, dtype=torch.bfloat16).normal_(generator=g)
+    w = (torch.randn(8, levels, 8, 3, 3, 3, generator=gw) * 0.2).to(torch.bfloat16).float()
+    yg = g8.conv_forward([apr], g8.regroup(xb), w.permute(1, 2, 0, 3, 4, 5).contiguous().to(DEV), ld)
+    got = g8.ungroup(yg).cpu()
+    del yg
+    ref = oracle.conv_forward([apr], xb.float().cpu(), w, ld)
+    compare(got, ref, 1e-2)
+
+
+def test_nuclei1024_whole_volume_tree_operators_and_gradients_match_the_oracle():
+    """configs[3], whole volume, against the oracle on every element: the mean-filled tree, max pool with its argmax
+    and the upsampling of the pooled tensor are bit-identical (same candidate and summation order); the gradients of
+    the 4 -> 4 fp32 stencil convolution are compared with the oracle run in float64 on the same values: input gradient to
+    rel 1e-5 of its scale, weight gradient (8.4e8 terms per element) to 1e-4."""
+    from oracle import oracle
+    _need(70)
+    apr, _ = make_config("nuclei1024")
+    apr.init_cuda()
+    n, c = apr.total_number_particles(), 2
+    levels = apr.level_max() - apr.level_min() + 1
+    ld0, ld1 = torch.zeros(1, dtype=torch.int32), torch.ones(1, dtype=torch.int32)
+    g = torch.Generator(device=DEV).manual_seed(21)
+    x = torch.empty(1, c, n, device=DEV).normal_(generator=g)
+    xc = x.cpu()
+    lib, plan, st = _ops._lib(), apr.plan(0), torch.cuda.current_stream().cuda_stream
+    nt = _ops.tree_parts(apr, 0)
+    tree = torch.empty(c, nt, device=DEV)
+    assert lib.aprnet_fill_tree_mean_f32(plan, 0, x.data_ptr(), n, c, tree.data_ptr(), nt, st) == 0
+    for ch in range(c):
+        assert torch.equal(tree[ch].cpu(), oracle.fill_tree_mean(apr, xc[0, ch], 0))
+    del tree
+    pooled, idx = _ops.maxpool_forward([apr], x, ld0)
+    ref, ref_idx = oracle.maxpool_forward([apr], xc, ld0)
+    assert torch.equal(pooled.cpu(), ref) and torch.equal(idx.cpu(), ref_idx)
+    del idx, ref_idx
+    up = _ops.upsample_const_forward([apr], pooled, ld1)
+    assert torch.equal(up.cpu(), oracle.upsample_const_forward([apr], ref, ld1))
+    del up, pooled, ref, x, xc
+    torch.cuda.empty_cache()
+    x = torch.empty(1, 4, n, device=DEV).normal_(generator=g)
+    gy = torch.empty(1, 4, n, device=DEV).normal_(generator=g)
+    w = torch.randn(4, levels, 4, 3, 3, 3, generator=torch.Generator().manual_seed(22)) * 0.2
+    gx, gw = _ops.conv_backward([apr], x, w.permute(1, 2, 0, 3, 4, 5).contiguous().to(DEV), gy, ld0)
+    # the oracle in float64 on the same fp32 values: a weight gradient is a sum of 8.4e8 terms per element, which the
+    # oracle's own fp32 running sums hold to about 2e-4 of its scale only
+    gx_ref, gw_ref = oracle.conv_backward([apr], x.cpu().double(), w.double(), gy.cpu().double(), ld0)
+    for ch in range(4):
+        scale = float(gx_ref[0, ch].abs().max())
+        assert float((gx[0, ch].cpu().double() - gx_ref[0, ch]).abs().max()) <= 1e-5 * scale
+    gw = gw.permute(2, 0, 1, 3, 4, 5).cpu().double()
+    # every element sums 8.4e8 products of fp32 values: 1e-4 of the scale (measured 1.7e-5; the reference's fp32 order 2e-4)
+    assert float((gw - gw_ref).abs().max()) <= 1e-4 * float(gw_ref.abs().max())
