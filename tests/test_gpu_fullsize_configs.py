@@ -15,6 +15,9 @@ DEV = "cuda:0"
 
 
 def _need(gb):
+    import gc
+    gc.collect()
+    torch.cuda.empty_cache()                  # what earlier tests left in torch's cache counts as free
     free, _total = torch.cuda.mem_get_info()
     if free < gb * 1e9:
         pytest.skip(f"needs about {gb} GB of free device memory, {free / 1e9:.0f} GB available")
@@ -32,7 +35,8 @@ def _absdot(a, b):
 def test_nuclei2048_whole_volume_tree_fill_and_conv_properties():
     """configs[2], whole 2048 x 2048 x 512 volume, 16 channels fp32: the tree mean of a constant field is that constant
     on every node, bit for bit; the identity stencil returns its input exactly (every particle is visited once and
-    reads its own cell); the parent-reading convolution is finite and repeats bit for bit."""
+    reads its own cell); the parent-reading convolution is finite and repeats bit for bit; with four channels it is
+    compared with the CPU oracle on every particle."""
     _need(150)
     apr, _ = make_config("nuclei2048")
     apr.init_cuda()
@@ -59,12 +63,22 @@ def test_nuclei2048_whole_volume_tree_fill_and_conv_properties():
     assert bool(torch.isfinite(y).all()) and float(y.abs().max()) > 0
     y2 = _ops.conv_forward([apr], x, wr, ld)
     assert torch.equal(y, y2)
+    del y, y2
+    # with four channels the CPU oracle finishes in seconds at this size: every particle, rel 1e-5 of the output scale
+    from oracle import oracle
+    w4 = torch.randn(4, levels, 4, 3, 3, 3, generator=torch.Generator().manual_seed(4)) * 0.2
+    x4 = x[:, :4].contiguous()
+    got = _ops.conv_forward([apr], x4, w4.permute(1, 2, 0, 3, 4, 5).contiguous().to(DEV), ld).cpu()
+    ref = oracle.conv_forward([apr], x4.cpu(), w4, ld)
+    for ch in range(4):
+        assert float((got[0, ch] - ref[0, ch]).abs().max()) <= 1e-5 * float(ref[0, ch].abs().max())
 
 
 def test_spots16k_whole_image_identity_adjoint_and_grouped_equals_planes():
     """configs[4], whole 16384^2 image, 1x5x5 64 -> 64 with bfloat16 features: the identity stencil copies the features
     exactly; the kernel on tensors grouped by eight channels returns bit for bit what the kernel on channel planes
-    returns; <conv(x), gy> = <x, dX> = <w, dW> to the bfloat16 rounding of the stored tensors."""
+    returns; <conv(x), gy> = <x, dX> = <w, dW> to the bfloat16 rounding of the stored tensors; with eight channels the
+    grouped kernel is compared with the CPU oracle on every particle."""
     _need(230)
     apr, _ = make_config("spots16k")
     apr.init_cuda()
@@ -97,6 +111,17 @@ def test_spots16k_whole_image_identity_adjoint_and_grouped_equals_planes():
     gx, gw = _ops.conv_backward([apr], x, w, gy, ld)
     assert abs(lhs - _dot(x, gx)) <= 1e-2 * ref
     assert abs(lhs - float((w.double() * gw.double()).sum())) <= 1e-2 * ref
+    del gx, gy
+    torch.cuda.empty_cache()
+    # eight channels against the CPU oracle on every particle (grouped tensors; stored values within 1e-2 of the scale of
+    # the fp32 result on the same bfloat16 inputs)
+    from oracle import oracle
+    x8 = x[:, :8].contiguous()
+    w8 = (torch.randn(8, levels, 8, 1, 5, 5, generator=torch.Generator().manual_seed(7)) * 0.1).to(torch.bfloat16).float()
+    got = g8.ungroup(g8.conv_forward([apr], g8.regroup(x8), w8.permute(1, 2, 0, 3, 4, 5).contiguous().to(DEV), ld)).cpu()
+    ref8 = oracle.conv_forward([apr], x8.float().cpu(), w8, ld)
+    for ch in range(8):
+        assert float((got[0, ch].float() - ref8[0, ch]).abs().max()) <= 1e-2 * float(ref8[0, ch].abs().max())
 
 
 def test_nuclei1024_whole_volume_conv_matches_the_oracle():
