@@ -50,6 +50,9 @@ struct HostAccess {
 struct bf16_t { uint16_t bits; };
 __host__ __device__ inline float bf16_to_float(bf16_t v) { return __builtin_bit_cast(float, (uint32_t)v.bits << 16); }
 __host__ __device__ inline bf16_t float_to_bf16(float f) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    return bf16_t{__builtin_bit_cast(uint16_t, (__bf16)f)};      // v_cvt_pk_bf16_f32: round to nearest even, NaN stays NaN
+#endif
     uint32_t u = __builtin_bit_cast(uint32_t, f);
     if ((u & 0x7fffffffu) > 0x7f800000u) return bf16_t{(uint16_t)((u >> 16) | 0x40u)};      // NaN stays NaN
     u += 0x7fffu + ((u >> 16) & 1u);
