@@ -481,6 +481,31 @@ def test_conv111_forward_bf16():
     close_bf16(got, ref)
 
 
+def test_bf16_results_round_to_nearest_even():
+    """What a kernel stores as bfloat16 is its fp32 result rounded to nearest, ties to even, overflow to infinity:
+    a 1x1x1 convolution of a channel of ones writes its fp32 weights, so every output equals the
+    weight rounded by torch (ties both ways, the last finite value and the first that rounds to infinity, random
+    bit patterns of normal numbers)."""
+    x, aprs, ld = batch([("3d_b", 0)], 4, torch.float32)
+    x[:] = 0
+    x[:, 0] = 1.0
+    special = [1.0, 1.0 + 2.0 ** -8, 1.0 + 3 * 2.0 ** -8, 1.0 + 2.0 ** -8 + 2.0 ** -20, 1.0 + 2.0 ** -7 - 2.0 ** -23,
+               -1.0 - 2.0 ** -8, -1.0 - 3 * 2.0 ** -8, 3.3895313892515355e38, 3.3961775292304601e38, 3.4e38, -3.4e38,
+               0.0, 2.0 ** -126, 2.0 ** -126 * (1 + 2.0 ** -8), 1e-30, 65504.0, 1.0 / 3.0]
+    g = torch.Generator().manual_seed(11)
+    bits = torch.randint(0x00800000, 0x7f000000, (64 - len(special),), generator=g, dtype=torch.int64)
+    bits = bits | (torch.randint(0, 2, bits.shape, generator=g, dtype=torch.int64) << 31)
+    rnd = (bits - (bits >> 31 << 32)).to(torch.int32).view(torch.float32)
+    w0 = torch.cat([torch.tensor(special, dtype=torch.float32), rnd])
+    w = torch.zeros(1, 64, 4, 1, 1, 1)
+    w[0, :, 0, 0, 0, 0] = w0
+    got = _ops.conv_forward(aprs, x.to(torch.bfloat16).to(DEV), w.to(DEV), ld)
+    want = w0.to(torch.bfloat16)
+    n = oracle.number_parts(aprs[0], 0)
+    for i in (0, n // 2, n - 1):
+        assert torch.equal(got[0, :, i].cpu().view(torch.int16), want.view(torch.int16)), i
+
+
 @pytest.mark.parametrize("bt", POOL_BATCHES[:4], ids=lambda b: "+".join(f"{n}@{d}" for n, d in b))
 def test_maxpool_upsample_bf16_bit_exact(bt):
     """Pool and upsample move values without arithmetic: bfloat16 results equal the oracle's on the same
