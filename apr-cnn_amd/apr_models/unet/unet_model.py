@@ -147,19 +147,35 @@ class APRUNet(nn.Module):
             level_deltas += 1
             skips.append(block(stage.conv, pooled))
             del pooled
+        hw = self.head.weight.detach().float()
+        hb = None if self.head.bias is None else self.head.bias.detach()
+
+        def last_conv_with_head(bb, inp, second=None):
+            # the network's last stencil convolution and the 1x1x1 head in one kernel: its 16 channels at full
+            # resolution are neither written nor read back
+            w = bb.conv.weight.detach().float()
+            bias = None if bb.conv.bias is None else bb.conv.bias.detach()
+            return g8.conv_head_forward(aprs, inp, restricted(bb.conv), level_deltas, bias, hw, hb, relu=True, x2=second)
+
         y = skips.pop()
-        for stage in self.decoder:
+        for si, stage in enumerate(self.decoder):
             skip = skips.pop()
             y = g8.upsample_const_forward(aprs, conv(stage.reduce_ch, y), level_deltas)
             level_deltas -= 1
-            out = conv(stage.conv.blocks[0], skip, y)
+            blocks = stage.conv.blocks
+            last = blocks[-1]
+            fuse_head = si == len(self.decoder) - 1 and tuple(last.conv.weight.shape[3:]) != (1, 1, 1) \
+                and g8.head_limits_ok(last.conv.weight.shape[1], hw)
+            if fuse_head and len(blocks) == 1:
+                return last_conv_with_head(last, skip, y)
+            out = conv(blocks[0], skip, y)
             y = skip = None
-            for bb in stage.conv.blocks[1:]:
+            for bb in blocks[1:-1] if fuse_head else blocks[1:]:
                 out = conv(bb, out)
+            if fuse_head:
+                return last_conv_with_head(last, out)
             y = out
             del out
-        hw = self.head.weight.detach().float()
-        hb = None if self.head.bias is None else self.head.bias.detach()
         return g8.conv111_forward(aprs, y, hw, level_deltas, hb, relu=False, grouped_output=False)
 
     def forward(self, x, aprs, level_deltas=None):

@@ -392,13 +392,23 @@ int conv_fwd_bf16(const aprnet_plan* cp, int d, int kz, int kx, int ky, const bf
 //   grouped output  Cout a multiple of 8
 int fill_tree_mean_g8(const aprnet_plan* p, int d, const bf16_t* x, int64_t ldx, int C, bf16_t* tree, int64_t ldt, hipStream_t st,
                       const NeedLists* need);
+// The 1x1x1 convolution that follows a layer inside its kernel (ConvArgs::head_w): out [C][ld] planes.
+struct ConvHead { const float* w = nullptr; const float* bias = nullptr; int S = 0, C = 0; bf16_t* out = nullptr; int64_t ld = 0; };
 int conv_fwd_bf16_layout(const aprnet_plan* cp, int d, int kz, int kx, int ky, const bf16_t* x, int64_t ldx, int C1, int x_g8, const float* w,
                          int S_exp, int Cout, const float* bias, bf16_t* y, int64_t ldy, int y_g8, bf16_t* tree_ws, int64_t ldt,
-                         hipStream_t st, const Fusion<bf16_t>& fu) {
+                         hipStream_t st, const Fusion<bf16_t>& fu, const ConvHead* head = nullptr) {
     aprnet_plan* p = const_cast<aprnet_plan*>(cp);
     if (int rc = check_level_delta(p, d, "conv_forward")) return rc;
     if (int rc = check_plane_size(p, d, 2, "conv_forward")) return rc;           // the plane input of a first layer: 32-bit offsets
     if (int rc = check_rows(ldx, p->number_parts(d), "conv_forward", "input")) return rc;
+    if (head) {
+        if (!head->w || !head->out || head->S <= 0 || head->C <= 0)
+            return fail(APRNET_ERR_INVALID_ARGUMENT, "conv_forward: head without weights or output");
+        if (!x_g8 || Cout > 16 || head->C > 4)
+            return fail(APRNET_ERR_UNSUPPORTED, "conv_forward: the fused head takes grouped input, at most 16 channels between "
+                                                "the two convolutions and at most 4 outputs");
+        if (int rc = check_rows(head->ld, p->number_parts(d), "conv_forward", "head output")) return rc;
+    } else
     if (int rc = check_rows(ldy, p->number_parts(d), "conv_forward", "output")) return rc;
     if (fu.C2 > 0) if (int rc = check_rows(fu.ldx2, p->number_parts(d), "conv_forward", "second input")) return rc;
     const int Cin = C1 + fu.C2;
@@ -420,6 +430,9 @@ int conv_fwd_bf16_layout(const aprnet_plan* cp, int d, int kz, int kx, int ky, c
     a.x = x; a.ldx = ldx; a.Cin = Cin; a.w = w; a.S_exp = S_exp; a.Cout = Cout; a.bias = bias; a.relu = fu.relu;
     a.y = y; a.ldy = ldy; a.y_g8 = y_g8; a.tree_data = tree_ws; a.ldt = ldt; a.Lc = p->lc(d); a.tree_off = p->tree_offset(a.Lc);
     a.x_count = p->number_parts(d); a.t_count = nt; a.c_split = C1;
+    if (head) {
+        a.head_w = head->w; a.head_b = head->bias; a.head_S = head->S; a.head_C = head->C; a.head_y = head->out; a.head_ld = head->ld;
+    }
     NeedLists need_store;
     const NeedLists* need = needed_nodes(p, d, code, tl, st, &need_store);
     if (!x_g8) {
@@ -483,6 +496,17 @@ int aprnet_conv_fwd_fused_bf16l(const aprnet_plan* p, int d, int kz, int kx, int
     if (int rc = read_fusion(fusion, &fu)) return rc;
     return conv_fwd_bf16_layout(p, d, kz, kx, ky, (const bf16_t*)x, ldx, Cin, x_grouped, w, S_exp, Cout, bias, (bf16_t*)y, ldy, y_grouped,
                                 (bf16_t*)tree_ws, ldt, (hipStream_t)st, fu);
+}
+int aprnet_conv_fwd_head_bf16g(const aprnet_plan* p, int d, int kz, int kx, int ky, const uint16_t* x, int64_t ldx, int Cin,
+                               const float* w, int S_exp, int Cout, const float* bias, uint16_t* tree_ws, int64_t ldt,
+                               const aprnet_conv_fusion* fusion, const float* head_w, int head_S, int head_C, const float* head_bias,
+                               uint16_t* out, int64_t ldo, void* st) {
+    Fusion<bf16_t> fu;
+    if (int rc = read_fusion(fusion, &fu)) return rc;
+    ConvHead head;
+    head.w = head_w; head.bias = head_bias; head.S = head_S; head.C = head_C; head.out = (bf16_t*)out; head.ld = ldo;
+    return conv_fwd_bf16_layout(p, d, kz, kx, ky, (const bf16_t*)x, ldx, Cin, 1, w, S_exp, Cout, bias, nullptr, 0, 0,
+                                (bf16_t*)tree_ws, ldt, (hipStream_t)st, fu, &head);
 }
 int aprnet_conv_fwd_fused_f32(const aprnet_plan* p, int d, int kz, int kx, int ky, const float* x, int64_t ldx, int Cin,
                               const float* w, int S_exp, int Cout, const float* bias, float* y, int64_t ldy, float* tree_ws,

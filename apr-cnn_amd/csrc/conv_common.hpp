@@ -44,6 +44,11 @@ struct ConvArgs {
     const T* xi2; int64_t xi2_ld;              // grouped second input: groups from c_split / 8 on (null: all groups in xi)
     int y_g8;                                  // bfloat16 forward: the output is grouped too, [Cout / 8][ldy][8]
     int big;                                   // bfloat16 forward on grouped input: 64-bit addresses (2^28 elements and more per group)
+    // bfloat16 forward on grouped input, at most 16 outputs: a 1x1x1 convolution of the result (after bias and clamp,
+    // rounded to bfloat16 as a stored result would be) follows inside the kernel and only its output is stored, as
+    // planes head_y [head_C][head_ld]; head_w [head_S][head_C][Cout] and head_b [head_C] (or null) in fp32; head_C <= 4.
+    // y is not written.  (null head_w: no head)
+    const float* head_w; const float* head_b; T* head_y; int64_t head_ld; int head_C, head_S;
     // backward only
     // gradients are accumulated in the computation type (fp32 for bfloat16 features)
     const T* gy; typename Num<T>::acc* gx; int64_t ldgx; typename Num<T>::acc* gtree; int64_t ldgt;

@@ -496,11 +496,14 @@ __global__ void interleave8_kernel(const bf16_t* __restrict__ x, int64_t ldx, co
 // MODE 0: forward.  MODE 1: input gradient (items = output gradient, results added atomically in fp32 to the place
 // each column names, as in the fp32 kernel; no pooled columns).
 // IL: the input comes regrouped (a.xi, a.ti), see above
-template <class G, int COH, int NB, bool FUSE, int MODE, bool IL, bool BIG, class Lists>
+// HEAD: the 1x1x1 convolution of the result follows here (see ConvArgs::head_w); head_a holds the A operands of the
+// head's weights for this tile's level (per lane: bfloat16 heads, then bfloat16 remainders), head_b4 its bias
+template <class G, int COH, int NB, bool FUSE, int MODE, bool IL, bool BIG, bool HEAD = false, class Lists>
 __device__ __forceinline__ void mfma_bf16_window(const ConvArgs<bf16_t>& a, int co0, int nc, int nitem, bool tree_items, int first,
                                                  const uint4* __restrict__ wl, const Lists& sh,
                                                  uint4* __restrict__ patch16, uint4* __restrict__ Wl16,
-                                                 const float* __restrict__ bias_l, const int* __restrict__ toff_l) {
+                                                 const float* __restrict__ bias_l, const int* __restrict__ toff_l,
+                                                 const uint4* __restrict__ head_a = nullptr, const float* __restrict__ head_b4 = nullptr) {
     constexpr int NSTEP = bf16_steps<G>();
     const int lane = lane_id();
     constexpr int NBA = NB > 0 ? NB : 1;
@@ -586,9 +589,42 @@ __device__ __forceinline__ void mfma_bf16_window(const ConvArgs<bf16_t>& a, int 
     }
 #undef APRNET_LOAD_WEIGHTS
 #undef APRNET_STORE_WEIGHTS
+    bf16x8 ha_hi, ha_lo;
+    if constexpr (HEAD) {
+        ha_hi = __builtin_bit_cast(bf16x8, head_a[lane]);
+        ha_lo = __builtin_bit_cast(bf16x8, head_a[64 + lane]);
+    }
 #pragma unroll
     for (int j = 0; j < NB; ++j) {
         const int col = ((first + G::NWAVE * j) << 4) + (lane & 15);
+        if constexpr (MODE == 0 && HEAD) {
+            // The head as one more matrix product: the lane's channels 4 g .. 4 g + 3 (g = lane / 16) of its column,
+            // rounded to bfloat16, are k-slots 8 g .. 8 g + 3 of a B operand (the other four slots are zero), the
+            // head's weights the A operand, each fp32 weight as a bfloat16 head plus a bfloat16 remainder (kept to
+            // 2^-16, as the stand-alone 1x1x1 kernel of grouped tensors keeps them); sums in fp32.  Output k of
+            // column n ends up in register k of lane n.  Every lane takes part (a matrix instruction reads the
+            // operand registers of all lanes, also of those whose column lies past the end); only the store is guarded.
+            const int g = lane >> 4;
+            float v[4];
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                v[r] = acc[j][0][r] + bias_l[4 * g + r];
+                if (a.relu) v[r] = v[r] < 0.f ? 0.f : v[r];
+            }
+            const unsigned lo = (unsigned)float_to_bf16(v[0]).bits | ((unsigned)float_to_bf16(v[1]).bits << 16);
+            const unsigned hi = (unsigned)float_to_bf16(v[2]).bits | ((unsigned)float_to_bf16(v[3]).bits << 16);
+            const bf16x8 bv = __builtin_bit_cast(bf16x8, make_uint4(lo, hi, 0u, 0u));
+            floatx4 hacc = {0.f, 0.f, 0.f, 0.f};
+            hacc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ha_hi, bv, hacc, 0, 0, 0);
+            hacc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ha_lo, bv, hacc, 0, 0, 0);
+            if (g == 0 && col < nc) {
+                const int64_t oh = ocol[j];
+#pragma unroll
+                for (int k = 0; k < 4; ++k)
+                    if (k < a.head_C) a.head_y[(int64_t)k * a.head_ld + oh] = float_to_bf16(hacc[k] + head_b4[k]);
+            }
+            continue;
+        }
         if (col >= nc) continue;
         int64_t o;
         if constexpr (IL) o = ocol[j]; else o = sh.col_idx[col];
@@ -640,7 +676,7 @@ __device__ __forceinline__ void mfma_bf16_window(const ConvArgs<bf16_t>& a, int 
 // three (80 registers, with spills): a third chain of windows per CU hides more of the memory round trips at the
 // start of every window than the spills cost (16->16 on the 23 M-particle APR 1.40 -> 1.28 ms; four workgroups at 64
 // registers: 2.39 ms; three for 32 outputs: 3.76 against 2.61 ms).
-template <class G, int COH, bool FUSE = false, int MODE = 0, bool IL = false, bool BIG = false>
+template <class G, int COH, bool FUSE = false, int MODE = 0, bool IL = false, bool BIG = false, bool HEAD = false>
 __global__ void __launch_bounds__(G::NT)
 __attribute__((amdgpu_waves_per_eu((COH == 1 && MODE == 0 && IL) ? 6 : 4, (COH == 1 && MODE == 0 && IL) ? 6 : 4)))
 conv_mfma_bf16_kernel(const ConvArgs<bf16_t> a) {
@@ -669,6 +705,27 @@ conv_mfma_bf16_kernel(const ConvArgs<bf16_t> a) {
     // per-lane copy through the whole kernel (the 16-output form no longer spills inside its matrix phase)
     __shared__ int toff_l[NSTEP * 4];
     if (threadIdx.x < NSTEP * 4) toff_l[threadIdx.x] = tap_offset_rt<G>(threadIdx.x);
+    __shared__ __attribute__((aligned(16))) uint4 head_a[HEAD ? 128 : 1];
+    __shared__ float head_b4[4];
+    if constexpr (HEAD) {
+        static_assert(COH == 1 && MODE == 0 && IL, "the head follows a forward layer of at most 16 outputs on grouped input");
+        const int hs = min(a.head_S - 1, a.Lc - L);
+        if (threadIdx.x < 64) {
+            // A[m = lane % 16][k = 8 (lane / 16) + i] = head weight of output m and channel 4 (lane / 16) + i for i < 4
+            const int m = threadIdx.x & 15, c0 = 4 * (threadIdx.x >> 4);
+            unsigned hi16[4], lo16[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const float wv = (m < a.head_C && c0 + i < a.Cout) ? a.head_w[((int64_t)hs * a.head_C + m) * a.Cout + c0 + i] : 0.f;
+                const bf16_t h = float_to_bf16(wv);
+                hi16[i] = h.bits;
+                lo16[i] = float_to_bf16(wv - bf16_to_float(h)).bits;
+            }
+            head_a[threadIdx.x] = make_uint4(hi16[0] | (hi16[1] << 16), hi16[2] | (hi16[3] << 16), 0u, 0u);
+            head_a[64 + threadIdx.x] = make_uint4(lo16[0] | (lo16[1] << 16), lo16[2] | (lo16[3] << 16), 0u, 0u);
+        }
+        if (threadIdx.x < 4) head_b4[threadIdx.x] = (a.head_b && (int)threadIdx.x < a.head_C) ? a.head_b[threadIdx.x] : 0.f;
+    }
     const int wb = a.tile_win[blockIdx.x], we = a.tile_win[blockIdx.x + 1];
     for (int w = wb; w < we; ++w) {
         const int win = w - wb;
@@ -684,11 +741,11 @@ conv_mfma_bf16_kernel(const ConvArgs<bf16_t> a) {
         const int first = (wave - (int)blockIdx.x - win) & (G::NWAVE - 1);
         const int nb = first < nblk ? (nblk - first + G::NWAVE - 1) / G::NWAVE : 0;
         switch (__builtin_amdgcn_readfirstlane(nb)) {
-            case 0: mfma_bf16_window<G, COH, 0, FUSE, MODE, IL, BIG>(a, co0, nc, nitem, tree_items, first, wl, gl, patch16, Wl16, bias_l, toff_l); break;
-            case 1: mfma_bf16_window<G, COH, 1, FUSE, MODE, IL, BIG>(a, co0, nc, nitem, tree_items, first, wl, gl, patch16, Wl16, bias_l, toff_l); break;
-            case 2: mfma_bf16_window<G, COH, 2, FUSE, MODE, IL, BIG>(a, co0, nc, nitem, tree_items, first, wl, gl, patch16, Wl16, bias_l, toff_l); break;
-            case 3: mfma_bf16_window<G, COH, 3, FUSE, MODE, IL, BIG>(a, co0, nc, nitem, tree_items, first, wl, gl, patch16, Wl16, bias_l, toff_l); break;
-            default: mfma_bf16_window<G, COH, 4, FUSE, MODE, IL, BIG>(a, co0, nc, nitem, tree_items, first, wl, gl, patch16, Wl16, bias_l, toff_l); break;
+            case 0: mfma_bf16_window<G, COH, 0, FUSE, MODE, IL, BIG, HEAD>(a, co0, nc, nitem, tree_items, first, wl, gl, patch16, Wl16, bias_l, toff_l, head_a, head_b4); break;
+            case 1: mfma_bf16_window<G, COH, 1, FUSE, MODE, IL, BIG, HEAD>(a, co0, nc, nitem, tree_items, first, wl, gl, patch16, Wl16, bias_l, toff_l, head_a, head_b4); break;
+            case 2: mfma_bf16_window<G, COH, 2, FUSE, MODE, IL, BIG, HEAD>(a, co0, nc, nitem, tree_items, first, wl, gl, patch16, Wl16, bias_l, toff_l, head_a, head_b4); break;
+            case 3: mfma_bf16_window<G, COH, 3, FUSE, MODE, IL, BIG, HEAD>(a, co0, nc, nitem, tree_items, first, wl, gl, patch16, Wl16, bias_l, toff_l, head_a, head_b4); break;
+            default: mfma_bf16_window<G, COH, 4, FUSE, MODE, IL, BIG, HEAD>(a, co0, nc, nitem, tree_items, first, wl, gl, patch16, Wl16, bias_l, toff_l, head_a, head_b4); break;
         }
         __syncthreads();        // the next window rewrites the patch
     }
@@ -754,6 +811,10 @@ static int launch_bf16(const ConvArgs<bf16_t>& a, int n_tiles, hipStream_t st, b
     } else if (dx) {
         if (coh == 1) hipLaunchKernelGGL((conv_mfma_bf16_kernel<G, 1, false, 1>), grid, dim3(G::NT), 0, st, a);
         else hipLaunchKernelGGL((conv_mfma_bf16_kernel<G, 2, false, 1>), grid, dim3(G::NT), 0, st, a);
+    } else if (a.head_w != nullptr) {       // the layer and the 1x1x1 head that follows it, grouped input, at most 16 outputs
+        if (a.xi == nullptr || coh != 1) return fail(APRNET_ERR_UNSUPPORTED, "conv_forward: the fused head takes grouped input and at most 16 channels");
+        if (a.big) hipLaunchKernelGGL((conv_mfma_bf16_kernel<G, 1, true, 0, true, true, true>), grid, dim3(G::NT), 0, st, a);
+        else hipLaunchKernelGGL((conv_mfma_bf16_kernel<G, 1, true, 0, true, false, true>), grid, dim3(G::NT), 0, st, a);
     } else if (a.xi != nullptr && a.big) {   // regrouped input of 2^28 elements and more per group: 64-bit addresses
         if (a.relu) {
             if (coh == 1) hipLaunchKernelGGL((conv_mfma_bf16_kernel<G, 1, true, 0, true, true>), grid, dim3(G::NT), 0, st, a);

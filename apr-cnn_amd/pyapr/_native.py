@@ -142,5 +142,7 @@ def hip():
     lib.aprnet_conv111_fwd_bf16g.argtypes = [vp, i32, vp, i64, i32, vp, i32, i32, vp, i32, vp, i64, i32, vp]
     lib.aprnet_conv_fwd_fused_bf16l.argtypes = [vp, i32, i32, i32, i32, vp, i64, i32, i32, vp, i32, i32, vp, vp, i64, i32,
                                                 vp, i64, vp, vp]
+    lib.aprnet_conv_fwd_head_bf16g.argtypes = [vp, i32, i32, i32, i32, vp, i64, i32, vp, i32, i32, vp, vp, i64, vp,
+                                               vp, i32, i32, vp, vp, i64, vp]
     _hip = lib
     return lib

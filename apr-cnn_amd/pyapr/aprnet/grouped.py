@@ -118,6 +118,54 @@ def conv_forward(aprs, x, weights, level_delta, bias=None, relu=False, x2=None, 
     return Grouped(out) if grouped_output else out
 
 
+def head_limits_ok(cout, head_weights):
+    """Whether conv_head_forward takes a layer of ``cout`` channels followed by this 1x1x1 head."""
+    return cout <= 16 and head_weights.shape[1] <= 4 and tuple(head_weights.shape[3:]) == (1, 1, 1) and head_weights.shape[2] == cout
+
+
+def conv_head_forward(aprs, x, weights, level_delta, bias, head_weights, head_bias=None, relu=True, x2=None):
+    """The last stencil convolution of a network and the 1x1x1 convolution that follows it (unet_model.py:94) in one
+    kernel: conv111(relu(conv(x) + bias)) without storing the layer's result.  ``x`` (and ``x2``) Grouped, weights
+    [S_exp, Cout <= 16, Cin, kz, kx, ky], head_weights [S, C <= 4, Cout, 1, 1, 1] (not expanded), fp32
+    -> [B, C, N] bfloat16 planes."""
+    _check_input(weights, "weights")
+    weights = weights.float()
+    bias = None if bias is None else bias.float().contiguous()
+    hw = head_weights.float().contiguous()
+    hb = None if head_bias is None else head_bias.float().contiguous()
+    s_exp, cout, cin, kz, kx, ky = weights.shape
+    if not head_limits_ok(cout, hw):
+        raise ValueError("the fused head takes at most 16 channels between the two convolutions and at most 4 outputs")
+    B, N = x.data.shape[0], x.data.shape[2]
+    c1, c2 = x.channels, (0 if x2 is None else x2.channels)
+    if c1 + c2 != cin:
+        raise ValueError("convolve: input tensor shape does not match weights tensor!")
+    if x2 is not None and (x2.data.shape[0] != B or x2.data.shape[2] != N):
+        raise ValueError("the second input must match the first in batch size and particle count")
+    d = _deltas(level_delta, len(aprs))
+    sizes = [number_particles(a, d[b]) for b, a in enumerate(aprs)]
+    if max(sizes) > N:
+        raise ValueError("input holds fewer particles than the APR at this level delta")
+    hs, hc = hw.shape[0], hw.shape[1]
+    out = torch.empty((B, hc, N), dtype=torch.bfloat16, device=x.data.device)
+    for b, nb in enumerate(sizes):             # slots behind a batch item's last particle, as conv111_forward leaves them
+        if nb < N:
+            out[b, :, nb:] = 0 if hb is None else hb.to(torch.bfloat16).view(-1, 1)
+    ld_tree = max(max(tree_parts(a, d[b]) for b, a in enumerate(aprs)), 1)
+    tree_ws = torch.empty((cin // 8, ld_tree, 8), dtype=torch.bfloat16, device=out.device)
+    plans = _plans(aprs, out.device)
+    with torch.cuda.device(out.device):
+        st = _stream()
+        for b in range(B):
+            fu = _ops._Fusion(_ptr(x2.data[b]) if x2 is not None else None, N, c2, 1 if relu else 0)
+            rc = _lib().aprnet_conv_fwd_head_bf16g(plans[b], d[b], kz, kx, ky, _ptr(x.data[b]), N, c1, _ptr(weights), s_exp, cout,
+                                                   None if bias is None else _ptr(bias), _ptr(tree_ws), ld_tree, C.byref(fu),
+                                                   _ptr(hw), hs, hc, None if hb is None else _ptr(hb), _ptr(out[b]), N, st)
+            if rc:
+                _raise(rc, "conv_head_forward failed")
+    return out
+
+
 def conv111_forward(aprs, x, weights, level_delta, bias=None, relu=False, grouped_output=True):
     """1x1x1 convolution of Grouped features; weights [S, Cout, Cin, 1, 1, 1] fp32 (not expanded)."""
     _check_input(weights, "weights")

@@ -311,6 +311,16 @@ int aprnet_conv111_g8_max_cin(void);
 int aprnet_conv_fwd_fused_bf16l(const aprnet_plan*, int level_delta, int kz, int kx, int ky, const uint16_t* x, int64_t ldx, int Cin,
                                 int x_grouped, const float* w, int S_exp, int Cout, const float* bias, uint16_t* y, int64_t ldy,
                                 int y_grouped, uint16_t* tree_ws, int64_t ld_tree, const aprnet_conv_fusion* fusion, void* stream);
+/* The last stencil convolution of a network together with the 1x1x1 convolution that follows it (the head of the
+ * APR-UNet: apr_models/apr_models/unet/unet_model.py:75-79, applied at :94 to the last UpConv block's output): x (and fusion->x2) grouped,
+ * Cout <= 16; the layer's result - after bias and fusion->relu, rounded to bfloat16 as aprnet_conv_fwd_fused_bf16l
+ * would store it - is not written; out [head_C][ldo] planes = Convolution<1,1,1>::forward of it with
+ * head_w [head_S][head_C][Cout] and head_bias [head_C] (or NULL), head_C <= 4, fp32 products and sums.  Saves one
+ * write and one read of the 16-channel tensor at the network's full resolution. */
+int aprnet_conv_fwd_head_bf16g(const aprnet_plan*, int level_delta, int kz, int kx, int ky, const uint16_t* x, int64_t ldx, int Cin,
+                               const float* w, int S_exp, int Cout, const float* bias, uint16_t* tree_ws, int64_t ld_tree,
+                               const aprnet_conv_fusion* fusion, const float* head_w, int head_S, int head_C,
+                               const float* head_bias, uint16_t* out, int64_t ldo, void* stream);
 
 /* Label and coordinate utilities of the StarDist networks (pyapr/aprnet/src/utils.hpp:86-333; CPU loops in the
  * reference, device kernels here).  Particle order = feature order at level_delta.  Images are dense device arrays

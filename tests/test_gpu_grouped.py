@@ -95,6 +95,55 @@ def test_grouped_convolution_with_64_bit_addresses(c1, c2, cout):
     assert torch.equal(planes, g8.conv_forward(aprs, xa, w, ld, bias, relu=False, x2=xb, grouped_output=False))
 
 
+@pytest.mark.parametrize("ksize", [(3, 3, 3), (1, 5, 5)], ids=["333", "155"])
+@pytest.mark.parametrize("c1,c2,cout,hc,hs", [(16, 0, 16, 3, 1), (16, 16, 16, 1, 2), (8, 0, 8, 4, 3), (24, 8, 16, 2, 1)])
+def test_convolution_with_fused_head_equals_the_two_operators(c1, c2, cout, hc, hs, ksize):
+    """The last stencil convolution and the 1x1x1 head in one kernel: the head sees the layer's result rounded to
+    bfloat16, as the stored tensor would hold it, and sums in fp32; against the same sums in float64 over the stored
+    result of the unfused layer the outputs agree to bfloat16 rounding (half a unit in the 8th mantissa bit of the
+    value, here 2^-8 of the row's absolute sum), also with 64-bit item addresses, where they are bit-identical."""
+    aprs, ld, x, g = _batch(c1 + c2, seed=9)
+    levels = max(a.level_max() - a.level_min() + 1 for a in aprs)
+    w = (torch.randn(levels, cout, c1 + c2, *ksize, generator=g) * 0.1).to(DEV)
+    bias = torch.randn(cout, generator=g).to(DEV)
+    hw = torch.randn(hs, hc, cout, 1, 1, 1, generator=g).to(DEV)
+    hb = torch.randn(hc, generator=g).to(DEV)
+    xa, xb = g8.regroup(x[:, :c1].contiguous()), (g8.regroup(x[:, c1:].contiguous()) if c2 else None)
+    mid = g8.ungroup(g8.conv_forward(aprs, xa, w, ld, bias, relu=True, x2=xb))            # [B, cout, N] bfloat16
+    got = g8.conv_head_forward(aprs, xa, w, ld, bias, hw, hb, relu=True, x2=xb)
+    assert got.shape == (2, hc, x.shape[2]) and got.dtype == torch.bfloat16
+    # the oracle's 1x1x1 convolution in float64 on the stored result of the unfused layer, and the same on absolute values
+    hw_cpu = hw.permute(2, 0, 1, 3, 4, 5).contiguous().double().cpu()
+    m = mid.double().cpu()
+    want = oracle.conv_forward(aprs, m, hw_cpu, ld) + hb.double().cpu().view(1, -1, 1)
+    bound = oracle.conv_forward(aprs, m.abs(), hw_cpu.abs(), ld) + hb.double().cpu().abs().view(1, -1, 1)
+    for b, apr in enumerate(aprs):
+        n = oracle.number_parts(apr, int(ld[b]))
+        err = (got[b, :, :n].double().cpu() - want[b, :, :n]).abs()
+        assert bool((err <= 2.0 ** -8 * bound[b, :, :n] + 1e-30).all()), float((err / (bound[b, :, :n] + 1e-30)).max())
+        tail = got[b, :, n:].float().cpu()
+        assert torch.equal(tail, hb.to(torch.bfloat16).float().cpu().view(-1, 1).expand_as(tail))
+    lib = _native.hip()
+    assert lib.aprnet_set_conv_path(15) == 0
+    try:
+        big = g8.conv_head_forward(aprs, xa, w, ld, bias, hw, hb, relu=True, x2=xb)
+    finally:
+        assert lib.aprnet_set_conv_path(14) == 0
+    assert torch.equal(big, got)
+
+
+def test_fused_head_refuses_what_it_does_not_take():
+    aprs, ld, x, g = _batch(32, seed=2)
+    levels = max(a.level_max() - a.level_min() + 1 for a in aprs)
+    xa = g8.regroup(x)
+    w32 = torch.randn(levels, 32, 32, 3, 3, 3, generator=g).to(DEV)
+    with pytest.raises(ValueError):
+        g8.conv_head_forward(aprs, xa, w32, ld, None, torch.randn(1, 2, 32, 1, 1, 1).to(DEV))       # 32 channels in between
+    w16 = torch.randn(levels, 16, 32, 3, 3, 3, generator=g).to(DEV)
+    with pytest.raises(ValueError):
+        g8.conv_head_forward(aprs, xa, w16, ld, None, torch.randn(1, 5, 16, 1, 1, 1).to(DEV))       # five outputs
+
+
 @pytest.mark.parametrize("cin", [1, 3])
 def test_first_layer_planes_in_grouped_out(cin):
     aprs, ld, x, g = _batch(cin, seed=3)
