@@ -805,12 +805,13 @@ def other_ops(apr, x, dev):
     torch.manual_seed(0)
     tnet = APRUNet(1, 3, depth=3, n_filters_base=16, n_stencils=2, norm="batch").to(dev).train()
     target = torch.randn(1, 3, xin.shape[2], device=dev)
+    torch.cuda.empty_cache()          # the step allocates other sizes than the inference runs before it left cached
 
     def train_step_bf16():
         for p_ in tnet.parameters():
             p_.grad = None
         torch.nn.functional.mse_loss(tnet(xinb, [apr]).float(), target).backward()
-    ms = _time(train_step_bf16, iters=2, warmup=1)
+    ms = _time(train_step_bf16, iters=3, warmup=2)
     res.append({"op": "apr_unet_train_step_bf16", "ms": ms, "particles_per_s": n0 / ms * 1e3,
                 "note": "the training step with bfloat16 features and feature gradients (fp32 parameters and accumulation)"})
     return res
