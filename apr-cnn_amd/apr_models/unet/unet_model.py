@@ -129,12 +129,12 @@ class APRUNet(nn.Module):
                 return kept[1]
             return _ops.restrict_kernel_forward(conv_module.weight.detach().float().contiguous(), levels)
 
-        def conv(bb, inp, second=None):
+        def conv(bb, inp, second=None, coarse=None):
             w = bb.conv.weight.detach().float()
             bias = None if bb.conv.bias is None else bb.conv.bias.detach()
             if tuple(w.shape[3:]) == (1, 1, 1):
                 return g8.conv111_forward(aprs, inp, w, level_deltas, bias, relu=True)
-            return g8.conv_forward(aprs, inp, restricted(bb.conv), level_deltas, bias, relu=True, x2=second)
+            return g8.conv_forward(aprs, inp, restricted(bb.conv), level_deltas, bias, relu=True, x2=second, x2_coarse=coarse)
 
         def block(cb, inp, second=None):
             for i, bb in enumerate(cb.blocks):
@@ -150,26 +150,28 @@ class APRUNet(nn.Module):
         hw = self.head.weight.detach().float()
         hb = None if self.head.bias is None else self.head.bias.detach()
 
-        def last_conv_with_head(bb, inp, second=None):
+        def last_conv_with_head(bb, inp, second=None, coarse=None):
             # the network's last stencil convolution and the 1x1x1 head in one kernel: its 16 channels at full
             # resolution are neither written nor read back
-            w = bb.conv.weight.detach().float()
             bias = None if bb.conv.bias is None else bb.conv.bias.detach()
-            return g8.conv_head_forward(aprs, inp, restricted(bb.conv), level_deltas, bias, hw, hb, relu=True, x2=second)
+            return g8.conv_head_forward(aprs, inp, restricted(bb.conv), level_deltas, bias, hw, hb, relu=True, x2=second,
+                                        x2_coarse=coarse)
 
         y = skips.pop()
         for si, stage in enumerate(self.decoder):
             skip = skips.pop()
-            y = g8.upsample_const_forward(aprs, conv(stage.reduce_ch, y), level_deltas)
+            z = conv(stage.reduce_ch, y)
+            y = g8.upsample_const_forward(aprs, z, level_deltas)
             level_deltas -= 1
+            # (the mean tree of the upsampled tensor is read off z: it holds what its nodes were upsampled from)
             blocks = stage.conv.blocks
             last = blocks[-1]
             fuse_head = si == len(self.decoder) - 1 and tuple(last.conv.weight.shape[3:]) != (1, 1, 1) \
                 and g8.head_limits_ok(last.conv.weight.shape[1], hw)
             if fuse_head and len(blocks) == 1:
-                return last_conv_with_head(last, skip, y)
-            out = conv(blocks[0], skip, y)
-            y = skip = None
+                return last_conv_with_head(last, skip, y, z)
+            out = conv(blocks[0], skip, y, z)
+            y = skip = z = None
             for bb in blocks[1:-1] if fuse_head else blocks[1:]:
                 out = conv(bb, out)
             if fuse_head:

@@ -248,6 +248,7 @@ static const NeedLists* needed_nodes(aprnet_plan* p, int d, int code, const Tile
 template <typename T>
 struct Fusion {
     const T* x2 = nullptr; int64_t ldx2 = 0; int C2 = 0; int relu = 0;
+    const T* x2_coarse = nullptr; int64_t ld_coarse = 0;      // grouped bfloat16 only: what x2 was upsampled from
 };
 template <typename T>
 static int read_fusion(const aprnet_conv_fusion* f, Fusion<T>* out) {
@@ -255,6 +256,7 @@ static int read_fusion(const aprnet_conv_fusion* f, Fusion<T>* out) {
     if (!f) return 0;
     if (f->C2 < 0 || (f->C2 > 0 && !f->x2)) return fail(APRNET_ERR_INVALID_ARGUMENT, "conv_forward: second input without data");
     if (f->C2 > 0) { out->x2 = (const T*)f->x2; out->ldx2 = f->ldx2; out->C2 = f->C2; }
+    if (f->C2 > 0 && f->x2_coarse) { out->x2_coarse = (const T*)f->x2_coarse; out->ld_coarse = f->ld_coarse; }
     out->relu = f->relu != 0;
     return 0;
 }
@@ -391,7 +393,9 @@ int conv_fwd_bf16(const aprnet_plan* cp, int d, int kz, int kx, int ky, const bf
 //   planes input    1 to 3 channels (the first layer of a network) on the pipelined kernel
 //   grouped output  Cout a multiple of 8
 int fill_tree_mean_g8(const aprnet_plan* p, int d, const bf16_t* x, int64_t ldx, int C, bf16_t* tree, int64_t ldt, hipStream_t st,
-                      const NeedLists* need);
+                      const NeedLists* need, bool particles_first = false);
+int tree_of_upsampled_g8(const aprnet_plan* p, int d, const bf16_t* z, int64_t ldz, int C, bf16_t* tree, int64_t ldt, hipStream_t st,
+                         const NeedLists* need);
 // The 1x1x1 convolution that follows a layer inside its kernel (ConvArgs::head_w): out [C][ld] planes.
 struct ConvHead { const float* w = nullptr; const float* bias = nullptr; int S = 0, C = 0; bf16_t* out = nullptr; int64_t ld = 0; };
 int conv_fwd_bf16_layout(const aprnet_plan* cp, int d, int kz, int kx, int ky, const bf16_t* x, int64_t ldx, int C1, int x_g8, const float* w,
@@ -418,6 +422,7 @@ int conv_fwd_bf16_layout(const aprnet_plan* cp, int d, int kz, int kx, int ky, c
         return fail(APRNET_ERR_UNSUPPORTED, "conv_forward: bfloat16 features are supported for the 3x3x3, 1x3x3 and 1x5x5 stencils");
     if (y_g8 && Cout % 8) return fail(APRNET_ERR_INVALID_ARGUMENT, "conv_forward: a grouped output holds a multiple of eight channels");
     if (x_g8 && (C1 % 8 || fu.C2 % 8)) return fail(APRNET_ERR_INVALID_ARGUMENT, "conv_forward: grouped inputs hold multiples of eight channels");
+    if (fu.x2_coarse && !x_g8) return fail(APRNET_ERR_UNSUPPORTED, "conv_forward: x2_coarse is taken with grouped inputs only");
     if (!x_g8 && (fu.C2 > 0 || !conv_narrow_supported(code, Cin)))
         return fail(APRNET_ERR_UNSUPPORTED, "conv_forward: a planes input with a grouped output is taken for 1 to 3 channels only");
     const int64_t nt = p->tree_parts(d);
@@ -443,8 +448,11 @@ int conv_fwd_bf16_layout(const aprnet_plan* cp, int d, int kz, int kx, int ky, c
         return done ? 0 : fail(APRNET_ERR_UNSUPPORTED, "conv_forward: the window lists of the plan are not available");
     }
     if (int rc = fill_tree_mean_g8(p, d, x, ldx, C1, tree_ws, ldt, st, need)) return rc;
-    if (fu.C2 > 0)
-        if (int rc = fill_tree_mean_g8(p, d, fu.x2, fu.ldx2, fu.C2, tree_ws + (int64_t)(C1 / 8) * ldt * 8, ldt, st, need)) return rc;
+    if (fu.C2 > 0) {
+        bf16_t* tree2 = tree_ws + (int64_t)(C1 / 8) * ldt * 8;
+        if (fu.x2_coarse) { if (int rc = tree_of_upsampled_g8(p, d, fu.x2_coarse, fu.ld_coarse, fu.C2, tree2, ldt, st, need)) return rc; }
+        else if (int rc = fill_tree_mean_g8(p, d, fu.x2, fu.ldx2, fu.C2, tree2, ldt, st, need)) return rc;
+    }
     if (tl.n == 0) return 0;
     if (int rc = set_lists(p, d, code, tl, a, st)) return rc;
     if (!a.tile_win) return fail(APRNET_ERR_UNSUPPORTED, "conv_forward: the window lists of the plan are not available");

@@ -98,16 +98,17 @@ __device__ __forceinline__ void fill_node_g8(const int32_t* children, int64_t n_
 
 __global__ void __launch_bounds__(GTB)
 fill_tree_level_g8_kernel(const int32_t* __restrict__ children, int64_t n_tree, int64_t t_begin, int64_t t_end, const bf16_t* __restrict__ x,
-                          int64_t ldx, bf16_t* __restrict__ tree, int64_t ldt, int64_t tree_off, int from_x) {
+                          int64_t ldx, bf16_t* __restrict__ tree, int64_t ldt, int64_t tree_off, int from_x, int tree_first) {
     const int64_t t = t_begin + (int64_t)blockIdx.x * GTB + threadIdx.x;
-    if (t < t_end) fill_node_g8(children, n_tree, t, x, ldx, tree, ldt, tree_off, from_x, from_x, blockIdx.y);
+    if (t < t_end) fill_node_g8(children, n_tree, t, x, ldx, tree, ldt, tree_off, from_x, tree_first, blockIdx.y);
 }
 
 __global__ void __launch_bounds__(GTB)
 fill_tree_list_g8_kernel(const int32_t* __restrict__ children, int64_t n_tree, const int32_t* __restrict__ nodes, int64_t count,
-                         const bf16_t* __restrict__ x, int64_t ldx, bf16_t* __restrict__ tree, int64_t ldt, int64_t tree_off, int from_x) {
+                         const bf16_t* __restrict__ x, int64_t ldx, bf16_t* __restrict__ tree, int64_t ldt, int64_t tree_off, int from_x,
+                         int tree_first) {
     const int64_t i = (int64_t)blockIdx.x * GTB + threadIdx.x;
-    if (i < count) fill_node_g8(children, n_tree, nodes[i], x, ldx, tree, ldt, tree_off, from_x, from_x, blockIdx.y);
+    if (i < count) fill_node_g8(children, n_tree, nodes[i], x, ldx, tree, ldt, tree_off, from_x, tree_first, blockIdx.y);
 }
 
 constexpr int G_MAX_COARSE = 12;
@@ -125,8 +126,10 @@ fill_tree_coarse_g8_kernel(const int32_t* __restrict__ children, int64_t n_tree,
 }
 
 // need: fill only the nodes a convolution reads (see need.hip); null: every node
+// particles_first: the level under the features sums its particles before its downsampled particles, as every other
+// level sums particles before tree nodes (for the tree of an upsampled tensor, see tree_of_upsampled_g8)
 int fill_tree_mean_g8(const aprnet_plan* p, int d, const bf16_t* x, int64_t ldx, int C, bf16_t* tree, int64_t ldt, hipStream_t st,
-                      const NeedLists* need) {
+                      const NeedLists* need, bool particles_first) {
     if (C <= 0 || (need && need->n_nodes == 0)) return 0;
     if (C % 8) return fail(APRNET_ERR_INVALID_ARGUMENT, "grouped features hold a multiple of eight channels");
     const int Lc = p->lc(d), G = C / 8;
@@ -148,10 +151,10 @@ int fill_tree_mean_g8(const aprnet_plan* p, int d, const bf16_t* x, int64_t ldx,
         if (need && !need->whole[l])
             hipLaunchKernelGGL(fill_tree_list_g8_kernel, dim3((unsigned)((need->cnt[l] + GTB - 1) / GTB), (unsigned)G), dim3(GTB), 0, st,
                                p->d_children, p->n_tree, need->d_nodes + need->off[l], need->cnt[l], x, ldx, tree, ldt,
-                               from_x ? p->tree_offset(Lc) : 0, from_x);
+                               from_x ? p->tree_offset(Lc) : 0, from_x, from_x && !particles_first);
         else
             hipLaunchKernelGGL(fill_tree_level_g8_kernel, dim3((unsigned)((e - b + GTB - 1) / GTB), (unsigned)G), dim3(GTB), 0, st, p->d_children,
-                               p->n_tree, b, e, x, ldx, tree, ldt, from_x ? p->tree_offset(Lc) : 0, from_x);
+                               p->n_tree, b, e, x, ldx, tree, ldt, from_x ? p->tree_offset(Lc) : 0, from_x, from_x && !particles_first);
     }
     GCoarse lv{};
     for (int l = l_coarse; l >= p->tree.level_min; --l)
@@ -159,6 +162,39 @@ int fill_tree_mean_g8(const aprnet_plan* p, int d, const bf16_t* x, int64_t ldx,
     if (lv.n > 0)
         hipLaunchKernelGGL(fill_tree_coarse_g8_kernel, dim3((unsigned)G), dim3(GTB), 0, st, p->d_children, p->n_tree, lv, x, ldx, tree, ldt);
     APRNET_LAUNCH_CHECK("fill_tree g8 kernels");
+    return 0;
+}
+
+// The mean tree of u = UpSampleConst(z) without reading u.  z lives at level delta d + 1: particles up to level Lc - 1,
+// then the nodes of level Lc - 1 in tree order ("downsampled particles").  The upsample gives all children of such a
+// node the node's value, so the node's mean in the tree of u is that value again (a sum of k <= 8 equal bfloat16
+// values and its division by k are exact in fp32), and below level Lc - 1 the tree of u is the tree of z.
+__global__ void __launch_bounds__(GTB)
+tree_level_from_coarse_g8_kernel(const int32_t* __restrict__ nodes, int64_t count, int64_t t_begin, int64_t n_copy,
+                                 const bf16_t* __restrict__ z, int64_t ldz, bf16_t* __restrict__ tree, int64_t ldt) {
+    const int64_t i = (int64_t)blockIdx.x * GTB + threadIdx.x;
+    if (i >= count) return;
+    const int64_t t = nodes ? (int64_t)nodes[i] : t_begin + i;
+    *g8_at(tree, ldt, blockIdx.y, t) = *g8_at(z, ldz, blockIdx.y, n_copy + (t - t_begin));
+}
+int tree_of_upsampled_g8(const aprnet_plan* p, int d, const bf16_t* z, int64_t ldz, int C, bf16_t* tree, int64_t ldt, hipStream_t st,
+                         const NeedLists* need) {
+    if (C <= 0 || (need && need->n_nodes == 0)) return 0;
+    if (C % 8) return fail(APRNET_ERR_INVALID_ARGUMENT, "grouped features hold a multiple of eight channels");
+    if (int rc = check_level_delta(p, d + 1, "conv_forward (x2_coarse)")) return rc;
+    if (int rc = check_rows(ldz, p->number_parts(d + 1), "conv_forward", "x2_coarse")) return rc;
+    const int Lc = p->lc(d), l = Lc - 1;
+    if (l > p->tree.level_max) return fail(APRNET_ERR_INVALID_ARGUMENT, "conv_forward: x2_coarse needs a level below the features");
+    // levels below Lc - 1: the tree of z (the lists of needed nodes name absolute levels, so they serve this fill too)
+    // (in the tree of u the nodes of level Lc - 1 are tree nodes, summed after the particles of their level)
+    if (int rc = fill_tree_mean_g8(p, d + 1, z, ldz, C, tree, ldt, st, need, true)) return rc;
+    const int64_t b = p->tree.level_begin(l), e = p->tree.level_end(l);
+    if (e <= b || (need && need->cnt[l] == 0)) return 0;
+    const bool listed = need && !need->whole[l];
+    const int64_t count = listed ? need->cnt[l] : e - b;
+    hipLaunchKernelGGL(tree_level_from_coarse_g8_kernel, dim3((unsigned)((count + GTB - 1) / GTB), (unsigned)(C / 8)), dim3(GTB), 0, st,
+                       listed ? need->d_nodes + need->off[l] : nullptr, count, b, p->apr.level_end(l), z, ldz, tree, ldt);
+    APRNET_LAUNCH_CHECK("tree_level_from_coarse_g8_kernel");
     return 0;
 }
 
@@ -438,7 +474,7 @@ int aprnet_fill_tree_mean_bf16g(const aprnet_plan* p, int d, const uint16_t* x, 
     if (int rc = check_rows(ldx, p->number_parts(d), "fill_tree_mean (grouped)", "input")) return rc;
     if (int rc = check_rows(ldt, p->tree_parts(d), "fill_tree_mean (grouped)", "tree work space")) return rc;
     APRNET_HIP_CHECK(hipSetDevice(p->device));
-    return fill_tree_mean_g8(p, d, (const bf16_t*)x, ldx, C, (bf16_t*)tree, ldt, (hipStream_t)st, nullptr);
+    return fill_tree_mean_g8(p, d, (const bf16_t*)x, ldx, C, (bf16_t*)tree, ldt, (hipStream_t)st, nullptr, false);
 }
 int aprnet_maxpool_fwd_bf16g(const aprnet_plan* p, int d, const uint16_t* x, int64_t ldx, int C, uint16_t* y, int64_t ldy, void* st) {
     if (int rc = check_level_delta(p, d, "maxpool_forward")) return rc;

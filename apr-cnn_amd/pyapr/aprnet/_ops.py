@@ -133,7 +133,8 @@ def restrict_kernel_backward(grad_weights, num_stencils):
 # ---------------------------------------------------------------------------------------- convolution
 class _Fusion(C.Structure):
     """aprnet_conv_fusion of the C ABI."""
-    _fields_ = [("x2", C.c_void_p), ("ldx2", C.c_int64), ("C2", C.c_int32), ("relu", C.c_int32)]
+    _fields_ = [("x2", C.c_void_p), ("ldx2", C.c_int64), ("C2", C.c_int32), ("relu", C.c_int32),
+                ("x2_coarse", C.c_void_p), ("ld_coarse", C.c_int64)]
 
 
 def conv_forward(aprs, x, weights, level_delta, bias=None, relu=False, x2=None):

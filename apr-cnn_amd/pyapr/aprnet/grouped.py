@@ -70,10 +70,21 @@ def ungroup(g, channels=None):
     return out
 
 
-def conv_forward(aprs, x, weights, level_delta, bias=None, relu=False, x2=None, grouped_output=True):
+def _fusion(x2, b, N, c2, relu, x2_coarse):
+    fu = _ops._Fusion(_ptr(x2.data[b]) if x2 is not None else None, N, c2, 1 if relu else 0)
+    if x2_coarse is not None:
+        if x2 is None or x2_coarse.channels != c2 or x2_coarse.data.shape[0] != x2.data.shape[0]:
+            raise ValueError("x2_coarse goes with a second input of the same batch size and channel count")
+        fu.x2_coarse, fu.ld_coarse = _ptr(x2_coarse.data[b]), x2_coarse.data.shape[2]
+    return fu
+
+
+def conv_forward(aprs, x, weights, level_delta, bias=None, relu=False, x2=None, grouped_output=True, x2_coarse=None):
     """Stencil convolution (3x3x3, 1x3x3, 1x5x5) on the bfloat16 matrix cores.  ``x``: Grouped, or a [B, C <= 3, N]
     bfloat16 plane tensor (the first layer of a network); ``x2``: optional Grouped second input whose channels follow
     those of x (the concatenation of a decoder stage).  weights [S_exp, Cout, Cin, kz, kx, ky] fp32.
+    ``x2_coarse``: the Grouped tensor at level_delta + 1 that x2 is the upsample_const_forward of; the mean tree of x2
+    is then read off it instead of computed from x2 (same values, an eighth of the reads).
     -> Grouped, or [B, Cout, N] planes with ``grouped_output=False``."""
     planes_in = not isinstance(x, Grouped)
     xd = x if planes_in else x.data
@@ -109,7 +120,7 @@ def conv_forward(aprs, x, weights, level_delta, bias=None, relu=False, x2=None, 
     with torch.cuda.device(xd.device):
         st = _stream()
         for b in range(B):
-            fu = _ops._Fusion(_ptr(x2.data[b]) if x2 is not None else None, N, c2, 1 if relu else 0)
+            fu = _fusion(x2, b, N, c2, relu, x2_coarse)
             rc = _lib().aprnet_conv_fwd_fused_bf16l(plans[b], d[b], kz, kx, ky, _ptr(xd[b]), N, c1, 0 if planes_in else 1, _ptr(weights),
                                                     s_exp, cout, None if bias is None else _ptr(bias), _ptr(out[b]), N,
                                                     1 if grouped_output else 0, _ptr(tree_ws), ld_tree, C.byref(fu), st)
@@ -123,7 +134,7 @@ def head_limits_ok(cout, head_weights):
     return cout <= 16 and head_weights.shape[1] <= 4 and tuple(head_weights.shape[3:]) == (1, 1, 1) and head_weights.shape[2] == cout
 
 
-def conv_head_forward(aprs, x, weights, level_delta, bias, head_weights, head_bias=None, relu=True, x2=None):
+def conv_head_forward(aprs, x, weights, level_delta, bias, head_weights, head_bias=None, relu=True, x2=None, x2_coarse=None):
     """The last stencil convolution of a network and the 1x1x1 convolution that follows it (unet_model.py:94) in one
     kernel: conv111(relu(conv(x) + bias)) without storing the layer's result.  ``x`` (and ``x2``) Grouped, weights
     [S_exp, Cout <= 16, Cin, kz, kx, ky], head_weights [S, C <= 4, Cout, 1, 1, 1] (not expanded), fp32
@@ -157,7 +168,7 @@ def conv_head_forward(aprs, x, weights, level_delta, bias, head_weights, head_bi
     with torch.cuda.device(out.device):
         st = _stream()
         for b in range(B):
-            fu = _ops._Fusion(_ptr(x2.data[b]) if x2 is not None else None, N, c2, 1 if relu else 0)
+            fu = _fusion(x2, b, N, c2, relu, x2_coarse)
             rc = _lib().aprnet_conv_fwd_head_bf16g(plans[b], d[b], kz, kx, ky, _ptr(x.data[b]), N, c1, _ptr(weights), s_exp, cout,
                                                    None if bias is None else _ptr(bias), _ptr(tree_ws), ld_tree, C.byref(fu),
                                                    _ptr(hw), hs, hc, None if hb is None else _ptr(hb), _ptr(out[b]), N, st)

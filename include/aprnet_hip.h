@@ -147,6 +147,11 @@ typedef struct aprnet_conv_fusion {
     int64_t ldx2;     /* the contraction, i.e. w has Cin + C2 input channels; NULL / 0 for a single input           */
     int32_t C2;
     int32_t relu;     /* nonzero: y = max(conv + bias, 0) */
+    const void* x2_coarse; /* grouped bfloat16 inputs only (aprnet_conv_fwd_fused_bf16l, aprnet_conv_fwd_head_bf16g), else NULL:  */
+    int64_t ld_coarse;     /* the tensor [C2 / 8][ld_coarse][8] at level_delta + 1 that x2 is the UpSampleConst of              */
+                           /* (UpConv.forward, unet_parts.py:79-83).  The mean tree of an upsampled tensor holds the values it   */
+                           /* was upsampled from, so the tree of x2 is taken from x2_coarse (an eighth of the values to read)   */
+                           /* instead of computed from x2; same results.  x2 itself is still read for the particles.             */
 } aprnet_conv_fusion;
 
 #define APRNET_DECL(T, SFX)                                                                                          \

@@ -132,6 +132,41 @@ def test_convolution_with_fused_head_equals_the_two_operators(c1, c2, cout, hc, 
     assert torch.equal(big, got)
 
 
+@pytest.mark.parametrize("ksize", [(3, 3, 3), (1, 3, 3)], ids=["333", "133"])
+@pytest.mark.parametrize("fill", [16, 17], ids=["needed-nodes", "whole-tree"])
+def test_tree_of_an_upsampled_second_input_is_read_off_its_source(fill, ksize):
+    """The second input of a decoder's first convolution is an upsampled tensor; its mean tree holds the values it was
+    upsampled from (a mean of equal values), so the convolution may read that tree off the source tensor instead of
+    computing it: bit-identical outputs, with the restricted and with the whole tree fill, with and without the head."""
+    aprs, ld, x, g = _batch(16, seed=4)
+    ld1 = ld + 1
+    n1 = max(oracle.number_parts(a, int(d)) for a, d in zip(aprs, ld1))
+    z = torch.randn(2, 24, n1, generator=g).to(torch.bfloat16)
+    for b, (a, d) in enumerate(zip(aprs, ld1)):
+        z[b, :, oracle.number_parts(a, int(d)):] = 0
+    zg = g8.regroup(z.to(DEV))
+    u = g8.upsample_const_forward(aprs, zg, ld1)
+    assert u.data.shape[2] == x.shape[2]
+    levels = max(a.level_max() - a.level_min() + 1 for a in aprs)
+    w = (torch.randn(levels, 16, 40, *ksize, generator=g) * 0.1).to(DEV)
+    bias = torch.randn(16, generator=g).to(DEV)
+    hw = torch.randn(1, 3, 16, 1, 1, 1, generator=g).to(DEV)
+    xa = g8.regroup(x)
+    lib = _native.hip()
+    assert lib.aprnet_set_conv_path(fill) == 0
+    try:
+        ref = g8.conv_forward(aprs, xa, w, ld, bias, relu=True, x2=u)
+        got = g8.conv_forward(aprs, xa, w, ld, bias, relu=True, x2=u, x2_coarse=zg)
+        href = g8.conv_head_forward(aprs, xa, w, ld, bias, hw, None, relu=True, x2=u)
+        hgot = g8.conv_head_forward(aprs, xa, w, ld, bias, hw, None, relu=True, x2=u, x2_coarse=zg)
+    finally:
+        assert lib.aprnet_set_conv_path(16) == 0
+    assert torch.equal(got.data, ref.data)
+    assert torch.equal(hgot, href)
+    with pytest.raises(ValueError):
+        g8.conv_forward(aprs, xa, w, ld, bias, relu=True, x2=u, x2_coarse=g8.regroup(z[:, :16].contiguous().to(DEV)))
+
+
 def test_fused_head_refuses_what_it_does_not_take():
     aprs, ld, x, g = _batch(32, seed=2)
     levels = max(a.level_max() - a.level_min() + 1 for a in aprs)
