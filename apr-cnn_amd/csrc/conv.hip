@@ -151,8 +151,9 @@ size_t conv_packed_floats(int code, int S_exp, int Cm, int Ck, bool transposed);
 int pack_conv_weights(int code, const float* w, int S_exp, int Cm, int Ck, bool transposed, float* packed, hipStream_t st);
 
 bool conv_narrow_supported(int code, int Cin);
-size_t conv_narrow_packed_floats(int code, int S_exp, int Cout, int Cin);
-int pack_conv_weights_narrow(int code, const float* w, int S_exp, int Cout, int Cin, float* packed, hipStream_t st);
+size_t conv_narrow_packed_floats(int code, int S_exp, int Cout, int Cin, bool bf16m);
+bool conv_narrow_bf16_math(int code, int Cin);
+int pack_conv_weights_narrow(int code, const float* w, int S_exp, int Cout, int Cin, float* packed, hipStream_t st, bool bf16m);
 int launch_conv_narrow(int code, const ConvArgs<float>& a, const WinLists& wl, hipStream_t st);
 int launch_conv_narrow(int code, const ConvArgs<bf16_t>& a, const WinLists& wl, hipStream_t st);
 static std::atomic<int> g_big_addr{0};       // bfloat16 forward on grouped tensors: 1 = 64-bit addresses also where 32-bit offsets would do
@@ -198,8 +199,10 @@ static int try_narrow(aprnet_plan* p, const ConvArgs<T>& a, int code, int d, con
     if (get_lists(p, d, code, tl, &wl, st) != 0) { (void)hipGetLastError(); return 0; }
     *done = true;
     ScratchLease lease;
-    if (int rc = lease.acquire(p, conv_narrow_packed_floats(code, a.S_exp, a.Cout, a.Cin) * sizeof(float), st)) return rc;
-    if (int rc = pack_conv_weights_narrow(code, (const float*)a.w, a.S_exp, a.Cout, a.Cin, (float*)p->d_scratch, st)) return rc;
+    // (bfloat16 features, one input channel, 3x3x3: the kernel's bfloat16 form and its image of the weights)
+    const bool bf16m = std::is_same<T, bf16_t>::value && conv_narrow_bf16_math(code, a.Cin);
+    if (int rc = lease.acquire(p, conv_narrow_packed_floats(code, a.S_exp, a.Cout, a.Cin, bf16m) * sizeof(float), st)) return rc;
+    if (int rc = pack_conv_weights_narrow(code, (const float*)a.w, a.S_exp, a.Cout, a.Cin, (float*)p->d_scratch, st, bf16m)) return rc;
     ConvArgs<T> b = a;
     b.w = (const float*)p->d_scratch;
     b.tile_win = wl.d_tile_win; b.win = wl.d_win;
@@ -345,7 +348,8 @@ int conv_fwd_bf16(const aprnet_plan* cp, int d, int kz, int kx, int ky, const bf
         return launch_fwd<bf16_t, G555, Chunk<float>::c555, 4>(a, tl.n, st);
     }
     if (conv_narrow_supported(code, Cin) && fu.C2 == 0) {
-        // a narrow first layer: fp32 products of the bfloat16 features on the pipelined kernel
+        // a narrow first layer on the pipelined kernel: one input channel of a 3x3x3 layer on the bfloat16 matrix
+        // instruction (weights rounded to bfloat16, as below), otherwise fp32 products of the bfloat16 features
         ConvArgs<bf16_t> n{};
         n.apr = p->dapr; n.tree = p->dtree; n.tiles = tl.d_tiles;
         n.x = x; n.ldx = ldx; n.Cin = Cin; n.w = w; n.S_exp = S_exp; n.Cout = Cout; n.bias = bias; n.relu = fu.relu;

@@ -57,6 +57,37 @@ __global__ void pack_weights_narrow_kernel(const float* __restrict__ w, int S_ex
     }
 }
 
+// bfloat16 features, one input channel, 3x3x3 (the first layer of a bfloat16 network): the 27 taps are the K of ONE
+// v_mfma_f32_16x16x32_bf16 per 16 columns instead of nine fp32 instructions; weights rounded to bfloat16, as in the
+// general bfloat16 kernel.  Slot i (0..7) of lane group g holds tap (row, dy), row = 3 dz + dx:
+//     g < 3:  rows 3 g, 3 g + 1 whole (slots 0-2, 3-5) and taps 0, 1 of row 3 g + 2 (slots 6, 7)
+//     g = 3:  tap 2 of rows 2, 5, 8 (slots 0, 3, 6); the other slots have zero weights
+// so every lane reads three runs of the patch, at cell + base A / B / C (+ 0, 1, 2): the same instructions for all lanes.
+__host__ __device__ inline int narrow_bf16_tap(int g, int i) {         // tap index row * 3 + dy of a slot, -1: none
+    if (g < 3) return (3 * g + i / 3) * 3 + i % 3;
+    return i % 3 == 0 ? (3 * (i / 3) + 2) * 3 + 2 : -1;
+}
+// packed[s][cb][h][lane]: the lane's 8 bfloat16 of the A operand (output channel (cb * COH + h) * 16 + lane % 16)
+__global__ void pack_weights_narrow_bf16_kernel(const float* __restrict__ w, int S_exp, int Cout, int COH, uint4* __restrict__ out) {
+    const int ncb = (Cout + 16 * COH - 1) / (16 * COH);
+    const unsigned n = (unsigned)S_exp * ncb * COH * 64;
+    for (unsigned e = blockIdx.x * blockDim.x + threadIdx.x; e < n; e += gridDim.x * blockDim.x) {
+        unsigned r = e;
+        const int lane = (int)(r % 64u); r /= 64u;
+        const int h = (int)(r % (unsigned)COH); r /= (unsigned)COH;
+        const int cb = (int)(r % (unsigned)ncb); r /= (unsigned)ncb;
+        const int s = (int)r;
+        const int co = (cb * COH + h) * 16 + (lane & 15), g = lane >> 4;
+        unsigned b[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const int t = narrow_bf16_tap(g, i);
+            b[i] = (t >= 0 && co < Cout) ? (unsigned)float_to_bf16(w[((int64_t)s * Cout + co) * 27 + t]).bits : 0u;
+        }
+        out[e] = make_uint4(b[0] | (b[1] << 16), b[2] | (b[3] << 16), b[4] | (b[5] << 16), b[6] | (b[7] << 16));
+    }
+}
+
 // two workgroups of eight waves per CU (three, at 80 registers with a few spills, ran slower: 2.0 against 1.25 ms)
 constexpr int NARROW_WAVES = 4;
 struct NarrowArgs {
@@ -69,15 +100,19 @@ struct NarrowArgs {
 
 // TREE: the windows may hold items that come from the tree (any level below the finest one of the call); without
 // it the tree loads, a third of a window's load instructions, are not issued at all
-template <typename T, class G, int CIN, int COH, bool TREE>
+// BM: the bfloat16 matrix instruction described above (bfloat16 features, CIN 1, 3x3x3)
+typedef __bf16 bf16x8n __attribute__((ext_vector_type(8)));
+template <typename T, class G, int CIN, int COH, bool TREE, bool BM = false>
 __global__ void __launch_bounds__(G::NT) __attribute__((amdgpu_waves_per_eu(NARROW_WAVES, NARROW_WAVES)))
 conv_narrow_kernel(const ConvArgs<T> a, const NarrowArgs na) {
+    static_assert(!BM || (std::is_same<T, bf16_t>::value && CIN == 1 && G::KZ == 3 && G::KX == 3 && G::KY == 3), "see narrow_bf16_tap");
     typedef NarrowShape<G, CIN> NS;
     constexpr int IPT = NS::IPT, NBW = ((G::MAXCOL + 15) / 16 + G::NWAVE - 1) / G::NWAVE;
     constexpr int PATCH = CIN * G::CH_STRIDE;
     static_assert((G::MAXCOL + 15) / 16 <= G::NWAVE * NBW, "a window must fit the accumulators of the block");
     __shared__ __attribute__((aligned(16))) float patch[3 * PATCH];
-    __shared__ float Wl[NS::STEPS * COH * 64];
+    __shared__ float Wl[BM ? 1 : NS::STEPS * COH * 64];
+    __shared__ __attribute__((aligned(16))) uint4 Wl16[BM ? COH * 64 : 1];
     __shared__ float bias_l[16 * COH];
 
     const int lane = lane_id();
@@ -97,6 +132,16 @@ conv_narrow_kernel(const ConvArgs<T> a, const NarrowArgs na) {
         int u = 4 * q + (lane >> 4);
         if (u >= NS::UNITS) u = 0;                       // zero weights: any cell the column really reads will do
         loff[q] = (u / G::KY) * G::CH_STRIDE + (u % G::KY) - G::TAP0;
+    }
+
+    // BM: the three runs of this lane group, relative to the column's cell
+    int runA = 0, runB = 0, runC = 0;
+    if constexpr (BM) {
+        auto row_off = [](int row) { return ((row / G::KX) * G::RX + (row % G::KX)) * G::RS; };
+        const int g = lane >> 4;
+        runA = (g < 3 ? row_off(3 * g) : row_off(2) + 2) - G::TAP0;
+        runB = (g < 3 ? row_off(3 * g + 1) : row_off(5) + 2) - G::TAP0;
+        runC = (g < 3 ? row_off(3 * g + 2) : row_off(8) + 2) - G::TAP0;
     }
 
     const __amdgpu_buffer_rsrc_t r_hdr = __builtin_amdgcn_make_buffer_rsrc(const_cast<int4*>(a.win), 0, (na.win0 + na.n_win) * 16, 0x00020000);
@@ -179,6 +224,11 @@ conv_narrow_kernel(const ConvArgs<T> a, const NarrowArgs na) {
     const int ncb = gridDim.y;
     auto stage_weights = [&](int level) {
         const int s_idx = min(a.S_exp - 1, a.Lc - level);
+        if constexpr (BM) {
+            const uint4* src16 = reinterpret_cast<const uint4*>(a.w) + ((int64_t)s_idx * ncb + blockIdx.y) * (COH * 64);
+            if (threadIdx.x < COH * 64) Wl16[threadIdx.x] = src16[threadIdx.x];
+            return;
+        }
         const float* src = a.w + ((int64_t)s_idx * ncb + blockIdx.y) * (NS::STEPS * COH * 64);
         for (int i = threadIdx.x; i < NS::STEPS * COH * 64; i += G::NT) Wl[i] = src[i];
     };
@@ -298,6 +348,30 @@ conv_narrow_kernel(const ConvArgs<T> a, const NarrowArgs na) {
             for (int h = 0; h < COH; ++h)
 #pragma unroll
                 for (int r = 0; r < 4; ++r) acc[j][h][r] = 0.f;
+        if constexpr (BM) {
+            if (nb > 0) {
+                lds_float* lp = (lds_float*)buf;
+                bf16x8n av[COH];
+#pragma unroll
+                for (int h = 0; h < COH; ++h) av[h] = __builtin_bit_cast(bf16x8n, Wl16[h * 64 + lane]);
+#pragma unroll
+                for (int j = 0; j < NBW; ++j) {
+                    if (j >= nb) break;                 // wave-uniform
+                    const int col = ((first + G::NWAVE * j) << 4) + (lane & 15);
+                    const int cell = col < nc ? (c0.pos[j] & (int)COL_CELL) : G::TAP0;
+                    lds_float* pa = lp + cell + runA; lds_float* pb = lp + cell + runB; lds_float* pc = lp + cell + runC;
+                    // the staged values are bfloat16 widened to fp32: the upper halves are the operand
+                    const unsigned f0 = __builtin_bit_cast(unsigned, pa[0]), f1 = __builtin_bit_cast(unsigned, pa[1]);
+                    const unsigned f2 = __builtin_bit_cast(unsigned, pa[2]), f3 = __builtin_bit_cast(unsigned, pb[0]);
+                    const unsigned f4 = __builtin_bit_cast(unsigned, pb[1]), f5 = __builtin_bit_cast(unsigned, pb[2]);
+                    const unsigned f6 = __builtin_bit_cast(unsigned, pc[0]), f7 = __builtin_bit_cast(unsigned, pc[1]);
+                    const bf16x8n bv = __builtin_bit_cast(bf16x8n, make_uint4(__builtin_amdgcn_perm(f1, f0, 0x07060302u), __builtin_amdgcn_perm(f3, f2, 0x07060302u),
+                                                                             __builtin_amdgcn_perm(f5, f4, 0x07060302u), __builtin_amdgcn_perm(f7, f6, 0x07060302u)));
+#pragma unroll
+                    for (int h = 0; h < COH; ++h) acc[j][h] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(av[h], bv, acc[j][h], 0, 0, 0);
+                }
+            }
+        } else
         if (nb > 0) {
             lds_float* lp = (lds_float*)buf;
             int bb[NBW][NS::Q];
@@ -343,17 +417,28 @@ template <class G> static void narrow_dims(int Cin, int* rows, int* q) {
 }
 static int narrow_coh(int Cout) { return Cout <= 16 ? 1 : 2; }
 
-size_t conv_narrow_packed_floats(int code, int S_exp, int Cout, int Cin) {
+// bfloat16 features on the bfloat16 matrix instruction (see narrow_bf16_tap)
+int bf16_math();
+bool conv_narrow_bf16_math(int code, int Cin) { return bf16_math() && code == 333 && Cin == 1; }
+size_t conv_narrow_packed_floats(int code, int S_exp, int Cout, int Cin, bool bf16m) {
+    if (bf16m) { const int coh = Cout <= 16 ? 1 : 2; return (size_t)S_exp * ((Cout + 16 * coh - 1) / (16 * coh)) * coh * 64 * 4; }
     int rows, q;
     if (code == 333) narrow_dims<N333>(Cin, &rows, &q); else if (code == 133) narrow_dims<N133>(Cin, &rows, &q); else narrow_dims<N155>(Cin, &rows, &q);
     const int coh = narrow_coh(Cout);
     return (size_t)S_exp * ((Cout + 16 * coh - 1) / (16 * coh)) * rows * q * coh * 64;
 }
 
-int pack_conv_weights_narrow(int code, const float* w, int S_exp, int Cout, int Cin, float* packed, hipStream_t st) {
+int pack_conv_weights_narrow(int code, const float* w, int S_exp, int Cout, int Cin, float* packed, hipStream_t st, bool bf16m) {
+    if (bf16m) {
+        const size_t n16 = conv_narrow_packed_floats(code, S_exp, Cout, Cin, true) / 4;
+        hipLaunchKernelGGL(pack_weights_narrow_bf16_kernel, dim3((unsigned)std::min<size_t>((n16 + 255) / 256, 1024)), dim3(256), 0, st, w, S_exp,
+                           Cout, Cout <= 16 ? 1 : 2, reinterpret_cast<uint4*>(packed));
+        APRNET_LAUNCH_CHECK("pack_weights_narrow_bf16_kernel");
+        return 0;
+    }
     int rows, q;
     if (code == 333) narrow_dims<N333>(Cin, &rows, &q); else if (code == 133) narrow_dims<N133>(Cin, &rows, &q); else narrow_dims<N155>(Cin, &rows, &q);
-    const size_t n = conv_narrow_packed_floats(code, S_exp, Cout, Cin);
+    const size_t n = conv_narrow_packed_floats(code, S_exp, Cout, Cin, false);
     const int ky = code % 10;
     hipLaunchKernelGGL(pack_weights_narrow_kernel, dim3((unsigned)std::min<size_t>((n + 255) / 256, 1024)), dim3(256), 0, st, w, S_exp, Cout, Cin,
                        ky, rows, q, narrow_coh(Cout), packed);
@@ -375,6 +460,19 @@ static int launch_narrow_cin(const ConvArgs<T>& a, const NarrowArgs& na, hipStre
         nb.n_win = part == 0 ? n_fine : na.n_win - n_fine;
         if (nb.n_win <= 0) continue;
         dim3 grid((unsigned)std::max(1, std::min(nb.n_win, 2 * cus)), (unsigned)((a.Cout + 16 * coh - 1) / (16 * coh)));
+        if constexpr (std::is_same<T, bf16_t>::value && CIN == 1 && G::KZ == 3) {
+            if (conv_narrow_bf16_math(333, 1)) {
+                if (part == 0) {
+                    if (coh == 1) hipLaunchKernelGGL((conv_narrow_kernel<T, G, CIN, 1, false, true>), grid, dim3(G::NT), 0, st, a, nb);
+                    else hipLaunchKernelGGL((conv_narrow_kernel<T, G, CIN, 2, false, true>), grid, dim3(G::NT), 0, st, a, nb);
+                } else {
+                    if (coh == 1) hipLaunchKernelGGL((conv_narrow_kernel<T, G, CIN, 1, true, true>), grid, dim3(G::NT), 0, st, a, nb);
+                    else hipLaunchKernelGGL((conv_narrow_kernel<T, G, CIN, 2, true, true>), grid, dim3(G::NT), 0, st, a, nb);
+                }
+                APRNET_LAUNCH_CHECK("conv_narrow_kernel");
+                continue;
+            }
+        }
         if (part == 0) {
             if (coh == 1) hipLaunchKernelGGL((conv_narrow_kernel<T, G, CIN, 1, false>), grid, dim3(G::NT), 0, st, a, nb);
             else hipLaunchKernelGGL((conv_narrow_kernel<T, G, CIN, 2, false>), grid, dim3(G::NT), 0, st, a, nb);

@@ -230,7 +230,8 @@ APRNET_DECL(double, f64)
  * Values are widened to fp32 on load, accumulated in fp32 and rounded to nearest even on store.  Weights
  * and bias are passed in fp32; the stencil convolution (3x3x3, 1x3x3, 1x5x5) rounds the weights to bfloat16
  * and multiplies on the bfloat16 matrix cores (aprnet_set_conv_path(3) keeps the weights and the products
- * in fp32; the 5x5x5 stencil has no matrix-core kernel and multiplies in fp32 on the vector-ALU kernel, forward
+ * in fp32; layers of 2 or 3 input channels, and one-channel layers of the 2-D stencils, keep fp32 weights and
+ * products; the 5x5x5 stencil has no matrix-core kernel and multiplies in fp32 on the vector-ALU kernel, forward
  * only).  Forward operators of the APR-UNet, plus the backward passes
  * of pool / upsample / tree fill and of the stencil convolution.  Argument meaning as
  * for the _f32 entry points. */
