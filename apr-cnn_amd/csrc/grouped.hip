@@ -106,9 +106,12 @@ fill_tree_level_g8_kernel(const int32_t* __restrict__ children, int64_t n_tree, 
 __global__ void __launch_bounds__(GTB)
 fill_tree_list_g8_kernel(const int32_t* __restrict__ children, int64_t n_tree, const int32_t* __restrict__ nodes, int64_t count,
                          const bf16_t* __restrict__ x, int64_t ldx, bf16_t* __restrict__ tree, int64_t ldt, int64_t tree_off, int from_x,
-                         int tree_first) {
+                         int tree_first, int G) {
     const int64_t i = (int64_t)blockIdx.x * GTB + threadIdx.x;
-    if (i < count) fill_node_g8(children, n_tree, nodes[i], x, ldx, tree, ldt, tree_off, from_x, tree_first, blockIdx.y);
+    if (i >= count) return;
+    const int64_t t = nodes[i];
+    // every channel group of the node in one thread: the list entry and the child table are read once
+    for (int q = 0; q < G; ++q) fill_node_g8(children, n_tree, t, x, ldx, tree, ldt, tree_off, from_x, tree_first, q);
 }
 
 constexpr int G_MAX_COARSE = 12;
@@ -149,9 +152,9 @@ int fill_tree_mean_g8(const aprnet_plan* p, int d, const bf16_t* x, int64_t ldx,
         const int from_x = (l + 1 == Lc);
         if (need && need->cnt[l] == 0) continue;
         if (need && !need->whole[l])
-            hipLaunchKernelGGL(fill_tree_list_g8_kernel, dim3((unsigned)((need->cnt[l] + GTB - 1) / GTB), (unsigned)G), dim3(GTB), 0, st,
+            hipLaunchKernelGGL(fill_tree_list_g8_kernel, dim3((unsigned)((need->cnt[l] + GTB - 1) / GTB)), dim3(GTB), 0, st,
                                p->d_children, p->n_tree, need->d_nodes + need->off[l], need->cnt[l], x, ldx, tree, ldt,
-                               from_x ? p->tree_offset(Lc) : 0, from_x, from_x && !particles_first);
+                               from_x ? p->tree_offset(Lc) : 0, from_x, from_x && !particles_first, G);
         else
             hipLaunchKernelGGL(fill_tree_level_g8_kernel, dim3((unsigned)((e - b + GTB - 1) / GTB), (unsigned)G), dim3(GTB), 0, st, p->d_children,
                                p->n_tree, b, e, x, ldx, tree, ldt, from_x ? p->tree_offset(Lc) : 0, from_x, from_x && !particles_first);
