@@ -98,9 +98,10 @@ __device__ __forceinline__ void fill_node_g8(const int32_t* children, int64_t n_
 
 __global__ void __launch_bounds__(GTB)
 fill_tree_level_g8_kernel(const int32_t* __restrict__ children, int64_t n_tree, int64_t t_begin, int64_t t_end, const bf16_t* __restrict__ x,
-                          int64_t ldx, bf16_t* __restrict__ tree, int64_t ldt, int64_t tree_off, int from_x, int tree_first) {
+                          int64_t ldx, bf16_t* __restrict__ tree, int64_t ldt, int64_t tree_off, int from_x, int tree_first, int G) {
     const int64_t t = t_begin + (int64_t)blockIdx.x * GTB + threadIdx.x;
-    if (t < t_end) fill_node_g8(children, n_tree, t, x, ldx, tree, ldt, tree_off, from_x, tree_first, blockIdx.y);
+    if (t >= t_end) return;
+    for (int q = 0; q < G; ++q) fill_node_g8(children, n_tree, t, x, ldx, tree, ldt, tree_off, from_x, tree_first, q);
 }
 
 __global__ void __launch_bounds__(GTB)
@@ -156,8 +157,8 @@ int fill_tree_mean_g8(const aprnet_plan* p, int d, const bf16_t* x, int64_t ldx,
                                p->d_children, p->n_tree, need->d_nodes + need->off[l], need->cnt[l], x, ldx, tree, ldt,
                                from_x ? p->tree_offset(Lc) : 0, from_x, from_x && !particles_first, G);
         else
-            hipLaunchKernelGGL(fill_tree_level_g8_kernel, dim3((unsigned)((e - b + GTB - 1) / GTB), (unsigned)G), dim3(GTB), 0, st, p->d_children,
-                               p->n_tree, b, e, x, ldx, tree, ldt, from_x ? p->tree_offset(Lc) : 0, from_x, from_x && !particles_first);
+            hipLaunchKernelGGL(fill_tree_level_g8_kernel, dim3((unsigned)((e - b + GTB - 1) / GTB)), dim3(GTB), 0, st, p->d_children,
+                               p->n_tree, b, e, x, ldx, tree, ldt, from_x ? p->tree_offset(Lc) : 0, from_x, from_x && !particles_first, G);
     }
     GCoarse lv{};
     for (int l = l_coarse; l >= p->tree.level_min; --l)
@@ -206,33 +207,37 @@ int tree_of_upsampled_g8(const aprnet_plan* p, int d, const bf16_t* z, int64_t l
 // downsampled particles, strict >, start value -1e17 (maxpool.hpp:51, 88-143).
 __global__ void __launch_bounds__(GTB)
 maxpool_g8_kernel(const int32_t* __restrict__ children, int64_t n_tree, int64_t n_copy, int64_t n_out, int64_t t_begin,
-                  const bf16_t* __restrict__ x, int64_t ldx, bf16_t* __restrict__ y, int64_t ldy, int64_t in_tree_off) {
+                  const bf16_t* __restrict__ x, int64_t ldx, int G, bf16_t* __restrict__ y, int64_t ldy, int64_t in_tree_off) {
     const int64_t i = (int64_t)blockIdx.x * GTB + threadIdx.x;
-    const int q = blockIdx.y;
     if (i >= n_out) return;
-    if (i < n_copy) { *g8_at(y, ldy, q, i) = *g8_at(x, ldx, q, i); return; }
+    if (i < n_copy) {
+        for (int q = 0; q < G; ++q) *g8_at(y, ldy, q, i) = *g8_at(x, ldx, q, i);
+        return;
+    }
     const int64_t t = t_begin + (i - n_copy);
-    int32_t ch[8];
+    int32_t ch[8];                        // read once for all channel groups
 #pragma unroll
     for (int s = 0; s < 8; ++s) ch[s] = children[(int64_t)s * n_tree + t];
-    uint4 raw[8];                         // unconditional loads, as in fill_node_g8
+    for (int q = 0; q < G; ++q) {
+        uint4 raw[8];                     // unconditional loads, as in fill_node_g8
 #pragma unroll
-    for (int s = 0; s < 8; ++s)
-        raw[s] = *g8_at(x, ldx, q, ch[s] >= 0 ? (int64_t)ch[s] : (ch[s] == NO_CHILD ? 0 : in_tree_off + ~ch[s]));
-    float best[8];
+        for (int s = 0; s < 8; ++s)
+            raw[s] = *g8_at(x, ldx, q, ch[s] >= 0 ? (int64_t)ch[s] : (ch[s] == NO_CHILD ? 0 : in_tree_off + ~ch[s]));
+        float best[8];
 #pragma unroll
-    for (int c = 0; c < 8; ++c) best[c] = -1e17f;
+        for (int c = 0; c < 8; ++c) best[c] = -1e17f;
 #pragma unroll
-    for (int pass = 0; pass < 2; ++pass)
+        for (int pass = 0; pass < 2; ++pass)
 #pragma unroll
-        for (int s = 0; s < 8; ++s) {
-            if (ch[s] == NO_CHILD || (pass == 0) != (ch[s] >= 0)) continue;
-            float f[8];
-            unpack8(raw[s], f);
+            for (int s = 0; s < 8; ++s) {
+                if (ch[s] == NO_CHILD || (pass == 0) != (ch[s] >= 0)) continue;
+                float f[8];
+                unpack8(raw[s], f);
 #pragma unroll
-            for (int c = 0; c < 8; ++c) if (f[c] > best[c]) best[c] = f[c];
-        }
-    *g8_at(y, ldy, q, i) = pack8(best);
+                for (int c = 0; c < 8; ++c) if (f[c] > best[c]) best[c] = f[c];
+            }
+        *g8_at(y, ldy, q, i) = pack8(best);
+    }
 }
 
 // upsample_fwd_kernel of tree_ops.hip: a downsampled particle's value goes to each of its children.  TWO lanes per
@@ -488,8 +493,8 @@ int aprnet_maxpool_fwd_bf16g(const aprnet_plan* p, int d, const uint16_t* x, int
     if (C <= 0 || n_out <= 0) return 0;
     if (ldy < n_out || ldx < p->number_parts(d)) return fail(APRNET_ERR_INVALID_ARGUMENT, "maxpool_forward: row shorter than the particle count");
     APRNET_HIP_CHECK(hipSetDevice(p->device));
-    hipLaunchKernelGGL(maxpool_g8_kernel, dim3((unsigned)((n_out + GTB - 1) / GTB), (unsigned)(C / 8)), dim3(GTB), 0, (hipStream_t)st,
-                       p->d_children, p->n_tree, n_copy, n_out, p->tree.level_begin(Lc - 1), (const bf16_t*)x, ldx, (bf16_t*)y, ldy,
+    hipLaunchKernelGGL(maxpool_g8_kernel, dim3((unsigned)((n_out + GTB - 1) / GTB)), dim3(GTB), 0, (hipStream_t)st,
+                       p->d_children, p->n_tree, n_copy, n_out, p->tree.level_begin(Lc - 1), (const bf16_t*)x, ldx, C / 8, (bf16_t*)y, ldy,
                        p->tree_offset(Lc));
     APRNET_LAUNCH_CHECK("maxpool_g8_kernel");
     return 0;
